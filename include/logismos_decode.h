@@ -1,0 +1,182 @@
+/*
+ * logismos_decode.h -- C ABI of the MI355X (gfx950) ragged-batch decode path.
+ *
+ * Every launcher follows the convention of the reference's HIP launchers
+ * (crates/kernels/src/matmul/hip/matmul_launchers.cpp:14-52,
+ *  crates/kernels/src/rms_norm/hip/rms_norm.hip:58-84,
+ *  crates/kernels/src/rope/hip/rope.hip:45-68):
+ *
+ *   - `extern "C"`, plain pointers and `int` dims, scalars by value, the
+ *     stream last;
+ *   - all pointers are caller-owned DEVICE memory, valid for the launch;
+ *     outputs never alias inputs; the launcher allocates and frees nothing;
+ *   - the launch is asynchronous on `stream`; nothing synchronises inside;
+ *   - the return value is the raw HIP status (`hipError_t` as uint32_t,
+ *     0 = success), the value the reference's Rust wrapper feeds to
+ *     `hipcore::ErrorKind::from_raw` (crates/hipcore/src/error.rs:125-150,
+ *     crates/kernels/src/matmul/mod.rs:140-186).  A shape the kernels cannot
+ *     address is rejected on the host before any launch with
+ *     hipErrorInvalidValue (1); nothing ever aborts;
+ *   - index arithmetic inside the kernels is 64-bit
+ *     (crates/kernels/src/matmul/hip/matmul_naive.hip:26-41).
+ *
+ * The library keeps no global mutable state and is re-entrant across
+ * streams (the reference's `Stream` is Send but not Sync,
+ * crates/hipcore/src/stream.rs:21-25: one caller thread per stream).
+ *
+ * The reference defines none of the data contracts below (its `sched`,
+ * paged `cache` and weight-`quant` crates are scaffolds); they extend the
+ * conventions it does define, cited at each item.
+ */
+#ifndef LOGISMOS_DECODE_H
+#define LOGISMOS_DECODE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Opaque stream handle: a `hipStream_t` (what `hipcore::Stream::raw()`
+ * yields, crates/hipcore/src/stream.rs).  NULL is the default stream. */
+typedef void* logismos_stream_t;
+
+/* Raw HIP status code. */
+typedef uint32_t logismos_status_t;
+
+/* ------------------------------------------------------------------------
+ * Data contracts
+ * ------------------------------------------------------------------------
+ *
+ * Paged KV pool.  K and V live in separate pools (the reference keeps K and
+ * V in separate per-layer buffers, crates/cache/src/flat.rs:84-89).  A pool
+ * is `[num_blocks][block_size][num_kv_heads][head_dim]` fp16, little-endian;
+ * one token row is `[num_kv_heads][head_dim]` contiguous, exactly a
+ * `FlatKvCache` row (`CacheLayout::row_elems`, crates/cache/src/flat.rs:36-69),
+ * and a block is `block_size` consecutive such rows.
+ *
+ * Block table.  int32, row-major `[num_seqs][max_blocks_per_seq]`; entry j of
+ * row s is the physical block that holds tokens [j*block_size,(j+1)*block_size)
+ * of sequence s.  Entries past ceil(context_len/block_size) are never read.
+ *
+ * Slot.  `slot = block_table[s][pos / block_size] * block_size + pos % block_size`
+ * (int64): the row index of token `pos` of sequence s inside a pool viewed as
+ * `[num_blocks*block_size][num_kv_heads*head_dim]`.
+ *
+ * cu_seqlens.  int32 exclusive prefix sum over the per-sequence number of NEW
+ * (query) tokens, leading 0, length num_seqs+1
+ * (research/14-gdn-aiter-preflight.md:338 is the only place the reference
+ * shows one: `[0,512,1536,2048]`).
+ *
+ * context_lens.  int32 `[num_seqs]`: tokens of the sequence visible to its
+ * LAST query token = prior context + new tokens.
+ *
+ * GQA.  Query head h reads KV head h / (num_q_heads / num_kv_heads)
+ * (`repeat_kv`, crates/transformers/src/attention.rs:366-382).
+ *
+ * Q8G32 weights (8-bit symmetric, group 32 along K; value-identical to ggml
+ * Q8_0, type id 8 in crates/loader/src/gguf.rs:57-78).  Device layout is
+ * planar: `qs` int8 `[N][K]` row-major and `d` fp16 `[N][K/32]`;
+ * w[n][k] = f16_to_f32(d[n][k/32]) * qs[n][k].
+ * `logismos_launch_repack_q8_0` converts ggml's 34-byte
+ * `{f16 d; int8 qs[32]}` blocks into it.
+ *
+ * Q4G128 weights (4-bit asymmetric, group 128 along K).  `qw` uint8
+ * `[N][K/2]`, element 2j in the low nibble of byte j and 2j+1 in the high
+ * nibble (index i at bit 4*i of a little-endian integer, the reference's
+ * only nibble convention: `pack_turbo4_indices`,
+ * crates/quant/src/lib.rs:272-285); `scale` fp16 `[N][K/128]`, `zero` fp16
+ * `[N][K/128]`; w[n][k] = (q - zero) * scale, q in [0,15].
+ */
+
+#define LOGISMOS_Q8_GROUP 32
+#define LOGISMOS_Q4_GROUP 128
+#define LOGISMOS_Q8_0_BLOCK_BYTES 34
+
+/* ------------------------------------------------------------------------
+ * Library identity / host-side shape guards (no device access; safe to call
+ * without a GPU).  The guards are the C counterpart of the reference's
+ * `check_matmul_shape` / `check_rope_shape` (crates/kernels/src/matmul/mod.rs:89-121,
+ * crates/kernels/src/rope/mod.rs:79-140): positive dims and every
+ * element-index product <= INT32_MAX.  They return 0 when the shape is
+ * accepted and hipErrorInvalidValue (1) otherwise; when `msg` is non-NULL a
+ * NUL-terminated reason is written into it (at most `msg_cap` bytes).
+ * ------------------------------------------------------------------------ */
+
+/* ABI version of this header; bumped on any signature change. */
+int logismos_decode_abi_version(void);
+
+/* The gfx target the kernels in this library were compiled for ("gfx950"). */
+const char* logismos_decode_offload_arch(void);
+
+logismos_status_t logismos_check_qgemv_q8g32_shape(int n, int k, char* msg, size_t msg_cap);
+
+logismos_status_t logismos_check_paged_attn_shape(int num_seqs, int total_tokens, int num_q_heads,
+                                                  int num_kv_heads, int head_dim, int block_size,
+                                                  int max_blocks_per_seq, int num_splits,
+                                                  char* msg, size_t msg_cap);
+
+/* ------------------------------------------------------------------------
+ * Quantized row-GEMV / GEMM
+ * ------------------------------------------------------------------------ */
+
+/* y[n] = sum_k x[k] * w[n][k], w in planar Q8G32.  x f32[K], y f32[N], fp32
+ * accumulation.  The quantized counterpart of `cpu_f32::linear_t` at m = 1
+ * (crates/kernels/src/cpu_f32/mod.rs:271-345: weight is `[out,in]`
+ * row-major).  Requires k % 32 == 0.  qs must be 16-byte aligned. */
+logismos_status_t logismos_launch_qgemv_q8g32_f32(const void* x_f32, const void* qs_i8,
+                                                  const void* d_f16, void* y_f32, int n, int k,
+                                                  logismos_stream_t stream);
+
+/* ggml Q8_0 block stream `[N][K/32]{f16 d; int8 qs[32]}` -> planar Q8G32. */
+logismos_status_t logismos_launch_repack_q8_0(const void* blocks_q8_0, void* qs_i8, void* d_f16,
+                                              int n, int k, logismos_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Paged attention (ragged batch: decode rows and chunked-prefill rows)
+ * ------------------------------------------------------------------------ */
+
+/* Number of KV partitions ("splits") the decode kernel should use for this
+ * problem size; pure host arithmetic, deterministic.  Pass the result both to
+ * the workspace query and to the launcher. */
+int logismos_paged_attn_num_splits(int num_seqs, int num_kv_heads, int block_size,
+                                   int max_blocks_per_seq);
+
+/* Bytes of split-K workspace the launcher needs for these arguments. */
+size_t logismos_paged_attn_workspace_bytes(int num_seqs, int num_q_heads, int head_dim,
+                                           int num_splits);
+
+/* out[t][h][:] = softmax_j( (q[t][h] . k[j][h/g]) * scale ) . v[j][h/g]
+ * over the keys j visible to query token t.
+ *
+ *   q, out          fp16 `[total_tokens][num_q_heads][head_dim]`
+ *   k_pool, v_pool  paged pools as described above
+ *   block_tables    int32 `[num_seqs][max_blocks_per_seq]`
+ *   cu_seqlens_q    int32 `[num_seqs+1]`; sequence s owns query tokens
+ *                   [cu[s], cu[s+1])
+ *   context_lens    int32 `[num_seqs]`
+ *   workspace       `logismos_paged_attn_workspace_bytes(...)` bytes, contents
+ *                   don't matter on entry; must not be shared by launches that
+ *                   can overlap in time
+ *   causal != 0     query token i (0-based) of a sequence with n new tokens
+ *                   and context c sees keys [0, c - n + i]; causal == 0: all c
+ *                   keys.  For n == 1 both coincide.
+ *
+ * The scale multiplies the dot product (it is not folded into q), as in
+ * `QwenAttention::forward` (crates/transformers/src/attention.rs:225-241);
+ * the softmax is fp32 and max-subtracted
+ * (`softmax_last_dim`, crates/kernels/src/cpu_f32/mod.rs:380-433); a query
+ * with no visible key yields zeros.  Requires head_dim == 128,
+ * block_size % 16 == 0, num_q_heads % num_kv_heads == 0 and a group size
+ * num_q_heads/num_kv_heads <= 8. */
+logismos_status_t logismos_launch_paged_attn_varlen_fp16(
+    const void* q_f16, const void* k_pool_f16, const void* v_pool_f16, const int32_t* block_tables,
+    const int32_t* cu_seqlens_q, const int32_t* context_lens, void* out_f16, void* workspace,
+    int num_seqs, int total_tokens, int num_q_heads, int num_kv_heads, int head_dim, int block_size,
+    int max_blocks_per_seq, int num_splits, float scale, int causal, logismos_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LOGISMOS_DECODE_H */
