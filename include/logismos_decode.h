@@ -112,10 +112,10 @@ const char* logismos_decode_offload_arch(void);
 
 logismos_status_t logismos_check_qgemv_q8g32_shape(int n, int k, char* msg, size_t msg_cap);
 
-logismos_status_t logismos_check_paged_attn_shape(int num_seqs, int total_tokens, int num_q_heads,
-                                                  int num_kv_heads, int head_dim, int block_size,
-                                                  int max_blocks_per_seq, int num_splits,
-                                                  char* msg, size_t msg_cap);
+logismos_status_t logismos_check_paged_attn_shape(int num_seqs, int total_tokens, int max_seqlen_q,
+                                                  int num_q_heads, int num_kv_heads, int head_dim,
+                                                  int block_size, int max_blocks_per_seq,
+                                                  int num_splits, char* msg, size_t msg_cap);
 
 /* ------------------------------------------------------------------------
  * Quantized row-GEMV / GEMM
@@ -156,6 +156,11 @@ size_t logismos_paged_attn_workspace_bytes(int num_seqs, int num_q_heads, int he
  *   cu_seqlens_q    int32 `[num_seqs+1]`; sequence s owns query tokens
  *                   [cu[s], cu[s+1])
  *   context_lens    int32 `[num_seqs]`
+ *   total_tokens    cu_seqlens_q[num_seqs]; max_seqlen_q: the largest number of
+ *                   new tokens of any sequence (both known to the host-side
+ *                   scheduler; 1 for a pure decode step)
+ *   num_splits      KV partitions per decode sequence (>= 1), e.g. from
+ *                   `logismos_paged_attn_num_splits`
  *   workspace       `logismos_paged_attn_workspace_bytes(...)` bytes, contents
  *                   don't matter on entry; must not be shared by launches that
  *                   can overlap in time
@@ -173,8 +178,26 @@ size_t logismos_paged_attn_workspace_bytes(int num_seqs, int num_q_heads, int he
 logismos_status_t logismos_launch_paged_attn_varlen_fp16(
     const void* q_f16, const void* k_pool_f16, const void* v_pool_f16, const int32_t* block_tables,
     const int32_t* cu_seqlens_q, const int32_t* context_lens, void* out_f16, void* workspace,
-    int num_seqs, int total_tokens, int num_q_heads, int num_kv_heads, int head_dim, int block_size,
-    int max_blocks_per_seq, int num_splits, float scale, int causal, logismos_stream_t stream);
+    int num_seqs, int total_tokens, int max_seqlen_q, int num_q_heads, int num_kv_heads,
+    int head_dim, int block_size, int max_blocks_per_seq, int num_splits, float scale, int causal,
+    logismos_stream_t stream);
+
+/* The same launch restricted to some of its phases (bitmask).  The full
+ * launcher runs, in order: the decode kernel (sequences with one new token,
+ * KV partitions in parallel), the prefill kernel (sequences with more than one
+ * new token; skipped when max_seqlen_q <= 1) and the merge of the decode
+ * partitions (skipped when num_splits == 1).  For callers that place the
+ * phases on different streams, and for per-kernel timing. */
+#define LOGISMOS_ATTN_PHASE_DECODE 1
+#define LOGISMOS_ATTN_PHASE_PREFILL 2
+#define LOGISMOS_ATTN_PHASE_MERGE 4
+#define LOGISMOS_ATTN_PHASE_ALL 7
+logismos_status_t logismos_launch_paged_attn_varlen_fp16_phases(
+    const void* q_f16, const void* k_pool_f16, const void* v_pool_f16, const int32_t* block_tables,
+    const int32_t* cu_seqlens_q, const int32_t* context_lens, void* out_f16, void* workspace,
+    int num_seqs, int total_tokens, int max_seqlen_q, int num_q_heads, int num_kv_heads,
+    int head_dim, int block_size, int max_blocks_per_seq, int num_splits, float scale, int causal,
+    int phases, logismos_stream_t stream);
 
 #ifdef __cplusplus
 }

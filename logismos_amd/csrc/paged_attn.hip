@@ -1,0 +1,456 @@
+// Ragged paged attention for gfx950 (head_dim 128, fp16 KV, fp32 softmax).
+//
+// One wave64 owns one (query token, KV head, KV partition) and serves the
+// whole GQA group of that KV head, so every K/V byte is fetched from HBM once
+// per group.  Work inside the wave, per tile of 16 keys (a tile never
+// straddles a KV block because block_size % 16 == 0):
+//
+//   * K: lane (tg = lane/16, c = lane%16) loads key c of the tile, 16-byte
+//     pieces tg, tg+4, tg+8, tg+12 of its 256-byte row, straight into the
+//     A-operand layout of v_mfma_f32_16x16x32_f16 (row = key, 8 consecutive
+//     contraction elements per lane).  The query group sits in registers as
+//     the B operand (column = head, same piece order), so four MFMAs give the
+//     16 keys x 16 heads score tile; lane (tg, c) ends up with the scores of
+//     head c for keys 4*tg..4*tg+3.
+//   * V: lane (tg, c) loads the 16-byte piece c of keys 4*tg..4*tg+3: each
+//     wave instruction covers four whole 256-byte rows.
+//   * The 16 lanes of a row (fixed tg) therefore hold both the scores and the
+//     values of the same four keys per tile: each row runs its own online
+//     softmax (running max / sum in the lanes c < G) with no traffic between
+//     rows; probabilities reach the value lanes through DPP row broadcasts and
+//     are applied with mixed-precision FMAs (fp16 value, fp32 accumulator).
+//   * The four rows are merged once at the end (log-sum-exp merge over
+//     ds_bpermute), then either normalised and written as fp16 (single
+//     partition) or written as an fp32 partial (m, l, acc) that the merge
+//     kernel combines across partitions.
+//
+// Tiles are double-buffered in registers: the loads of tile i+1 are in flight
+// while tile i is consumed.  Physical block ids come through scalar loads.
+//
+// Algorithmic HBM bytes per (sequence, KV head): ctx * 2 * 256 (K and V rows)
+// + G * 256 * 2 (q, out) + 4 * ceil(ctx/block_size) (block table).
+#include "device_utils.hpp"
+#include "launch_common.hpp"
+
+#include <hip/hip_fp16.h>
+#include <math.h>
+
+namespace lg {
+
+constexpr int kHeadDim = 128;
+constexpr int kTileKeys = 16;
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct KvTile {
+    half8_t k[4];
+    half8_t v[4];
+};
+
+struct AttnParams {
+    const _Float16* q;
+    const _Float16* k_pool;
+    const _Float16* v_pool;
+    const int32_t* block_tables;
+    const int32_t* cu_seqlens_q;
+    const int32_t* context_lens;
+    _Float16* out;
+    float* ws_acc;  // [num_seqs][num_splits][hq][128]
+    float* ws_ml;   // [num_seqs][num_splits][hq][2]
+    int num_seqs;
+    int hq;
+    int hkv;
+    int block_size;
+    int max_blocks_per_seq;
+    int num_splits;
+    int part_tokens;  // keys per partition (multiple of 16)
+    float scale_log2e;
+    int causal;
+};
+
+// DECODE = true : grid (num_splits, hkv, num_seqs); sequences with exactly one
+//                 new token, keys split into partitions of part_tokens.
+// DECODE = false: grid (max_seqlen_q, hkv, num_seqs); one wave per query token
+//                 of the sequences with more than one new token, whole visible
+//                 context in one partition.
+template <int G, bool DECODE>
+__global__ __launch_bounds__(64) void paged_attn_kernel(const AttnParams p) {
+    const int lane = threadIdx.x;
+    const int tg = lane >> 4;
+    const int c = lane & 15;
+    const int kvh = blockIdx.y;
+    const int s = blockIdx.z;
+
+    const int t0 = p.cu_seqlens_q[s];
+    const int n_new = p.cu_seqlens_q[s + 1] - t0;
+    const int ctx = p.context_lens[s];
+    int t, vis, tok_begin, tok_end, split;
+    if constexpr (DECODE) {
+        if (n_new != 1) return;
+        t = t0;
+        vis = ctx;
+        split = blockIdx.x;
+        tok_begin = split * p.part_tokens;
+    } else {
+        const int i = blockIdx.x;
+        if (n_new <= 1 || i >= n_new) return;
+        t = t0 + i;
+        vis = p.causal ? (ctx - n_new + i + 1) : ctx;
+        vis = vis > ctx ? ctx : vis;
+        split = 0;
+        tok_begin = 0;
+    }
+    if (vis <= 0) {
+        // no visible key: zeros (softmax over zero columns)
+        if (split == 0 && c < G) {
+            half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+            _Float16* o = p.out + ((int64_t)t * p.hq + kvh * G + c) * kHeadDim;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) *reinterpret_cast<half8_t*>(o + 8 * (tg + 4 * j)) = z;
+        }
+        return;
+    }
+    if (tok_begin >= vis) return;
+    tok_end = DECODE ? min(vis, tok_begin + p.part_tokens) : vis;
+    const int num_parts = DECODE ? (vis + p.part_tokens - 1) / p.part_tokens : 1;
+    const int ntiles = (tok_end - tok_begin + kTileKeys - 1) / kTileKeys;
+
+    // ---- query group as the MFMA B operand: column = head c, piece tg + 4j
+    half8_t qreg[4];
+    {
+        const half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+        const _Float16* qp =
+            p.q + ((int64_t)t * p.hq + kvh * G + (c < G ? c : 0)) * kHeadDim + 8 * tg;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            qreg[j] = (c < G) ? *reinterpret_cast<const half8_t*>(qp + 32 * j) : z;
+    }
+
+    // ---- tile loader.  The physical block id is a scalar load (wave-uniform
+    // address), so waiting for it never waits for the vector loads in flight.
+    const int32_t* bt_row = p.block_tables + (int64_t)s * p.max_blocks_per_seq;
+
+    // lane-constant element offsets inside a tile (row stride = hkv * 128)
+    const unsigned row_stride = (unsigned)p.hkv * kHeadDim;
+    const unsigned k_lane_off = (unsigned)c * row_stride;
+    unsigned v_lane_off[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v_lane_off[i] = (unsigned)(4 * tg + i) * row_stride;
+
+    auto load_tile = [&](int tile, KvTile& kv) {
+        const int tok_base = __builtin_amdgcn_readfirstlane(tok_begin + tile * kTileKeys);
+        const int blk_idx = tok_base / p.block_size;
+        const int blk = bt_row[blk_idx];
+        // wave-uniform 64-bit base of the tile's first row, this KV head
+        const int64_t row_base = (int64_t)blk * p.block_size + (tok_base - blk_idx * p.block_size);
+        const int64_t base = (row_base * p.hkv + kvh) * kHeadDim;
+        const _Float16* kb = p.k_pool + base;
+        const _Float16* vb = p.v_pool + base;
+        // keys past the end of the partition re-read its last key (their
+        // probability is forced to zero below); never touches another block
+        const unsigned last_off = (unsigned)(tok_end - 1 - tok_base) * row_stride;
+        const unsigned ko = min(k_lane_off, last_off) + 8u * tg;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) kv.k[j] = *reinterpret_cast<const half8_t*>(kb + ko + 32 * j);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const unsigned vo = min(v_lane_off[i], last_off) + 8u * c;
+            kv.v[i] = *reinterpret_cast<const half8_t*>(vb + vo);
+        }
+    };
+
+    float m = -INFINITY;  // running max (log2 domain), meaningful in lanes c < G
+    float l = 0.0f;       // running sum
+    float acc[G][8];
+#pragma unroll
+    for (int h = 0; h < G; ++h)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[h][e] = 0.0f;
+
+    auto compute_tile = [&](int tile, const KvTile& kv) {
+        float4_t sacc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kv.k[j], qreg[j], sacc, 0, 0, 0);
+        const int tok0 = tok_begin + tile * kTileKeys + 4 * tg;
+        float sc[4];
+        float mx = m;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            sc[r] = (tok0 + r < tok_end) ? sacc[r] * p.scale_log2e : -INFINITY;
+            mx = fmaxf(mx, sc[r]);
+        }
+        const float msafe = (mx == -INFINITY) ? 0.0f : mx;
+        const float alpha = fast_exp2(m - msafe);
+        float pr[4];
+        float psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            pr[r] = fast_exp2(sc[r] - msafe);
+            psum += pr[r];
+        }
+        l = l * alpha + psum;
+        m = mx;
+        static_for<G>([&](auto hc) {
+            constexpr int h = decltype(hc)::value;
+            const float a = row_bcast<h>(alpha);
+            const float p0 = row_bcast<h>(pr[0]);
+            const float p1 = row_bcast<h>(pr[1]);
+            const float p2 = row_bcast<h>(pr[2]);
+            const float p3 = row_bcast<h>(pr[3]);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float v = acc[h][e] * a;
+                v = fmaf(p0, (float)kv.v[0][e], v);
+                v = fmaf(p1, (float)kv.v[1][e], v);
+                v = fmaf(p2, (float)kv.v[2][e], v);
+                v = fmaf(p3, (float)kv.v[3][e], v);
+                acc[h][e] = v;
+            }
+        });
+    };
+
+    // Register double buffer, two tiles per iteration in one straight-line
+    // body: every iteration issues the same loads (the tile index is clamped;
+    // a tile past the end re-reads the last one and is fully masked in
+    // compute_tile), so the loads of the next tile stay in flight while the
+    // current one is consumed and the wait counts stay exact.
+    KvTile buf0, buf1;
+    const int last_tile = ntiles - 1;
+    load_tile(0, buf0);
+    for (int tile = 0; tile < ntiles; tile += 2) {
+        load_tile(min(tile + 1, last_tile), buf1);
+        __builtin_amdgcn_sched_barrier(0);  // keep the prefetch above the math
+        compute_tile(tile, buf0);
+        __builtin_amdgcn_sched_barrier(0);
+        load_tile(min(tile + 2, last_tile), buf0);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_tile(tile + 1, buf1);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // ---- merge the four rows of the wave, then write
+    static_for<G>([&](auto hc) {
+        constexpr int h = decltype(hc)::value;
+        float mh = row_bcast<h>(m);
+        float lh = row_bcast<h>(l);
+#pragma unroll
+        for (int mask = 16; mask <= 32; mask <<= 1) {
+            const float mo = shfl_xor_f32(mh, mask);
+            const float mn = fmaxf(mh, mo);
+            const float msafe = (mn == -INFINITY) ? 0.0f : mn;
+            const float f = fast_exp2(mh - msafe);
+            lh *= f;
+            lh += shfl_xor_f32(lh, mask);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float v = acc[h][e] * f;
+                acc[h][e] = v + shfl_xor_f32(v, mask);
+            }
+            mh = mn;
+        }
+        if (tg == (h & 3)) {
+            const int head = kvh * G + h;
+            if (num_parts == 1) {
+                const float inv = 1.0f / lh;
+                half8_t o;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[e] = (_Float16)(acc[h][e] * inv);
+                *reinterpret_cast<half8_t*>(p.out + ((int64_t)t * p.hq + head) * kHeadDim + 8 * c) = o;
+            } else {
+                const int64_t idx = ((int64_t)s * p.num_splits + split) * p.hq + head;
+                float4_t a0 = {acc[h][0], acc[h][1], acc[h][2], acc[h][3]};
+                float4_t a1 = {acc[h][4], acc[h][5], acc[h][6], acc[h][7]};
+                float* dst = p.ws_acc + idx * kHeadDim + 8 * c;
+                *reinterpret_cast<float4_t*>(dst) = a0;
+                *reinterpret_cast<float4_t*>(dst + 4) = a1;
+                if (c == 0) {
+                    p.ws_ml[idx * 2] = mh;
+                    p.ws_ml[idx * 2 + 1] = lh;
+                }
+            }
+        }
+    });
+}
+
+// Combines the partials of the decode sequences that used more than one
+// partition.  grid (hq, num_seqs), 128 threads = one per output element.
+__global__ __launch_bounds__(128) void paged_attn_merge_kernel(const AttnParams p) {
+    const int s = blockIdx.y;
+    const int h = blockIdx.x;
+    const int d = threadIdx.x;
+    const int t0 = p.cu_seqlens_q[s];
+    if (p.cu_seqlens_q[s + 1] - t0 != 1) return;
+    const int ctx = p.context_lens[s];
+    const int np = (ctx + p.part_tokens - 1) / p.part_tokens;
+    if (np <= 1) return;
+    const int64_t base = ((int64_t)s * p.num_splits) * p.hq + h;
+    float mmax = -INFINITY;
+    for (int i = 0; i < np; ++i) mmax = fmaxf(mmax, p.ws_ml[(base + (int64_t)i * p.hq) * 2]);
+    float num = 0.0f, den = 0.0f;
+    for (int i = 0; i < np; ++i) {
+        const int64_t idx = base + (int64_t)i * p.hq;
+        const float f = fast_exp2(p.ws_ml[idx * 2] - mmax);
+        den = fmaf(f, p.ws_ml[idx * 2 + 1], den);
+        num = fmaf(f, p.ws_acc[idx * kHeadDim + d], num);
+    }
+    p.out[((int64_t)t0 * p.hq + h) * kHeadDim + d] = (_Float16)(num / den);
+}
+
+static int part_tokens_for(int block_size, int max_blocks_per_seq, int num_splits) {
+    const int64_t max_ctx = (int64_t)block_size * max_blocks_per_seq;
+    int64_t part = (max_ctx + num_splits - 1) / num_splits;
+    part = (part + kTileKeys - 1) / kTileKeys * kTileKeys;
+    return (int)part;
+}
+
+template <int G>
+static hipError_t launch_group(const AttnParams& p, int max_seqlen_q, int phases,
+                               hipStream_t stream) {
+    dim3 block(64);
+    if (phases & LOGISMOS_ATTN_PHASE_DECODE) {
+        dim3 grid_d(p.num_splits, p.hkv, p.num_seqs);
+        paged_attn_kernel<G, true><<<grid_d, block, 0, stream>>>(p);
+    }
+    if ((phases & LOGISMOS_ATTN_PHASE_PREFILL) && max_seqlen_q > 1) {
+        dim3 grid_p(max_seqlen_q, p.hkv, p.num_seqs);
+        paged_attn_kernel<G, false><<<grid_p, block, 0, stream>>>(p);
+    }
+    if ((phases & LOGISMOS_ATTN_PHASE_MERGE) && p.num_splits > 1) {
+        dim3 grid_m(p.hq, p.num_seqs);
+        paged_attn_merge_kernel<<<grid_m, dim3(128), 0, stream>>>(p);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace lg
+
+extern "C" logismos_status_t logismos_check_paged_attn_shape(int num_seqs, int total_tokens,
+                                                             int max_seqlen_q, int num_q_heads,
+                                                             int num_kv_heads, int head_dim,
+                                                             int block_size, int max_blocks_per_seq,
+                                                             int num_splits, char* msg,
+                                                             size_t msg_cap) {
+    const char* k = "paged_attn_varlen_fp16";
+    struct {
+        int v;
+        const char* name;
+    } pos[] = {{num_seqs, "num_seqs"},         {num_q_heads, "num_q_heads"},
+               {num_kv_heads, "num_kv_heads"}, {head_dim, "head_dim"},
+               {block_size, "block_size"},     {max_blocks_per_seq, "max_blocks_per_seq"},
+               {num_splits, "num_splits"}};
+    for (auto& e : pos)
+        if (e.v <= 0) return lg::reject(msg, msg_cap, "%s: %s must be positive, got %d", k, e.name, e.v);
+    if (total_tokens < 0 || max_seqlen_q < 0)
+        return lg::reject(msg, msg_cap, "%s: total_tokens / max_seqlen_q must be >= 0", k);
+    if (max_seqlen_q > total_tokens)
+        return lg::reject(msg, msg_cap, "%s: max_seqlen_q = %d exceeds total_tokens = %d", k,
+                          max_seqlen_q, total_tokens);
+    if (head_dim != lg::kHeadDim)
+        return lg::reject(msg, msg_cap, "%s: head_dim must be 128, got %d", k, head_dim);
+    if (block_size % 16 != 0)
+        return lg::reject(msg, msg_cap, "%s: block_size = %d is not a multiple of 16", k, block_size);
+    if (num_q_heads % num_kv_heads != 0)
+        return lg::reject(msg, msg_cap, "%s: num_q_heads = %d is not a multiple of num_kv_heads = %d",
+                          k, num_q_heads, num_kv_heads);
+    if (num_q_heads / num_kv_heads > 8)
+        return lg::reject(msg, msg_cap, "%s: GQA group size %d exceeds 8", k,
+                          num_q_heads / num_kv_heads);
+    if (num_seqs > 65535 || num_kv_heads > 65535)
+        return lg::reject(msg, msg_cap, "%s: num_seqs and num_kv_heads must be <= 65535", k);
+    const int64_t i32max = INT32_MAX;
+    if ((int64_t)total_tokens * num_q_heads * head_dim > i32max)
+        return lg::reject(msg, msg_cap, "%s: total_tokens*num_q_heads*head_dim exceeds i32::MAX", k);
+    if ((int64_t)block_size * max_blocks_per_seq > i32max)
+        return lg::reject(msg, msg_cap, "%s: block_size*max_blocks_per_seq exceeds i32::MAX", k);
+    if ((int64_t)num_seqs * max_blocks_per_seq > i32max)
+        return lg::reject(msg, msg_cap, "%s: num_seqs*max_blocks_per_seq exceeds i32::MAX", k);
+    if ((int64_t)num_seqs * num_splits * num_q_heads > i32max / 130)
+        return lg::reject(msg, msg_cap, "%s: split-K workspace index exceeds i32::MAX", k);
+    return 0;
+}
+
+extern "C" int logismos_paged_attn_num_splits(int num_seqs, int num_kv_heads, int block_size,
+                                              int max_blocks_per_seq) {
+    if (num_seqs <= 0 || num_kv_heads <= 0 || block_size <= 0 || max_blocks_per_seq <= 0) return 1;
+    // Aim at ~4096 waves over the chip if every sequence were full length,
+    // with partitions of 64..512 keys.
+    const int64_t max_ctx = (int64_t)block_size * max_blocks_per_seq;
+    int64_t part = (int64_t)num_seqs * num_kv_heads * max_ctx / 4096;
+    if (part < 64) part = 64;
+    if (part > 512) part = 512;
+    part = (part + 15) / 16 * 16;
+    int64_t splits = (max_ctx + part - 1) / part;
+    if (splits < 1) splits = 1;
+    if (splits > 4096) splits = 4096;
+    return (int)splits;
+}
+
+extern "C" size_t logismos_paged_attn_workspace_bytes(int num_seqs, int num_q_heads, int head_dim,
+                                                      int num_splits) {
+    if (num_seqs <= 0 || num_q_heads <= 0 || head_dim <= 0 || num_splits <= 1) return 0;
+    return (size_t)num_seqs * (size_t)num_splits * (size_t)num_q_heads * (size_t)(head_dim + 2) *
+           sizeof(float);
+}
+
+extern "C" logismos_status_t logismos_launch_paged_attn_varlen_fp16(
+    const void* q_f16, const void* k_pool_f16, const void* v_pool_f16, const int32_t* block_tables,
+    const int32_t* cu_seqlens_q, const int32_t* context_lens, void* out_f16, void* workspace,
+    int num_seqs, int total_tokens, int max_seqlen_q, int num_q_heads, int num_kv_heads,
+    int head_dim, int block_size, int max_blocks_per_seq, int num_splits, float scale, int causal,
+    logismos_stream_t stream) {
+    return logismos_launch_paged_attn_varlen_fp16_phases(
+        q_f16, k_pool_f16, v_pool_f16, block_tables, cu_seqlens_q, context_lens, out_f16, workspace,
+        num_seqs, total_tokens, max_seqlen_q, num_q_heads, num_kv_heads, head_dim, block_size,
+        max_blocks_per_seq, num_splits, scale, causal, LOGISMOS_ATTN_PHASE_ALL, stream);
+}
+
+extern "C" logismos_status_t logismos_launch_paged_attn_varlen_fp16_phases(
+    const void* q_f16, const void* k_pool_f16, const void* v_pool_f16, const int32_t* block_tables,
+    const int32_t* cu_seqlens_q, const int32_t* context_lens, void* out_f16, void* workspace,
+    int num_seqs, int total_tokens, int max_seqlen_q, int num_q_heads, int num_kv_heads,
+    int head_dim, int block_size, int max_blocks_per_seq, int num_splits, float scale, int causal,
+    int phases, logismos_stream_t stream) {
+    if (logismos_check_paged_attn_shape(num_seqs, total_tokens, max_seqlen_q, num_q_heads,
+                                        num_kv_heads, head_dim, block_size, max_blocks_per_seq,
+                                        num_splits, nullptr, 0) != 0)
+        return hipErrorInvalidValue;
+    if (total_tokens == 0) return hipSuccess;
+    if (!q_f16 || !k_pool_f16 || !v_pool_f16 || !block_tables || !cu_seqlens_q || !context_lens ||
+        !out_f16)
+        return hipErrorInvalidValue;
+    if (num_splits > 1 && !workspace) return hipErrorInvalidValue;
+
+    lg::AttnParams p;
+    p.q = static_cast<const _Float16*>(q_f16);
+    p.k_pool = static_cast<const _Float16*>(k_pool_f16);
+    p.v_pool = static_cast<const _Float16*>(v_pool_f16);
+    p.block_tables = block_tables;
+    p.cu_seqlens_q = cu_seqlens_q;
+    p.context_lens = context_lens;
+    p.out = static_cast<_Float16*>(out_f16);
+    p.ws_acc = static_cast<float*>(workspace);
+    p.ws_ml = p.ws_acc ? p.ws_acc + (size_t)num_seqs * num_splits * num_q_heads * lg::kHeadDim
+                       : nullptr;
+    p.num_seqs = num_seqs;
+    p.hq = num_q_heads;
+    p.hkv = num_kv_heads;
+    p.block_size = block_size;
+    p.max_blocks_per_seq = max_blocks_per_seq;
+    p.num_splits = num_splits;
+    p.part_tokens = lg::part_tokens_for(block_size, max_blocks_per_seq, num_splits);
+    p.scale_log2e = scale * lg::kLog2e;
+    p.causal = causal;
+
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (num_q_heads / num_kv_heads) {
+        case 1: return lg::launch_group<1>(p, max_seqlen_q, phases, st);
+        case 2: return lg::launch_group<2>(p, max_seqlen_q, phases, st);
+        case 3: return lg::launch_group<3>(p, max_seqlen_q, phases, st);
+        case 4: return lg::launch_group<4>(p, max_seqlen_q, phases, st);
+        case 5: return lg::launch_group<5>(p, max_seqlen_q, phases, st);
+        case 6: return lg::launch_group<6>(p, max_seqlen_q, phases, st);
+        case 7: return lg::launch_group<7>(p, max_seqlen_q, phases, st);
+        case 8: return lg::launch_group<8>(p, max_seqlen_q, phases, st);
+        default: return hipErrorInvalidValue;
+    }
+}

@@ -1,0 +1,148 @@
+"""Python mirror of the reference's ``kernels::launch_*`` wrappers for the
+decode path (crates/kernels/src/matmul/mod.rs:140-186 is the template):
+host-side shape guard -> FFI call with raw device pointers, i32 dims and the
+raw stream -> non-zero status becomes ``LaunchError`` carrying the classified
+kind.  The library is loaded from ``logismos_amd/lib``; there is no fallback.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+from . import hip
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "liblogismos_kernels.so")
+
+_lib = None
+
+
+class NoGpuBuild(RuntimeError):
+    """`Error::NoGpuBuild` (crates/kernels/src/error.rs:55-63): the kernel archive is absent."""
+
+
+class UnsupportedShape(ValueError):
+    """`Error::UnsupportedShape` (crates/kernels/src/error.rs:44-53)."""
+
+    def __init__(self, kernel: str, msg: str):
+        self.kernel, self.msg = kernel, msg
+        super().__init__(f"kernel {kernel}: unsupported shape: {msg}")
+
+
+class LaunchError(RuntimeError):
+    """`Error::Launch` (crates/kernels/src/error.rs:27-42)."""
+
+    def __init__(self, kernel: str, code: int):
+        self.kernel, self.code, self.kind = kernel, int(code), hip.error_kind(code)
+        super().__init__(f"kernel {kernel}: launch failed: {self.kind} (code {self.code})")
+
+
+_vp, _i, _f, _sz = C.c_void_p, C.c_int, C.c_float, C.c_size_t
+
+_SIGNATURES = {
+    "logismos_decode_abi_version": (C.c_int, []),
+    "logismos_decode_offload_arch": (C.c_char_p, []),
+    "logismos_check_qgemv_q8g32_shape": (C.c_uint32, [_i, _i, C.c_char_p, _sz]),
+    "logismos_check_paged_attn_shape": (C.c_uint32, [_i] * 9 + [C.c_char_p, _sz]),
+    "logismos_launch_qgemv_q8g32_f32": (C.c_uint32, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
+    "logismos_launch_repack_q8_0": (C.c_uint32, [_vp, _vp, _vp, _i, _i, _vp]),
+    "logismos_paged_attn_num_splits": (C.c_int, [_i, _i, _i, _i]),
+    "logismos_paged_attn_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "logismos_launch_paged_attn_varlen_fp16":
+        (C.c_uint32, [_vp] * 8 + [_i] * 9 + [_f, _i, _vp]),
+    "logismos_launch_paged_attn_varlen_fp16_phases":
+        (C.c_uint32, [_vp] * 8 + [_i] * 9 + [_f, _i, _i, _vp]),
+}
+
+ATTN_PHASE_DECODE, ATTN_PHASE_PREFILL, ATTN_PHASE_MERGE, ATTN_PHASE_ALL = 1, 2, 4, 7
+
+
+def library() -> C.CDLL:
+    """Loads the C-ABI library; raises NoGpuBuild when it was never built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise NoGpuBuild(f"{LIB_PATH} is missing: run `python -m logismos_amd.build` "
+                             "(needs hipcc); there is no CPU fallback")
+        hip._runtime()
+        lib = C.CDLL(LIB_PATH)
+        for name, (restype, argtypes) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = restype, argtypes
+        _lib = lib
+    return _lib
+
+
+def exported_symbols() -> list[str]:
+    return sorted(_SIGNATURES)
+
+
+def _raw(stream) -> C.c_void_p | None:
+    return stream.raw if stream is not None else None
+
+
+def _ptr(x) -> C.c_void_p:
+    return x.ptr if isinstance(x, hip.DeviceBuffer) else x
+
+
+def _guard(kernel: str, check_fn, *dims) -> None:
+    msg = C.create_string_buffer(256)
+    if check_fn(*dims, msg, len(msg)) != 0:
+        raise UnsupportedShape(kernel, msg.value.decode())
+
+
+def _status(kernel: str, code: int) -> None:
+    if code != 0:
+        raise LaunchError(kernel, code)
+
+
+def check_qgemv_q8g32_shape(n: int, k: int) -> None:
+    _guard("qgemv_q8g32_f32", library().logismos_check_qgemv_q8g32_shape, n, k)
+
+
+def launch_qgemv_q8g32_f32(x, qs, d, y, n: int, k: int, stream=None) -> None:
+    check_qgemv_q8g32_shape(n, k)
+    _status("qgemv_q8g32_f32", library().logismos_launch_qgemv_q8g32_f32(
+        _ptr(x), _ptr(qs), _ptr(d), _ptr(y), n, k, _raw(stream)))
+
+
+def launch_repack_q8_0(blocks, qs, d, n: int, k: int, stream=None) -> None:
+    check_qgemv_q8g32_shape(n, k)
+    _status("repack_q8_0", library().logismos_launch_repack_q8_0(
+        _ptr(blocks), _ptr(qs), _ptr(d), n, k, _raw(stream)))
+
+
+def paged_attn_num_splits(num_seqs, num_kv_heads, block_size, max_blocks_per_seq) -> int:
+    return library().logismos_paged_attn_num_splits(num_seqs, num_kv_heads, block_size,
+                                                    max_blocks_per_seq)
+
+
+def paged_attn_workspace_bytes(num_seqs, num_q_heads, head_dim, num_splits) -> int:
+    return library().logismos_paged_attn_workspace_bytes(num_seqs, num_q_heads, head_dim,
+                                                         num_splits)
+
+
+def check_paged_attn_shape(num_seqs, total_tokens, max_seqlen_q, num_q_heads, num_kv_heads,
+                           head_dim, block_size, max_blocks_per_seq, num_splits) -> None:
+    _guard("paged_attn_varlen_fp16", library().logismos_check_paged_attn_shape, num_seqs,
+           total_tokens, max_seqlen_q, num_q_heads, num_kv_heads, head_dim, block_size,
+           max_blocks_per_seq, num_splits)
+
+
+def launch_paged_attn_varlen_fp16(q, k_pool, v_pool, block_tables, cu_seqlens_q, context_lens, out,
+                                  workspace, num_seqs, total_tokens, max_seqlen_q, num_q_heads,
+                                  num_kv_heads, head_dim, block_size, max_blocks_per_seq,
+                                  num_splits, scale, causal=True, stream=None,
+                                  phases=None) -> None:
+    check_paged_attn_shape(num_seqs, total_tokens, max_seqlen_q, num_q_heads, num_kv_heads,
+                           head_dim, block_size, max_blocks_per_seq, num_splits)
+    args = (_ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables), _ptr(cu_seqlens_q),
+            _ptr(context_lens), _ptr(out), _ptr(workspace) if workspace is not None else None,
+            num_seqs, total_tokens, max_seqlen_q, num_q_heads, num_kv_heads, head_dim, block_size,
+            max_blocks_per_seq, num_splits, float(scale), 1 if causal else 0)
+    if phases is None:
+        code = library().logismos_launch_paged_attn_varlen_fp16(*args, _raw(stream))
+    else:
+        code = library().logismos_launch_paged_attn_varlen_fp16_phases(*args, int(phases),
+                                                                       _raw(stream))
+    _status("paged_attn_varlen_fp16", code)

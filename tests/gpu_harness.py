@@ -1,0 +1,76 @@
+"""Host glue used by the GPU tests, smoke() and bench.py: uploads a case,
+calls the C-ABI launchers, downloads results."""
+from __future__ import annotations
+
+import numpy as np
+
+from logismos_amd import hip, kernels
+
+
+class PagedAttnRunner:
+    def __init__(self, case, num_splits=None, causal=True, stream=None):
+        self.case = case
+        self.stream = stream
+        self.causal = causal
+        c = case
+        self.num_seqs = len(c["context_lens"])
+        self.total_tokens = int(c["cu_seqlens"][-1])
+        self.max_seqlen_q = int(c["new_tokens"].max()) if self.num_seqs else 0
+        self.num_splits = num_splits or kernels.paged_attn_num_splits(
+            self.num_seqs, c["hkv"], c["block_size"], c["max_blocks"])
+        self.q = hip.DeviceBuffer.from_numpy(c["q"])
+        self.k_pool = hip.DeviceBuffer.from_numpy(c["k_pool"])
+        self.v_pool = hip.DeviceBuffer.from_numpy(c["v_pool"])
+        self.bt = hip.DeviceBuffer.from_numpy(c["block_tables"])
+        self.cu = hip.DeviceBuffer.from_numpy(c["cu_seqlens"])
+        self.ctx = hip.DeviceBuffer.from_numpy(c["context_lens"])
+        self.out = hip.DeviceBuffer(max(c["q"].nbytes, 16))
+        self.out.fill(0xFF)  # NaN pattern: unwritten outputs are caught
+        ws = kernels.paged_attn_workspace_bytes(self.num_seqs, c["hq"], c["d"], self.num_splits)
+        self.ws = hip.DeviceBuffer(max(ws, 16))
+        self.ws.fill(0xFF)
+
+    def launch(self, phases=None, k_pool=None, v_pool=None):
+        c = self.case
+        kernels.launch_paged_attn_varlen_fp16(
+            self.q, k_pool or self.k_pool, v_pool or self.v_pool, self.bt, self.cu, self.ctx,
+            self.out, self.ws, self.num_seqs, self.total_tokens, self.max_seqlen_q, c["hq"],
+            c["hkv"], c["d"], c["block_size"], c["max_blocks"], self.num_splits, c["scale"],
+            self.causal, self.stream, phases)
+
+    def result(self) -> np.ndarray:
+        (self.stream.synchronize() if self.stream else hip.synchronize())
+        return self.out.to_numpy(np.float16, self.case["q"].shape)
+
+
+class QgemvQ8Runner:
+    def __init__(self, x, qs, d, n, k, stream=None):
+        self.n, self.k, self.stream = n, k, stream
+        self.x = hip.DeviceBuffer.from_numpy(np.ascontiguousarray(x, np.float32))
+        self.qs = hip.DeviceBuffer.from_numpy(np.ascontiguousarray(qs, np.int8))
+        self.d = hip.DeviceBuffer.from_numpy(np.ascontiguousarray(d).view(np.uint16))
+        self.y = hip.DeviceBuffer(n * 4)
+        self.y.fill(0xFF)
+
+    def launch(self):
+        kernels.launch_qgemv_q8g32_f32(self.x, self.qs, self.d, self.y, self.n, self.k, self.stream)
+
+    def result(self) -> np.ndarray:
+        (self.stream.synchronize() if self.stream else hip.synchronize())
+        return self.y.to_numpy(np.float32, (self.n,))
+
+
+def assert_parity(got, want, max_abs=2e-3, max_rel=1e-2, what=""):
+    """Tolerance of the decode path for fp16/bf16 outputs with fp32 accumulation:
+    every element within max_abs OR within max_rel of the oracle (relative error
+    with the reference's denominator floor, crates/kernels/tests/matmul_parity.rs:83-99)."""
+    got = np.asarray(got, np.float32)
+    want = np.asarray(want, np.float32)
+    assert got.shape == want.shape, (got.shape, want.shape)
+    assert np.isfinite(got).all(), f"{what}: non-finite output"
+    err = np.abs(got - want)
+    rel = err / np.maximum(np.abs(want), 1e-3)
+    bad = (err > max_abs) & (rel > max_rel)
+    assert not bad.any(), (f"{what}: {int(bad.sum())} elements out of tolerance; "
+                           f"max_abs={err.max():.3e} max_rel={rel.max():.3e}")
+    return float(err.max()), float(rel.max())

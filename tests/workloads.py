@@ -1,0 +1,70 @@
+"""Seeded synthetic inputs shared by the parity tests, smoke() and bench.py.
+
+Everything is generated on the host with numpy's PCG64 (same numpy on every
+box of this image), then uploaded: the oracle and the GPU see identical bytes.
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+
+SEED = 0x10615
+
+
+def paged_case(rng, new_tokens, prior_ctx, hq, hkv, d=128, block_size=16, spare_frac=0.25,
+               kv_std=1.0):
+    """Ragged paged-attention inputs: pools shared by all sequences, physical
+    block ids a random permutation, block-table tail entries poisoned."""
+    new = np.asarray(new_tokens, np.int32)
+    prior = np.asarray(prior_ctx, np.int32)
+    ctx = (new + prior).astype(np.int32)
+    nblk = [(int(c) + block_size - 1) // block_size for c in ctx]
+    total_blocks = sum(nblk) + max(1, int(sum(nblk) * spare_frac))
+    perm = rng.permutation(total_blocks).astype(np.int32)
+    max_blocks = max(max(nblk), 1)
+    bt = np.full((len(new), max_blocks), 0x3FFFFFF, np.int32)
+    o = 0
+    for s, nb in enumerate(nblk):
+        bt[s, :nb] = perm[o:o + nb]
+        o += nb
+    rows = total_blocks * block_size
+    k_pool = (rng.standard_normal((rows, hkv * d), np.float32) * kv_std).astype(np.float16)
+    v_pool = (rng.standard_normal((rows, hkv * d), np.float32) * kv_std).astype(np.float16)
+    cu = np.concatenate([[0], np.cumsum(new)]).astype(np.int32)
+    q = rng.standard_normal((int(cu[-1]), hq, d), np.float32).astype(np.float16)
+    return dict(q=q, k_pool=k_pool, v_pool=v_pool, block_tables=bt, cu_seqlens=cu,
+                context_lens=ctx, new_tokens=new, prior_ctx=prior, hq=hq, hkv=hkv, d=d,
+                block_size=block_size, max_blocks=max_blocks, scale=1.0 / math.sqrt(d))
+
+
+def config2(seed=SEED + 1):
+    """Ragged paged decode, Qwen2-1.5B geometry: 16 sequences, ctx ~ U{64..2048},
+    12 query / 2 KV heads, head_dim 128, block 16, one query token each."""
+    rng = np.random.default_rng(seed)
+    ctx = rng.integers(64, 2049, size=16)
+    return paged_case(rng, np.ones(16, np.int32), ctx - 1, hq=12, hkv=2)
+
+
+def config1(seed=SEED):
+    """Q8G32 GEMV, Qwen2-1.5B MLP up-proj: x 1x1536 ~N(0,1), W 8960x1536 ~N(0,0.02)."""
+    rng = np.random.default_rng(seed)
+    n, k = 8960, 1536
+    x = rng.standard_normal(k, np.float32)
+    w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
+    return dict(x=x, w=w, n=n, k=k)
+
+
+def paged_attn_algorithmic_bytes(case) -> int:
+    """K and V rows read once per sequence, q and out, block-table entries read,
+    cu_seqlens and context_lens."""
+    ctx = case["context_lens"].astype(np.int64)
+    row_bytes = case["hkv"] * case["d"] * 2
+    kv = int(ctx.sum()) * 2 * row_bytes
+    qo = 2 * case["q"].size * 2
+    bt = 4 * int(((ctx + case["block_size"] - 1) // case["block_size"]).sum())
+    return kv + qo + bt + 4 * (2 * len(ctx) + 1)
+
+
+def qgemv_q8_algorithmic_bytes(n, k) -> int:
+    return n * k + n * (k // 32) * 2 + 4 * k + 4 * n
