@@ -199,6 +199,18 @@ logismos_status_t logismos_launch_paged_attn_varlen_fp16_phases(
     int head_dim, int block_size, int max_blocks_per_seq, int num_splits, float scale, int causal,
     int phases, logismos_stream_t stream);
 
+/* ------------------------------------------------------------------------
+ * Memory-system probes (measurement aids; the reference has no counterpart,
+ * its only timing helper is the hipEvent pair of
+ * crates/kernels/examples/gemm_bench.rs:120-128).  A plain copy and a plain
+ * read of `bytes` bytes (multiple of 16, 16-byte aligned): the achievable HBM
+ * ceiling of the box, and the calibration for FETCH_SIZE / WRITE_SIZE.
+ * ------------------------------------------------------------------------ */
+logismos_status_t logismos_launch_probe_copy(const void* src, void* dst, size_t bytes,
+                                             logismos_stream_t stream);
+logismos_status_t logismos_launch_probe_read(const void* src, void* sink_u32, size_t bytes,
+                                             logismos_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

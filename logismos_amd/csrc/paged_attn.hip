@@ -73,11 +73,20 @@ struct AttnParams {
 //                 of the sequences with more than one new token, whole visible
 //                 context in one partition.
 template <int G, bool DECODE>
-__global__ __launch_bounds__(64) void paged_attn_kernel(const AttnParams p) {
-    const int lane = threadIdx.x;
+#ifdef LG_EXP_WGH
+__global__ __launch_bounds__(64 * LG_EXP_WGH) void paged_attn_kernel
+#else
+__global__ __launch_bounds__(64) void paged_attn_kernel
+#endif
+(const AttnParams p) {
+    const int lane = threadIdx.x & 63;
     const int tg = lane >> 4;
     const int c = lane & 15;
+#ifdef LG_EXP_WGH
+    const int kvh = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);
+#else
     const int kvh = blockIdx.y;
+#endif
     const int s = blockIdx.z;
 
     const int t0 = p.cu_seqlens_q[s];
@@ -148,9 +157,17 @@ __global__ __launch_bounds__(64) void paged_attn_kernel(const AttnParams p) {
         // keys past the end of the partition re-read its last key (their
         // probability is forced to zero below); never touches another block
         const unsigned last_off = (unsigned)(tok_end - 1 - tok_base) * row_stride;
+#ifdef LG_EXP_KCOAL
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const unsigned vo = min(v_lane_off[i], last_off) + 8u * c;
+            kv.k[i] = *reinterpret_cast<const half8_t*>(kb + vo);
+        }
+#else
         const unsigned ko = min(k_lane_off, last_off) + 8u * tg;
 #pragma unroll
         for (int j = 0; j < 4; ++j) kv.k[j] = *reinterpret_cast<const half8_t*>(kb + ko + 32 * j);
+#endif
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const unsigned vo = min(v_lane_off[i], last_off) + 8u * c;
@@ -214,8 +231,27 @@ __global__ __launch_bounds__(64) void paged_attn_kernel(const AttnParams p) {
     // a tile past the end re-reads the last one and is fully masked in
     // compute_tile), so the loads of the next tile stay in flight while the
     // current one is consumed and the wait counts stay exact.
-    KvTile buf0, buf1;
     const int last_tile = ntiles - 1;
+#ifdef LG_EXP_PF2
+    KvTile bufa, bufb, bufc;
+    load_tile(0, bufa);
+    load_tile(min(1, last_tile), bufb);
+    for (int tile = 0; tile < ntiles; tile += 3) {
+        load_tile(min(tile + 2, last_tile), bufc);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_tile(tile, bufa);
+        __builtin_amdgcn_sched_barrier(0);
+        load_tile(min(tile + 3, last_tile), bufa);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_tile(tile + 1, bufb);
+        __builtin_amdgcn_sched_barrier(0);
+        load_tile(min(tile + 4, last_tile), bufb);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_tile(tile + 2, bufc);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+#else
+    KvTile buf0, buf1;
     load_tile(0, buf0);
     for (int tile = 0; tile < ntiles; tile += 2) {
         load_tile(min(tile + 1, last_tile), buf1);
@@ -227,6 +263,7 @@ __global__ __launch_bounds__(64) void paged_attn_kernel(const AttnParams p) {
         compute_tile(tile + 1, buf1);
         __builtin_amdgcn_sched_barrier(0);
     }
+#endif
 
     // ---- merge the four rows of the wave, then write
     static_for<G>([&](auto hc) {
@@ -273,27 +310,74 @@ __global__ __launch_bounds__(64) void paged_attn_kernel(const AttnParams p) {
 }
 
 // Combines the partials of the decode sequences that used more than one
-// partition.  grid (hq, num_seqs), 128 threads = one per output element.
-__global__ __launch_bounds__(128) void paged_attn_merge_kernel(const AttnParams p) {
+// partition.  grid (hq, num_seqs), 256 threads: wave w folds partitions
+// w, w+4, ... (four independent partials in flight per round, two output
+// elements per lane), then the four waves are folded through LDS.
+__global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams p) {
     const int s = blockIdx.y;
     const int h = blockIdx.x;
-    const int d = threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int w = threadIdx.x >> 6;
     const int t0 = p.cu_seqlens_q[s];
     if (p.cu_seqlens_q[s + 1] - t0 != 1) return;
     const int ctx = p.context_lens[s];
     const int np = (ctx + p.part_tokens - 1) / p.part_tokens;
     if (np <= 1) return;
     const int64_t base = ((int64_t)s * p.num_splits) * p.hq + h;
-    float mmax = -INFINITY;
-    for (int i = 0; i < np; ++i) mmax = fmaxf(mmax, p.ws_ml[(base + (int64_t)i * p.hq) * 2]);
-    float num = 0.0f, den = 0.0f;
-    for (int i = 0; i < np; ++i) {
-        const int64_t idx = base + (int64_t)i * p.hq;
-        const float f = fast_exp2(p.ws_ml[idx * 2] - mmax);
-        den = fmaf(f, p.ws_ml[idx * 2 + 1], den);
-        num = fmaf(f, p.ws_acc[idx * kHeadDim + d], num);
+
+    float M = -INFINITY, den = 0.0f, n0 = 0.0f, n1 = 0.0f;
+    for (int i0 = w; i0 < np; i0 += 16) {
+        float mj[4], lj[4], a0[4], a1[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = i0 + 4 * j;
+            const bool valid = i < np;
+            const int64_t idx = base + (int64_t)(valid ? i : i0) * p.hq;
+            const float mv = p.ws_ml[idx * 2];
+            const float lv = p.ws_ml[idx * 2 + 1];
+            const float* a = p.ws_acc + idx * kHeadDim + 2 * lane;
+            const float av0 = a[0], av1 = a[1];
+            mj[j] = valid ? mv : -INFINITY;
+            lj[j] = valid ? lv : 0.0f;
+            a0[j] = valid ? av0 : 0.0f;
+            a1[j] = valid ? av1 : 0.0f;
+        }
+        float mx = M;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) mx = fmaxf(mx, mj[j]);
+        const float f = fast_exp2(M - mx);  // partition 0 of the round is valid: mx is finite
+        den *= f;
+        n0 *= f;
+        n1 *= f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float g = fast_exp2(mj[j] - mx);
+            den = fmaf(g, lj[j], den);
+            n0 = fmaf(g, a0[j], n0);
+            n1 = fmaf(g, a1[j], n1);
+        }
+        M = mx;
     }
-    p.out[((int64_t)t0 * p.hq + h) * kHeadDim + d] = (_Float16)(num / den);
+    __shared__ float sm[4], sden[4], sn[4][kHeadDim];
+    if (lane == 0) {
+        sm[w] = M;
+        sden[w] = den;
+    }
+    sn[w][2 * lane] = n0;
+    sn[w][2 * lane + 1] = n1;
+    __syncthreads();
+    if (threadIdx.x < kHeadDim) {
+        const int d = threadIdx.x;
+        float mx = fmaxf(fmaxf(sm[0], sm[1]), fmaxf(sm[2], sm[3]));
+        float num = 0.0f, dd = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float g = fast_exp2(sm[j] - mx);  // a wave without partitions has m = -inf: g = 0
+            dd = fmaf(g, sden[j], dd);
+            num = fmaf(g, sn[j][d], num);
+        }
+        p.out[((int64_t)t0 * p.hq + h) * kHeadDim + d] = (_Float16)(num / dd);
+    }
 }
 
 static int part_tokens_for(int block_size, int max_blocks_per_seq, int num_splits) {
@@ -308,8 +392,14 @@ static hipError_t launch_group(const AttnParams& p, int max_seqlen_q, int phases
                                hipStream_t stream) {
     dim3 block(64);
     if (phases & LOGISMOS_ATTN_PHASE_DECODE) {
+#ifdef LG_EXP_WGH
+        const int wpb = (p.hkv % LG_EXP_WGH == 0) ? LG_EXP_WGH : 1;
+        dim3 grid_d(p.num_splits, p.hkv / wpb, p.num_seqs);
+        paged_attn_kernel<G, true><<<grid_d, dim3(64 * wpb), 0, stream>>>(p);
+#else
         dim3 grid_d(p.num_splits, p.hkv, p.num_seqs);
         paged_attn_kernel<G, true><<<grid_d, block, 0, stream>>>(p);
+#endif
     }
     if ((phases & LOGISMOS_ATTN_PHASE_PREFILL) && max_seqlen_q > 1) {
         dim3 grid_p(max_seqlen_q, p.hkv, p.num_seqs);
@@ -317,7 +407,7 @@ static hipError_t launch_group(const AttnParams& p, int max_seqlen_q, int phases
     }
     if ((phases & LOGISMOS_ATTN_PHASE_MERGE) && p.num_splits > 1) {
         dim3 grid_m(p.hq, p.num_seqs);
-        paged_attn_merge_kernel<<<grid_m, dim3(128), 0, stream>>>(p);
+        paged_attn_merge_kernel<<<grid_m, dim3(256), 0, stream>>>(p);
     }
     return hipGetLastError();
 }

@@ -12,7 +12,9 @@ import os
 from . import hip
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "liblogismos_kernels.so")
+# LOGISMOS_KERNELS_LIB points at an alternative build of the same ABI.
+LIB_PATH = os.environ.get("LOGISMOS_KERNELS_LIB") or os.path.join(_HERE, "lib",
+                                                                 "liblogismos_kernels.so")
 
 _lib = None
 
@@ -52,6 +54,8 @@ _SIGNATURES = {
         (C.c_uint32, [_vp] * 8 + [_i] * 9 + [_f, _i, _vp]),
     "logismos_launch_paged_attn_varlen_fp16_phases":
         (C.c_uint32, [_vp] * 8 + [_i] * 9 + [_f, _i, _i, _vp]),
+    "logismos_launch_probe_copy": (C.c_uint32, [_vp, _vp, _sz, _vp]),
+    "logismos_launch_probe_read": (C.c_uint32, [_vp, _vp, _sz, _vp]),
 }
 
 ATTN_PHASE_DECODE, ATTN_PHASE_PREFILL, ATTN_PHASE_MERGE, ATTN_PHASE_ALL = 1, 2, 4, 7
@@ -146,3 +150,13 @@ def launch_paged_attn_varlen_fp16(q, k_pool, v_pool, block_tables, cu_seqlens_q,
         code = library().logismos_launch_paged_attn_varlen_fp16_phases(*args, int(phases),
                                                                        _raw(stream))
     _status("paged_attn_varlen_fp16", code)
+
+
+def launch_probe_copy(src, dst, nbytes: int, stream=None) -> None:
+    _status("probe_copy", library().logismos_launch_probe_copy(_ptr(src), _ptr(dst), nbytes,
+                                                               _raw(stream)))
+
+
+def launch_probe_read(src, sink, nbytes: int, stream=None) -> None:
+    _status("probe_read", library().logismos_launch_probe_read(_ptr(src), _ptr(sink), nbytes,
+                                                               _raw(stream)))

@@ -68,3 +68,11 @@ def paged_attn_algorithmic_bytes(case) -> int:
 
 def qgemv_q8_algorithmic_bytes(n, k) -> int:
     return n * k + n * (k // 32) * 2 + 4 * k + 4 * n
+
+
+def config5_attention(seed=SEED + 5, num_seqs=32, lo=256, hi=8192):
+    """One layer's attention of the Qwen3-8B-geometry decode step: 32 live sequences,
+    ctx ~ U{256..8192}, 32 query / 8 KV heads, head_dim 128, block 16."""
+    rng = np.random.default_rng(seed)
+    ctx = rng.integers(lo, hi + 1, size=num_seqs)
+    return paged_case(rng, np.ones(num_seqs, np.int32), ctx - 1, hq=32, hkv=8, spare_frac=0.05)
