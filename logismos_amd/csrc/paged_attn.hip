@@ -39,6 +39,7 @@ namespace lg {
 
 constexpr int kHeadDim = 128;
 constexpr int kTileKeys = 16;
+constexpr int kMaxHeadWaves = 8;  // waves (KV heads) per workgroup
 constexpr float kLog2e = 1.4426950408889634f;
 
 struct KvTile {
@@ -67,26 +68,19 @@ struct AttnParams {
     int causal;
 };
 
-// DECODE = true : grid (num_splits, hkv, num_seqs); sequences with exactly one
-//                 new token, keys split into partitions of part_tokens.
-// DECODE = false: grid (max_seqlen_q, hkv, num_seqs); one wave per query token
+// DECODE = true : grid (num_splits, hkv / waves, num_seqs); sequences with exactly
+//                 one new token, keys split into partitions of part_tokens.
+// DECODE = false: grid (max_seqlen_q, hkv / waves, num_seqs); one wave per query token
 //                 of the sequences with more than one new token, whole visible
 //                 context in one partition.
 template <int G, bool DECODE>
-#ifdef LG_EXP_WGH
-__global__ __launch_bounds__(64 * LG_EXP_WGH) void paged_attn_kernel
-#else
-__global__ __launch_bounds__(64) void paged_attn_kernel
-#endif
-(const AttnParams p) {
+__global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_kernel(const AttnParams p) {
     const int lane = threadIdx.x & 63;
     const int tg = lane >> 4;
     const int c = lane & 15;
-#ifdef LG_EXP_WGH
+    // the waves of a workgroup are consecutive KV heads of the same keys: together
+    // they stream whole token rows (hkv * 256 contiguous bytes)
     const int kvh = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);
-#else
-    const int kvh = blockIdx.y;
-#endif
     const int s = blockIdx.z;
 
     const int t0 = p.cu_seqlens_q[s];
@@ -157,17 +151,9 @@ __global__ __launch_bounds__(64) void paged_attn_kernel
         // keys past the end of the partition re-read its last key (their
         // probability is forced to zero below); never touches another block
         const unsigned last_off = (unsigned)(tok_end - 1 - tok_base) * row_stride;
-#ifdef LG_EXP_KCOAL
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const unsigned vo = min(v_lane_off[i], last_off) + 8u * c;
-            kv.k[i] = *reinterpret_cast<const half8_t*>(kb + vo);
-        }
-#else
         const unsigned ko = min(k_lane_off, last_off) + 8u * tg;
 #pragma unroll
         for (int j = 0; j < 4; ++j) kv.k[j] = *reinterpret_cast<const half8_t*>(kb + ko + 32 * j);
-#endif
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const unsigned vo = min(v_lane_off[i], last_off) + 8u * c;
@@ -232,25 +218,6 @@ __global__ __launch_bounds__(64) void paged_attn_kernel
     // compute_tile), so the loads of the next tile stay in flight while the
     // current one is consumed and the wait counts stay exact.
     const int last_tile = ntiles - 1;
-#ifdef LG_EXP_PF2
-    KvTile bufa, bufb, bufc;
-    load_tile(0, bufa);
-    load_tile(min(1, last_tile), bufb);
-    for (int tile = 0; tile < ntiles; tile += 3) {
-        load_tile(min(tile + 2, last_tile), bufc);
-        __builtin_amdgcn_sched_barrier(0);
-        compute_tile(tile, bufa);
-        __builtin_amdgcn_sched_barrier(0);
-        load_tile(min(tile + 3, last_tile), bufa);
-        __builtin_amdgcn_sched_barrier(0);
-        compute_tile(tile + 1, bufb);
-        __builtin_amdgcn_sched_barrier(0);
-        load_tile(min(tile + 4, last_tile), bufb);
-        __builtin_amdgcn_sched_barrier(0);
-        compute_tile(tile + 2, bufc);
-        __builtin_amdgcn_sched_barrier(0);
-    }
-#else
     KvTile buf0, buf1;
     load_tile(0, buf0);
     for (int tile = 0; tile < ntiles; tile += 2) {
@@ -263,7 +230,6 @@ __global__ __launch_bounds__(64) void paged_attn_kernel
         compute_tile(tile + 1, buf1);
         __builtin_amdgcn_sched_barrier(0);
     }
-#endif
 
     // ---- merge the four rows of the wave, then write
     static_for<G>([&](auto hc) {
@@ -390,19 +356,20 @@ static int part_tokens_for(int block_size, int max_blocks_per_seq, int num_split
 template <int G>
 static hipError_t launch_group(const AttnParams& p, int max_seqlen_q, int phases,
                                hipStream_t stream) {
-    dim3 block(64);
+    // waves per workgroup: the largest divisor of hkv that is <= kMaxHeadWaves
+    int wpb = 1;
+    for (int w = kMaxHeadWaves; w > 1; --w)
+        if (p.hkv % w == 0) {
+            wpb = w;
+            break;
+        }
+    dim3 block(64 * wpb);
     if (phases & LOGISMOS_ATTN_PHASE_DECODE) {
-#ifdef LG_EXP_WGH
-        const int wpb = (p.hkv % LG_EXP_WGH == 0) ? LG_EXP_WGH : 1;
         dim3 grid_d(p.num_splits, p.hkv / wpb, p.num_seqs);
-        paged_attn_kernel<G, true><<<grid_d, dim3(64 * wpb), 0, stream>>>(p);
-#else
-        dim3 grid_d(p.num_splits, p.hkv, p.num_seqs);
         paged_attn_kernel<G, true><<<grid_d, block, 0, stream>>>(p);
-#endif
     }
     if ((phases & LOGISMOS_ATTN_PHASE_PREFILL) && max_seqlen_q > 1) {
-        dim3 grid_p(max_seqlen_q, p.hkv, p.num_seqs);
+        dim3 grid_p(max_seqlen_q, p.hkv / wpb, p.num_seqs);
         paged_attn_kernel<G, false><<<grid_p, block, 0, stream>>>(p);
     }
     if ((phases & LOGISMOS_ATTN_PHASE_MERGE) && p.num_splits > 1) {

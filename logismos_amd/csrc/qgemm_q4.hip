@@ -1,0 +1,258 @@
+// Q4G128 dequant-fused row-GEMV / GEMM for gfx950:
+//   y[b][n] = bf16( sum_k x[b][k] * (q[n][k] - zero[n][k/128]) * scale[n][k/128] )
+//
+// Nibbles are never converted one by one.  OR-ing a nibble into the mantissa
+// of the bf16 constant 128.0 (0x4300) yields the bf16 number 128 + q exactly,
+// two per 32-bit register:  ((w >> 4s) & 0x000F000F) | 0x43004300  holds
+// elements s and s+4 of the 8 nibbles of w.  Both kernels contract these
+// "128 + q" values against x and remove the offset per group:
+//   sum_k x_k (q_k - z) s  =  s * ( sum_k x_k (128 + q_k)  -  (128 + z) * sum_k x_k ).
+// x is staged once per workgroup in LDS, already permuted to the (s, s+4)
+// pair order, next to the per-chunk / per-group sums of x.
+//
+// Batch <= 4 (bandwidth-bound GEMV): VALU path.  One wave owns R rows; a lane
+// reads 16 bytes (32 nibbles) of each row per step, unpacks them once and
+// feeds v_dot2_f32_bf16 for every batch row.
+//
+// Batch >= 5: MFMA path (see qgemm_q4g128_mfma_kernel below).
+//
+// Algorithmic bytes per call: n*k/2 (nibbles) + n*(k/128)*4 (scale, zero)
+// + b*k*2 (x) + b*n*2 (y).
+#include "device_utils.hpp"
+#include "launch_common.hpp"
+
+#include <hip/hip_fp16.h>
+
+namespace lg {
+
+__device__ __forceinline__ float bf16_lo_to_f32(unsigned v) { return __uint_as_float(v << 16); }
+__device__ __forceinline__ float bf16_hi_to_f32(unsigned v) {
+    return __uint_as_float(v & 0xffff0000u);
+}
+__device__ __forceinline__ unsigned short f32_to_bf16_rne(float f) {
+    unsigned u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (unsigned short)(u >> 16);
+}
+__device__ __forceinline__ float dot2_bf16(unsigned a, unsigned b, float c) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a),
+                                           __builtin_bit_cast(bf16x2_t, b), c, false);
+}
+
+// 8 consecutive bf16 (x0..x7 in four dwords) -> pairs (x0,x4) (x1,x5) (x2,x6) (x3,x7)
+__device__ __forceinline__ uint4_t pair_order(uint4_t d) {
+    uint4_t o;
+    o[0] = (d[0] & 0xffffu) | (d[2] << 16);
+    o[1] = (d[0] >> 16) | (d[2] & 0xffff0000u);
+    o[2] = (d[1] & 0xffffu) | (d[3] << 16);
+    o[3] = (d[1] >> 16) | (d[3] & 0xffff0000u);
+    return o;
+}
+__device__ __forceinline__ float sum8_bf16(uint4_t d) {
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s += bf16_lo_to_f32(d[i]) + bf16_hi_to_f32(d[i]);
+    return s;
+}
+
+constexpr unsigned kNibMask = 0x000F000Fu;
+constexpr unsigned kBf16Magic = 0x43004300u;  // (128.0, 128.0)
+
+// ---------------------------------------------------------------------------
+// VALU path, batch B <= 4.  grid = ceil(n / (4*R)), block = 256 (4 waves).
+// LDS: xp [B][4][nchunks] uint4 (x in pair order, piece-major so that a wave
+// reads consecutive 16-byte words) and xs [B][nchunks] float (sum of x over
+// the 32 elements of a chunk).
+// ---------------------------------------------------------------------------
+template <int B, int R>
+__global__ __launch_bounds__(256) void qgemv_q4g128_kernel(const uint16_t* __restrict__ x,
+                                                           const uint8_t* __restrict__ qw,
+                                                           const __half* __restrict__ scale,
+                                                           const __half* __restrict__ zero,
+                                                           uint16_t* __restrict__ y, int n, int k) {
+    extern __shared__ uint4_t lds[];
+    const int nchunks = k >> 5;  // 32 elements = 16 bytes of nibbles
+    const int groups = k >> 7;
+    uint4_t* xp = lds;
+    float* xs = reinterpret_cast<float*>(lds + (size_t)B * 4 * nchunks);
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * R;
+    const int64_t row_bytes = k >> 1;
+
+    // first step's weights go in flight before x is staged
+    uint4_t w_next[R];
+    {
+        const int c = lane < nchunks ? lane : nchunks - 1;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int64_t row = (row0 + r < n) ? (row0 + r) : (int64_t)(n - 1);
+            w_next[r] = *reinterpret_cast<const uint4_t*>(qw + row * row_bytes + (int64_t)c * 16);
+        }
+    }
+
+    for (int idx = threadIdx.x; idx < B * nchunks; idx += 256) {
+        const int b = idx / nchunks, c = idx - b * nchunks;
+        const uint4_t* src = reinterpret_cast<const uint4_t*>(x + (int64_t)b * k + (int64_t)c * 32);
+        float s = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint4_t d = src[j];
+            s += sum8_bf16(d);
+            xp[((size_t)b * 4 + j) * nchunks + c] = pair_order(d);
+        }
+        xs[b * nchunks + c] = s;
+    }
+    __syncthreads();
+    if (row0 >= n) return;
+
+    float acc[R][B];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int b = 0; b < B; ++b) acc[r][b] = 0.0f;
+
+    // The magic constant lives in a VGPR the optimiser cannot see through, so
+    // that (w & mask) | magic is one v_and_or_b32 (a VOP3 takes no literal and
+    // at most one scalar operand on this target).
+    unsigned magic;
+    asm volatile("v_mov_b32 %0, 0x43004300" : "=v"(magic));
+
+    for (int c0 = 0; c0 < nchunks; c0 += kWave) {
+        const int c = c0 + lane;
+        const bool live = c < nchunks;
+        const int cc = live ? c : nchunks - 1;
+        uint4_t w[R];
+        __half sc[R], zr[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int64_t row = (row0 + r < n) ? (row0 + r) : (int64_t)(n - 1);
+            w[r] = w_next[r];
+            sc[r] = scale[row * groups + (cc >> 2)];
+            zr[r] = zero[row * groups + (cc >> 2)];
+        }
+        {   // next step's weights (clamped: the last step re-reads its own chunk)
+            const int cn = (c0 + kWave + lane) < nchunks ? (c0 + kWave + lane) : cc;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int64_t row = (row0 + r < n) ? (row0 + r) : (int64_t)(n - 1);
+                w_next[r] =
+                    *reinterpret_cast<const uint4_t*>(qw + row * row_bytes + (int64_t)cn * 16);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+
+        float raw[R][B];
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int b = 0; b < B; ++b) raw[r][b] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            uint4_t xv[B];
+#pragma unroll
+            for (int b = 0; b < B; ++b) xv[b] = xp[((size_t)b * 4 + j) * nchunks + cc];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const unsigned wd = w[r][j];
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const unsigned h = ((wd >> (4 * s)) & kNibMask) | magic;
+#pragma unroll
+                    for (int b = 0; b < B; ++b) raw[r][b] = dot2_bf16(h, xv[b][s], raw[r][b]);
+                }
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+            const float xsum = live ? xs[b * nchunks + cc] : 0.0f;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const float sf = live ? __half2float(sc[r]) : 0.0f;
+                const float off = 128.0f + __half2float(zr[r]);
+                acc[r][b] = fmaf(sf, fmaf(-off, xsum, raw[r][b]), acc[r][b]);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+            const float total = wave_sum(acc[r][b]);
+            if (lane == 0 && row0 + r < n) y[(int64_t)b * n + row0 + r] = f32_to_bf16_rne(total);
+        }
+}
+
+template <int B, int R>
+static hipError_t launch_gemv(const void* x, const void* qw, const void* scale, const void* zero,
+                              void* y, int n, int k, hipStream_t stream) {
+    const int nchunks = k / 32;
+    const size_t lds = (size_t)B * nchunks * (4 * 16 + 4);
+    auto kern = qgemv_q4g128_kernel<B, R>;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+    }
+    const int rows_per_block = 4 * R;
+    dim3 grid((n + rows_per_block - 1) / rows_per_block), block(256);
+    kern<<<grid, block, lds, stream>>>(static_cast<const uint16_t*>(x),
+                                       static_cast<const uint8_t*>(qw),
+                                       static_cast<const __half*>(scale),
+                                       static_cast<const __half*>(zero),
+                                       static_cast<uint16_t*>(y), n, k);
+    return hipGetLastError();
+}
+
+template <int B>
+static hipError_t launch_gemv_b(const void* x, const void* qw, const void* scale, const void* zero,
+                                void* y, int n, int k, hipStream_t stream) {
+    // rows per wave: enough waves to cover the chip several times over
+    if (n >= 8192) return launch_gemv<B, 4>(x, qw, scale, zero, y, n, k, stream);
+    if (n >= 4096) return launch_gemv<B, 2>(x, qw, scale, zero, y, n, k, stream);
+    return launch_gemv<B, 1>(x, qw, scale, zero, y, n, k, stream);
+}
+
+constexpr size_t kMaxLds = 160 * 1024;
+
+}  // namespace lg
+
+extern "C" logismos_status_t logismos_check_qgemm_q4g128_shape(int b, int n, int k, char* msg,
+                                                               size_t msg_cap) {
+    const char* kn = "qgemm_q4g128_bf16";
+    if (b <= 0) return lg::reject(msg, msg_cap, "%s: batch must be positive, got %d", kn, b);
+    if (n <= 0) return lg::reject(msg, msg_cap, "%s: N must be positive, got %d", kn, n);
+    if (k <= 0) return lg::reject(msg, msg_cap, "%s: K must be positive, got %d", kn, k);
+    if (k % 128 != 0)
+        return lg::reject(msg, msg_cap, "%s: K = %d is not a multiple of the group size 128", kn, k);
+    if (b > 4)
+        return lg::reject(msg, msg_cap, "%s: batch %d exceeds the supported maximum of 4", kn, b);
+    if ((int64_t)n * k > (int64_t)INT32_MAX)
+        return lg::reject(msg, msg_cap, "%s: N*K = %lld exceeds i32::MAX", kn,
+                          (long long)((int64_t)n * k));
+    if ((int64_t)b * n > (int64_t)INT32_MAX || (int64_t)b * k > (int64_t)INT32_MAX)
+        return lg::reject(msg, msg_cap, "%s: batch*N or batch*K exceeds i32::MAX", kn);
+    if ((size_t)b * (k / 32) * 68 > lg::kMaxLds)
+        return lg::reject(msg, msg_cap, "%s: batch*K = %lld does not fit the LDS staging of x", kn,
+                          (long long)((int64_t)b * k));
+    return 0;
+}
+
+extern "C" logismos_status_t logismos_launch_qgemm_q4g128_bf16(
+    const void* x_bf16, const void* qw_u8, const void* scale_f16, const void* zero_f16,
+    void* y_bf16, int b, int n, int k, logismos_stream_t stream) {
+    if (logismos_check_qgemm_q4g128_shape(b, n, k, nullptr, 0) != 0) return hipErrorInvalidValue;
+    if (!x_bf16 || !qw_u8 || !scale_f16 || !zero_f16 || !y_bf16) return hipErrorInvalidValue;
+    if ((reinterpret_cast<uintptr_t>(qw_u8) & 15u) || (reinterpret_cast<uintptr_t>(x_bf16) & 15u))
+        return hipErrorInvalidValue;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (b) {
+        case 1: return lg::launch_gemv_b<1>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, n, k, st);
+        case 2: return lg::launch_gemv_b<2>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, n, k, st);
+        case 3: return lg::launch_gemv_b<3>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, n, k, st);
+        case 4: return lg::launch_gemv_b<4>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, n, k, st);
+        default: return hipErrorInvalidValue;
+    }
+}

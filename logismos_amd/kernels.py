@@ -47,6 +47,8 @@ _SIGNATURES = {
     "logismos_check_qgemv_q8g32_shape": (C.c_uint32, [_i, _i, C.c_char_p, _sz]),
     "logismos_check_paged_attn_shape": (C.c_uint32, [_i] * 9 + [C.c_char_p, _sz]),
     "logismos_launch_qgemv_q8g32_f32": (C.c_uint32, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
+    "logismos_check_qgemm_q4g128_shape": (C.c_uint32, [_i, _i, _i, C.c_char_p, _sz]),
+    "logismos_launch_qgemm_q4g128_bf16": (C.c_uint32, [_vp] * 5 + [_i, _i, _i, _vp]),
     "logismos_launch_repack_q8_0": (C.c_uint32, [_vp, _vp, _vp, _i, _i, _vp]),
     "logismos_paged_attn_num_splits": (C.c_int, [_i, _i, _i, _i]),
     "logismos_paged_attn_workspace_bytes": (_sz, [_i, _i, _i, _i]),
@@ -108,6 +110,16 @@ def launch_qgemv_q8g32_f32(x, qs, d, y, n: int, k: int, stream=None) -> None:
     check_qgemv_q8g32_shape(n, k)
     _status("qgemv_q8g32_f32", library().logismos_launch_qgemv_q8g32_f32(
         _ptr(x), _ptr(qs), _ptr(d), _ptr(y), n, k, _raw(stream)))
+
+
+def check_qgemm_q4g128_shape(b: int, n: int, k: int) -> None:
+    _guard("qgemm_q4g128_bf16", library().logismos_check_qgemm_q4g128_shape, b, n, k)
+
+
+def launch_qgemm_q4g128_bf16(x, qw, scale, zero, y, b: int, n: int, k: int, stream=None) -> None:
+    check_qgemm_q4g128_shape(b, n, k)
+    _status("qgemm_q4g128_bf16", library().logismos_launch_qgemm_q4g128_bf16(
+        _ptr(x), _ptr(qw), _ptr(scale), _ptr(zero), _ptr(y), b, n, k, _raw(stream)))
 
 
 def launch_repack_q8_0(blocks, qs, d, n: int, k: int, stream=None) -> None:

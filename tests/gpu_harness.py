@@ -60,6 +60,26 @@ class QgemvQ8Runner:
         return self.y.to_numpy(np.float32, (self.n,))
 
 
+class QgemmQ4Runner:
+    def __init__(self, x_bf16_bits, qw, scale, zero, b, n, k, stream=None):
+        self.b, self.n, self.k, self.stream = b, n, k, stream
+        self.x = hip.DeviceBuffer.from_numpy(np.ascontiguousarray(x_bf16_bits, np.uint16))
+        self.qw = hip.DeviceBuffer.from_numpy(np.ascontiguousarray(qw, np.uint8))
+        self.scale = hip.DeviceBuffer.from_numpy(np.ascontiguousarray(scale).view(np.uint16))
+        self.zero = hip.DeviceBuffer.from_numpy(np.ascontiguousarray(zero).view(np.uint16))
+        self.y = hip.DeviceBuffer(b * n * 2)
+        self.y.fill(0xFF)
+
+    def launch(self, qw=None, scale=None, zero=None):
+        kernels.launch_qgemm_q4g128_bf16(self.x, qw or self.qw, scale or self.scale,
+                                         zero or self.zero, self.y, self.b, self.n, self.k,
+                                         self.stream)
+
+    def result_bits(self) -> np.ndarray:
+        (self.stream.synchronize() if self.stream else hip.synchronize())
+        return self.y.to_numpy(np.uint16, (self.b, self.n))
+
+
 def assert_parity(got, want, max_abs=2e-3, max_rel=1e-2, what=""):
     """Tolerance of the decode path for fp16/bf16 outputs with fp32 accumulation:
     every element within max_abs OR within max_rel of the oracle (relative error

@@ -98,3 +98,14 @@ def test_num_splits_and_workspace_are_pure_functions():
     assert ns >= 1
     assert kernels.paged_attn_workspace_bytes(32, 32, 128, ns) == 32 * ns * 32 * 130 * 4
     assert kernels.paged_attn_workspace_bytes(32, 32, 128, 1) == 0
+
+
+@pytest.mark.parametrize("b,n,k,frag", [
+    (0, 8, 128, "batch must be positive"), (1, 0, 128, "N must be positive"),
+    (1, 8, 64, "multiple of the group size 128"), (1, 1 << 20, 1 << 12, "exceeds i32::MAX"),
+])
+def test_qgemm_q4_shape_guard(b, n, k, frag):
+    with pytest.raises(kernels.UnsupportedShape) as e:
+        kernels.check_qgemm_q4g128_shape(b, n, k)
+    assert frag in str(e.value)
+    kernels.check_qgemm_q4g128_shape(1, 12288, 4096)

@@ -1,0 +1,71 @@
+"""GPU parity: Q4G128 dequant-fused GEMV/GEMM vs the CPU oracle, through the C ABI.
+
+Tolerance (bf16 outputs, fp32 accumulation): 2e-3 max-abs or 1e-2 relative.
+"""
+import numpy as np
+import pytest
+
+import oracle as O
+from tests import workloads
+from tests.gpu_harness import QgemmQ4Runner, assert_parity
+
+pytestmark = pytest.mark.gpu
+
+_cache = {}
+
+
+def _config3():
+    if "c3" not in _cache:
+        c = workloads.config3()
+        qw, s, z = O.quantize_q4g128(c["w"], c["n"], c["k"])
+        _cache["c3"] = (c, qw, s, z)
+    return _cache["c3"]
+
+
+def _run(x_f32, qw, s, z, b, n, k):
+    xb = O.f32_to_bf16_bits(x_f32[:b])
+    r = QgemmQ4Runner(xb, qw, s, z, b, n, k)
+    r.launch()
+    got = O.bf16_bits_to_f32(r.result_bits())
+    want = O.bf16_bits_to_f32(O.qgemm_q4g128_bf16(xb, qw, s, z, b, n, k))
+    return got, want
+
+
+@pytest.mark.parametrize("b", [1, 2, 4])
+def test_config3_matches_oracle(b):
+    c, qw, s, z = _config3()
+    got, want = _run(c["x"], qw, s, z, b, c["n"], c["k"])
+    assert_parity(got, want, what=f"qgemm_q4 config 3 batch {b}")
+
+
+@pytest.mark.parametrize("b,n,k", [(1, 1, 128), (3, 5, 256), (2, 17, 1152), (4, 1000, 2048),
+                                   (1, 4096, 12288), (4, 4100, 4096), (3, 1024, 4096)])
+def test_ragged_shapes(b, n, k):
+    rng = np.random.default_rng(b * 1000003 + n * 101 + k)
+    w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
+    x = rng.standard_normal((b, k), np.float32)
+    qw, s, z = O.quantize_q4g128(w, n, k)
+    got, want = _run(x, qw, s, z, b, n, k)
+    assert_parity(got, want, what=f"qgemm_q4 {b}x{n}x{k}")
+
+
+def test_one_hot_x_reads_back_the_dequantised_column():
+    # orientation, nibble order and zero-point handling in one exact check
+    rng = np.random.default_rng(8)
+    n, k = 64, 256
+    w = rng.standard_normal((n, k), np.float32)
+    qw, s, z = O.quantize_q4g128(w, n, k)
+    wd = O.dequantize_q4g128(qw, s, z, n, k)
+    for col in (0, 1, 5, 127, 128, 255):
+        x = np.zeros((1, k), np.float32)
+        x[0, col] = 1.0
+        got, _ = _run(x, qw, s, z, 1, n, k)
+        want = O.bf16_bits_to_f32(O.f32_to_bf16_bits(wd[:, col]))
+        assert np.abs(got[0] - want).max() <= np.abs(want).max() * 2.0**-7, col
+
+
+def test_batch_rows_are_independent():
+    c, qw, s, z = _config3()
+    got4, _ = _run(c["x"], qw, s, z, 4, c["n"], c["k"])
+    got1, _ = _run(c["x"][2:3], qw, s, z, 1, c["n"], c["k"])
+    assert np.array_equal(got4[2], got1[0])

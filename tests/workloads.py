@@ -76,3 +76,15 @@ def config5_attention(seed=SEED + 5, num_seqs=32, lo=256, hi=8192):
     rng = np.random.default_rng(seed)
     ctx = rng.integers(lo, hi + 1, size=num_seqs)
     return paged_case(rng, np.ones(num_seqs, np.int32), ctx - 1, hq=32, hkv=8, spare_frac=0.05)
+
+
+def config3(seed=SEED + 3, n=12288, k=4096, max_batch=16):
+    """Q4G128 GEMV/GEMM at Qwen-8B geometry: W 12288x4096 ~N(0,0.02), x bf16 ~N(0,1)."""
+    rng = np.random.default_rng(seed)
+    w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
+    x = rng.standard_normal((max_batch, k), np.float32)
+    return dict(w=w, x=x, n=n, k=k)
+
+
+def qgemm_q4_algorithmic_bytes(b, n, k) -> int:
+    return n * k // 2 + n * (k // 128) * 4 + b * k * 2 + b * n * 2
