@@ -132,13 +132,21 @@ logismos_status_t logismos_launch_qgemv_q8g32_f32(const void* x_f32, const void*
 /* y[b][n] = sum_k x[b][k] * w[n][k], w in Q4G128.  x bf16 `[B][K]`, y bf16
  * `[B][N]`, fp32 accumulation, one rounding at the end: `cpu_f32::linear_t`
  * (crates/kernels/src/cpu_f32/mod.rs:271-345) over the dequantised matrix with
- * m = B.  Batch 1..4 runs the bandwidth-bound VALU GEMV, larger batches the
- * MFMA kernel.  Requires k % 128 == 0; x and qw 16-byte aligned. */
+ * m = B <= 32.  Batch 1..4 runs the bandwidth-bound VALU GEMV, larger batches
+ * the MFMA kernel.  Requires k % 128 == 0; x and qw 16-byte aligned. */
 logismos_status_t logismos_check_qgemm_q4g128_shape(int b, int n, int k, char* msg, size_t msg_cap);
 logismos_status_t logismos_launch_qgemm_q4g128_bf16(const void* x_bf16, const void* qw_u8,
                                                     const void* scale_f16, const void* zero_f16,
                                                     void* y_bf16, int b, int n, int k,
                                                     logismos_stream_t stream);
+
+/* The same product forced onto the MFMA kernel for any batch 1..32 (the default
+ * launcher uses it from batch 5): lets a caller or a benchmark compare the two
+ * paths on identical inputs. */
+logismos_status_t logismos_launch_qgemm_q4g128_bf16_mfma(const void* x_bf16, const void* qw_u8,
+                                                         const void* scale_f16,
+                                                         const void* zero_f16, void* y_bf16, int b,
+                                                         int n, int k, logismos_stream_t stream);
 
 /* ggml Q8_0 block stream `[N][K/32]{f16 d; int8 qs[32]}` -> planar Q8G32. */
 logismos_status_t logismos_launch_repack_q8_0(const void* blocks_q8_0, void* qs_i8, void* d_f16,

@@ -49,6 +49,7 @@ _SIGNATURES = {
     "logismos_launch_qgemv_q8g32_f32": (C.c_uint32, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
     "logismos_check_qgemm_q4g128_shape": (C.c_uint32, [_i, _i, _i, C.c_char_p, _sz]),
     "logismos_launch_qgemm_q4g128_bf16": (C.c_uint32, [_vp] * 5 + [_i, _i, _i, _vp]),
+    "logismos_launch_qgemm_q4g128_bf16_mfma": (C.c_uint32, [_vp] * 5 + [_i, _i, _i, _vp]),
     "logismos_launch_repack_q8_0": (C.c_uint32, [_vp, _vp, _vp, _i, _i, _vp]),
     "logismos_paged_attn_num_splits": (C.c_int, [_i, _i, _i, _i]),
     "logismos_paged_attn_workspace_bytes": (_sz, [_i, _i, _i, _i]),
@@ -116,10 +117,13 @@ def check_qgemm_q4g128_shape(b: int, n: int, k: int) -> None:
     _guard("qgemm_q4g128_bf16", library().logismos_check_qgemm_q4g128_shape, b, n, k)
 
 
-def launch_qgemm_q4g128_bf16(x, qw, scale, zero, y, b: int, n: int, k: int, stream=None) -> None:
+def launch_qgemm_q4g128_bf16(x, qw, scale, zero, y, b: int, n: int, k: int, stream=None,
+                             force_mfma: bool = False) -> None:
     check_qgemm_q4g128_shape(b, n, k)
-    _status("qgemm_q4g128_bf16", library().logismos_launch_qgemm_q4g128_bf16(
-        _ptr(x), _ptr(qw), _ptr(scale), _ptr(zero), _ptr(y), b, n, k, _raw(stream)))
+    fn = (library().logismos_launch_qgemm_q4g128_bf16_mfma if force_mfma
+          else library().logismos_launch_qgemm_q4g128_bf16)
+    _status("qgemm_q4g128_bf16", fn(_ptr(x), _ptr(qw), _ptr(scale), _ptr(zero), _ptr(y), b, n, k,
+                                    _raw(stream)))
 
 
 def launch_repack_q8_0(blocks, qs, d, n: int, k: int, stream=None) -> None:

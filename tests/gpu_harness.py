@@ -70,10 +70,10 @@ class QgemmQ4Runner:
         self.y = hip.DeviceBuffer(b * n * 2)
         self.y.fill(0xFF)
 
-    def launch(self, qw=None, scale=None, zero=None):
+    def launch(self, qw=None, scale=None, zero=None, force_mfma=False):
         kernels.launch_qgemm_q4g128_bf16(self.x, qw or self.qw, scale or self.scale,
                                          zero or self.zero, self.y, self.b, self.n, self.k,
-                                         self.stream)
+                                         self.stream, force_mfma)
 
     def result_bits(self) -> np.ndarray:
         (self.stream.synchronize() if self.stream else hip.synchronize())

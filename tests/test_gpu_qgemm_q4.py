@@ -22,20 +22,39 @@ def _config3():
     return _cache["c3"]
 
 
-def _run(x_f32, qw, s, z, b, n, k):
+def _run(x_f32, qw, s, z, b, n, k, force_mfma=False):
     xb = O.f32_to_bf16_bits(x_f32[:b])
     r = QgemmQ4Runner(xb, qw, s, z, b, n, k)
-    r.launch()
+    r.launch(force_mfma=force_mfma)
     got = O.bf16_bits_to_f32(r.result_bits())
     want = O.bf16_bits_to_f32(O.qgemm_q4g128_bf16(xb, qw, s, z, b, n, k))
     return got, want
 
 
-@pytest.mark.parametrize("b", [1, 2, 4])
+@pytest.mark.parametrize("b", [1, 2, 4, 8, 16])
 def test_config3_matches_oracle(b):
     c, qw, s, z = _config3()
     got, want = _run(c["x"], qw, s, z, b, c["n"], c["k"])
     assert_parity(got, want, what=f"qgemm_q4 config 3 batch {b}")
+
+
+@pytest.mark.parametrize("b", [1, 3, 4])
+def test_config3_mfma_path_at_small_batch(b):
+    c, qw, s, z = _config3()
+    got, want = _run(c["x"], qw, s, z, b, c["n"], c["k"], force_mfma=True)
+    assert_parity(got, want, what=f"qgemm_q4 config 3 batch {b} (mfma)")
+
+
+@pytest.mark.parametrize("b,n,k", [(5, 16, 128), (7, 33, 256), (8, 17, 1152), (16, 1000, 2048),
+                                   (9, 4096, 12288), (32, 4100, 4096), (17, 1024, 4096),
+                                   (32, 12288, 4096), (32, 4096, 12288), (24, 70000, 256)])
+def test_mfma_ragged_shapes(b, n, k):
+    rng = np.random.default_rng(b * 1000003 + n * 101 + k)
+    w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
+    x = rng.standard_normal((b, k), np.float32)
+    qw, s, z = O.quantize_q4g128(w, n, k)
+    got, want = _run(x, qw, s, z, b, n, k)
+    assert_parity(got, want, what=f"qgemm_q4 mfma {b}x{n}x{k}")
 
 
 @pytest.mark.parametrize("b,n,k", [(1, 1, 128), (3, 5, 256), (2, 17, 1152), (4, 1000, 2048),
