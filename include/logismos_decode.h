@@ -132,8 +132,8 @@ logismos_status_t logismos_launch_qgemv_q8g32_f32(const void* x_f32, const void*
 /* y[b][n] = sum_k x[b][k] * w[n][k], w in Q4G128.  x bf16 `[B][K]`, y bf16
  * `[B][N]`, fp32 accumulation, one rounding at the end: `cpu_f32::linear_t`
  * (crates/kernels/src/cpu_f32/mod.rs:271-345) over the dequantised matrix with
- * m = B <= 32.  Batch 1..4 runs the bandwidth-bound VALU GEMV, larger batches
- * the MFMA kernel.  Requires k % 128 == 0; x and qw 16-byte aligned. */
+ * m = B <= 32.  Batch 1..2 runs the bandwidth-bound VALU GEMV (in-register nibble
+ * unpack, v_dot2), batch >= 3 the MFMA kernel (measured crossover on MI355X).  Requires k % 128 == 0; x and qw 16-byte aligned. */
 logismos_status_t logismos_check_qgemm_q4g128_shape(int b, int n, int k, char* msg, size_t msg_cap);
 logismos_status_t logismos_launch_qgemm_q4g128_bf16(const void* x_bf16, const void* qw_u8,
                                                     const void* scale_f16, const void* zero_f16,
@@ -141,7 +141,7 @@ logismos_status_t logismos_launch_qgemm_q4g128_bf16(const void* x_bf16, const vo
                                                     logismos_stream_t stream);
 
 /* The same product forced onto the MFMA kernel for any batch 1..32 (the default
- * launcher uses it from batch 5): lets a caller or a benchmark compare the two
+ * launcher uses it from batch 3): lets a caller or a benchmark compare the two
  * paths on identical inputs. */
 logismos_status_t logismos_launch_qgemm_q4g128_bf16_mfma(const void* x_bf16, const void* qw_u8,
                                                          const void* scale_f16,

@@ -219,173 +219,192 @@ static hipError_t launch_gemv_b(const void* x, const void* qw, const void* scale
 // MFMA path, batch 5..32.  y^T is computed: the weight tile is the B operand
 // of v_mfma_f32_16x16x32_bf16 (column = weight row n, 8 contraction elements
 // per lane = one dword of nibbles turned into four bf16 pairs), x is the A
-// operand (row = batch index) read from LDS, so that the four results a lane
-// holds all belong to ONE weight row and need only that row's scale / zero.
+// operand (row = batch index), so that the four results a lane holds all
+// belong to ONE weight row and need only that row's scale / zero.
 //
-// A workgroup owns TL tiles of 16 weight rows and splits K KQ ways: wave
-// (tl, kq) handles, in every slab of KQ*GPB groups, the GPB consecutive groups
-// [slab*KQ*GPB + kq*GPB, +GPB) of its tile.  One 16-byte load per lane covers a
-// whole group (128 nibbles) of a row: lane (n = lane%16, kc = lane/16) reads
-// bytes [64 g + 16 kc, +16) of row n; its dword t feeds MFMA t, which therefore
-// contracts over k = 128 g + 32 kc + 8 t + (0..7), kc = 0..3.  The loads of the
-// next slab are issued before the current one is consumed (register double
-// buffer).  x of the slab sits in LDS as xl[batch][k/8] (16-byte words in pair
-// order) next to xg[group][batch], the per-group sums of x.
-// The KQ partial results of a tile are folded through LDS at the end.
+// A workgroup owns T tiles of 16 weight rows and ALL of K, split across its W
+// waves: in phase p, wave w owns the GW consecutive groups starting at
+// (p*W + w)*GW.  Its slice of x (all batch rows, GW*128 columns) is loaded
+// straight from global memory (L2-resident) into MFMA A-operand registers once
+// per phase and reused for every tile; one 16-byte load per lane covers a whole
+// group (128 nibbles) of a weight row: lane (n = lane%16, kc = lane/16) reads
+// bytes [64 g + 16 kc, +16) of row n, its dword t feeds MFMA t, which therefore
+// contracts over k = 128 g + 32 kc + 8 t + (0..7), kc = 0..3.  Every load of a
+// phase is issued before any of it is consumed.  Waves never wait for each
+// other while streaming: every wave keeps its partial results in its own LDS
+// slot (LDS float atomics on shared accumulators measured 2-4x slower for the
+// whole kernel), and the slots are summed once after the only barrier.  scale / zero of the
+// workgroup's rows are staged in LDS with one coalesced copy (per-lane 2-byte
+// loads from 16 different rows per instruction are what this avoids).
 // ---------------------------------------------------------------------------
-template <int BT, int GPB>
+template <int BT, int GW, int T>
 __global__ __launch_bounds__(1024) void qgemm_q4g128_mfma_kernel(
     const uint16_t* __restrict__ x, const uint8_t* __restrict__ qw,
     const __half* __restrict__ scale, const __half* __restrict__ zero, uint16_t* __restrict__ y,
-    int b, int n, int k, int tl_count, int kq_count) {
+    int b, int n, int k) {
     extern __shared__ uint4_t lds[];
-    constexpr int BP = BT * 16;  // padded batch
+    constexpr int BP = BT * 16;
     const int groups = k >> 7;
-    const int slab_groups = kq_count * GPB;
-    const int num_slabs = (groups + slab_groups - 1) / slab_groups;
-    // xl[batch][chunk] with a row stride == 1 (mod 16) 16-byte words: the 16 batch
-    // rows a quad reads for one chunk then fall into 16 different bank groups
-    const int qs = slab_groups * 16 + 1;
-    uint4_t* xl = lds;                                                // [BP][qs]
-    float* xg = reinterpret_cast<float*>(lds + (size_t)BP * qs);      // [slab_groups][BP]
+    float* yl = reinterpret_cast<float*>(lds);  // [waves][T][BP][16] partial results
+    __half* sz = reinterpret_cast<__half*>(yl + (size_t)(blockDim.x >> 6) * T * BP * 16);
+    // sz: scale [T*16][groups], then zero [T*16][groups]
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int nwaves = blockDim.x >> 6;
-    const int tl = wave / kq_count;
-    const int kq = wave - tl * kq_count;
-    const int col = lane & 15;  // weight row inside the tile / batch row of the A operand
+    const int col = lane & 15;
     const int kc = lane >> 4;
-    const int64_t tile = (int64_t)blockIdx.x * tl_count + tl;
-    const int64_t row_raw = tile * 16 + col;
-    const int64_t row = row_raw < n ? row_raw : (int64_t)(n - 1);
-    const uint8_t* wrow = qw + row * (int64_t)(k >> 1) + kc * 16;
-    const __half* srow = scale + row * groups;
-    const __half* zrow = zero + row * groups;
+    const int64_t row0 = (int64_t)blockIdx.x * T * 16;
+    const int rows_here = (int)min((int64_t)(T * 16), (int64_t)n - row0);
 
     unsigned magic;
     asm volatile("v_mov_b32 %0, 0x43004300" : "=v"(magic));
 
-    uint4_t wbuf[2][GPB];
-    auto load_slab = [&](int slab, uint4_t (&dst)[GPB]) {
-        const int g0 = slab * slab_groups + kq * GPB;
+    struct Phase {
+        uint4_t xa[GW][4][BT];
+        uint4_t w[T][GW];
+    };
+    const uint8_t* wrow[T];
 #pragma unroll
-        for (int i = 0; i < GPB; ++i) {
+    for (int ti = 0; ti < T; ++ti) {
+        const int r = ti * 16 + col;
+        wrow[ti] = qw + (row0 + (r < rows_here ? r : rows_here - 1)) * (int64_t)(k >> 1) + kc * 16;
+    }
+    const uint16_t* xrow[BT];
+#pragma unroll
+    for (int bt = 0; bt < BT; ++bt) {
+        const int bi = bt * 16 + col;
+        xrow[bt] = x + (int64_t)(bi < b ? bi : b - 1) * k + kc * 32;
+    }
+    auto issue = [&](int phase, Phase& ph) {
+        const int g0 = (phase * nwaves + wave) * GW;
+#pragma unroll
+        for (int i = 0; i < GW; ++i) {
             const int g = (g0 + i) < groups ? (g0 + i) : (groups - 1);
-            dst[i] = *reinterpret_cast<const uint4_t*>(wrow + (int64_t)g * 64);
+#pragma unroll
+            for (int bt = 0; bt < BT; ++bt)
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#ifdef LG_EXP_NOXLOAD
+                    ph.xa[i][t][bt] = uint4_t{0x3f803f80u, (unsigned)g, 0x3f803f80u, (unsigned)lane};
+#else
+                    ph.xa[i][t][bt] =
+                        *reinterpret_cast<const uint4_t*>(xrow[bt] + (int64_t)g * 128 + t * 8);
+#endif
         }
+#pragma unroll
+        for (int ti = 0; ti < T; ++ti)
+#pragma unroll
+            for (int i = 0; i < GW; ++i) {
+                const int g = (g0 + i) < groups ? (g0 + i) : (groups - 1);
+#ifdef LG_EXP_NOWLOAD
+                ph.w[ti][i] = uint4_t{0x12345678u, (unsigned)g, 0x9abcdef0u, (unsigned)lane};
+#else
+                ph.w[ti][i] = *reinterpret_cast<const uint4_t*>(wrow[ti] + (int64_t)g * 64);
+#endif
+            }
     };
 
-    float4_t yacc[BT];
-#pragma unroll
-    for (int t = 0; t < BT; ++t) yacc[t] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    const int num_phases = (groups + nwaves * GW - 1) / (nwaves * GW);
+    Phase ph;
+    issue(0, ph);
+    __builtin_amdgcn_sched_barrier(0);
 
-    auto compute_slab = [&](int slab, const uint4_t (&w)[GPB]) {
-        const int g0 = slab * slab_groups + kq * GPB;
+    float* yw = yl + (size_t)wave * T * BP * 16;
+    // while the first loads fly: stage scale / zero
+    {
+        const int count = rows_here * groups;
+        const __half* s0 = scale + row0 * groups;
+        const __half* z0 = zero + row0 * groups;
+        for (int i = threadIdx.x; i < count; i += blockDim.x) {
+            sz[i] = s0[i];
+            sz[T * 16 * groups + i] = z0[i];
+        }
+    }
+    __syncthreads();
+    const __half* zl = sz + T * 16 * groups;
+
+    for (int phase = 0; phase < num_phases; ++phase) {
+        if (phase > 0) {
+            issue(phase, ph);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        const int g0 = (phase * nwaves + wave) * GW;
+        // x slice: pair order in place, per-group sums of x in result layout
+        float xsum[GW][BT][4];
 #pragma unroll
-        for (int i = 0; i < GPB; ++i) {
-            const int g = g0 + i;
-            if (g < groups) {  // wave-uniform
-                const float sf = __half2float(srow[g]);
-                const float off = 128.0f + __half2float(zrow[g]);
-                const int gl = kq * GPB + i;  // group index inside the slab
-                float4_t acc[BT];
+        for (int i = 0; i < GW; ++i)
 #pragma unroll
-                for (int t = 0; t < BT; ++t) acc[t] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+            for (int bt = 0; bt < BT; ++bt) {
+                float part = 0.0f;
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
-                    const unsigned wd = w[i][t];
+                    part += sum8_bf16(ph.xa[i][t][bt]);
+                    ph.xa[i][t][bt] = pair_order(ph.xa[i][t][bt]);
+                }
+                part += shfl_xor_f32(part, 16);
+                part += shfl_xor_f32(part, 32);  // sum over the group for batch row `col`
+#pragma unroll
+                for (int e = 0; e < 4; ++e) xsum[i][bt][e] = __shfl(part, 4 * kc + e, kWave);
+            }
+#pragma unroll
+        for (int ti = 0; ti < T; ++ti) {
+            float4_t ysum[BT];
+#pragma unroll
+            for (int bt = 0; bt < BT; ++bt) ysum[bt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+            const int r = ti * 16 + col;
+            const int rl = r < rows_here ? r : rows_here - 1;
+#pragma unroll
+            for (int i = 0; i < GW; ++i) {
+                const bool valid = (g0 + i) < groups;  // wave-uniform
+                const int g = valid ? (g0 + i) : (groups - 1);
+                const float sf = __half2float(sz[rl * groups + g]);
+                const float off = 128.0f + __half2float(zl[rl * groups + g]);
+                float4_t acc[BT];
+#pragma unroll
+                for (int bt = 0; bt < BT; ++bt) acc[bt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const unsigned wd = ph.w[ti][i][t];
                     uint4_t h;
 #pragma unroll
-                    for (int s = 0; s < 4; ++s) h[s] = ((wd >> (4 * s)) & kNibMask) | magic;
+                    for (int sft = 0; sft < 4; ++sft)
+                        h[sft] = ((wd >> (4 * sft)) & kNibMask) | magic;
                     const bf16x8_t bop = __builtin_bit_cast(bf16x8_t, h);
-                    const int q = gl * 16 + 4 * kc + t;
 #pragma unroll
-                    for (int bt = 0; bt < BT; ++bt) {
-                        const bf16x8_t aop =
-                            __builtin_bit_cast(bf16x8_t, xl[(size_t)(bt * 16 + col) * qs + q]);
-                        acc[bt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aop, bop, acc[bt], 0, 0, 0);
+                    for (int bt = 0; bt < BT; ++bt)
+                        acc[bt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            __builtin_bit_cast(bf16x8_t, ph.xa[i][t][bt]), bop, acc[bt], 0, 0, 0);
+                }
+#pragma unroll
+                for (int bt = 0; bt < BT; ++bt)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float v = fmaf(sf, fmaf(-off, xsum[i][bt][e], acc[bt][e]), ysum[bt][e]);
+                        ysum[bt][e] = valid ? v : ysum[bt][e];
                     }
-                }
-#pragma unroll
-                for (int bt = 0; bt < BT; ++bt) {
-                    const float4_t xsum =
-                        *reinterpret_cast<const float4_t*>(xg + (size_t)gl * BP + bt * 16 + 4 * kc);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        yacc[bt][e] = fmaf(sf, fmaf(-off, xsum[e], acc[bt][e]), yacc[bt][e]);
-                }
             }
-        }
-    };
-
-    auto stage_x = [&](int slab) {
-        const int g_begin = slab * slab_groups;
-        const int g_count = min(slab_groups, groups - g_begin);
-        const int chunks = g_count * 16;  // 8-element chunks in the slab
-        for (int idx = threadIdx.x; idx < chunks * BP; idx += blockDim.x) {
-            const int bi = idx / chunks, q = idx - bi * chunks;
-            uint4_t d = uint4_t{0u, 0u, 0u, 0u};
-            if (bi < b)
-                d = *reinterpret_cast<const uint4_t*>(x + (int64_t)bi * k + (int64_t)g_begin * 128 +
-                                                      (int64_t)q * 8);
-            xl[(size_t)bi * qs + q] = pair_order(d);
-        }
-        __syncthreads();
-        // per-group sums from the staged chunks (16 chunks per group)
-        for (int idx = threadIdx.x; idx < g_count * BP; idx += blockDim.x) {
-            const int gl = idx / BP, bi = idx - gl * BP;
-            float sum = 0.0f;
 #pragma unroll
-            for (int q = 0; q < 16; ++q) sum += sum8_bf16(xl[(size_t)bi * qs + gl * 16 + q]);
-            xg[(size_t)gl * BP + bi] = sum;
-        }
-    };
-
-    load_slab(0, wbuf[0]);
-    for (int slab = 0; slab < num_slabs; slab += 2) {
-        load_slab(min(slab + 1, num_slabs - 1), wbuf[1]);
-        __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();  // everyone is done with the previous slab's x
-        stage_x(slab);
-        __syncthreads();
-        compute_slab(slab, wbuf[0]);
-        if (slab + 1 >= num_slabs) break;  // uniform
-        load_slab(min(slab + 2, num_slabs - 1), wbuf[0]);
-        __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();
-        stage_x(slab + 1);
-        __syncthreads();
-        compute_slab(slab + 1, wbuf[1]);
-    }
-
-    // ---- fold the KQ partials of each tile through LDS, store bf16
-    __syncthreads();
-    float4_t* red = reinterpret_cast<float4_t*>(lds);  // [nwaves][BT][64]
+            for (int bt = 0; bt < BT; ++bt)
 #pragma unroll
-    for (int bt = 0; bt < BT; ++bt) red[((size_t)wave * BT + bt) * 64 + lane] = yacc[bt];
-    __syncthreads();
-    if (kq == 0) {
-#pragma unroll
-        for (int bt = 0; bt < BT; ++bt) {
-            float4_t sum = yacc[bt];
-            for (int j = 1; j < kq_count; ++j) {
-                const float4_t o = red[((size_t)(wave + j) * BT + bt) * 64 + lane];
-                sum[0] += o[0];
-                sum[1] += o[1];
-                sum[2] += o[2];
-                sum[3] += o[3];
-            }
-            if (row_raw < n) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int bi = bt * 16 + 4 * kc + e;
-                    if (bi < b) y[(int64_t)bi * n + row_raw] = f32_to_bf16_rne(sum[e]);
+                for (int e = 0; e < 4; ++e)
+{
+                    // this wave's own slot: no other wave touches it before the barrier
+                    float* slot = &yw[(ti * BP + bt * 16 + 4 * kc + e) * 16 + col];
+                    *slot = (phase == 0) ? ysum[bt][e] : (*slot + ysum[bt][e]);
                 }
-            }
         }
     }
-    (void)nwaves;
+    __syncthreads();
+    for (int i = threadIdx.x; i < T * BP * 16; i += blockDim.x) {
+        const int c = i & 15;
+        const int bi = (i >> 4) % BP;
+        const int ti = i / (BP * 16);
+        const int r = ti * 16 + c;
+        float sum = 0.0f;
+        for (int w = 0; w < nwaves; ++w) sum += yl[(size_t)w * T * BP * 16 + i];
+        if (r < rows_here && bi < b) y[(int64_t)bi * n + row0 + r] = f32_to_bf16_rne(sum);
+    }
 }
 
 static int device_cu_count() {
@@ -400,54 +419,40 @@ static int device_cu_count() {
     return count;
 }
 
-template <int BT>
-static hipError_t launch_mfma(const void* x, const void* qw, const void* scale, const void* zero,
-                              void* y, int b, int n, int k, hipStream_t stream) {
+template <int BT, int GW, int T>
+static hipError_t launch_mfma_t(const void* x, const void* qw, const void* scale, const void* zero,
+                                void* y, int b, int n, int k, hipStream_t stream) {
     const int groups = k / 128;
     const int tiles = (n + 15) / 16;
-    const int cus = device_cu_count();
-    int tl = (tiles + cus - 1) / cus;  // tiles per workgroup
-    if (tl > 4) tl = 4;
-    int kq = 1;
-    while (tl * kq * 2 <= 16 && kq * 2 <= groups) kq *= 2;
-    // groups per wave per slab: LDS holds kq*gpb groups of x for BT*16 batch rows
-    // (4 KiB per group per batch tile); keep it within 128 KiB
-    int gpb = 32 / (kq * BT);
-    const int gpb_max = BT == 1 ? 8 : 4;  // register budget of the weight double buffer
-    if (gpb > gpb_max) gpb = gpb_max;
-    if (gpb < 1) gpb = 1;
-    while (gpb > 1 && kq * (gpb / 2) >= groups) gpb /= 2;  // do not stage more than K
-    const int slab_groups = kq * gpb;
-    const size_t lds_x =
-        (size_t)(slab_groups * 16 + 1) * BT * 16 * 16 + (size_t)slab_groups * BT * 16 * 4;
-    const size_t lds_red = (size_t)tl * kq * BT * 64 * 16;
-    const size_t lds = lds_x > lds_red ? lds_x : lds_red;
-    const int grid = (tiles + tl - 1) / tl;
-    dim3 block(64 * tl * kq);
-#define LG_LAUNCH_MFMA(GPB)                                                                      \
-    {                                                                                            \
-        auto kern = qgemm_q4g128_mfma_kernel<BT, GPB>;                                           \
-        if (lds > 64 * 1024) {                                                                   \
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),              \
-                                               hipFuncAttributeMaxDynamicSharedMemorySize,       \
-                                               (int)lds);                                        \
-            if (e != hipSuccess) return e;                                                       \
-        }                                                                                        \
-        kern<<<dim3(grid), block, lds, stream>>>(                                                \
-            static_cast<const uint16_t*>(x), static_cast<const uint8_t*>(qw),                    \
-            static_cast<const __half*>(scale), static_cast<const __half*>(zero),                 \
-            static_cast<uint16_t*>(y), b, n, k, tl, kq);                                         \
+    int waves = (groups + GW - 1) / GW;
+    if (waves > 16) waves = 16;
+    const size_t lds =
+        (size_t)waves * T * BT * 16 * 16 * 4 + (size_t)2 * T * 16 * groups * 2;
+    auto kern = qgemm_q4g128_mfma_kernel<BT, GW, T>;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
     }
-    switch (gpb) {
-        case 8:
-            if constexpr (BT == 1) LG_LAUNCH_MFMA(8)
-            break;
-        case 4: LG_LAUNCH_MFMA(4) break;
-        case 2: LG_LAUNCH_MFMA(2) break;
-        default: LG_LAUNCH_MFMA(1) break;
-    }
-#undef LG_LAUNCH_MFMA
+    kern<<<dim3((tiles + T - 1) / T), dim3(64 * waves), lds, stream>>>(
+        static_cast<const uint16_t*>(x), static_cast<const uint8_t*>(qw),
+        static_cast<const __half*>(scale), static_cast<const __half*>(zero),
+        static_cast<uint16_t*>(y), b, n, k);
     return hipGetLastError();
+}
+
+template <int BT, int GW>
+static hipError_t launch_mfma(const void* x, const void* qw, const void* scale, const void* zero,
+                              void* y, int b, int n, int k, hipStream_t stream) {
+    const int tiles = (n + 15) / 16;
+    const int cus = device_cu_count();
+    const int t = (tiles + cus - 1) / cus;  // row tiles per workgroup
+    if constexpr (BT == 2) {  // one group per wave: registers allow six tiles
+        if (t >= 6) return launch_mfma_t<BT, GW, 6>(x, qw, scale, zero, y, b, n, k, stream);
+    }
+    if (t >= 3) return launch_mfma_t<BT, GW, 3>(x, qw, scale, zero, y, b, n, k, stream);
+    if (t == 2) return launch_mfma_t<BT, GW, 2>(x, qw, scale, zero, y, b, n, k, stream);
+    return launch_mfma_t<BT, GW, 1>(x, qw, scale, zero, y, b, n, k, stream);
 }
 
 constexpr size_t kMaxLds = 160 * 1024;
@@ -488,13 +493,12 @@ static logismos_status_t qgemm_q4_dispatch(const void* x_bf16, const void* qw_u8
         switch (b) {
             case 1: return lg::launch_gemv_b<1>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, n, k, st);
             case 2: return lg::launch_gemv_b<2>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, n, k, st);
-            case 3: return lg::launch_gemv_b<3>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, n, k, st);
-            case 4: return lg::launch_gemv_b<4>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, n, k, st);
-            default: break;
+            default: break;  // batch 3 and 4: the MFMA kernel is faster (measured crossover)
         }
     }
-    if (b <= 16) return lg::launch_mfma<1>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, b, n, k, st);
-    return lg::launch_mfma<2>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, b, n, k, st);
+    if (b <= 16)
+        return lg::launch_mfma<1, 2>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, b, n, k, st);
+    return lg::launch_mfma<2, 1>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, b, n, k, st);
 }
 
 extern "C" logismos_status_t logismos_launch_qgemm_q4g128_bf16(
