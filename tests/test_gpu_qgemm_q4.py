@@ -84,7 +84,14 @@ def test_one_hot_x_reads_back_the_dequantised_column():
 
 
 def test_batch_rows_are_independent():
+    # a batch row's result does not depend on its neighbours or its position
     c, qw, s, z = _config3()
-    got4, _ = _run(c["x"], qw, s, z, 4, c["n"], c["k"])
-    got1, _ = _run(c["x"][2:3], qw, s, z, 1, c["n"], c["k"])
-    assert np.array_equal(got4[2], got1[0])
+    n, k = c["n"], c["k"]
+    got4, _ = _run(c["x"], qw, s, z, 4, n, k)                 # MFMA kernel
+    got3, _ = _run(c["x"][[2, 0, 1]], qw, s, z, 3, n, k)      # MFMA kernel, row 2 first
+    assert np.array_equal(got4[2], got3[0])
+    got2, _ = _run(c["x"], qw, s, z, 2, n, k)                 # VALU GEMV
+    got1, _ = _run(c["x"][1:2], qw, s, z, 1, n, k)
+    assert np.array_equal(got2[1], got1[0])
+    # the two kernels agree to bf16 rounding
+    assert_parity(got4[1], got2[1], what="mfma vs gemv")
