@@ -219,6 +219,74 @@ logismos_status_t logismos_launch_paged_attn_varlen_fp16_phases(
     int phases, logismos_stream_t stream);
 
 /* ------------------------------------------------------------------------
+ * Ragged packing and KV writes
+ * ------------------------------------------------------------------------ */
+
+/* From per-sequence counts to the packed-batch index buffers, on the GPU:
+ *   cu_seqlens[0] = 0, cu_seqlens[s+1] = cu_seqlens[s] + new_tokens[s]
+ *   context_lens[s] = prior_ctx[s] + new_tokens[s]
+ *   slot_mapping[cu_seqlens[s] + i] = slot of position prior_ctx[s] + i of sequence s
+ *                                     (-1 when that position lies past max_blocks)
+ * new_tokens, prior_ctx int32 `[num_seqs]` (negative values count as 0);
+ * slot_mapping int64 `[sum new_tokens]`.  The host never needs the total. */
+logismos_status_t logismos_check_pack_ragged_shape(int num_seqs, int block_size, int max_blocks,
+                                                   char* msg, size_t msg_cap);
+logismos_status_t logismos_launch_pack_ragged(const int32_t* new_tokens, const int32_t* prior_ctx,
+                                              const int32_t* block_tables, int32_t* cu_seqlens,
+                                              int64_t* slot_mapping, int32_t* context_lens,
+                                              int num_seqs, int block_size, int max_blocks,
+                                              logismos_stream_t stream);
+
+/* Row t of k_new / v_new (fp16 `[total_tokens][num_kv_heads*head_dim]`, the rows
+ * `KvCache::put` takes, crates/cache/src/lib.rs:57-64) is written to pool row
+ * slot_mapping[t]; negative slots are skipped.  num_kv_heads*head_dim % 8 == 0. */
+logismos_status_t logismos_launch_kv_write_fp16(const void* k_new_f16, const void* v_new_f16,
+                                                void* k_pool_f16, void* v_pool_f16,
+                                                const int64_t* slot_mapping, int total_tokens,
+                                                int num_kv_heads, int head_dim,
+                                                logismos_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Small operators of the decode step (gfx950 versions of the reference's
+ * cpu_f32 contracts, crates/kernels/src/cpu_f32/mod.rs)
+ * ------------------------------------------------------------------------ */
+
+/* h[r][:] += y[r][:] (skipped when y_bf16 == NULL), then
+ * out[r][:] = bf16( h * (1/sqrt(mean(h^2)+eps)) * w ): the pre-norm residual
+ * step of a layer (crates/encoders/src/stella.rs:190-206) over `rms_norm`
+ * (crates/kernels/src/cpu_f32/mod.rs:137-159).  h fp32 `[rows][n]` in place,
+ * w fp32 `[n]`. */
+logismos_status_t logismos_launch_add_rms_norm_bf16(void* h_f32, const void* y_bf16,
+                                                    const void* w_f32, void* out_bf16, int rows,
+                                                    int n, float eps, logismos_stream_t stream);
+
+/* Splits qkv (bf16 `[T][(hq+2*hkv)*128]`, q heads, then k heads, then v heads),
+ * applies RoPE in the halves convention (`rope_halves_in_place`,
+ * crates/kernels/src/cpu_f32/mod.rs:502-547) to q and k with the token's
+ * position (clamped to [0, max_pos)), and writes q as fp16 `[T][hq][128]`, k and
+ * v as fp16 rows of the paged pools at slot_mapping[t] (negative: skipped).
+ * cos / sin: fp32 `[max_pos][64]` (`build_rope_table_f32`, :599-619). */
+logismos_status_t logismos_launch_rope_kv_write_fp16(
+    const void* qkv_bf16, const int32_t* positions, const void* cos_f32, const void* sin_f32,
+    const int64_t* slot_mapping, void* q_out_f16, void* k_pool_f16, void* v_pool_f16,
+    int total_tokens, int num_q_heads, int num_kv_heads, int head_dim, int max_pos,
+    logismos_stream_t stream);
+
+/* out[t][j] = bf16( silu(gate) * up ), gate_up bf16 `[rows][2*inter]` = gate | up
+ * (`SwiGluMlp::forward`, crates/transformers/src/mlp.rs:82-125; `silu`,
+ * `hadamard`, crates/kernels/src/cpu_f32/mod.rs:349-374). */
+logismos_status_t logismos_launch_silu_mul_bf16(const void* gate_up_bf16, void* out_bf16, int rows,
+                                                int inter, logismos_stream_t stream);
+
+logismos_status_t logismos_launch_cast_f16_bf16(const void* in_f16, void* out_bf16, size_t count,
+                                                logismos_stream_t stream);
+
+/* out[r] = first index of the maximum of logits[r][:] (`decode::greedy`,
+ * crates/decode/src/lib.rs:73-83: strict >, the first maximum wins). */
+logismos_status_t logismos_launch_greedy_f32(const void* logits_f32, void* out_u32, int rows, int n,
+                                             logismos_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * Memory-system probes (measurement aids; the reference has no counterpart,
  * its only timing helper is the hipEvent pair of
  * crates/kernels/examples/gemm_bench.rs:120-128).  A plain copy and a plain

@@ -1,0 +1,217 @@
+// The small operators of a decode step, gfx950 versions of the contracts the
+// reference's CPU op set defines (crates/kernels/src/cpu_f32/mod.rs):
+// residual add + RMSNorm, RoPE (halves convention) fused with the KV write,
+// SiLU * up, fp16 -> bf16 cast, greedy argmax.  All are tiny at decode batch
+// sizes: they exist to keep the step on the GPU between the big kernels.
+#include "device_utils.hpp"
+#include "launch_common.hpp"
+
+#include <hip/hip_fp16.h>
+#include <math.h>
+
+namespace lg {
+
+__device__ __forceinline__ float bf16_to_f32(unsigned short v) {
+    return __uint_as_float((unsigned)v << 16);
+}
+__device__ __forceinline__ unsigned short f32_to_bf16(float f) {
+    unsigned u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (unsigned short)(u >> 16);
+}
+
+// h[r][:] += y[r][:] (when y != nullptr); out[r][:] = bf16(h * inv_rms * w).
+// One workgroup of 256 threads per row.
+__global__ __launch_bounds__(256) void add_rms_norm_kernel(float* __restrict__ h,
+                                                           const uint16_t* __restrict__ y,
+                                                           const float* __restrict__ w,
+                                                           uint16_t* __restrict__ out, int n,
+                                                           float eps) {
+    const int64_t row = blockIdx.x;
+    float* hr = h + row * n;
+    float sum_sq = 0.0f;
+    for (int j = threadIdx.x; j < n; j += 256) {
+        float v = hr[j];
+        if (y) {
+            v += bf16_to_f32(y[row * n + j]);
+            hr[j] = v;
+        }
+        sum_sq = fmaf(v, v, sum_sq);
+    }
+    __shared__ float part[4];
+    sum_sq = wave_sum(sum_sq);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = sum_sq;
+    __syncthreads();
+    const float total = part[0] + part[1] + part[2] + part[3];
+    const float inv = 1.0f / sqrtf(total / (float)n + eps);
+    for (int j = threadIdx.x; j < n; j += 256) out[row * n + j] = f32_to_bf16(hr[j] * inv * w[j]);
+}
+
+// grid (hq + 2*hkv, total_tokens), 64 threads: thread i rotates elements i and
+// i + d/2 (d = 128).  q heads go to q_out (fp16); k heads, rotated, and v heads,
+// as they are, go to the pools at the token's slot.
+__global__ __launch_bounds__(64) void rope_kv_write_kernel(
+    const uint16_t* __restrict__ qkv, const int32_t* __restrict__ positions,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    const int64_t* __restrict__ slot_mapping, __half* __restrict__ q_out,
+    __half* __restrict__ k_pool, __half* __restrict__ v_pool, int hq, int hkv, int max_pos) {
+    constexpr int D = 128, HALF = 64;
+    const int head = blockIdx.x;
+    const int64_t t = blockIdx.y;
+    const int i = threadIdx.x;
+    const uint16_t* src = qkv + (t * (hq + 2 * hkv) + head) * D;
+    const float x0 = bf16_to_f32(src[i]);
+    const float x1 = bf16_to_f32(src[i + HALF]);
+    if (head < hq + hkv) {
+        int pos = positions[t];
+        pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
+        const float c = cos_t[(int64_t)pos * HALF + i];
+        const float s = sin_t[(int64_t)pos * HALF + i];
+        const float y0 = x0 * c - x1 * s;
+        const float y1 = x0 * s + x1 * c;
+        if (head < hq) {
+            __half* dst = q_out + (t * hq + head) * D;
+            dst[i] = __float2half_rn(y0);
+            dst[i + HALF] = __float2half_rn(y1);
+        } else {
+            const int64_t slot = slot_mapping[t];
+            if (slot < 0) return;
+            __half* dst = k_pool + (slot * hkv + (head - hq)) * D;
+            dst[i] = __float2half_rn(y0);
+            dst[i + HALF] = __float2half_rn(y1);
+        }
+    } else {
+        const int64_t slot = slot_mapping[t];
+        if (slot < 0) return;
+        __half* dst = v_pool + (slot * hkv + (head - hq - hkv)) * D;
+        dst[i] = __float2half_rn(x0);
+        dst[i + HALF] = __float2half_rn(x1);
+    }
+}
+
+// out[t][j] = bf16( silu(gate[t][j]) * up[t][j] ), gate_up = [t][gate(0..inter) | up(0..inter)]
+__global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restrict__ gate_up,
+                                                       uint16_t* __restrict__ out, int inter,
+                                                       int64_t total) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int64_t t = idx / inter;
+    const int64_t j = idx - t * inter;
+    const float g = bf16_to_f32(gate_up[t * 2 * inter + j]);
+    const float u = bf16_to_f32(gate_up[t * 2 * inter + inter + j]);
+    const float sg = g / (1.0f + expf(-g));
+    out[idx] = f32_to_bf16(sg * u);
+}
+
+__global__ __launch_bounds__(256) void cast_f16_bf16_kernel(const __half* __restrict__ in,
+                                                            uint16_t* __restrict__ out,
+                                                            int64_t total) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx < total) out[idx] = f32_to_bf16(__half2float(in[idx]));
+}
+
+// One workgroup per row: first index of the maximum (strict >, ties keep the lower index).
+__global__ __launch_bounds__(256) void greedy_kernel(const float* __restrict__ logits,
+                                                     uint32_t* __restrict__ out, int n) {
+    const int64_t row = blockIdx.x;
+    const float* lr = logits + row * n;
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+    for (int j = threadIdx.x; j < n; j += 256) {
+        const float v = lr[j];
+        if (v > best) {
+            best = v;
+            best_i = j;
+        }
+    }
+    __shared__ float sb[256];
+    __shared__ int si[256];
+    sb[threadIdx.x] = best;
+    si[threadIdx.x] = best_i;
+    __syncthreads();
+    for (int off = 128; off > 0; off >>= 1) {
+        if ((int)threadIdx.x < off) {
+            const float ov = sb[threadIdx.x + off];
+            const int oi = si[threadIdx.x + off];
+            if (ov > sb[threadIdx.x] || (ov == sb[threadIdx.x] && oi < si[threadIdx.x])) {
+                sb[threadIdx.x] = ov;
+                si[threadIdx.x] = oi;
+            }
+        }
+        __syncthreads();
+    }
+    // all -inf (or NaN-only) rows: index 0, like the CPU loop that never updates
+    if (threadIdx.x == 0) out[row] = si[0] == 0x7fffffff ? 0u : (uint32_t)si[0];
+}
+
+}  // namespace lg
+
+extern "C" logismos_status_t logismos_launch_add_rms_norm_bf16(void* h_f32, const void* y_bf16,
+                                                               const void* w_f32, void* out_bf16,
+                                                               int rows, int n, float eps,
+                                                               logismos_stream_t stream) {
+    if (rows <= 0 || n <= 0 || (int64_t)rows * n > (int64_t)INT32_MAX) return hipErrorInvalidValue;
+    if (!h_f32 || !w_f32 || !out_bf16) return hipErrorInvalidValue;
+    lg::add_rms_norm_kernel<<<dim3(rows), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<float*>(h_f32), static_cast<const uint16_t*>(y_bf16),
+        static_cast<const float*>(w_f32), static_cast<uint16_t*>(out_bf16), n, eps);
+    return hipGetLastError();
+}
+
+extern "C" logismos_status_t logismos_launch_rope_kv_write_fp16(
+    const void* qkv_bf16, const int32_t* positions, const void* cos_f32, const void* sin_f32,
+    const int64_t* slot_mapping, void* q_out_f16, void* k_pool_f16, void* v_pool_f16,
+    int total_tokens, int num_q_heads, int num_kv_heads, int head_dim, int max_pos,
+    logismos_stream_t stream) {
+    if (total_tokens < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || max_pos <= 0)
+        return hipErrorInvalidValue;
+    if (head_dim != 128 || total_tokens > 65535) return hipErrorInvalidValue;
+    if ((int64_t)total_tokens * (num_q_heads + 2 * num_kv_heads) * head_dim > (int64_t)INT32_MAX)
+        return hipErrorInvalidValue;
+    if (total_tokens == 0) return hipSuccess;
+    if (!qkv_bf16 || !positions || !cos_f32 || !sin_f32 || !slot_mapping || !q_out_f16 ||
+        !k_pool_f16 || !v_pool_f16)
+        return hipErrorInvalidValue;
+    dim3 grid(num_q_heads + 2 * num_kv_heads, total_tokens);
+    lg::rope_kv_write_kernel<<<grid, dim3(64), 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<const uint16_t*>(qkv_bf16), positions, static_cast<const float*>(cos_f32),
+        static_cast<const float*>(sin_f32), slot_mapping, static_cast<__half*>(q_out_f16),
+        static_cast<__half*>(k_pool_f16), static_cast<__half*>(v_pool_f16), num_q_heads,
+        num_kv_heads, max_pos);
+    return hipGetLastError();
+}
+
+extern "C" logismos_status_t logismos_launch_silu_mul_bf16(const void* gate_up_bf16,
+                                                           void* out_bf16, int rows, int inter,
+                                                           logismos_stream_t stream) {
+    if (rows <= 0 || inter <= 0 || (int64_t)rows * inter * 2 > (int64_t)INT32_MAX)
+        return hipErrorInvalidValue;
+    if (!gate_up_bf16 || !out_bf16) return hipErrorInvalidValue;
+    const int64_t total = (int64_t)rows * inter;
+    lg::silu_mul_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                          static_cast<hipStream_t>(stream)>>>(
+        static_cast<const uint16_t*>(gate_up_bf16), static_cast<uint16_t*>(out_bf16), inter, total);
+    return hipGetLastError();
+}
+
+extern "C" logismos_status_t logismos_launch_cast_f16_bf16(const void* in_f16, void* out_bf16,
+                                                           size_t count,
+                                                           logismos_stream_t stream) {
+    if (count == 0) return hipSuccess;
+    if (!in_f16 || !out_bf16 || count > (size_t)INT32_MAX) return hipErrorInvalidValue;
+    lg::cast_f16_bf16_kernel<<<dim3((unsigned)((count + 255) / 256)), dim3(256), 0,
+                               static_cast<hipStream_t>(stream)>>>(
+        static_cast<const __half*>(in_f16), static_cast<uint16_t*>(out_bf16), (int64_t)count);
+    return hipGetLastError();
+}
+
+extern "C" logismos_status_t logismos_launch_greedy_f32(const void* logits_f32, void* out_u32,
+                                                        int rows, int n,
+                                                        logismos_stream_t stream) {
+    if (rows <= 0 || n <= 0 || (int64_t)rows * n > (int64_t)INT32_MAX) return hipErrorInvalidValue;
+    if (!logits_f32 || !out_u32) return hipErrorInvalidValue;
+    lg::greedy_kernel<<<dim3(rows), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<const float*>(logits_f32), static_cast<uint32_t*>(out_u32), n);
+    return hipGetLastError();
+}

@@ -57,6 +57,14 @@ _SIGNATURES = {
         (C.c_uint32, [_vp] * 8 + [_i] * 9 + [_f, _i, _vp]),
     "logismos_launch_paged_attn_varlen_fp16_phases":
         (C.c_uint32, [_vp] * 8 + [_i] * 9 + [_f, _i, _i, _vp]),
+    "logismos_check_pack_ragged_shape": (C.c_uint32, [_i, _i, _i, C.c_char_p, _sz]),
+    "logismos_launch_pack_ragged": (C.c_uint32, [_vp] * 6 + [_i, _i, _i, _vp]),
+    "logismos_launch_kv_write_fp16": (C.c_uint32, [_vp] * 5 + [_i, _i, _i, _vp]),
+    "logismos_launch_add_rms_norm_bf16": (C.c_uint32, [_vp] * 4 + [_i, _i, _f, _vp]),
+    "logismos_launch_rope_kv_write_fp16": (C.c_uint32, [_vp] * 8 + [_i] * 5 + [_vp]),
+    "logismos_launch_silu_mul_bf16": (C.c_uint32, [_vp, _vp, _i, _i, _vp]),
+    "logismos_launch_cast_f16_bf16": (C.c_uint32, [_vp, _vp, _sz, _vp]),
+    "logismos_launch_greedy_f32": (C.c_uint32, [_vp, _vp, _i, _i, _vp]),
     "logismos_launch_probe_copy": (C.c_uint32, [_vp, _vp, _sz, _vp]),
     "logismos_launch_probe_read": (C.c_uint32, [_vp, _vp, _sz, _vp]),
 }
@@ -176,3 +184,48 @@ def launch_probe_copy(src, dst, nbytes: int, stream=None) -> None:
 def launch_probe_read(src, sink, nbytes: int, stream=None) -> None:
     _status("probe_read", library().logismos_launch_probe_read(_ptr(src), _ptr(sink), nbytes,
                                                                _raw(stream)))
+
+
+def launch_pack_ragged(new_tokens, prior_ctx, block_tables, cu_seqlens, slot_mapping, context_lens,
+                       num_seqs: int, block_size: int, max_blocks: int, stream=None) -> None:
+    _guard("pack_ragged", library().logismos_check_pack_ragged_shape, num_seqs, block_size,
+           max_blocks)
+    _status("pack_ragged", library().logismos_launch_pack_ragged(
+        _ptr(new_tokens), _ptr(prior_ctx), _ptr(block_tables), _ptr(cu_seqlens),
+        _ptr(slot_mapping), _ptr(context_lens), num_seqs, block_size, max_blocks, _raw(stream)))
+
+
+def launch_kv_write_fp16(k_new, v_new, k_pool, v_pool, slot_mapping, total_tokens: int,
+                         num_kv_heads: int, head_dim: int, stream=None) -> None:
+    _status("kv_write_fp16", library().logismos_launch_kv_write_fp16(
+        _ptr(k_new), _ptr(v_new), _ptr(k_pool), _ptr(v_pool), _ptr(slot_mapping), total_tokens,
+        num_kv_heads, head_dim, _raw(stream)))
+
+
+def launch_add_rms_norm_bf16(h, y, w, out, rows: int, n: int, eps: float, stream=None) -> None:
+    _status("add_rms_norm_bf16", library().logismos_launch_add_rms_norm_bf16(
+        _ptr(h), _ptr(y) if y is not None else None, _ptr(w), _ptr(out), rows, n, float(eps),
+        _raw(stream)))
+
+
+def launch_rope_kv_write_fp16(qkv, positions, cos, sin, slot_mapping, q_out, k_pool, v_pool,
+                              total_tokens: int, hq: int, hkv: int, head_dim: int, max_pos: int,
+                              stream=None) -> None:
+    _status("rope_kv_write_fp16", library().logismos_launch_rope_kv_write_fp16(
+        _ptr(qkv), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping), _ptr(q_out),
+        _ptr(k_pool), _ptr(v_pool), total_tokens, hq, hkv, head_dim, max_pos, _raw(stream)))
+
+
+def launch_silu_mul_bf16(gate_up, out, rows: int, inter: int, stream=None) -> None:
+    _status("silu_mul_bf16", library().logismos_launch_silu_mul_bf16(
+        _ptr(gate_up), _ptr(out), rows, inter, _raw(stream)))
+
+
+def launch_cast_f16_bf16(src, dst, count: int, stream=None) -> None:
+    _status("cast_f16_bf16", library().logismos_launch_cast_f16_bf16(
+        _ptr(src), _ptr(dst), count, _raw(stream)))
+
+
+def launch_greedy_f32(logits, out, rows: int, n: int, stream=None) -> None:
+    _status("greedy_f32", library().logismos_launch_greedy_f32(
+        _ptr(logits), _ptr(out), rows, n, _raw(stream)))

@@ -1,0 +1,95 @@
+"""GPU parity of the small decode-step operators vs the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+
+import oracle as O
+from oracle import decode_step as OS
+from logismos_amd import hip, kernels
+from tests.gpu_harness import assert_parity
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("rows,n,with_y", [(1, 128, False), (5, 1536, True), (32, 4096, True),
+                                           (3, 1000, True)])
+def test_add_rms_norm(rows, n, with_y):
+    rng = np.random.default_rng(rows * n)
+    h = rng.standard_normal((rows, n), np.float32)
+    y = O.f32_to_bf16_bits(rng.standard_normal((rows, n), np.float32)) if with_y else None
+    w = (1 + 0.02 * rng.standard_normal(n)).astype(np.float32)
+    d_h = hip.DeviceBuffer.from_numpy(h)
+    d_y = hip.DeviceBuffer.from_numpy(y) if with_y else None
+    d_out = hip.DeviceBuffer(rows * n * 2)
+    kernels.launch_add_rms_norm_bf16(d_h, d_y, hip.DeviceBuffer.from_numpy(w), d_out, rows, n, 1e-6)
+    hip.synchronize()
+    h_ref = h.copy()
+    want = OS.add_rms_norm_bf16(h_ref, y, w, 1e-6)
+    # the residual add is one fp32 add: bit-exact
+    assert np.array_equal(d_h.to_numpy(np.float32, (rows, n)), h_ref)
+    got = O.bf16_bits_to_f32(d_out.to_numpy(np.uint16, (rows, n)))
+    assert_parity(got, O.bf16_bits_to_f32(want), max_abs=2e-3, max_rel=1e-2, what="add_rms_norm")
+
+
+def test_rope_kv_write_matches_oracle_and_reference_table():
+    rng = np.random.default_rng(21)
+    t, hq, hkv, d, bs, nblk, max_pos = 7, 8, 2, 128, 16, 12, 4096
+    qkv = O.f32_to_bf16_bits(rng.standard_normal((t, (hq + 2 * hkv) * d), np.float32))
+    positions = np.array([0, 1, 17, 4095, 300, 5000, 2], np.int32)  # 5000 clamps to 4095
+    slots = rng.permutation(nblk * bs)[:t].astype(np.int64)
+    slots[3] = -1
+    cos, sin = O.build_rope_table_f32(max_pos, d, 1_000_000.0)
+    k_pool = rng.standard_normal((nblk * bs, hkv * d), np.float32).astype(np.float16)
+    v_pool = rng.standard_normal((nblk * bs, hkv * d), np.float32).astype(np.float16)
+    d_kp, d_vp = hip.DeviceBuffer.from_numpy(k_pool), hip.DeviceBuffer.from_numpy(v_pool)
+    d_q = hip.DeviceBuffer(t * hq * d * 2)
+    kernels.launch_rope_kv_write_fp16(
+        hip.DeviceBuffer.from_numpy(qkv), hip.DeviceBuffer.from_numpy(positions),
+        hip.DeviceBuffer.from_numpy(cos), hip.DeviceBuffer.from_numpy(sin),
+        hip.DeviceBuffer.from_numpy(slots), d_q, d_kp, d_vp, t, hq, hkv, d, max_pos)
+    hip.synchronize()
+    q_want = OS.rope_kv_write(qkv, positions, cos, sin, slots, k_pool, v_pool, hq, hkv, d)
+    q_got = d_q.to_numpy(np.float16, (t, hq, d))
+    # fp32 rotate of two products then one fp16 rounding: allow 1 ulp (fma contraction)
+    assert_parity(q_got, q_want, max_abs=1e-3, max_rel=2e-3, what="rope q")
+    assert_parity(d_kp.to_numpy(np.float16, k_pool.shape), k_pool, max_abs=1e-3, max_rel=2e-3,
+                  what="rope k pool")
+    # v is copied unrotated: bit-exact (bf16 -> fp16 is exact or the same rounding)
+    assert np.array_equal(d_vp.to_numpy(np.float16, v_pool.shape).view(np.uint16),
+                          v_pool.view(np.uint16))
+    # position 0 is the identity rotation
+    x0 = O.bf16_bits_to_f32(qkv[0]).reshape(hq + 2 * hkv, d)[:hq]
+    assert np.array_equal(q_got[0], x0.astype(np.float16))
+
+
+def test_silu_mul_and_cast():
+    rng = np.random.default_rng(22)
+    rows, inter = 5, 1000
+    gu = O.f32_to_bf16_bits(rng.standard_normal((rows, 2 * inter), np.float32) * 3)
+    d_out = hip.DeviceBuffer(rows * inter * 2)
+    kernels.launch_silu_mul_bf16(hip.DeviceBuffer.from_numpy(gu), d_out, rows, inter)
+    hip.synchronize()
+    got = O.bf16_bits_to_f32(d_out.to_numpy(np.uint16, (rows, inter)))
+    assert_parity(got, O.bf16_bits_to_f32(OS.silu_mul_bf16(gu, inter)), what="silu_mul")
+    a = rng.standard_normal(777, np.float32).astype(np.float16)
+    d_b = hip.DeviceBuffer(777 * 2)
+    kernels.launch_cast_f16_bf16(hip.DeviceBuffer.from_numpy(a), d_b, 777)
+    hip.synchronize()
+    assert np.array_equal(d_b.to_numpy(np.uint16, (777,)), OS.cast_f16_bf16(a))
+
+
+def test_greedy_first_maximum_wins():
+    """crates/decode/src/lib.rs:90-92 plus a vocabulary-sized row"""
+    rng = np.random.default_rng(23)
+    rows, n = 4, 151936
+    logits = rng.standard_normal((rows, n), np.float32)
+    logits[0, :3] = [0.0, 2.0, 2.0]
+    logits[0, 3:] = -1.0
+    logits[1, [5, 70000, 150000]] = 9.0       # three equal maxima: index 5
+    logits[2, :] = -np.inf                     # all -inf: index 0
+    d_out = hip.DeviceBuffer(rows * 4)
+    kernels.launch_greedy_f32(hip.DeviceBuffer.from_numpy(logits), d_out, rows, n)
+    hip.synchronize()
+    got = d_out.to_numpy(np.uint32, (rows,))
+    want = [O.greedy(logits[r]) for r in range(rows)]
+    assert got.tolist() == want
+    assert got[0] == 1 and got[1] == 5 and got[2] == 0
