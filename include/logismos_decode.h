@@ -287,6 +287,64 @@ logismos_status_t logismos_launch_greedy_f32(const void* logits_f32, void* out_u
                                              logismos_stream_t stream);
 
 /* ------------------------------------------------------------------------
+ * Decode step: one new token for each of num_seqs <= 32 live sequences through
+ * num_layers pre-norm layers (`StellaLayer::forward` order,
+ * crates/encoders/src/stella.rs:190-206; attention and SwiGLU arithmetic of
+ * crates/transformers/src/{attention,mlp}.rs) with Q4G128 weights and the paged
+ * fp16 KV cache.  The reference has no decoder yet (crates/decoders/src/lib.rs).
+ *
+ * Per layer: h += previous projection; xn = RMSNorm(h); qkv = xn.Wqkv^T;
+ * RoPE(q,k), K/V appended at slot_mapping; paged attention; h += attn.Wo^T;
+ * xn = RMSNorm(h); act = silu(xn.Wgate^T) * (xn.Wup^T); down projection.
+ * Wqkv stacks the q, k and v projections (rows: hq*128, hkv*128, hkv*128),
+ * Wgate_up stacks gate and up (intermediate rows each).  After the last layer
+ * out = bf16(RMSNorm(h) * final_norm_w).  All launches are asynchronous on
+ * `stream`; `workspace` needs logismos_decode_step_workspace_bytes() bytes,
+ * 256-byte aligned, contents don't matter.
+ * ------------------------------------------------------------------------ */
+typedef struct {
+    const void* qw;    /* uint8 [N][K/2] */
+    const void* scale; /* fp16  [N][K/128] */
+    const void* zero;  /* fp16  [N][K/128] */
+} logismos_q4_weight_t;
+
+typedef struct {
+    int num_layers, hidden, num_q_heads, num_kv_heads, head_dim, intermediate;
+    float rms_eps;
+    int block_size, max_blocks_per_seq, max_pos;
+} logismos_decode_config_t;
+
+typedef struct {
+    const void* norm1_w_f32; /* [hidden] */
+    const void* norm2_w_f32; /* [hidden] */
+    logismos_q4_weight_t qkv, o, gate_up, down;
+    void* k_pool_f16; /* this layer's paged pools */
+    void* v_pool_f16;
+} logismos_decode_layer_t;
+
+typedef struct {
+    void* hidden_f32;             /* [num_seqs][hidden], in: embeddings, out: last residual */
+    void* out_bf16;               /* [num_seqs][hidden] */
+    const void* final_norm_w_f32; /* [hidden] */
+    const int32_t* block_tables;  /* [num_seqs][max_blocks_per_seq] */
+    const int32_t* cu_seqlens;    /* [num_seqs+1] = 0,1,2,... */
+    const int32_t* context_lens;  /* [num_seqs], including the new token */
+    const int32_t* positions;     /* [num_seqs] = context_lens - 1 */
+    const int64_t* slot_mapping;  /* [num_seqs] */
+    const void* rope_cos_f32;     /* [max_pos][64] */
+    const void* rope_sin_f32;
+    int num_seqs;
+    int num_splits;
+} logismos_decode_batch_t;
+
+size_t logismos_decode_step_workspace_bytes(const logismos_decode_config_t* cfg, int num_seqs,
+                                            int num_splits);
+logismos_status_t logismos_launch_decode_step(const logismos_decode_config_t* cfg,
+                                              const logismos_decode_layer_t* layers,
+                                              const logismos_decode_batch_t* batch, void* workspace,
+                                              logismos_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * Memory-system probes (measurement aids; the reference has no counterpart,
  * its only timing helper is the hipEvent pair of
  * crates/kernels/examples/gemm_bench.rs:120-128).  A plain copy and a plain

@@ -1,0 +1,120 @@
+// One continuous-batching decode step (one new token per live sequence) as a
+// sequence of asynchronous launches on one stream: the executor the reference
+// does not have yet (crates/decoders/src/lib.rs is a scaffold), written against
+// the launchers of this library only.  Nothing is allocated, nothing
+// synchronises; a caller may capture the whole step into a HIP graph.
+#include "launch_common.hpp"
+
+#include <math.h>
+
+namespace {
+
+struct Workspace {
+    char* xn;        // bf16 [B][hidden]
+    char* qkv;       // bf16 [B][(hq+2hkv)*d]
+    char* q;         // f16  [B][hq*d]
+    char* attn;      // f16  [B][hq*d]
+    char* attn_b;    // bf16 [B][hq*d]
+    char* proj;      // bf16 [B][hidden]      (o projection, then down projection)
+    char* gate_up;   // bf16 [B][2*inter]
+    char* act;       // bf16 [B][inter]
+    char* attn_ws;   // split-K workspace
+    size_t total;
+};
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+Workspace carve(const logismos_decode_config_t& c, int b, int num_splits, char* base) {
+    Workspace w{};
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        char* p = base ? base + off : nullptr;
+        off += align256(bytes);
+        return p;
+    };
+    const size_t qd = (size_t)c.num_q_heads * c.head_dim;
+    const size_t kvd = (size_t)c.num_kv_heads * c.head_dim;
+    w.xn = take((size_t)b * c.hidden * 2);
+    w.qkv = take((size_t)b * (qd + 2 * kvd) * 2);
+    w.q = take((size_t)b * qd * 2);
+    w.attn = take((size_t)b * qd * 2);
+    w.attn_b = take((size_t)b * qd * 2);
+    w.proj = take((size_t)b * c.hidden * 2);
+    w.gate_up = take((size_t)b * 2 * c.intermediate * 2);
+    w.act = take((size_t)b * c.intermediate * 2);
+    w.attn_ws = take(logismos_paged_attn_workspace_bytes(b, c.num_q_heads, c.head_dim, num_splits));
+    w.total = off;
+    return w;
+}
+
+bool config_ok(const logismos_decode_config_t* c, int b) {
+    if (!c || b <= 0 || b > 32) return false;
+    if (c->num_layers <= 0 || c->hidden <= 0 || c->intermediate <= 0 || c->max_pos <= 0)
+        return false;
+    if (c->head_dim != 128 || c->num_q_heads <= 0 || c->num_kv_heads <= 0) return false;
+    if (c->hidden % 128 != 0 || c->intermediate % 128 != 0) return false;
+    if (((int64_t)c->num_q_heads * c->head_dim) % 128 != 0) return false;
+    return true;
+}
+
+}  // namespace
+
+extern "C" size_t logismos_decode_step_workspace_bytes(const logismos_decode_config_t* cfg,
+                                                       int num_seqs, int num_splits) {
+    if (!config_ok(cfg, num_seqs) || num_splits <= 0) return 0;
+    return carve(*cfg, num_seqs, num_splits, nullptr).total;
+}
+
+#define LG_TRY(call)                                  \
+    do {                                              \
+        logismos_status_t st__ = (call);              \
+        if (st__ != 0) return st__;                   \
+    } while (0)
+
+extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_config_t* cfg,
+                                                         const logismos_decode_layer_t* layers,
+                                                         const logismos_decode_batch_t* batch,
+                                                         void* workspace,
+                                                         logismos_stream_t stream) {
+    if (!cfg || !layers || !batch || !workspace) return hipErrorInvalidValue;
+    const int b = batch->num_seqs;
+    if (!config_ok(cfg, b) || batch->num_splits <= 0) return hipErrorInvalidValue;
+    if (reinterpret_cast<uintptr_t>(workspace) & 255u) return hipErrorInvalidValue;
+    const logismos_decode_config_t& c = *cfg;
+    const Workspace w = carve(c, b, batch->num_splits, static_cast<char*>(workspace));
+    const int qd = c.num_q_heads * c.head_dim;
+    const int kvd = c.num_kv_heads * c.head_dim;
+    const float scale = 1.0f / sqrtf((float)c.head_dim);
+
+    const void* residual = nullptr;  // what the next add_rms_norm folds into h
+    for (int l = 0; l < c.num_layers; ++l) {
+        const logismos_decode_layer_t& L = layers[l];
+        LG_TRY(logismos_launch_add_rms_norm_bf16(batch->hidden_f32, residual, L.norm1_w_f32, w.xn, b,
+                                                 c.hidden, c.rms_eps, stream));
+        LG_TRY(logismos_launch_qgemm_q4g128_bf16(w.xn, L.qkv.qw, L.qkv.scale, L.qkv.zero, w.qkv, b,
+                                                 qd + 2 * kvd, c.hidden, stream));
+        LG_TRY(logismos_launch_rope_kv_write_fp16(w.qkv, batch->positions, batch->rope_cos_f32,
+                                                  batch->rope_sin_f32, batch->slot_mapping, w.q,
+                                                  L.k_pool_f16, L.v_pool_f16, b, c.num_q_heads,
+                                                  c.num_kv_heads, c.head_dim, c.max_pos, stream));
+        LG_TRY(logismos_launch_paged_attn_varlen_fp16(
+            w.q, L.k_pool_f16, L.v_pool_f16, batch->block_tables, batch->cu_seqlens,
+            batch->context_lens, w.attn, w.attn_ws, b, b, 1, c.num_q_heads, c.num_kv_heads,
+            c.head_dim, c.block_size, c.max_blocks_per_seq, batch->num_splits, scale, 1, stream));
+        LG_TRY(logismos_launch_cast_f16_bf16(w.attn, w.attn_b, (size_t)b * qd, stream));
+        LG_TRY(logismos_launch_qgemm_q4g128_bf16(w.attn_b, L.o.qw, L.o.scale, L.o.zero, w.proj, b,
+                                                 c.hidden, qd, stream));
+        LG_TRY(logismos_launch_add_rms_norm_bf16(batch->hidden_f32, w.proj, L.norm2_w_f32, w.xn, b,
+                                                 c.hidden, c.rms_eps, stream));
+        LG_TRY(logismos_launch_qgemm_q4g128_bf16(w.xn, L.gate_up.qw, L.gate_up.scale,
+                                                 L.gate_up.zero, w.gate_up, b, 2 * c.intermediate,
+                                                 c.hidden, stream));
+        LG_TRY(logismos_launch_silu_mul_bf16(w.gate_up, w.act, b, c.intermediate, stream));
+        LG_TRY(logismos_launch_qgemm_q4g128_bf16(w.act, L.down.qw, L.down.scale, L.down.zero, w.proj,
+                                                 b, c.hidden, c.intermediate, stream));
+        residual = w.proj;
+    }
+    LG_TRY(logismos_launch_add_rms_norm_bf16(batch->hidden_f32, residual, batch->final_norm_w_f32,
+                                             batch->out_bf16, b, c.hidden, c.rms_eps, stream));
+    return 0;
+}

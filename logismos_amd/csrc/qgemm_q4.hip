@@ -446,10 +446,7 @@ static hipError_t launch_mfma(const void* x, const void* qw, const void* scale, 
                               void* y, int b, int n, int k, hipStream_t stream) {
     const int tiles = (n + 15) / 16;
     const int cus = device_cu_count();
-    const int t = (tiles + cus - 1) / cus;  // row tiles per workgroup
-    if constexpr (BT == 2) {  // one group per wave: registers allow six tiles
-        if (t >= 6) return launch_mfma_t<BT, GW, 6>(x, qw, scale, zero, y, b, n, k, stream);
-    }
+    const int t = (tiles + cus - 1) / cus;  // row tiles per workgroup (LDS slots cap it at 3)
     if (t >= 3) return launch_mfma_t<BT, GW, 3>(x, qw, scale, zero, y, b, n, k, stream);
     if (t == 2) return launch_mfma_t<BT, GW, 2>(x, qw, scale, zero, y, b, n, k, stream);
     return launch_mfma_t<BT, GW, 1>(x, qw, scale, zero, y, b, n, k, stream);

@@ -65,11 +65,36 @@ _SIGNATURES = {
     "logismos_launch_silu_mul_bf16": (C.c_uint32, [_vp, _vp, _i, _i, _vp]),
     "logismos_launch_cast_f16_bf16": (C.c_uint32, [_vp, _vp, _sz, _vp]),
     "logismos_launch_greedy_f32": (C.c_uint32, [_vp, _vp, _i, _i, _vp]),
+    "logismos_decode_step_workspace_bytes": (_sz, [_vp, _i, _i]),
+    "logismos_launch_decode_step": (C.c_uint32, [_vp, _vp, _vp, _vp, _vp]),
     "logismos_launch_probe_copy": (C.c_uint32, [_vp, _vp, _sz, _vp]),
     "logismos_launch_probe_read": (C.c_uint32, [_vp, _vp, _sz, _vp]),
 }
 
 ATTN_PHASE_DECODE, ATTN_PHASE_PREFILL, ATTN_PHASE_MERGE, ATTN_PHASE_ALL = 1, 2, 4, 7
+
+
+class Q4Weight(C.Structure):
+    _fields_ = [("qw", _vp), ("scale", _vp), ("zero", _vp)]
+
+
+class DecodeConfig(C.Structure):
+    _fields_ = [("num_layers", _i), ("hidden", _i), ("num_q_heads", _i), ("num_kv_heads", _i),
+                ("head_dim", _i), ("intermediate", _i), ("rms_eps", _f), ("block_size", _i),
+                ("max_blocks_per_seq", _i), ("max_pos", _i)]
+
+
+class DecodeLayer(C.Structure):
+    _fields_ = [("norm1_w_f32", _vp), ("norm2_w_f32", _vp), ("qkv", Q4Weight), ("o", Q4Weight),
+                ("gate_up", Q4Weight), ("down", Q4Weight), ("k_pool_f16", _vp),
+                ("v_pool_f16", _vp)]
+
+
+class DecodeBatch(C.Structure):
+    _fields_ = [("hidden_f32", _vp), ("out_bf16", _vp), ("final_norm_w_f32", _vp),
+                ("block_tables", _vp), ("cu_seqlens", _vp), ("context_lens", _vp),
+                ("positions", _vp), ("slot_mapping", _vp), ("rope_cos_f32", _vp),
+                ("rope_sin_f32", _vp), ("num_seqs", _i), ("num_splits", _i)]
 
 
 def library() -> C.CDLL:
@@ -229,3 +254,13 @@ def launch_cast_f16_bf16(src, dst, count: int, stream=None) -> None:
 def launch_greedy_f32(logits, out, rows: int, n: int, stream=None) -> None:
     _status("greedy_f32", library().logismos_launch_greedy_f32(
         _ptr(logits), _ptr(out), rows, n, _raw(stream)))
+
+
+def decode_step_workspace_bytes(cfg: DecodeConfig, num_seqs: int, num_splits: int) -> int:
+    return library().logismos_decode_step_workspace_bytes(C.byref(cfg), num_seqs, num_splits)
+
+
+def launch_decode_step(cfg: DecodeConfig, layers, batch: DecodeBatch, workspace, stream=None) -> None:
+    """`layers` is a ctypes array of DecodeLayer (host memory)."""
+    _status("decode_step", library().logismos_launch_decode_step(
+        C.byref(cfg), C.cast(layers, _vp), C.byref(batch), _ptr(workspace), _raw(stream)))

@@ -80,6 +80,98 @@ class QgemmQ4Runner:
         return self.y.to_numpy(np.uint16, (self.b, self.n))
 
 
+def _val(p):
+    return p.ptr.value if isinstance(p, hip.DeviceBuffer) else p
+
+
+class DecodeStepRunner:
+    """Uploads a decode-step problem (see oracle/decode_step.py for the dict layout) and runs
+    logismos_launch_decode_step.  `layer_bufs` keeps the device buffers alive."""
+
+    def __init__(self, cfg, layers, batch, num_splits=None, stream=None, share_layer_data=False):
+        self.cfg_d, self.stream = cfg, stream
+        b = batch["h"].shape[0]
+        self.b = b
+        max_blocks = batch["block_tables"].shape[1]
+        self.num_splits = num_splits or kernels.paged_attn_num_splits(b, cfg["hkv"],
+                                                                      cfg["block_size"], max_blocks)
+        half = cfg["d"] // 2
+        self.cfg = kernels.DecodeConfig(len(layers), cfg["hidden"], cfg["hq"], cfg["hkv"], cfg["d"],
+                                        cfg["inter"], cfg["eps"], cfg["block_size"], max_blocks,
+                                        batch["cos"].size // half)
+        up = hip.DeviceBuffer.from_numpy
+        self.keep = []
+
+        def w3(t):
+            bufs = [up(np.ascontiguousarray(t[0])), up(np.ascontiguousarray(t[1]).view(np.uint16)),
+                    up(np.ascontiguousarray(t[2]).view(np.uint16))]
+            self.keep += bufs
+            return kernels.Q4Weight(*[_val(x) for x in bufs])
+
+        self.layers = (kernels.DecodeLayer * len(layers))()
+        self.pools = []
+        first = None
+        for i, L in enumerate(layers):
+            if share_layer_data and first is not None:
+                # same weights, own pools (device-to-device copies): timing runs only
+                src = first
+                kp, vp = hip.DeviceBuffer(src[6].nbytes), hip.DeviceBuffer(src[7].nbytes)
+                kp.copy_from_device(src[6], src[6].nbytes)
+                vp.copy_from_device(src[7], src[7].nbytes)
+                q4 = []
+                for j in range(2, 6):
+                    trio = []
+                    for buf in src[j]:
+                        nb = hip.DeviceBuffer(buf.nbytes)
+                        nb.copy_from_device(buf, buf.nbytes)
+                        trio.append(nb)
+                    q4.append(trio)
+                n1, n2 = src[0], src[1]
+            else:
+                n1, n2 = up(L["norm1"].astype(np.float32)), up(L["norm2"].astype(np.float32))
+                q4 = []
+                for name in ("qkv", "o", "gate_up", "down"):
+                    t = L[name]
+                    q4.append([up(np.ascontiguousarray(t[0])),
+                               up(np.ascontiguousarray(t[1]).view(np.uint16)),
+                               up(np.ascontiguousarray(t[2]).view(np.uint16))])
+                kp, vp = up(L["k_pool"]), up(L["v_pool"])
+                if first is None:
+                    first = (n1, n2, q4[0], q4[1], q4[2], q4[3], kp, vp)
+            self.keep += [n1, n2, kp, vp] + [x for t in q4 for x in t]
+            self.pools.append((kp, vp))
+            lay = self.layers[i]
+            lay.norm1_w_f32, lay.norm2_w_f32 = _val(n1), _val(n2)
+            for name, trio in zip(("qkv", "o", "gate_up", "down"), q4):
+                setattr(lay, name, kernels.Q4Weight(*[_val(x) for x in trio]))
+            lay.k_pool_f16, lay.v_pool_f16 = _val(kp), _val(vp)
+
+        self.h = up(batch["h"].astype(np.float32))
+        self.out = hip.DeviceBuffer(b * cfg["hidden"] * 2)
+        self.out.fill(0xFF)
+        names = ("block_tables", "cu_seqlens", "context_lens", "positions")
+        self.idx = {n: up(np.ascontiguousarray(batch[n], np.int32)) for n in names}
+        self.slots = up(np.ascontiguousarray(batch["slots"], np.int64))
+        self.cos, self.sin = up(batch["cos"]), up(batch["sin"])
+        self.fnorm = up(batch["final_norm"].astype(np.float32))
+        self.batch = kernels.DecodeBatch(
+            _val(self.h), _val(self.out), _val(self.fnorm), _val(self.idx["block_tables"]),
+            _val(self.idx["cu_seqlens"]), _val(self.idx["context_lens"]),
+            _val(self.idx["positions"]), _val(self.slots), _val(self.cos), _val(self.sin), b,
+            self.num_splits)
+        ws = kernels.decode_step_workspace_bytes(self.cfg, b, self.num_splits)
+        assert ws > 0
+        self.ws = hip.DeviceBuffer(ws)
+        self.ws.fill(0xFF)
+
+    def launch(self):
+        kernels.launch_decode_step(self.cfg, self.layers, self.batch, self.ws, self.stream)
+
+    def result_bits(self) -> np.ndarray:
+        (self.stream.synchronize() if self.stream else hip.synchronize())
+        return self.out.to_numpy(np.uint16, (self.b, self.cfg_d["hidden"]))
+
+
 def assert_parity(got, want, max_abs=2e-3, max_rel=1e-2, what=""):
     """Tolerance of the decode path for fp16/bf16 outputs with fp32 accumulation:
     every element within max_abs OR within max_rel of the oracle (relative error

@@ -88,3 +88,45 @@ def config3(seed=SEED + 3, n=12288, k=4096, max_batch=16):
 
 def qgemm_q4_algorithmic_bytes(b, n, k) -> int:
     return n * k // 2 + n * (k // 128) * 4 + b * k * 2 + b * n * 2
+
+
+def decode_step_problem(rng, num_layers, hidden, hq, hkv, inter, ctx, d=128, block_size=16,
+                        max_pos=None, eps=1e-6, theta=1e6, random_nibbles=False):
+    """A decode-step problem: `ctx[s]` is the context of sequence s INCLUDING the new token.
+    Weights ~N(0,0.02) quantised to Q4G128 by the oracle (or raw random nibbles/scales when
+    random_nibbles, for timing-only runs), RMSNorm gains 1+N(0,0.02), RoPE theta 1e6."""
+    import oracle as O
+    ctx = np.asarray(ctx, np.int32)
+    b = len(ctx)
+    max_pos = max_pos or int(ctx.max()) + 1
+
+    def q4(n, k):
+        if random_nibbles:
+            qw = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+            s = (rng.random((n, k // 128), np.float32) * 0.004 + 0.004).astype(np.float16)
+            z = (rng.random((n, k // 128), np.float32) * 2 + 6.5).astype(np.float16)
+            return qw, s, z
+        w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
+        return O.quantize_q4g128(w, n, k)
+
+    base = paged_case(rng, np.ones(b, np.int32), ctx - 1, hq=hq, hkv=hkv, d=d,
+                      block_size=block_size, spare_frac=0.05)
+    layers = []
+    for _ in range(num_layers):
+        rows = base["k_pool"].shape[0]
+        layers.append(dict(
+            norm1=(1 + 0.02 * rng.standard_normal(hidden)).astype(np.float32),
+            norm2=(1 + 0.02 * rng.standard_normal(hidden)).astype(np.float32),
+            qkv=q4((hq + 2 * hkv) * d, hidden), o=q4(hidden, hq * d),
+            gate_up=q4(2 * inter, hidden), down=q4(hidden, inter),
+            k_pool=rng.standard_normal((rows, hkv * d), np.float32).astype(np.float16),
+            v_pool=rng.standard_normal((rows, hkv * d), np.float32).astype(np.float16)))
+    cos, sin = O.build_rope_table_f32(max_pos, d, theta)
+    cu, slots, ctx_lens, _ = O.pack_ragged(np.ones(b, np.int32), ctx - 1, base["block_tables"],
+                                           block_size)
+    batch = dict(h=rng.standard_normal((b, hidden), np.float32),
+                 block_tables=base["block_tables"], cu_seqlens=cu, context_lens=ctx_lens,
+                 positions=(ctx - 1).astype(np.int32), slots=slots, cos=cos, sin=sin,
+                 final_norm=(1 + 0.02 * rng.standard_normal(hidden)).astype(np.float32))
+    cfg = dict(hidden=hidden, hq=hq, hkv=hkv, d=d, inter=inter, eps=eps, block_size=block_size)
+    return cfg, layers, batch
