@@ -3,12 +3,14 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
-A step is one pass of the hot path over one batch of synthetic input that is
-already resident in HBM.  Prints ONE JSON line.  `value` is algorithmic bytes
-of a step / wall time of a step (GB/s); `roofline` prices the dominant kernel
-alone (HIP events around back-to-back launches of only that kernel on the
-launch stream); `cpu_baseline` is the CPU oracle timed on this box's host
-cores on a bounded sample of the same workload.
+A step is one continuous-batching decode step (config 5 of the baseline: 32
+live sequences, Qwen3-8B-style geometry) over synthetic inputs already resident
+in HBM.  Prints ONE JSON line.  `value` is decode tokens per second;
+`roofline` prices the dominant kernel alone (HIP events around back-to-back
+launches of only the paged-attention decode kernel on the launch stream);
+`cpu_baseline` is the CPU oracle timed on this box's host cores on a bounded
+sample of the same workload.  The per-kernel legs (configs 1-3) are reported in
+the same line under their own keys.
 
 Cold-HBM timing: the KV pools (or weights) are replicated so that consecutive
 steps touch different memory and the replicas together exceed twice the
@@ -207,12 +209,172 @@ def bench_qgemv_q8(args):
             "cpu_baseline_GBps": round(algo * reps / el / 1e9, 2), "cpu_cores": cores}
 
 
+def bench_q4(args):
+    """Config 3: Q4G128 12288x4096 at batch 1..16 (cold weights)."""
+    import oracle as O
+    rng = np.random.default_rng(workloads.SEED + 3)
+    n, k = 12288, 4096
+    qw = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+    s = (rng.random((n, k // 128), np.float32) * 0.004 + 0.004).astype(np.float16)
+    z = (rng.random((n, k // 128), np.float32) * 2 + 6.5).astype(np.float16)
+    x = O.f32_to_bf16_bits(rng.standard_normal((16, k), np.float32))
+    stream = hip.Stream()
+    out = {}
+    from tests.gpu_harness import QgemmQ4Runner
+    for b in (1, 2, 4, 8, 16):
+        r = QgemmQ4Runner(x[:b], qw, s, z, b, n, k, stream=stream)
+        copies = max(2, -(-COLD_BYTES // qw.nbytes))
+        qws = replicate(r.qw, copies)
+        algo = workloads.qgemm_q4_algorithmic_bytes(b, n, k)
+        ms, _, _ = time_launches(stream, [(lambda q=q: r.launch(qw=q)) for q in qws], args.steps,
+                                 args.warmup)
+        out[f"b{b}"] = {"us": round(ms * 1e3, 2), "GBps": round(algo / ms / 1e6, 1),
+                        "kernel": "gemv" if b <= 2 else "mfma"}
+        del r, qws
+    return {"workload": "config 3: Q4G128 GEMV/GEMM 12288x4096, x bf16, cold weights", **out}
+
+
+def bench_decode_step(args):
+    """Config 5: full decode step, Qwen3-8B-style geometry, 32 live sequences."""
+    import oracle as O
+    from oracle import decode_step as OS
+    from tests.gpu_harness import DecodeStepRunner
+    rng = np.random.default_rng(workloads.SEED + 5)
+    S, L, hidden, hq, hkv, inter, bs = 32, 36, 4096, 32, 8, 12288, 16
+    steps, warmup = args.steps_c5, args.warmup_c5
+    total_steps = steps + warmup + 2
+    ctx0 = rng.integers(256, 8193, size=S).astype(np.int64)
+    # per-step contexts: every sequence grows by one token per step; each step one sequence
+    # finishes and a new one (context U[256,8192], its prefill not part of the step) takes
+    # its row and its blocks
+    ctx_steps = np.zeros((total_steps, S), np.int64)
+    cur = ctx0.copy()
+    for i in range(total_steps):
+        cur[i % S] = rng.integers(256, 8193)
+        ctx_steps[i] = cur
+        cur = cur + 1
+    max_ctx = int(ctx_steps.max()) + 1
+    cfg, layers, batch = workloads.decode_step_problem(
+        rng, num_layers=1, hidden=hidden, hq=hq, hkv=hkv, inter=inter,
+        ctx=np.full(S, max_ctx), max_pos=max_ctx + 1, random_nibbles=True)
+    max_blocks = batch["block_tables"].shape[1]
+    stream = hip.Stream()
+
+    # ---- CPU baseline + parity on a bounded sample: ONE layer of step 0
+    b0 = dict(batch, h=batch["h"].copy())
+    prior0 = (ctx_steps[0] - 1).astype(np.int32)
+    cu, slots, ctx_l, _ = O.pack_ragged(np.ones(S, np.int32), prior0, batch["block_tables"], bs)
+    b0.update(cu_seqlens=cu, slots=slots, context_lens=ctx_l, positions=prior0)
+    g1 = DecodeStepRunner(cfg, layers, b0, stream=stream)
+    g1.launch()
+    got = O.bf16_bits_to_f32(g1.result_bits())
+    del g1
+    cores = physical_cores()
+    O.set_num_threads(cores)
+    import copy
+    lay_cpu = copy.deepcopy(layers)
+    t0 = time.perf_counter()
+    want = O.bf16_bits_to_f32(OS.decode_step(cfg, lay_cpu, dict(b0, h=batch["h"].copy())))
+    cpu_s = time.perf_counter() - t0
+    del lay_cpu
+    rel_l2 = float(np.linalg.norm(got - want) / np.linalg.norm(want))
+
+    # ---- the 36-layer problem on the device (layer data replicated device-to-device)
+    r = DecodeStepRunner(cfg, layers * L, b0, stream=stream, share_layer_data=True)
+    d_prior = hip.DeviceBuffer.from_numpy((ctx_steps - 1).astype(np.int32))   # [steps][S]
+    d_ones = hip.DeviceBuffer.from_numpy(np.ones(S, np.int32))
+    d_cur_prior = r.idx["positions"]    # positions == prior context of the new token
+
+    def one_step(i, graph):
+        d_cur_prior.copy_from_device_async(d_prior, 4 * S, stream, src_offset=4 * S * i)
+        graph.launch()
+
+    g = hip.Graph(stream)
+    with g:
+        kernels.launch_pack_ragged(d_ones, d_cur_prior, r.idx["block_tables"],
+                                   r.idx["cu_seqlens"], r.slots, r.idx["context_lens"], S, bs,
+                                   max_blocks, stream)
+        r.launch()
+    for i in range(warmup):
+        one_step(i, g)
+    stream.synchronize()
+    e0, e1 = hip.Event(), hip.Event()
+    hip.synchronize()
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for i in range(steps):
+        one_step(warmup + i, g)
+    e1.record(stream)
+    e1.synchronize()
+    hip.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ms_step = e0.elapsed_ms(e1) / steps
+
+    # ---- the dominant kernel alone: paged-attention decode at this shape, rotating layers
+    sum_ctx = float(ctx_steps[warmup:warmup + steps].sum()) / steps
+    c_attn = dict(q=np.zeros((S, hq, 128), np.float16), hq=hq, hkv=hkv, d=128, block_size=bs,
+                  max_blocks=max_blocks, scale=1.0 / np.sqrt(128.0))
+    d_q = hip.DeviceBuffer(S * hq * 128 * 2)
+    d_q.fill(0x3C)
+    d_o = hip.DeviceBuffer(S * hq * 128 * 2)
+    ns = r.num_splits
+    d_ws = hip.DeviceBuffer(max(16, kernels.paged_attn_workspace_bytes(S, hq, 128, ns)))
+
+    def attn(l):
+        kp, vp = r.pools[l]
+        return lambda: kernels.launch_paged_attn_varlen_fp16(
+            d_q, kp, vp, r.idx["block_tables"], r.idx["cu_seqlens"], r.idx["context_lens"], d_o,
+            d_ws, S, S, 1, hq, hkv, 128, bs, max_blocks, ns, c_attn["scale"], True, stream,
+            kernels.ATTN_PHASE_DECODE)
+    ctx_now = r.idx["context_lens"].to_numpy(np.int32, (S,)).astype(np.int64)
+    attn_bytes = int(ctx_now.sum()) * 2 * hkv * 128 * 2 + 2 * S * hq * 128 * 2 + \
+        4 * int(((ctx_now + bs - 1) // bs).sum()) + 4 * (2 * S + 1)
+    ms_attn, _, _ = time_launches(stream, [attn(l) for l in range(L)], 72, 8)
+
+    per_layer_w = sum(int(np.asarray(t[0]).nbytes + np.asarray(t[1]).nbytes +
+                          np.asarray(t[2]).nbytes)
+                      for t in (layers[0][k] for k in ("qkv", "o", "gate_up", "down")))
+    algo_step = L * per_layer_w + sum_ctx * L * 2 * hkv * 128 * 2
+    tok_s = S / (ms_step * 1e-3)
+    achieved = attn_bytes / (ms_attn * 1e-3) / 1e9
+    return {
+        "metric": "decode tok/s @ batch 32 (paged-attn + quant GEMV path)",
+        "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "config 5: continuous-batching decode step, Qwen3-8B-style geometry "
+                               "(36 layers, hidden 4096, 32 q / 8 kv heads, head_dim 128, MLP "
+                               "12288, RMSNorm, RoPE theta 1e6), Q4G128 weights, 32 live sequences, "
+                               "contexts U[256,8192], one finishing and one admitted per step, "
+                               "fp16 paged KV block 16; embedding and lm_head not included",
+                   "mean_sum_ctx": round(sum_ctx, 1), "num_splits": ns,
+                   "algorithmic_bytes_per_step": int(algo_step),
+                   "step_GBps": round(algo_step / (ms_step * 1e-3) / 1e9, 1),
+                   "step_frac_of_hbm_peak": round(algo_step / (ms_step * 1e-3) / 1e9 /
+                                                  HBM_PEAK_GBPS, 4),
+                   "hip_graph": True, "gpu_side_packing": True},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "paged_attn_kernel<4,decode> (one layer of the step)",
+                     "ms_per_launch": round(ms_attn, 5), "algorithmic_bytes_per_launch": attn_bytes},
+        "cpu_baseline": {"value": round(S / (cpu_s * L), 3), "unit": "tok/s", "cores": cores,
+                         "kind": "port",
+                         "sample": f"one of the 36 layers of step 0 ({cpu_s:.2f} s on the CPU "
+                                   "oracle), scaled by 36"},
+        "parity_rel_l2_vs_oracle_one_layer": rel_l2,
+        "host_wall_ms_per_step": round(wall_ms, 4),
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--steps", type=int, default=None,
+                    help="timed steps (default 20 decode steps; 200 launches for the kernel legs)")
+    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--cpu-seconds", type=float, default=5.0)
+    ap.add_argument("--skip-kernels", action="store_true",
+                    help="only the decode-step line, without the per-kernel legs")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; every workload is the full single-GPU "
@@ -221,8 +383,17 @@ def main():
         sys.exit("bench.py: no HIP device visible; there is no CPU fallback to time")
     hip.set_device(0)
     kernels.library()
-    line = bench_paged_decode(args)
-    line["qgemv_q8"] = bench_qgemv_q8(args)
+    args.steps_c5 = args.steps if args.steps is not None else 20
+    args.warmup_c5 = args.warmup if args.warmup is not None else 3
+    line = bench_decode_step(args)
+    if not args.skip_kernels:
+        args.steps, args.warmup = 200, 20
+        c2 = bench_paged_decode(args)
+        line["paged_attn_config2"] = {k: c2[k] for k in ("value", "unit", "ms_per_step", "config",
+                                                          "roofline", "cpu_baseline",
+                                                          "parity_max_abs_vs_oracle")}
+        line["qgemv_q8_config1"] = bench_qgemv_q8(args)
+        line["qgemm_q4_config3"] = bench_q4(args)
     print(json.dumps(line))
 
 

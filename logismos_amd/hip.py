@@ -177,6 +177,13 @@ class DeviceBuffer:
         check(_runtime().hipMemcpy(self.offset(dst_offset), src.offset(src_offset),
                                    C.c_size_t(nbytes), C.c_int(3)), "hipMemcpy(D2D)")
 
+    def copy_from_device_async(self, src: "DeviceBuffer", nbytes: int, stream: "Stream",
+                               dst_offset: int = 0, src_offset: int = 0) -> None:
+        assert dst_offset + nbytes <= self.nbytes and src_offset + nbytes <= src.nbytes
+        check(_runtime().hipMemcpyAsync(self.offset(dst_offset), src.offset(src_offset),
+                                        C.c_size_t(nbytes), C.c_int(3), stream.raw),
+              "hipMemcpyAsync(D2D)")
+
     def fill(self, byte: int) -> None:
         check(_runtime().hipMemset(self._p, C.c_int(byte), C.c_size_t(self.nbytes)), "hipMemset")
 
