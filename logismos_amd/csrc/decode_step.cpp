@@ -97,11 +97,12 @@ extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_c
                                                   batch->rope_sin_f32, batch->slot_mapping, w.q,
                                                   L.k_pool_f16, L.v_pool_f16, b, c.num_q_heads,
                                                   c.num_kv_heads, c.head_dim, c.max_pos, stream));
-        LG_TRY(logismos_launch_paged_attn_varlen_fp16(
+        // attention writes bf16 directly: its output only feeds the o projection
+        LG_TRY(lg::paged_attn_launch(
             w.q, L.k_pool_f16, L.v_pool_f16, batch->block_tables, batch->cu_seqlens,
-            batch->context_lens, w.attn, w.attn_ws, b, b, 1, c.num_q_heads, c.num_kv_heads,
-            c.head_dim, c.block_size, c.max_blocks_per_seq, batch->num_splits, scale, 1, stream));
-        LG_TRY(logismos_launch_cast_f16_bf16(w.attn, w.attn_b, (size_t)b * qd, stream));
+            batch->context_lens, w.attn_b, w.attn_ws, b, b, 1, c.num_q_heads, c.num_kv_heads,
+            c.head_dim, c.block_size, c.max_blocks_per_seq, batch->num_splits, scale, 1,
+            LOGISMOS_ATTN_PHASE_ALL, 1, stream));
         LG_TRY(logismos_launch_qgemm_q4g128_bf16(w.attn_b, L.o.qw, L.o.scale, L.o.zero, w.proj, b,
                                                  c.hidden, qd, stream));
         LG_TRY(logismos_launch_add_rms_norm_bf16(batch->hidden_f32, w.proj, L.norm2_w_f32, w.xn, b,

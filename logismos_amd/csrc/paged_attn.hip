@@ -66,7 +66,19 @@ struct AttnParams {
     int part_tokens;  // keys per partition (multiple of 16)
     float scale_log2e;
     int causal;
+    int out_bf16;  // write `out` as bf16 instead of fp16 (the step executor feeds a bf16 GEMM)
 };
+
+__device__ __forceinline__ unsigned short attn_out_elem(float v, int out_bf16) {
+    if (out_bf16) {
+        unsigned u = __float_as_uint(v);
+        if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40u);
+        u += 0x7fffu + ((u >> 16) & 1u);
+        return (unsigned short)(u >> 16);
+    }
+    const _Float16 hv = (_Float16)v;
+    return __builtin_bit_cast(unsigned short, hv);
+}
 
 // DECODE = true : grid (num_splits, hkv / waves, num_seqs); sequences with exactly
 //                 one new token, keys split into partitions of part_tokens.
@@ -255,10 +267,12 @@ __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_kernel(const At
             const int head = kvh * G + h;
             if (num_parts == 1) {
                 const float inv = 1.0f / lh;
-                half8_t o;
+                uint4_t o;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) o[e] = (_Float16)(acc[h][e] * inv);
-                *reinterpret_cast<half8_t*>(p.out + ((int64_t)t * p.hq + head) * kHeadDim + 8 * c) = o;
+                for (int e = 0; e < 4; ++e)
+                    o[e] = (unsigned)attn_out_elem(acc[h][2 * e] * inv, p.out_bf16) |
+                           ((unsigned)attn_out_elem(acc[h][2 * e + 1] * inv, p.out_bf16) << 16);
+                *reinterpret_cast<uint4_t*>(p.out + ((int64_t)t * p.hq + head) * kHeadDim + 8 * c) = o;
             } else {
                 const int64_t idx = ((int64_t)s * p.num_splits + split) * p.hq + head;
                 float4_t a0 = {acc[h][0], acc[h][1], acc[h][2], acc[h][3]};
@@ -342,7 +356,8 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams 
             dd = fmaf(g, sden[j], dd);
             num = fmaf(g, sn[j][d], num);
         }
-        p.out[((int64_t)t0 * p.hq + h) * kHeadDim + d] = (_Float16)(num / dd);
+        reinterpret_cast<unsigned short*>(p.out)[((int64_t)t0 * p.hq + h) * kHeadDim + d] =
+            attn_out_elem(num / dd, p.out_bf16);
     }
 }
 
@@ -467,6 +482,18 @@ extern "C" logismos_status_t logismos_launch_paged_attn_varlen_fp16_phases(
     int num_seqs, int total_tokens, int max_seqlen_q, int num_q_heads, int num_kv_heads,
     int head_dim, int block_size, int max_blocks_per_seq, int num_splits, float scale, int causal,
     int phases, logismos_stream_t stream) {
+    return lg::paged_attn_launch(q_f16, k_pool_f16, v_pool_f16, block_tables, cu_seqlens_q,
+                                 context_lens, out_f16, workspace, num_seqs, total_tokens,
+                                 max_seqlen_q, num_q_heads, num_kv_heads, head_dim, block_size,
+                                 max_blocks_per_seq, num_splits, scale, causal, phases, 0, stream);
+}
+
+logismos_status_t lg::paged_attn_launch(
+    const void* q_f16, const void* k_pool_f16, const void* v_pool_f16, const int32_t* block_tables,
+    const int32_t* cu_seqlens_q, const int32_t* context_lens, void* out_f16, void* workspace,
+    int num_seqs, int total_tokens, int max_seqlen_q, int num_q_heads, int num_kv_heads,
+    int head_dim, int block_size, int max_blocks_per_seq, int num_splits, float scale, int causal,
+    int phases, int out_bf16, logismos_stream_t stream) {
     if (logismos_check_paged_attn_shape(num_seqs, total_tokens, max_seqlen_q, num_q_heads,
                                         num_kv_heads, head_dim, block_size, max_blocks_per_seq,
                                         num_splits, nullptr, 0) != 0)
@@ -497,6 +524,7 @@ extern "C" logismos_status_t logismos_launch_paged_attn_varlen_fp16_phases(
     p.part_tokens = lg::part_tokens_for(block_size, max_blocks_per_seq, num_splits);
     p.scale_log2e = scale * lg::kLog2e;
     p.causal = causal;
+    p.out_bf16 = out_bf16;
 
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (num_q_heads / num_kv_heads) {

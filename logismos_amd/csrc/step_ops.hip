@@ -22,30 +22,74 @@ __device__ __forceinline__ unsigned short f32_to_bf16(float f) {
 }
 
 // h[r][:] += y[r][:] (when y != nullptr); out[r][:] = bf16(h * inv_rms * w).
-// One workgroup of 256 threads per row.
-__global__ __launch_bounds__(256) void add_rms_norm_kernel(float* __restrict__ h,
-                                                           const uint16_t* __restrict__ y,
-                                                           const float* __restrict__ w,
-                                                           uint16_t* __restrict__ out, int n,
-                                                           float eps) {
+// One workgroup of 1024 threads per row, four consecutive elements per thread
+// per pass kept in registers (a 4096-wide row is a single pass: one read of h,
+// one write of h, one write of out).
+constexpr int kNormThreads = 1024;
+constexpr int kNormMaxPasses = 4;  // rows up to 16384 wide stay in registers
+
+__global__ __launch_bounds__(kNormThreads) void add_rms_norm_kernel(
+    float* __restrict__ h, const uint16_t* __restrict__ y, const float* __restrict__ w,
+    uint16_t* __restrict__ out, int n, float eps) {
     const int64_t row = blockIdx.x;
     float* hr = h + row * n;
+    const bool vec = (n & 3) == 0 && n <= 4 * kNormThreads * kNormMaxPasses;
+    __shared__ float part[kNormThreads / 64];
+    float4_t v[kNormMaxPasses];
     float sum_sq = 0.0f;
-    for (int j = threadIdx.x; j < n; j += 256) {
-        float v = hr[j];
-        if (y) {
-            v += bf16_to_f32(y[row * n + j]);
-            hr[j] = v;
+    if (vec) {
+#pragma unroll
+        for (int p = 0; p < kNormMaxPasses; ++p) {
+            const int j = (p * kNormThreads + (int)threadIdx.x) * 4;
+            if (j < n) {
+                v[p] = *reinterpret_cast<const float4_t*>(hr + j);
+                if (y) {
+                    const uint2_t yy = *reinterpret_cast<const uint2_t*>(y + row * n + j);
+                    v[p][0] += __uint_as_float(yy[0] << 16);
+                    v[p][1] += __uint_as_float(yy[0] & 0xffff0000u);
+                    v[p][2] += __uint_as_float(yy[1] << 16);
+                    v[p][3] += __uint_as_float(yy[1] & 0xffff0000u);
+                    *reinterpret_cast<float4_t*>(hr + j) = v[p];
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sum_sq = fmaf(v[p][e], v[p][e], sum_sq);
+            }
         }
-        sum_sq = fmaf(v, v, sum_sq);
+    } else {
+        for (int j = threadIdx.x; j < n; j += kNormThreads) {
+            float t = hr[j];
+            if (y) {
+                t += bf16_to_f32(y[row * n + j]);
+                hr[j] = t;
+            }
+            sum_sq = fmaf(t, t, sum_sq);
+        }
     }
-    __shared__ float part[4];
     sum_sq = wave_sum(sum_sq);
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = sum_sq;
     __syncthreads();
-    const float total = part[0] + part[1] + part[2] + part[3];
+    float total = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kNormThreads / 64; ++i) total += part[i];
     const float inv = 1.0f / sqrtf(total / (float)n + eps);
-    for (int j = threadIdx.x; j < n; j += 256) out[row * n + j] = f32_to_bf16(hr[j] * inv * w[j]);
+    if (vec) {
+#pragma unroll
+        for (int p = 0; p < kNormMaxPasses; ++p) {
+            const int j = (p * kNormThreads + (int)threadIdx.x) * 4;
+            if (j < n) {
+                const float4_t ww = *reinterpret_cast<const float4_t*>(w + j);
+                uint2_t o;
+                o[0] = (unsigned)f32_to_bf16(v[p][0] * inv * ww[0]) |
+                       ((unsigned)f32_to_bf16(v[p][1] * inv * ww[1]) << 16);
+                o[1] = (unsigned)f32_to_bf16(v[p][2] * inv * ww[2]) |
+                       ((unsigned)f32_to_bf16(v[p][3] * inv * ww[3]) << 16);
+                *reinterpret_cast<uint2_t*>(out + row * n + j) = o;
+            }
+        }
+    } else {
+        for (int j = threadIdx.x; j < n; j += kNormThreads)
+            out[row * n + j] = f32_to_bf16(hr[j] * inv * w[j]);
+    }
 }
 
 // grid (hq + 2*hkv, total_tokens), 64 threads: thread i rotates elements i and
@@ -153,7 +197,8 @@ extern "C" logismos_status_t logismos_launch_add_rms_norm_bf16(void* h_f32, cons
                                                                logismos_stream_t stream) {
     if (rows <= 0 || n <= 0 || (int64_t)rows * n > (int64_t)INT32_MAX) return hipErrorInvalidValue;
     if (!h_f32 || !w_f32 || !out_bf16) return hipErrorInvalidValue;
-    lg::add_rms_norm_kernel<<<dim3(rows), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+    lg::add_rms_norm_kernel<<<dim3(rows), dim3(lg::kNormThreads), 0,
+                              static_cast<hipStream_t>(stream)>>>(
         static_cast<float*>(h_f32), static_cast<const uint16_t*>(y_bf16),
         static_cast<const float*>(w_f32), static_cast<uint16_t*>(out_bf16), n, eps);
     return hipGetLastError();

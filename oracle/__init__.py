@@ -402,18 +402,24 @@ def paged_gather_fp16(pool, block_table_row, ctx, block_size, row_elems):
     return out.view(np.float16)
 
 
+_paged_attn_f32 = _sig("oracle_paged_attn_varlen_fp16_f32out", None, _vp, _vp, _vp, _vp, _vp, _vp,
+                       _vp, _sz, _sz, _sz, _sz, _sz, _sz, C.c_float, C.c_int)
+
+
 def paged_attn_varlen_fp16(q, k_pool, v_pool, block_tables, cu_seqlens_q, context_lens,
-                           num_q_heads, num_kv_heads, head_dim, block_size, scale, causal=True):
+                           num_q_heads, num_kv_heads, head_dim, block_size, scale, causal=True,
+                           f32_out=False):
     q, k_pool, v_pool = _u16(q), _u16(k_pool), _u16(v_pool)
     block_tables = np.ascontiguousarray(block_tables, dtype=np.int32)
     cu = np.ascontiguousarray(cu_seqlens_q, dtype=np.int32)
     ctx = np.ascontiguousarray(context_lens, dtype=np.int32)
     num_seqs = ctx.size
-    out = np.zeros(q.shape, np.uint16)
-    _paged_attn(_p(q), _p(k_pool), _p(v_pool), _p(block_tables), _p(cu), _p(ctx), _p(out),
-                num_seqs, num_q_heads, num_kv_heads, head_dim, block_size,
-                block_tables.shape[1] if num_seqs else 0, scale, 1 if causal else 0)
-    return out.view(np.float16)
+    out = np.zeros(q.shape, np.float32 if f32_out else np.uint16)
+    (_paged_attn_f32 if f32_out else _paged_attn)(
+        _p(q), _p(k_pool), _p(v_pool), _p(block_tables), _p(cu), _p(ctx), _p(out), num_seqs,
+        num_q_heads, num_kv_heads, head_dim, block_size,
+        block_tables.shape[1] if num_seqs else 0, scale, 1 if causal else 0)
+    return out if f32_out else out.view(np.float16)
 
 
 # ---------------------------------------------------------------- metric / threads

@@ -12,7 +12,7 @@ part of the definition and are the ones the GPU path uses:
   normed activations ........ bf16   (input of every quantized GEMM)
   GEMM outputs .............. bf16   (fp32 accumulation, one rounding)
   q, and K/V in the cache ... fp16   (RoPE in fp32 on the bf16 GEMM output)
-  attention output .......... fp16 -> bf16 for the o projection
+  attention output .......... bf16   (one rounding of the fp32 result; feeds the o projection)
   silu(gate) * up ........... bf16
 """
 from __future__ import annotations
@@ -92,8 +92,8 @@ def decode_step(cfg, layers, batch, trace=None):
         attn = O.paged_attn_varlen_fp16(q16, L["k_pool"], L["v_pool"], batch["block_tables"],
                                         batch["cu_seqlens"], batch["context_lens"], cfg["hq"],
                                         cfg["hkv"], cfg["d"], cfg["block_size"],
-                                        1.0 / np.sqrt(np.float32(cfg["d"])), True)
-        o = _gemm(cast_f16_bf16(attn.reshape(b, -1)), L["o"], b)
+                                        1.0 / np.sqrt(np.float32(cfg["d"])), True, f32_out=True)
+        o = _gemm(O.f32_to_bf16_bits(attn.reshape(b, -1)), L["o"], b)
         xn2 = add_rms_norm_bf16(h, o, L["norm2"], cfg["eps"])
         gu = _gemm(xn2, L["gate_up"], b)
         act = silu_mul_bf16(gu, cfg["inter"])

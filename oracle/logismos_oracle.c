@@ -602,12 +602,12 @@ void oracle_paged_gather_fp16(const uint16_t* pool, const int32_t* block_table_r
  * q head h -> kv head h / groups (:366-382).  Visible keys of query token i
  * (n new tokens, context c): causal ? [0, c-n+i] : [0, c).  No visible key =>
  * zeros (softmax_last_dim over n = 0 columns).  Output rounded to fp16 once. */
-void oracle_paged_attn_varlen_fp16(const uint16_t* q, const uint16_t* k_pool,
-                                   const uint16_t* v_pool, const int32_t* block_tables,
-                                   const int32_t* cu_seqlens_q, const int32_t* context_lens,
-                                   uint16_t* out, size_t num_seqs, size_t num_q_heads,
-                                   size_t num_kv_heads, size_t head_dim, size_t block_size,
-                                   size_t max_blocks_per_seq, float scale, int causal) {
+static void paged_attn_core(const uint16_t* q, const uint16_t* k_pool, const uint16_t* v_pool,
+                            const int32_t* block_tables, const int32_t* cu_seqlens_q,
+                            const int32_t* context_lens, uint16_t* out, float* out_f32,
+                            size_t num_seqs, size_t num_q_heads, size_t num_kv_heads,
+                            size_t head_dim, size_t block_size, size_t max_blocks_per_seq,
+                            float scale, int causal) {
     size_t groups = num_q_heads / num_kv_heads;
     size_t row = num_kv_heads * head_dim;
 #pragma omp parallel for schedule(dynamic, 1)
@@ -651,7 +651,10 @@ void oracle_paged_attn_varlen_fp16(const uint16_t* q, const uint16_t* k_pool,
                     float p = probs[j];
                     for (size_t e = 0; e < head_dim; ++e) of[e] += p * vr[e];
                 }
-                oracle_f32_to_f16_n(of, out + qoff, head_dim);
+                if (out_f32)
+                    memcpy(out_f32 + qoff, of, head_dim * sizeof(float));
+                else
+                    oracle_f32_to_f16_n(of, out + qoff, head_dim);
             }
         }
         free(kh);
@@ -663,6 +666,31 @@ void oracle_paged_attn_varlen_fp16(const uint16_t* q, const uint16_t* k_pool,
         free(qf);
         free(of);
     }
+}
+
+void oracle_paged_attn_varlen_fp16(const uint16_t* q, const uint16_t* k_pool,
+                                   const uint16_t* v_pool, const int32_t* block_tables,
+                                   const int32_t* cu_seqlens_q, const int32_t* context_lens,
+                                   uint16_t* out, size_t num_seqs, size_t num_q_heads,
+                                   size_t num_kv_heads, size_t head_dim, size_t block_size,
+                                   size_t max_blocks_per_seq, float scale, int causal) {
+    paged_attn_core(q, k_pool, v_pool, block_tables, cu_seqlens_q, context_lens, out, NULL,
+                    num_seqs, num_q_heads, num_kv_heads, head_dim, block_size, max_blocks_per_seq,
+                    scale, causal);
+}
+
+/* The same attention with the fp32 result before its final rounding (the decode
+ * step rounds it to bf16 once, for the o projection). */
+void oracle_paged_attn_varlen_fp16_f32out(const uint16_t* q, const uint16_t* k_pool,
+                                          const uint16_t* v_pool, const int32_t* block_tables,
+                                          const int32_t* cu_seqlens_q,
+                                          const int32_t* context_lens, float* out,
+                                          size_t num_seqs, size_t num_q_heads,
+                                          size_t num_kv_heads, size_t head_dim, size_t block_size,
+                                          size_t max_blocks_per_seq, float scale, int causal) {
+    paged_attn_core(q, k_pool, v_pool, block_tables, cu_seqlens_q, context_lens, NULL, out,
+                    num_seqs, num_q_heads, num_kv_heads, head_dim, block_size, max_blocks_per_seq,
+                    scale, causal);
 }
 
 /* ------------------------------------------------------------------ metric / threads */

@@ -119,6 +119,14 @@ void oracle_paged_attn_varlen_fp16(const uint16_t* q, const uint16_t* k_pool,
                                    size_t num_kv_heads, size_t head_dim, size_t block_size,
                                    size_t max_blocks_per_seq, float scale, int causal);
 
+void oracle_paged_attn_varlen_fp16_f32out(const uint16_t* q, const uint16_t* k_pool,
+                                          const uint16_t* v_pool, const int32_t* block_tables,
+                                          const int32_t* cu_seqlens_q,
+                                          const int32_t* context_lens, float* out,
+                                          size_t num_seqs, size_t num_q_heads,
+                                          size_t num_kv_heads, size_t head_dim, size_t block_size,
+                                          size_t max_blocks_per_seq, float scale, int causal);
+
 /* ---- parity metric of the reference's GPU tests (crates/kernels/tests/matmul_parity.rs:83-99) */
 void oracle_parity_metric_f32(const float* got, const float* want, size_t n, float* max_abs,
                               float* max_rel);
