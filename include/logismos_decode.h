@@ -148,6 +148,21 @@ logismos_status_t logismos_launch_qgemm_q4g128_bf16_mfma(const void* x_bf16, con
                                                          const void* zero_f16, void* y_bf16, int b,
                                                          int n, int k, logismos_stream_t stream);
 
+/* Split-K form for a decode batch (b <= 32): fp32 partial products
+ *   parts[j][b][n] = sum over K part j of x[b][k] * w[n][k],  j < J,
+ * whose sum over j is the product.  Workgroups are tall (up to 256 weight rows
+ * by a short K part) so that the x each one needs is small next to its weights;
+ * the J parts are added by the consumer (the `_f32p` operators below), which
+ * keeps the result deterministic and un-rounded.  J depends on (b, n, k) only:
+ * `logismos_qgemm_q4g128_splitk_parts` returns it (0 for a rejected shape);
+ * `parts_f32` needs J*b*n*4 bytes. */
+int logismos_qgemm_q4g128_splitk_parts(int b, int n, int k);
+logismos_status_t logismos_launch_qgemm_q4g128_f32_splitk(const void* x_bf16, const void* qw_u8,
+                                                          const void* scale_f16,
+                                                          const void* zero_f16, void* parts_f32,
+                                                          int b, int n, int k,
+                                                          logismos_stream_t stream);
+
 /* ggml Q8_0 block stream `[N][K/32]{f16 d; int8 qs[32]}` -> planar Q8G32. */
 logismos_status_t logismos_launch_repack_q8_0(const void* blocks_q8_0, void* qs_i8, void* d_f16,
                                               int n, int k, logismos_stream_t stream);
@@ -279,6 +294,22 @@ logismos_status_t logismos_launch_silu_mul_bf16(const void* gate_up_bf16, void* 
                                                 int inter, logismos_stream_t stream);
 
 logismos_status_t logismos_launch_cast_f16_bf16(const void* in_f16, void* out_bf16, size_t count,
+                                                logismos_stream_t stream);
+
+/* The same three operators reading the fp32 split-K parts of the preceding GEMM
+ * (`parts[j]` is a whole `[rows][width]` matrix; the operator adds the
+ * num_parts of them in order, without intermediate rounding). */
+logismos_status_t logismos_launch_add_rms_norm_f32p(void* h_f32, const void* parts_f32,
+                                                    int num_parts, const void* w_f32,
+                                                    void* out_bf16, int rows, int n, float eps,
+                                                    logismos_stream_t stream);
+logismos_status_t logismos_launch_rope_kv_write_f32p(
+    const void* qkv_parts_f32, int num_parts, const int32_t* positions, const void* cos_f32,
+    const void* sin_f32, const int64_t* slot_mapping, void* q_out_f16, void* k_pool_f16,
+    void* v_pool_f16, int total_tokens, int num_q_heads, int num_kv_heads, int head_dim,
+    int max_pos, logismos_stream_t stream);
+logismos_status_t logismos_launch_silu_mul_f32p(const void* parts_f32, int num_parts,
+                                                void* out_bf16, int rows, int inter,
                                                 logismos_stream_t stream);
 
 /* out[r] = first index of the maximum of logits[r][:] (`decode::greedy`,

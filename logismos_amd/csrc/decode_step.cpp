@@ -11,14 +11,14 @@ namespace {
 
 struct Workspace {
     char* xn;        // bf16 [B][hidden]
-    char* qkv;       // bf16 [B][(hq+2hkv)*d]
+    char* qkv;       // f32  [Jqkv][B][(hq+2hkv)*d]   split-K parts
     char* q;         // f16  [B][hq*d]
-    char* attn;      // f16  [B][hq*d]
     char* attn_b;    // bf16 [B][hq*d]
-    char* proj;      // bf16 [B][hidden]      (o projection, then down projection)
-    char* gate_up;   // bf16 [B][2*inter]
+    char* proj;      // f32  [max(Jo,Jdown)][B][hidden]  (o projection, then down projection)
+    char* gate_up;   // f32  [Jgu][B][2*inter]
     char* act;       // bf16 [B][inter]
-    char* attn_ws;   // split-K workspace
+    char* attn_ws;   // split-K workspace of the attention
+    int j_qkv, j_o, j_gu, j_down;
     size_t total;
 };
 
@@ -34,13 +34,17 @@ Workspace carve(const logismos_decode_config_t& c, int b, int num_splits, char* 
     };
     const size_t qd = (size_t)c.num_q_heads * c.head_dim;
     const size_t kvd = (size_t)c.num_kv_heads * c.head_dim;
+    w.j_qkv = logismos_qgemm_q4g128_splitk_parts(b, (int)(qd + 2 * kvd), c.hidden);
+    w.j_o = logismos_qgemm_q4g128_splitk_parts(b, c.hidden, (int)qd);
+    w.j_gu = logismos_qgemm_q4g128_splitk_parts(b, 2 * c.intermediate, c.hidden);
+    w.j_down = logismos_qgemm_q4g128_splitk_parts(b, c.hidden, c.intermediate);
+    const int j_proj = w.j_o > w.j_down ? w.j_o : w.j_down;
     w.xn = take((size_t)b * c.hidden * 2);
-    w.qkv = take((size_t)b * (qd + 2 * kvd) * 2);
+    w.qkv = take((size_t)w.j_qkv * b * (qd + 2 * kvd) * 4);
     w.q = take((size_t)b * qd * 2);
-    w.attn = take((size_t)b * qd * 2);
     w.attn_b = take((size_t)b * qd * 2);
-    w.proj = take((size_t)b * c.hidden * 2);
-    w.gate_up = take((size_t)b * 2 * c.intermediate * 2);
+    w.proj = take((size_t)j_proj * b * c.hidden * 4);
+    w.gate_up = take((size_t)w.j_gu * b * 2 * c.intermediate * 4);
     w.act = take((size_t)b * c.intermediate * 2);
     w.attn_ws = take(logismos_paged_attn_workspace_bytes(b, c.num_q_heads, c.head_dim, num_splits));
     w.total = off;
@@ -86,36 +90,39 @@ extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_c
     const int kvd = c.num_kv_heads * c.head_dim;
     const float scale = 1.0f / sqrtf((float)c.head_dim);
 
-    const void* residual = nullptr;  // what the next add_rms_norm folds into h
+    int res_parts = 0;  // split-K parts of the projection the next add_rms_norm folds into h
     for (int l = 0; l < c.num_layers; ++l) {
         const logismos_decode_layer_t& L = layers[l];
-        LG_TRY(logismos_launch_add_rms_norm_bf16(batch->hidden_f32, residual, L.norm1_w_f32, w.xn, b,
-                                                 c.hidden, c.rms_eps, stream));
-        LG_TRY(logismos_launch_qgemm_q4g128_bf16(w.xn, L.qkv.qw, L.qkv.scale, L.qkv.zero, w.qkv, b,
-                                                 qd + 2 * kvd, c.hidden, stream));
-        LG_TRY(logismos_launch_rope_kv_write_fp16(w.qkv, batch->positions, batch->rope_cos_f32,
-                                                  batch->rope_sin_f32, batch->slot_mapping, w.q,
-                                                  L.k_pool_f16, L.v_pool_f16, b, c.num_q_heads,
-                                                  c.num_kv_heads, c.head_dim, c.max_pos, stream));
+        LG_TRY(logismos_launch_add_rms_norm_f32p(batch->hidden_f32, w.proj, res_parts,
+                                                 L.norm1_w_f32, w.xn, b, c.hidden, c.rms_eps,
+                                                 stream));
+        LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk(w.xn, L.qkv.qw, L.qkv.scale, L.qkv.zero,
+                                                       w.qkv, b, qd + 2 * kvd, c.hidden, stream));
+        LG_TRY(logismos_launch_rope_kv_write_f32p(
+            w.qkv, w.j_qkv, batch->positions, batch->rope_cos_f32, batch->rope_sin_f32,
+            batch->slot_mapping, w.q, L.k_pool_f16, L.v_pool_f16, b, c.num_q_heads, c.num_kv_heads,
+            c.head_dim, c.max_pos, stream));
         // attention writes bf16 directly: its output only feeds the o projection
         LG_TRY(lg::paged_attn_launch(
             w.q, L.k_pool_f16, L.v_pool_f16, batch->block_tables, batch->cu_seqlens,
             batch->context_lens, w.attn_b, w.attn_ws, b, b, 1, c.num_q_heads, c.num_kv_heads,
             c.head_dim, c.block_size, c.max_blocks_per_seq, batch->num_splits, scale, 1,
             LOGISMOS_ATTN_PHASE_ALL, 1, stream));
-        LG_TRY(logismos_launch_qgemm_q4g128_bf16(w.attn_b, L.o.qw, L.o.scale, L.o.zero, w.proj, b,
-                                                 c.hidden, qd, stream));
-        LG_TRY(logismos_launch_add_rms_norm_bf16(batch->hidden_f32, w.proj, L.norm2_w_f32, w.xn, b,
-                                                 c.hidden, c.rms_eps, stream));
-        LG_TRY(logismos_launch_qgemm_q4g128_bf16(w.xn, L.gate_up.qw, L.gate_up.scale,
-                                                 L.gate_up.zero, w.gate_up, b, 2 * c.intermediate,
-                                                 c.hidden, stream));
-        LG_TRY(logismos_launch_silu_mul_bf16(w.gate_up, w.act, b, c.intermediate, stream));
-        LG_TRY(logismos_launch_qgemm_q4g128_bf16(w.act, L.down.qw, L.down.scale, L.down.zero, w.proj,
-                                                 b, c.hidden, c.intermediate, stream));
-        residual = w.proj;
+        LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk(w.attn_b, L.o.qw, L.o.scale, L.o.zero,
+                                                       w.proj, b, c.hidden, qd, stream));
+        LG_TRY(logismos_launch_add_rms_norm_f32p(batch->hidden_f32, w.proj, w.j_o, L.norm2_w_f32,
+                                                 w.xn, b, c.hidden, c.rms_eps, stream));
+        LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk(w.xn, L.gate_up.qw, L.gate_up.scale,
+                                                       L.gate_up.zero, w.gate_up, b,
+                                                       2 * c.intermediate, c.hidden, stream));
+        LG_TRY(logismos_launch_silu_mul_f32p(w.gate_up, w.j_gu, w.act, b, c.intermediate, stream));
+        LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk(w.act, L.down.qw, L.down.scale, L.down.zero,
+                                                       w.proj, b, c.hidden, c.intermediate,
+                                                       stream));
+        res_parts = w.j_down;
     }
-    LG_TRY(logismos_launch_add_rms_norm_bf16(batch->hidden_f32, residual, batch->final_norm_w_f32,
-                                             batch->out_bf16, b, c.hidden, c.rms_eps, stream));
+    LG_TRY(logismos_launch_add_rms_norm_f32p(batch->hidden_f32, w.proj, res_parts,
+                                             batch->final_norm_w_f32, batch->out_bf16, b, c.hidden,
+                                             c.rms_eps, stream));
     return 0;
 }

@@ -20,43 +20,11 @@
 // + b*k*2 (x) + b*n*2 (y).
 #include "device_utils.hpp"
 #include "launch_common.hpp"
+#include "q4_common.hpp"
 
 #include <hip/hip_fp16.h>
 
 namespace lg {
-
-__device__ __forceinline__ float bf16_lo_to_f32(unsigned v) { return __uint_as_float(v << 16); }
-__device__ __forceinline__ float bf16_hi_to_f32(unsigned v) {
-    return __uint_as_float(v & 0xffff0000u);
-}
-__device__ __forceinline__ unsigned short f32_to_bf16_rne(float f) {
-    unsigned u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (unsigned short)(u >> 16);
-}
-__device__ __forceinline__ float dot2_bf16(unsigned a, unsigned b, float c) {
-    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a),
-                                           __builtin_bit_cast(bf16x2_t, b), c, false);
-}
-
-// 8 consecutive bf16 (x0..x7 in four dwords) -> pairs (x0,x4) (x1,x5) (x2,x6) (x3,x7)
-__device__ __forceinline__ uint4_t pair_order(uint4_t d) {
-    uint4_t o;
-    o[0] = (d[0] & 0xffffu) | (d[2] << 16);
-    o[1] = (d[0] >> 16) | (d[2] & 0xffff0000u);
-    o[2] = (d[1] & 0xffffu) | (d[3] << 16);
-    o[3] = (d[1] >> 16) | (d[3] & 0xffff0000u);
-    return o;
-}
-__device__ __forceinline__ float sum8_bf16(uint4_t d) {
-    float s = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) s += bf16_lo_to_f32(d[i]) + bf16_hi_to_f32(d[i]);
-    return s;
-}
-
-constexpr unsigned kNibMask = 0x000F000Fu;
 
 // ---------------------------------------------------------------------------
 // VALU path, batch B <= 4.  grid = ceil(n / (4*R)), block = 256 (4 waves).
@@ -405,18 +373,6 @@ __global__ __launch_bounds__(1024) void qgemm_q4g128_mfma_kernel(
         for (int w = 0; w < nwaves; ++w) sum += yl[(size_t)w * T * BP * 16 + i];
         if (r < rows_here && bi < b) y[(int64_t)bi * n + row0 + r] = f32_to_bf16_rne(sum);
     }
-}
-
-static int device_cu_count() {
-    static const int count = [] {
-        int dev = 0, cus = 0;
-        if (hipGetDevice(&dev) != hipSuccess) return 256;
-        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-            cus <= 0)
-            return 256;
-        return cus;
-    }();
-    return count;
 }
 
 template <int BT, int GW, int T>

@@ -29,8 +29,9 @@ constexpr int kNormThreads = 1024;
 constexpr int kNormMaxPasses = 4;  // rows up to 16384 wide stay in registers
 
 __global__ __launch_bounds__(kNormThreads) void add_rms_norm_kernel(
-    float* __restrict__ h, const uint16_t* __restrict__ y, const float* __restrict__ w,
-    uint16_t* __restrict__ out, int n, float eps) {
+    float* __restrict__ h, const uint16_t* __restrict__ y, const float* __restrict__ yp,
+    int num_parts, int64_t part_stride, const float* __restrict__ w, uint16_t* __restrict__ out,
+    int n, float eps) {
     const int64_t row = blockIdx.x;
     float* hr = h + row * n;
     const bool vec = (n & 3) == 0 && n <= 4 * kNormThreads * kNormMaxPasses;
@@ -50,6 +51,17 @@ __global__ __launch_bounds__(kNormThreads) void add_rms_norm_kernel(
                     v[p][2] += __uint_as_float(yy[1] << 16);
                     v[p][3] += __uint_as_float(yy[1] & 0xffff0000u);
                     *reinterpret_cast<float4_t*>(hr + j) = v[p];
+                } else if (yp) {
+                    // fp32 partial sums of a split-K projection, added in part order
+                    for (int q = 0; q < num_parts; ++q) {
+                        const float4_t t4 = *reinterpret_cast<const float4_t*>(
+                            yp + (int64_t)q * part_stride + row * n + j);
+                        v[p][0] += t4[0];
+                        v[p][1] += t4[1];
+                        v[p][2] += t4[2];
+                        v[p][3] += t4[3];
+                    }
+                    *reinterpret_cast<float4_t*>(hr + j) = v[p];
                 }
 #pragma unroll
                 for (int e = 0; e < 4; ++e) sum_sq = fmaf(v[p][e], v[p][e], sum_sq);
@@ -60,6 +72,9 @@ __global__ __launch_bounds__(kNormThreads) void add_rms_norm_kernel(
             float t = hr[j];
             if (y) {
                 t += bf16_to_f32(y[row * n + j]);
+                hr[j] = t;
+            } else if (yp) {
+                for (int q = 0; q < num_parts; ++q) t += yp[(int64_t)q * part_stride + row * n + j];
                 hr[j] = t;
             }
             sum_sq = fmaf(t, t, sum_sq);
@@ -96,7 +111,8 @@ __global__ __launch_bounds__(kNormThreads) void add_rms_norm_kernel(
 // i + d/2 (d = 128).  q heads go to q_out (fp16); k heads, rotated, and v heads,
 // as they are, go to the pools at the token's slot.
 __global__ __launch_bounds__(64) void rope_kv_write_kernel(
-    const uint16_t* __restrict__ qkv, const int32_t* __restrict__ positions,
+    const uint16_t* __restrict__ qkv, const float* __restrict__ qkv_parts, int num_parts,
+    int64_t part_stride, const int32_t* __restrict__ positions,
     const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     const int64_t* __restrict__ slot_mapping, __half* __restrict__ q_out,
     __half* __restrict__ k_pool, __half* __restrict__ v_pool, int hq, int hkv, int max_pos) {
@@ -104,9 +120,17 @@ __global__ __launch_bounds__(64) void rope_kv_write_kernel(
     const int head = blockIdx.x;
     const int64_t t = blockIdx.y;
     const int i = threadIdx.x;
-    const uint16_t* src = qkv + (t * (hq + 2 * hkv) + head) * D;
-    const float x0 = bf16_to_f32(src[i]);
-    const float x1 = bf16_to_f32(src[i + HALF]);
+    const int64_t off = (t * (hq + 2 * hkv) + head) * D;
+    float x0 = 0.0f, x1 = 0.0f;
+    if (qkv) {
+        x0 = bf16_to_f32(qkv[off + i]);
+        x1 = bf16_to_f32(qkv[off + i + HALF]);
+    } else {
+        for (int q = 0; q < num_parts; ++q) {
+            x0 += qkv_parts[(int64_t)q * part_stride + off + i];
+            x1 += qkv_parts[(int64_t)q * part_stride + off + i + HALF];
+        }
+    }
     if (head < hq + hkv) {
         int pos = positions[t];
         pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
@@ -136,14 +160,24 @@ __global__ __launch_bounds__(64) void rope_kv_write_kernel(
 
 // out[t][j] = bf16( silu(gate[t][j]) * up[t][j] ), gate_up = [t][gate(0..inter) | up(0..inter)]
 __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restrict__ gate_up,
+                                                       const float* __restrict__ parts,
+                                                       int num_parts, int64_t part_stride,
                                                        uint16_t* __restrict__ out, int inter,
                                                        int64_t total) {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= total) return;
     const int64_t t = idx / inter;
     const int64_t j = idx - t * inter;
-    const float g = bf16_to_f32(gate_up[t * 2 * inter + j]);
-    const float u = bf16_to_f32(gate_up[t * 2 * inter + inter + j]);
+    float g = 0.0f, u = 0.0f;
+    if (gate_up) {
+        g = bf16_to_f32(gate_up[t * 2 * inter + j]);
+        u = bf16_to_f32(gate_up[t * 2 * inter + inter + j]);
+    } else {
+        for (int q = 0; q < num_parts; ++q) {
+            g += parts[(int64_t)q * part_stride + t * 2 * inter + j];
+            u += parts[(int64_t)q * part_stride + t * 2 * inter + inter + j];
+        }
+    }
     const float sg = g / (1.0f + expf(-g));
     out[idx] = f32_to_bf16(sg * u);
 }
@@ -199,8 +233,25 @@ extern "C" logismos_status_t logismos_launch_add_rms_norm_bf16(void* h_f32, cons
     if (!h_f32 || !w_f32 || !out_bf16) return hipErrorInvalidValue;
     lg::add_rms_norm_kernel<<<dim3(rows), dim3(lg::kNormThreads), 0,
                               static_cast<hipStream_t>(stream)>>>(
-        static_cast<float*>(h_f32), static_cast<const uint16_t*>(y_bf16),
+        static_cast<float*>(h_f32), static_cast<const uint16_t*>(y_bf16), nullptr, 0, 0,
         static_cast<const float*>(w_f32), static_cast<uint16_t*>(out_bf16), n, eps);
+    return hipGetLastError();
+}
+
+extern "C" logismos_status_t logismos_launch_add_rms_norm_f32p(void* h_f32, const void* parts_f32,
+                                                               int num_parts, const void* w_f32,
+                                                               void* out_bf16, int rows, int n,
+                                                               float eps,
+                                                               logismos_stream_t stream) {
+    if (rows <= 0 || n <= 0 || (int64_t)rows * n > (int64_t)INT32_MAX) return hipErrorInvalidValue;
+    if (!h_f32 || !w_f32 || !out_bf16 || num_parts < 0 || (num_parts > 0 && !parts_f32))
+        return hipErrorInvalidValue;
+    lg::add_rms_norm_kernel<<<dim3(rows), dim3(lg::kNormThreads), 0,
+                              static_cast<hipStream_t>(stream)>>>(
+        static_cast<float*>(h_f32), nullptr,
+        num_parts > 0 ? static_cast<const float*>(parts_f32) : nullptr, num_parts,
+        (int64_t)rows * n, static_cast<const float*>(w_f32), static_cast<uint16_t*>(out_bf16), n,
+        eps);
     return hipGetLastError();
 }
 
@@ -220,10 +271,49 @@ extern "C" logismos_status_t logismos_launch_rope_kv_write_fp16(
         return hipErrorInvalidValue;
     dim3 grid(num_q_heads + 2 * num_kv_heads, total_tokens);
     lg::rope_kv_write_kernel<<<grid, dim3(64), 0, static_cast<hipStream_t>(stream)>>>(
-        static_cast<const uint16_t*>(qkv_bf16), positions, static_cast<const float*>(cos_f32),
+        static_cast<const uint16_t*>(qkv_bf16), nullptr, 0, 0, positions,
+        static_cast<const float*>(cos_f32),
         static_cast<const float*>(sin_f32), slot_mapping, static_cast<__half*>(q_out_f16),
         static_cast<__half*>(k_pool_f16), static_cast<__half*>(v_pool_f16), num_q_heads,
         num_kv_heads, max_pos);
+    return hipGetLastError();
+}
+
+extern "C" logismos_status_t logismos_launch_rope_kv_write_f32p(
+    const void* qkv_parts_f32, int num_parts, const int32_t* positions, const void* cos_f32,
+    const void* sin_f32, const int64_t* slot_mapping, void* q_out_f16, void* k_pool_f16,
+    void* v_pool_f16, int total_tokens, int num_q_heads, int num_kv_heads, int head_dim,
+    int max_pos, logismos_stream_t stream) {
+    if (total_tokens < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || max_pos <= 0 || num_parts <= 0)
+        return hipErrorInvalidValue;
+    if (head_dim != 128 || total_tokens > 65535) return hipErrorInvalidValue;
+    const int64_t width = (int64_t)(num_q_heads + 2 * num_kv_heads) * head_dim;
+    if ((int64_t)total_tokens * width > (int64_t)INT32_MAX) return hipErrorInvalidValue;
+    if (total_tokens == 0) return hipSuccess;
+    if (!qkv_parts_f32 || !positions || !cos_f32 || !sin_f32 || !slot_mapping || !q_out_f16 ||
+        !k_pool_f16 || !v_pool_f16)
+        return hipErrorInvalidValue;
+    dim3 grid(num_q_heads + 2 * num_kv_heads, total_tokens);
+    lg::rope_kv_write_kernel<<<grid, dim3(64), 0, static_cast<hipStream_t>(stream)>>>(
+        nullptr, static_cast<const float*>(qkv_parts_f32), num_parts, (int64_t)total_tokens * width,
+        positions, static_cast<const float*>(cos_f32), static_cast<const float*>(sin_f32),
+        slot_mapping, static_cast<__half*>(q_out_f16), static_cast<__half*>(k_pool_f16),
+        static_cast<__half*>(v_pool_f16), num_q_heads, num_kv_heads, max_pos);
+    return hipGetLastError();
+}
+
+extern "C" logismos_status_t logismos_launch_silu_mul_f32p(const void* parts_f32, int num_parts,
+                                                           void* out_bf16, int rows, int inter,
+                                                           logismos_stream_t stream) {
+    if (rows <= 0 || inter <= 0 || num_parts <= 0 ||
+        (int64_t)rows * inter * 2 > (int64_t)INT32_MAX)
+        return hipErrorInvalidValue;
+    if (!parts_f32 || !out_bf16) return hipErrorInvalidValue;
+    const int64_t total = (int64_t)rows * inter;
+    lg::silu_mul_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                          static_cast<hipStream_t>(stream)>>>(
+        nullptr, static_cast<const float*>(parts_f32), num_parts, (int64_t)rows * 2 * inter,
+        static_cast<uint16_t*>(out_bf16), inter, total);
     return hipGetLastError();
 }
 
@@ -236,7 +326,8 @@ extern "C" logismos_status_t logismos_launch_silu_mul_bf16(const void* gate_up_b
     const int64_t total = (int64_t)rows * inter;
     lg::silu_mul_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
                           static_cast<hipStream_t>(stream)>>>(
-        static_cast<const uint16_t*>(gate_up_bf16), static_cast<uint16_t*>(out_bf16), inter, total);
+        static_cast<const uint16_t*>(gate_up_bf16), nullptr, 0, 0,
+        static_cast<uint16_t*>(out_bf16), inter, total);
     return hipGetLastError();
 }
 

@@ -67,6 +67,11 @@ _SIGNATURES = {
     "logismos_launch_greedy_f32": (C.c_uint32, [_vp, _vp, _i, _i, _vp]),
     "logismos_decode_step_workspace_bytes": (_sz, [_vp, _i, _i]),
     "logismos_launch_decode_step": (C.c_uint32, [_vp, _vp, _vp, _vp, _vp]),
+    "logismos_qgemm_q4g128_splitk_parts": (C.c_int, [_i, _i, _i]),
+    "logismos_launch_qgemm_q4g128_f32_splitk": (C.c_uint32, [_vp] * 5 + [_i, _i, _i, _vp]),
+    "logismos_launch_add_rms_norm_f32p": (C.c_uint32, [_vp, _vp, _i, _vp, _vp, _i, _i, _f, _vp]),
+    "logismos_launch_rope_kv_write_f32p": (C.c_uint32, [_vp, _i] + [_vp] * 7 + [_i] * 5 + [_vp]),
+    "logismos_launch_silu_mul_f32p": (C.c_uint32, [_vp, _i, _vp, _i, _i, _vp]),
     "logismos_launch_probe_copy": (C.c_uint32, [_vp, _vp, _sz, _vp]),
     "logismos_launch_probe_read": (C.c_uint32, [_vp, _vp, _sz, _vp]),
 }
@@ -264,3 +269,35 @@ def launch_decode_step(cfg: DecodeConfig, layers, batch: DecodeBatch, workspace,
     """`layers` is a ctypes array of DecodeLayer (host memory)."""
     _status("decode_step", library().logismos_launch_decode_step(
         C.byref(cfg), C.cast(layers, _vp), C.byref(batch), _ptr(workspace), _raw(stream)))
+
+
+def qgemm_q4g128_splitk_parts(b: int, n: int, k: int) -> int:
+    return library().logismos_qgemm_q4g128_splitk_parts(b, n, k)
+
+
+def launch_qgemm_q4g128_f32_splitk(x, qw, scale, zero, parts, b: int, n: int, k: int,
+                                   stream=None) -> None:
+    check_qgemm_q4g128_shape(b, n, k)
+    _status("qgemm_q4g128_f32_splitk", library().logismos_launch_qgemm_q4g128_f32_splitk(
+        _ptr(x), _ptr(qw), _ptr(scale), _ptr(zero), _ptr(parts), b, n, k, _raw(stream)))
+
+
+def launch_add_rms_norm_f32p(h, parts, num_parts: int, w, out, rows: int, n: int, eps: float,
+                             stream=None) -> None:
+    _status("add_rms_norm_f32p", library().logismos_launch_add_rms_norm_f32p(
+        _ptr(h), _ptr(parts) if parts is not None else None, num_parts, _ptr(w), _ptr(out), rows,
+        n, float(eps), _raw(stream)))
+
+
+def launch_rope_kv_write_f32p(parts, num_parts: int, positions, cos, sin, slot_mapping, q_out,
+                              k_pool, v_pool, total_tokens: int, hq: int, hkv: int, head_dim: int,
+                              max_pos: int, stream=None) -> None:
+    _status("rope_kv_write_f32p", library().logismos_launch_rope_kv_write_f32p(
+        _ptr(parts), num_parts, _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping),
+        _ptr(q_out), _ptr(k_pool), _ptr(v_pool), total_tokens, hq, hkv, head_dim, max_pos,
+        _raw(stream)))
+
+
+def launch_silu_mul_f32p(parts, num_parts: int, out, rows: int, inter: int, stream=None) -> None:
+    _status("silu_mul_f32p", library().logismos_launch_silu_mul_f32p(
+        _ptr(parts), num_parts, _ptr(out), rows, inter, _raw(stream)))

@@ -353,6 +353,18 @@ def dequantize_q4g128(qw, scale, zero, n, k):
     return w
 
 
+_qgemm_q4_f32 = _sig("oracle_qgemm_q4g128_f32", None, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz)
+
+
+def qgemm_q4g128_f32(x_bf16_bits, qw, scale, zero, b, n, k):
+    x = _u16(x_bf16_bits)
+    qw = np.ascontiguousarray(qw, dtype=np.uint8)
+    scale, zero = _u16(scale), _u16(zero)
+    y = np.empty((b, n), np.float32)
+    _qgemm_q4_f32(_p(x), _p(qw), _p(scale), _p(zero), _p(y), b, n, k)
+    return y
+
+
 def qgemm_q4g128_bf16(x_bf16_bits, qw, scale, zero, b, n, k):
     x = _u16(x_bf16_bits)
     qw = np.ascontiguousarray(qw, dtype=np.uint8)

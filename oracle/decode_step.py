@@ -10,8 +10,8 @@ part of the definition and are the ones the GPU path uses:
 
   hidden state h ............ fp32
   normed activations ........ bf16   (input of every quantized GEMM)
-  GEMM outputs .............. bf16   (fp32 accumulation, one rounding)
-  q, and K/V in the cache ... fp16   (RoPE in fp32 on the bf16 GEMM output)
+  GEMM outputs .............. fp32   (consumed un-rounded by the next operator)
+  q, and K/V in the cache ... fp16   (RoPE in fp32 on the fp32 GEMM output)
   attention output .......... bf16   (one rounding of the fp32 result; feeds the o projection)
   silu(gate) * up ........... bf16
 """
@@ -22,19 +22,23 @@ import numpy as np
 import oracle as O
 
 
-def add_rms_norm_bf16(h: np.ndarray, y_bits, w, eps: float) -> np.ndarray:
-    """h (fp32, [rows, n]) += y (bf16 bits) in place; returns bf16 bits of rms_norm(h) * w."""
+def add_rms_norm_bf16(h: np.ndarray, y, w, eps: float) -> np.ndarray:
+    """h (fp32, [rows, n]) += y in place (y: bf16 bits, or fp32); returns bf16 bits of
+    rms_norm(h) * w."""
     rows, n = h.shape
-    if y_bits is not None:
-        h += O.bf16_bits_to_f32(y_bits).reshape(rows, n)
+    if y is not None:
+        y = np.asarray(y)
+        h += (y if y.dtype == np.float32 else O.bf16_bits_to_f32(y)).reshape(rows, n)
     return O.f32_to_bf16_bits(O.rms_norm(h, w, rows, n, eps)).reshape(rows, n)
 
 
-def rope_kv_write(qkv_bits, positions, cos, sin, slots, k_pool, v_pool, hq, hkv, d=128):
-    """qkv bf16 bits [T, (hq+2hkv)*d] -> q fp16 [T,hq,d]; roped k and v written into the pools."""
-    t = qkv_bits.shape[0]
+def rope_kv_write(qkv, positions, cos, sin, slots, k_pool, v_pool, hq, hkv, d=128):
+    """qkv (bf16 bits or fp32) [T, (hq+2hkv)*d] -> q fp16 [T,hq,d]; roped k and v written into
+    the pools."""
+    qkv = np.asarray(qkv)
+    t = qkv.shape[0]
     half = d // 2
-    x = O.bf16_bits_to_f32(qkv_bits).reshape(t, hq + 2 * hkv, d)
+    x = (qkv if qkv.dtype == np.float32 else O.bf16_bits_to_f32(qkv)).reshape(t, hq + 2 * hkv, d)
     q = np.ascontiguousarray(x[:, :hq]).reshape(t * hq, d)
     k = np.ascontiguousarray(x[:, hq:hq + hkv]).reshape(t * hkv, d)
     v = np.ascontiguousarray(x[:, hq + hkv:]).reshape(t, hkv * d)
@@ -53,8 +57,9 @@ def rope_kv_write(qkv_bits, positions, cos, sin, slots, k_pool, v_pool, hq, hkv,
     return q16
 
 
-def silu_mul_bf16(gate_up_bits, inter):
-    x = O.bf16_bits_to_f32(gate_up_bits)
+def silu_mul_bf16(gate_up, inter):
+    gate_up = np.asarray(gate_up)
+    x = gate_up if gate_up.dtype == np.float32 else O.bf16_bits_to_f32(gate_up)
     rows = x.shape[0]
     g = np.ascontiguousarray(x[:, :inter])
     u = np.ascontiguousarray(x[:, inter:])
@@ -68,7 +73,7 @@ def cast_f16_bf16(a16):
 def _gemm(x_bits, w, b):
     qw, s, z = w
     n, k = qw.shape[0], qw.shape[1] * 2
-    return O.qgemm_q4g128_bf16(np.ascontiguousarray(x_bits), qw, s, z, b, n, k)
+    return O.qgemm_q4g128_f32(np.ascontiguousarray(x_bits), qw, s, z, b, n, k)
 
 
 def decode_step(cfg, layers, batch, trace=None):

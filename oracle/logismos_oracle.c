@@ -504,9 +504,9 @@ void oracle_dequantize_q4g128(const uint8_t* qw, const uint16_t* scale, const ui
 /* linear_t (crates/kernels/src/cpu_f32/mod.rs:271-345) over the dequantised
  * matrix with bf16 activations: y[b][n] = bf16( sum_k x[b][k] * ((q-z)*s) ),
  * ascending k, fp32 accumulation, one rounding at the end. */
-void oracle_qgemm_q4g128_bf16(const uint16_t* x_bf16, const uint8_t* qw, const uint16_t* scale,
-                              const uint16_t* zero, uint16_t* y_bf16, size_t b, size_t n,
-                              size_t k) {
+static void qgemm_q4g128_core(const uint16_t* x_bf16, const uint8_t* qw, const uint16_t* scale,
+                              const uint16_t* zero, uint16_t* y_bf16, float* y_f32, size_t b,
+                              size_t n, size_t k) {
     size_t groups = k / 128;
     float* xf = (float*)malloc(b * k * sizeof(float));
     oracle_bf16_to_f32_n(x_bf16, xf, b * k);
@@ -528,12 +528,28 @@ void oracle_qgemm_q4g128_bf16(const uint16_t* x_bf16, const uint8_t* qw, const u
                 const float* xr = xf + bi * k;
                 float acc = 0.0f;
                 for (size_t c = 0; c < k; ++c) acc += xr[c] * wrow[c];
-                y_bf16[bi * n + (size_t)r] = oracle_f32_to_bf16(acc);
+                if (y_f32)
+                    y_f32[bi * n + (size_t)r] = acc;
+                else
+                    y_bf16[bi * n + (size_t)r] = oracle_f32_to_bf16(acc);
             }
         }
         free(wrow);
     }
     free(xf);
+}
+
+void oracle_qgemm_q4g128_bf16(const uint16_t* x_bf16, const uint8_t* qw, const uint16_t* scale,
+                              const uint16_t* zero, uint16_t* y_bf16, size_t b, size_t n,
+                              size_t k) {
+    qgemm_q4g128_core(x_bf16, qw, scale, zero, y_bf16, NULL, b, n, k);
+}
+
+/* The same product before its final rounding (the decode step keeps GEMM
+ * results in fp32 until the next operator). */
+void oracle_qgemm_q4g128_f32(const uint16_t* x_bf16, const uint8_t* qw, const uint16_t* scale,
+                             const uint16_t* zero, float* y_f32, size_t b, size_t n, size_t k) {
+    qgemm_q4g128_core(x_bf16, qw, scale, zero, NULL, y_f32, b, n, k);
 }
 
 /* ------------------------------------------------------------------ ragged packing / paged KV */

@@ -102,6 +102,9 @@ void oracle_qgemm_q4g128_bf16(const uint16_t* x_bf16, const uint8_t* qw, const u
                               const uint16_t* zero, uint16_t* y_bf16, size_t b, size_t n,
                               size_t k);
 
+void oracle_qgemm_q4g128_f32(const uint16_t* x_bf16, const uint8_t* qw, const uint16_t* scale,
+                             const uint16_t* zero, float* y_f32, size_t b, size_t n, size_t k);
+
 /* ---- ragged packing / paged KV */
 int oracle_pack_ragged(const int32_t* new_tokens, const int32_t* prior_ctx,
                        const int32_t* block_tables, int32_t* cu_seqlens, int64_t* slot_mapping,

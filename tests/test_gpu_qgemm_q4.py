@@ -95,3 +95,42 @@ def test_batch_rows_are_independent():
     assert np.array_equal(got2[1], got1[0])
     # the two kernels agree to bf16 rounding
     assert_parity(got4[1], got2[1], what="mfma vs gemv")
+
+
+# ------------------------------------------------------------------ split-K form (fp32 parts)
+def _run_splitk(x_f32, qw, s, z, b, n, k):
+    from logismos_amd import hip, kernels
+    xb = O.f32_to_bf16_bits(x_f32[:b])
+    j = kernels.qgemm_q4g128_splitk_parts(b, n, k)
+    assert j >= 1
+    d_parts = hip.DeviceBuffer(j * b * n * 4)
+    d_parts.fill(0xFF)
+    kernels.launch_qgemm_q4g128_f32_splitk(
+        hip.DeviceBuffer.from_numpy(xb), hip.DeviceBuffer.from_numpy(np.ascontiguousarray(qw)),
+        hip.DeviceBuffer.from_numpy(np.ascontiguousarray(s).view(np.uint16)),
+        hip.DeviceBuffer.from_numpy(np.ascontiguousarray(z).view(np.uint16)), d_parts, b, n, k)
+    hip.synchronize()
+    parts = d_parts.to_numpy(np.float32, (j, b, n))
+    assert np.isfinite(parts).all()
+    return parts.sum(axis=0, dtype=np.float32), O.qgemm_q4g128_f32(xb, qw, s, z, b, n, k), j
+
+
+@pytest.mark.parametrize("b", [1, 8, 16, 32])
+def test_splitk_config3_matches_oracle(b):
+    c, qw, s, z = _config3()
+    x = np.concatenate([c["x"], c["x"][::-1]])  # 32 rows
+    got, want, _ = _run_splitk(x, qw, s, z, b, c["n"], c["k"])
+    # fp32 result of fp32 accumulation: only the summation order differs
+    assert_parity(got, want, max_abs=2e-4, max_rel=1e-3, what=f"qgemm_q4 split-K batch {b}")
+
+
+@pytest.mark.parametrize("b,n,k", [(32, 6144, 4096), (32, 4096, 4096), (32, 24576, 4096),
+                                   (32, 4096, 12288), (5, 16, 128), (17, 33, 384),
+                                   (32, 1000, 1152), (31, 4100, 2048), (9, 70000, 256)])
+def test_splitk_ragged_shapes(b, n, k):
+    rng = np.random.default_rng(b * 1000003 + n * 101 + k)
+    w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
+    x = rng.standard_normal((b, k), np.float32)
+    qw, s, z = O.quantize_q4g128(w, n, k)
+    got, want, j = _run_splitk(x, qw, s, z, b, n, k)
+    assert_parity(got, want, max_abs=2e-4, max_rel=1e-3, what=f"split-K {b}x{n}x{k} (J={j})")

@@ -93,3 +93,63 @@ def test_greedy_first_maximum_wins():
     want = [O.greedy(logits[r]) for r in range(rows)]
     assert got.tolist() == want
     assert got[0] == 1 and got[1] == 5 and got[2] == 0
+
+
+def test_f32_parts_variants_add_the_parts_in_order():
+    rng = np.random.default_rng(24)
+    rows, n, j = 6, 2048, 3
+    # add_rms_norm over three fp32 parts
+    h = rng.standard_normal((rows, n), np.float32)
+    parts = rng.standard_normal((j, rows, n), np.float32)
+    w = (1 + 0.02 * rng.standard_normal(n)).astype(np.float32)
+    d_h, d_out = hip.DeviceBuffer.from_numpy(h), hip.DeviceBuffer(rows * n * 2)
+    kernels.launch_add_rms_norm_f32p(d_h, hip.DeviceBuffer.from_numpy(parts), j,
+                                     hip.DeviceBuffer.from_numpy(w), d_out, rows, n, 1e-6)
+    hip.synchronize()
+    y = (parts[0] + parts[1]) + parts[2]            # same order: bit-exact residual
+    h_ref = h + parts[0]
+    h_ref += parts[1]
+    h_ref += parts[2]
+    assert np.array_equal(d_h.to_numpy(np.float32, (rows, n)), h_ref)
+    want = O.f32_to_bf16_bits(O.rms_norm(h_ref, w, rows, n, 1e-6)).reshape(rows, n)
+    assert_parity(O.bf16_bits_to_f32(d_out.to_numpy(np.uint16, (rows, n))),
+                  O.bf16_bits_to_f32(want), what="add_rms_norm_f32p")
+    # zero parts: plain RMSNorm of h
+    d_h2 = hip.DeviceBuffer.from_numpy(h)
+    kernels.launch_add_rms_norm_f32p(d_h2, None, 0, hip.DeviceBuffer.from_numpy(w), d_out, rows, n,
+                                     1e-6)
+    hip.synchronize()
+    assert np.array_equal(d_h2.to_numpy(np.float32, (rows, n)), h)
+
+    # silu_mul over two parts
+    inter = 1000
+    gp = rng.standard_normal((2, rows, 2 * inter), np.float32)
+    d_o = hip.DeviceBuffer(rows * inter * 2)
+    kernels.launch_silu_mul_f32p(hip.DeviceBuffer.from_numpy(gp), 2, d_o, rows, inter)
+    hip.synchronize()
+    want = OS.silu_mul_bf16(gp[0] + gp[1], inter)
+    assert_parity(O.bf16_bits_to_f32(d_o.to_numpy(np.uint16, (rows, inter))),
+                  O.bf16_bits_to_f32(want), what="silu_mul_f32p")
+
+    # rope over two parts
+    t, hq, hkv, d, bs, nblk, max_pos = 5, 4, 2, 128, 16, 8, 512
+    qp = rng.standard_normal((2, t, (hq + 2 * hkv) * d), np.float32)
+    positions = np.array([0, 3, 511, 17, 100], np.int32)
+    slots = rng.permutation(nblk * bs)[:t].astype(np.int64)
+    cos, sin = O.build_rope_table_f32(max_pos, d, 1_000_000.0)
+    k_pool = np.zeros((nblk * bs, hkv * d), np.float16)
+    v_pool = np.zeros((nblk * bs, hkv * d), np.float16)
+    d_kp, d_vp = hip.DeviceBuffer.from_numpy(k_pool), hip.DeviceBuffer.from_numpy(v_pool)
+    d_q = hip.DeviceBuffer(t * hq * d * 2)
+    kernels.launch_rope_kv_write_f32p(
+        hip.DeviceBuffer.from_numpy(qp), 2, hip.DeviceBuffer.from_numpy(positions),
+        hip.DeviceBuffer.from_numpy(cos), hip.DeviceBuffer.from_numpy(sin),
+        hip.DeviceBuffer.from_numpy(slots), d_q, d_kp, d_vp, t, hq, hkv, d, max_pos)
+    hip.synchronize()
+    q_want = OS.rope_kv_write(qp[0] + qp[1], positions, cos, sin, slots, k_pool, v_pool, hq, hkv, d)
+    assert_parity(d_q.to_numpy(np.float16, (t, hq, d)), q_want, max_abs=1e-3, max_rel=2e-3,
+                  what="rope_f32p q")
+    assert_parity(d_kp.to_numpy(np.float16, k_pool.shape), k_pool, max_abs=1e-3, max_rel=2e-3,
+                  what="rope_f32p k")
+    assert np.array_equal(d_vp.to_numpy(np.float16, v_pool.shape).view(np.uint16),
+                          v_pool.view(np.uint16))
