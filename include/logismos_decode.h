@@ -163,6 +163,22 @@ logismos_status_t logismos_launch_qgemm_q4g128_f32_splitk(const void* x_bf16, co
                                                           int b, int n, int k,
                                                           logismos_stream_t stream);
 
+/* Prepared activations.  The MFMA kernels want x in "pair order" with per-group
+ * sums; a producer that writes x in that form once saves every GEMM workgroup
+ * from rebuilding it.  Layout (b <= 32 rows, BP = 16 for b <= 16 else 32):
+ *   uint4 xp[K/8][BP]    8 consecutive bf16 x0..x7 of row r, chunk c, stored as
+ *                        the pairs (x0,x4) (x1,x5) (x2,x6) (x3,x7)
+ *   float xg[K/128][BP]  sum of the bf16 values of each group of 128, after xp.
+ * `logismos_q4_xprep_bytes` sizes the buffer, `logismos_launch_q4_prepare_x_bf16`
+ * converts a plain bf16 `[b][K]` matrix, `..._splitk_xprep` consumes it.  The
+ * step operators below can emit it directly (`out_prepared != 0`). */
+size_t logismos_q4_xprep_bytes(int b, int k);
+logismos_status_t logismos_launch_q4_prepare_x_bf16(const void* x_bf16, void* x_prepared, int b,
+                                                    int k, logismos_stream_t stream);
+logismos_status_t logismos_launch_qgemm_q4g128_f32_splitk_xprep(
+    const void* x_prepared, const void* qw_u8, const void* scale_f16, const void* zero_f16,
+    void* parts_f32, int b, int n, int k, logismos_stream_t stream);
+
 /* ggml Q8_0 block stream `[N][K/32]{f16 d; int8 qs[32]}` -> planar Q8G32. */
 logismos_status_t logismos_launch_repack_q8_0(const void* blocks_q8_0, void* qs_i8, void* d_f16,
                                               int n, int k, logismos_stream_t stream);
@@ -311,6 +327,16 @@ logismos_status_t logismos_launch_rope_kv_write_f32p(
 logismos_status_t logismos_launch_silu_mul_f32p(const void* parts_f32, int num_parts,
                                                 void* out_bf16, int rows, int inter,
                                                 logismos_stream_t stream);
+
+/* The same with the result in the prepared layout of the next GEMM (rows <= 32,
+ * width % 128 == 0; see `logismos_q4_xprep_bytes`). */
+logismos_status_t logismos_launch_add_rms_norm_f32p_xprep(void* h_f32, const void* parts_f32,
+                                                          int num_parts, const void* w_f32,
+                                                          void* x_prepared, int rows, int n,
+                                                          float eps, logismos_stream_t stream);
+logismos_status_t logismos_launch_silu_mul_f32p_xprep(const void* parts_f32, int num_parts,
+                                                      void* x_prepared, int rows, int inter,
+                                                      logismos_stream_t stream);
 
 /* out[r] = first index of the maximum of logits[r][:] (`decode::greedy`,
  * crates/decode/src/lib.rs:73-83: strict >, the first maximum wins). */

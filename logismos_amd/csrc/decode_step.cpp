@@ -10,13 +10,13 @@
 namespace {
 
 struct Workspace {
-    char* xn;        // bf16 [B][hidden]
+    char* xn;        // prepared activations of width hidden (input of qkv / gate_up)
     char* qkv;       // f32  [Jqkv][B][(hq+2hkv)*d]   split-K parts
     char* q;         // f16  [B][hq*d]
-    char* attn_b;    // bf16 [B][hq*d]
+    char* attn_b;    // prepared activations of width hq*d (input of the o projection)
     char* proj;      // f32  [max(Jo,Jdown)][B][hidden]  (o projection, then down projection)
     char* gate_up;   // f32  [Jgu][B][2*inter]
-    char* act;       // bf16 [B][inter]
+    char* act;       // prepared activations of width inter (input of the down projection)
     char* attn_ws;   // split-K workspace of the attention
     int j_qkv, j_o, j_gu, j_down;
     size_t total;
@@ -39,13 +39,13 @@ Workspace carve(const logismos_decode_config_t& c, int b, int num_splits, char* 
     w.j_gu = logismos_qgemm_q4g128_splitk_parts(b, 2 * c.intermediate, c.hidden);
     w.j_down = logismos_qgemm_q4g128_splitk_parts(b, c.hidden, c.intermediate);
     const int j_proj = w.j_o > w.j_down ? w.j_o : w.j_down;
-    w.xn = take((size_t)b * c.hidden * 2);
+    w.xn = take(logismos_q4_xprep_bytes(b, c.hidden));
     w.qkv = take((size_t)w.j_qkv * b * (qd + 2 * kvd) * 4);
     w.q = take((size_t)b * qd * 2);
-    w.attn_b = take((size_t)b * qd * 2);
+    w.attn_b = take(logismos_q4_xprep_bytes(b, (int)qd));
     w.proj = take((size_t)j_proj * b * c.hidden * 4);
     w.gate_up = take((size_t)w.j_gu * b * 2 * c.intermediate * 4);
-    w.act = take((size_t)b * c.intermediate * 2);
+    w.act = take(logismos_q4_xprep_bytes(b, c.intermediate));
     w.attn_ws = take(logismos_paged_attn_workspace_bytes(b, c.num_q_heads, c.head_dim, num_splits));
     w.total = off;
     return w;
@@ -93,32 +93,34 @@ extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_c
     int res_parts = 0;  // split-K parts of the projection the next add_rms_norm folds into h
     for (int l = 0; l < c.num_layers; ++l) {
         const logismos_decode_layer_t& L = layers[l];
-        LG_TRY(logismos_launch_add_rms_norm_f32p(batch->hidden_f32, w.proj, res_parts,
-                                                 L.norm1_w_f32, w.xn, b, c.hidden, c.rms_eps,
-                                                 stream));
-        LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk(w.xn, L.qkv.qw, L.qkv.scale, L.qkv.zero,
-                                                       w.qkv, b, qd + 2 * kvd, c.hidden, stream));
+        LG_TRY(logismos_launch_add_rms_norm_f32p_xprep(batch->hidden_f32, w.proj, res_parts,
+                                                       L.norm1_w_f32, w.xn, b, c.hidden, c.rms_eps,
+                                                       stream));
+        LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk_xprep(
+            w.xn, L.qkv.qw, L.qkv.scale, L.qkv.zero, w.qkv, b, qd + 2 * kvd, c.hidden, stream));
         LG_TRY(logismos_launch_rope_kv_write_f32p(
             w.qkv, w.j_qkv, batch->positions, batch->rope_cos_f32, batch->rope_sin_f32,
             batch->slot_mapping, w.q, L.k_pool_f16, L.v_pool_f16, b, c.num_q_heads, c.num_kv_heads,
             c.head_dim, c.max_pos, stream));
-        // attention writes bf16 directly: its output only feeds the o projection
+        // attention writes the prepared layout directly: its output only feeds the o projection
         LG_TRY(lg::paged_attn_launch(
             w.q, L.k_pool_f16, L.v_pool_f16, batch->block_tables, batch->cu_seqlens,
             batch->context_lens, w.attn_b, w.attn_ws, b, b, 1, c.num_q_heads, c.num_kv_heads,
             c.head_dim, c.block_size, c.max_blocks_per_seq, batch->num_splits, scale, 1,
-            LOGISMOS_ATTN_PHASE_ALL, 1, stream));
-        LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk(w.attn_b, L.o.qw, L.o.scale, L.o.zero,
-                                                       w.proj, b, c.hidden, qd, stream));
-        LG_TRY(logismos_launch_add_rms_norm_f32p(batch->hidden_f32, w.proj, w.j_o, L.norm2_w_f32,
-                                                 w.xn, b, c.hidden, c.rms_eps, stream));
-        LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk(w.xn, L.gate_up.qw, L.gate_up.scale,
-                                                       L.gate_up.zero, w.gate_up, b,
-                                                       2 * c.intermediate, c.hidden, stream));
-        LG_TRY(logismos_launch_silu_mul_f32p(w.gate_up, w.j_gu, w.act, b, c.intermediate, stream));
-        LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk(w.act, L.down.qw, L.down.scale, L.down.zero,
-                                                       w.proj, b, c.hidden, c.intermediate,
+            LOGISMOS_ATTN_PHASE_ALL, 2, stream));
+        LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk_xprep(w.attn_b, L.o.qw, L.o.scale, L.o.zero,
+                                                             w.proj, b, c.hidden, qd, stream));
+        LG_TRY(logismos_launch_add_rms_norm_f32p_xprep(batch->hidden_f32, w.proj, w.j_o,
+                                                       L.norm2_w_f32, w.xn, b, c.hidden, c.rms_eps,
                                                        stream));
+        LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk_xprep(w.xn, L.gate_up.qw, L.gate_up.scale,
+                                                             L.gate_up.zero, w.gate_up, b,
+                                                             2 * c.intermediate, c.hidden, stream));
+        LG_TRY(logismos_launch_silu_mul_f32p_xprep(w.gate_up, w.j_gu, w.act, b, c.intermediate,
+                                                   stream));
+        LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk_xprep(w.act, L.down.qw, L.down.scale,
+                                                             L.down.zero, w.proj, b, c.hidden,
+                                                             c.intermediate, stream));
         res_parts = w.j_down;
     }
     LG_TRY(logismos_launch_add_rms_norm_f32p(batch->hidden_f32, w.proj, res_parts,

@@ -31,6 +31,7 @@
 // + G * 256 * 2 (q, out) + 4 * ceil(ctx/block_size) (block table).
 #include "device_utils.hpp"
 #include "launch_common.hpp"
+#include "q4_common.hpp"
 
 #include <hip/hip_fp16.h>
 #include <math.h>
@@ -66,7 +67,10 @@ struct AttnParams {
     int part_tokens;  // keys per partition (multiple of 16)
     float scale_log2e;
     int causal;
-    int out_bf16;  // write `out` as bf16 instead of fp16 (the step executor feeds a bf16 GEMM)
+    // 0: fp16 [T][hq][128]; 1: bf16, same shape; 2: the prepared layout of the following
+    // Q4G128 GEMM (x = [out_rows][hq*128], see q4_common.hpp) -- what the step executor uses
+    int out_bf16;
+    int out_rows;
 };
 
 __device__ __forceinline__ unsigned short attn_out_elem(float v, int out_bf16) {
@@ -118,9 +122,21 @@ __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_kernel(const At
         // no visible key: zeros (softmax over zero columns)
         if (split == 0 && c < G) {
             half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
-            _Float16* o = p.out + ((int64_t)t * p.hq + kvh * G + c) * kHeadDim;
+            if (p.out_bf16 == 2) {
+                const int bp = xprep_bp(p.out_rows);
+                const int head = kvh * G + c;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) *reinterpret_cast<half8_t*>(o + 8 * (tg + 4 * j)) = z;
+                for (int j = 0; j < 4; ++j)
+                    reinterpret_cast<half8_t*>(p.out)[(int64_t)(head * 16 + tg + 4 * j) * bp + t] = z;
+                if (tg == 0)
+                    reinterpret_cast<float*>(
+                        reinterpret_cast<char*>(p.out) +
+                        xprep_xg_offset(p.out_rows, p.hq * kHeadDim))[(int64_t)head * bp + t] = 0.0f;
+            } else {
+                _Float16* o = p.out + ((int64_t)t * p.hq + kvh * G + c) * kHeadDim;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) *reinterpret_cast<half8_t*>(o + 8 * (tg + 4 * j)) = z;
+            }
         }
         return;
     }
@@ -272,7 +288,20 @@ __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_kernel(const At
                 for (int e = 0; e < 4; ++e)
                     o[e] = (unsigned)attn_out_elem(acc[h][2 * e] * inv, p.out_bf16) |
                            ((unsigned)attn_out_elem(acc[h][2 * e + 1] * inv, p.out_bf16) << 16);
-                *reinterpret_cast<uint4_t*>(p.out + ((int64_t)t * p.hq + head) * kHeadDim + 8 * c) = o;
+                if (p.out_bf16 == 2) {
+                    // a head is one group of 128: the 16 lanes of this row hold its 16 chunks
+                    const float gs = row16_sum(sum8_bf16(o));
+                    const int bp = xprep_bp(p.out_rows);
+                    reinterpret_cast<uint4_t*>(p.out)[(int64_t)(head * 16 + c) * bp + t] =
+                        pair_order(o);
+                    if (c == 0)
+                        reinterpret_cast<float*>(
+                            reinterpret_cast<char*>(p.out) +
+                            xprep_xg_offset(p.out_rows, p.hq * kHeadDim))[(int64_t)head * bp + t] = gs;
+                } else {
+                    *reinterpret_cast<uint4_t*>(p.out + ((int64_t)t * p.hq + head) * kHeadDim +
+                                                8 * c) = o;
+                }
             } else {
                 const int64_t idx = ((int64_t)s * p.num_splits + split) * p.hq + head;
                 float4_t a0 = {acc[h][0], acc[h][1], acc[h][2], acc[h][3]};
@@ -339,6 +368,7 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams 
         M = mx;
     }
     __shared__ float sm[4], sden[4], sn[4][kHeadDim];
+    __shared__ __attribute__((aligned(16))) unsigned short sout[kHeadDim];
     if (lane == 0) {
         sm[w] = M;
         sden[w] = den;
@@ -356,8 +386,25 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams 
             dd = fmaf(g, sden[j], dd);
             num = fmaf(g, sn[j][d], num);
         }
-        reinterpret_cast<unsigned short*>(p.out)[((int64_t)t0 * p.hq + h) * kHeadDim + d] =
-            attn_out_elem(num / dd, p.out_bf16);
+        const unsigned short ov = attn_out_elem(num / dd, p.out_bf16);
+        if (p.out_bf16 != 2)
+            reinterpret_cast<unsigned short*>(p.out)[((int64_t)t0 * p.hq + h) * kHeadDim + d] = ov;
+        else
+            sout[d] = ov;
+    }
+    if (p.out_bf16 == 2) {
+        __syncthreads();
+        if (threadIdx.x < 16) {
+            const int c = threadIdx.x;
+            const uint4_t o = reinterpret_cast<const uint4_t*>(sout)[c];
+            const float gs = row16_sum(sum8_bf16(o));
+            const int bp = xprep_bp(p.out_rows);
+            reinterpret_cast<uint4_t*>(p.out)[(int64_t)(h * 16 + c) * bp + t0] = pair_order(o);
+            if (c == 0)
+                reinterpret_cast<float*>(
+                    reinterpret_cast<char*>(p.out) +
+                    xprep_xg_offset(p.out_rows, p.hq * kHeadDim))[(int64_t)h * bp + t0] = gs;
+        }
     }
 }
 
@@ -525,6 +572,7 @@ logismos_status_t lg::paged_attn_launch(
     p.scale_log2e = scale * lg::kLog2e;
     p.causal = causal;
     p.out_bf16 = out_bf16;
+    p.out_rows = total_tokens;
 
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (num_q_heads / num_kv_heads) {

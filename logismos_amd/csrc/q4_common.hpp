@@ -40,6 +40,20 @@ __device__ __forceinline__ float sum8_bf16(uint4_t d) {
 constexpr unsigned kNibMask = 0x000F000Fu;
 
 
+// "Prepared" form of a batch of activations for the Q4G128 MFMA kernels: what the
+// kernels otherwise build in LDS per workgroup, built once by the producer.
+//   xp  uint4 [K/8][BP]   chunk c of batch row r: its 8 bf16 in pair order
+//   xg  float [K/128][BP] sum of the (bf16-rounded) x over each group
+// BP = 16 for up to 16 batch rows, else 32; rows >= b are never read for a stored
+// result (row i of the MFMA A operand only reaches row i of the product).
+__host__ __device__ inline int xprep_bp(int b) { return b <= 16 ? 16 : 32; }
+__host__ __device__ inline size_t xprep_xg_offset(int b, int k) {
+    return (size_t)(k / 8) * xprep_bp(b) * 16;
+}
+__host__ __device__ inline size_t xprep_bytes(int b, int k) {
+    return xprep_xg_offset(b, k) + (size_t)(k / 128) * xprep_bp(b) * 4;
+}
+
 inline int device_cu_count() {
     static const int count = [] {
         int dev = 0, cus = 0;

@@ -12,9 +12,9 @@
 // coalesced copy, and the K parts of different workgroups are summed by the
 // consumer instead of through shared accumulators.
 //
-// Per workgroup (1024 threads): x part -> LDS in pair order (+ per-group sums of
-// x), scale/zero of its rows and groups -> LDS; wave w owns row tile w, w+16, ..
-// and for each issues its GP 16-byte loads per lane (one per group) up front.
+// Per workgroup (4 waves): x part -> LDS in pair order (+ per-group sums of x),
+// scale/zero of its rows and groups -> LDS; every wave owns TW row tiles and
+// issues their TW*GP 16-byte loads per lane (one per tile and group) up front.
 // Dequantisation is the same magic-number trick as in qgemm_q4.hip; the weight
 // tile is the MFMA B operand, x from LDS the A operand.  Loads retire in order,
 // so x, scale and zero are requested BEFORE the weights: waiting for them does
@@ -25,30 +25,37 @@
 
 #include <hip/hip_fp16.h>
 #include <math.h>
+#include <stdlib.h>
 
 namespace lg {
 
-constexpr int kSplitkThreads = 1024;
+constexpr int kSplitkWaves = 4;
+constexpr int kSplitkThreads = 64 * kSplitkWaves;
 
-template <int BT, int GP>
+// BT batch tiles of 16 rows of x, GP groups per K part, TW row tiles per wave
+// (a workgroup owns 4*TW*16 weight rows).  Small workgroups on purpose: several
+// are resident per CU at different stages (staging x / waiting for weights /
+// MFMA), which overlaps what a single big workgroup would serialise.
+template <int BT, int GP, int TW, bool PREP>
 __global__ __launch_bounds__(kSplitkThreads) void qgemm_q4g128_splitk_kernel(
     const uint16_t* __restrict__ x, const uint8_t* __restrict__ qw,
     const __half* __restrict__ scale, const __half* __restrict__ zero, float* __restrict__ part,
-    int b, int n, int k, int tiles_per_wg) {
+    int b, int n, int k) {
     extern __shared__ uint4_t lds[];
     constexpr int BP = BT * 16;
-    constexpr int QS = GP * 16 + 1;  // row stride of xl in 16-byte words, == 1 (mod 16)
+    // xl: PREP ? [GP*16 chunks][BP] (the prepared layout itself) : [BP][QS], QS == 1 (mod 16)
+    constexpr int QS = GP * 16 + 1;
+    constexpr int ROWS = kSplitkWaves * TW * 16;
     const int groups = k >> 7;
     const int j = blockIdx.y;
     const int g0 = j * GP;
     const int gcount = min(GP, groups - g0);
-    const int rows_wg = tiles_per_wg * 16;
-    const int64_t row0 = (int64_t)blockIdx.x * rows_wg;
-    const int rows_here = (int)min((int64_t)rows_wg, (int64_t)n - row0);
+    const int64_t row0 = (int64_t)blockIdx.x * ROWS;
+    const int rows_here = (int)min((int64_t)ROWS, (int64_t)n - row0);
 
-    uint4_t* xl = lds;                                          // [BP][QS]
-    float* xg = reinterpret_cast<float*>(lds + BP * QS);        // [GP][BP]
-    __half* szl = reinterpret_cast<__half*>(xg + GP * BP);      // scale [rows_wg][GP], zero [..]
+    uint4_t* xl = lds;                                      // [BP][QS]
+    float* xg = reinterpret_cast<float*>(lds + BP * QS);    // [GP][BP]
+    __half* szl = reinterpret_cast<__half*>(xg + GP * BP);  // scale [ROWS][GP], zero [ROWS][GP]
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -61,17 +68,30 @@ __global__ __launch_bounds__(kSplitkThreads) void qgemm_q4g128_splitk_kernel(
     // ---- requests, in the order they must retire: x, scale/zero, weights
     constexpr int U = (BP * GP * 16 + kSplitkThreads - 1) / kSplitkThreads;
     const int chunks = gcount * 16;
-    const int x_total = chunks * b;
+    const int x_total = PREP ? chunks * BP : chunks * b;
     uint4_t xd[U];
+    float xgd = 0.0f;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const int idx = u * kSplitkThreads + (int)threadIdx.x;
         const int idc = idx < x_total ? idx : x_total - 1;
-        const int bi = idc / chunks, q = idc - bi * chunks;
-        xd[u] = *reinterpret_cast<const uint4_t*>(x + (int64_t)bi * k + (int64_t)g0 * 128 +
-                                                  (int64_t)q * 8);
+        if constexpr (PREP) {
+            // the K part of the prepared x is one contiguous block of 16-byte words
+            xd[u] = reinterpret_cast<const uint4_t*>(x)[(int64_t)g0 * 16 * BP + idc];
+        } else {
+            const int bi = idc / chunks, q = idc - bi * chunks;
+            xd[u] = *reinterpret_cast<const uint4_t*>(x + (int64_t)bi * k + (int64_t)g0 * 128 +
+                                                      (int64_t)q * 8);
+        }
     }
-    constexpr int SZU = (256 * GP + kSplitkThreads - 1) / kSplitkThreads;  // rows_wg <= 256
+    if constexpr (PREP) {
+        static_assert(GP * BP <= kSplitkThreads, "one group sum per thread");
+        const float* xg_src = reinterpret_cast<const float*>(
+            reinterpret_cast<const char*>(x) + xprep_xg_offset(b, k));
+        const int t = (int)threadIdx.x < gcount * BP ? (int)threadIdx.x : 0;
+        xgd = xg_src[(int64_t)g0 * BP + t];
+    }
+    constexpr int SZU = (ROWS * GP + kSplitkThreads - 1) / kSplitkThreads;
     const int sz_total = rows_here * gcount;
     __half sd[SZU], zd[SZU];
 #pragma unroll
@@ -84,32 +104,43 @@ __global__ __launch_bounds__(kSplitkThreads) void qgemm_q4g128_splitk_kernel(
     }
     __builtin_amdgcn_sched_barrier(0);
 
-    auto load_tile = [&](int t, uint4_t (&w)[GP]) {
-        const int r = t * 16 + col;
+    // this wave's TW tiles: rows (wave*TW + t)*16 .. +16
+    uint4_t w[TW][GP];
+#pragma unroll
+    for (int t = 0; t < TW; ++t) {
+        const int r = (wave * TW + t) * 16 + col;
         const uint8_t* wrow =
             qw + (row0 + (r < rows_here ? r : rows_here - 1)) * (int64_t)(k >> 1) + kc * 16;
 #pragma unroll
         for (int i = 0; i < GP; ++i) {
             const int g = (i < gcount) ? (g0 + i) : (g0 + gcount - 1);
-            w[i] = *reinterpret_cast<const uint4_t*>(wrow + (int64_t)g * 64);
+#ifdef LG_EXP_NOWLOAD
+            w[t][i] = uint4_t{0x12345678u, (unsigned)g, 0x9abcdef0u, (unsigned)lane};
+#else
+            w[t][i] = *reinterpret_cast<const uint4_t*>(wrow + (int64_t)g * 64);
+#endif
         }
-    };
-    uint4_t w[GP];
-    int t = wave;
-    if (t < tiles_per_wg) load_tile(t, w);
+    }
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- x, scale, zero into LDS
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const int idx = u * kSplitkThreads + (int)threadIdx.x;
-        const int idc = idx < x_total ? idx : x_total - 1;
-        const int bi = idc / chunks, q = idc - bi * chunks;
-        const float gs = row16_sum(sum8_bf16(xd[u]));  // 16 chunks of a group = 16 lanes
-        if (idx < x_total) {
-            xl[bi * QS + q] = pair_order(xd[u]);
-            if ((lane & 15) == 0) xg[(q >> 4) * BP + bi] = gs;
+        if constexpr (PREP) {
+            if (idx < x_total) xl[idx] = xd[u];
+        } else {
+            const int idc = idx < x_total ? idx : x_total - 1;
+            const int bi = idc / chunks, q = idc - bi * chunks;
+            const float gs = row16_sum(sum8_bf16(xd[u]));  // 16 chunks of a group = 16 lanes
+            if (idx < x_total) {
+                xl[bi * QS + q] = pair_order(xd[u]);
+                if ((lane & 15) == 0) xg[(q >> 4) * BP + bi] = gs;
+            }
         }
+    }
+    if constexpr (PREP) {
+        if ((int)threadIdx.x < gcount * BP) xg[threadIdx.x] = xgd;
     }
 #pragma unroll
     for (int u = 0; u < SZU; ++u) {
@@ -117,15 +148,15 @@ __global__ __launch_bounds__(kSplitkThreads) void qgemm_q4g128_splitk_kernel(
         if (idx < sz_total) {
             const int r = idx / gcount, g = idx - r * gcount;
             szl[r * GP + g] = sd[u];
-            szl[rows_wg * GP + r * GP + g] = zd[u];
+            szl[ROWS * GP + r * GP + g] = zd[u];
         }
     }
     __syncthreads();
-    const __half* zl = szl + rows_wg * GP;
+    const __half* zl = szl + ROWS * GP;
 
-    for (; t < tiles_per_wg; t += kSplitkThreads / 64) {
-        if (t != wave) load_tile(t, w);
-        const int r = t * 16 + col;
+#pragma unroll
+    for (int t = 0; t < TW; ++t) {
+        const int r = (wave * TW + t) * 16 + col;
         const int rl = r < rows_here ? r : rows_here - 1;
         float4_t ysum[BT];
 #pragma unroll
@@ -140,7 +171,7 @@ __global__ __launch_bounds__(kSplitkThreads) void qgemm_q4g128_splitk_kernel(
             for (int bt = 0; bt < BT; ++bt) acc[bt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int s4 = 0; s4 < 4; ++s4) {
-                const unsigned wd = w[i][s4];
+                const unsigned wd = w[t][i][s4];
                 uint4_t h;
 #pragma unroll
                 for (int sft = 0; sft < 4; ++sft) h[sft] = ((wd >> (4 * sft)) & kNibMask) | magic;
@@ -149,8 +180,9 @@ __global__ __launch_bounds__(kSplitkThreads) void qgemm_q4g128_splitk_kernel(
 #pragma unroll
                 for (int bt = 0; bt < BT; ++bt)
                     acc[bt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                        __builtin_bit_cast(bf16x8_t, xl[(bt * 16 + col) * QS + q]), bop, acc[bt], 0,
-                        0, 0);
+                        __builtin_bit_cast(bf16x8_t, PREP ? xl[q * BP + bt * 16 + col]
+                                                          : xl[(bt * 16 + col) * QS + q]),
+                        bop, acc[bt], 0, 0, 0);
             }
 #pragma unroll
             for (int bt = 0; bt < BT; ++bt) {
@@ -162,6 +194,9 @@ __global__ __launch_bounds__(kSplitkThreads) void qgemm_q4g128_splitk_kernel(
                     ysum[bt][e] = valid ? v : ysum[bt][e];
                 }
             }
+            // one group at a time: without this the scheduler hoists the LDS reads of
+            // every group (GP*4*BT operands of four registers) and spills
+            __builtin_amdgcn_sched_barrier(0);
         }
         if (r < rows_here) {
 #pragma unroll
@@ -169,22 +204,27 @@ __global__ __launch_bounds__(kSplitkThreads) void qgemm_q4g128_splitk_kernel(
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int bi = bt * 16 + 4 * kc + e;
-                    if (bi < b) part[((int64_t)j * b + bi) * n + row0 + r] = ysum[bt][e];
+#ifdef LG_EXP_NOSTORE
+                    if (bi < b && ysum[bt][e] == 12345.678f)
+#else
+                    if (bi < b)
+#endif
+                        part[((int64_t)j * b + bi) * n + row0 + r] = ysum[bt][e];
                 }
         }
     }
 }
 
 struct SplitkPlan {
-    int tiles_per_wg;  // 16-row tiles per workgroup (rows = 16 * tiles_per_wg <= 256)
-    int gp;            // groups per K part
-    int parts;         // J = ceil(groups / gp)
+    int tw;     // row tiles per wave (rows per workgroup = 64 * tw)
+    int gp;     // groups per K part
+    int parts;  // J = ceil(groups / gp)
 };
 
 // Deterministic in (b, n, k) and the CU count.  Cost relative to the weight
 // bytes: 1 (weights) + x re-reads (128/R per 32 batch rows, served by L2)
-// + partial write + read (4/gp per 32 batch rows), times the idle fraction when
-// fewer workgroups than CUs exist.
+// + partial write + read (4/gp per 32 batch rows, mostly cache-resident), times
+// the idle fraction when the workgroups do not fill the CUs evenly.
 static SplitkPlan splitk_plan(int b, int n, int k) {
     const int groups = k / 128;
     const int tiles = (n + 15) / 16;
@@ -192,59 +232,68 @@ static SplitkPlan splitk_plan(int b, int n, int k) {
     const double bs = (double)b / 32.0;
     SplitkPlan best{1, 1, groups};
     double best_cost = 1e30;
-    const int tpws[] = {4, 8, 16};
-    const int gps[] = {1, 2, 4, 8};
-    for (int tpw : tpws)
+#ifdef LG_EXP_PLAN_ENV
+    if (const char* e = getenv("LG_PLAN")) {
+        int gp = 1, tw = 1;
+        if (sscanf(e, "%d,%d", &gp, &tw) == 2) return SplitkPlan{tw, gp, (groups + gp - 1) / gp};
+    }
+#endif
+    const int tws[] = {1, 2, 4};
+    const int gps[] = {1, 2, 4};
+    for (int tw : tws)
         for (int gp : gps) {
             if (gp > groups && gp != 1) continue;
+            if (b > 16 && tw * gp > 8) continue;  // register budget with two batch tiles
             const int parts = (groups + gp - 1) / gp;
+            const int tpw = kSplitkWaves * tw;
             const long wgs = (long)((tiles + tpw - 1) / tpw) * parts;
             const double r = 16.0 * tpw;
-            double cost = 1.0 + 0.35 * bs * 128.0 / r + bs * 4.0 / gp;
-            const double waves_of_wgs = (double)wgs / cus;
-            // a partially filled last round of workgroups idles part of the chip
-            const double rounds = waves_of_wgs <= 1.0 ? 1.0 : ceil(waves_of_wgs);
-            cost *= rounds / waves_of_wgs;
+            double cost = 1.0 + 0.35 * bs * 128.0 / r + 0.5 * bs * 4.0 / gp;
+            // four workgroups fit a CU: count rounds of 4*cus workgroups
+            const double fill = (double)wgs / (4.0 * cus);
+            const double rounds = fill <= 1.0 ? 1.0 : ceil(fill);
+            cost *= rounds / (fill < 0.25 ? 0.25 : fill);
             if (cost < best_cost) {
                 best_cost = cost;
-                best = SplitkPlan{tpw, gp, parts};
+                best = SplitkPlan{tw, gp, parts};
             }
         }
     return best;
 }
 
-template <int BT, int GP>
+template <int BT, int GP, int TW, bool PREP>
 static hipError_t launch_splitk(const void* x, const void* qw, const void* scale, const void* zero,
                                 void* part, int b, int n, int k, const SplitkPlan& plan,
                                 hipStream_t stream) {
     constexpr int BP = BT * 16;
+    constexpr int ROWS = kSplitkWaves * TW * 16;
     const int tiles = (n + 15) / 16;
-    const size_t lds = (size_t)BP * (GP * 16 + 1) * 16 + (size_t)GP * BP * 4 +
-                       (size_t)2 * plan.tiles_per_wg * 16 * GP * 2;
-    auto kern = qgemm_q4g128_splitk_kernel<BT, GP>;
-    if (lds > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-    }
-    dim3 grid((tiles + plan.tiles_per_wg - 1) / plan.tiles_per_wg, plan.parts);
+    const size_t lds =
+        (size_t)BP * (GP * 16 + 1) * 16 + (size_t)GP * BP * 4 + (size_t)2 * ROWS * GP * 2;
+    auto kern = qgemm_q4g128_splitk_kernel<BT, GP, TW, PREP>;
+    dim3 grid((tiles + kSplitkWaves * TW - 1) / (kSplitkWaves * TW), plan.parts);
     kern<<<grid, dim3(kSplitkThreads), lds, stream>>>(
         static_cast<const uint16_t*>(x), static_cast<const uint8_t*>(qw),
         static_cast<const __half*>(scale), static_cast<const __half*>(zero),
-        static_cast<float*>(part), b, n, k, plan.tiles_per_wg);
+        static_cast<float*>(part), b, n, k);
     return hipGetLastError();
 }
 
-template <int BT>
+template <int BT, bool PREP>
 static hipError_t launch_splitk_bt(const void* x, const void* qw, const void* scale,
                                    const void* zero, void* part, int b, int n, int k,
                                    const SplitkPlan& plan, hipStream_t stream) {
-    switch (plan.gp) {
-        case 1: return launch_splitk<BT, 1>(x, qw, scale, zero, part, b, n, k, plan, stream);
-        case 2: return launch_splitk<BT, 2>(x, qw, scale, zero, part, b, n, k, plan, stream);
-        case 4: return launch_splitk<BT, 4>(x, qw, scale, zero, part, b, n, k, plan, stream);
-        default: return launch_splitk<BT, 8>(x, qw, scale, zero, part, b, n, k, plan, stream);
+#define LG_SPLITK_CASE(GP, TW)                                                                  \
+    if (plan.gp == GP && plan.tw == TW)                                                         \
+        return launch_splitk<BT, GP, TW, PREP>(x, qw, scale, zero, part, b, n, k, plan, stream);
+    LG_SPLITK_CASE(1, 1) LG_SPLITK_CASE(1, 2) LG_SPLITK_CASE(1, 4)
+    LG_SPLITK_CASE(2, 1) LG_SPLITK_CASE(2, 2) LG_SPLITK_CASE(2, 4)
+    LG_SPLITK_CASE(4, 1) LG_SPLITK_CASE(4, 2)
+    if constexpr (BT == 1) {
+        LG_SPLITK_CASE(4, 4)
     }
+#undef LG_SPLITK_CASE
+    return hipErrorInvalidValue;
 }
 
 }  // namespace lg
@@ -254,17 +303,79 @@ extern "C" int logismos_qgemm_q4g128_splitk_parts(int b, int n, int k) {
     return lg::splitk_plan(b, n, k).parts;
 }
 
-extern "C" logismos_status_t logismos_launch_qgemm_q4g128_f32_splitk(
-    const void* x_bf16, const void* qw_u8, const void* scale_f16, const void* zero_f16,
-    void* parts_f32, int b, int n, int k, logismos_stream_t stream) {
+static logismos_status_t splitk_dispatch(const void* x, bool prepared, const void* qw_u8,
+                                         const void* scale_f16, const void* zero_f16,
+                                         void* parts_f32, int b, int n, int k,
+                                         logismos_stream_t stream) {
     if (logismos_check_qgemm_q4g128_shape(b, n, k, nullptr, 0) != 0) return hipErrorInvalidValue;
-    if (!x_bf16 || !qw_u8 || !scale_f16 || !zero_f16 || !parts_f32) return hipErrorInvalidValue;
-    if ((reinterpret_cast<uintptr_t>(qw_u8) & 15u) || (reinterpret_cast<uintptr_t>(x_bf16) & 15u))
+    if (!x || !qw_u8 || !scale_f16 || !zero_f16 || !parts_f32) return hipErrorInvalidValue;
+    if ((reinterpret_cast<uintptr_t>(qw_u8) & 15u) || (reinterpret_cast<uintptr_t>(x) & 15u))
         return hipErrorInvalidValue;
     const lg::SplitkPlan plan = lg::splitk_plan(b, n, k);
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (prepared) {
+        if (b <= 16)
+            return lg::launch_splitk_bt<1, true>(x, qw_u8, scale_f16, zero_f16, parts_f32, b, n, k,
+                                                 plan, st);
+        return lg::launch_splitk_bt<2, true>(x, qw_u8, scale_f16, zero_f16, parts_f32, b, n, k, plan,
+                                             st);
+    }
     if (b <= 16)
-        return lg::launch_splitk_bt<1>(x_bf16, qw_u8, scale_f16, zero_f16, parts_f32, b, n, k, plan,
-                                       st);
-    return lg::launch_splitk_bt<2>(x_bf16, qw_u8, scale_f16, zero_f16, parts_f32, b, n, k, plan, st);
+        return lg::launch_splitk_bt<1, false>(x, qw_u8, scale_f16, zero_f16, parts_f32, b, n, k,
+                                              plan, st);
+    return lg::launch_splitk_bt<2, false>(x, qw_u8, scale_f16, zero_f16, parts_f32, b, n, k, plan,
+                                          st);
+}
+
+extern "C" logismos_status_t logismos_launch_qgemm_q4g128_f32_splitk(
+    const void* x_bf16, const void* qw_u8, const void* scale_f16, const void* zero_f16,
+    void* parts_f32, int b, int n, int k, logismos_stream_t stream) {
+    return splitk_dispatch(x_bf16, false, qw_u8, scale_f16, zero_f16, parts_f32, b, n, k, stream);
+}
+
+extern "C" logismos_status_t logismos_launch_qgemm_q4g128_f32_splitk_xprep(
+    const void* x_prepared, const void* qw_u8, const void* scale_f16, const void* zero_f16,
+    void* parts_f32, int b, int n, int k, logismos_stream_t stream) {
+    return splitk_dispatch(x_prepared, true, qw_u8, scale_f16, zero_f16, parts_f32, b, n, k, stream);
+}
+
+extern "C" size_t logismos_q4_xprep_bytes(int b, int k) {
+    if (b <= 0 || b > 32 || k <= 0 || k % 128 != 0) return 0;
+    return lg::xprep_bytes(b, k);
+}
+
+namespace lg {
+// bf16 x [b][k] -> prepared form; one thread per 8-element chunk
+__global__ __launch_bounds__(256) void q4_prepare_x_kernel(const uint16_t* __restrict__ x,
+                                                           void* __restrict__ xprep, int b, int k) {
+    const int bp = xprep_bp(b);
+    const int chunks = k >> 3;
+    const int idx = blockIdx.x * 256 + threadIdx.x;  // chunk-major inside a batch row
+    const int bi = idx / chunks, c = idx - bi * chunks;
+    const bool live = bi < b;
+    uint4_t d = uint4_t{0u, 0u, 0u, 0u};
+    if (live) d = *reinterpret_cast<const uint4_t*>(x + (int64_t)bi * k + (int64_t)c * 8);
+    const float gs = row16_sum(sum8_bf16(d));
+    if (live) {
+        reinterpret_cast<uint4_t*>(xprep)[(int64_t)c * bp + bi] = pair_order(d);
+        if ((threadIdx.x & 15) == 0)
+            reinterpret_cast<float*>(reinterpret_cast<char*>(xprep) +
+                                     xprep_xg_offset(b, k))[(int64_t)(c >> 4) * bp + bi] = gs;
+    }
+}
+}  // namespace lg
+
+extern "C" logismos_status_t logismos_launch_q4_prepare_x_bf16(const void* x_bf16, void* x_prepared,
+                                                               int b, int k,
+                                                               logismos_stream_t stream) {
+    if (b <= 0 || b > 32 || k <= 0 || k % 128 != 0 || (int64_t)b * k > (int64_t)INT32_MAX)
+        return hipErrorInvalidValue;
+    if (!x_bf16 || !x_prepared || (reinterpret_cast<uintptr_t>(x_bf16) & 15u) ||
+        (reinterpret_cast<uintptr_t>(x_prepared) & 15u))
+        return hipErrorInvalidValue;
+    const int items = b * (k / 8);
+    lg::q4_prepare_x_kernel<<<dim3((items + 255) / 256), dim3(256), 0,
+                              static_cast<hipStream_t>(stream)>>>(
+        static_cast<const uint16_t*>(x_bf16), x_prepared, b, k);
+    return hipGetLastError();
 }

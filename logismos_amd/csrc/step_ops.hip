@@ -5,6 +5,7 @@
 // sizes: they exist to keep the step on the GPU between the big kernels.
 #include "device_utils.hpp"
 #include "launch_common.hpp"
+#include "q4_common.hpp"
 
 #include <hip/hip_fp16.h>
 #include <math.h>
@@ -104,6 +105,143 @@ __global__ __launch_bounds__(kNormThreads) void add_rms_norm_kernel(
     } else {
         for (int j = threadIdx.x; j < n; j += kNormThreads)
             out[row * n + j] = f32_to_bf16(hr[j] * inv * w[j]);
+    }
+}
+
+// The step's form of the same operator: y arrives as fp32 split-K parts and the
+// normed row leaves in the prepared layout of the next Q4G128 GEMM (pair order
+// + per-group sums).  512 threads per row, eight consecutive elements (one
+// 16-byte chunk of the output) per thread and pass; n % 128 == 0.
+constexpr int kPrepThreads = 512;
+constexpr int kPrepMaxPasses = 4;  // rows up to 16384 wide
+
+__global__ __launch_bounds__(kPrepThreads) void add_rms_norm_xprep_kernel(
+    float* __restrict__ h, const float* __restrict__ yp, int num_parts, int64_t part_stride,
+    const float* __restrict__ w, void* __restrict__ xprep, int rows, int n, float eps) {
+    const int64_t row = blockIdx.x;
+    float* hr = h + row * n;
+    float v[kPrepMaxPasses][8];
+    float sum_sq = 0.0f;
+#pragma unroll
+    for (int p = 0; p < kPrepMaxPasses; ++p) {
+        const int j = (p * kPrepThreads + (int)threadIdx.x) * 8;
+        if (j < n) {
+            const float4_t a = *reinterpret_cast<const float4_t*>(hr + j);
+            const float4_t b = *reinterpret_cast<const float4_t*>(hr + j + 4);
+            float4_t s0 = a, s1 = b;
+            // h + part 0 + part 1 + ... in this order; four loads in flight per round
+            for (int q0 = 0; q0 < num_parts; q0 += 4) {
+                float4_t t0[4], t1[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int q = (q0 + u) < num_parts ? (q0 + u) : q0;
+                    const float* src = yp + (int64_t)q * part_stride + row * n + j;
+                    t0[u] = *reinterpret_cast<const float4_t*>(src);
+                    t1[u] = *reinterpret_cast<const float4_t*>(src + 4);
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    if (q0 + u < num_parts) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            s0[e] += t0[u][e];
+                            s1[e] += t1[u][e];
+                        }
+                    }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                v[p][e] = s0[e];
+                v[p][4 + e] = s1[e];
+            }
+            if (num_parts > 0) {
+                *reinterpret_cast<float4_t*>(hr + j) = float4_t{v[p][0], v[p][1], v[p][2], v[p][3]};
+                *reinterpret_cast<float4_t*>(hr + j + 4) =
+                    float4_t{v[p][4], v[p][5], v[p][6], v[p][7]};
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sum_sq = fmaf(v[p][e], v[p][e], sum_sq);
+        }
+    }
+    __shared__ float part[kPrepThreads / 64];
+    sum_sq = wave_sum(sum_sq);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = sum_sq;
+    __syncthreads();
+    float total = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kPrepThreads / 64; ++i) total += part[i];
+    const float inv = 1.0f / sqrtf(total / (float)n + eps);
+    const int bp = xprep_bp(rows);
+    uint4_t* xp = reinterpret_cast<uint4_t*>(xprep);
+    float* xg = reinterpret_cast<float*>(reinterpret_cast<char*>(xprep) + xprep_xg_offset(rows, n));
+#pragma unroll
+    for (int p = 0; p < kPrepMaxPasses; ++p) {
+        const int c = p * kPrepThreads + (int)threadIdx.x;  // chunk index
+        const int j = c * 8;
+        const bool live = j < n;  // uniform over each group of 16 threads (n % 128 == 0)
+        uint4_t o = {0u, 0u, 0u, 0u};
+        if (live) {
+            const float4_t w0 = *reinterpret_cast<const float4_t*>(w + j);
+            const float4_t w1 = *reinterpret_cast<const float4_t*>(w + j + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float lo = v[p][2 * e] * inv * (2 * e < 4 ? w0[2 * e] : w1[2 * e - 4]);
+                const float hi = v[p][2 * e + 1] * inv * (2 * e + 1 < 4 ? w0[2 * e + 1] : w1[2 * e - 3]);
+                o[e] = (unsigned)f32_to_bf16(lo) | ((unsigned)f32_to_bf16(hi) << 16);
+            }
+        }
+        const float gs = row16_sum(sum8_bf16(o));
+        if (live) {
+            xp[(int64_t)c * bp + row] = pair_order(o);
+            if ((threadIdx.x & 15) == 0) xg[(int64_t)(c >> 4) * bp + row] = gs;
+        }
+    }
+}
+
+// act = silu(gate) * up from the fp32 parts of the gate_up GEMM, written in the
+// prepared layout of the down projection.  One thread per 8 outputs.
+__global__ __launch_bounds__(256) void silu_mul_xprep_kernel(const float* __restrict__ parts,
+                                                             int num_parts, int64_t part_stride,
+                                                             void* __restrict__ xprep, int rows,
+                                                             int inter) {
+    const int chunks = inter >> 3;
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    const int t = idx / chunks, c = idx - t * chunks;
+    const bool live = t < rows;  // uniform over groups of 16 threads (inter % 128 == 0)
+    uint4_t o = {0u, 0u, 0u, 0u};
+    if (live) {
+        float g[8], u[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) g[e] = u[e] = 0.0f;
+        const int64_t base = (int64_t)t * 2 * inter + (int64_t)c * 8;
+        for (int q = 0; q < num_parts; ++q) {
+            const float* src = parts + (int64_t)q * part_stride + base;
+            const float4_t g0 = *reinterpret_cast<const float4_t*>(src);
+            const float4_t g1 = *reinterpret_cast<const float4_t*>(src + 4);
+            const float4_t u0 = *reinterpret_cast<const float4_t*>(src + inter);
+            const float4_t u1 = *reinterpret_cast<const float4_t*>(src + inter + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                g[e] += g0[e];
+                g[4 + e] += g1[e];
+                u[e] += u0[e];
+                u[4 + e] += u1[e];
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float a = g[2 * e] / (1.0f + expf(-g[2 * e])) * u[2 * e];
+            const float b = g[2 * e + 1] / (1.0f + expf(-g[2 * e + 1])) * u[2 * e + 1];
+            o[e] = (unsigned)f32_to_bf16(a) | ((unsigned)f32_to_bf16(b) << 16);
+        }
+    }
+    const float gs = row16_sum(sum8_bf16(o));
+    if (live) {
+        const int bp = xprep_bp(rows);
+        reinterpret_cast<uint4_t*>(xprep)[(int64_t)c * bp + t] = pair_order(o);
+        if ((threadIdx.x & 15) == 0)
+            reinterpret_cast<float*>(reinterpret_cast<char*>(xprep) +
+                                     xprep_xg_offset(rows, inter))[(int64_t)(c >> 4) * bp + t] = gs;
     }
 }
 
@@ -349,5 +487,36 @@ extern "C" logismos_status_t logismos_launch_greedy_f32(const void* logits_f32, 
     if (!logits_f32 || !out_u32) return hipErrorInvalidValue;
     lg::greedy_kernel<<<dim3(rows), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
         static_cast<const float*>(logits_f32), static_cast<uint32_t*>(out_u32), n);
+    return hipGetLastError();
+}
+
+extern "C" logismos_status_t logismos_launch_add_rms_norm_f32p_xprep(
+    void* h_f32, const void* parts_f32, int num_parts, const void* w_f32, void* x_prepared, int rows,
+    int n, float eps, logismos_stream_t stream) {
+    if (rows <= 0 || rows > 32 || n <= 0 || n % 128 != 0 ||
+        n > 8 * lg::kPrepThreads * lg::kPrepMaxPasses)
+        return hipErrorInvalidValue;
+    if (!h_f32 || !w_f32 || !x_prepared || num_parts < 0 || (num_parts > 0 && !parts_f32))
+        return hipErrorInvalidValue;
+    lg::add_rms_norm_xprep_kernel<<<dim3(rows), dim3(lg::kPrepThreads), 0,
+                                    static_cast<hipStream_t>(stream)>>>(
+        static_cast<float*>(h_f32), static_cast<const float*>(parts_f32), num_parts,
+        (int64_t)rows * n, static_cast<const float*>(w_f32), x_prepared, rows, n, eps);
+    return hipGetLastError();
+}
+
+extern "C" logismos_status_t logismos_launch_silu_mul_f32p_xprep(const void* parts_f32,
+                                                                 int num_parts, void* x_prepared,
+                                                                 int rows, int inter,
+                                                                 logismos_stream_t stream) {
+    if (rows <= 0 || rows > 32 || inter <= 0 || inter % 128 != 0 || num_parts <= 0 ||
+        (int64_t)rows * inter * 2 > (int64_t)INT32_MAX)
+        return hipErrorInvalidValue;
+    if (!parts_f32 || !x_prepared) return hipErrorInvalidValue;
+    const int items = rows * (inter / 8);
+    lg::silu_mul_xprep_kernel<<<dim3((items + 255) / 256), dim3(256), 0,
+                                static_cast<hipStream_t>(stream)>>>(
+        static_cast<const float*>(parts_f32), num_parts, (int64_t)rows * 2 * inter, x_prepared, rows,
+        inter);
     return hipGetLastError();
 }

@@ -72,6 +72,12 @@ _SIGNATURES = {
     "logismos_launch_add_rms_norm_f32p": (C.c_uint32, [_vp, _vp, _i, _vp, _vp, _i, _i, _f, _vp]),
     "logismos_launch_rope_kv_write_f32p": (C.c_uint32, [_vp, _i] + [_vp] * 7 + [_i] * 5 + [_vp]),
     "logismos_launch_silu_mul_f32p": (C.c_uint32, [_vp, _i, _vp, _i, _i, _vp]),
+    "logismos_q4_xprep_bytes": (_sz, [_i, _i]),
+    "logismos_launch_q4_prepare_x_bf16": (C.c_uint32, [_vp, _vp, _i, _i, _vp]),
+    "logismos_launch_qgemm_q4g128_f32_splitk_xprep": (C.c_uint32, [_vp] * 5 + [_i, _i, _i, _vp]),
+    "logismos_launch_add_rms_norm_f32p_xprep":
+        (C.c_uint32, [_vp, _vp, _i, _vp, _vp, _i, _i, _f, _vp]),
+    "logismos_launch_silu_mul_f32p_xprep": (C.c_uint32, [_vp, _i, _vp, _i, _i, _vp]),
     "logismos_launch_probe_copy": (C.c_uint32, [_vp, _vp, _sz, _vp]),
     "logismos_launch_probe_read": (C.c_uint32, [_vp, _vp, _sz, _vp]),
 }
@@ -276,10 +282,21 @@ def qgemm_q4g128_splitk_parts(b: int, n: int, k: int) -> int:
 
 
 def launch_qgemm_q4g128_f32_splitk(x, qw, scale, zero, parts, b: int, n: int, k: int,
-                                   stream=None) -> None:
+                                   stream=None, prepared: bool = False) -> None:
     check_qgemm_q4g128_shape(b, n, k)
-    _status("qgemm_q4g128_f32_splitk", library().logismos_launch_qgemm_q4g128_f32_splitk(
-        _ptr(x), _ptr(qw), _ptr(scale), _ptr(zero), _ptr(parts), b, n, k, _raw(stream)))
+    fn = (library().logismos_launch_qgemm_q4g128_f32_splitk_xprep if prepared
+          else library().logismos_launch_qgemm_q4g128_f32_splitk)
+    _status("qgemm_q4g128_f32_splitk", fn(_ptr(x), _ptr(qw), _ptr(scale), _ptr(zero), _ptr(parts),
+                                          b, n, k, _raw(stream)))
+
+
+def q4_xprep_bytes(b: int, k: int) -> int:
+    return library().logismos_q4_xprep_bytes(b, k)
+
+
+def launch_q4_prepare_x_bf16(x, xprep, b: int, k: int, stream=None) -> None:
+    _status("q4_prepare_x_bf16", library().logismos_launch_q4_prepare_x_bf16(
+        _ptr(x), _ptr(xprep), b, k, _raw(stream)))
 
 
 def launch_add_rms_norm_f32p(h, parts, num_parts: int, w, out, rows: int, n: int, eps: float,
@@ -301,3 +318,16 @@ def launch_rope_kv_write_f32p(parts, num_parts: int, positions, cos, sin, slot_m
 def launch_silu_mul_f32p(parts, num_parts: int, out, rows: int, inter: int, stream=None) -> None:
     _status("silu_mul_f32p", library().logismos_launch_silu_mul_f32p(
         _ptr(parts), num_parts, _ptr(out), rows, inter, _raw(stream)))
+
+
+def launch_add_rms_norm_f32p_xprep(h, parts, num_parts: int, w, xprep, rows: int, n: int,
+                                   eps: float, stream=None) -> None:
+    _status("add_rms_norm_f32p_xprep", library().logismos_launch_add_rms_norm_f32p_xprep(
+        _ptr(h), _ptr(parts) if parts is not None else None, num_parts, _ptr(w), _ptr(xprep), rows,
+        n, float(eps), _raw(stream)))
+
+
+def launch_silu_mul_f32p_xprep(parts, num_parts: int, xprep, rows: int, inter: int,
+                               stream=None) -> None:
+    _status("silu_mul_f32p_xprep", library().logismos_launch_silu_mul_f32p_xprep(
+        _ptr(parts), num_parts, _ptr(xprep), rows, inter, _raw(stream)))

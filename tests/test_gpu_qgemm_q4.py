@@ -98,17 +98,24 @@ def test_batch_rows_are_independent():
 
 
 # ------------------------------------------------------------------ split-K form (fp32 parts)
-def _run_splitk(x_f32, qw, s, z, b, n, k):
+def _run_splitk(x_f32, qw, s, z, b, n, k, prepared=False):
     from logismos_amd import hip, kernels
     xb = O.f32_to_bf16_bits(x_f32[:b])
     j = kernels.qgemm_q4g128_splitk_parts(b, n, k)
     assert j >= 1
     d_parts = hip.DeviceBuffer(j * b * n * 4)
     d_parts.fill(0xFF)
+    d_x = hip.DeviceBuffer.from_numpy(xb)
+    if prepared:
+        d_xp = hip.DeviceBuffer(kernels.q4_xprep_bytes(b, k))
+        d_xp.fill(0xFF)  # padding rows stay NaN: they must not leak into stored results
+        kernels.launch_q4_prepare_x_bf16(d_x, d_xp, b, k)
+        d_x = d_xp
     kernels.launch_qgemm_q4g128_f32_splitk(
-        hip.DeviceBuffer.from_numpy(xb), hip.DeviceBuffer.from_numpy(np.ascontiguousarray(qw)),
+        d_x, hip.DeviceBuffer.from_numpy(np.ascontiguousarray(qw)),
         hip.DeviceBuffer.from_numpy(np.ascontiguousarray(s).view(np.uint16)),
-        hip.DeviceBuffer.from_numpy(np.ascontiguousarray(z).view(np.uint16)), d_parts, b, n, k)
+        hip.DeviceBuffer.from_numpy(np.ascontiguousarray(z).view(np.uint16)), d_parts, b, n, k,
+        prepared=prepared)
     hip.synchronize()
     parts = d_parts.to_numpy(np.float32, (j, b, n))
     assert np.isfinite(parts).all()
@@ -134,3 +141,16 @@ def test_splitk_ragged_shapes(b, n, k):
     qw, s, z = O.quantize_q4g128(w, n, k)
     got, want, j = _run_splitk(x, qw, s, z, b, n, k)
     assert_parity(got, want, max_abs=2e-4, max_rel=1e-3, what=f"split-K {b}x{n}x{k} (J={j})")
+
+
+@pytest.mark.parametrize("b,n,k", [(32, 6144, 4096), (32, 4096, 12288), (5, 16, 128),
+                                   (17, 33, 384), (16, 1000, 1152), (31, 4100, 2048)])
+def test_splitk_with_prepared_x_is_bit_identical(b, n, k):
+    rng = np.random.default_rng(b * 1000003 + n * 101 + k + 1)
+    w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
+    x = rng.standard_normal((b, k), np.float32)
+    qw, s, z = O.quantize_q4g128(w, n, k)
+    plain, want, _ = _run_splitk(x, qw, s, z, b, n, k)
+    prep, _, _ = _run_splitk(x, qw, s, z, b, n, k, prepared=True)
+    assert np.array_equal(plain, prep)
+    assert_parity(prep, want, max_abs=2e-4, max_rel=1e-3, what="split-K, prepared x")

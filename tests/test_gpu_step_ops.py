@@ -153,3 +153,56 @@ def test_f32_parts_variants_add_the_parts_in_order():
                   what="rope_f32p k")
     assert np.array_equal(d_vp.to_numpy(np.float16, v_pool.shape).view(np.uint16),
                           v_pool.view(np.uint16))
+
+
+def _unprepare(buf, b, k):
+    """prepared layout -> (bf16 bits [b][k], group sums [b][k/128])"""
+    bp = 16 if b <= 16 else 32
+    chunks = k // 8
+    xp = buf[: chunks * bp * 16].view(np.uint16).reshape(chunks, bp, 8)
+    # pair order (x0,x4)(x1,x5)(x2,x6)(x3,x7) -> natural
+    nat = np.empty_like(xp)
+    nat[..., [0, 4, 1, 5, 2, 6, 3, 7]] = xp
+    x = nat.transpose(1, 0, 2).reshape(bp, k)[:b]
+    xg = buf[chunks * bp * 16:].view(np.float32).reshape(k // 128, bp).T[:b]
+    return x, xg
+
+
+def test_prepared_layout_producers_match_the_plain_ones():
+    rng = np.random.default_rng(25)
+    rows, n, j = 20, 4096, 5
+    h = rng.standard_normal((rows, n), np.float32)
+    parts = rng.standard_normal((j, rows, n), np.float32)
+    w = (1 + 0.02 * rng.standard_normal(n)).astype(np.float32)
+    d_w, d_parts = hip.DeviceBuffer.from_numpy(w), hip.DeviceBuffer.from_numpy(parts)
+    d_h1, d_h2 = hip.DeviceBuffer.from_numpy(h), hip.DeviceBuffer.from_numpy(h)
+    d_plain = hip.DeviceBuffer(rows * n * 2)
+    d_prep = hip.DeviceBuffer(kernels.q4_xprep_bytes(rows, n))
+    kernels.launch_add_rms_norm_f32p(d_h1, d_parts, j, d_w, d_plain, rows, n, 1e-6)
+    kernels.launch_add_rms_norm_f32p_xprep(d_h2, d_parts, j, d_w, d_prep, rows, n, 1e-6)
+    hip.synchronize()
+    assert np.array_equal(d_h1.to_numpy(np.float32, (rows, n)), d_h2.to_numpy(np.float32, (rows, n)))
+    x, xg = _unprepare(d_prep.to_numpy(np.uint8, (d_prep.nbytes,)), rows, n)
+    plain = d_plain.to_numpy(np.uint16, (rows, n))
+    # the two kernels reduce the sum of squares in a different order: allow one bf16 ulp
+    assert_parity(O.bf16_bits_to_f32(x), O.bf16_bits_to_f32(plain), max_abs=1e-6, max_rel=8e-3,
+                  what="prepared add_rms_norm")
+    assert np.abs(xg - O.bf16_bits_to_f32(x).reshape(rows, n // 128, 128).sum(axis=2)).max() < 1e-3
+
+    inter = 1536
+    gp = rng.standard_normal((3, rows, 2 * inter), np.float32)
+    d_gp = hip.DeviceBuffer.from_numpy(gp)
+    d_o = hip.DeviceBuffer(rows * inter * 2)
+    d_op = hip.DeviceBuffer(kernels.q4_xprep_bytes(rows, inter))
+    kernels.launch_silu_mul_f32p(d_gp, 3, d_o, rows, inter)
+    kernels.launch_silu_mul_f32p_xprep(d_gp, 3, d_op, rows, inter)
+    hip.synchronize()
+    x, xg = _unprepare(d_op.to_numpy(np.uint8, (d_op.nbytes,)), rows, inter)
+    assert np.array_equal(x, d_o.to_numpy(np.uint16, (rows, inter)))
+    assert np.abs(xg - O.bf16_bits_to_f32(x).reshape(rows, inter // 128, 128).sum(axis=2)).max() < 1e-3
+    # prepare kernel on the plain output gives the same bytes
+    d_op2 = hip.DeviceBuffer(kernels.q4_xprep_bytes(rows, inter))
+    kernels.launch_q4_prepare_x_bf16(d_o, d_op2, rows, inter)
+    hip.synchronize()
+    x2, xg2 = _unprepare(d_op2.to_numpy(np.uint8, (d_op2.nbytes,)), rows, inter)
+    assert np.array_equal(x2, x) and np.array_equal(xg2, xg)
