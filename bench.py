@@ -9,7 +9,7 @@ in HBM.  Prints ONE JSON line.  `value` is decode tokens per second;
 `roofline` prices the dominant kernel alone (HIP events around back-to-back
 launches of only the paged-attention decode kernel on the launch stream);
 `cpu_baseline` is the CPU oracle timed on this box's host cores on a bounded
-sample of the same workload.  The per-kernel legs (configs 1-3) are reported in
+sample of the same workload.  The per-kernel legs (configs 1-4) are reported in
 the same line under their own keys.
 
 Cold-HBM timing: the KV pools (or weights) are replicated so that consecutive
@@ -170,6 +170,107 @@ def bench_paged_decode(args):
                          "sample": f"{reps} passes of the same config-2 batch in {el:.1f} s"},
         "parity_max_abs_vs_oracle": max_abs,
         "host_wall_ms_per_step": round(wall_ms, 5),
+    }
+
+
+def bench_mixed_config4(args):
+    """Config 4: 48 decode rows + 16 prefill chunks of 512 tokens in one packed token buffer.
+    One step = GPU-side packing (cu_seqlens, slot mapping, context lengths), the K/V rows of
+    the new tokens scattered into the paged pools, ragged attention over the whole batch."""
+    import oracle as O
+    case = workloads.config4()
+    stream = hip.Stream()
+    rng = np.random.default_rng(99)
+    S = len(case["new_tokens"])
+    T = int(case["cu_seqlens"][-1])
+    row = case["hkv"] * case["d"]
+    k_new = rng.standard_normal((T, row), np.float32).astype(np.float16)
+    v_new = rng.standard_normal((T, row), np.float32).astype(np.float16)
+    cu_h, slots_h, ctx_h, _ = O.pack_ragged(case["new_tokens"], case["prior_ctx"],
+                                            case["block_tables"], case["block_size"])
+    # the attention runner reads what the packer wrote on the GPU, not host-built copies
+    r = PagedAttnRunner(case, stream=stream)
+    d_new = hip.DeviceBuffer.from_numpy(case["new_tokens"])
+    d_prior = hip.DeviceBuffer.from_numpy(case["prior_ctx"])
+    d_slots = hip.DeviceBuffer(T * 8)
+    r.cu.fill(0xFF)
+    r.ctx.fill(0xFF)
+    d_knew = hip.DeviceBuffer.from_numpy(k_new)
+    d_vnew = hip.DeviceBuffer.from_numpy(v_new)
+
+    def pack():
+        kernels.launch_pack_ragged(d_new, d_prior, r.bt, r.cu, d_slots, r.ctx, S,
+                                   case["block_size"], case["max_blocks"], stream)
+
+    def write():
+        kernels.launch_kv_write_fp16(d_knew, d_vnew, r.k_pool, r.v_pool, d_slots, T, case["hkv"],
+                                     case["d"], stream)
+
+    def step():
+        pack()
+        write()
+        r.launch()
+
+    step()
+    got = r.result()
+    pack_ok = (np.array_equal(r.cu.to_numpy(np.int32, (S + 1,)), cu_h)
+               and np.array_equal(d_slots.to_numpy(np.int64, (T,)), slots_h)
+               and np.array_equal(r.ctx.to_numpy(np.int32, (S,)), ctx_h))
+    # parity sample: the prefill chunk with the shortest context and three decode rows, as a
+    # reduced batch for the oracle over the pools with the new rows written
+    kp, vp = case["k_pool"].copy(), case["v_pool"].copy()
+    kp[slots_h] = k_new
+    vp[slots_h] = v_new
+    pre = [s for s in range(S) if case["new_tokens"][s] > 1]
+    dec = [s for s in range(S) if case["new_tokens"][s] == 1]
+    pick = [min(pre, key=lambda s: case["context_lens"][s])] + \
+        sorted(dec, key=lambda s: case["context_lens"][s])[:3]
+    sub_q = np.concatenate([case["q"][cu_h[s]:cu_h[s + 1]] for s in pick])
+    sub_cu = np.concatenate([[0], np.cumsum(case["new_tokens"][pick])]).astype(np.int32)
+    want = O.paged_attn_varlen_fp16(sub_q, kp, vp, case["block_tables"][pick], sub_cu,
+                                    case["context_lens"][pick], case["hq"], case["hkv"],
+                                    case["d"], case["block_size"], case["scale"], True)
+    sub_got = np.concatenate([got[cu_h[s]:cu_h[s + 1]] for s in pick])
+    max_abs = float(np.abs(sub_got.astype(np.float32) - want.astype(np.float32)).max())
+
+    steps, warmup = max(10, args.steps // 10), 3
+    ms_step, wall_ms, graphed = time_launches(stream, [step], steps, warmup)
+    ms_pack, _, _ = time_launches(stream, [pack], steps, warmup)
+    ms_write, _, _ = time_launches(stream, [write], steps, warmup)
+    ms_pre, _, _ = time_launches(
+        stream, [lambda: r.launch(phases=kernels.ATTN_PHASE_PREFILL)], steps, warmup)
+    ms_dec, _, _ = time_launches(
+        stream, [lambda: r.launch(phases=kernels.ATTN_PHASE_DECODE)], steps, warmup)
+    ms_merge, _, _ = time_launches(
+        stream, [lambda: r.launch(phases=kernels.ATTN_PHASE_MERGE)], steps, warmup)
+
+    is_dec = case["new_tokens"] == 1
+    sub = lambda m: {**case, "new_tokens": case["new_tokens"][m],  # noqa: E731
+                     "context_lens": case["context_lens"][m]}
+    flops_pre = workloads.paged_attn_flops(sub(~is_dec))
+    ctx_dec = case["context_lens"][is_dec].astype(np.int64)
+    dec_bytes = int(ctx_dec.sum()) * 2 * row * 2
+    return {
+        "metric": "mixed chunked-prefill + decode attention step, new tokens/s",
+        "value": round(T / (ms_step * 1e-3), 1), "unit": "tokens/s",
+        "ms_per_step": round(ms_step, 4), "steps": steps, "warmup": warmup, "dtype": "f16",
+        "config": {"workload": "config 4: 48 decode rows (ctx log-uniform 128..32768) + 16 prefill "
+                               "chunks x 512 tokens (prior 0..8192), 32 q / 8 kv heads, head_dim "
+                               "128, block 16; one layer's packing + KV write + attention",
+                   "total_new_tokens": T, "sum_ctx": int(case["context_lens"].sum()),
+                   "num_splits": r.num_splits, "hip_graph": graphed},
+        "kernels_ms": {"pack_ragged": round(ms_pack, 4), "kv_write": round(ms_write, 4),
+                       "prefill": round(ms_pre, 4), "decode": round(ms_dec, 4),
+                       "merge": round(ms_merge, 4)},
+        "roofline": {"bound": "mfma", "achieved": round(flops_pre / (ms_pre * 1e-3) / 1e12, 1),
+                     "peak": 2500.0, "unit": "TFLOP/s",
+                     "frac": round(flops_pre / (ms_pre * 1e-3) / 1e12 / 2500.0, 4),
+                     "traffic": None, "kernel": "paged_attn_prefill_kernel<4,2>",
+                     "flops_per_launch": flops_pre},
+        "decode_rows_GBps": round(dec_bytes / (ms_dec * 1e-3) / 1e9, 1),
+        "gpu_packing_bit_exact": bool(pack_ok),
+        "parity_max_abs_vs_oracle": max_abs,
+        "parity_sample": f"sequences {pick} (1 prefill chunk, 3 decode rows)",
     }
 
 
@@ -392,6 +493,7 @@ def main():
         line["paged_attn_config2"] = {k: c2[k] for k in ("value", "unit", "ms_per_step", "config",
                                                           "roofline", "cpu_baseline",
                                                           "parity_max_abs_vs_oracle")}
+        line["mixed_prefill_decode_config4"] = bench_mixed_config4(args)
         line["qgemv_q8_config1"] = bench_qgemv_q8(args)
         line["qgemm_q4_config3"] = bench_q4(args)
     print(json.dumps(line))

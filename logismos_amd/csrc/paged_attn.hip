@@ -84,12 +84,10 @@ __device__ __forceinline__ unsigned short attn_out_elem(float v, int out_bf16) {
     return __builtin_bit_cast(unsigned short, hv);
 }
 
-// DECODE = true : grid (num_splits, hkv / waves, num_seqs); sequences with exactly
-//                 one new token, keys split into partitions of part_tokens.
-// DECODE = false: grid (max_seqlen_q, hkv / waves, num_seqs); one wave per query token
-//                 of the sequences with more than one new token, whole visible
-//                 context in one partition.
-template <int G, bool DECODE>
+// Decode rows: grid (num_splits, hkv / waves, num_seqs); sequences with exactly one
+// new token, keys split into partitions of part_tokens.  Sequences with more new
+// tokens belong to paged_attn_prefill_kernel below.
+template <int G>
 __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_kernel(const AttnParams p) {
     const int lane = threadIdx.x & 63;
     const int tg = lane >> 4;
@@ -102,22 +100,11 @@ __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_kernel(const At
     const int t0 = p.cu_seqlens_q[s];
     const int n_new = p.cu_seqlens_q[s + 1] - t0;
     const int ctx = p.context_lens[s];
-    int t, vis, tok_begin, tok_end, split;
-    if constexpr (DECODE) {
-        if (n_new != 1) return;
-        t = t0;
-        vis = ctx;
-        split = blockIdx.x;
-        tok_begin = split * p.part_tokens;
-    } else {
-        const int i = blockIdx.x;
-        if (n_new <= 1 || i >= n_new) return;
-        t = t0 + i;
-        vis = p.causal ? (ctx - n_new + i + 1) : ctx;
-        vis = vis > ctx ? ctx : vis;
-        split = 0;
-        tok_begin = 0;
-    }
+    if (n_new != 1) return;
+    const int t = t0;
+    const int vis = ctx;
+    const int split = blockIdx.x;
+    const int tok_begin = split * p.part_tokens;
     if (vis <= 0) {
         // no visible key: zeros (softmax over zero columns)
         if (split == 0 && c < G) {
@@ -141,8 +128,8 @@ __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_kernel(const At
         return;
     }
     if (tok_begin >= vis) return;
-    tok_end = DECODE ? min(vis, tok_begin + p.part_tokens) : vis;
-    const int num_parts = DECODE ? (vis + p.part_tokens - 1) / p.part_tokens : 1;
+    const int tok_end = min(vis, tok_begin + p.part_tokens);
+    const int num_parts = (vis + p.part_tokens - 1) / p.part_tokens;
     const int ntiles = (tok_end - tok_begin + kTileKeys - 1) / kTileKeys;
 
     // ---- query group as the MFMA B operand: column = head c, piece tg + 4j
@@ -408,6 +395,297 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams 
     }
 }
 
+// ---------------------------------------------------------------------------
+// Chunked prefill: sequences with more than one new token.
+//
+// A workgroup of four waves owns one (sequence, KV head, tile of query tokens)
+// and streams the visible keys once, in tiles of 32, through LDS; the whole GQA
+// group shares them.  A wave owns 32*CT score columns, a column being one
+// (query token, head of the group) pair, and keeps their queries in registers.
+// Per key tile and column tile:
+//
+//   S^T[32 keys x 32 cols] = K[32 x 128] . Q^T       8 x v_mfma_f32_32x32x16_f16
+//   online softmax per column (fp32; a column lives in lanes c and c + 32)
+//   O^T[128 x 32 cols]   += V^T[128 x 32 keys] . P   8 x v_mfma_f32_32x32x16_f16
+//
+// The C layout of S^T (lane (hl, c): keys 8g + 4hl + i of column c) is, read as
+// "slot e = 4*(g%2) + i of MFMA g/2", already a B-operand layout, so P never
+// leaves its lane; V is written to LDS transposed ([d][key], two keys per
+// 32-bit store) so that the matching A operand is two 8-byte reads.
+//
+// K/V tiles travel HBM/L2 -> registers -> LDS, double-buffered, one barrier per
+// tile; the loads of tile i+1 are issued before the math of tile i.
+// grid (hkv, query tiles, num_seqs): with hkv a multiple of 8 every XCD (and its
+// L2) serves the same KV heads for all query tiles; later query tiles (more
+// visible keys under the causal mask) are dispatched first.
+constexpr int kPfKeys = 32;
+constexpr int kPfWaves = 4;
+constexpr int kKsStride = kHeadDim + 8;  // halfs per K row in LDS (272 B)
+constexpr int kVtStride = kPfKeys + 4;   // halfs per V^T row in LDS (72 B)
+constexpr int kKsElems = kPfKeys * kKsStride;
+constexpr int kVtElems = kHeadDim * kVtStride;
+constexpr int kStageStride = kHeadDim + 8;
+
+struct PfRegs {
+    uint4_t k[2];
+    uint4_t v[2];
+};
+
+template <int G, int CT>
+__global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const AttnParams p) {
+    constexpr int COLS = 32 * CT;   // score columns per wave
+    constexpr int TPW = COLS / G;   // query tokens per wave
+    constexpr int QT = kPfWaves * TPW;
+    static_assert(TPW >= 1, "group does not fit a wave");
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int w = tid >> 6;
+    const int hl = lane >> 5;
+    const int c = lane & 31;
+    const int kvh = blockIdx.x;
+    const int s = blockIdx.z;
+
+    const int t0 = p.cu_seqlens_q[s];
+    const int n_new = p.cu_seqlens_q[s + 1] - t0;
+    if (n_new <= 1) return;
+    const int qtile = gridDim.y - 1 - blockIdx.y;
+    const int i0 = qtile * QT;
+    if (i0 >= n_new) return;
+    const int ctx = p.context_lens[s];
+
+    // visible keys of new token i: the prior context and the new tokens up to itself
+    auto limit_of = [&](int i) {
+        int v = p.causal ? (ctx - n_new + i + 1) : ctx;
+        v = v > ctx ? ctx : v;
+        return v < 0 ? 0 : v;
+    };
+    const int kmax = limit_of(min(n_new, i0 + QT) - 1);  // keys this workgroup streams
+    const int ntiles = (kmax + kPfKeys - 1) / kPfKeys;
+    const int wi0 = i0 + w * TPW;  // first token of this wave
+    const bool wave_active = wi0 < n_new;
+    const int wave_max = wave_active ? limit_of(min(n_new, wi0 + TPW) - 1) : 0;
+    const int wave_min = wave_active ? limit_of(wi0) : 0;
+
+    __shared__ __attribute__((aligned(16))) _Float16 smem[2 * kKsElems + 2 * kVtElems];
+    static_assert(kPfWaves * 32 * kStageStride <= 2 * kKsElems + 2 * kVtElems, "stage fits");
+    _Float16* Ks = smem;
+    _Float16* Vt = smem + 2 * kKsElems;
+
+    // ---- columns of this lane and their queries (B operand: column c, d = 16j + 8hl ..)
+    int col_tok[CT], col_head[CT], col_lim[CT];
+    bool col_valid[CT];
+    half8_t qreg[CT][8];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const int j = 32 * ct + c;
+        const int tok = j / G;
+        col_head[ct] = kvh * G + (j - tok * G);
+        col_tok[ct] = wi0 + tok;
+        col_valid[ct] = tok < TPW && col_tok[ct] < n_new;
+        // columns without a query are never masked and never written
+        col_lim[ct] = col_valid[ct] ? limit_of(col_tok[ct]) : INT32_MAX;
+        const half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+        const int tq = col_valid[ct] ? col_tok[ct] : i0;
+        const _Float16* qp = p.q + ((int64_t)(t0 + tq) * p.hq + col_head[ct]) * kHeadDim + 8 * hl;
+#pragma unroll
+        for (int jj = 0; jj < 8; ++jj)
+            qreg[ct][jj] = col_valid[ct] ? *reinterpret_cast<const half8_t*>(qp + 16 * jj) : z;
+    }
+
+    // ---- tile movement: thread (kp = tid / 16, piece = tid % 16) carries the 16-byte
+    // piece of keys 2kp and 2kp + 1, of K and of V
+    const int kp = tid >> 4;
+    const int piece = tid & 15;
+    const int32_t* bt_row = p.block_tables + (int64_t)s * p.max_blocks_per_seq;
+    auto gload = [&](int tile, PfRegs& r) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            // keys past the end re-read the last streamed key; they are masked below
+            const int kidx = min(tile * kPfKeys + 2 * kp + u, kmax - 1);
+            const int bi = kidx / p.block_size;
+            const int64_t slot = (int64_t)bt_row[bi] * p.block_size + (kidx - bi * p.block_size);
+            const int64_t off = (slot * p.hkv + kvh) * kHeadDim + 8 * piece;
+            r.k[u] = *reinterpret_cast<const uint4_t*>(p.k_pool + off);
+            r.v[u] = *reinterpret_cast<const uint4_t*>(p.v_pool + off);
+        }
+    };
+    auto lstore = [&](int buf, const PfRegs& r) {
+        _Float16* ks = Ks + buf * kKsElems;
+        _Float16* vt = Vt + buf * kVtElems;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+            *reinterpret_cast<uint4_t*>(ks + (2 * kp + u) * kKsStride + 8 * piece) = r.k[u];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            // (key 2kp, key 2kp+1) of element e as one 32-bit word
+            const unsigned sel = (e & 1) ? 0x07060302u : 0x05040100u;
+            const unsigned pr = __builtin_amdgcn_perm(r.v[1][e >> 1], r.v[0][e >> 1], sel);
+            *reinterpret_cast<unsigned*>(vt + (8 * piece + e) * kVtStride + 2 * kp) = pr;
+        }
+    };
+
+    float m[CT], l[CT];
+    float16_t oacc[CT][4];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        m[ct] = -INFINITY;
+        l[ct] = 0.0f;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[ct][dt][r] = 0.0f;
+    }
+
+    auto compute = [&](int tile, int buf) {
+        const _Float16* ks = Ks + buf * kKsElems;
+        const _Float16* vt = Vt + buf * kVtElems;
+        const int key0 = tile * kPfKeys;
+        half8_t ka[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            ka[j] = *reinterpret_cast<const half8_t*>(ks + c * kKsStride + 16 * j + 8 * hl);
+        const bool need_mask = key0 + kPfKeys > wave_min;
+        half8_t pb[CT][2];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            float16_t sacc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sacc[r] = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[j], qreg[ct][j], sacc, 0, 0, 0);
+            float sc[16];
+            float mx = m[ct];
+            if (need_mask) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int key = key0 + 8 * (r >> 2) + 4 * hl + (r & 3);
+                    sc[r] = key < col_lim[ct] ? sacc[r] * p.scale_log2e : -INFINITY;
+                    mx = fmaxf(mx, sc[r]);
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    sc[r] = sacc[r] * p.scale_log2e;
+                    mx = fmaxf(mx, sc[r]);
+                }
+            }
+            mx = fmaxf(mx, shfl_xor_f32(mx, 32));
+            const float msafe = (mx == -INFINITY) ? 0.0f : mx;
+            const float alpha = fast_exp2(m[ct] - msafe);
+            float psum = 0.0f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float pv = fast_exp2(sc[r] - msafe);
+                psum += pv;
+                pb[ct][r >> 3][r & 7] = (_Float16)pv;
+            }
+            l[ct] = l[ct] * alpha + psum;
+            m[ct] = mx;
+            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+                for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) oacc[ct][dt][r] *= alpha;
+            }
+        }
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) {
+#pragma unroll
+            for (int kh = 0; kh < 2; ++kh) {
+                const _Float16* vp = vt + (32 * dt + c) * kVtStride + 16 * kh + 4 * hl;
+                const half4_t v0 = *reinterpret_cast<const half4_t*>(vp);
+                const half4_t v1 = *reinterpret_cast<const half4_t*>(vp + 8);
+                const half8_t va = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct)
+                    oacc[ct][dt] =
+                        __builtin_amdgcn_mfma_f32_32x32x16_f16(va, pb[ct][kh], oacc[ct][dt], 0, 0, 0);
+            }
+        }
+    };
+
+    if (ntiles > 0) {
+        PfRegs regs;
+        gload(0, regs);
+        lstore(0, regs);
+        __syncthreads();
+        for (int tile = 0; tile < ntiles; ++tile) {
+            const bool more = tile + 1 < ntiles;
+            if (more) gload(tile + 1, regs);
+            if (tile * kPfKeys < wave_max) compute(tile, tile & 1);
+            if (more) lstore((tile + 1) & 1, regs);
+            __syncthreads();
+        }
+    }
+
+    // ---- normalise, stage through this wave's LDS slice, write 16-byte pieces
+    _Float16* stage = smem + w * 32 * kStageStride;
+    unsigned short* stage_u = reinterpret_cast<unsigned short*>(stage);
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const float lt = l[ct] + shfl_xor_f32(l[ct], 32);
+        const float inv = lt > 0.0f ? 1.0f / lt : 0.0f;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                uint2_t o;
+#pragma unroll
+                for (int e = 0; e < 2; ++e)
+                    o[e] = (unsigned)attn_out_elem(oacc[ct][dt][4 * g + 2 * e] * inv, p.out_bf16) |
+                           ((unsigned)attn_out_elem(oacc[ct][dt][4 * g + 2 * e + 1] * inv, p.out_bf16)
+                            << 16);
+                *reinterpret_cast<uint2_t*>(stage_u + c * kStageStride + 32 * dt + 8 * g + 4 * hl) = o;
+            }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int pass = 0; pass < 8; ++pass) {
+            const int col = (lane >> 4) + 4 * pass;
+            const int chunk = lane & 15;
+            const uint4_t o =
+                *reinterpret_cast<const uint4_t*>(stage_u + col * kStageStride + 8 * chunk);
+            const int j = 32 * ct + col;
+            const int tok = j / G;
+            const int head = kvh * G + (j - tok * G);
+            const int ti = wi0 + tok;
+            const bool valid = tok < TPW && ti < n_new;
+            const int t = t0 + ti;
+            if (p.out_bf16 == 2) {
+                const float gs = row16_sum(sum8_bf16(o));
+                if (valid) {
+                    const int bp = xprep_bp(p.out_rows);
+                    reinterpret_cast<uint4_t*>(p.out)[(int64_t)(head * 16 + chunk) * bp + t] =
+                        pair_order(o);
+                    if (chunk == 0)
+                        reinterpret_cast<float*>(
+                            reinterpret_cast<char*>(p.out) +
+                            xprep_xg_offset(p.out_rows, p.hq * kHeadDim))[(int64_t)head * bp + t] = gs;
+                }
+            } else if (valid) {
+                *reinterpret_cast<uint4_t*>(p.out + ((int64_t)t * p.hq + head) * kHeadDim +
+                                            8 * chunk) = o;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+template <int G>
+static void launch_prefill(const AttnParams& p, int max_seqlen_q, hipStream_t stream) {
+    // two column tiles per wave once the chunk is long enough to fill the wider tile
+    constexpr int QT1 = kPfWaves * (32 / G);
+    constexpr int QT2 = kPfWaves * (64 / G);
+    if (max_seqlen_q > QT1) {
+        dim3 grid(p.hkv, (max_seqlen_q + QT2 - 1) / QT2, p.num_seqs);
+        paged_attn_prefill_kernel<G, 2><<<grid, dim3(64 * kPfWaves), 0, stream>>>(p);
+    } else {
+        dim3 grid(p.hkv, (max_seqlen_q + QT1 - 1) / QT1, p.num_seqs);
+        paged_attn_prefill_kernel<G, 1><<<grid, dim3(64 * kPfWaves), 0, stream>>>(p);
+    }
+}
+
 static int part_tokens_for(int block_size, int max_blocks_per_seq, int num_splits) {
     const int64_t max_ctx = (int64_t)block_size * max_blocks_per_seq;
     int64_t part = (max_ctx + num_splits - 1) / num_splits;
@@ -428,11 +706,10 @@ static hipError_t launch_group(const AttnParams& p, int max_seqlen_q, int phases
     dim3 block(64 * wpb);
     if (phases & LOGISMOS_ATTN_PHASE_DECODE) {
         dim3 grid_d(p.num_splits, p.hkv / wpb, p.num_seqs);
-        paged_attn_kernel<G, true><<<grid_d, block, 0, stream>>>(p);
+        paged_attn_kernel<G><<<grid_d, block, 0, stream>>>(p);
     }
     if ((phases & LOGISMOS_ATTN_PHASE_PREFILL) && max_seqlen_q > 1) {
-        dim3 grid_p(max_seqlen_q, p.hkv / wpb, p.num_seqs);
-        paged_attn_kernel<G, false><<<grid_p, block, 0, stream>>>(p);
+        launch_prefill<G>(p, max_seqlen_q, stream);
     }
     if ((phases & LOGISMOS_ATTN_PHASE_MERGE) && p.num_splits > 1) {
         dim3 grid_m(p.hq, p.num_seqs);

@@ -97,6 +97,80 @@ def test_mixed_chunked_prefill_and_decode_small():
     _check(c, causal=True, num_splits=7, what="mixed causal split 7")
 
 
+@pytest.mark.parametrize("hq,hkv", [(4, 4), (4, 2), (12, 4), (8, 2), (10, 2), (12, 2), (14, 2),
+                                    (16, 2), (32, 8)])
+def test_chunked_prefill_gqa_group_sizes(hq, hkv):
+    # chunk lengths on both sides of the query-tile and key-tile edges, with and
+    # without prior context, next to decode rows
+    rng = np.random.default_rng(40 + hq + hkv)
+    new = [31, 1, 32, 33, 2, 64, 65, 129, 7]
+    prior = [0, 77, 5, 100, 31, 0, 333, 17, 1]
+    c = workloads.paged_case(rng, new, prior, hq=hq, hkv=hkv)
+    _check(c, causal=True, what=f"prefill causal {hq}/{hkv}")
+    _check(c, causal=False, what=f"prefill non-causal {hq}/{hkv}")
+
+
+@pytest.mark.parametrize("block_size", [16, 32, 128])
+def test_chunked_prefill_block_sizes(block_size):
+    rng = np.random.default_rng(50 + block_size)
+    c = workloads.paged_case(rng, [100, 1, 40], [300, 50, 0], hq=8, hkv=2, block_size=block_size)
+    _check(c, what=f"prefill block {block_size}")
+
+
+def test_chunked_prefill_512_token_chunks_with_prior_context():
+    # config-4 chunk shape at Qwen3-8B head geometry, contexts the oracle finishes quickly
+    rng = np.random.default_rng(41)
+    c = workloads.paged_case(rng, [512, 1, 512, 200, 1], [0, 700, 1000, 77, 12], hq=32, hkv=8)
+    _check(c, what="512-token chunks")
+
+
+def test_chunked_prefill_peaked_softmax():
+    rng = np.random.default_rng(42)
+    c = workloads.paged_case(rng, [96, 1], [200, 10], hq=8, hkv=2)
+    c["scale"] = 4.0
+    _check(c, what="prefill peaked softmax")
+
+
+def test_config4_prefill_rows_agree_with_decode_rows_at_full_size():
+    # Size-independent property at config 4's full size: under the causal mask, new
+    # token i of a chunk attends to exactly the keys a decode row with context
+    # prior + i + 1 would, so the prefill kernel must reproduce what the (oracle-checked)
+    # decode kernel gives for the same query over the same block table.
+    c = workloads.config4()
+    r = PagedAttnRunner(c)
+    r.launch()
+    got = r.result()
+    assert np.isfinite(got.astype(np.float32)).all()
+    rng = np.random.default_rng(43)
+    pre = [s for s in range(len(c["new_tokens"])) if c["new_tokens"][s] > 1]
+    picks = [(s, int(i)) for s in pre for i in rng.choice(int(c["new_tokens"][s]), 3, replace=False)]
+    picks += [(pre[0], 0), (pre[-1], int(c["new_tokens"][pre[-1]]) - 1)]
+    d = dict(c)
+    d["q"] = np.stack([c["q"][c["cu_seqlens"][s] + i] for s, i in picks])
+    d["block_tables"] = np.stack([c["block_tables"][s] for s, _ in picks])
+    d["new_tokens"] = np.ones(len(picks), np.int32)
+    d["context_lens"] = np.array([c["prior_ctx"][s] + i + 1 for s, i in picks], np.int32)
+    d["prior_ctx"] = d["context_lens"] - 1
+    d["cu_seqlens"] = np.arange(len(picks) + 1, dtype=np.int32)
+    rd = PagedAttnRunner(d)
+    rd.launch()
+    want = rd.result()
+    rows = np.stack([got[c["cu_seqlens"][s] + i] for s, i in picks])
+    assert_parity(rows, want, what="config 4 prefill rows vs decode rows")
+    # and the decode rows of the mixed batch against the oracle on a reduced copy
+    dec = [s for s in range(len(c["new_tokens"])) if c["new_tokens"][s] == 1][:6]
+    e = dict(c)
+    e["q"] = np.stack([c["q"][c["cu_seqlens"][s]] for s in dec])
+    e["block_tables"] = np.stack([c["block_tables"][s] for s in dec])
+    e["new_tokens"] = np.ones(len(dec), np.int32)
+    e["context_lens"] = c["context_lens"][dec]
+    e["prior_ctx"] = e["context_lens"] - 1
+    e["cu_seqlens"] = np.arange(len(dec) + 1, dtype=np.int32)
+    want_dec = _oracle(e)
+    rows_dec = np.stack([got[c["cu_seqlens"][s]] for s in dec])
+    assert_parity(rows_dec, want_dec, what="config 4 decode rows vs oracle")
+
+
 def test_zero_context_and_empty_sequences():
     rng = np.random.default_rng(5)
     c = workloads.paged_case(rng, [1, 0, 1, 3], [0, 5, 40, 0], hq=4, hkv=2)

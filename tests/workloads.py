@@ -13,9 +13,11 @@ SEED = 0x10615
 
 
 def paged_case(rng, new_tokens, prior_ctx, hq, hkv, d=128, block_size=16, spare_frac=0.25,
-               kv_std=1.0):
+               kv_std=1.0, pool_period_rows=None):
     """Ragged paged-attention inputs: pools shared by all sequences, physical
-    block ids a random permutation, block-table tail entries poisoned."""
+    block ids a random permutation, block-table tail entries poisoned.  With
+    pool_period_rows the pools repeat that many random rows (full-size cases whose
+    pools would take minutes to draw)."""
     new = np.asarray(new_tokens, np.int32)
     prior = np.asarray(prior_ctx, np.int32)
     ctx = (new + prior).astype(np.int32)
@@ -29,8 +31,13 @@ def paged_case(rng, new_tokens, prior_ctx, hq, hkv, d=128, block_size=16, spare_
         bt[s, :nb] = perm[o:o + nb]
         o += nb
     rows = total_blocks * block_size
-    k_pool = (rng.standard_normal((rows, hkv * d), np.float32) * kv_std).astype(np.float16)
-    v_pool = (rng.standard_normal((rows, hkv * d), np.float32) * kv_std).astype(np.float16)
+    def pool():
+        n = min(rows, pool_period_rows or rows)
+        base = (rng.standard_normal((n, hkv * d), np.float32) * kv_std).astype(np.float16)
+        return base if n == rows else np.resize(base, (rows, hkv * d))
+
+    k_pool = pool()
+    v_pool = pool()
     cu = np.concatenate([[0], np.cumsum(new)]).astype(np.int32)
     q = rng.standard_normal((int(cu[-1]), hq, d), np.float32).astype(np.float16)
     return dict(q=q, k_pool=k_pool, v_pool=v_pool, block_tables=bt, cu_seqlens=cu,
@@ -76,6 +83,43 @@ def config5_attention(seed=SEED + 5, num_seqs=32, lo=256, hi=8192):
     rng = np.random.default_rng(seed)
     ctx = rng.integers(lo, hi + 1, size=num_seqs)
     return paged_case(rng, np.ones(num_seqs, np.int32), ctx - 1, hq=32, hkv=8, spare_frac=0.05)
+
+
+def config4(seed=SEED + 4, num_decode=48, num_prefill=16, chunk=512, max_decode_ctx=32768,
+            max_prior=8192, hq=32, hkv=8, pool_period_rows=8191):
+    """Mixed chunked-prefill + decode ragged batch, Qwen3-8B attention geometry: 48 decode
+    rows (contexts log-uniform 128..32768) interleaved with 16 prefill chunks of 512 tokens
+    (prior context uniform 0..8192), one packed token buffer."""
+    rng = np.random.default_rng(seed)
+    dec_ctx = np.exp(rng.uniform(np.log(128.0), np.log(float(max_decode_ctx)), num_decode))
+    dec_ctx = np.clip(np.rint(dec_ctx).astype(np.int64), 128, max_decode_ctx)
+    pre_prior = rng.integers(0, max_prior + 1, size=num_prefill)
+    kind = np.array([0] * num_decode + [1] * num_prefill)
+    rng.shuffle(kind)
+    new, prior = [], []
+    di = pi = 0
+    for kd in kind:
+        if kd == 0:
+            new.append(1)
+            prior.append(int(dec_ctx[di]) - 1)
+            di += 1
+        else:
+            new.append(chunk)
+            prior.append(int(pre_prior[pi]))
+            pi += 1
+    return paged_case(rng, new, prior, hq=hq, hkv=hkv, spare_frac=0.02,
+                      pool_period_rows=pool_period_rows)
+
+
+def paged_attn_flops(case, causal=True) -> int:
+    """QK^T and PV multiply-adds (x2) over the visible (query, key) pairs."""
+    new = case["new_tokens"].astype(np.int64)
+    ctx = case["context_lens"].astype(np.int64)
+    if causal:
+        pairs = new * (ctx - new) + new * (new + 1) // 2
+    else:
+        pairs = new * ctx
+    return int(pairs.sum()) * case["hq"] * case["d"] * 4
 
 
 def config3(seed=SEED + 3, n=12288, k=4096, max_batch=16):
