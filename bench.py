@@ -476,6 +476,10 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=5.0)
     ap.add_argument("--skip-kernels", action="store_true",
                     help="only the decode-step line, without the per-kernel legs")
+    ap.add_argument("--workload", default="all",
+                    choices=["all", "step", "config1", "config2", "config3", "config4"],
+                    help="all: the decode-step line with every leg inside it (default); "
+                         "otherwise only that workload's own JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; every workload is the full single-GPU "
@@ -486,8 +490,15 @@ def main():
     kernels.library()
     args.steps_c5 = args.steps if args.steps is not None else 20
     args.warmup_c5 = args.warmup if args.warmup is not None else 3
+    if args.workload in ("config1", "config2", "config3", "config4"):
+        args.steps = args.steps if args.steps is not None else 200
+        args.warmup = args.warmup if args.warmup is not None else 20
+        leg = {"config1": bench_qgemv_q8, "config2": bench_paged_decode, "config3": bench_q4,
+               "config4": bench_mixed_config4}[args.workload]
+        print(json.dumps(leg(args)))
+        return
     line = bench_decode_step(args)
-    if not args.skip_kernels:
+    if not args.skip_kernels and args.workload == "all":
         args.steps, args.warmup = 200, 20
         c2 = bench_paged_decode(args)
         line["paged_attn_config2"] = {k: c2[k] for k in ("value", "unit", "ms_per_step", "config",

@@ -253,23 +253,15 @@ __global__ __launch_bounds__(1024) void qgemm_q4g128_mfma_kernel(
             for (int bt = 0; bt < BT; ++bt)
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
-#ifdef LG_EXP_NOXLOAD
-                    ph.xa[i][t][bt] = uint4_t{0x3f803f80u, (unsigned)g, 0x3f803f80u, (unsigned)lane};
-#else
                     ph.xa[i][t][bt] =
                         *reinterpret_cast<const uint4_t*>(xrow[bt] + (int64_t)g * 128 + t * 8);
-#endif
         }
 #pragma unroll
         for (int ti = 0; ti < T; ++ti)
 #pragma unroll
             for (int i = 0; i < GW; ++i) {
                 const int g = (g0 + i) < groups ? (g0 + i) : (groups - 1);
-#ifdef LG_EXP_NOWLOAD
-                ph.w[ti][i] = uint4_t{0x12345678u, (unsigned)g, 0x9abcdef0u, (unsigned)lane};
-#else
                 ph.w[ti][i] = *reinterpret_cast<const uint4_t*>(wrow[ti] + (int64_t)g * 64);
-#endif
             }
     };
 

@@ -114,11 +114,7 @@ __global__ __launch_bounds__(kSplitkThreads) void qgemm_q4g128_splitk_kernel(
 #pragma unroll
         for (int i = 0; i < GP; ++i) {
             const int g = (i < gcount) ? (g0 + i) : (g0 + gcount - 1);
-#ifdef LG_EXP_NOWLOAD
-            w[t][i] = uint4_t{0x12345678u, (unsigned)g, 0x9abcdef0u, (unsigned)lane};
-#else
             w[t][i] = *reinterpret_cast<const uint4_t*>(wrow + (int64_t)g * 64);
-#endif
         }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -204,11 +200,7 @@ __global__ __launch_bounds__(kSplitkThreads) void qgemm_q4g128_splitk_kernel(
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int bi = bt * 16 + 4 * kc + e;
-#ifdef LG_EXP_NOSTORE
-                    if (bi < b && ysum[bt][e] == 12345.678f)
-#else
                     if (bi < b)
-#endif
                         part[((int64_t)j * b + bi) * n + row0 + r] = ysum[bt][e];
                 }
         }
@@ -232,12 +224,6 @@ static SplitkPlan splitk_plan(int b, int n, int k) {
     const double bs = (double)b / 32.0;
     SplitkPlan best{1, 1, groups};
     double best_cost = 1e30;
-#ifdef LG_EXP_PLAN_ENV
-    if (const char* e = getenv("LG_PLAN")) {
-        int gp = 1, tw = 1;
-        if (sscanf(e, "%d,%d", &gp, &tw) == 2) return SplitkPlan{tw, gp, (groups + gp - 1) / gp};
-    }
-#endif
     const int tws[] = {1, 2, 4};
     const int gps[] = {1, 2, 4};
     for (int tw : tws)
