@@ -35,6 +35,7 @@ from tests import workloads  # noqa: E402
 from tests.gpu_harness import PagedAttnRunner, QgemvQ8Runner  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
+PMC_CAL_BYTES = 256 << 20  # bytes the calibration copy reads (and writes)
 COLD_BYTES = 640 << 20  # replicas together exceed 2x the 256 MiB Infinity Cache
 
 
@@ -63,6 +64,19 @@ def physical_cores() -> int:
     except AttributeError:
         pass
     return max(1, n)
+
+
+def measured_traffic(summary: str):
+    """HBM bytes per launch from a committed hardware-counter summary under profiles/ (the
+    counters cannot be read from inside this process); None when there is none."""
+    try:
+        with open(os.path.join(ROOT, "profiles", summary)) as f:
+            for ln in f:
+                if ln.strip().startswith("traffic_bytes_per_launch:"):
+                    return int(ln.split(":")[1])
+    except OSError:
+        pass
+    return None
 
 
 def time_launches(stream, fns, steps, warmup, use_graph=True):
@@ -431,6 +445,13 @@ def bench_decode_step(args):
     attn_bytes = int(ctx_now.sum()) * 2 * hkv * 128 * 2 + 2 * S * hq * 128 * 2 + \
         4 * int(((ctx_now + bs - 1) // bs).sum()) + 4 * (2 * S + 1)
     ms_attn, _, _ = time_launches(stream, [attn(l) for l in range(L)], 72, 8)
+    # one plain copy of known size (outside every timed region): the dispatch that hardware
+    # counter runs of this command are scaled by
+    cal = hip.DeviceBuffer(2 * PMC_CAL_BYTES)
+    cal.fill(0x11)
+    kernels.launch_probe_copy(cal, cal.offset(PMC_CAL_BYTES), PMC_CAL_BYTES, stream)
+    stream.synchronize()
+    del cal
 
     per_layer_w = sum(int(np.asarray(t[0]).nbytes + np.asarray(t[1]).nbytes +
                           np.asarray(t[2]).nbytes)
@@ -455,7 +476,12 @@ def bench_decode_step(args):
                                                   HBM_PEAK_GBPS, 4),
                    "hip_graph": True, "gpu_side_packing": True},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": measured_traffic("paged_attn_decode_config5_pmc.txt")
+                     if (steps, warmup) == (20, 3) else None,
+                     "traffic_source": "profiles/paged_attn_decode_config5_pmc.txt (rocprofv3 "
+                                       "--pmc FETCH_SIZE / WRITE_SIZE of this command at its "
+                                       "default steps, bytes per launch)",
                      "kernel": "paged_attn_kernel<4,decode> (one layer of the step)",
                      "ms_per_launch": round(ms_attn, 5), "algorithmic_bytes_per_launch": attn_bytes},
         "cpu_baseline": {"value": round(S / (cpu_s * L), 3), "unit": "tok/s", "cores": cores,
