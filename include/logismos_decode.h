@@ -222,7 +222,8 @@ size_t logismos_paged_attn_workspace_bytes(int num_seqs, int num_q_heads, int he
  * `QwenAttention::forward` (crates/transformers/src/attention.rs:225-241);
  * the softmax is fp32 and max-subtracted
  * (`softmax_last_dim`, crates/kernels/src/cpu_f32/mod.rs:380-433); a query
- * with no visible key yields zeros.  Requires head_dim == 128,
+ * with no visible key yields zeros.  `scale` must be finite and > 0 (else
+ * hipErrorInvalidValue).  Requires head_dim == 128,
  * block_size % 16 == 0, num_q_heads % num_kv_heads == 0 and a group size
  * num_q_heads/num_kv_heads <= 8. */
 logismos_status_t logismos_launch_paged_attn_varlen_fp16(

@@ -425,6 +425,7 @@ constexpr int kVtStride = kPfKeys + 4;   // halfs per V^T row in LDS (72 B)
 constexpr int kKsElems = kPfKeys * kKsStride;
 constexpr int kVtElems = kHeadDim * kVtStride;
 constexpr int kStageStride = kHeadDim + 8;
+constexpr float kLazyLog2 = 8.0f;  // headroom of the lazily updated softmax maximum
 
 struct PfRegs {
     uint4_t k[2];
@@ -464,7 +465,6 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
     const int ntiles = (kmax + kPfKeys - 1) / kPfKeys;
     const int wi0 = i0 + w * TPW;  // first token of this wave
     const bool wave_active = wi0 < n_new;
-    const int wave_max = wave_active ? limit_of(min(n_new, wi0 + TPW) - 1) : 0;
     const int wave_min = wave_active ? limit_of(wi0) : 0;
 
     __shared__ __attribute__((aligned(16))) _Float16 smem[2 * kKsElems + 2 * kVtElems];
@@ -494,20 +494,51 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
     }
 
     // ---- tile movement: thread (kp = tid / 16, piece = tid % 16) carries the 16-byte
-    // piece of keys 2kp and 2kp + 1, of K and of V
+    // piece of keys 2kp and 2kp + 1, of K and of V.  The eight keys a wave carries sit in
+    // one KV block (8-aligned, block_size % 16 == 0, and a key past the end re-reads key
+    // kmax - 1 of that same block or, when the whole group is past the end, of its own
+    // block), so the physical block id is one scalar load per wave and tile.
     const int kp = tid >> 4;
     const int piece = tid & 15;
     const int32_t* bt_row = p.block_tables + (int64_t)s * p.max_blocks_per_seq;
-    auto gload = [&](int tile, PfRegs& r) {
+    const int wave_key0 = __builtin_amdgcn_readfirstlane(8 * w);
+    struct PfAddr {
+        int blk;   // physical block (wave-uniform)
+        int rel0;  // tile * 32 - first key of that block (may be negative)
+    };
+    // Block cursor of this wave, advanced one tile (32 keys) per call without divisions:
+    // [cur_base, cur_base + block_size) holds key cur_pos = tile * 32 + wave_key0.  Once
+    // cur_pos passes the last streamed key the block of that key is used instead.
+    const int last_key = kmax - 1;
+    const int last_bi = (last_key > 0 ? last_key : 0) / p.block_size;
+    const int last_base = last_bi * p.block_size;
+    int cur_pos = wave_key0, cur_bi = 0, cur_base = 0;
+    auto next_addr = [&]() {
+        while (cur_pos >= cur_base + p.block_size) {
+            cur_base += p.block_size;
+            ++cur_bi;
+        }
+        const bool past = cur_pos > last_key;
+        const int bi = past ? last_bi : cur_bi;
+        const int base = past ? last_base : cur_base;
+        PfAddr a{bt_row[bi], cur_pos - wave_key0 - base};
+        cur_pos += kPfKeys;
+        return a;
+    };
+    const unsigned row_stride = (unsigned)p.hkv * kHeadDim;           // elements per token row
+    const int64_t blk_stride = (int64_t)p.block_size * row_stride;    // elements per block
+    const unsigned lane_const = (unsigned)kvh * kHeadDim + 8u * piece;
+    auto gload = [&](int tile, const PfAddr& a, PfRegs& r) {
+        const _Float16* kb = p.k_pool + (int64_t)a.blk * blk_stride;  // wave-uniform
+        const _Float16* vb = p.v_pool + (int64_t)a.blk * blk_stride;
+        const int rel_last = last_key - tile * kPfKeys + a.rel0;      // of key kmax - 1
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             // keys past the end re-read the last streamed key; they are masked below
-            const int kidx = min(tile * kPfKeys + 2 * kp + u, kmax - 1);
-            const int bi = kidx / p.block_size;
-            const int64_t slot = (int64_t)bt_row[bi] * p.block_size + (kidx - bi * p.block_size);
-            const int64_t off = (slot * p.hkv + kvh) * kHeadDim + 8 * piece;
-            r.k[u] = *reinterpret_cast<const uint4_t*>(p.k_pool + off);
-            r.v[u] = *reinterpret_cast<const uint4_t*>(p.v_pool + off);
+            const int rel = min(a.rel0 + 2 * kp + u, rel_last);
+            const unsigned off = __umul24((unsigned)rel, row_stride) + lane_const;
+            r.k[u] = *reinterpret_cast<const uint4_t*>(kb + off);
+            r.v[u] = *reinterpret_cast<const uint4_t*>(vb + off);
         }
     };
     auto lstore = [&](int buf, const PfRegs& r) {
@@ -555,40 +586,63 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
 #pragma unroll
             for (int j = 0; j < 8; ++j)
                 sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[j], qreg[ct][j], sacc, 0, 0, 0);
+            // raw scores of this lane's 16 keys; masked ones become -inf
             float sc[16];
-            float mx = m[ct];
+            float tm = -INFINITY;
             if (need_mask) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int key = key0 + 8 * (r >> 2) + 4 * hl + (r & 3);
-                    sc[r] = key < col_lim[ct] ? sacc[r] * p.scale_log2e : -INFINITY;
-                    mx = fmaxf(mx, sc[r]);
+                    sc[r] = key < col_lim[ct] ? sacc[r] : -INFINITY;
+                    tm = fmaxf(tm, sc[r]);
                 }
             } else {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    sc[r] = sacc[r] * p.scale_log2e;
-                    mx = fmaxf(mx, sc[r]);
+                    sc[r] = sacc[r];
+                    tm = fmaxf(tm, sc[r]);
                 }
             }
-            mx = fmaxf(mx, shfl_xor_f32(mx, 32));
-            const float msafe = (mx == -INFINITY) ? 0.0f : mx;
-            const float alpha = fast_exp2(m[ct] - msafe);
-            float psum = 0.0f;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float pv = fast_exp2(sc[r] - msafe);
-                psum += pv;
-                pb[ct][r >> 3][r & 7] = (_Float16)pv;
-            }
-            l[ct] = l[ct] * alpha + psum;
-            m[ct] = mx;
-            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+            tm = fmaxf(tm, shfl_xor_f32(tm, 32)) * p.scale_log2e;
+            // Lazy reference maximum: the column's exponentials stay relative to m[ct]
+            // until a tile maximum exceeds it by more than 2^kLazyLog2 (probabilities are
+            // then at most 2^kLazyLog2, well inside fp16 and fp32 range), so the
+            // accumulators are rescaled a few times per column instead of per tile.
+            const bool raise = tm > m[ct] + kLazyLog2;
+            if (__builtin_expect(__builtin_amdgcn_ballot_w64(raise) != 0, 0)) {
+                const float alpha = raise ? fast_exp2(m[ct] - tm) : 1.0f;
+                m[ct] = raise ? tm : m[ct];
+                l[ct] *= alpha;
+                // The accumulators live in accumulation registers (they are MFMA operands
+                // everywhere else); scaling them in place here keeps this rare path from
+                // pulling them into ordinary registers around every tile.
 #pragma unroll
                 for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) oacc[ct][dt][r] *= alpha;
+                    for (int r = 0; r < 16; ++r) {
+                        float x = oacc[ct][dt][r], tmp;
+                        // (not volatile: touches no memory, so the loads around it keep
+                        // their scalar form)
+                        asm("v_accvgpr_read_b32 %1, %0\n\t"
+                            "s_nop 1\n\t"
+                            "v_mul_f32 %1, %1, %2\n\t"
+                            "s_nop 1\n\t"
+                            "v_accvgpr_write_b32 %0, %1\n\t"
+                            "s_nop 3"
+                            : "+a"(x), "=&v"(tmp)
+                            : "v"(alpha));
+                        oacc[ct][dt][r] = x;
+                    }
             }
+            const float nm = (m[ct] == -INFINITY) ? 0.0f : -m[ct];
+            float psum = 0.0f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float pv = fast_exp2(fmaf(sc[r], p.scale_log2e, nm));
+                psum += pv;
+                pb[ct][r >> 3][r & 7] = (_Float16)pv;
+            }
+            l[ct] += psum;
         }
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt) {
@@ -606,16 +660,34 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
         }
     };
 
+    // Two tiles of loads stay in flight: the rows of tile t + 2 are requested before the
+    // math of tile t and written to LDS after the math of tile t + 1; block ids run one
+    // tile further ahead through the scalar cache.  The body is straight-line for two
+    // tiles (tiles past the end repeat clamped loads and are fully masked), which keeps the
+    // wait counts exact.  Every wave does the math of every tile of the workgroup (a tile
+    // beyond a wave's own columns is fully masked there): the waves meet at the barrier
+    // anyway, and an unconditional body keeps the accumulators in place.
     if (ntiles > 0) {
-        PfRegs regs;
-        gload(0, regs);
-        lstore(0, regs);
+        PfRegs ra, rb;
+        PfAddr a0 = next_addr(), a1 = next_addr(), an = next_addr();
+        gload(0, a0, ra);
+        gload(1, a1, rb);
+        lstore(0, ra);
         __syncthreads();
-        for (int tile = 0; tile < ntiles; ++tile) {
-            const bool more = tile + 1 < ntiles;
-            if (more) gload(tile + 1, regs);
-            if (tile * kPfKeys < wave_max) compute(tile, tile & 1);
-            if (more) lstore((tile + 1) & 1, regs);
+        for (int tile = 0; tile < ntiles; tile += 2) {
+            PfAddr an2 = next_addr();
+            gload(tile + 2, an, ra);
+            __builtin_amdgcn_sched_barrier(0);
+            compute(tile, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            lstore(1, rb);
+            __syncthreads();
+            an = next_addr();
+            gload(tile + 3, an2, rb);
+            __builtin_amdgcn_sched_barrier(0);
+            compute(tile + 1, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            lstore(0, ra);
             __syncthreads();
         }
     }
@@ -758,6 +830,8 @@ extern "C" logismos_status_t logismos_check_paged_attn_shape(int num_seqs, int t
         return lg::reject(msg, msg_cap, "%s: total_tokens*num_q_heads*head_dim exceeds i32::MAX", k);
     if ((int64_t)block_size * max_blocks_per_seq > i32max)
         return lg::reject(msg, msg_cap, "%s: block_size*max_blocks_per_seq exceeds i32::MAX", k);
+    if ((int64_t)block_size * num_kv_heads * head_dim > i32max)
+        return lg::reject(msg, msg_cap, "%s: block_size*num_kv_heads*head_dim exceeds i32::MAX", k);
     if ((int64_t)num_seqs * max_blocks_per_seq > i32max)
         return lg::reject(msg, msg_cap, "%s: num_seqs*max_blocks_per_seq exceeds i32::MAX", k);
     if ((int64_t)num_seqs * num_splits * num_q_heads > i32max / 130)
@@ -822,6 +896,7 @@ logismos_status_t lg::paged_attn_launch(
                                         num_kv_heads, head_dim, block_size, max_blocks_per_seq,
                                         num_splits, nullptr, 0) != 0)
         return hipErrorInvalidValue;
+    if (!(scale > 0.0f) || !(scale < INFINITY)) return hipErrorInvalidValue;
     if (total_tokens == 0) return hipSuccess;
     if (!q_f16 || !k_pool_f16 || !v_pool_f16 || !block_tables || !cu_seqlens_q || !context_lens ||
         !out_f16)
