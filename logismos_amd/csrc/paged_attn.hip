@@ -398,7 +398,7 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams 
 // ---------------------------------------------------------------------------
 // Chunked prefill: sequences with more than one new token.
 //
-// A workgroup of four waves owns one (sequence, KV head, tile of query tokens)
+// A workgroup of W waves owns one (sequence, KV head, tile of query tokens)
 // and streams the visible keys once, in tiles of 32, through LDS; the whole GQA
 // group shares them.  A wave owns 32*CT score columns, a column being one
 // (query token, head of the group) pair, and keeps their queries in registers.
@@ -419,7 +419,6 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams 
 // L2) serves the same KV heads for all query tiles; later query tiles (more
 // visible keys under the causal mask) are dispatched first.
 constexpr int kPfKeys = 32;
-constexpr int kPfWaves = 4;
 constexpr int kKsStride = kHeadDim + 8;  // halfs per K row in LDS (272 B)
 constexpr int kVtStride = kPfKeys + 4;   // halfs per V^T row in LDS (72 B)
 constexpr int kKsElems = kPfKeys * kKsStride;
@@ -427,16 +426,20 @@ constexpr int kVtElems = kHeadDim * kVtStride;
 constexpr int kStageStride = kHeadDim + 8;
 constexpr float kLazyLog2 = 8.0f;  // headroom of the lazily updated softmax maximum
 
+// W = 4: every thread moves two K and two V pieces per tile; W = 8 (two waves per SIMD,
+// which lets one wave's softmax overlap the other's MFMAs): waves 0-3 move K, 4-7 move V.
+template <int W>
 struct PfRegs {
-    uint4_t k[2];
-    uint4_t v[2];
+    uint4_t x[W == 4 ? 2 : 1][2];  // [K, V][key of the pair]
 };
 
-template <int G, int CT>
-__global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const AttnParams p) {
+template <int G, int CT, int W>
+__global__ __launch_bounds__(64 * W) void paged_attn_prefill_kernel(const AttnParams p) {
+    static_assert(W == 4 || W == 8, "4 or 8 waves");
     constexpr int COLS = 32 * CT;   // score columns per wave
     constexpr int TPW = COLS / G;   // query tokens per wave
-    constexpr int QT = kPfWaves * TPW;
+    constexpr int QT = W * TPW;
+    constexpr int NR = W == 4 ? 2 : 1;  // pools a thread moves
     static_assert(TPW >= 1, "group does not fit a wave");
 
     const int tid = threadIdx.x;
@@ -468,7 +471,7 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
     const int wave_min = wave_active ? limit_of(wi0) : 0;
 
     __shared__ __attribute__((aligned(16))) _Float16 smem[2 * kKsElems + 2 * kVtElems];
-    static_assert(kPfWaves * 32 * kStageStride <= 2 * kKsElems + 2 * kVtElems, "stage fits");
+    static_assert(W * 16 * kStageStride <= 2 * kKsElems + 2 * kVtElems, "stage fits");
     _Float16* Ks = smem;
     _Float16* Vt = smem + 2 * kKsElems;
 
@@ -498,10 +501,11 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
     // one KV block (8-aligned, block_size % 16 == 0, and a key past the end re-reads key
     // kmax - 1 of that same block or, when the whole group is past the end, of its own
     // block), so the physical block id is one scalar load per wave and tile.
-    const int kp = tid >> 4;
+    const int kp = (tid & 255) >> 4;
     const int piece = tid & 15;
+    const int role0 = W == 4 ? 0 : (w >> 2);  // first pool this thread moves (0 = K, 1 = V)
     const int32_t* bt_row = p.block_tables + (int64_t)s * p.max_blocks_per_seq;
-    const int wave_key0 = __builtin_amdgcn_readfirstlane(8 * w);
+    const int wave_key0 = __builtin_amdgcn_readfirstlane(8 * (w & 3));
     struct PfAddr {
         int blk;   // physical block (wave-uniform)
         int rel0;  // tile * 32 - first key of that block (may be negative)
@@ -528,31 +532,41 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
     const unsigned row_stride = (unsigned)p.hkv * kHeadDim;           // elements per token row
     const int64_t blk_stride = (int64_t)p.block_size * row_stride;    // elements per block
     const unsigned lane_const = (unsigned)kvh * kHeadDim + 8u * piece;
-    auto gload = [&](int tile, const PfAddr& a, PfRegs& r) {
-        const _Float16* kb = p.k_pool + (int64_t)a.blk * blk_stride;  // wave-uniform
-        const _Float16* vb = p.v_pool + (int64_t)a.blk * blk_stride;
+    auto gload = [&](int tile, const PfAddr& a, PfRegs<W>& r) {
         const int rel_last = last_key - tile * kPfKeys + a.rel0;      // of key kmax - 1
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            // keys past the end re-read the last streamed key; they are masked below
-            const int rel = min(a.rel0 + 2 * kp + u, rel_last);
-            const unsigned off = __umul24((unsigned)rel, row_stride) + lane_const;
-            r.k[u] = *reinterpret_cast<const uint4_t*>(kb + off);
-            r.v[u] = *reinterpret_cast<const uint4_t*>(vb + off);
+        for (int rr = 0; rr < NR; ++rr) {
+            const _Float16* pool = (role0 + rr) ? p.v_pool : p.k_pool;
+            const _Float16* pb = pool + (int64_t)a.blk * blk_stride;  // wave-uniform
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                // keys past the end re-read the last streamed key; they are masked below
+                const int rel = min(a.rel0 + 2 * kp + u, rel_last);
+                const unsigned off = __umul24((unsigned)rel, row_stride) + lane_const;
+                r.x[rr][u] = *reinterpret_cast<const uint4_t*>(pb + off);
+            }
         }
     };
-    auto lstore = [&](int buf, const PfRegs& r) {
+    auto lstore = [&](int buf, const PfRegs<W>& r) {
         _Float16* ks = Ks + buf * kKsElems;
         _Float16* vt = Vt + buf * kVtElems;
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
-            *reinterpret_cast<uint4_t*>(ks + (2 * kp + u) * kKsStride + 8 * piece) = r.k[u];
+        for (int rr = 0; rr < NR; ++rr) {
+            if ((role0 + rr) == 0) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            // (key 2kp, key 2kp+1) of element e as one 32-bit word
-            const unsigned sel = (e & 1) ? 0x07060302u : 0x05040100u;
-            const unsigned pr = __builtin_amdgcn_perm(r.v[1][e >> 1], r.v[0][e >> 1], sel);
-            *reinterpret_cast<unsigned*>(vt + (8 * piece + e) * kVtStride + 2 * kp) = pr;
+                for (int u = 0; u < 2; ++u)
+                    *reinterpret_cast<uint4_t*>(ks + (2 * kp + u) * kKsStride + 8 * piece) =
+                        r.x[rr][u];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    // (key 2kp, key 2kp+1) of element e as one 32-bit word
+                    const unsigned sel = (e & 1) ? 0x07060302u : 0x05040100u;
+                    const unsigned pr =
+                        __builtin_amdgcn_perm(r.x[rr][1][e >> 1], r.x[rr][0][e >> 1], sel);
+                    *reinterpret_cast<unsigned*>(vt + (8 * piece + e) * kVtStride + 2 * kp) = pr;
+                }
+            }
         }
     };
 
@@ -668,7 +682,7 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
     // beyond a wave's own columns is fully masked there): the waves meet at the barrier
     // anyway, and an unconditional body keeps the accumulators in place.
     if (ntiles > 0) {
-        PfRegs ra, rb;
+        PfRegs<W> ra, rb;
         PfAddr a0 = next_addr(), a1 = next_addr(), an = next_addr();
         gload(0, a0, ra);
         gload(1, a1, rb);
@@ -692,69 +706,79 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
         }
     }
 
-    // ---- normalise, stage through this wave's LDS slice, write 16-byte pieces
-    _Float16* stage = smem + w * 32 * kStageStride;
-    unsigned short* stage_u = reinterpret_cast<unsigned short*>(stage);
+    // ---- normalise, stage through this wave's LDS slice (16 columns at a time), write
+    // 16-byte pieces
+    unsigned short* stage_u = reinterpret_cast<unsigned short*>(smem) + w * 16 * kStageStride;
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
         const float lt = l[ct] + shfl_xor_f32(l[ct], 32);
         const float inv = lt > 0.0f ? 1.0f / lt : 0.0f;
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+        for (int hf = 0; hf < 2; ++hf) {
+            if ((c >> 4) == hf) {
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                uint2_t o;
+                for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-                for (int e = 0; e < 2; ++e)
-                    o[e] = (unsigned)attn_out_elem(oacc[ct][dt][4 * g + 2 * e] * inv, p.out_bf16) |
-                           ((unsigned)attn_out_elem(oacc[ct][dt][4 * g + 2 * e + 1] * inv, p.out_bf16)
-                            << 16);
-                *reinterpret_cast<uint2_t*>(stage_u + c * kStageStride + 32 * dt + 8 * g + 4 * hl) = o;
+                    for (int g = 0; g < 4; ++g) {
+                        uint2_t o;
+#pragma unroll
+                        for (int e = 0; e < 2; ++e)
+                            o[e] = (unsigned)attn_out_elem(oacc[ct][dt][4 * g + 2 * e] * inv,
+                                                           p.out_bf16) |
+                                   ((unsigned)attn_out_elem(oacc[ct][dt][4 * g + 2 * e + 1] * inv,
+                                                            p.out_bf16)
+                                    << 16);
+                        *reinterpret_cast<uint2_t*>(stage_u + (c & 15) * kStageStride + 32 * dt +
+                                                    8 * g + 4 * hl) = o;
+                    }
             }
-        __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int pass = 0; pass < 8; ++pass) {
-            const int col = (lane >> 4) + 4 * pass;
-            const int chunk = lane & 15;
-            const uint4_t o =
-                *reinterpret_cast<const uint4_t*>(stage_u + col * kStageStride + 8 * chunk);
-            const int j = 32 * ct + col;
-            const int tok = j / G;
-            const int head = kvh * G + (j - tok * G);
-            const int ti = wi0 + tok;
-            const bool valid = tok < TPW && ti < n_new;
-            const int t = t0 + ti;
-            if (p.out_bf16 == 2) {
-                const float gs = row16_sum(sum8_bf16(o));
-                if (valid) {
-                    const int bp = xprep_bp(p.out_rows);
-                    reinterpret_cast<uint4_t*>(p.out)[(int64_t)(head * 16 + chunk) * bp + t] =
-                        pair_order(o);
-                    if (chunk == 0)
-                        reinterpret_cast<float*>(
-                            reinterpret_cast<char*>(p.out) +
-                            xprep_xg_offset(p.out_rows, p.hq * kHeadDim))[(int64_t)head * bp + t] = gs;
+            for (int pass = 0; pass < 4; ++pass) {
+                const int col = (lane >> 4) + 4 * pass;  // within this half
+                const int chunk = lane & 15;
+                const uint4_t o =
+                    *reinterpret_cast<const uint4_t*>(stage_u + col * kStageStride + 8 * chunk);
+                const int j = 32 * ct + 16 * hf + col;
+                const int tok = j / G;
+                const int head = kvh * G + (j - tok * G);
+                const int ti = wi0 + tok;
+                const bool valid = tok < TPW && ti < n_new;
+                const int t = t0 + ti;
+                if (p.out_bf16 == 2) {
+                    const float gs = row16_sum(sum8_bf16(o));
+                    if (valid) {
+                        const int bp = xprep_bp(p.out_rows);
+                        reinterpret_cast<uint4_t*>(p.out)[(int64_t)(head * 16 + chunk) * bp + t] =
+                            pair_order(o);
+                        if (chunk == 0)
+                            reinterpret_cast<float*>(
+                                reinterpret_cast<char*>(p.out) +
+                                xprep_xg_offset(p.out_rows, p.hq * kHeadDim))[(int64_t)head * bp + t] =
+                                gs;
+                    }
+                } else if (valid) {
+                    *reinterpret_cast<uint4_t*>(p.out + ((int64_t)t * p.hq + head) * kHeadDim +
+                                                8 * chunk) = o;
                 }
-            } else if (valid) {
-                *reinterpret_cast<uint4_t*>(p.out + ((int64_t)t * p.hq + head) * kHeadDim +
-                                            8 * chunk) = o;
             }
+            __builtin_amdgcn_wave_barrier();
         }
-        __builtin_amdgcn_wave_barrier();
     }
 }
 
 template <int G>
 static void launch_prefill(const AttnParams& p, int max_seqlen_q, hipStream_t stream) {
-    // two column tiles per wave once the chunk is long enough to fill the wider tile
-    constexpr int QT1 = kPfWaves * (32 / G);
-    constexpr int QT2 = kPfWaves * (64 / G);
-    if (max_seqlen_q > QT1) {
-        dim3 grid(p.hkv, (max_seqlen_q + QT2 - 1) / QT2, p.num_seqs);
-        paged_attn_prefill_kernel<G, 2><<<grid, dim3(64 * kPfWaves), 0, stream>>>(p);
+    // eight waves of one column tile each (two waves per SIMD) once the chunk fills that
+    // many query tokens; four waves for short chunks
+    constexpr int QT4 = 4 * (32 / G);
+    constexpr int QT8 = 8 * (32 / G);
+    if (max_seqlen_q > QT4) {
+        dim3 grid(p.hkv, (max_seqlen_q + QT8 - 1) / QT8, p.num_seqs);
+        paged_attn_prefill_kernel<G, 1, 8><<<grid, dim3(512), 0, stream>>>(p);
     } else {
-        dim3 grid(p.hkv, (max_seqlen_q + QT1 - 1) / QT1, p.num_seqs);
-        paged_attn_prefill_kernel<G, 1><<<grid, dim3(64 * kPfWaves), 0, stream>>>(p);
+        dim3 grid(p.hkv, (max_seqlen_q + QT4 - 1) / QT4, p.num_seqs);
+        paged_attn_prefill_kernel<G, 1, 4><<<grid, dim3(256), 0, stream>>>(p);
     }
 }
 
