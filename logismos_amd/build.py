@@ -34,6 +34,14 @@ HIPCC_FLAGS = [
 ]
 
 
+# Per-source additions.  paged_attn.hip: MFMA results stay in ordinary VGPRs (the
+# kernels fit in 256 registers; the default accumulation-register form costs the
+# prefill kernel ~50 register-to-register moves per key tile around its softmax).
+EXTRA_FLAGS = {
+    "paged_attn.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+}
+
+
 def hipcc() -> str:
     exe = os.environ.get("HIPCC") or shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(exe) and not shutil.which(exe):
@@ -47,7 +55,8 @@ def sources() -> list[str]:
 
 def _compile(src: str) -> str:
     obj = os.path.join(OBJDIR, os.path.basename(src) + ".o")
-    cmd = [hipcc(), *HIPCC_FLAGS, "-x", "hip", "-c", src, "-o", obj]
+    cmd = [hipcc(), *HIPCC_FLAGS, *EXTRA_FLAGS.get(os.path.basename(src), []), "-x", "hip", "-c",
+           src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{r.stderr}")

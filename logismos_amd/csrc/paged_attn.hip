@@ -398,11 +398,11 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams 
 // ---------------------------------------------------------------------------
 // Chunked prefill: sequences with more than one new token.
 //
-// A workgroup of W waves owns one (sequence, KV head, tile of query tokens)
-// and streams the visible keys once, in tiles of 32, through LDS; the whole GQA
-// group shares them.  A wave owns 32*CT score columns, a column being one
-// (query token, head of the group) pair, and keeps their queries in registers.
-// Per key tile and column tile:
+// A workgroup of eight waves (two per SIMD) owns one (sequence, KV head, tile of
+// query tokens) and streams the visible keys once, in tiles of 32, through LDS;
+// the whole GQA group shares them.  A wave owns 32 score columns, a column being
+// one (query token, head of the group) pair, and keeps their queries in
+// registers.  Per key tile:
 //
 //   S^T[32 keys x 32 cols] = K[32 x 128] . Q^T       8 x v_mfma_f32_32x32x16_f16
 //   online softmax per column (fp32; a column lives in lanes c and c + 32)
@@ -413,12 +413,17 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams 
 // leaves its lane; V is written to LDS transposed ([d][key], two keys per
 // 32-bit store) so that the matching A operand is two 8-byte reads.
 //
-// K/V tiles travel HBM/L2 -> registers -> LDS, double-buffered, one barrier per
-// tile; the loads of tile i+1 are issued before the math of tile i.
+// Schedule of one iteration (tile t): request K rows of tile t+3 / V rows of tile
+// t+2 from memory; issue the MFMAs of S(t+1); read V(t) from LDS; softmax of S(t)
+// on the VALU while those MFMAs run; O += P.V(t); write K(t+2) / V(t+1) to LDS;
+// barrier.  K therefore runs one tile ahead of V in the two-deep LDS rings.
+// Waves 0-3 move K, waves 4-7 move V.  The softmax maximum is updated lazily (see
+// kLazyLog2), which makes accumulator rescaling rare.
 // grid (hkv, query tiles, num_seqs): with hkv a multiple of 8 every XCD (and its
 // L2) serves the same KV heads for all query tiles; later query tiles (more
 // visible keys under the causal mask) are dispatched first.
 constexpr int kPfKeys = 32;
+constexpr int kPfWaves = 8;
 constexpr int kKsStride = kHeadDim + 8;  // halfs per K row in LDS (272 B)
 constexpr int kVtStride = kPfKeys + 4;   // halfs per V^T row in LDS (72 B)
 constexpr int kKsElems = kPfKeys * kKsStride;
@@ -426,20 +431,14 @@ constexpr int kVtElems = kHeadDim * kVtStride;
 constexpr int kStageStride = kHeadDim + 8;
 constexpr float kLazyLog2 = 8.0f;  // headroom of the lazily updated softmax maximum
 
-// W = 4: every thread moves two K and two V pieces per tile; W = 8 (two waves per SIMD,
-// which lets one wave's softmax overlap the other's MFMAs): waves 0-3 move K, 4-7 move V.
-template <int W>
 struct PfRegs {
-    uint4_t x[W == 4 ? 2 : 1][2];  // [K, V][key of the pair]
+    uint4_t x[2];  // the two keys of this thread's pair
 };
 
-template <int G, int CT, int W>
-__global__ __launch_bounds__(64 * W) void paged_attn_prefill_kernel(const AttnParams p) {
-    static_assert(W == 4 || W == 8, "4 or 8 waves");
-    constexpr int COLS = 32 * CT;   // score columns per wave
-    constexpr int TPW = COLS / G;   // query tokens per wave
-    constexpr int QT = W * TPW;
-    constexpr int NR = W == 4 ? 2 : 1;  // pools a thread moves
+template <int G>
+__global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const AttnParams p) {
+    constexpr int TPW = 32 / G;  // query tokens per wave
+    constexpr int QT = kPfWaves * TPW;
     static_assert(TPW >= 1, "group does not fit a wave");
 
     const int tid = threadIdx.x;
@@ -467,48 +466,44 @@ __global__ __launch_bounds__(64 * W) void paged_attn_prefill_kernel(const AttnPa
     const int kmax = limit_of(min(n_new, i0 + QT) - 1);  // keys this workgroup streams
     const int ntiles = (kmax + kPfKeys - 1) / kPfKeys;
     const int wi0 = i0 + w * TPW;  // first token of this wave
-    const bool wave_active = wi0 < n_new;
-    const int wave_min = wave_active ? limit_of(wi0) : 0;
+    const int wave_min = wi0 < n_new ? limit_of(wi0) : 0;
 
     __shared__ __attribute__((aligned(16))) _Float16 smem[2 * kKsElems + 2 * kVtElems];
-    static_assert(W * 16 * kStageStride <= 2 * kKsElems + 2 * kVtElems, "stage fits");
+    static_assert(kPfWaves * 16 * kStageStride <= 2 * kKsElems + 2 * kVtElems, "stage fits");
     _Float16* Ks = smem;
     _Float16* Vt = smem + 2 * kKsElems;
 
-    // ---- columns of this lane and their queries (B operand: column c, d = 16j + 8hl ..)
-    int col_tok[CT], col_head[CT], col_lim[CT];
-    bool col_valid[CT];
-    half8_t qreg[CT][8];
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        const int j = 32 * ct + c;
-        const int tok = j / G;
-        col_head[ct] = kvh * G + (j - tok * G);
-        col_tok[ct] = wi0 + tok;
-        col_valid[ct] = tok < TPW && col_tok[ct] < n_new;
-        // columns without a query are never masked and never written
-        col_lim[ct] = col_valid[ct] ? limit_of(col_tok[ct]) : INT32_MAX;
+    // ---- column of this lane and its query (B operand: column c, d = 16j + 8hl ..)
+    const int col_tok_l = c / G;
+    const int col_head = kvh * G + (c - col_tok_l * G);
+    const int col_tok = wi0 + col_tok_l;
+    const bool col_valid = col_tok_l < TPW && col_tok < n_new;
+    // columns without a query are never masked and never written
+    const int col_lim = col_valid ? limit_of(col_tok) : INT32_MAX;
+    half8_t qreg[8];
+    {
         const half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
-        const int tq = col_valid[ct] ? col_tok[ct] : i0;
-        const _Float16* qp = p.q + ((int64_t)(t0 + tq) * p.hq + col_head[ct]) * kHeadDim + 8 * hl;
+        const int tq = col_valid ? col_tok : i0;
+        const _Float16* qp = p.q + ((int64_t)(t0 + tq) * p.hq + col_head) * kHeadDim + 8 * hl;
 #pragma unroll
-        for (int jj = 0; jj < 8; ++jj)
-            qreg[ct][jj] = col_valid[ct] ? *reinterpret_cast<const half8_t*>(qp + 16 * jj) : z;
+        for (int j = 0; j < 8; ++j)
+            qreg[j] = col_valid ? *reinterpret_cast<const half8_t*>(qp + 16 * j) : z;
     }
 
-    // ---- tile movement: thread (kp = tid / 16, piece = tid % 16) carries the 16-byte
-    // piece of keys 2kp and 2kp + 1, of K and of V.  The eight keys a wave carries sit in
-    // one KV block (8-aligned, block_size % 16 == 0, and a key past the end re-reads key
-    // kmax - 1 of that same block or, when the whole group is past the end, of its own
-    // block), so the physical block id is one scalar load per wave and tile.
+    // ---- tile movement: thread (kp, piece) of a four-wave half carries the 16-byte piece
+    // of keys 2kp and 2kp + 1 of its pool.  The eight keys a wave carries sit in one KV
+    // block (8-aligned, block_size % 16 == 0, and a key past the end re-reads key kmax - 1
+    // of that same block or, when the whole group is past the end, of its own block), so the
+    // physical block id is one scalar load per wave and tile.
     const int kp = (tid & 255) >> 4;
     const int piece = tid & 15;
-    const int role0 = W == 4 ? 0 : (w >> 2);  // first pool this thread moves (0 = K, 1 = V)
+    const bool moves_v = __builtin_amdgcn_readfirstlane(w >> 2) != 0;
     const int32_t* bt_row = p.block_tables + (int64_t)s * p.max_blocks_per_seq;
     const int wave_key0 = __builtin_amdgcn_readfirstlane(8 * (w & 3));
     struct PfAddr {
         int blk;   // physical block (wave-uniform)
         int rel0;  // tile * 32 - first key of that block (may be negative)
+        int tile;
     };
     // Block cursor of this wave, advanced one tile (32 keys) per call without divisions:
     // [cur_base, cur_base + block_size) holds key cur_pos = tile * 32 + wave_key0.  Once
@@ -516,192 +511,192 @@ __global__ __launch_bounds__(64 * W) void paged_attn_prefill_kernel(const AttnPa
     const int last_key = kmax - 1;
     const int last_bi = (last_key > 0 ? last_key : 0) / p.block_size;
     const int last_base = last_bi * p.block_size;
-    int cur_pos = wave_key0, cur_bi = 0, cur_base = 0;
+    int cur_tile = 0, cur_bi = 0, cur_base = 0;
     auto next_addr = [&]() {
-        while (cur_pos >= cur_base + p.block_size) {
+        const int pos = cur_tile * kPfKeys + wave_key0;
+        while (pos >= cur_base + p.block_size) {
             cur_base += p.block_size;
             ++cur_bi;
         }
-        const bool past = cur_pos > last_key;
+        const bool past = pos > last_key;
         const int bi = past ? last_bi : cur_bi;
         const int base = past ? last_base : cur_base;
-        PfAddr a{bt_row[bi], cur_pos - wave_key0 - base};
-        cur_pos += kPfKeys;
+        PfAddr a{bt_row[bi], cur_tile * kPfKeys - base, cur_tile};
+        ++cur_tile;
         return a;
     };
-    const unsigned row_stride = (unsigned)p.hkv * kHeadDim;           // elements per token row
-    const int64_t blk_stride = (int64_t)p.block_size * row_stride;    // elements per block
+    const unsigned row_stride = (unsigned)p.hkv * kHeadDim;         // elements per token row
+    const int64_t blk_stride = (int64_t)p.block_size * row_stride;  // elements per block
     const unsigned lane_const = (unsigned)kvh * kHeadDim + 8u * piece;
-    auto gload = [&](int tile, const PfAddr& a, PfRegs<W>& r) {
-        const int rel_last = last_key - tile * kPfKeys + a.rel0;      // of key kmax - 1
+    const _Float16* pool = moves_v ? p.v_pool : p.k_pool;
+    auto gload = [&](const PfAddr& a, PfRegs& r) {
+        const _Float16* pb = pool + (int64_t)a.blk * blk_stride;   // wave-uniform
+        const int rel_last = last_key - a.tile * kPfKeys + a.rel0;  // of key kmax - 1
 #pragma unroll
-        for (int rr = 0; rr < NR; ++rr) {
-            const _Float16* pool = (role0 + rr) ? p.v_pool : p.k_pool;
-            const _Float16* pb = pool + (int64_t)a.blk * blk_stride;  // wave-uniform
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                // keys past the end re-read the last streamed key; they are masked below
-                const int rel = min(a.rel0 + 2 * kp + u, rel_last);
-                const unsigned off = __umul24((unsigned)rel, row_stride) + lane_const;
-                r.x[rr][u] = *reinterpret_cast<const uint4_t*>(pb + off);
-            }
+        for (int u = 0; u < 2; ++u) {
+            // keys past the end re-read the last streamed key; they are masked below
+            const int rel = min(a.rel0 + 2 * kp + u, rel_last);
+            const unsigned off = __umul24((unsigned)rel, row_stride) + lane_const;
+            r.x[u] = *reinterpret_cast<const uint4_t*>(pb + off);
         }
     };
-    auto lstore = [&](int buf, const PfRegs<W>& r) {
-        _Float16* ks = Ks + buf * kKsElems;
-        _Float16* vt = Vt + buf * kVtElems;
+    // K rows as they are; V transposed, (key 2kp, key 2kp+1) of element e as one word
+    auto lstore = [&](int buf, const PfRegs& r) {
+        if (!moves_v) {
+            _Float16* ks = Ks + buf * kKsElems;
 #pragma unroll
-        for (int rr = 0; rr < NR; ++rr) {
-            if ((role0 + rr) == 0) {
+            for (int u = 0; u < 2; ++u)
+                *reinterpret_cast<uint4_t*>(ks + (2 * kp + u) * kKsStride + 8 * piece) = r.x[u];
+        } else {
+            _Float16* vt = Vt + buf * kVtElems;
 #pragma unroll
-                for (int u = 0; u < 2; ++u)
-                    *reinterpret_cast<uint4_t*>(ks + (2 * kp + u) * kKsStride + 8 * piece) =
-                        r.x[rr][u];
-            } else {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    // (key 2kp, key 2kp+1) of element e as one 32-bit word
-                    const unsigned sel = (e & 1) ? 0x07060302u : 0x05040100u;
-                    const unsigned pr =
-                        __builtin_amdgcn_perm(r.x[rr][1][e >> 1], r.x[rr][0][e >> 1], sel);
-                    *reinterpret_cast<unsigned*>(vt + (8 * piece + e) * kVtStride + 2 * kp) = pr;
-                }
+            for (int e = 0; e < 8; ++e) {
+                const unsigned sel = (e & 1) ? 0x07060302u : 0x05040100u;
+                const unsigned pr = __builtin_amdgcn_perm(r.x[1][e >> 1], r.x[0][e >> 1], sel);
+                *reinterpret_cast<unsigned*>(vt + (8 * piece + e) * kVtStride + 2 * kp) = pr;
             }
         }
     };
 
-    float m[CT], l[CT];
-    float16_t oacc[CT][4];
+    float m = -INFINITY, l = 0.0f;
+    float16_t oacc[4];
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        m[ct] = -INFINITY;
-        l[ct] = 0.0f;
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.0f;
+
+    // S^T of one key tile: K from LDS as the A operand
+    auto qk = [&](int buf) {
+        const _Float16* ks = Ks + buf * kKsElems + c * kKsStride + 8 * hl;
+        half8_t ka[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ka[j] = *reinterpret_cast<const half8_t*>(ks + 16 * j);
+        float16_t sacc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sacc[r] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[j], qreg[j], sacc, 0, 0, 0);
+        return sacc;
+    };
+    struct VTile {
+        half8_t a[4][2];
+    };
+    auto vread = [&](int buf, VTile& v) {
+        const _Float16* vt = Vt + buf * kVtElems + c * kVtStride + 4 * hl;
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[ct][dt][r] = 0.0f;
-    }
-
-    auto compute = [&](int tile, int buf) {
-        const _Float16* ks = Ks + buf * kKsElems;
-        const _Float16* vt = Vt + buf * kVtElems;
-        const int key0 = tile * kPfKeys;
-        half8_t ka[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-            ka[j] = *reinterpret_cast<const half8_t*>(ks + c * kKsStride + 16 * j + 8 * hl);
-        const bool need_mask = key0 + kPfKeys > wave_min;
-        half8_t pb[CT][2];
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            float16_t sacc;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) sacc[r] = 0.0f;
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-                sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[j], qreg[ct][j], sacc, 0, 0, 0);
-            // raw scores of this lane's 16 keys; masked ones become -inf
-            float sc[16];
-            float tm = -INFINITY;
-            if (need_mask) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int key = key0 + 8 * (r >> 2) + 4 * hl + (r & 3);
-                    sc[r] = key < col_lim[ct] ? sacc[r] : -INFINITY;
-                    tm = fmaxf(tm, sc[r]);
-                }
-            } else {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    sc[r] = sacc[r];
-                    tm = fmaxf(tm, sc[r]);
-                }
-            }
-            tm = fmaxf(tm, shfl_xor_f32(tm, 32)) * p.scale_log2e;
-            // Lazy reference maximum: the column's exponentials stay relative to m[ct]
-            // until a tile maximum exceeds it by more than 2^kLazyLog2 (probabilities are
-            // then at most 2^kLazyLog2, well inside fp16 and fp32 range), so the
-            // accumulators are rescaled a few times per column instead of per tile.
-            const bool raise = tm > m[ct] + kLazyLog2;
-            if (__builtin_expect(__builtin_amdgcn_ballot_w64(raise) != 0, 0)) {
-                const float alpha = raise ? fast_exp2(m[ct] - tm) : 1.0f;
-                m[ct] = raise ? tm : m[ct];
-                l[ct] *= alpha;
-                // The accumulators live in accumulation registers (they are MFMA operands
-                // everywhere else); scaling them in place here keeps this rare path from
-                // pulling them into ordinary registers around every tile.
-#pragma unroll
-                for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        float x = oacc[ct][dt][r], tmp;
-                        // (not volatile: touches no memory, so the loads around it keep
-                        // their scalar form)
-                        asm("v_accvgpr_read_b32 %1, %0\n\t"
-                            "s_nop 1\n\t"
-                            "v_mul_f32 %1, %1, %2\n\t"
-                            "s_nop 1\n\t"
-                            "v_accvgpr_write_b32 %0, %1\n\t"
-                            "s_nop 3"
-                            : "+a"(x), "=&v"(tmp)
-                            : "v"(alpha));
-                        oacc[ct][dt][r] = x;
-                    }
-            }
-            const float nm = (m[ct] == -INFINITY) ? 0.0f : -m[ct];
-            float psum = 0.0f;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float pv = fast_exp2(fmaf(sc[r], p.scale_log2e, nm));
-                psum += pv;
-                pb[ct][r >> 3][r & 7] = (_Float16)pv;
-            }
-            l[ct] += psum;
-        }
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt) {
-#pragma unroll
             for (int kh = 0; kh < 2; ++kh) {
-                const _Float16* vp = vt + (32 * dt + c) * kVtStride + 16 * kh + 4 * hl;
+                const _Float16* vp = vt + 32 * dt * kVtStride + 16 * kh;
                 const half4_t v0 = *reinterpret_cast<const half4_t*>(vp);
                 const half4_t v1 = *reinterpret_cast<const half4_t*>(vp + 8);
-                const half8_t va = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+                v.a[dt][kh] = half8_t{v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+            }
+    };
+    // online softmax of one score tile; returns P as the two B operands of P.V
+    auto softmax = [&](int tile, const float16_t& sacc, half8_t (&pb)[2]) {
+        const int key0 = tile * kPfKeys;
+        float sc[16];
+        float tm = -INFINITY;
+        if (key0 + kPfKeys > wave_min) {  // some column of this wave may be masked here
 #pragma unroll
-                for (int ct = 0; ct < CT; ++ct)
-                    oacc[ct][dt] =
-                        __builtin_amdgcn_mfma_f32_32x32x16_f16(va, pb[ct][kh], oacc[ct][dt], 0, 0, 0);
+            for (int r = 0; r < 16; ++r) {
+                const int key = key0 + 8 * (r >> 2) + 4 * hl + (r & 3);
+                sc[r] = key < col_lim ? sacc[r] : -INFINITY;
+                tm = fmaxf(tm, sc[r]);
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                sc[r] = sacc[r];
+                tm = fmaxf(tm, sc[r]);
             }
         }
+        tm = fmaxf(tm, shfl_xor_f32(tm, 32)) * p.scale_log2e;
+        // Lazy reference maximum: the column's exponentials stay relative to m until a
+        // tile maximum exceeds it by more than 2^kLazyLog2 (probabilities are then at most
+        // 2^kLazyLog2, well inside fp16 and fp32 range), so the accumulators are rescaled
+        // a few times per column instead of per tile.
+        const bool raise = tm > m + kLazyLog2;
+        if (__builtin_expect(__builtin_amdgcn_ballot_w64(raise) != 0, 0)) {
+            const float alpha = raise ? fast_exp2(m - tm) : 1.0f;
+            m = raise ? tm : m;
+            l *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+        }
+        const float nm = (m == -INFINITY) ? 0.0f : -m;
+        float psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float pv = fast_exp2(fmaf(sc[r], p.scale_log2e, nm));
+            psum += pv;
+            pb[r >> 3][r & 7] = (_Float16)pv;
+        }
+        l += psum;
+    };
+    auto pv = [&](const VTile& v, const half8_t (&pb)[2]) {
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int kh = 0; kh < 2; ++kh)
+                oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(v.a[dt][kh], pb[kh], oacc[dt], 0, 0, 0);
     };
 
-    // Two tiles of loads stay in flight: the rows of tile t + 2 are requested before the
-    // math of tile t and written to LDS after the math of tile t + 1; block ids run one
-    // tile further ahead through the scalar cache.  The body is straight-line for two
-    // tiles (tiles past the end repeat clamped loads and are fully masked), which keeps the
-    // wait counts exact.  Every wave does the math of every tile of the workgroup (a tile
-    // beyond a wave's own columns is fully masked there): the waves meet at the barrier
-    // anyway, and an unconditional body keeps the accumulators in place.
+    // The body is straight-line for two tiles (tiles past the end repeat clamped loads and
+    // are fully masked), which keeps the wait counts exact.  Every wave does the math of
+    // every tile of the workgroup (a tile beyond a wave's own columns is fully masked
+    // there): the waves meet at the barrier anyway.
     if (ntiles > 0) {
-        PfRegs<W> ra, rb;
-        PfAddr a0 = next_addr(), a1 = next_addr(), an = next_addr();
-        gload(0, a0, ra);
-        gload(1, a1, rb);
-        lstore(0, ra);
+        PfRegs ra, rb;
+        // K waves start one tile ahead of V waves
+        {
+            PfAddr a = next_addr();
+            gload(a, ra);
+            if (!moves_v) {
+                a = next_addr();
+                gload(a, rb);
+                lstore(0, ra);
+                lstore(1, rb);
+                a = next_addr();
+                gload(a, ra);  // K(2) in flight
+            } else {
+                lstore(0, ra);
+                a = next_addr();
+                gload(a, ra);  // V(1) in flight
+            }
+        }
+        PfAddr an = next_addr();
         __syncthreads();
+        float16_t s_cur = qk(0);
         for (int tile = 0; tile < ntiles; tile += 2) {
+            // ---- tile (K(tile+1) in K buffer 1, V(tile) in V buffer 0)
             PfAddr an2 = next_addr();
-            gload(tile + 2, an, ra);
+            gload(an, rb);  // K(tile+3) / V(tile+2)
             __builtin_amdgcn_sched_barrier(0);
-            compute(tile, 0);
+            float16_t s_nxt = qk(1);
+            VTile v;
+            vread(0, v);
+            half8_t pb[2];
+            softmax(tile, s_cur, pb);
+            pv(v, pb);
             __builtin_amdgcn_sched_barrier(0);
-            lstore(1, rb);
+            // K(tile+2) -> K buffer 0, V(tile+1) -> V buffer 1
+            lstore(moves_v ? 1 : 0, ra);
             __syncthreads();
+            // ---- tile + 1 (K(tile+2) in K buffer 0, V(tile+1) in V buffer 1)
             an = next_addr();
-            gload(tile + 3, an2, rb);
+            gload(an2, ra);  // K(tile+4) / V(tile+3)
             __builtin_amdgcn_sched_barrier(0);
-            compute(tile + 1, 1);
+            s_cur = qk(0);
+            vread(1, v);
+            softmax(tile + 1, s_nxt, pb);
+            pv(v, pb);
             __builtin_amdgcn_sched_barrier(0);
-            lstore(0, ra);
+            lstore(moves_v ? 0 : 1, rb);
             __syncthreads();
         }
     }
@@ -709,77 +704,65 @@ __global__ __launch_bounds__(64 * W) void paged_attn_prefill_kernel(const AttnPa
     // ---- normalise, stage through this wave's LDS slice (16 columns at a time), write
     // 16-byte pieces
     unsigned short* stage_u = reinterpret_cast<unsigned short*>(smem) + w * 16 * kStageStride;
+    const float lt = l + shfl_xor_f32(l, 32);
+    const float inv = lt > 0.0f ? 1.0f / lt : 0.0f;
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        const float lt = l[ct] + shfl_xor_f32(l[ct], 32);
-        const float inv = lt > 0.0f ? 1.0f / lt : 0.0f;
+    for (int hf = 0; hf < 2; ++hf) {
+        if ((c >> 4) == hf) {
 #pragma unroll
-        for (int hf = 0; hf < 2; ++hf) {
-            if ((c >> 4) == hf) {
+            for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-                for (int dt = 0; dt < 4; ++dt)
+                for (int g = 0; g < 4; ++g) {
+                    uint2_t o;
 #pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        uint2_t o;
-#pragma unroll
-                        for (int e = 0; e < 2; ++e)
-                            o[e] = (unsigned)attn_out_elem(oacc[ct][dt][4 * g + 2 * e] * inv,
-                                                           p.out_bf16) |
-                                   ((unsigned)attn_out_elem(oacc[ct][dt][4 * g + 2 * e + 1] * inv,
-                                                            p.out_bf16)
-                                    << 16);
-                        *reinterpret_cast<uint2_t*>(stage_u + (c & 15) * kStageStride + 32 * dt +
-                                                    8 * g + 4 * hl) = o;
-                    }
-            }
-            __builtin_amdgcn_wave_barrier();
-#pragma unroll
-            for (int pass = 0; pass < 4; ++pass) {
-                const int col = (lane >> 4) + 4 * pass;  // within this half
-                const int chunk = lane & 15;
-                const uint4_t o =
-                    *reinterpret_cast<const uint4_t*>(stage_u + col * kStageStride + 8 * chunk);
-                const int j = 32 * ct + 16 * hf + col;
-                const int tok = j / G;
-                const int head = kvh * G + (j - tok * G);
-                const int ti = wi0 + tok;
-                const bool valid = tok < TPW && ti < n_new;
-                const int t = t0 + ti;
-                if (p.out_bf16 == 2) {
-                    const float gs = row16_sum(sum8_bf16(o));
-                    if (valid) {
-                        const int bp = xprep_bp(p.out_rows);
-                        reinterpret_cast<uint4_t*>(p.out)[(int64_t)(head * 16 + chunk) * bp + t] =
-                            pair_order(o);
-                        if (chunk == 0)
-                            reinterpret_cast<float*>(
-                                reinterpret_cast<char*>(p.out) +
-                                xprep_xg_offset(p.out_rows, p.hq * kHeadDim))[(int64_t)head * bp + t] =
-                                gs;
-                    }
-                } else if (valid) {
-                    *reinterpret_cast<uint4_t*>(p.out + ((int64_t)t * p.hq + head) * kHeadDim +
-                                                8 * chunk) = o;
+                    for (int e = 0; e < 2; ++e)
+                        o[e] = (unsigned)attn_out_elem(oacc[dt][4 * g + 2 * e] * inv, p.out_bf16) |
+                               ((unsigned)attn_out_elem(oacc[dt][4 * g + 2 * e + 1] * inv,
+                                                        p.out_bf16)
+                                << 16);
+                    *reinterpret_cast<uint2_t*>(stage_u + (c & 15) * kStageStride + 32 * dt +
+                                                8 * g + 4 * hl) = o;
                 }
-            }
-            __builtin_amdgcn_wave_barrier();
         }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int pass = 0; pass < 4; ++pass) {
+            const int col = (lane >> 4) + 4 * pass;  // within this half
+            const int chunk = lane & 15;
+            const uint4_t o =
+                *reinterpret_cast<const uint4_t*>(stage_u + col * kStageStride + 8 * chunk);
+            const int j = 16 * hf + col;
+            const int tok = j / G;
+            const int head = kvh * G + (j - tok * G);
+            const int ti = wi0 + tok;
+            const bool valid = tok < TPW && ti < n_new;
+            const int t = t0 + ti;
+            if (p.out_bf16 == 2) {
+                const float gs = row16_sum(sum8_bf16(o));
+                if (valid) {
+                    const int bp = xprep_bp(p.out_rows);
+                    reinterpret_cast<uint4_t*>(p.out)[(int64_t)(head * 16 + chunk) * bp + t] =
+                        pair_order(o);
+                    if (chunk == 0)
+                        reinterpret_cast<float*>(
+                            reinterpret_cast<char*>(p.out) +
+                            xprep_xg_offset(p.out_rows, p.hq * kHeadDim))[(int64_t)head * bp + t] =
+                            gs;
+                }
+            } else if (valid) {
+                *reinterpret_cast<uint4_t*>(p.out + ((int64_t)t * p.hq + head) * kHeadDim +
+                                            8 * chunk) = o;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
     }
 }
 
 template <int G>
 static void launch_prefill(const AttnParams& p, int max_seqlen_q, hipStream_t stream) {
-    // eight waves of one column tile each (two waves per SIMD) once the chunk fills that
-    // many query tokens; four waves for short chunks
-    constexpr int QT4 = 4 * (32 / G);
-    constexpr int QT8 = 8 * (32 / G);
-    if (max_seqlen_q > QT4) {
-        dim3 grid(p.hkv, (max_seqlen_q + QT8 - 1) / QT8, p.num_seqs);
-        paged_attn_prefill_kernel<G, 1, 8><<<grid, dim3(512), 0, stream>>>(p);
-    } else {
-        dim3 grid(p.hkv, (max_seqlen_q + QT4 - 1) / QT4, p.num_seqs);
-        paged_attn_prefill_kernel<G, 1, 4><<<grid, dim3(256), 0, stream>>>(p);
-    }
+    constexpr int QT = kPfWaves * (32 / G);
+    dim3 grid(p.hkv, (max_seqlen_q + QT - 1) / QT, p.num_seqs);
+    paged_attn_prefill_kernel<G><<<grid, dim3(64 * kPfWaves), 0, stream>>>(p);
 }
 
 static int part_tokens_for(int block_size, int max_blocks_per_seq, int num_splits) {
