@@ -403,6 +403,98 @@ logismos_status_t logismos_launch_decode_step(const logismos_decode_config_t* cf
                                               logismos_stream_t stream);
 
 /* ------------------------------------------------------------------------
+ * Paged KV cache (host object over device pools)
+ * ------------------------------------------------------------------------ */
+
+/* Rows [start_pos, start_pos + n_tokens) of ONE sequence, contiguous fp16
+ * `[n_tokens][num_kv_heads*head_dim]`, to / from the pools through the
+ * sequence's block-table row (device int32): the device side of
+ * `KvCache::put` and `KvCache::get` (crates/cache/src/lib.rs:57-68; row order
+ * and bytes as `FlatKvCache`, crates/cache/src/flat.rs:180-304). */
+logismos_status_t logismos_launch_kv_append_fp16(const void* k_new_f16, const void* v_new_f16,
+                                                 void* k_pool_f16, void* v_pool_f16,
+                                                 const int32_t* block_table_row, int start_pos,
+                                                 int n_tokens, int num_kv_heads, int head_dim,
+                                                 int block_size, logismos_stream_t stream);
+logismos_status_t logismos_launch_kv_gather_fp16(const void* k_pool_f16, const void* v_pool_f16,
+                                                 const int32_t* block_table_row, void* k_out_f16,
+                                                 void* v_out_f16, int start_pos, int n_tokens,
+                                                 int num_kv_heads, int head_dim, int block_size,
+                                                 logismos_stream_t stream);
+
+/* `CacheLayout` (crates/cache/src/flat.rs:36-69) for a paged cache: max_seq_len
+ * = block_size * max_blocks_per_seq; dtype is fp16. */
+typedef struct {
+    int num_layers;
+    int num_kv_heads;
+    int head_dim;
+    int block_size;         /* rows per block, multiple of 16 */
+    int num_blocks;         /* blocks in every layer's K pool and V pool */
+    int max_seqs;           /* sequence slots */
+    int max_blocks_per_seq; /* width of the block table */
+} logismos_paged_kv_layout_t;
+
+typedef struct logismos_paged_kv_cache logismos_paged_kv_cache_t;
+
+/* Results: the variants of the reference's cache `Error`
+ * (crates/cache/src/error.rs) that apply, plus the pool-specific ones. */
+enum {
+    LOGISMOS_KV_OK = 0,
+    LOGISMOS_KV_LAYER_OUT_OF_RANGE = 1,   /* Error::LayerOutOfRange */
+    LOGISMOS_KV_LEN_OVERFLOW = 2,         /* Error::LenOverflow */
+    LOGISMOS_KV_READ_BEYOND_WRITTEN = 3,  /* Error::ReadBeyondWritten */
+    LOGISMOS_KV_SHAPE_MISMATCH = 4,       /* Error::ShapeMismatch */
+    LOGISMOS_KV_BAD_SEQ = 5,              /* sequence id not open */
+    LOGISMOS_KV_OUT_OF_BLOCKS = 6,        /* free list exhausted */
+    LOGISMOS_KV_OUT_OF_SEQS = 7,          /* no free sequence slot */
+    LOGISMOS_KV_HIP_ERROR = 8             /* allocation, copy or launch failed */
+};
+
+/* The paged implementation the `KvCache` trait was left open for
+ * (crates/cache/src/lib.rs:9-13,51-82), one instance per device; create and
+ * destroy allocate and free device memory (the current device), nothing else does.
+ * put / get / len_of / num_layers / reset keep the trait's meaning per sequence:
+ *   put     appends n_tokens rows to (seq, layer); refuses LayerOutOfRange and
+ *           LenOverflow like FlatKvCache::put (crates/cache/src/flat.rs:180-255);
+ *           takes blocks from the free list as the sequence grows
+ *   get     gathers the first len rows into contiguous buffers; refuses
+ *           ReadBeyondWritten like FlatKvCache::get (:257-304)
+ *   len_of  written rows, or -1 where the trait returns None
+ *   reset   every open sequence back to length zero, its blocks freed
+ * open_seq / close_seq admit and retire a sequence; reserve makes the block
+ * table cover total_rows rows ahead of a step whose kernels write the rows
+ * themselves (`logismos_launch_rope_kv_write_*`), and advance then records
+ * those rows as written.  k_pool / v_pool / block_tables return the device
+ * pointers the attention and packing entry points take (block table row of
+ * sequence s at `block_tables + s * max_blocks_per_seq`; entries without a
+ * block hold 0x3FFFFFFF).  Copies and launches go to `stream`; one caller
+ * thread at a time per cache. */
+int logismos_paged_kv_cache_create(const logismos_paged_kv_layout_t* layout,
+                                   logismos_paged_kv_cache_t** out);
+void logismos_paged_kv_cache_destroy(logismos_paged_kv_cache_t* cache);
+int logismos_paged_kv_cache_open_seq(logismos_paged_kv_cache_t* cache, int* seq_id);
+int logismos_paged_kv_cache_close_seq(logismos_paged_kv_cache_t* cache, int seq_id);
+int logismos_paged_kv_cache_reserve(logismos_paged_kv_cache_t* cache, int seq_id,
+                                    int64_t total_rows, logismos_stream_t stream);
+int logismos_paged_kv_cache_advance(logismos_paged_kv_cache_t* cache, int seq_id, int layer_idx,
+                                    int n_tokens);
+int logismos_paged_kv_cache_put(logismos_paged_kv_cache_t* cache, int seq_id, int layer_idx,
+                                const void* k_f16, const void* v_f16, int n_tokens,
+                                logismos_stream_t stream);
+int logismos_paged_kv_cache_get(const logismos_paged_kv_cache_t* cache, int seq_id, int layer_idx,
+                                int64_t len, void* k_out_f16, void* v_out_f16,
+                                logismos_stream_t stream);
+int64_t logismos_paged_kv_cache_len_of(const logismos_paged_kv_cache_t* cache, int seq_id,
+                                       int layer_idx);
+int logismos_paged_kv_cache_num_layers(const logismos_paged_kv_cache_t* cache);
+void logismos_paged_kv_cache_reset(logismos_paged_kv_cache_t* cache);
+int logismos_paged_kv_cache_free_blocks(const logismos_paged_kv_cache_t* cache);
+void* logismos_paged_kv_cache_k_pool(const logismos_paged_kv_cache_t* cache, int layer_idx);
+void* logismos_paged_kv_cache_v_pool(const logismos_paged_kv_cache_t* cache, int layer_idx);
+const int32_t* logismos_paged_kv_cache_block_tables(const logismos_paged_kv_cache_t* cache);
+const int32_t* logismos_paged_kv_cache_block_tables_host(const logismos_paged_kv_cache_t* cache);
+
+/* ------------------------------------------------------------------------
  * Memory-system probes (measurement aids; the reference has no counterpart,
  * its only timing helper is the hipEvent pair of
  * crates/kernels/examples/gemm_bench.rs:120-128).  A plain copy and a plain

@@ -63,7 +63,80 @@ __global__ __launch_bounds__(256) void kv_write_kernel(const uint4_t* __restrict
     v_pool[slot * row_vec + j] = v_new[idx];
 }
 
+// One sequence's rows [start_pos, start_pos + n_tokens) <-> contiguous rows, through the
+// sequence's block-table row.  TO_POOL: contiguous -> pool (append); else pool -> contiguous
+// (gather).  16 bytes per lane.
+template <bool TO_POOL>
+__global__ __launch_bounds__(256) void kv_seq_copy_kernel(uint4_t* __restrict__ k_flat,
+                                                          uint4_t* __restrict__ v_flat,
+                                                          uint4_t* __restrict__ k_pool,
+                                                          uint4_t* __restrict__ v_pool,
+                                                          const int32_t* __restrict__ bt_row,
+                                                          int start_pos, int n_tokens, int row_vec,
+                                                          int block_size) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (int64_t)n_tokens * row_vec) return;
+    const int t = (int)(idx / row_vec);
+    const int64_t j = idx - (int64_t)t * row_vec;
+    const int pos = start_pos + t;
+    const int bi = pos / block_size;
+    const int64_t slot = (int64_t)bt_row[bi] * block_size + (pos - bi * block_size);
+    if (TO_POOL) {
+        k_pool[slot * row_vec + j] = k_flat[idx];
+        v_pool[slot * row_vec + j] = v_flat[idx];
+    } else {
+        k_flat[idx] = k_pool[slot * row_vec + j];
+        v_flat[idx] = v_pool[slot * row_vec + j];
+    }
+}
+
 }  // namespace lg
+
+static logismos_status_t kv_seq_copy(bool to_pool, void* k_flat, void* v_flat, void* k_pool,
+                                     void* v_pool, const int32_t* bt_row, int start_pos,
+                                     int n_tokens, int num_kv_heads, int head_dim, int block_size,
+                                     logismos_stream_t stream) {
+    if (start_pos < 0 || n_tokens < 0 || num_kv_heads <= 0 || head_dim <= 0 || block_size <= 0)
+        return hipErrorInvalidValue;
+    const int64_t row_elems = (int64_t)num_kv_heads * head_dim;
+    if (row_elems % 8 != 0 || row_elems > INT32_MAX) return hipErrorInvalidValue;
+    if ((int64_t)start_pos + n_tokens > (int64_t)INT32_MAX) return hipErrorInvalidValue;
+    if (n_tokens == 0) return hipSuccess;
+    if (!k_flat || !v_flat || !k_pool || !v_pool || !bt_row) return hipErrorInvalidValue;
+    const int row_vec = (int)(row_elems / 8);
+    const int64_t items = (int64_t)n_tokens * row_vec;
+    const dim3 grid((unsigned)((items + 255) / 256));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    auto* kf = static_cast<lg::uint4_t*>(k_flat);
+    auto* vf = static_cast<lg::uint4_t*>(v_flat);
+    auto* kp = static_cast<lg::uint4_t*>(k_pool);
+    auto* vp = static_cast<lg::uint4_t*>(v_pool);
+    if (to_pool)
+        lg::kv_seq_copy_kernel<true><<<grid, dim3(256), 0, st>>>(kf, vf, kp, vp, bt_row, start_pos,
+                                                                 n_tokens, row_vec, block_size);
+    else
+        lg::kv_seq_copy_kernel<false><<<grid, dim3(256), 0, st>>>(kf, vf, kp, vp, bt_row, start_pos,
+                                                                  n_tokens, row_vec, block_size);
+    return hipGetLastError();
+}
+
+extern "C" logismos_status_t logismos_launch_kv_append_fp16(
+    const void* k_new_f16, const void* v_new_f16, void* k_pool_f16, void* v_pool_f16,
+    const int32_t* block_table_row, int start_pos, int n_tokens, int num_kv_heads, int head_dim,
+    int block_size, logismos_stream_t stream) {
+    return kv_seq_copy(true, const_cast<void*>(k_new_f16), const_cast<void*>(v_new_f16), k_pool_f16,
+                       v_pool_f16, block_table_row, start_pos, n_tokens, num_kv_heads, head_dim,
+                       block_size, stream);
+}
+
+extern "C" logismos_status_t logismos_launch_kv_gather_fp16(
+    const void* k_pool_f16, const void* v_pool_f16, const int32_t* block_table_row, void* k_out_f16,
+    void* v_out_f16, int start_pos, int n_tokens, int num_kv_heads, int head_dim, int block_size,
+    logismos_stream_t stream) {
+    return kv_seq_copy(false, k_out_f16, v_out_f16, const_cast<void*>(k_pool_f16),
+                       const_cast<void*>(v_pool_f16), block_table_row, start_pos, n_tokens,
+                       num_kv_heads, head_dim, block_size, stream);
+}
 
 extern "C" logismos_status_t logismos_check_pack_ragged_shape(int num_seqs, int block_size,
                                                               int max_blocks, char* msg,

@@ -133,6 +133,26 @@ class Event:
             pass
 
 
+class DevicePtrView:
+    """Borrowed device memory (owned by someone else, e.g. a cache's pool): read-back only."""
+
+    def __init__(self, ptr: C.c_void_p, nbytes: int):
+        self._p = C.c_void_p(ptr.value if isinstance(ptr, C.c_void_p) else int(ptr))
+        self.nbytes = int(nbytes)
+
+    @property
+    def ptr(self) -> C.c_void_p:
+        return self._p
+
+    def to_numpy(self, dtype, shape=None) -> np.ndarray:
+        out = np.empty(self.nbytes // np.dtype(dtype).itemsize if shape is None else shape, dtype)
+        assert out.nbytes <= self.nbytes
+        if out.nbytes:
+            check(_runtime().hipMemcpy(out.ctypes.data_as(C.c_void_p), self._p,
+                                       C.c_size_t(out.nbytes), C.c_int(2)), "hipMemcpy(D2H)")
+        return out
+
+
 class DeviceBuffer:
     """Owned device allocation (`hipcore::DeviceBuffer`, crates/hipcore/src/memory.rs)."""
 

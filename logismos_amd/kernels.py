@@ -78,11 +78,34 @@ _SIGNATURES = {
     "logismos_launch_add_rms_norm_f32p_xprep":
         (C.c_uint32, [_vp, _vp, _i, _vp, _vp, _i, _i, _f, _vp]),
     "logismos_launch_silu_mul_f32p_xprep": (C.c_uint32, [_vp, _i, _vp, _i, _i, _vp]),
+    "logismos_launch_kv_append_fp16": (C.c_uint32, [_vp] * 5 + [_i] * 5 + [_vp]),
+    "logismos_launch_kv_gather_fp16": (C.c_uint32, [_vp] * 5 + [_i] * 5 + [_vp]),
+    "logismos_paged_kv_cache_create": (C.c_int, [_vp, C.POINTER(_vp)]),
+    "logismos_paged_kv_cache_destroy": (None, [_vp]),
+    "logismos_paged_kv_cache_open_seq": (C.c_int, [_vp, C.POINTER(C.c_int)]),
+    "logismos_paged_kv_cache_close_seq": (C.c_int, [_vp, _i]),
+    "logismos_paged_kv_cache_reserve": (C.c_int, [_vp, _i, C.c_int64, _vp]),
+    "logismos_paged_kv_cache_advance": (C.c_int, [_vp, _i, _i, _i]),
+    "logismos_paged_kv_cache_put": (C.c_int, [_vp, _i, _i, _vp, _vp, _i, _vp]),
+    "logismos_paged_kv_cache_get": (C.c_int, [_vp, _i, _i, C.c_int64, _vp, _vp, _vp]),
+    "logismos_paged_kv_cache_len_of": (C.c_int64, [_vp, _i, _i]),
+    "logismos_paged_kv_cache_num_layers": (C.c_int, [_vp]),
+    "logismos_paged_kv_cache_reset": (None, [_vp]),
+    "logismos_paged_kv_cache_free_blocks": (C.c_int, [_vp]),
+    "logismos_paged_kv_cache_k_pool": (_vp, [_vp, _i]),
+    "logismos_paged_kv_cache_v_pool": (_vp, [_vp, _i]),
+    "logismos_paged_kv_cache_block_tables": (_vp, [_vp]),
+    "logismos_paged_kv_cache_block_tables_host": (_vp, [_vp]),
     "logismos_launch_probe_copy": (C.c_uint32, [_vp, _vp, _sz, _vp]),
     "logismos_launch_probe_read": (C.c_uint32, [_vp, _vp, _sz, _vp]),
 }
 
 ATTN_PHASE_DECODE, ATTN_PHASE_PREFILL, ATTN_PHASE_MERGE, ATTN_PHASE_ALL = 1, 2, 4, 7
+
+
+class PagedKvLayout(C.Structure):
+    _fields_ = [("num_layers", _i), ("num_kv_heads", _i), ("head_dim", _i), ("block_size", _i),
+                ("num_blocks", _i), ("max_seqs", _i), ("max_blocks_per_seq", _i)]
 
 
 class Q4Weight(C.Structure):
@@ -133,7 +156,7 @@ def _raw(stream) -> C.c_void_p | None:
 
 
 def _ptr(x) -> C.c_void_p:
-    return x.ptr if isinstance(x, hip.DeviceBuffer) else x
+    return x.ptr if isinstance(x, (hip.DeviceBuffer, hip.DevicePtrView)) else x
 
 
 def _guard(kernel: str, check_fn, *dims) -> None:
