@@ -177,7 +177,7 @@ def bench_paged_decode(args):
                    "hip_graph": graphed},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "paged_attn_kernel<6,decode>", "ms_per_launch": round(ms_dec, 5),
+                     "kernel": "paged_attn_balanced_kernel<6>", "ms_per_launch": round(ms_dec, 5),
                      "warm_cache_GBps": round(algo / (ms_warm * 1e-3) / 1e9, 1)},
         "cpu_baseline": {"value": round(cpu_gbps, 2), "unit": "GB/s", "cores": cores,
                          "kind": "port",
@@ -482,7 +482,7 @@ def bench_decode_step(args):
                      "traffic_source": "profiles/paged_attn_decode_config5_pmc.txt (rocprofv3 "
                                        "--pmc FETCH_SIZE / WRITE_SIZE of this command at its "
                                        "default steps, bytes per launch)",
-                     "kernel": "paged_attn_kernel<4,decode> (one layer of the step)",
+                     "kernel": "paged_attn_balanced_kernel<4> (decode rows, one layer of the step)",
                      "ms_per_launch": round(ms_attn, 5), "algorithmic_bytes_per_launch": attn_bytes},
         "cpu_baseline": {"value": round(S / (cpu_s * L), 3), "unit": "tok/s", "cores": cores,
                          "kind": "port",

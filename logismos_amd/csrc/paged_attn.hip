@@ -56,15 +56,16 @@ struct AttnParams {
     const int32_t* cu_seqlens_q;
     const int32_t* context_lens;
     _Float16* out;
-    float* ws_acc;  // [num_seqs][num_splits][hq][128]
-    float* ws_ml;   // [num_seqs][num_splits][hq][2]
+    float* ws_acc;  // [slot][hq][128], slot < num_seqs * num_splits
+    float* ws_ml;   // [slot][hq][2]
     int num_seqs;
     int hq;
     int hkv;
     int block_size;
     int max_blocks_per_seq;
     int num_splits;
-    int part_tokens;  // keys per partition (multiple of 16)
+    int part_tokens;  // keys per partition (multiple of 16), static split only
+    int num_workers;  // > 0: balanced decode (see paged_attn_balanced_kernel), else static split
     float scale_log2e;
     int causal;
     // 0: fp16 [T][hq][128]; 1: bf16, same shape; 2: the prepared layout of the following
@@ -84,52 +85,41 @@ __device__ __forceinline__ unsigned short attn_out_elem(float v, int out_bf16) {
     return __builtin_bit_cast(unsigned short, hv);
 }
 
-// Decode rows: grid (num_splits, hkv / waves, num_seqs); sequences with exactly one
-// new token, keys split into partitions of part_tokens.  Sequences with more new
-// tokens belong to paged_attn_prefill_kernel below.
+// Output row of a query with no visible key: zeros (softmax over zero columns).
 template <int G>
-__global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_kernel(const AttnParams p) {
+__device__ __forceinline__ void attn_write_zero_row(const AttnParams& p, int t, int kvh, int lane) {
+    const int tg = lane >> 4;
+    const int c = lane & 15;
+    if (c >= G) return;
+    half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (p.out_bf16 == 2) {
+        const int bp = xprep_bp(p.out_rows);
+        const int head = kvh * G + c;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            reinterpret_cast<half8_t*>(p.out)[(int64_t)(head * 16 + tg + 4 * j) * bp + t] = z;
+        if (tg == 0)
+            reinterpret_cast<float*>(reinterpret_cast<char*>(p.out) +
+                                     xprep_xg_offset(p.out_rows, p.hq * kHeadDim))[(int64_t)head * bp + t] =
+                0.0f;
+    } else {
+        _Float16* o = p.out + ((int64_t)t * p.hq + kvh * G + c) * kHeadDim;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) *reinterpret_cast<half8_t*>(o + 8 * (tg + 4 * j)) = z;
+    }
+}
+
+// One wave: keys [tok_begin, tok_end) (tok_begin a multiple of 16, the range not empty)
+// of decode sequence s, KV head kvh, query token t.  `single`: the range is the whole
+// context and the normalised output is written; otherwise the partial (m, l, acc) goes to
+// workspace slot `slot`.
+template <int G>
+__device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t, int kvh,
+                                               int tok_begin, int tok_end, bool single,
+                                               int64_t slot) {
     const int lane = threadIdx.x & 63;
     const int tg = lane >> 4;
     const int c = lane & 15;
-    // the waves of a workgroup are consecutive KV heads of the same keys: together
-    // they stream whole token rows (hkv * 256 contiguous bytes)
-    const int kvh = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    const int s = blockIdx.z;
-
-    const int t0 = p.cu_seqlens_q[s];
-    const int n_new = p.cu_seqlens_q[s + 1] - t0;
-    const int ctx = p.context_lens[s];
-    if (n_new != 1) return;
-    const int t = t0;
-    const int vis = ctx;
-    const int split = blockIdx.x;
-    const int tok_begin = split * p.part_tokens;
-    if (vis <= 0) {
-        // no visible key: zeros (softmax over zero columns)
-        if (split == 0 && c < G) {
-            half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (p.out_bf16 == 2) {
-                const int bp = xprep_bp(p.out_rows);
-                const int head = kvh * G + c;
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    reinterpret_cast<half8_t*>(p.out)[(int64_t)(head * 16 + tg + 4 * j) * bp + t] = z;
-                if (tg == 0)
-                    reinterpret_cast<float*>(
-                        reinterpret_cast<char*>(p.out) +
-                        xprep_xg_offset(p.out_rows, p.hq * kHeadDim))[(int64_t)head * bp + t] = 0.0f;
-            } else {
-                _Float16* o = p.out + ((int64_t)t * p.hq + kvh * G + c) * kHeadDim;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) *reinterpret_cast<half8_t*>(o + 8 * (tg + 4 * j)) = z;
-            }
-        }
-        return;
-    }
-    if (tok_begin >= vis) return;
-    const int tok_end = min(vis, tok_begin + p.part_tokens);
-    const int num_parts = (vis + p.part_tokens - 1) / p.part_tokens;
     const int ntiles = (tok_end - tok_begin + kTileKeys - 1) / kTileKeys;
 
     // ---- query group as the MFMA B operand: column = head c, piece tg + 4j
@@ -268,7 +258,7 @@ __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_kernel(const At
         }
         if (tg == (h & 3)) {
             const int head = kvh * G + h;
-            if (num_parts == 1) {
+            if (single) {
                 const float inv = 1.0f / lh;
                 uint4_t o;
 #pragma unroll
@@ -290,7 +280,7 @@ __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_kernel(const At
                                                 8 * c) = o;
                 }
             } else {
-                const int64_t idx = ((int64_t)s * p.num_splits + split) * p.hq + head;
+                const int64_t idx = slot * p.hq + head;
                 float4_t a0 = {acc[h][0], acc[h][1], acc[h][2], acc[h][3]};
                 float4_t a1 = {acc[h][4], acc[h][5], acc[h][6], acc[h][7]};
                 float* dst = p.ws_acc + idx * kHeadDim + 8 * c;
@@ -305,6 +295,116 @@ __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_kernel(const At
     });
 }
 
+// Decode rows, static split: grid (num_splits, hkv / waves, num_seqs); sequences with
+// exactly one new token, keys split into partitions of part_tokens.  The waves of a
+// workgroup are consecutive KV heads of the same keys: together they stream whole token
+// rows (hkv * 256 contiguous bytes).  Sequences with more new tokens belong to
+// paged_attn_prefill_kernel below.
+template <int G>
+__global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_kernel(const AttnParams p) {
+    const int lane = threadIdx.x & 63;
+    const int kvh = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int s = blockIdx.z;
+    const int t = p.cu_seqlens_q[s];
+    if (p.cu_seqlens_q[s + 1] - t != 1) return;
+    const int ctx = p.context_lens[s];
+    const int split = blockIdx.x;
+    if (ctx <= 0) {
+        if (split == 0) attn_write_zero_row<G>(p, t, kvh, lane);
+        return;
+    }
+    const int tok_begin = split * p.part_tokens;
+    if (tok_begin >= ctx) return;
+    const int num_parts = (ctx + p.part_tokens - 1) / p.part_tokens;
+    attn_partition<G>(p, s, t, kvh, tok_begin, min(ctx, tok_begin + p.part_tokens), num_parts == 1,
+                      (int64_t)s * p.num_splits + split);
+}
+
+// 16-key tiles sequence s contributes to the decode stream
+__device__ __forceinline__ int decode_tiles(const AttnParams& p, int s) {
+    const int n_new = p.cu_seqlens_q[s + 1] - p.cu_seqlens_q[s];
+    const int ctx = p.context_lens[s];
+    return (n_new == 1 && ctx > 0) ? (ctx + kTileKeys - 1) / kTileKeys : 0;
+}
+
+constexpr int kMaxBalancedSeqs = 2048;  // prefix table held in LDS
+constexpr int kMinWorkerTiles = 8;      // a worker streams at least 128 keys
+
+__device__ __forceinline__ int worker_tiles(int total_tiles, int num_workers) {
+    const int r = (total_tiles + num_workers - 1) / num_workers;
+    return r < kMinWorkerTiles ? kMinWorkerTiles : r;
+}
+
+// Decode rows, balanced: the key tiles of all decode sequences form one stream (sequence
+// after sequence); worker w (a workgroup, grid.x = num_workers, one per CU's worth of
+// waves) takes tiles [w*R, (w+1)*R) of it, R = ceil(total / num_workers), whichever
+// sequences they belong to.  Every worker therefore reads the same number of bytes,
+// whatever the context lengths are: with static partitions 288 equal workgroups on 256
+// CUs take two rounds, and the measured rate drops from 5.6 to 4.3 TB/s.  A worker's
+// piece of sequence s is written to workspace slot w + s (the pieces of one sequence get
+// consecutive slots since both w and s only grow along the stream); a sequence that lies
+// inside one worker is finished there.
+template <int G>
+__global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_balanced_kernel(const AttnParams p) {
+    __shared__ int pt[kMaxBalancedSeqs + 1];  // exclusive prefix of decode tiles
+    const int lane = threadIdx.x & 63;
+    const int kvh = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int S = p.num_seqs;
+    if (threadIdx.x < 64) {
+        const int per = (S + 63) / 64;
+        int sum = 0;
+        for (int i = 0; i < per; ++i) {
+            const int s = lane * per + i;
+            if (s < S) sum += decode_tiles(p, s);
+        }
+        int incl = sum;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int v = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += v;
+        }
+        int run = incl - sum;
+        for (int i = 0; i < per; ++i) {
+            const int s = lane * per + i;
+            if (s < S) {
+                pt[s] = run;
+                run += decode_tiles(p, s);
+            }
+        }
+        if (lane == 63) pt[S] = incl;
+    }
+    __syncthreads();
+    // LDS reads land in vector registers: make the (wave-uniform) values scalar again so
+    // that block ids keep coming through scalar loads
+    const int total = __builtin_amdgcn_readfirstlane(pt[S]);
+    const int w = blockIdx.x;
+    const int R = worker_tiles(total, p.num_workers);
+    const int64_t tb64 = (int64_t)w * R;
+    if (tb64 >= total) return;
+    const int tb = (int)tb64;
+    const int te = (int)min((int64_t)total, tb64 + R);
+    // the sequence holding tile tb: the largest s with pt[s] <= tb (it has tiles, since
+    // pt[s + 1] > tb)
+    int lo = 0, hi = S;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (__builtin_amdgcn_readfirstlane(pt[mid]) <= tb) lo = mid;
+        else hi = mid;
+    }
+    int tcur = tb;
+    for (int s = lo; tcur < te; ++s) {
+        const int seq_begin = __builtin_amdgcn_readfirstlane(pt[s]);
+        const int seq_end = __builtin_amdgcn_readfirstlane(pt[s + 1]);
+        if (seq_end <= tcur) continue;  // a sequence without decode tiles
+        const int seg_end = min(te, seq_end);
+        const int ctx = p.context_lens[s];
+        const bool single = tcur == seq_begin && seg_end == seq_end;
+        attn_partition<G>(p, s, p.cu_seqlens_q[s], kvh, (tcur - seq_begin) * kTileKeys,
+                          min(ctx, (seg_end - seq_begin) * kTileKeys), single, (int64_t)w + s);
+        tcur = seg_end;
+    }
+}
+
 // Combines the partials of the decode sequences that used more than one
 // partition.  grid (hq, num_seqs), 256 threads: wave w folds partitions
 // w, w+4, ... (four independent partials in flight per round, two output
@@ -317,9 +417,50 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams 
     const int t0 = p.cu_seqlens_q[s];
     if (p.cu_seqlens_q[s + 1] - t0 != 1) return;
     const int ctx = p.context_lens[s];
-    const int np = (ctx + p.part_tokens - 1) / p.part_tokens;
-    if (np <= 1) return;
-    const int64_t base = ((int64_t)s * p.num_splits) * p.hq + h;
+    __shared__ float sm[4], sden[4], sn[4][kHeadDim];
+    __shared__ __attribute__((aligned(16))) unsigned short sout[kHeadDim];
+    __shared__ int red[2][4];
+    int np;              // partials of this sequence
+    int64_t first_slot;  // of its first partial
+    bool zero_row = false;
+    if (p.num_workers > 0) {
+        // balanced decode: recompute where this sequence sits in the stream of key tiles
+        int before = 0, total = 0;
+        for (int i = threadIdx.x; i < p.num_seqs; i += 256) {
+            const int nt = decode_tiles(p, i);
+            total += nt;
+            before += i < s ? nt : 0;
+        }
+#pragma unroll
+        for (int mask = 32; mask >= 1; mask >>= 1) {
+            total += __shfl_xor(total, mask, 64);
+            before += __shfl_xor(before, mask, 64);
+        }
+        if (lane == 0) {
+            red[0][w] = total;
+            red[1][w] = before;
+        }
+        __syncthreads();
+        total = red[0][0] + red[0][1] + red[0][2] + red[0][3];
+        before = red[1][0] + red[1][1] + red[1][2] + red[1][3];
+        const int nt = ctx > 0 ? (ctx + kTileKeys - 1) / kTileKeys : 0;
+        if (nt == 0) {
+            zero_row = true;  // the stream has no tile of this row: nobody wrote it
+            np = 0;
+            first_slot = 0;
+        } else {
+            const int R = worker_tiles(total, p.num_workers);
+            const int w_first = before / R;
+            np = (before + nt - 1) / R - w_first + 1;
+            first_slot = (int64_t)w_first + s;
+            if (np <= 1) return;
+        }
+    } else {
+        np = (ctx + p.part_tokens - 1) / p.part_tokens;
+        first_slot = (int64_t)s * p.num_splits;
+        if (np <= 1) return;
+    }
+    const int64_t base = first_slot * p.hq + h;
 
     float M = -INFINITY, den = 0.0f, n0 = 0.0f, n1 = 0.0f;
     for (int i0 = w; i0 < np; i0 += 16) {
@@ -354,8 +495,6 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams 
         }
         M = mx;
     }
-    __shared__ float sm[4], sden[4], sn[4][kHeadDim];
-    __shared__ __attribute__((aligned(16))) unsigned short sout[kHeadDim];
     if (lane == 0) {
         sm[w] = M;
         sden[w] = den;
@@ -373,7 +512,7 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams 
             dd = fmaf(g, sden[j], dd);
             num = fmaf(g, sn[j][d], num);
         }
-        const unsigned short ov = attn_out_elem(num / dd, p.out_bf16);
+        const unsigned short ov = zero_row ? (unsigned short)0 : attn_out_elem(num / dd, p.out_bf16);
         if (p.out_bf16 != 2)
             reinterpret_cast<unsigned short*>(p.out)[((int64_t)t0 * p.hq + h) * kHeadDim + d] = ov;
         else
@@ -765,6 +904,18 @@ static void launch_prefill(const AttnParams& p, int max_seqlen_q, hipStream_t st
     paged_attn_prefill_kernel<G><<<grid, dim3(64 * kPfWaves), 0, stream>>>(p);
 }
 
+// Workers of the balanced decode kernel: eight waves per CU (one wave = one KV head of one
+// worker), limited by the workspace the caller sized for num_splits partials per sequence
+// (slots used: at most workers + num_seqs - 1).  0: static split (one partition, or more
+// sequences than the prefix table holds).
+static int balanced_workers(int num_seqs, int num_kv_heads, int num_splits) {
+    if (num_splits <= 1 || num_seqs > kMaxBalancedSeqs) return 0;
+    int64_t target = (int64_t)device_cu_count() * kMaxHeadWaves / num_kv_heads;
+    if (target < 1) target = 1;
+    const int64_t cap = (int64_t)num_seqs * (num_splits - 1);
+    return (int)(target < cap ? target : cap);
+}
+
 static int part_tokens_for(int block_size, int max_blocks_per_seq, int num_splits) {
     const int64_t max_ctx = (int64_t)block_size * max_blocks_per_seq;
     int64_t part = (max_ctx + num_splits - 1) / num_splits;
@@ -784,8 +935,13 @@ static hipError_t launch_group(const AttnParams& p, int max_seqlen_q, int phases
         }
     dim3 block(64 * wpb);
     if (phases & LOGISMOS_ATTN_PHASE_DECODE) {
-        dim3 grid_d(p.num_splits, p.hkv / wpb, p.num_seqs);
-        paged_attn_kernel<G><<<grid_d, block, 0, stream>>>(p);
+        if (p.num_workers > 0) {
+            dim3 grid_d(p.num_workers, p.hkv / wpb, 1);
+            paged_attn_balanced_kernel<G><<<grid_d, block, 0, stream>>>(p);
+        } else {
+            dim3 grid_d(p.num_splits, p.hkv / wpb, p.num_seqs);
+            paged_attn_kernel<G><<<grid_d, block, 0, stream>>>(p);
+        }
     }
     if ((phases & LOGISMOS_ATTN_PHASE_PREFILL) && max_seqlen_q > 1) {
         launch_prefill<G>(p, max_seqlen_q, stream);
@@ -849,8 +1005,17 @@ extern "C" logismos_status_t logismos_check_paged_attn_shape(int num_seqs, int t
 extern "C" int logismos_paged_attn_num_splits(int num_seqs, int num_kv_heads, int block_size,
                                               int max_blocks_per_seq) {
     if (num_seqs <= 0 || num_kv_heads <= 0 || block_size <= 0 || max_blocks_per_seq <= 0) return 1;
-    // Aim at ~4096 waves over the chip if every sequence were full length,
-    // with partitions of 64..512 keys.
+    if (num_seqs <= lg::kMaxBalancedSeqs) {
+        // balanced decode: enough partial slots for one worker per CU's worth of waves
+        int64_t target = (int64_t)lg::device_cu_count() * lg::kMaxHeadWaves / num_kv_heads;
+        if (target < 1) target = 1;
+        int64_t splits = (target + num_seqs - 1) / num_seqs + 1;
+        if (splits < 2) splits = 2;
+        if (splits > 4096) splits = 4096;
+        return (int)splits;
+    }
+    // static split: aim at ~4096 waves over the chip if every sequence were full length,
+    // with partitions of 64..512 keys
     const int64_t max_ctx = (int64_t)block_size * max_blocks_per_seq;
     int64_t part = (int64_t)num_seqs * num_kv_heads * max_ctx / 4096;
     if (part < 64) part = 64;
@@ -928,6 +1093,7 @@ logismos_status_t lg::paged_attn_launch(
     p.max_blocks_per_seq = max_blocks_per_seq;
     p.num_splits = num_splits;
     p.part_tokens = lg::part_tokens_for(block_size, max_blocks_per_seq, num_splits);
+    p.num_workers = lg::balanced_workers(num_seqs, num_kv_heads, num_splits);
     p.scale_log2e = scale * lg::kLog2e;
     p.causal = causal;
     p.out_bf16 = out_bf16;
