@@ -215,8 +215,10 @@ struct SplitkPlan {
 
 // Deterministic in (b, n, k) and the CU count.  Cost relative to the weight
 // bytes: 1 (weights) + x re-reads (128/R per 32 batch rows, served by L2)
-// + partial write + read (4/gp per 32 batch rows, mostly cache-resident), times
-// the idle fraction when the workgroups do not fill the CUs evenly.
+// + the fp32 parts (4/gp per 32 batch rows, written here and read back by the
+// consumer, whose few workgroups read them slowly: weighted 1.5), times a mild
+// penalty when the workgroups do not fill the CUs evenly (measured kernels lose far
+// less than the idle fraction suggests, because fewer resident workgroups run faster).
 static SplitkPlan splitk_plan(int b, int n, int k) {
     const int groups = k / 128;
     const int tiles = (n + 15) / 16;
@@ -225,20 +227,23 @@ static SplitkPlan splitk_plan(int b, int n, int k) {
     SplitkPlan best{1, 1, groups};
     double best_cost = 1e30;
     const int tws[] = {1, 2, 4};
-    const int gps[] = {1, 2, 4};
+    const int gps[] = {1, 2, 4, 8};
     for (int tw : tws)
         for (int gp : gps) {
             if (gp > groups && gp != 1) continue;
             if (b > 16 && tw * gp > 8) continue;  // register budget with two batch tiles
+            if (gp == 8 && tw > 2) continue;      // instantiated: (8,1), (8,2)
             const int parts = (groups + gp - 1) / gp;
             const int tpw = kSplitkWaves * tw;
             const long wgs = (long)((tiles + tpw - 1) / tpw) * parts;
             const double r = 16.0 * tpw;
-            double cost = 1.0 + 0.35 * bs * 128.0 / r + 0.5 * bs * 4.0 / gp;
-            // four workgroups fit a CU: count rounds of 4*cus workgroups
-            const double fill = (double)wgs / (4.0 * cus);
-            const double rounds = fill <= 1.0 ? 1.0 : ceil(fill);
-            cost *= rounds / (fill < 0.25 ? 0.25 : fill);
+            double cost = 1.0 + 0.35 * bs * 128.0 / r + 1.5 * bs * 4.0 / gp;
+            // resident workgroups per CU: four, two when the x part takes 64 KiB of LDS
+            const double fill = (double)wgs / ((gp == 8 ? 2.0 : 4.0) * cus);
+            if (fill <= 1.0)
+                cost *= 1.0 + 0.3 * (1.0 - fill);
+            else
+                cost *= 1.0 + 0.5 * (ceil(fill) / fill - 1.0);
             if (cost < best_cost) {
                 best_cost = cost;
                 best = SplitkPlan{tw, gp, parts};
@@ -257,6 +262,13 @@ static hipError_t launch_splitk(const void* x, const void* qw, const void* scale
     const size_t lds =
         (size_t)BP * (GP * 16 + 1) * 16 + (size_t)GP * BP * 4 + (size_t)2 * ROWS * GP * 2;
     auto kern = qgemm_q4g128_splitk_kernel<BT, GP, TW, PREP>;
+    if (lds > 64 * 1024) {
+        // above the default dynamic-LDS limit: opt in once per instantiation
+        static const hipError_t opt = hipFuncSetAttribute(
+            reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+            160 * 1024 - 1024);
+        if (opt != hipSuccess) return opt;
+    }
     dim3 grid((tiles + kSplitkWaves * TW - 1) / (kSplitkWaves * TW), plan.parts);
     kern<<<grid, dim3(kSplitkThreads), lds, stream>>>(
         static_cast<const uint16_t*>(x), static_cast<const uint8_t*>(qw),
@@ -275,6 +287,7 @@ static hipError_t launch_splitk_bt(const void* x, const void* qw, const void* sc
     LG_SPLITK_CASE(1, 1) LG_SPLITK_CASE(1, 2) LG_SPLITK_CASE(1, 4)
     LG_SPLITK_CASE(2, 1) LG_SPLITK_CASE(2, 2) LG_SPLITK_CASE(2, 4)
     LG_SPLITK_CASE(4, 1) LG_SPLITK_CASE(4, 2)
+    LG_SPLITK_CASE(8, 1) LG_SPLITK_CASE(8, 2)
     if constexpr (BT == 1) {
         LG_SPLITK_CASE(4, 4)
     }
