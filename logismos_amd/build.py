@@ -39,6 +39,7 @@ HIPCC_FLAGS = [
 # prefill kernel ~50 register-to-register moves per key tile around its softmax).
 EXTRA_FLAGS = {
     "paged_attn.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "qgemm_q4_splitk.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
 }
 
 

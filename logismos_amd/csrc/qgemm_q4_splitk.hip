@@ -77,7 +77,8 @@ __global__ __launch_bounds__(kSplitkThreads) void qgemm_q4g128_splitk_kernel(
         const int idc = idx < x_total ? idx : x_total - 1;
         if constexpr (PREP) {
             // the K part of the prepared x is one contiguous block of 16-byte words
-            xd[u] = reinterpret_cast<const uint4_t*>(x)[(int64_t)g0 * 16 * BP + idc];
+            const uint4_t* xb = reinterpret_cast<const uint4_t*>(x) + (int64_t)g0 * 16 * BP;
+            xd[u] = xb[(unsigned)idc];
         } else {
             const int bi = idc / chunks, q = idc - bi * chunks;
             xd[u] = *reinterpret_cast<const uint4_t*>(x + (int64_t)bi * k + (int64_t)g0 * 128 +
@@ -91,31 +92,34 @@ __global__ __launch_bounds__(kSplitkThreads) void qgemm_q4g128_splitk_kernel(
         const int t = (int)threadIdx.x < gcount * BP ? (int)threadIdx.x : 0;
         xgd = xg_src[(int64_t)g0 * BP + t];
     }
+    // scale / zero of (row r, group g): thread idx -> r = idx / GP, g = idx % GP; rows and
+    // groups past the end repeat the last valid one (their products are dropped below)
     constexpr int SZU = (ROWS * GP + kSplitkThreads - 1) / kSplitkThreads;
-    const int sz_total = rows_here * gcount;
+    const __half* sbase = scale + row0 * groups + g0;  // workgroup-uniform
+    const __half* zbase = zero + row0 * groups + g0;
     __half sd[SZU], zd[SZU];
 #pragma unroll
     for (int u = 0; u < SZU; ++u) {
         const int idx = u * kSplitkThreads + (int)threadIdx.x;
-        const int idc = idx < sz_total ? idx : sz_total - 1;
-        const int r = idc / gcount, g = idc - r * gcount;
-        sd[u] = scale[(row0 + r) * groups + g0 + g];
-        zd[u] = zero[(row0 + r) * groups + g0 + g];
+        const int r = min(idx / GP, rows_here - 1), g = min(idx % GP, gcount - 1);
+        const unsigned off = (unsigned)r * (unsigned)groups + (unsigned)g;
+        sd[u] = sbase[off];
+        zd[u] = zbase[off];
     }
     __builtin_amdgcn_sched_barrier(0);
 
     // this wave's TW tiles: rows (wave*TW + t)*16 .. +16
     uint4_t w[TW][GP];
+    const uint8_t* wbase = qw + row0 * (int64_t)(k >> 1) + (int64_t)g0 * 64;  // uniform
 #pragma unroll
     for (int t = 0; t < TW; ++t) {
         const int r = (wave * TW + t) * 16 + col;
-        const uint8_t* wrow =
-            qw + (row0 + (r < rows_here ? r : rows_here - 1)) * (int64_t)(k >> 1) + kc * 16;
+        const unsigned woff =
+            (unsigned)(r < rows_here ? r : rows_here - 1) * (unsigned)(k >> 1) + (unsigned)kc * 16u;
 #pragma unroll
-        for (int i = 0; i < GP; ++i) {
-            const int g = (i < gcount) ? (g0 + i) : (g0 + gcount - 1);
-            w[t][i] = *reinterpret_cast<const uint4_t*>(wrow + (int64_t)g * 64);
-        }
+        for (int i = 0; i < GP; ++i)
+            w[t][i] = *reinterpret_cast<const uint4_t*>(wbase + woff +
+                                                        64u * (unsigned)(i < gcount ? i : gcount - 1));
     }
     __builtin_amdgcn_sched_barrier(0);
 
@@ -141,10 +145,9 @@ __global__ __launch_bounds__(kSplitkThreads) void qgemm_q4g128_splitk_kernel(
 #pragma unroll
     for (int u = 0; u < SZU; ++u) {
         const int idx = u * kSplitkThreads + (int)threadIdx.x;
-        if (idx < sz_total) {
-            const int r = idx / gcount, g = idx - r * gcount;
-            szl[r * GP + g] = sd[u];
-            szl[ROWS * GP + r * GP + g] = zd[u];
+        if (idx < ROWS * GP) {
+            szl[idx] = sd[u];
+            szl[ROWS * GP + idx] = zd[u];
         }
     }
     __syncthreads();
@@ -159,9 +162,11 @@ __global__ __launch_bounds__(kSplitkThreads) void qgemm_q4g128_splitk_kernel(
         for (int bt = 0; bt < BT; ++bt) ysum[bt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int i = 0; i < GP; ++i) {
+            // a group past the end of K (last part only): scale 0, operands of group 0
             const bool valid = i < gcount;  // uniform
-            const float sf = __half2float(szl[rl * GP + (valid ? i : 0)]);
-            const float off = 128.0f + __half2float(zl[rl * GP + (valid ? i : 0)]);
+            const int ix = valid ? i : 0;
+            const float sf = valid ? __half2float(szl[rl * GP + i]) : 0.0f;
+            const float off = 128.0f + __half2float(zl[rl * GP + ix]);
             float4_t acc[BT];
 #pragma unroll
             for (int bt = 0; bt < BT; ++bt) acc[bt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
@@ -172,7 +177,7 @@ __global__ __launch_bounds__(kSplitkThreads) void qgemm_q4g128_splitk_kernel(
 #pragma unroll
                 for (int sft = 0; sft < 4; ++sft) h[sft] = ((wd >> (4 * sft)) & kNibMask) | magic;
                 const bf16x8_t bop = __builtin_bit_cast(bf16x8_t, h);
-                const int q = i * 16 + 4 * kc + s4;
+                const int q = ix * 16 + 4 * kc + s4;
 #pragma unroll
                 for (int bt = 0; bt < BT; ++bt)
                     acc[bt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
@@ -183,25 +188,23 @@ __global__ __launch_bounds__(kSplitkThreads) void qgemm_q4g128_splitk_kernel(
 #pragma unroll
             for (int bt = 0; bt < BT; ++bt) {
                 const float4_t xsum =
-                    *reinterpret_cast<const float4_t*>(xg + i * BP + bt * 16 + 4 * kc);
+                    *reinterpret_cast<const float4_t*>(xg + ix * BP + bt * 16 + 4 * kc);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float v = fmaf(sf, fmaf(-off, xsum[e], acc[bt][e]), ysum[bt][e]);
-                    ysum[bt][e] = valid ? v : ysum[bt][e];
-                }
+                for (int e = 0; e < 4; ++e)
+                    ysum[bt][e] = fmaf(sf, fmaf(-off, xsum[e], acc[bt][e]), ysum[bt][e]);
             }
             // one group at a time: without this the scheduler hoists the LDS reads of
             // every group (GP*4*BT operands of four registers) and spills
             __builtin_amdgcn_sched_barrier(0);
         }
         if (r < rows_here) {
+            float* pbase = part + (int64_t)j * b * n + row0;  // uniform
 #pragma unroll
             for (int bt = 0; bt < BT; ++bt)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int bi = bt * 16 + 4 * kc + e;
-                    if (bi < b)
-                        part[((int64_t)j * b + bi) * n + row0 + r] = ysum[bt][e];
+                    if (bi < b) pbase[(unsigned)bi * (unsigned)n + (unsigned)r] = ysum[bt][e];
                 }
         }
     }
