@@ -40,6 +40,7 @@ HIPCC_FLAGS = [
 EXTRA_FLAGS = {
     "paged_attn.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "qgemm_q4_splitk.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "qgemm_q4_stream.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
 }
 
 

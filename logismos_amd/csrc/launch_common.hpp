@@ -30,4 +30,12 @@ logismos_status_t paged_attn_launch(
     int head_dim, int block_size, int max_blocks_per_seq, int num_splits, float scale, int causal,
     int phases, int out_bf16, logismos_stream_t stream);
 
+// Streaming Q4G128 GEMM over prepared activations (qgemm_q4_stream.hip): steps per worker
+// for this shape (0: not applicable, use the split-K kernel) and the launch.  K parts are
+// 8 groups there, so a shape it applies to has K/1024 parts.
+int stream_steps(int b, int n, int k);
+hipError_t qgemm_q4_stream_launch(const void* xprep, const void* qw, const void* scale,
+                                  const void* zero, void* part, int b, int n, int k, int steps,
+                                  hipStream_t stream);
+
 }  // namespace lg

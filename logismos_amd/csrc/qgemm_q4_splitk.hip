@@ -227,6 +227,8 @@ static SplitkPlan splitk_plan(int b, int n, int k) {
     const int tiles = (n + 15) / 16;
     const int cus = device_cu_count();
     const double bs = (double)b / 32.0;
+    // shapes the streaming kernel takes (prepared x) use its K parts in both entry points
+    if (stream_steps(b, n, k) > 0) return SplitkPlan{1, 8, groups / 8};
     SplitkPlan best{1, 1, groups};
     double best_cost = 1e30;
     const int tws[] = {1, 2, 4};
@@ -316,6 +318,9 @@ static logismos_status_t splitk_dispatch(const void* x, bool prepared, const voi
     const lg::SplitkPlan plan = lg::splitk_plan(b, n, k);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (prepared) {
+        if (const int steps = lg::stream_steps(b, n, k))
+            return lg::qgemm_q4_stream_launch(x, qw_u8, scale_f16, zero_f16, parts_f32, b, n, k,
+                                              steps, st);
         if (b <= 16)
             return lg::launch_splitk_bt<1, true>(x, qw_u8, scale_f16, zero_f16, parts_f32, b, n, k,
                                                  plan, st);

@@ -144,7 +144,11 @@ def test_splitk_ragged_shapes(b, n, k):
 
 
 @pytest.mark.parametrize("b,n,k", [(32, 6144, 4096), (32, 4096, 12288), (5, 16, 128),
-                                   (17, 33, 384), (16, 1000, 1152), (31, 4100, 2048)])
+                                   (17, 33, 384), (16, 1000, 1152), (31, 4100, 2048),
+                                   # shapes the streaming kernel takes: whole and ragged row
+                                   # tiles, one and two batch tiles, one to twelve K parts
+                                   (32, 24576, 4096), (16, 24576, 4096), (32, 24570, 2048),
+                                   (7, 45003, 1024), (3, 12288, 4096)])
 def test_splitk_with_prepared_x_is_bit_identical(b, n, k):
     rng = np.random.default_rng(b * 1000003 + n * 101 + k + 1)
     w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
