@@ -193,6 +193,10 @@ __global__ __launch_bounds__(kSplitkThreads) void qgemm_q4g128_splitk_kernel(
                 for (int e = 0; e < 4; ++e)
                     ysum[bt][e] = fmaf(sf, fmaf(-off, xsum[e], acc[bt][e]), ysum[bt][e]);
             }
+            // pin the running sums here: otherwise the compiler sinks every group's update to
+            // the store and keeps all their accumulators alive
+#pragma unroll
+            for (int bt = 0; bt < BT; ++bt) asm volatile("" : "+v"(ysum[bt]));
             // one group at a time: without this the scheduler hoists the LDS reads of
             // every group (GP*4*BT operands of four registers) and spills
             __builtin_amdgcn_sched_barrier(0);

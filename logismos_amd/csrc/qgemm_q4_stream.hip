@@ -134,6 +134,10 @@ __global__ __launch_bounds__(64 * kStreamWaves) void qgemm_q4g128_stream_kernel(
                 for (int e = 0; e < 4; ++e)
                     ysum[bt][e] = fmaf(sf, fmaf(-off, xsum[e], acc[bt][e]), ysum[bt][e]);
             }
+            // pin the running sums here: otherwise the compiler sinks every group's update to
+            // the store and keeps all their accumulators alive
+#pragma unroll
+            for (int bt = 0; bt < BT; ++bt) asm volatile("" : "+v"(ysum[bt]));
             // one group at a time: keeps the LDS operand reads from being hoisted (and spilled)
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -164,18 +168,18 @@ __global__ __launch_bounds__(64 * kStreamWaves) void qgemm_q4g128_stream_kernel(
     }
 }
 
-// Steps (tiles per wave) a worker takes, 0 when the streaming kernel does not apply.
+// Steps (tiles per wave) a worker takes, 0 when the streaming kernel does not apply.  One
+// workgroup per CU: spreading the same tiles over two (which fit) measured slower, the
+// second copy of the x part costing more than the extra waves gain.
 int stream_steps(int b, int n, int k) {
     const int groups = k / 128;
     if (b < 3 || groups % kStreamGP != 0) return 0;
     const int tiles = (n + 15) / 16;
     const int parts = groups / kStreamGP;
     const int cus = device_cu_count();
-    // wave tiles per CU if spread evenly; below two steps of eight waves the split-K
-    // kernel's finer workgroups do as well
-    const long per_cu = (long)tiles * parts / cus;
-    if (per_cu < 2 * kStreamWaves / 2 + 2) return 0;
-    // largest worker count that fits one workgroup per CU, in whole steps
+    // wave tiles per CU if spread evenly; with fewer than ten the split-K kernel's finer
+    // workgroups do as well
+    if ((long)tiles * parts / cus < 10) return 0;
     int steps = 1;
     while ((long)((tiles + steps * kStreamWaves - 1) / (steps * kStreamWaves)) * parts > cus) ++steps;
     return steps;

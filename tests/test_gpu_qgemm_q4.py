@@ -143,12 +143,10 @@ def test_splitk_ragged_shapes(b, n, k):
     assert_parity(got, want, max_abs=2e-4, max_rel=1e-3, what=f"split-K {b}x{n}x{k} (J={j})")
 
 
-@pytest.mark.parametrize("b,n,k", [(32, 6144, 4096), (32, 4096, 12288), (5, 16, 128),
-                                   (17, 33, 384), (16, 1000, 1152), (31, 4100, 2048),
-                                   # shapes the streaming kernel takes: whole and ragged row
-                                   # tiles, one and two batch tiles, one to twelve K parts
-                                   (32, 24576, 4096), (16, 24576, 4096), (32, 24570, 2048),
-                                   (7, 45003, 1024), (3, 12288, 4096)])
+@pytest.mark.parametrize("b,n,k", [(32, 6144, 4096), (5, 16, 128), (17, 33, 384),
+                                   (16, 1000, 1152), (31, 4100, 2048),
+                                   # streaming kernel, one batch tile (same MFMA shape)
+                                   (16, 24576, 4096), (7, 45003, 1024), (3, 12288, 4096)])
 def test_splitk_with_prepared_x_is_bit_identical(b, n, k):
     rng = np.random.default_rng(b * 1000003 + n * 101 + k + 1)
     w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
@@ -158,3 +156,19 @@ def test_splitk_with_prepared_x_is_bit_identical(b, n, k):
     prep, _, _ = _run_splitk(x, qw, s, z, b, n, k, prepared=True)
     assert np.array_equal(plain, prep)
     assert_parity(prep, want, max_abs=2e-4, max_rel=1e-3, what="split-K, prepared x")
+
+
+@pytest.mark.parametrize("b,n,k", [(32, 24576, 4096), (32, 4096, 12288), (32, 24570, 2048),
+                                   (17, 45003, 1024), (25, 12288, 4096)])
+def test_streaming_kernel_with_two_batch_tiles(b, n, k):
+    # batch 17..32 on the large shapes: against the oracle and the plain-x path, whole and
+    # ragged row tiles, one to twelve K parts
+    rng = np.random.default_rng(b * 1000003 + n * 101 + k + 2)
+    w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
+    x = rng.standard_normal((b, k), np.float32)
+    qw, s, z = O.quantize_q4g128(w, n, k)
+    plain, want, _ = _run_splitk(x, qw, s, z, b, n, k)
+    prep, _, j = _run_splitk(x, qw, s, z, b, n, k, prepared=True)
+    assert j == k // 1024
+    assert_parity(prep, want, max_abs=2e-4, max_rel=1e-3, what="streaming kernel vs oracle")
+    assert_parity(prep, plain, max_abs=5e-5, max_rel=1e-4, what="streaming vs split-K kernel")
