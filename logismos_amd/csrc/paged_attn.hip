@@ -904,12 +904,24 @@ static void launch_prefill(const AttnParams& p, int max_seqlen_q, hipStream_t st
     paged_attn_prefill_kernel<G><<<grid, dim3(64 * kPfWaves), 0, stream>>>(p);
 }
 
+// Small batches stay on the static split: when every partition of every sequence is
+// resident at once there is no second round to balance away, and the balanced kernel's
+// prologue (prefix table, search) costs more than it saves (config 2: 12.7 vs 18 us).
+// The bound is on what the block tables could hold, the only size the host knows.
+static bool small_decode_batch(int num_seqs, int num_kv_heads, int block_size,
+                               int max_blocks_per_seq) {
+    return (int64_t)num_seqs * num_kv_heads * block_size * max_blocks_per_seq <= 200000;
+}
+
 // Workers of the balanced decode kernel: eight waves per CU (one wave = one KV head of one
 // worker), limited by the workspace the caller sized for num_splits partials per sequence
-// (slots used: at most workers + num_seqs - 1).  0: static split (one partition, or more
-// sequences than the prefix table holds).
-static int balanced_workers(int num_seqs, int num_kv_heads, int num_splits) {
-    if (num_splits <= 1 || num_seqs > kMaxBalancedSeqs) return 0;
+// (slots used: at most workers + num_seqs - 1).  0: static split (one partition, a small
+// batch, or more sequences than the prefix table holds).
+static int balanced_workers(int num_seqs, int num_kv_heads, int block_size, int max_blocks_per_seq,
+                            int num_splits) {
+    if (num_splits <= 1 || num_seqs > kMaxBalancedSeqs ||
+        small_decode_batch(num_seqs, num_kv_heads, block_size, max_blocks_per_seq))
+        return 0;
     int64_t target = (int64_t)device_cu_count() * kMaxHeadWaves / num_kv_heads;
     if (target < 1) target = 1;
     const int64_t cap = (int64_t)num_seqs * (num_splits - 1);
@@ -1005,7 +1017,8 @@ extern "C" logismos_status_t logismos_check_paged_attn_shape(int num_seqs, int t
 extern "C" int logismos_paged_attn_num_splits(int num_seqs, int num_kv_heads, int block_size,
                                               int max_blocks_per_seq) {
     if (num_seqs <= 0 || num_kv_heads <= 0 || block_size <= 0 || max_blocks_per_seq <= 0) return 1;
-    if (num_seqs <= lg::kMaxBalancedSeqs) {
+    if (num_seqs <= lg::kMaxBalancedSeqs &&
+        !lg::small_decode_batch(num_seqs, num_kv_heads, block_size, max_blocks_per_seq)) {
         // balanced decode: enough partial slots for one worker per CU's worth of waves
         int64_t target = (int64_t)lg::device_cu_count() * lg::kMaxHeadWaves / num_kv_heads;
         if (target < 1) target = 1;
@@ -1093,7 +1106,8 @@ logismos_status_t lg::paged_attn_launch(
     p.max_blocks_per_seq = max_blocks_per_seq;
     p.num_splits = num_splits;
     p.part_tokens = lg::part_tokens_for(block_size, max_blocks_per_seq, num_splits);
-    p.num_workers = lg::balanced_workers(num_seqs, num_kv_heads, num_splits);
+    p.num_workers =
+        lg::balanced_workers(num_seqs, num_kv_heads, block_size, max_blocks_per_seq, num_splits);
     p.scale_log2e = scale * lg::kLog2e;
     p.causal = causal;
     p.out_bf16 = out_bf16;

@@ -171,6 +171,36 @@ def test_config4_prefill_rows_agree_with_decode_rows_at_full_size():
     assert_parity(rows_dec, want_dec, what="config 4 decode rows vs oracle")
 
 
+@pytest.mark.parametrize("hq,hkv", [(1, 1), (4, 2), (12, 2), (12, 4), (32, 8), (8, 1), (16, 16),
+                                    (14, 2)])
+def test_balanced_decode_kernel_gqa_group_sizes(hq, hkv):
+    # wide block tables put even a small batch on the balanced decode kernel (one stream of
+    # key tiles split evenly over the workers): ragged contexts around the tile and worker
+    # edges, rows with one visible key, a zero-context row, prefill rows in between
+    rng = np.random.default_rng(60 + hq + hkv)
+    new = [1, 1, 1, 9, 1, 1, 1, 0, 1, 1]
+    prior = [0, 15, 16, 40, 127, 128, 1000, 5, 2047, 333]
+    c = workloads.paged_case(rng, new, prior, hq=hq, hkv=hkv, min_max_blocks=8192)
+    c["context_lens"][9] = 0
+    for ns in (2, 5, 64):
+        _check(c, num_splits=ns, what=f"balanced {hq}/{hkv} splits {ns}")
+    r = PagedAttnRunner(c)
+    r.launch()
+    got = r.result()
+    t = int(c["cu_seqlens"][9])
+    assert (got[t] == 0).all()
+
+
+def test_balanced_decode_kernel_many_short_sequences():
+    # more sequences than workers' worth of tiles: most workers cross several sequences
+    rng = np.random.default_rng(61)
+    n = 300
+    prior = rng.integers(0, 40, size=n)
+    c = workloads.paged_case(rng, np.ones(n, np.int32), prior, hq=8, hkv=2, min_max_blocks=512)
+    _check(c, what="300 short sequences")
+    _check(c, num_splits=2, what="300 short sequences, 2 splits")
+
+
 def test_zero_context_and_empty_sequences():
     rng = np.random.default_rng(5)
     c = workloads.paged_case(rng, [1, 0, 1, 3], [0, 5, 40, 0], hq=4, hkv=2)

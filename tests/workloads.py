@@ -13,18 +13,19 @@ SEED = 0x10615
 
 
 def paged_case(rng, new_tokens, prior_ctx, hq, hkv, d=128, block_size=16, spare_frac=0.25,
-               kv_std=1.0, pool_period_rows=None):
+               kv_std=1.0, pool_period_rows=None, min_max_blocks=1):
     """Ragged paged-attention inputs: pools shared by all sequences, physical
     block ids a random permutation, block-table tail entries poisoned.  With
     pool_period_rows the pools repeat that many random rows (full-size cases whose
-    pools would take minutes to draw)."""
+    pools would take minutes to draw); min_max_blocks widens the block tables (the launch
+    heuristics size their work by what the tables could hold)."""
     new = np.asarray(new_tokens, np.int32)
     prior = np.asarray(prior_ctx, np.int32)
     ctx = (new + prior).astype(np.int32)
     nblk = [(int(c) + block_size - 1) // block_size for c in ctx]
     total_blocks = sum(nblk) + max(1, int(sum(nblk) * spare_frac))
     perm = rng.permutation(total_blocks).astype(np.int32)
-    max_blocks = max(max(nblk), 1)
+    max_blocks = max(max(nblk), min_max_blocks, 1)
     bt = np.full((len(new), max_blocks), 0x3FFFFFF, np.int32)
     o = 0
     for s, nb in enumerate(nblk):
