@@ -209,8 +209,15 @@ size_t logismos_paged_attn_workspace_bytes(int num_seqs, int num_q_heads, int he
  *   total_tokens    cu_seqlens_q[num_seqs]; max_seqlen_q: the largest number of
  *                   new tokens of any sequence (both known to the host-side
  *                   scheduler; 1 for a pure decode step)
- *   num_splits      KV partitions per decode sequence (>= 1), e.g. from
- *                   `logismos_paged_attn_num_splits`
+ *   num_splits      partial results the workspace can hold per decode sequence
+ *                   (>= 1), e.g. from `logismos_paged_attn_num_splits`.  1: every
+ *                   sequence is one partition.  Small batches: each context is
+ *                   cut into num_splits static partitions.  Otherwise the key
+ *                   tiles of all decode sequences are split evenly over one
+ *                   worker per CU (at most num_seqs*(num_splits-1) workers), so
+ *                   the work per CU does not depend on how the context lengths
+ *                   are distributed; the result does not depend on num_splits
+ *                   beyond fp32 summation order
  *   workspace       `logismos_paged_attn_workspace_bytes(...)` bytes, contents
  *                   don't matter on entry; must not be shared by launches that
  *                   can overlap in time
