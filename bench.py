@@ -346,6 +346,21 @@ def bench_q4(args):
         out[f"b{b}"] = {"us": round(ms * 1e3, 2), "GBps": round(algo / ms / 1e6, 1),
                         "kernel": "gemv" if b <= 2 else "mfma"}
         del r, qws
+    # the same matrix size as ggml Q4_0 weights through the Q4G32 GEMV (x fp32, batch 1)
+    qw32 = hip.DeviceBuffer.from_numpy(qw)
+    sc32 = hip.DeviceBuffer.from_numpy(
+        (rng.random((n, k // 32), np.float32) * 0.004 + 0.004).astype(np.float16))
+    mn32 = hip.DeviceBuffer.from_numpy(
+        (rng.random((n, k // 32), np.float32) * -0.06).astype(np.float16))
+    x32 = hip.DeviceBuffer.from_numpy(rng.standard_normal(k, np.float32))
+    y32 = hip.DeviceBuffer(n * 4)
+    qws = replicate(qw32, max(2, -(-COLD_BYTES // qw.nbytes)))
+    algo32 = n * k // 2 + n * (k // 32) * 4 + 4 * k + 4 * n
+    ms, _, _ = time_launches(
+        stream, [(lambda q=q: kernels.launch_qgemv_q4g32_f32(x32, q, sc32, mn32, y32, n, k, stream))
+                 for q in qws], args.steps, args.warmup)
+    out["q4g32_b1"] = {"us": round(ms * 1e3, 2), "GBps": round(algo32 / ms / 1e6, 1),
+                       "kernel": "qgemv_q4g32 (ggml Q4_0/Q4_1 arithmetic, x fp32)"}
     return {"workload": "config 3: Q4G128 GEMV/GEMM 12288x4096, x bf16, cold weights", **out}
 
 

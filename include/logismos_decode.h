@@ -82,6 +82,17 @@ typedef uint32_t logismos_status_t;
  * `logismos_launch_repack_q8_0` converts ggml's 34-byte
  * `{f16 d; int8 qs[32]}` blocks into it.
  *
+ * Q4G32 weights (4-bit, group 32 along K: the arithmetic of ggml Q4_1, type id
+ * 3, and of Q4_0, id 2, in crates/loader/src/gguf.rs:57-78).  Planar: `qw`
+ * uint8 `[N][K/2]`, element k in the low (k even) or high (k odd) nibble of
+ * byte k/2 (the nibble order of `pack_turbo4_indices`,
+ * crates/quant/src/lib.rs:272-285); `scale` fp16 `[N][K/32]`, `min` fp16
+ * `[N][K/32]`; w[n][k] = q * scale + min.  `logismos_launch_repack_q4_1`
+ * converts ggml's 20-byte `{f16 d; f16 m; u8 qs[16]}` blocks (scale = d,
+ * min = m) and `logismos_launch_repack_q4_0` its 18-byte `{f16 d; u8 qs[16]}`
+ * blocks (scale = d, min = -8 d, so that q*d + min = (q - 8)*d); ggml keeps
+ * value j in the low and value j + 16 in the high nibble of byte j.
+ *
  * Q4G128 weights (4-bit asymmetric, group 128 along K).  `qw` uint8
  * `[N][K/2]`, element 2j in the low nibble of byte j and 2j+1 in the high
  * nibble (index i at bit 4*i of a little-endian integer, the reference's
@@ -178,6 +189,24 @@ logismos_status_t logismos_launch_q4_prepare_x_bf16(const void* x_bf16, void* x_
 logismos_status_t logismos_launch_qgemm_q4g128_f32_splitk_xprep(
     const void* x_prepared, const void* qw_u8, const void* scale_f16, const void* zero_f16,
     void* parts_f32, int b, int n, int k, logismos_stream_t stream);
+
+/* y[n] = sum_k x[k] * (q[n][k] * scale[n][k/32] + min[n][k/32]): `linear_t` at m = 1
+ * (crates/kernels/src/cpu_f32/mod.rs:271-345) over Q4G32 weights; x, y fp32;
+ * K % 32 == 0, N*K <= i32::MAX; qw and x 16-byte aligned. */
+logismos_status_t logismos_check_qgemv_q4g32_shape(int n, int k, char* msg, size_t msg_cap);
+logismos_status_t logismos_launch_qgemv_q4g32_f32(const void* x_f32, const void* qw_u8,
+                                                  const void* scale_f16, const void* min_f16,
+                                                  void* y_f32, int n, int k,
+                                                  logismos_stream_t stream);
+
+/* ggml Q4_0 / Q4_1 block streams `[N][K/32]` (the tensors the loader rejects today,
+ * crates/loader/src/gguf.rs:127-145,397-406) -> planar Q4G32.  blocks 2-byte aligned. */
+logismos_status_t logismos_launch_repack_q4_0(const void* blocks_q4_0, void* qw_u8,
+                                              void* scale_f16, void* min_f16, int n, int k,
+                                              logismos_stream_t stream);
+logismos_status_t logismos_launch_repack_q4_1(const void* blocks_q4_1, void* qw_u8,
+                                              void* scale_f16, void* min_f16, int n, int k,
+                                              logismos_stream_t stream);
 
 /* ggml Q8_0 block stream `[N][K/32]{f16 d; int8 qs[32]}` -> planar Q8G32. */
 logismos_status_t logismos_launch_repack_q8_0(const void* blocks_q8_0, void* qs_i8, void* d_f16,

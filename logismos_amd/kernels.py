@@ -51,6 +51,10 @@ _SIGNATURES = {
     "logismos_launch_qgemm_q4g128_bf16": (C.c_uint32, [_vp] * 5 + [_i, _i, _i, _vp]),
     "logismos_launch_qgemm_q4g128_bf16_mfma": (C.c_uint32, [_vp] * 5 + [_i, _i, _i, _vp]),
     "logismos_launch_repack_q8_0": (C.c_uint32, [_vp, _vp, _vp, _i, _i, _vp]),
+    "logismos_check_qgemv_q4g32_shape": (C.c_uint32, [_i, _i, C.c_char_p, _sz]),
+    "logismos_launch_qgemv_q4g32_f32": (C.c_uint32, [_vp] * 5 + [_i, _i, _vp]),
+    "logismos_launch_repack_q4_0": (C.c_uint32, [_vp] * 4 + [_i, _i, _vp]),
+    "logismos_launch_repack_q4_1": (C.c_uint32, [_vp] * 4 + [_i, _i, _vp]),
     "logismos_paged_attn_num_splits": (C.c_int, [_i, _i, _i, _i]),
     "logismos_paged_attn_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "logismos_launch_paged_attn_varlen_fp16":
@@ -168,6 +172,26 @@ def _guard(kernel: str, check_fn, *dims) -> None:
 def _status(kernel: str, code: int) -> None:
     if code != 0:
         raise LaunchError(kernel, code)
+
+
+def check_qgemv_q4g32_shape(n: int, k: int) -> None:
+    _guard("qgemv_q4g32_f32", library().logismos_check_qgemv_q4g32_shape, n, k)
+
+
+def launch_qgemv_q4g32_f32(x, qw, scale, minv, y, n: int, k: int, stream=None) -> None:
+    check_qgemv_q4g32_shape(n, k)
+    _status("qgemv_q4g32_f32", library().logismos_launch_qgemv_q4g32_f32(
+        _ptr(x), _ptr(qw), _ptr(scale), _ptr(minv), _ptr(y), n, k, _raw(stream)))
+
+
+def launch_repack_q4_blocks(blocks, qw, scale, minv, n: int, k: int, has_min: bool,
+                            stream=None) -> None:
+    """ggml Q4_1 (has_min) or Q4_0 block stream -> planar Q4G32."""
+    check_qgemv_q4g32_shape(n, k)
+    fn = (library().logismos_launch_repack_q4_1 if has_min
+          else library().logismos_launch_repack_q4_0)
+    _status("repack_q4_1" if has_min else "repack_q4_0",
+            fn(_ptr(blocks), _ptr(qw), _ptr(scale), _ptr(minv), n, k, _raw(stream)))
 
 
 def check_qgemv_q8g32_shape(n: int, k: int) -> None:

@@ -293,6 +293,58 @@ def unpack_nibbles(packed, n):
     return out
 
 
+_quant_q4_0 = _sig("oracle_quantize_q4_0_blocks", None, _vp, _vp, _sz, _sz)
+_quant_q4_1 = _sig("oracle_quantize_q4_1_blocks", None, _vp, _vp, _sz, _sz)
+_dequant_q4_0 = _sig("oracle_dequantize_q4_0_blocks", None, _vp, _vp, _sz, _sz)
+_dequant_q4_1 = _sig("oracle_dequantize_q4_1_blocks", None, _vp, _vp, _sz, _sz)
+_q4_blocks_to_planar = _sig("oracle_q4_blocks_to_q4g32", None, _vp, C.c_int, _vp, _vp, _vp, _sz,
+                            _sz)
+_dequant_q4g32 = _sig("oracle_dequantize_q4g32", None, _vp, _vp, _vp, _vp, _sz, _sz)
+_qgemv_q4g32 = _sig("oracle_qgemv_q4g32_f32", None, _vp, _vp, _vp, _vp, _vp, _sz, _sz)
+
+
+def quantize_q4_blocks(w, n, k, has_min):
+    """ggml Q4_0 (has_min False, 18-byte blocks) or Q4_1 (True, 20-byte blocks) stream."""
+    w = _f32(w)
+    assert w.size == n * k and k % 32 == 0
+    blocks = np.empty(n * (k // 32) * (20 if has_min else 18), np.uint8)
+    (_quant_q4_1 if has_min else _quant_q4_0)(_p(w), _p(blocks), n, k)
+    return blocks
+
+
+def dequantize_q4_blocks(blocks, n, k, has_min):
+    blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+    w = np.empty((n, k), np.float32)
+    (_dequant_q4_1 if has_min else _dequant_q4_0)(_p(blocks), _p(w), n, k)
+    return w
+
+
+def q4_blocks_to_q4g32(blocks, n, k, has_min):
+    blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+    qw = np.empty((n, k // 2), np.uint8)
+    scale = np.empty((n, k // 32), np.uint16)
+    minv = np.empty((n, k // 32), np.uint16)
+    _q4_blocks_to_planar(_p(blocks), 1 if has_min else 0, _p(qw), _p(scale), _p(minv), n, k)
+    return qw, scale.view(np.float16), minv.view(np.float16)
+
+
+def dequantize_q4g32(qw, scale, minv, n, k):
+    qw = np.ascontiguousarray(qw, dtype=np.uint8)
+    scale, minv = _u16(scale), _u16(minv)
+    w = np.empty((n, k), np.float32)
+    _dequant_q4g32(_p(qw), _p(scale), _p(minv), _p(w), n, k)
+    return w
+
+
+def qgemv_q4g32_f32(x, qw, scale, minv, n, k):
+    x = _f32(x)
+    qw = np.ascontiguousarray(qw, dtype=np.uint8)
+    scale, minv = _u16(scale), _u16(minv)
+    y = np.empty(n, np.float32)
+    _qgemv_q4g32(_p(x), _p(qw), _p(scale), _p(minv), _p(y), n, k)
+    return y
+
+
 def quantize_q8g32(w, n, k):
     w = _f32(w)
     assert w.size == n * k and k % 32 == 0

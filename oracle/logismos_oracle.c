@@ -447,6 +447,162 @@ void oracle_qgemv_q8g32_f32(const float* x, const int8_t* qs, const uint16_t* d,
     }
 }
 
+/* ------------------------------------------------- ggml Q4_0 / Q4_1 and Q4G32 */
+
+/* ggml's 4-bit block formats, the ids the reference parses and rejects (`GgmlType::Q4_0 = 2`,
+ * `Q4_1 = 3`, crates/loader/src/gguf.rs:57-78,127-145).  The reference holds neither the
+ * structs nor arithmetic for them and names no ggml version; what follows restates ggml's
+ * published definitions (ggml-common.h `block_q4_0` = {f16 d; u8 qs[16]}, 18 bytes, and
+ * `block_q4_1` = {f16 d; f16 m; u8 qs[16]}, 20 bytes, for 32 values; ggml-quants.c
+ * `quantize_row_q4_0_ref`, `quantize_row_q4_1_ref`, `dequantize_row_q4_0`,
+ * `dequantize_row_q4_1`): byte j of qs holds value j in its low nibble and value j + 16 in its
+ * high nibble; Q4_0: w = (q - 8) * d; Q4_1: w = q * d + m. */
+void oracle_quantize_q4_0_blocks(const float* w, uint8_t* blocks, size_t n, size_t k) {
+    size_t groups = k / 32;
+#pragma omp parallel for schedule(static)
+    for (long r = 0; r < (long)n; ++r)
+        for (size_t g = 0; g < groups; ++g) {
+            const float* src = w + (size_t)r * k + g * 32;
+            float amax = 0.0f, max = 0.0f; /* the value of largest magnitude, with its sign */
+            for (int i = 0; i < 32; ++i)
+                if (amax < fabsf(src[i])) {
+                    amax = fabsf(src[i]);
+                    max = src[i];
+                }
+            const float d = max / -8.0f;
+            const float id = d != 0.0f ? 1.0f / d : 0.0f;
+            uint8_t* blk = blocks + ((size_t)r * groups + g) * 18;
+            uint16_t dh = oracle_f32_to_f16(d);
+            blk[0] = (uint8_t)(dh & 0xff);
+            blk[1] = (uint8_t)(dh >> 8);
+            for (int j = 0; j < 16; ++j) {
+                const float x0 = src[j] * id, x1 = src[16 + j] * id;
+                int q0 = (int)(int8_t)(x0 + 8.5f), q1 = (int)(int8_t)(x1 + 8.5f);
+                if (q0 > 15) q0 = 15;
+                if (q1 > 15) q1 = 15;
+                blk[2 + j] = (uint8_t)(q0 | (q1 << 4));
+            }
+        }
+}
+
+void oracle_quantize_q4_1_blocks(const float* w, uint8_t* blocks, size_t n, size_t k) {
+    size_t groups = k / 32;
+#pragma omp parallel for schedule(static)
+    for (long r = 0; r < (long)n; ++r)
+        for (size_t g = 0; g < groups; ++g) {
+            const float* src = w + (size_t)r * k + g * 32;
+            float mn = src[0], mx = src[0];
+            for (int i = 1; i < 32; ++i) {
+                if (src[i] < mn) mn = src[i];
+                if (src[i] > mx) mx = src[i];
+            }
+            const float d = (mx - mn) / 15.0f;
+            const float id = d != 0.0f ? 1.0f / d : 0.0f;
+            uint8_t* blk = blocks + ((size_t)r * groups + g) * 20;
+            uint16_t dh = oracle_f32_to_f16(d), mh = oracle_f32_to_f16(mn);
+            blk[0] = (uint8_t)(dh & 0xff);
+            blk[1] = (uint8_t)(dh >> 8);
+            blk[2] = (uint8_t)(mh & 0xff);
+            blk[3] = (uint8_t)(mh >> 8);
+            for (int j = 0; j < 16; ++j) {
+                const float x0 = (src[j] - mn) * id, x1 = (src[16 + j] - mn) * id;
+                int q0 = (int)(int8_t)(x0 + 0.5f), q1 = (int)(int8_t)(x1 + 0.5f);
+                if (q0 > 15) q0 = 15;
+                if (q1 > 15) q1 = 15;
+                blk[4 + j] = (uint8_t)(q0 | (q1 << 4));
+            }
+        }
+}
+
+void oracle_dequantize_q4_0_blocks(const uint8_t* blocks, float* w, size_t n, size_t k) {
+    size_t groups = k / 32;
+    for (size_t r = 0; r < n; ++r)
+        for (size_t g = 0; g < groups; ++g) {
+            const uint8_t* blk = blocks + (r * groups + g) * 18;
+            const float d = oracle_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+            float* dst = w + r * k + g * 32;
+            for (int j = 0; j < 16; ++j) {
+                dst[j] = (float)((int)(blk[2 + j] & 0x0F) - 8) * d;
+                dst[j + 16] = (float)((int)(blk[2 + j] >> 4) - 8) * d;
+            }
+        }
+}
+
+void oracle_dequantize_q4_1_blocks(const uint8_t* blocks, float* w, size_t n, size_t k) {
+    size_t groups = k / 32;
+    for (size_t r = 0; r < n; ++r)
+        for (size_t g = 0; g < groups; ++g) {
+            const uint8_t* blk = blocks + (r * groups + g) * 20;
+            const float d = oracle_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+            const float m = oracle_f16_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
+            float* dst = w + r * k + g * 32;
+            for (int j = 0; j < 16; ++j) {
+                dst[j] = (float)(blk[4 + j] & 0x0F) * d + m;
+                dst[j + 16] = (float)(blk[4 + j] >> 4) * d + m;
+            }
+        }
+}
+
+/* Planar Q4G32 [DEFINED BY BUILD], what the GPU GEMV reads: nibbles uint8 [N][K/2] in k
+ * order, low nibble first (the reference's only nibble order, `pack_turbo4_indices`,
+ * crates/quant/src/lib.rs:272-285), fp16 scale [N][K/32], fp16 min [N][K/32];
+ * w = q * scale + min.  Q4_1 maps onto it unchanged (scale = d, min = m); Q4_0 with
+ * scale = d and min = -8 * d, which is exact in fp16 short of overflow, and then
+ * q * d + (-8 d) differs from (q - 8) * d by at most one fp32 rounding. */
+void oracle_q4_blocks_to_q4g32(const uint8_t* blocks, int has_min, uint8_t* qw, uint16_t* scale,
+                               uint16_t* minv, size_t n, size_t k) {
+    size_t groups = k / 32;
+    const size_t bsz = has_min ? 20 : 18;
+    for (size_t r = 0; r < n; ++r)
+        for (size_t g = 0; g < groups; ++g) {
+            const uint8_t* blk = blocks + (r * groups + g) * bsz;
+            const uint16_t dh = (uint16_t)(blk[0] | (blk[1] << 8));
+            scale[r * groups + g] = dh;
+            minv[r * groups + g] = has_min ? (uint16_t)(blk[2] | (blk[3] << 8))
+                                           : oracle_f32_to_f16(-8.0f * oracle_f16_to_f32(dh));
+            const uint8_t* qs = blk + (has_min ? 4 : 2);
+            uint8_t* dst = qw + r * (k / 2) + g * 16;
+            for (int t = 0; t < 8; ++t) {
+                dst[t] = (uint8_t)((qs[2 * t] & 0x0F) | ((qs[2 * t + 1] & 0x0F) << 4));
+                dst[8 + t] = (uint8_t)((qs[2 * t] >> 4) | ((qs[2 * t + 1] >> 4) << 4));
+            }
+        }
+}
+
+void oracle_dequantize_q4g32(const uint8_t* qw, const uint16_t* scale, const uint16_t* minv,
+                             float* w, size_t n, size_t k) {
+    size_t groups = k / 32;
+    for (size_t r = 0; r < n; ++r)
+        for (size_t c = 0; c < k; ++c) {
+            const uint8_t byte = qw[r * (k / 2) + c / 2];
+            const float q = (float)((c & 1) ? (byte >> 4) : (byte & 0x0F));
+            w[r * k + c] = q * oracle_f16_to_f32(scale[r * groups + c / 32]) +
+                           oracle_f16_to_f32(minv[r * groups + c / 32]);
+        }
+}
+
+/* linear_t at m = 1 (crates/kernels/src/cpu_f32/mod.rs:271-345) over the dequantised
+ * matrix, ascending k, fp32. */
+void oracle_qgemv_q4g32_f32(const float* x, const uint8_t* qw, const uint16_t* scale,
+                            const uint16_t* minv, float* y, size_t n, size_t k) {
+    size_t groups = k / 32;
+#pragma omp parallel for schedule(static)
+    for (long r = 0; r < (long)n; ++r) {
+        float acc = 0.0f;
+        for (size_t g = 0; g < groups; ++g) {
+            const float s = oracle_f16_to_f32(scale[(size_t)r * groups + g]);
+            const float m = oracle_f16_to_f32(minv[(size_t)r * groups + g]);
+            for (int i = 0; i < 32; ++i) {
+                const size_t c = g * 32 + i;
+                const uint8_t byte = qw[(size_t)r * (k / 2) + c / 2];
+                const float q = (float)((c & 1) ? (byte >> 4) : (byte & 0x0F));
+                acc += x[c] * (q * s + m);
+            }
+        }
+        y[r] = acc;
+    }
+}
+
 /* ------------------------------------------------------------------ Q4G128 */
 
 /* 4-bit asymmetric, group 128: scale = (max-min)/15, zero = -min/scale, both

@@ -93,6 +93,18 @@ void oracle_q8_0_blocks_to_q8g32(const uint8_t* blocks, int8_t* qs, uint16_t* d,
 void oracle_qgemv_q8g32_f32(const float* x, const int8_t* qs, const uint16_t* d, float* y,
                             size_t n, size_t k);
 
+/* ---- ggml Q4_0 / Q4_1 blocks (18 / 20 bytes per 32 values) and planar Q4G32 */
+void oracle_quantize_q4_0_blocks(const float* w, uint8_t* blocks, size_t n, size_t k);
+void oracle_quantize_q4_1_blocks(const float* w, uint8_t* blocks, size_t n, size_t k);
+void oracle_dequantize_q4_0_blocks(const uint8_t* blocks, float* w, size_t n, size_t k);
+void oracle_dequantize_q4_1_blocks(const uint8_t* blocks, float* w, size_t n, size_t k);
+void oracle_q4_blocks_to_q4g32(const uint8_t* blocks, int has_min, uint8_t* qw, uint16_t* scale,
+                               uint16_t* minv, size_t n, size_t k);
+void oracle_dequantize_q4g32(const uint8_t* qw, const uint16_t* scale, const uint16_t* minv,
+                             float* w, size_t n, size_t k);
+void oracle_qgemv_q4g32_f32(const float* x, const uint8_t* qw, const uint16_t* scale,
+                            const uint16_t* minv, float* y, size_t n, size_t k);
+
 /* ---- Q4G128 */
 void oracle_quantize_q4g128(const float* w, uint8_t* qw, uint16_t* scale, uint16_t* zero, size_t n,
                             size_t k);
