@@ -486,6 +486,102 @@ def paged_attn_varlen_fp16(q, k_pool, v_pool, block_tables, cu_seqlens_q, contex
     return out if f32_out else out.view(np.float16)
 
 
+# ---------------------------------------------------------------- TurboQuant 3-bit KV
+_t3_codebook = _sig("oracle_turbo3_codebook", None, _vp)
+_fwht = _sig("oracle_fwht_128", None, _vp)
+_t3_pack = _sig("oracle_pack_turbo3_indices", C.c_int, _vp, _vp)
+_t3_unpack = _sig("oracle_unpack_turbo3_indices", None, _vp, _vp)
+_t3_encode = _sig("oracle_encode_turbo3_0_head", None, _vp, _vp)
+_t3_decode = _sig("oracle_decode_turbo3_0_head", None, _vp, _vp)
+_t3_kv_write = _sig("oracle_kv_write_turbo3", None, _vp, _vp, _vp, _vp, _vp, _sz, _sz)
+_t3_gather = _sig("oracle_paged_gather_turbo3", None, _vp, _vp, _sz, _sz, _sz, _vp)
+_t3_attn = _sig("oracle_paged_attn_varlen_turbo3", None, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz,
+                _sz, _sz, _sz, _sz, C.c_float, C.c_int)
+TURBO3_BYTES_PER_HEAD = 56
+
+
+def turbo3_codebook():
+    out = np.empty(8, np.float32)
+    _t3_codebook(_p(out))
+    return out
+
+
+def fwht_128(data):
+    d = _f32(data).copy()
+    assert d.size == 128
+    _fwht(_p(d))
+    return d
+
+
+def pack_turbo3_indices(idx):
+    idx = np.ascontiguousarray(idx, dtype=np.uint8)
+    assert idx.size == 32
+    out = np.empty(12, np.uint8)
+    pos = _t3_pack(_p(idx), _p(out))
+    if pos >= 0:
+        raise ValueError(f"turbo3 index out of range at position {pos}: {int(idx[pos])} > 7")
+    return out
+
+
+def unpack_turbo3_indices(packed):
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    assert packed.size == 12
+    out = np.empty(32, np.uint8)
+    _t3_unpack(_p(packed), _p(out))
+    return out
+
+
+def encode_turbo3_0_head(values):
+    v = _f32(values)
+    if v.size != 128:
+        raise ValueError(f"invalid head dim: got {v.size}, expected 128")
+    out = np.empty(56, np.uint8)
+    _t3_encode(_p(v), _p(out))
+    return out
+
+
+def decode_turbo3_0_head(blocks):
+    b = np.ascontiguousarray(blocks, dtype=np.uint8)
+    if b.size != 56:
+        raise ValueError(f"invalid block count: got {b.size} bytes, expected 56")
+    out = np.empty(128, np.float32)
+    _t3_decode(_p(b), _p(out))
+    return out
+
+
+def kv_write_turbo3(k_new, v_new, k_pool, v_pool, slot_mapping, num_kv_heads):
+    """In place: k_pool / v_pool uint8 [rows][num_kv_heads*56]."""
+    k_new, v_new = _u16(k_new), _u16(v_new)
+    slots = np.ascontiguousarray(slot_mapping, dtype=np.int64)
+    assert k_pool.dtype == np.uint8 and k_pool.flags.c_contiguous
+    assert v_pool.dtype == np.uint8 and v_pool.flags.c_contiguous
+    _t3_kv_write(_p(k_new), _p(v_new), _p(k_pool), _p(v_pool), _p(slots), slots.size, num_kv_heads)
+
+
+def paged_gather_turbo3(pool, block_table_row, ctx, block_size, num_kv_heads):
+    pool = np.ascontiguousarray(pool, dtype=np.uint8)
+    bt = np.ascontiguousarray(block_table_row, dtype=np.int32)
+    out = np.empty((ctx, num_kv_heads * 128), np.float32)
+    _t3_gather(_p(pool), _p(bt), ctx, block_size, num_kv_heads, _p(out))
+    return out
+
+
+def paged_attn_varlen_turbo3(q, k_pool, v_pool, block_tables, cu_seqlens_q, context_lens,
+                             num_q_heads, num_kv_heads, block_size, scale, causal=True):
+    q = _u16(q)
+    k_pool = np.ascontiguousarray(k_pool, dtype=np.uint8)
+    v_pool = np.ascontiguousarray(v_pool, dtype=np.uint8)
+    block_tables = np.ascontiguousarray(block_tables, dtype=np.int32)
+    cu = np.ascontiguousarray(cu_seqlens_q, dtype=np.int32)
+    ctx = np.ascontiguousarray(context_lens, dtype=np.int32)
+    num_seqs = ctx.size
+    out = np.zeros(q.shape, np.uint16)
+    _t3_attn(_p(q), _p(k_pool), _p(v_pool), _p(block_tables), _p(cu), _p(ctx), _p(out), num_seqs,
+             num_q_heads, num_kv_heads, block_size, block_tables.shape[1] if num_seqs else 0,
+             scale, 1 if causal else 0)
+    return out.view(np.float16)
+
+
 # ---------------------------------------------------------------- metric / threads
 _metric = _sig("oracle_parity_metric_f32", None, _vp, _vp, _sz, C.POINTER(C.c_float),
                C.POINTER(C.c_float))

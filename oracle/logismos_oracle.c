@@ -767,6 +767,135 @@ void oracle_paged_gather_fp16(const uint16_t* pool, const int32_t* block_table_r
     }
 }
 
+/* ------------------------------------------------------------------ TurboQuant 3-bit KV */
+
+/* `TURBO3_CODEBOOK` (crates/quant/src/lib.rs:66-80): Lloyd-Max centroids, verbatim. */
+static const float kTurbo3Codebook[8] = {
+    -0.1883972972f, -0.1181399059f, -0.0665857641f, -0.0216044751f,
+    0.0216041461f,  0.0665854520f,  0.1181396281f,  0.1883970748f,
+};
+
+void oracle_turbo3_codebook(float* out8) { memcpy(out8, kTurbo3Codebook, sizeof kTurbo3Codebook); }
+
+/* `fwht_128` (crates/quant/src/lib.rs:88-113): butterflies h = 1, 2, .., 64 over chunks
+ * of 2h (lo += hi, hi = lo - hi), then every value times the f32 literal 1/sqrt(128). */
+void oracle_fwht_128(float* data) {
+    for (size_t h = 1; h < 128; h *= 2)
+        for (size_t c = 0; c < 128; c += 2 * h)
+            for (size_t i = 0; i < h; ++i) {
+                float x = data[c + i], y = data[c + h + i];
+                data[c + i] = x + y;
+                data[c + h + i] = x - y;
+            }
+    const float scale = 0.08838834764831844f;
+    for (size_t i = 0; i < 128; ++i) data[i] *= scale;
+}
+
+/* `nearest_centroid` (crates/quant/src/lib.rs:119-126): argmin |v - c| by total order,
+ * the first minimum wins (Iterator::min_by keeps the first of equal elements). */
+static uint8_t turbo3_nearest(float v) {
+    int best = 0;
+    float bd = fabsf(v - kTurbo3Codebook[0]);
+    for (int i = 1; i < 8; ++i) {
+        float d = fabsf(v - kTurbo3Codebook[i]);
+        /* total_cmp: a NaN distance (v NaN) compares greater than every number */
+        if (d < bd) {
+            bd = d;
+            best = i;
+        }
+    }
+    return (uint8_t)best;
+}
+
+/* `pack_turbo3_indices` / `unpack_turbo3_indices` (crates/quant/src/lib.rs:224-268):
+ * index i occupies bits [3i, 3i+3) of a little-endian 96-bit integer.  Returns the
+ * position of the first index > 7, or -1. */
+int oracle_pack_turbo3_indices(const uint8_t* idx32, uint8_t* packed12) {
+    memset(packed12, 0, 12);
+    for (int i = 0; i < 32; ++i) {
+        if (idx32[i] > 7) return i;
+        int bit = 3 * i;
+        packed12[bit >> 3] |= (uint8_t)(idx32[i] << (bit & 7));
+        if ((bit & 7) > 5) packed12[(bit >> 3) + 1] |= (uint8_t)(idx32[i] >> (8 - (bit & 7)));
+    }
+    return -1;
+}
+
+void oracle_unpack_turbo3_indices(const uint8_t* packed12, uint8_t* idx32) {
+    for (int i = 0; i < 32; ++i) {
+        int bit = 3 * i;
+        unsigned v = packed12[bit >> 3] >> (bit & 7);
+        if ((bit & 7) > 5) v |= (unsigned)packed12[(bit >> 3) + 1] << (8 - (bit & 7));
+        idx32[i] = (uint8_t)(v & 7u);
+    }
+}
+
+/* `encode_turbo3_0_head` (crates/quant/src/lib.rs:316-353): L2 norm (sequential fp32 sum
+ * of squares, sqrt), v / norm (zeros when norm <= 1e-12), FWHT, nearest centroid, pack; the
+ * fp16 norm is stored in each of the four 14-byte blocks {norm_f16_le[2], packed[12]}. */
+void oracle_encode_turbo3_0_head(const float* values128, uint8_t* out56) {
+    float sum_sq = 0.0f;
+    for (int i = 0; i < 128; ++i) sum_sq += values128[i] * values128[i];
+    const float norm = sqrtf(sum_sq);
+    const uint16_t nh = oracle_f32_to_f16(norm);
+    float t[128];
+    for (int i = 0; i < 128; ++i) t[i] = norm > 1e-12f ? values128[i] / norm : 0.0f;
+    oracle_fwht_128(t);
+    for (int b = 0; b < 4; ++b) {
+        uint8_t idx[32];
+        for (int i = 0; i < 32; ++i) idx[i] = turbo3_nearest(t[b * 32 + i]);
+        uint8_t* blk = out56 + 14 * b;
+        blk[0] = (uint8_t)(nh & 0xff);
+        blk[1] = (uint8_t)(nh >> 8);
+        oracle_pack_turbo3_indices(idx, blk + 2);
+    }
+}
+
+/* `decode_turbo3_0_head` (crates/quant/src/lib.rs:376-413): centroids, FWHT, times the
+ * norm of the FIRST block. */
+void oracle_decode_turbo3_0_head(const uint8_t* in56, float* values128) {
+    for (int b = 0; b < 4; ++b) {
+        uint8_t idx[32];
+        oracle_unpack_turbo3_indices(in56 + 14 * b + 2, idx);
+        for (int i = 0; i < 32; ++i) values128[b * 32 + i] = kTurbo3Codebook[idx[i]];
+    }
+    oracle_fwht_128(values128);
+    const float norm = oracle_f16_to_f32((uint16_t)(in56[0] | (in56[1] << 8)));
+    for (int i = 0; i < 128; ++i) values128[i] *= norm;
+}
+
+/* Paged turbo3 pools [DEFINED BY BUILD]: the fp16 pools with every 128-value head row
+ * replaced by its 56 encoded bytes: `[num_blocks][block_size][num_kv_heads][56]`, same
+ * block tables and slots.  Writing = `KvCache::put` of encoded rows: k_new / v_new fp16
+ * `[T][num_kv_heads][128]`, widened to f32 and encoded head by head. */
+void oracle_kv_write_turbo3(const uint16_t* k_new, const uint16_t* v_new, uint8_t* k_pool,
+                            uint8_t* v_pool, const int64_t* slot_mapping, size_t total_tokens,
+                            size_t num_kv_heads) {
+#pragma omp parallel for schedule(static)
+    for (long t = 0; t < (long)total_tokens; ++t) {
+        int64_t slot = slot_mapping[t];
+        if (slot < 0) continue;
+        for (size_t h = 0; h < num_kv_heads; ++h) {
+            float f[128];
+            oracle_f16_to_f32_n(k_new + ((size_t)t * num_kv_heads + h) * 128, f, 128);
+            oracle_encode_turbo3_0_head(f, k_pool + ((size_t)slot * num_kv_heads + h) * 56);
+            oracle_f16_to_f32_n(v_new + ((size_t)t * num_kv_heads + h) * 128, f, 128);
+            oracle_encode_turbo3_0_head(f, v_pool + ((size_t)slot * num_kv_heads + h) * 56);
+        }
+    }
+}
+
+/* First ctx rows of a sequence, decoded to f32 `[ctx][num_kv_heads*128]`. */
+void oracle_paged_gather_turbo3(const uint8_t* pool, const int32_t* block_table_row, size_t ctx,
+                                size_t block_size, size_t num_kv_heads, float* out) {
+    for (size_t j = 0; j < ctx; ++j) {
+        size_t slot = (size_t)block_table_row[j / block_size] * block_size + j % block_size;
+        for (size_t h = 0; h < num_kv_heads; ++h)
+            oracle_decode_turbo3_0_head(pool + (slot * num_kv_heads + h) * 56,
+                                        out + (j * num_kv_heads + h) * 128);
+    }
+}
+
 /* Ragged paged attention.  Per sequence: gather K/V (above), then for every
  * query token the SDPA arithmetic of crates/transformers/src/attention.rs:225-296
  * -- dot in fp32 (ascending d), times scale AFTER the dot, softmax_last_dim
@@ -774,14 +903,16 @@ void oracle_paged_gather_fp16(const uint16_t* pool, const int32_t* block_table_r
  * q head h -> kv head h / groups (:366-382).  Visible keys of query token i
  * (n new tokens, context c): causal ? [0, c-n+i] : [0, c).  No visible key =>
  * zeros (softmax_last_dim over n = 0 columns).  Output rounded to fp16 once. */
-static void paged_attn_core(const uint16_t* q, const uint16_t* k_pool, const uint16_t* v_pool,
-                            const int32_t* block_tables, const int32_t* cu_seqlens_q,
+static void paged_attn_core(const uint16_t* q, const void* k_pool_any, const void* v_pool_any,
+                            int turbo3, const int32_t* block_tables, const int32_t* cu_seqlens_q,
                             const int32_t* context_lens, uint16_t* out, float* out_f32,
                             size_t num_seqs, size_t num_q_heads, size_t num_kv_heads,
                             size_t head_dim, size_t block_size, size_t max_blocks_per_seq,
                             float scale, int causal) {
     size_t groups = num_q_heads / num_kv_heads;
     size_t row = num_kv_heads * head_dim;
+    const uint16_t* k_pool = (const uint16_t*)k_pool_any;
+    const uint16_t* v_pool = (const uint16_t*)v_pool_any;
 #pragma omp parallel for schedule(dynamic, 1)
     for (long s = 0; s < (long)num_seqs; ++s) {
         long ctx = context_lens[s];
@@ -798,10 +929,17 @@ static void paged_attn_core(const uint16_t* q, const uint16_t* k_pool, const uin
         float* qf = (float*)malloc(head_dim * sizeof(float));
         float* of = (float*)malloc(head_dim * sizeof(float));
         const int32_t* bt = block_tables + (size_t)s * max_blocks_per_seq;
-        oracle_paged_gather_fp16(k_pool, bt, ctxu, block_size, row, kh);
-        oracle_paged_gather_fp16(v_pool, bt, ctxu, block_size, row, vh);
-        oracle_f16_to_f32_n(kh, kf, ctxu * row);
-        oracle_f16_to_f32_n(vh, vf, ctxu * row);
+        if (turbo3) {
+            oracle_paged_gather_turbo3((const uint8_t*)k_pool_any, bt, ctxu, block_size,
+                                       num_kv_heads, kf);
+            oracle_paged_gather_turbo3((const uint8_t*)v_pool_any, bt, ctxu, block_size,
+                                       num_kv_heads, vf);
+        } else {
+            oracle_paged_gather_fp16(k_pool, bt, ctxu, block_size, row, kh);
+            oracle_paged_gather_fp16(v_pool, bt, ctxu, block_size, row, vh);
+            oracle_f16_to_f32_n(kh, kf, ctxu * row);
+            oracle_f16_to_f32_n(vh, vf, ctxu * row);
+        }
         for (long i = 0; i < n_new; ++i) {
             long vis = causal ? (ctx - n_new + i + 1) : ctx;
             if (vis < 0) vis = 0;
@@ -846,7 +984,7 @@ void oracle_paged_attn_varlen_fp16(const uint16_t* q, const uint16_t* k_pool,
                                    uint16_t* out, size_t num_seqs, size_t num_q_heads,
                                    size_t num_kv_heads, size_t head_dim, size_t block_size,
                                    size_t max_blocks_per_seq, float scale, int causal) {
-    paged_attn_core(q, k_pool, v_pool, block_tables, cu_seqlens_q, context_lens, out, NULL,
+    paged_attn_core(q, k_pool, v_pool, 0, block_tables, cu_seqlens_q, context_lens, out, NULL,
                     num_seqs, num_q_heads, num_kv_heads, head_dim, block_size, max_blocks_per_seq,
                     scale, causal);
 }
@@ -860,8 +998,22 @@ void oracle_paged_attn_varlen_fp16_f32out(const uint16_t* q, const uint16_t* k_p
                                           size_t num_seqs, size_t num_q_heads,
                                           size_t num_kv_heads, size_t head_dim, size_t block_size,
                                           size_t max_blocks_per_seq, float scale, int causal) {
-    paged_attn_core(q, k_pool, v_pool, block_tables, cu_seqlens_q, context_lens, NULL, out,
+    paged_attn_core(q, k_pool, v_pool, 0, block_tables, cu_seqlens_q, context_lens, NULL, out,
                     num_seqs, num_q_heads, num_kv_heads, head_dim, block_size, max_blocks_per_seq,
+                    scale, causal);
+}
+
+/* The same attention over turbo3 pools: every visible K / V head row is decoded with
+ * `decode_turbo3_0_head` (f32) and then used exactly as the widened fp16 rows are above;
+ * head_dim is 128. */
+void oracle_paged_attn_varlen_turbo3(const uint16_t* q, const uint8_t* k_pool,
+                                     const uint8_t* v_pool, const int32_t* block_tables,
+                                     const int32_t* cu_seqlens_q, const int32_t* context_lens,
+                                     uint16_t* out, size_t num_seqs, size_t num_q_heads,
+                                     size_t num_kv_heads, size_t block_size,
+                                     size_t max_blocks_per_seq, float scale, int causal) {
+    paged_attn_core(q, k_pool, v_pool, 1, block_tables, cu_seqlens_q, context_lens, out, NULL,
+                    num_seqs, num_q_heads, num_kv_heads, 128, block_size, max_blocks_per_seq,
                     scale, causal);
 }
 

@@ -142,6 +142,25 @@ void oracle_paged_attn_varlen_fp16_f32out(const uint16_t* q, const uint16_t* k_p
                                           size_t num_kv_heads, size_t head_dim, size_t block_size,
                                           size_t max_blocks_per_seq, float scale, int causal);
 
+/* ---- TurboQuant 3-bit KV codec (crates/quant/src/lib.rs) and attention over turbo3 pools */
+void oracle_turbo3_codebook(float* out8);
+void oracle_fwht_128(float* data);
+int oracle_pack_turbo3_indices(const uint8_t* idx32, uint8_t* packed12);
+void oracle_unpack_turbo3_indices(const uint8_t* packed12, uint8_t* idx32);
+void oracle_encode_turbo3_0_head(const float* values128, uint8_t* out56);
+void oracle_decode_turbo3_0_head(const uint8_t* in56, float* values128);
+void oracle_kv_write_turbo3(const uint16_t* k_new, const uint16_t* v_new, uint8_t* k_pool,
+                            uint8_t* v_pool, const int64_t* slot_mapping, size_t total_tokens,
+                            size_t num_kv_heads);
+void oracle_paged_gather_turbo3(const uint8_t* pool, const int32_t* block_table_row, size_t ctx,
+                                size_t block_size, size_t num_kv_heads, float* out);
+void oracle_paged_attn_varlen_turbo3(const uint16_t* q, const uint8_t* k_pool,
+                                     const uint8_t* v_pool, const int32_t* block_tables,
+                                     const int32_t* cu_seqlens_q, const int32_t* context_lens,
+                                     uint16_t* out, size_t num_seqs, size_t num_q_heads,
+                                     size_t num_kv_heads, size_t block_size,
+                                     size_t max_blocks_per_seq, float scale, int causal);
+
 /* ---- parity metric of the reference's GPU tests (crates/kernels/tests/matmul_parity.rs:83-99) */
 void oracle_parity_metric_f32(const float* got, const float* want, size_t n, float* max_abs,
                               float* max_rel);
