@@ -531,6 +531,34 @@ const int32_t* logismos_paged_kv_cache_block_tables(const logismos_paged_kv_cach
 const int32_t* logismos_paged_kv_cache_block_tables_host(const logismos_paged_kv_cache_t* cache);
 
 /* ------------------------------------------------------------------------
+ * TurboQuant 3-bit KV (`turbo3_0`, crates/quant/src/lib.rs)
+ * ------------------------------------------------------------------------
+ * turbo3 pools hold every 128-value head row as four 14-byte blocks
+ * `{norm_f16_le[2], packed_indices[12]}` (`Turbo3Block`, crates/quant/src/lib.rs:129-172;
+ * 56 bytes per head, 4.57x smaller than fp16): `[num_blocks][block_size][num_kv_heads][56]`
+ * bytes, 2-byte aligned, with the slots and block tables of the fp16 pools.
+ * head_dim is 128 (`TURBOQUANT_HEAD_DIM`). */
+
+/* `encode_turbo3_0_head` (crates/quant/src/lib.rs:316-353) of every head of row t of
+ * k_new / v_new (fp16 `[total_tokens][num_kv_heads][128]`, widened to f32), written to pool
+ * row slot_mapping[t] (negative: skipped).  Bytes identical to the reference function's. */
+logismos_status_t logismos_launch_kv_write_turbo3(const void* k_new_f16, const void* v_new_f16,
+                                                  void* k_pool_t3, void* v_pool_t3,
+                                                  const int64_t* slot_mapping, int total_tokens,
+                                                  int num_kv_heads, logismos_stream_t stream);
+
+/* `decode_turbo3_0_head` (crates/quant/src/lib.rs:376-413) of rows
+ * [start_pos, start_pos + n_tokens) of one sequence (block_table_row: device int32) into
+ * f32 `[n_tokens][num_kv_heads][128]`; values identical to the reference function's. */
+logismos_status_t logismos_launch_kv_gather_turbo3_f32(const void* k_pool_t3,
+                                                       const void* v_pool_t3,
+                                                       const int32_t* block_table_row,
+                                                       void* k_out_f32, void* v_out_f32,
+                                                       int start_pos, int n_tokens,
+                                                       int num_kv_heads, int block_size,
+                                                       logismos_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * Memory-system probes (measurement aids; the reference has no counterpart,
  * its only timing helper is the hipEvent pair of
  * crates/kernels/examples/gemm_bench.rs:120-128).  A plain copy and a plain

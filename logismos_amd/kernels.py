@@ -100,6 +100,8 @@ _SIGNATURES = {
     "logismos_paged_kv_cache_v_pool": (_vp, [_vp, _i]),
     "logismos_paged_kv_cache_block_tables": (_vp, [_vp]),
     "logismos_paged_kv_cache_block_tables_host": (_vp, [_vp]),
+    "logismos_launch_kv_write_turbo3": (C.c_uint32, [_vp] * 5 + [_i, _i, _vp]),
+    "logismos_launch_kv_gather_turbo3_f32": (C.c_uint32, [_vp] * 5 + [_i] * 4 + [_vp]),
     "logismos_launch_probe_copy": (C.c_uint32, [_vp, _vp, _sz, _vp]),
     "logismos_launch_probe_read": (C.c_uint32, [_vp, _vp, _sz, _vp]),
 }
@@ -276,6 +278,21 @@ def launch_pack_ragged(new_tokens, prior_ctx, block_tables, cu_seqlens, slot_map
     _status("pack_ragged", library().logismos_launch_pack_ragged(
         _ptr(new_tokens), _ptr(prior_ctx), _ptr(block_tables), _ptr(cu_seqlens),
         _ptr(slot_mapping), _ptr(context_lens), num_seqs, block_size, max_blocks, _raw(stream)))
+
+
+def launch_kv_write_turbo3(k_new, v_new, k_pool, v_pool, slot_mapping, total_tokens: int,
+                           num_kv_heads: int, stream=None) -> None:
+    _status("kv_write_turbo3", library().logismos_launch_kv_write_turbo3(
+        _ptr(k_new), _ptr(v_new), _ptr(k_pool), _ptr(v_pool), _ptr(slot_mapping), total_tokens,
+        num_kv_heads, _raw(stream)))
+
+
+def launch_kv_gather_turbo3_f32(k_pool, v_pool, block_table_row, k_out, v_out, start_pos: int,
+                                n_tokens: int, num_kv_heads: int, block_size: int,
+                                stream=None) -> None:
+    _status("kv_gather_turbo3_f32", library().logismos_launch_kv_gather_turbo3_f32(
+        _ptr(k_pool), _ptr(v_pool), _ptr(block_table_row), _ptr(k_out), _ptr(v_out), start_pos,
+        n_tokens, num_kv_heads, block_size, _raw(stream)))
 
 
 def launch_kv_write_fp16(k_new, v_new, k_pool, v_pool, slot_mapping, total_tokens: int,
