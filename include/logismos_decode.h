@@ -558,6 +558,22 @@ logismos_status_t logismos_launch_kv_gather_turbo3_f32(const void* k_pool_t3,
                                                        int num_kv_heads, int block_size,
                                                        logismos_stream_t stream);
 
+/* `logismos_launch_paged_attn_varlen_fp16` over turbo3 pools, for decode rows
+ * (every sequence has 0 or 1 new tokens: max_seqlen_q <= 1, else
+ * hipErrorInvalidValue): out = softmax(q . K^T * scale) . V with K and V the rows
+ * `decode_turbo3_0_head` (crates/quant/src/lib.rs:376-413) would return.  The decode is
+ * fused into the gather: since a decoded row is norm * H c with H the orthonormal,
+ * symmetric transform of `fwht_128` (:88-113), the kernel transforms each query once,
+ * multiplies with the centroid values c (as fp16) and transforms each output once;
+ * nothing is decoded to memory.  Same workspace, num_splits and block tables as the
+ * fp16 entry point; head_dim is 128; fp16 q and out. */
+logismos_status_t logismos_launch_paged_attn_varlen_turbo3(
+    const void* q_f16, const void* k_pool_t3, const void* v_pool_t3, const int32_t* block_tables,
+    const int32_t* cu_seqlens_q, const int32_t* context_lens, void* out_f16, void* workspace,
+    int num_seqs, int total_tokens, int max_seqlen_q, int num_q_heads, int num_kv_heads,
+    int block_size, int max_blocks_per_seq, int num_splits, float scale,
+    logismos_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Memory-system probes (measurement aids; the reference has no counterpart,
  * its only timing helper is the hipEvent pair of

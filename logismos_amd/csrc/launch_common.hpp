@@ -22,13 +22,14 @@ inline logismos_status_t reject(char* msg, size_t cap, const char* fmt, ...) {
 }
 
 // Library-internal form of the paged-attention launcher: the public one with the
-// output element type selectable (fp16, or bf16 for the step executor).
+// output element type selectable (fp16, or bf16 for the step executor) and the pools either
+// fp16 or turbo3 (kv_turbo3 != 0: decode rows only).
 logismos_status_t paged_attn_launch(
     const void* q_f16, const void* k_pool_f16, const void* v_pool_f16, const int32_t* block_tables,
     const int32_t* cu_seqlens_q, const int32_t* context_lens, void* out, void* workspace,
     int num_seqs, int total_tokens, int max_seqlen_q, int num_q_heads, int num_kv_heads,
     int head_dim, int block_size, int max_blocks_per_seq, int num_splits, float scale, int causal,
-    int phases, int out_bf16, logismos_stream_t stream);
+    int phases, int out_bf16, int kv_turbo3, logismos_stream_t stream);
 
 // Streaming Q4G128 GEMM over prepared activations (qgemm_q4_stream.hip): steps per worker
 // for this shape (0: not applicable, use the split-K kernel) and the launch.  K parts are

@@ -85,6 +85,114 @@ __device__ __forceinline__ unsigned short attn_out_elem(float v, int out_bf16) {
     return __builtin_bit_cast(unsigned short, hv);
 }
 
+// ---- TurboQuant 3-bit pools (crates/quant/src/lib.rs): a head row is four 14-byte blocks
+// {fp16 norm, 32 x 3-bit centroid indices}.  With H the (orthonormal, symmetric) transform of
+// `fwht_128`, a decoded row is norm * H c, so q . k = norm * (H q) . c and
+// sum_j p_j v_j = H sum_j (p_j norm_j) c_j: the kernel transforms q once, works on the
+// centroid values themselves and transforms the result once.
+struct KvTileT3 {
+    unsigned k[4], v[4];  // 24 index bits (8 values) each, in bits 8..31
+    unsigned short kn[4], vn[4];
+};
+
+// fp16 bits of `TURBO3_CODEBOOK` (RNE): b207 af90 ac43 a588 2588 2c43 2f90 3207; tables of
+// their low and high bytes for v_perm_b32
+constexpr unsigned kT3LoLo = 0x88439007u, kT3LoHi = 0x07904388u;
+constexpr unsigned kT3HiLo = 0xa5acafb2u, kT3HiHi = 0x322f2c25u;
+
+// four 3-bit indices (12 bits) -> four fp16 centroids (two dwords)
+__device__ __forceinline__ void turbo3_decode4(unsigned x12, unsigned& w0, unsigned& w1) {
+    const unsigned t = (x12 | (x12 << 10)) & 0x003F003Fu;
+    const unsigned u = (t | (t << 5)) & 0x07070707u;  // one index per byte
+    const unsigned lob = __builtin_amdgcn_perm(kT3LoHi, kT3LoLo, u);
+    const unsigned hib = __builtin_amdgcn_perm(kT3HiHi, kT3HiLo, u);
+    w0 = __builtin_amdgcn_perm(hib, lob, 0x05010400u);
+    w1 = __builtin_amdgcn_perm(hib, lob, 0x07030602u);
+}
+
+// the dword loaded one byte before a 3-byte group -> its eight fp16 centroids
+__device__ __forceinline__ half8_t turbo3_decode8(unsigned dword) {
+    const unsigned x = dword >> 8;
+    unsigned w0, w1, w2, w3;
+    turbo3_decode4(x & 0xFFFu, w0, w1);
+    turbo3_decode4(x >> 12, w2, w3);
+    const uint4_t o = {w0, w1, w2, w3};
+    return __builtin_bit_cast(half8_t, o);
+}
+
+__device__ __forceinline__ unsigned load_u32_unaligned(const uint8_t* ptr) {
+    unsigned v;
+    __builtin_memcpy(&v, ptr, 4);
+    return v;
+}
+
+// fwht_128 of a head held by the 4 lanes tg of a column as x[j][i] = element 8*(tg + 4j) + i
+__device__ __forceinline__ void fwht_pieces(float (&x)[4][8]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int h = 1; h < 8; h <<= 1)
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if ((i & h) == 0) {
+                    const float a = x[j][i], b = x[j][i + h];
+                    x[j][i] = a + b;
+                    x[j][i + h] = a - b;
+                }
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int mask = 16; mask <= 32; mask <<= 1) {
+        const bool hi = (lane & mask) != 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float o = shfl_xor_f32(x[j][i], mask);
+                x[j][i] = hi ? o - x[j][i] : x[j][i] + o;
+            }
+    }
+#pragma unroll
+    for (int h = 1; h < 4; h <<= 1)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if ((j & h) == 0)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float a = x[j][i], b = x[j + h][i];
+                    x[j][i] = a + b;
+                    x[j + h][i] = a - b;
+                }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[j][i] *= 0.08838834764831844f;
+}
+
+// fwht_128 of a head held by the 16 lanes c of a row as x[e] = element 8c + e
+__device__ __forceinline__ void fwht_row(float (&x)[8]) {
+#pragma unroll
+    for (int h = 1; h < 8; h <<= 1)
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if ((i & h) == 0) {
+                const float a = x[i], b = x[i + h];
+                x[i] = a + b;
+                x[i + h] = a - b;
+            }
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int mask = 1; mask <= 8; mask <<= 1) {
+        const bool hi = (lane & mask) != 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float o = shfl_xor_f32(x[i], mask);
+            x[i] = hi ? o - x[i] : x[i] + o;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] *= 0.08838834764831844f;
+}
+
 // Output row of a query with no visible key: zeros (softmax over zero columns).
 template <int G>
 __device__ __forceinline__ void attn_write_zero_row(const AttnParams& p, int t, int kvh, int lane) {
@@ -113,7 +221,7 @@ __device__ __forceinline__ void attn_write_zero_row(const AttnParams& p, int t, 
 // of decode sequence s, KV head kvh, query token t.  `single`: the range is the whole
 // context and the normalised output is written; otherwise the partial (m, l, acc) goes to
 // workspace slot `slot`.
-template <int G>
+template <int G, bool T3>
 __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t, int kvh,
                                                int tok_begin, int tok_end, bool single,
                                                int64_t slot) {
@@ -131,6 +239,18 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
 #pragma unroll
         for (int j = 0; j < 4; ++j)
             qreg[j] = (c < G) ? *reinterpret_cast<const half8_t*>(qp + 32 * j) : z;
+        if constexpr (T3) {
+            float x[4][8];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) x[j][i] = (float)qreg[j][i];
+            fwht_pieces(x);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) qreg[j][i] = (_Float16)x[j][i];
+        }
     }
 
     // ---- tile loader.  The physical block id is a scalar load (wave-uniform
@@ -144,12 +264,35 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
 #pragma unroll
     for (int i = 0; i < 4; ++i) v_lane_off[i] = (unsigned)(4 * tg + i) * row_stride;
 
-    auto load_tile = [&](int tile, KvTile& kv) {
+    using Tile = typename std::conditional<T3, KvTileT3, KvTile>::type;
+    // turbo3: byte offsets inside a tile (row stride = hkv * 56); a lane reads the dword
+    // that starts one byte before its 3-byte group, which never leaves the head row
+    const unsigned row_bytes = (unsigned)p.hkv * 56u;
+    const unsigned k3_piece = 14u * 0u + 1u + 3u * tg;                 // + 14 * j
+    const unsigned v3_piece = 14u * (c >> 2) + 1u + 3u * (c & 3);
+    auto load_tile = [&](int tile, Tile& kv) {
         const int tok_base = __builtin_amdgcn_readfirstlane(tok_begin + tile * kTileKeys);
         const int blk_idx = tok_base / p.block_size;
         const int blk = bt_row[blk_idx];
         // wave-uniform 64-bit base of the tile's first row, this KV head
         const int64_t row_base = (int64_t)blk * p.block_size + (tok_base - blk_idx * p.block_size);
+        if constexpr (T3) {
+            const int64_t base = (row_base * p.hkv + kvh) * 56;
+            const uint8_t* kb = reinterpret_cast<const uint8_t*>(p.k_pool) + base;
+            const uint8_t* vb = reinterpret_cast<const uint8_t*>(p.v_pool) + base;
+            const unsigned last_off = (unsigned)(tok_end - 1 - tok_base) * row_bytes;
+            const unsigned ko = min((unsigned)c * row_bytes, last_off) + k3_piece;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) kv.k[j] = load_u32_unaligned(kb + ko + 14u * j);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const unsigned ro = min((unsigned)(4 * tg + i) * row_bytes, last_off);
+                kv.v[i] = load_u32_unaligned(vb + ro + v3_piece);
+                kv.kn[i] = *reinterpret_cast<const unsigned short*>(kb + ro);
+                kv.vn[i] = *reinterpret_cast<const unsigned short*>(vb + ro);
+            }
+            return;
+        }
         const int64_t base = (row_base * p.hkv + kvh) * kHeadDim;
         const _Float16* kb = p.k_pool + base;
         const _Float16* vb = p.v_pool + base;
@@ -157,12 +300,15 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
         // probability is forced to zero below); never touches another block
         const unsigned last_off = (unsigned)(tok_end - 1 - tok_base) * row_stride;
         const unsigned ko = min(k_lane_off, last_off) + 8u * tg;
+        if constexpr (!T3) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) kv.k[j] = *reinterpret_cast<const half8_t*>(kb + ko + 32 * j);
+            for (int j = 0; j < 4; ++j)
+                kv.k[j] = *reinterpret_cast<const half8_t*>(kb + ko + 32 * j);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const unsigned vo = min(v_lane_off[i], last_off) + 8u * c;
-            kv.v[i] = *reinterpret_cast<const half8_t*>(vb + vo);
+            for (int i = 0; i < 4; ++i) {
+                const unsigned vo = min(v_lane_off[i], last_off) + 8u * c;
+                kv.v[i] = *reinterpret_cast<const half8_t*>(vb + vo);
+            }
         }
     };
 
@@ -174,7 +320,20 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[h][e] = 0.0f;
 
-    auto compute_tile = [&](int tile, const KvTile& kv) {
+    auto compute_tile = [&](int tile, const Tile& raw) {
+        KvTile kv;
+        float kn[4], vn[4];
+        if constexpr (T3) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                kv.k[j] = turbo3_decode8(raw.k[j]);
+                kv.v[j] = turbo3_decode8(raw.v[j]);
+                kn[j] = __half2float(__builtin_bit_cast(__half, raw.kn[j])) * p.scale_log2e;
+                vn[j] = __half2float(__builtin_bit_cast(__half, raw.vn[j]));
+            }
+        } else {
+            kv = raw;
+        }
         float4_t sacc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int j = 0; j < 4; ++j)
@@ -184,7 +343,8 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
         float mx = m;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            sc[r] = (tok0 + r < tok_end) ? sacc[r] * p.scale_log2e : -INFINITY;
+            const float sv = T3 ? sacc[r] * kn[r] : sacc[r] * p.scale_log2e;
+            sc[r] = (tok0 + r < tok_end) ? sv : -INFINITY;
             mx = fmaxf(mx, sc[r]);
         }
         const float msafe = (mx == -INFINITY) ? 0.0f : mx;
@@ -198,6 +358,11 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
         }
         l = l * alpha + psum;
         m = mx;
+        if constexpr (T3) {
+            // the value rows are unit-scale centroids: their norms ride on the probabilities
+#pragma unroll
+            for (int r = 0; r < 4; ++r) pr[r] *= vn[r];
+        }
         static_for<G>([&](auto hc) {
             constexpr int h = decltype(hc)::value;
             const float a = row_bcast<h>(alpha);
@@ -223,7 +388,7 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
     // compute_tile), so the loads of the next tile stay in flight while the
     // current one is consumed and the wait counts stay exact.
     const int last_tile = ntiles - 1;
-    KvTile buf0, buf1;
+    Tile buf0, buf1;
     load_tile(0, buf0);
     for (int tile = 0; tile < ntiles; tile += 2) {
         load_tile(min(tile + 1, last_tile), buf1);
@@ -256,6 +421,7 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
             }
             mh = mn;
         }
+        if constexpr (T3) fwht_row(acc[h]);  // back from the centroid domain (all rows alike)
         if (tg == (h & 3)) {
             const int head = kvh * G + h;
             if (single) {
@@ -300,7 +466,7 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
 // workgroup are consecutive KV heads of the same keys: together they stream whole token
 // rows (hkv * 256 contiguous bytes).  Sequences with more new tokens belong to
 // paged_attn_prefill_kernel below.
-template <int G>
+template <int G, bool T3>
 __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_kernel(const AttnParams p) {
     const int lane = threadIdx.x & 63;
     const int kvh = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -316,8 +482,8 @@ __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_kernel(const At
     const int tok_begin = split * p.part_tokens;
     if (tok_begin >= ctx) return;
     const int num_parts = (ctx + p.part_tokens - 1) / p.part_tokens;
-    attn_partition<G>(p, s, t, kvh, tok_begin, min(ctx, tok_begin + p.part_tokens), num_parts == 1,
-                      (int64_t)s * p.num_splits + split);
+    attn_partition<G, T3>(p, s, t, kvh, tok_begin, min(ctx, tok_begin + p.part_tokens),
+                          num_parts == 1, (int64_t)s * p.num_splits + split);
 }
 
 // 16-key tiles sequence s contributes to the decode stream
@@ -344,7 +510,7 @@ __device__ __forceinline__ int worker_tiles(int total_tiles, int num_workers) {
 // piece of sequence s is written to workspace slot w + s (the pieces of one sequence get
 // consecutive slots since both w and s only grow along the stream); a sequence that lies
 // inside one worker is finished there.
-template <int G>
+template <int G, bool T3>
 __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_balanced_kernel(const AttnParams p) {
     __shared__ int pt[kMaxBalancedSeqs + 1];  // exclusive prefix of decode tiles
     const int lane = threadIdx.x & 63;
@@ -399,8 +565,8 @@ __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_balanced_kernel
         const int seg_end = min(te, seq_end);
         const int ctx = p.context_lens[s];
         const bool single = tcur == seq_begin && seg_end == seq_end;
-        attn_partition<G>(p, s, p.cu_seqlens_q[s], kvh, (tcur - seq_begin) * kTileKeys,
-                          min(ctx, (seg_end - seq_begin) * kTileKeys), single, (int64_t)w + s);
+        attn_partition<G, T3>(p, s, p.cu_seqlens_q[s], kvh, (tcur - seq_begin) * kTileKeys,
+                              min(ctx, (seg_end - seq_begin) * kTileKeys), single, (int64_t)w + s);
         tcur = seg_end;
     }
 }
@@ -935,7 +1101,7 @@ static int part_tokens_for(int block_size, int max_blocks_per_seq, int num_split
     return (int)part;
 }
 
-template <int G>
+template <int G, bool T3>
 static hipError_t launch_group(const AttnParams& p, int max_seqlen_q, int phases,
                                hipStream_t stream) {
     // waves per workgroup: the largest divisor of hkv that is <= kMaxHeadWaves
@@ -949,14 +1115,15 @@ static hipError_t launch_group(const AttnParams& p, int max_seqlen_q, int phases
     if (phases & LOGISMOS_ATTN_PHASE_DECODE) {
         if (p.num_workers > 0) {
             dim3 grid_d(p.num_workers, p.hkv / wpb, 1);
-            paged_attn_balanced_kernel<G><<<grid_d, block, 0, stream>>>(p);
+            paged_attn_balanced_kernel<G, T3><<<grid_d, block, 0, stream>>>(p);
         } else {
             dim3 grid_d(p.num_splits, p.hkv / wpb, p.num_seqs);
-            paged_attn_kernel<G><<<grid_d, block, 0, stream>>>(p);
+            paged_attn_kernel<G, T3><<<grid_d, block, 0, stream>>>(p);
         }
     }
-    if ((phases & LOGISMOS_ATTN_PHASE_PREFILL) && max_seqlen_q > 1) {
-        launch_prefill<G>(p, max_seqlen_q, stream);
+    if constexpr (!T3) {
+        if ((phases & LOGISMOS_ATTN_PHASE_PREFILL) && max_seqlen_q > 1)
+            launch_prefill<G>(p, max_seqlen_q, stream);
     }
     if ((phases & LOGISMOS_ATTN_PHASE_MERGE) && p.num_splits > 1) {
         dim3 grid_m(p.hq, p.num_seqs);
@@ -1068,7 +1235,23 @@ extern "C" logismos_status_t logismos_launch_paged_attn_varlen_fp16_phases(
     return lg::paged_attn_launch(q_f16, k_pool_f16, v_pool_f16, block_tables, cu_seqlens_q,
                                  context_lens, out_f16, workspace, num_seqs, total_tokens,
                                  max_seqlen_q, num_q_heads, num_kv_heads, head_dim, block_size,
-                                 max_blocks_per_seq, num_splits, scale, causal, phases, 0, stream);
+                                 max_blocks_per_seq, num_splits, scale, causal, phases, 0, 0,
+                                 stream);
+}
+
+extern "C" logismos_status_t logismos_launch_paged_attn_varlen_turbo3(
+    const void* q_f16, const void* k_pool_t3, const void* v_pool_t3, const int32_t* block_tables,
+    const int32_t* cu_seqlens_q, const int32_t* context_lens, void* out_f16, void* workspace,
+    int num_seqs, int total_tokens, int max_seqlen_q, int num_q_heads, int num_kv_heads,
+    int block_size, int max_blocks_per_seq, int num_splits, float scale,
+    logismos_stream_t stream) {
+    if ((reinterpret_cast<uintptr_t>(k_pool_t3) | reinterpret_cast<uintptr_t>(v_pool_t3)) & 1u)
+        return hipErrorInvalidValue;
+    return lg::paged_attn_launch(q_f16, k_pool_t3, v_pool_t3, block_tables, cu_seqlens_q,
+                                 context_lens, out_f16, workspace, num_seqs, total_tokens,
+                                 max_seqlen_q, num_q_heads, num_kv_heads, 128, block_size,
+                                 max_blocks_per_seq, num_splits, scale, 1,
+                                 LOGISMOS_ATTN_PHASE_ALL, 0, 1, stream);
 }
 
 logismos_status_t lg::paged_attn_launch(
@@ -1076,7 +1259,8 @@ logismos_status_t lg::paged_attn_launch(
     const int32_t* cu_seqlens_q, const int32_t* context_lens, void* out_f16, void* workspace,
     int num_seqs, int total_tokens, int max_seqlen_q, int num_q_heads, int num_kv_heads,
     int head_dim, int block_size, int max_blocks_per_seq, int num_splits, float scale, int causal,
-    int phases, int out_bf16, logismos_stream_t stream) {
+    int phases, int out_bf16, int kv_turbo3, logismos_stream_t stream) {
+    if (kv_turbo3 && max_seqlen_q > 1) return hipErrorInvalidValue;  // decode rows only
     if (logismos_check_paged_attn_shape(num_seqs, total_tokens, max_seqlen_q, num_q_heads,
                                         num_kv_heads, head_dim, block_size, max_blocks_per_seq,
                                         num_splits, nullptr, 0) != 0)
@@ -1115,14 +1299,30 @@ logismos_status_t lg::paged_attn_launch(
 
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (num_q_heads / num_kv_heads) {
-        case 1: return lg::launch_group<1>(p, max_seqlen_q, phases, st);
-        case 2: return lg::launch_group<2>(p, max_seqlen_q, phases, st);
-        case 3: return lg::launch_group<3>(p, max_seqlen_q, phases, st);
-        case 4: return lg::launch_group<4>(p, max_seqlen_q, phases, st);
-        case 5: return lg::launch_group<5>(p, max_seqlen_q, phases, st);
-        case 6: return lg::launch_group<6>(p, max_seqlen_q, phases, st);
-        case 7: return lg::launch_group<7>(p, max_seqlen_q, phases, st);
-        case 8: return lg::launch_group<8>(p, max_seqlen_q, phases, st);
+        case 1:
+            return kv_turbo3 ? lg::launch_group<1, true>(p, max_seqlen_q, phases, st)
+                             : lg::launch_group<1, false>(p, max_seqlen_q, phases, st);
+        case 2:
+            return kv_turbo3 ? lg::launch_group<2, true>(p, max_seqlen_q, phases, st)
+                             : lg::launch_group<2, false>(p, max_seqlen_q, phases, st);
+        case 3:
+            return kv_turbo3 ? lg::launch_group<3, true>(p, max_seqlen_q, phases, st)
+                             : lg::launch_group<3, false>(p, max_seqlen_q, phases, st);
+        case 4:
+            return kv_turbo3 ? lg::launch_group<4, true>(p, max_seqlen_q, phases, st)
+                             : lg::launch_group<4, false>(p, max_seqlen_q, phases, st);
+        case 5:
+            return kv_turbo3 ? lg::launch_group<5, true>(p, max_seqlen_q, phases, st)
+                             : lg::launch_group<5, false>(p, max_seqlen_q, phases, st);
+        case 6:
+            return kv_turbo3 ? lg::launch_group<6, true>(p, max_seqlen_q, phases, st)
+                             : lg::launch_group<6, false>(p, max_seqlen_q, phases, st);
+        case 7:
+            return kv_turbo3 ? lg::launch_group<7, true>(p, max_seqlen_q, phases, st)
+                             : lg::launch_group<7, false>(p, max_seqlen_q, phases, st);
+        case 8:
+            return kv_turbo3 ? lg::launch_group<8, true>(p, max_seqlen_q, phases, st)
+                             : lg::launch_group<8, false>(p, max_seqlen_q, phases, st);
         default: return hipErrorInvalidValue;
     }
 }

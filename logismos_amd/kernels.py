@@ -100,6 +100,8 @@ _SIGNATURES = {
     "logismos_paged_kv_cache_v_pool": (_vp, [_vp, _i]),
     "logismos_paged_kv_cache_block_tables": (_vp, [_vp]),
     "logismos_paged_kv_cache_block_tables_host": (_vp, [_vp]),
+    "logismos_launch_paged_attn_varlen_turbo3":
+        (C.c_uint32, [_vp] * 8 + [_i] * 8 + [_f, _vp]),
     "logismos_launch_kv_write_turbo3": (C.c_uint32, [_vp] * 5 + [_i, _i, _vp]),
     "logismos_launch_kv_gather_turbo3_f32": (C.c_uint32, [_vp] * 5 + [_i] * 4 + [_vp]),
     "logismos_launch_probe_copy": (C.c_uint32, [_vp, _vp, _sz, _vp]),
@@ -278,6 +280,19 @@ def launch_pack_ragged(new_tokens, prior_ctx, block_tables, cu_seqlens, slot_map
     _status("pack_ragged", library().logismos_launch_pack_ragged(
         _ptr(new_tokens), _ptr(prior_ctx), _ptr(block_tables), _ptr(cu_seqlens),
         _ptr(slot_mapping), _ptr(context_lens), num_seqs, block_size, max_blocks, _raw(stream)))
+
+
+def launch_paged_attn_varlen_turbo3(q, k_pool, v_pool, block_tables, cu_seqlens_q, context_lens,
+                                    out, workspace, num_seqs, total_tokens, max_seqlen_q,
+                                    num_q_heads, num_kv_heads, block_size, max_blocks_per_seq,
+                                    num_splits, scale, stream=None) -> None:
+    check_paged_attn_shape(num_seqs, total_tokens, max_seqlen_q, num_q_heads, num_kv_heads, 128,
+                           block_size, max_blocks_per_seq, num_splits)
+    _status("paged_attn_varlen_turbo3", library().logismos_launch_paged_attn_varlen_turbo3(
+        _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables), _ptr(cu_seqlens_q),
+        _ptr(context_lens), _ptr(out), _ptr(workspace) if workspace is not None else None,
+        num_seqs, total_tokens, max_seqlen_q, num_q_heads, num_kv_heads, block_size,
+        max_blocks_per_seq, num_splits, float(scale), _raw(stream)))
 
 
 def launch_kv_write_turbo3(k_new, v_new, k_pool, v_pool, slot_mapping, total_tokens: int,

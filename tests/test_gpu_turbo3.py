@@ -112,3 +112,95 @@ def test_encode_then_decode_round_trip_on_the_gpu():
             assert np.array_equal(got[t, h], O.decode_turbo3_0_head(O.encode_turbo3_0_head(kf[t, h])))
     rel = np.linalg.norm(got - kf, axis=2) / np.linalg.norm(kf, axis=2)
     assert rel.max() < 0.25
+
+
+# ------------------------------------------------------------------ attention over turbo3 pools
+def _turbo3_pools(c):
+    """Encodes the fp16 pools of a paged case row by row (on the CPU oracle)."""
+    rows, hkv = c["k_pool"].shape[0], c["hkv"]
+    kp = np.zeros((rows, hkv * 56), np.uint8)
+    vp = np.zeros((rows, hkv * 56), np.uint8)
+    O.kv_write_turbo3(c["k_pool"], c["v_pool"], kp, vp, np.arange(rows, dtype=np.int64), hkv)
+    return kp, vp
+
+
+def _attn_turbo3(c, kp, vp, num_splits=None):
+    S = len(c["context_lens"])
+    T = int(c["cu_seqlens"][-1])
+    ns = num_splits or kernels.paged_attn_num_splits(S, c["hkv"], c["block_size"], c["max_blocks"])
+    out = hip.DeviceBuffer(max(16, c["q"].nbytes))
+    out.fill(0xFF)
+    ws = hip.DeviceBuffer(max(16, kernels.paged_attn_workspace_bytes(S, c["hq"], 128, ns)))
+    ws.fill(0xFF)
+    kernels.launch_paged_attn_varlen_turbo3(
+        _dev(c["q"]), _dev(kp), _dev(vp), _dev(c["block_tables"]), _dev(c["cu_seqlens"]),
+        _dev(c["context_lens"]), out, ws, S, T, int(c["new_tokens"].max()), c["hq"], c["hkv"],
+        c["block_size"], c["max_blocks"], ns, c["scale"])
+    hip.synchronize()
+    return out.to_numpy(np.float16, c["q"].shape)
+
+
+def _oracle_t3(c, kp, vp):
+    return O.paged_attn_varlen_turbo3(c["q"], kp, vp, c["block_tables"], c["cu_seqlens"],
+                                      c["context_lens"], c["hq"], c["hkv"], c["block_size"],
+                                      c["scale"], True)
+
+
+@pytest.mark.parametrize("hq,hkv", [(1, 1), (4, 2), (12, 2), (32, 8), (8, 1), (14, 2)])
+def test_turbo3_attention_gqa_group_sizes(hq, hkv):
+    rng = np.random.default_rng(70 + hq + hkv)
+    new = [1, 1, 1, 1, 1, 0, 1]
+    prior = [0, 15, 16, 127, 1000, 5, 333]
+    c = workloads.paged_case(rng, new, prior, hq=hq, hkv=hkv)
+    kp, vp = _turbo3_pools(c)
+    want = _oracle_t3(c, kp, vp)
+    for ns in (1, 3, 16):
+        assert_parity(_attn_turbo3(c, kp, vp, ns), want, what=f"turbo3 {hq}/{hkv} splits {ns}")
+
+
+def test_turbo3_attention_balanced_kernel_and_zero_context():
+    rng = np.random.default_rng(71)
+    new = np.ones(12, np.int32)
+    prior = [0, 40, 2047, 16, 511, 300, 1, 999, 64, 65, 129, 700]
+    c = workloads.paged_case(rng, new, prior, hq=8, hkv=2, min_max_blocks=8192)
+    c["context_lens"][3] = 0
+    kp, vp = _turbo3_pools(c)
+    want = _oracle_t3(c, kp, vp)
+    got = _attn_turbo3(c, kp, vp)
+    assert (got[3] == 0).all() and (want[3] == 0).all()
+    assert_parity(got, want, what="turbo3 balanced")
+    assert_parity(_attn_turbo3(c, kp, vp, 5), want, what="turbo3 balanced, 5 splits")
+
+
+def test_turbo3_attention_tracks_fp16_attention_over_the_same_rows():
+    # the codec's error, not the kernel's: turbo3 attention stays close to fp16 attention
+    # over the rows it was encoded from (loose bound; values ~N(0,1), outputs ~0.1..1)
+    rng = np.random.default_rng(72)
+    c = workloads.paged_case(rng, [1, 1], [600, 90], hq=8, hkv=2)
+    kp, vp = _turbo3_pools(c)
+    got = _attn_turbo3(c, kp, vp).astype(np.float32)
+    ref = O.paged_attn_varlen_fp16(c["q"], c["k_pool"], c["v_pool"], c["block_tables"],
+                                   c["cu_seqlens"], c["context_lens"], 8, 2, 128, 16, c["scale"],
+                                   True).astype(np.float32)
+    assert np.abs(got - ref).max() < 0.35 and np.corrcoef(got.ravel(), ref.ravel())[0, 1] > 0.8
+
+
+def test_turbo3_attention_rejects_prefill_rows():
+    rng = np.random.default_rng(73)
+    c = workloads.paged_case(rng, [1, 4], [10, 20], hq=4, hkv=2)
+    kp, vp = _turbo3_pools(c)
+    with pytest.raises(kernels.LaunchError):
+        _attn_turbo3(c, kp, vp)
+
+
+def test_put_encode_then_attend_round_trip_on_the_gpu():
+    # new rows encoded by the GPU writer into turbo3 pools, then attended to: the same
+    # bytes and the same result as the CPU path end to end
+    rng = np.random.default_rng(74)
+    c = workloads.paged_case(rng, np.ones(3, np.int32), [70, 5, 300], hq=8, hkv=2)
+    rows = c["k_pool"].shape[0]
+    kp, vp = _encode_gpu(c["k_pool"], c["v_pool"], np.arange(rows, dtype=np.int64), rows, 2)
+    kp_h, vp_h = _turbo3_pools(c)
+    assert np.array_equal(kp.to_numpy(np.uint8, kp_h.shape), kp_h)
+    got = _attn_turbo3(c, kp_h, vp_h)
+    assert_parity(got, _oracle_t3(c, kp_h, vp_h), what="turbo3 put -> attend")
