@@ -279,13 +279,51 @@ def bench_mixed_config4(args):
         "roofline": {"bound": "mfma", "achieved": round(flops_pre / (ms_pre * 1e-3) / 1e12, 1),
                      "peak": 2500.0, "unit": "TFLOP/s",
                      "frac": round(flops_pre / (ms_pre * 1e-3) / 1e12 / 2500.0, 4),
-                     "traffic": None, "kernel": "paged_attn_prefill_kernel<4,2>",
+                     "traffic": None, "kernel": "paged_attn_prefill_kernel<4>",
                      "flops_per_launch": flops_pre},
         "decode_rows_GBps": round(dec_bytes / (ms_dec * 1e-3) / 1e9, 1),
         "gpu_packing_bit_exact": bool(pack_ok),
         "parity_max_abs_vs_oracle": max_abs,
         "parity_sample": f"sequences {pick} (1 prefill chunk, 3 decode rows)",
     }
+
+
+def bench_turbo3(args):
+    """One layer's decode attention of config 5 over TurboQuant 3-bit pools (56 bytes per
+    head row instead of 256), next to the fp16 pools it was encoded from."""
+    case = workloads.config5_attention()
+    stream = hip.Stream()
+    S, hq, hkv = len(case["context_lens"]), case["hq"], case["hkv"]
+    r = PagedAttnRunner(case, stream=stream)
+    rows = case["k_pool"].shape[0]
+    slots = hip.DeviceBuffer.from_numpy(np.arange(rows, dtype=np.int64))
+    copies = 3   # 3 x 2 x 0.3 GB of fp16 pools > 2 x Infinity Cache
+    kps, vps = replicate(r.k_pool, copies), replicate(r.v_pool, copies)
+    t3 = []
+    for k, v in zip(kps, vps):
+        kp, vp = hip.DeviceBuffer(rows * hkv * 56), hip.DeviceBuffer(rows * hkv * 56)
+        kernels.launch_kv_write_turbo3(k, v, kp, vp, slots, rows, hkv, stream)
+        t3.append((kp, vp))
+    stream.synchronize()
+    ns = r.num_splits
+
+    def turbo(kp, vp):
+        return lambda: kernels.launch_paged_attn_varlen_turbo3(
+            r.q, kp, vp, r.bt, r.cu, r.ctx, r.out, r.ws, S, S, 1, hq, hkv, case["block_size"],
+            case["max_blocks"], ns, case["scale"], stream)
+    ms16, _, _ = time_launches(stream, [(lambda k=k, v=v: r.launch(k_pool=k, v_pool=v))
+                                        for k, v in zip(kps, vps)], 60, 6)
+    ms3, _, _ = time_launches(stream, [turbo(k, v) for k, v in t3], 60, 6)
+    ctx = int(case["context_lens"].sum())
+    return {"workload": "config 5 attention (32 seqs, ctx U[256,8192], 32 q / 8 kv heads), one "
+                        "layer, decode + merge; turbo3 = TurboQuant 3-bit KV, decode fused",
+            "sum_ctx": ctx,
+            "fp16": {"us": round(ms16 * 1e3, 1), "kv_bytes": ctx * 4096,
+                     "GBps": round(ctx * 4096 / ms16 / 1e6, 1)},
+            "turbo3": {"us": round(ms3 * 1e3, 1), "kv_bytes": ctx * 896,
+                       "GBps": round(ctx * 896 / ms3 / 1e6, 1)},
+            "keys_per_us": {"fp16": round(ctx / (ms16 * 1e3), 1),
+                            "turbo3": round(ctx / (ms3 * 1e3), 1)}}
 
 
 def bench_qgemv_q8(args):
@@ -546,6 +584,7 @@ def main():
                                                           "roofline", "cpu_baseline",
                                                           "parity_max_abs_vs_oracle")}
         line["mixed_prefill_decode_config4"] = bench_mixed_config4(args)
+        line["paged_attn_turbo3_config5"] = bench_turbo3(args)
         line["qgemv_q8_config1"] = bench_qgemv_q8(args)
         line["qgemm_q4_config3"] = bench_q4(args)
     print(json.dumps(line))
