@@ -177,7 +177,8 @@ def bench_paged_decode(args):
                    "hip_graph": graphed},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "paged_attn_balanced_kernel<6>", "ms_per_launch": round(ms_dec, 5),
+                     "kernel": "paged_attn_kernel<6> (static split; a batch this small stays off the "
+                               "balanced kernel)", "ms_per_launch": round(ms_dec, 5),
                      "warm_cache_GBps": round(algo / (ms_warm * 1e-3) / 1e9, 1)},
         "cpu_baseline": {"value": round(cpu_gbps, 2), "unit": "GB/s", "cores": cores,
                          "kind": "port",
