@@ -380,6 +380,29 @@ logismos_status_t logismos_launch_silu_mul_f32p_xprep(const void* parts_f32, int
 logismos_status_t logismos_launch_greedy_f32(const void* logits_f32, void* out_u32, int rows, int n,
                                              logismos_stream_t stream);
 
+/* Vocabulary projection and token selection in one pass: logits = x . W^T over Q4G128
+ * weights `[n][k]` (x in the prepared layout, rows = b <= 32, k % 1024 == 0), then
+ * out_tokens[r] = `decode::greedy` of row r (crates/decode/src/lib.rs:73-83: strict >, the
+ * first maximum wins; a row with no value above -inf gives 0).  The logits never go to
+ * memory unless `logits_f32` (`[b][n]`, may be NULL) asks for them.  `workspace`:
+ * logismos_qgemm_q4g128_greedy_workspace_bytes() bytes, 4-byte aligned, contents don't matter. */
+logismos_status_t logismos_check_qgemm_q4g128_greedy_shape(int b, int n, int k, char* msg,
+                                                           size_t msg_cap);
+size_t logismos_qgemm_q4g128_greedy_workspace_bytes(int b, int n, int k);
+logismos_status_t logismos_launch_qgemm_q4g128_greedy_xprep(
+    const void* x_prepared, const void* qw_u8, const void* scale_f16, const void* zero_f16,
+    void* out_tokens_u32, void* logits_f32, void* workspace, int b, int n, int k,
+    logismos_stream_t stream);
+
+/* out[r][:] = table[ids[r]][:] as fp32, table `[vocab][hidden]` fp32 or bf16; an id >= vocab
+ * gives a zero row (`embed_lookup`, crates/kernels/src/cpu_f32/mod.rs:106-127). */
+logismos_status_t logismos_launch_embed_lookup_f32(const void* table_f32, const void* ids_u32,
+                                                   void* out_f32, int rows, int hidden,
+                                                   long long vocab, logismos_stream_t stream);
+logismos_status_t logismos_launch_embed_lookup_bf16(const void* table_bf16, const void* ids_u32,
+                                                    void* out_f32, int rows, int hidden,
+                                                    long long vocab, logismos_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Decode step: one new token for each of num_seqs <= 32 live sequences through
  * num_layers pre-norm layers (`StellaLayer::forward` order,
@@ -392,9 +415,17 @@ logismos_status_t logismos_launch_greedy_f32(const void* logits_f32, void* out_u
  * xn = RMSNorm(h); act = silu(xn.Wgate^T) * (xn.Wup^T); down projection.
  * Wqkv stacks the q, k and v projections (rows: hq*128, hkv*128, hkv*128),
  * Wgate_up stacks gate and up (intermediate rows each).  After the last layer
- * out = bf16(RMSNorm(h) * final_norm_w).  All launches are asynchronous on
- * `stream`; `workspace` needs logismos_decode_step_workspace_bytes() bytes,
- * 256-byte aligned, contents don't matter.
+ * out = bf16(RMSNorm(h) * final_norm_w).
+ *
+ * Tokens in, tokens out (both optional, cfg->vocab > 0): with `token_ids` the step first
+ * fills hidden_f32 from `embed_table_bf16` (`embed_lookup`,
+ * crates/kernels/src/cpu_f32/mod.rs:106-127: an id outside the vocabulary is a zero row);
+ * with `lm_head` it ends with the vocabulary projection of the normed state and
+ * `decode::greedy` per sequence (crates/decode/src/lib.rs:73-83) into `out_tokens_u32`
+ * (and the fp32 logits into `logits_f32` if that is not NULL); `out_bf16` may then be NULL.
+ *
+ * All launches are asynchronous on `stream`; `workspace` needs
+ * logismos_decode_step_workspace_bytes() bytes, 256-byte aligned, contents don't matter.
  * ------------------------------------------------------------------------ */
 typedef struct {
     const void* qw;    /* uint8 [N][K/2] */
@@ -406,6 +437,7 @@ typedef struct {
     int num_layers, hidden, num_q_heads, num_kv_heads, head_dim, intermediate;
     float rms_eps;
     int block_size, max_blocks_per_seq, max_pos;
+    int vocab; /* rows of the embedding table and of lm_head; 0 when neither is used */
 } logismos_decode_config_t;
 
 typedef struct {
@@ -429,6 +461,11 @@ typedef struct {
     const void* rope_sin_f32;
     int num_seqs;
     int num_splits;
+    const uint32_t* token_ids;           /* [num_seqs] or NULL: hidden_f32 is the input */
+    const void* embed_table_bf16;        /* [vocab][hidden], with token_ids */
+    const logismos_q4_weight_t* lm_head; /* [vocab][hidden] Q4G128 (host pointer) or NULL */
+    void* out_tokens_u32;                /* [num_seqs], with lm_head */
+    void* logits_f32;                    /* [num_seqs][vocab] or NULL */
 } logismos_decode_batch_t;
 
 size_t logismos_decode_step_workspace_bytes(const logismos_decode_config_t* cfg, int num_seqs,

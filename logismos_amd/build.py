@@ -41,6 +41,7 @@ EXTRA_FLAGS = {
     "paged_attn.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "qgemm_q4_splitk.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "qgemm_q4_stream.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "qgemm_q4_greedy.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
 }
 
 

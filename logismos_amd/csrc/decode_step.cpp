@@ -18,6 +18,7 @@ struct Workspace {
     char* gate_up;   // f32  [Jgu][B][2*inter]
     char* act;       // prepared activations of width inter (input of the down projection)
     char* attn_ws;   // split-K workspace of the attention
+    char* head_ws;   // per-workgroup candidates of the token selection (vocab > 0)
     int j_qkv, j_o, j_gu, j_down;
     size_t total;
 };
@@ -47,6 +48,9 @@ Workspace carve(const logismos_decode_config_t& c, int b, int num_splits, char* 
     w.gate_up = take((size_t)w.j_gu * b * 2 * c.intermediate * 4);
     w.act = take(logismos_q4_xprep_bytes(b, c.intermediate));
     w.attn_ws = take(logismos_paged_attn_workspace_bytes(b, c.num_q_heads, c.head_dim, num_splits));
+    w.head_ws = c.vocab > 0
+                    ? take(logismos_qgemm_q4g128_greedy_workspace_bytes(b, c.vocab, c.hidden))
+                    : nullptr;
     w.total = off;
     return w;
 }
@@ -58,6 +62,9 @@ bool config_ok(const logismos_decode_config_t* c, int b) {
     if (c->head_dim != 128 || c->num_q_heads <= 0 || c->num_kv_heads <= 0) return false;
     if (c->hidden % 128 != 0 || c->intermediate % 128 != 0) return false;
     if (((int64_t)c->num_q_heads * c->head_dim) % 128 != 0) return false;
+    if (c->vocab < 0) return false;
+    if (c->vocab > 0 && logismos_check_qgemm_q4g128_greedy_shape(b, c->vocab, c->hidden, nullptr, 0))
+        return false;
     return true;
 }
 
@@ -85,11 +92,20 @@ extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_c
     if (!config_ok(cfg, b) || batch->num_splits <= 0) return hipErrorInvalidValue;
     if (reinterpret_cast<uintptr_t>(workspace) & 255u) return hipErrorInvalidValue;
     const logismos_decode_config_t& c = *cfg;
+    const bool tokens_in = batch->token_ids != nullptr;
+    const bool tokens_out = batch->lm_head != nullptr;
+    if ((tokens_in || tokens_out) && c.vocab <= 0) return hipErrorInvalidValue;
+    if (tokens_in && !batch->embed_table_bf16) return hipErrorInvalidValue;
+    if (tokens_out && !batch->out_tokens_u32) return hipErrorInvalidValue;
+    if (!tokens_out && !batch->out_bf16) return hipErrorInvalidValue;
     const Workspace w = carve(c, b, batch->num_splits, static_cast<char*>(workspace));
     const int qd = c.num_q_heads * c.head_dim;
     const int kvd = c.num_kv_heads * c.head_dim;
     const float scale = 1.0f / sqrtf((float)c.head_dim);
 
+    if (tokens_in)
+        LG_TRY(logismos_launch_embed_lookup_bf16(batch->embed_table_bf16, batch->token_ids,
+                                                 batch->hidden_f32, b, c.hidden, c.vocab, stream));
     int res_parts = 0;  // split-K parts of the projection the next add_rms_norm folds into h
     for (int l = 0; l < c.num_layers; ++l) {
         const logismos_decode_layer_t& L = layers[l];
@@ -123,8 +139,21 @@ extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_c
                                                              c.intermediate, stream));
         res_parts = w.j_down;
     }
-    LG_TRY(logismos_launch_add_rms_norm_f32p(batch->hidden_f32, w.proj, res_parts,
-                                             batch->final_norm_w_f32, batch->out_bf16, b, c.hidden,
-                                             c.rms_eps, stream));
+    if (tokens_out) {
+        // the normed state in the layout of the vocabulary projection, then the projection
+        // with the token choice fused into it
+        LG_TRY(logismos_launch_add_rms_norm_f32p_xprep(batch->hidden_f32, w.proj, res_parts,
+                                                       batch->final_norm_w_f32, w.xn, b, c.hidden,
+                                                       c.rms_eps, stream));
+        res_parts = 0;  // folded into h by the call above
+        const logismos_q4_weight_t& H = *batch->lm_head;
+        LG_TRY(logismos_launch_qgemm_q4g128_greedy_xprep(w.xn, H.qw, H.scale, H.zero,
+                                                         batch->out_tokens_u32, batch->logits_f32,
+                                                         w.head_ws, b, c.vocab, c.hidden, stream));
+    }
+    if (batch->out_bf16)
+        LG_TRY(logismos_launch_add_rms_norm_f32p(batch->hidden_f32, w.proj, res_parts,
+                                                 batch->final_norm_w_f32, batch->out_bf16, b,
+                                                 c.hidden, c.rms_eps, stream));
     return 0;
 }

@@ -361,6 +361,29 @@ __global__ __launch_bounds__(256) void greedy_kernel(const float* __restrict__ l
     if (threadIdx.x == 0) out[row] = si[0] == 0x7fffffff ? 0u : (uint32_t)si[0];
 }
 
+// out[r][:] = table[ids[r]][:] widened to fp32; an id outside the vocabulary gives a zero row
+// (`embed_lookup`, crates/kernels/src/cpu_f32/mod.rs:106-127).
+template <bool BF16>
+__global__ __launch_bounds__(256) void embed_lookup_kernel(const void* __restrict__ table,
+                                                           const uint32_t* __restrict__ ids,
+                                                           float* __restrict__ out, int hidden,
+                                                           int64_t vocab) {
+    const int64_t row = blockIdx.x;
+    const uint32_t id = ids[row];
+    const bool valid = (int64_t)id < vocab;
+    float* o = out + row * hidden;
+    for (int j = threadIdx.x; j < hidden; j += 256) {
+        float v = 0.0f;
+        if (valid) {
+            if constexpr (BF16)
+                v = bf16_to_f32(static_cast<const uint16_t*>(table)[(int64_t)id * hidden + j]);
+            else
+                v = static_cast<const float*>(table)[(int64_t)id * hidden + j];
+        }
+        o[j] = v;
+    }
+}
+
 }  // namespace lg
 
 extern "C" logismos_status_t logismos_launch_add_rms_norm_bf16(void* h_f32, const void* y_bf16,
@@ -519,4 +542,38 @@ extern "C" logismos_status_t logismos_launch_silu_mul_f32p_xprep(const void* par
         static_cast<const float*>(parts_f32), num_parts, (int64_t)rows * 2 * inter, x_prepared, rows,
         inter);
     return hipGetLastError();
+}
+
+static logismos_status_t embed_lookup_launch(const void* table, const void* ids_u32, void* out_f32,
+                                             int rows, int hidden, int64_t vocab, bool bf16,
+                                             logismos_stream_t stream) {
+    if (rows <= 0 || hidden <= 0 || vocab <= 0 || (int64_t)rows * hidden > (int64_t)INT32_MAX)
+        return hipErrorInvalidValue;
+    if (!table || !ids_u32 || !out_f32) return hipErrorInvalidValue;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (bf16)
+        lg::embed_lookup_kernel<true><<<dim3(rows), dim3(256), 0, st>>>(
+            table, static_cast<const uint32_t*>(ids_u32), static_cast<float*>(out_f32), hidden,
+            vocab);
+    else
+        lg::embed_lookup_kernel<false><<<dim3(rows), dim3(256), 0, st>>>(
+            table, static_cast<const uint32_t*>(ids_u32), static_cast<float*>(out_f32), hidden,
+            vocab);
+    return hipGetLastError();
+}
+
+extern "C" logismos_status_t logismos_launch_embed_lookup_f32(const void* table_f32,
+                                                              const void* ids_u32, void* out_f32,
+                                                              int rows, int hidden,
+                                                              long long vocab,
+                                                              logismos_stream_t stream) {
+    return embed_lookup_launch(table_f32, ids_u32, out_f32, rows, hidden, vocab, false, stream);
+}
+
+extern "C" logismos_status_t logismos_launch_embed_lookup_bf16(const void* table_bf16,
+                                                               const void* ids_u32, void* out_f32,
+                                                               int rows, int hidden,
+                                                               long long vocab,
+                                                               logismos_stream_t stream) {
+    return embed_lookup_launch(table_bf16, ids_u32, out_f32, rows, hidden, vocab, true, stream);
 }

@@ -69,6 +69,11 @@ _SIGNATURES = {
     "logismos_launch_silu_mul_bf16": (C.c_uint32, [_vp, _vp, _i, _i, _vp]),
     "logismos_launch_cast_f16_bf16": (C.c_uint32, [_vp, _vp, _sz, _vp]),
     "logismos_launch_greedy_f32": (C.c_uint32, [_vp, _vp, _i, _i, _vp]),
+    "logismos_check_qgemm_q4g128_greedy_shape": (C.c_uint32, [_i, _i, _i, C.c_char_p, _sz]),
+    "logismos_qgemm_q4g128_greedy_workspace_bytes": (_sz, [_i, _i, _i]),
+    "logismos_launch_qgemm_q4g128_greedy_xprep": (C.c_uint32, [_vp] * 7 + [_i, _i, _i, _vp]),
+    "logismos_launch_embed_lookup_f32": (C.c_uint32, [_vp, _vp, _vp, _i, _i, C.c_longlong, _vp]),
+    "logismos_launch_embed_lookup_bf16": (C.c_uint32, [_vp, _vp, _vp, _i, _i, C.c_longlong, _vp]),
     "logismos_decode_step_workspace_bytes": (_sz, [_vp, _i, _i]),
     "logismos_launch_decode_step": (C.c_uint32, [_vp, _vp, _vp, _vp, _vp]),
     "logismos_qgemm_q4g128_splitk_parts": (C.c_int, [_i, _i, _i]),
@@ -123,7 +128,7 @@ class Q4Weight(C.Structure):
 class DecodeConfig(C.Structure):
     _fields_ = [("num_layers", _i), ("hidden", _i), ("num_q_heads", _i), ("num_kv_heads", _i),
                 ("head_dim", _i), ("intermediate", _i), ("rms_eps", _f), ("block_size", _i),
-                ("max_blocks_per_seq", _i), ("max_pos", _i)]
+                ("max_blocks_per_seq", _i), ("max_pos", _i), ("vocab", _i)]
 
 
 class DecodeLayer(C.Structure):
@@ -136,7 +141,9 @@ class DecodeBatch(C.Structure):
     _fields_ = [("hidden_f32", _vp), ("out_bf16", _vp), ("final_norm_w_f32", _vp),
                 ("block_tables", _vp), ("cu_seqlens", _vp), ("context_lens", _vp),
                 ("positions", _vp), ("slot_mapping", _vp), ("rope_cos_f32", _vp),
-                ("rope_sin_f32", _vp), ("num_seqs", _i), ("num_splits", _i)]
+                ("rope_sin_f32", _vp), ("num_seqs", _i), ("num_splits", _i),
+                ("token_ids", _vp), ("embed_table_bf16", _vp), ("lm_head", C.POINTER(Q4Weight)),
+                ("out_tokens_u32", _vp), ("logits_f32", _vp)]
 
 
 def library() -> C.CDLL:
@@ -344,6 +351,31 @@ def launch_cast_f16_bf16(src, dst, count: int, stream=None) -> None:
 def launch_greedy_f32(logits, out, rows: int, n: int, stream=None) -> None:
     _status("greedy_f32", library().logismos_launch_greedy_f32(
         _ptr(logits), _ptr(out), rows, n, _raw(stream)))
+
+
+def check_qgemm_q4g128_greedy_shape(b: int, n: int, k: int) -> None:
+    _guard("qgemm_q4g128_greedy", library().logismos_check_qgemm_q4g128_greedy_shape, b, n, k)
+
+
+def qgemm_q4g128_greedy_workspace_bytes(b: int, n: int, k: int) -> int:
+    return library().logismos_qgemm_q4g128_greedy_workspace_bytes(b, n, k)
+
+
+def launch_qgemm_q4g128_greedy_xprep(x_prepared, qw, scale, zero, out_tokens, logits, workspace,
+                                     b: int, n: int, k: int, stream=None) -> None:
+    """Vocabulary projection + greedy token per batch row; `logits` may be None."""
+    check_qgemm_q4g128_greedy_shape(b, n, k)
+    _status("qgemm_q4g128_greedy", library().logismos_launch_qgemm_q4g128_greedy_xprep(
+        _ptr(x_prepared), _ptr(qw), _ptr(scale), _ptr(zero), _ptr(out_tokens),
+        _ptr(logits) if logits is not None else None, _ptr(workspace), b, n, k, _raw(stream)))
+
+
+def launch_embed_lookup(table, ids, out, rows: int, hidden: int, vocab: int, bf16: bool,
+                        stream=None) -> None:
+    fn = (library().logismos_launch_embed_lookup_bf16 if bf16
+          else library().logismos_launch_embed_lookup_f32)
+    _status("embed_lookup", fn(_ptr(table), _ptr(ids), _ptr(out), rows, hidden, vocab,
+                               _raw(stream)))
 
 
 def decode_step_workspace_bytes(cfg: DecodeConfig, num_seqs: int, num_splits: int) -> int:

@@ -83,11 +83,18 @@ def decode_step(cfg, layers, batch, trace=None):
     layers: list of dict(norm1, qkv, o, norm2, gate_up, down, k_pool, v_pool); each weight a
             (qw, scale, zero) triple; pools are updated in place
     batch:  dict(h [B, hidden] fp32 (updated in place), block_tables, cu_seqlens, context_lens,
-            positions, slots, cos, sin, final_norm)
+            positions, slots, cos, sin, final_norm); optionally token_ids (uint32 [B]) with
+            embed_table (bf16 bits [vocab, hidden]): h is first filled by `embed_lookup`; and
+            lm_head (a Q4G128 triple [vocab, hidden]): the step ends with the vocabulary
+            projection and `greedy`, leaving batch["logits"] (fp32) and batch["tokens"]
     Returns the final normed hidden state as bf16 bits.
     """
     b = batch["h"].shape[0]
     h = batch["h"]
+    if batch.get("token_ids") is not None:
+        vocab, hidden = batch["embed_table"].shape
+        table = O.bf16_bits_to_f32(batch["embed_table"])
+        h[:] = O.embed_lookup(table, hidden, vocab, batch["token_ids"]).reshape(b, hidden)
     y = None
     for li, L in enumerate(layers):
         xn = add_rms_norm_bf16(h, y, L["norm1"], cfg["eps"])
@@ -106,4 +113,8 @@ def decode_step(cfg, layers, batch, trace=None):
         if trace is not None:
             trace.append(dict(xn=xn, qkv=qkv, q=q16, attn=attn, o=o, xn2=xn2, gu=gu, act=act,
                               down=y, h=h.copy()))
-    return add_rms_norm_bf16(h, y, batch["final_norm"], cfg["eps"])
+    out = add_rms_norm_bf16(h, y, batch["final_norm"], cfg["eps"])
+    if batch.get("lm_head") is not None:
+        batch["logits"] = _gemm(out, batch["lm_head"], b)
+        batch["tokens"] = np.array([O.greedy(r) for r in batch["logits"]], np.uint32)
+    return out

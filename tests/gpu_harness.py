@@ -2,6 +2,8 @@
 calls the C-ABI launchers, downloads results."""
 from __future__ import annotations
 
+import ctypes as C
+
 import numpy as np
 
 from logismos_amd import hip, kernels
@@ -98,7 +100,8 @@ class DecodeStepRunner:
         half = cfg["d"] // 2
         self.cfg = kernels.DecodeConfig(len(layers), cfg["hidden"], cfg["hq"], cfg["hkv"], cfg["d"],
                                         cfg["inter"], cfg["eps"], cfg["block_size"], max_blocks,
-                                        batch["cos"].size // half)
+                                        batch["cos"].size // half,
+                                        batch["lm_head"][0].shape[0] if "lm_head" in batch else 0)
         up = hip.DeviceBuffer.from_numpy
         self.keep = []
 
@@ -159,6 +162,21 @@ class DecodeStepRunner:
             _val(self.idx["cu_seqlens"]), _val(self.idx["context_lens"]),
             _val(self.idx["positions"]), _val(self.slots), _val(self.cos), _val(self.sin), b,
             self.num_splits)
+        self.vocab = self.cfg.vocab
+        if self.vocab:
+            # tokens in (embedding lookup) and tokens out (vocabulary projection + greedy)
+            self.token_ids = up(np.ascontiguousarray(batch["token_ids"], np.uint32))
+            self.embed = up(np.ascontiguousarray(batch["embed_table"], np.uint16))
+            self.head = w3(batch["lm_head"])
+            self.tokens = hip.DeviceBuffer(b * 4)
+            self.tokens.fill(0xFF)
+            self.logits = hip.DeviceBuffer(b * self.vocab * 4)
+            self.logits.fill(0xFF)
+            self.batch.token_ids = _val(self.token_ids)
+            self.batch.embed_table_bf16 = _val(self.embed)
+            self.batch.lm_head = C.pointer(self.head)
+            self.batch.out_tokens_u32 = _val(self.tokens)
+            self.batch.logits_f32 = _val(self.logits)
         ws = kernels.decode_step_workspace_bytes(self.cfg, b, self.num_splits)
         assert ws > 0
         self.ws = hip.DeviceBuffer(ws)
@@ -170,6 +188,12 @@ class DecodeStepRunner:
     def result_bits(self) -> np.ndarray:
         (self.stream.synchronize() if self.stream else hip.synchronize())
         return self.out.to_numpy(np.uint16, (self.b, self.cfg_d["hidden"]))
+
+    def result_tokens(self):
+        """(tokens uint32 [B], logits fp32 [B, vocab]) of a step with an lm_head."""
+        (self.stream.synchronize() if self.stream else hip.synchronize())
+        return (self.tokens.to_numpy(np.uint32, (self.b,)),
+                self.logits.to_numpy(np.float32, (self.b, self.vocab)))
 
 
 def assert_parity(got, want, max_abs=2e-3, max_rel=1e-2, what=""):

@@ -67,3 +67,43 @@ def test_step_is_deterministic_and_split_invariant():
     _, c, _, _, _ = _run_both(cfg, layers, batch, num_splits=8)
     assert np.array_equal(a, b)
     assert _rel_l2(c, a) < 5e-3
+
+
+def test_tokens_in_tokens_out():
+    # embedding lookup in front, vocabulary projection + greedy behind: token ids to token ids
+    rng = np.random.default_rng(34)
+    vocab = 5003
+    cfg, layers, batch = workloads.decode_step_problem(
+        rng, num_layers=2, hidden=1024, hq=8, hkv=2, inter=2048, ctx=[1, 17, 300, 64, 999, 5],
+        vocab=vocab)
+    batch["token_ids"][3] = vocab  # outside the vocabulary: a zero embedding row
+    r, got, want, lay, bat = _run_both(cfg, layers, batch)
+    assert _rel_l2(got, want) < 5e-3
+    tokens, logits = r.result_tokens()
+    assert np.isfinite(logits).all()
+    assert _rel_l2(logits, bat["logits"]) < 6e-3
+    # the selection rule exactly, on the logits the step stored
+    assert np.array_equal(tokens, np.array([O.greedy(x) for x in logits], np.uint32))
+    # and the oracle's token wherever its winner is clear of the logit error
+    err = float(np.abs(logits - bat["logits"]).max())
+    top2 = np.sort(bat["logits"], axis=1)[:, -2:]
+    clear = (top2[:, 1] - top2[:, 0]) > 4 * err
+    assert clear.any()
+    assert np.array_equal(tokens[clear], bat["tokens"][clear])
+    h_gpu = r.h.to_numpy(np.float32, bat["h"].shape)
+    assert _rel_l2(h_gpu, bat["h"]) < 5e-3
+
+
+def test_tokens_out_without_the_bf16_state_or_logits():
+    rng = np.random.default_rng(35)
+    cfg, layers, batch = workloads.decode_step_problem(
+        rng, num_layers=1, hidden=1024, hq=8, hkv=2, inter=2048, ctx=[40, 7, 129], vocab=3000)
+    full = DecodeStepRunner(cfg, layers, batch)
+    full.launch()
+    want, _ = full.result_tokens()
+    lean = DecodeStepRunner(cfg, layers, batch)
+    lean.batch.out_bf16 = None
+    lean.batch.logits_f32 = None
+    lean.launch()
+    got, _ = lean.result_tokens()
+    assert np.array_equal(got, want)
