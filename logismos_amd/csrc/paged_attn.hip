@@ -719,25 +719,28 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams 
 // The C layout of S^T (lane (hl, c): keys 8g + 4hl + i of column c) is, read as
 // "slot e = 4*(g%2) + i of MFMA g/2", already a B-operand layout, so P never
 // leaves its lane; V is written to LDS transposed ([d][key], two keys per
-// 32-bit store) so that the matching A operand is two 8-byte reads.
+// 32-bit store, keys in P's slot order) so that the matching A operand is one
+// 16-byte read.
 //
-// Schedule of one iteration (tile t): request K rows of tile t+3 / V rows of tile
-// t+2 from memory; issue the MFMAs of S(t+1); read V(t) from LDS; softmax of S(t)
-// on the VALU while those MFMAs run; O += P.V(t); write K(t+2) / V(t+1) to LDS;
-// barrier.  K therefore runs one tile ahead of V in the two-deep LDS rings.
-// Waves 0-3 move K, waves 4-7 move V.  The softmax maximum is updated lazily (see
-// kLazyLog2), which makes accumulator rescaling rare.
+// Schedule of one step (tile t): request K rows of tile t+3 / V rows of tile t+1
+// from memory; then, in one block of interleaved instructions, the MFMAs of
+// S(t+1) and of O += P(t-1).V(t-1) with the softmax of S(t) between them (the
+// MFMAs of a step do not depend on its VALU work); write K(t+2) / V(t) to LDS;
+// barrier.  The LDS rings are two deep.  Waves 0-3 move K, waves 4-7 move V.
+// The softmax maximum is updated lazily (see kLazyLog2), which makes accumulator
+// rescaling rare.
 // grid (hkv, query tiles, num_seqs): with hkv a multiple of 8 every XCD (and its
 // L2) serves the same KV heads for all query tiles; later query tiles (more
 // visible keys under the causal mask) are dispatched first.
 constexpr int kPfKeys = 32;
 constexpr int kPfWaves = 8;
 constexpr int kKsStride = kHeadDim + 8;  // halfs per K row in LDS (272 B)
-constexpr int kVtStride = kPfKeys + 4;   // halfs per V^T row in LDS (72 B)
+constexpr int kVtStride = kPfKeys + 8;   // halfs per V^T row in LDS (80 B: 16-byte reads stay aligned)
 constexpr int kKsElems = kPfKeys * kKsStride;
 constexpr int kVtElems = kHeadDim * kVtStride;
 constexpr int kStageStride = kHeadDim + 8;
 constexpr float kLazyLog2 = 8.0f;  // headroom of the lazily updated softmax maximum
+constexpr int kPfRankMax = 512;    // sequences ordered by length inside the kernel
 
 struct PfRegs {
     uint4_t x[2];  // the two keys of this thread's pair
@@ -755,7 +758,38 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
     const int hl = lane >> 5;
     const int c = lane & 31;
     const int kvh = blockIdx.x;
-    const int s = blockIdx.z;
+
+    // ---- which sequence this workgroup takes.  Workgroups start in the order of their
+    // linear index and a CU takes the next one when it is done, so long sequences should
+    // come first: blockIdx.z picks the sequence whose context has that rank in descending
+    // order.  The query tiles of a sequence stay adjacent (blockIdx.y, later tiles first):
+    // they stream the same keys at about the same time and share them in L2 -- ordering
+    // single (sequence, tile) items by length balanced as well but ran 13 % slower.
+    // (16 chunks of 512 tokens, prior contexts 0..8192: in grid order the last CU ends 24 %
+    // after the average one, in this order 1 %.)  More sequences than kPfRankMax: grid order.
+    int pick = blockIdx.z;
+    if ((int)gridDim.z <= kPfRankMax) {
+        __shared__ int rank_keys[kPfRankMax];
+        __shared__ int rank_pick;
+        const int nseq = gridDim.z;
+        if (tid < nseq)
+            rank_keys[tid] = (p.cu_seqlens_q[tid + 1] - p.cu_seqlens_q[tid] > 1)
+                                 ? max(p.context_lens[tid], 0) + 1
+                                 : 0;
+        __syncthreads();
+        if (tid < nseq) {
+            const int mine = rank_keys[tid];
+            int rank = 0;
+            for (int j = 0; j < nseq; ++j) {
+                const int other = rank_keys[j];
+                rank += (other > mine || (other == mine && j < tid)) ? 1 : 0;
+            }
+            if (rank == pick) rank_pick = tid;
+        }
+        __syncthreads();
+        pick = rank_pick;
+    }
+    const int s = __builtin_amdgcn_readfirstlane(pick);
 
     const int t0 = p.cu_seqlens_q[s];
     const int n_new = p.cu_seqlens_q[s + 1] - t0;
@@ -848,6 +882,9 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
             r.x[u] = *reinterpret_cast<const uint4_t*>(pb + off);
         }
     };
+    // column (in halfs) of this thread's key pair inside a V^T row (see lstore)
+    const int vt_pos = ((2 * kp) & ~12) | (((2 * kp) & 4) << 1) | (((2 * kp) & 8) >> 1);
+    const int vt_col = 8 * ((vt_pos >> 3) ^ ((piece >> 1) & 3)) + (vt_pos & 7);
     // K rows as they are; V transposed, (key 2kp, key 2kp+1) of element e as one word
     auto lstore = [&](int buf, const PfRegs& r) {
         if (!moves_v) {
@@ -856,12 +893,16 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
             for (int u = 0; u < 2; ++u)
                 *reinterpret_cast<uint4_t*>(ks + (2 * kp + u) * kKsStride + 8 * piece) = r.x[u];
         } else {
-            _Float16* vt = Vt + buf * kVtElems;
+            // Key k of a 16-key slab sits at position swap(bit 2, bit 3) of k, the order in
+            // which the P operand holds it, so that a lane's 8 keys are one 16-byte read; the
+            // four 16-byte chunks of a row are XOR-swizzled by (row / 16) % 4, which makes
+            // these transposed 4-byte stores two-way instead of eight-way bank conflicts
+            _Float16* vt = Vt + buf * kVtElems + vt_col;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const unsigned sel = (e & 1) ? 0x07060302u : 0x05040100u;
                 const unsigned pr = __builtin_amdgcn_perm(r.x[1][e >> 1], r.x[0][e >> 1], sel);
-                *reinterpret_cast<unsigned*>(vt + (8 * piece + e) * kVtStride + 2 * kp) = pr;
+                *reinterpret_cast<unsigned*>(vt + (8 * piece + e) * kVtStride) = pr;
             }
         }
     };
@@ -873,51 +914,78 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.0f;
 
-    // S^T of one key tile: K from LDS as the A operand
-    auto qk = [&](int buf) {
-        const _Float16* ks = Ks + buf * kKsElems + c * kKsStride + 8 * hl;
-        half8_t ka[8];
+    // The three stages of a key tile t -- S(t) = K.Q^T on the matrix pipe, F(t) the online
+    // softmax on the VALU, O(t) = V^T.P on the matrix pipe -- run software-pipelined: step t
+    // issues S(t+1) and O(t-1) around F(t), so the MFMAs of a step do not depend on its VALU
+    // work and the two can be interleaved instruction by instruction inside ONE wave (the
+    // waves of a workgroup move in lock-step between barriers and cannot hide each other's
+    // phases).  P(t-1) and the operands are carried in registers from step to step.
+    half8_t p_prev[2];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) ka[j] = *reinterpret_cast<const half8_t*>(ks + 16 * j);
+    for (int kh = 0; kh < 2; ++kh) p_prev[kh] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    float16_t s_cur;
+    // lane part of a V^T operand address: row c of a 32-row block, the lane's half of a
+    // 16-key slab, under the chunk swizzle of lstore
+    const int vt_lane = c * kVtStride + 8 * (hl ^ (c >> 4));
+
+    // S^T of the first key tile (the steps compute every later one)
+    auto qk_first = [&]() {
+        const _Float16* ks = Ks + c * kKsStride + 8 * hl;
         float16_t sacc;
 #pragma unroll
         for (int r = 0; r < 16; ++r) sacc[r] = 0.0f;
 #pragma unroll
         for (int j = 0; j < 8; ++j)
-            sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[j], qreg[j], sacc, 0, 0, 0);
+            sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                *reinterpret_cast<const half8_t*>(ks + 16 * j), qreg[j], sacc, 0, 0, 0);
         return sacc;
     };
-    struct VTile {
-        half8_t a[4][2];
-    };
-    auto vread = [&](int buf, VTile& v) {
-        const _Float16* vt = Vt + buf * kVtElems + c * kVtStride + 4 * hl;
+    // O += V^T(buffer buf) . P
+    auto pv_from = [&](int buf, const half8_t (&pb)[2]) {
+        const _Float16* vt = Vt + buf * kVtElems + vt_lane;
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+        for (int kh = 0; kh < 2; ++kh)
 #pragma unroll
-            for (int kh = 0; kh < 2; ++kh) {
-                const _Float16* vp = vt + 32 * dt * kVtStride + 16 * kh;
-                const half4_t v0 = *reinterpret_cast<const half4_t*>(vp);
-                const half4_t v1 = *reinterpret_cast<const half4_t*>(vp + 8);
-                v.a[dt][kh] = half8_t{v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-            }
+            for (int dt = 0; dt < 4; ++dt)
+                oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                    *reinterpret_cast<const half8_t*>(vt + 32 * dt * kVtStride +
+                                                      16 * (kh ^ (dt & 1))),
+                    pb[kh], oacc[dt], 0, 0, 0);
     };
-    // online softmax of one score tile; returns P as the two B operands of P.V
-    auto softmax = [&](int tile, const float16_t& sacc, half8_t (&pb)[2]) {
+    // One step: tile t with S(t) in s_cur; K(t+1) in K buffer 1-H, V(t-1) in V buffer 1-H.
+    // Leaves S(t+1) in s_cur and P(t) in p_prev.  MASKED: some column may not see all keys
+    // of the tile (then the mask costs 48 VALU instructions and a branch splits the block).
+    auto step = [&](auto masked_c, auto h_c, int tile) {
+        constexpr bool MASKED = decltype(masked_c)::value != 0;
+        constexpr int H = decltype(h_c)::value;
+        const _Float16* ks = Ks + (1 - H) * kKsElems + c * kKsStride + 8 * hl;
+        const _Float16* vt = Vt + (1 - H) * kVtElems + vt_lane;
+        // operands in the order the MFMAs below take them
+        half8_t ka[8], va[2][4];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            ka[j] = *reinterpret_cast<const half8_t*>(ks + 16 * j);
+            va[j >> 2][j & 3] = *reinterpret_cast<const half8_t*>(
+                vt + 32 * (j & 3) * kVtStride + 16 * ((j >> 2) ^ (j & 1)));
+        }
+
+        // ---- F(t), first part: tile maximum and the lazily raised reference maximum
         const int key0 = tile * kPfKeys;
         float sc[16];
         float tm = -INFINITY;
-        if (key0 + kPfKeys > wave_min) {  // some column of this wave may be masked here
+        bool plain = true;
+        if constexpr (MASKED) plain = key0 + kPfKeys <= wave_min;
+        if (plain) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int key = key0 + 8 * (r >> 2) + 4 * hl + (r & 3);
-                sc[r] = key < col_lim ? sacc[r] : -INFINITY;
+                sc[r] = s_cur[r];
                 tm = fmaxf(tm, sc[r]);
             }
         } else {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                sc[r] = sacc[r];
+                const int key = key0 + 8 * (r >> 2) + 4 * hl + (r & 3);
+                sc[r] = key < col_lim ? s_cur[r] : -INFINITY;
                 tm = fmaxf(tm, sc[r]);
             }
         }
@@ -927,40 +995,66 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
         // 2^kLazyLog2, well inside fp16 and fp32 range), so the accumulators are rescaled
         // a few times per column instead of per tile.
         const bool raise = tm > m + kLazyLog2;
-        if (__builtin_expect(__builtin_amdgcn_ballot_w64(raise) != 0, 0)) {
-            const float alpha = raise ? fast_exp2(m - tm) : 1.0f;
-            m = raise ? tm : m;
-            l *= alpha;
-#pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
-        }
+        const float alpha = raise ? fast_exp2(m - tm) : 1.0f;
+        m = raise ? tm : m;
         const float nm = (m == -INFINITY) ? 0.0f : -m;
+
+        // ---- S(t+1) and O(t-1) on the matrix pipe (alternating: consecutive MFMAs are
+        // independent), the exponentials of F(t) on the VALU
+        float16_t s_nxt;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s_nxt[r] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            s_nxt = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[j], qreg[j], s_nxt, 0, 0, 0);
+            oacc[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[j >> 2][j & 3], p_prev[j >> 2],
+                                                                 oacc[j & 3], 0, 0, 0);
+        }
         float psum = 0.0f;
+        half8_t pb[2];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const float pv = fast_exp2(fmaf(sc[r], p.scale_log2e, nm));
             psum += pv;
             pb[r >> 3][r & 7] = (_Float16)pv;
         }
-        l += psum;
-    };
-    auto pv = [&](const VTile& v, const half8_t (&pb)[2]) {
+        l = fmaf(l, alpha, psum);
+        if constexpr (!MASKED) {
+            // Order of the block: the first eight operand reads, then 16 MFMAs, each followed
+            // by the read of the operand eight MFMAs ahead (into the registers just freed) and
+            // by its share of the VALU work
+            __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+            for (int g = 0; g < 16; ++g) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                if (g < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+            }
+        }
+        // keep F(t) in this block: its results are only used by the next step, and the
+        // compiler would otherwise sink the exponentials out from under the MFMAs
+        asm volatile("" : "+v"(pb[0]), "+v"(pb[1]), "+v"(l));
+        // O(t-1) was accumulated relative to the old reference: rescale after it
+        if (__builtin_expect(__builtin_amdgcn_ballot_w64(raise) != 0, 0)) {
 #pragma unroll
-            for (int kh = 0; kh < 2; ++kh)
-                oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(v.a[dt][kh], pb[kh], oacc[dt], 0, 0, 0);
+            for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+        }
+        s_cur = s_nxt;
+        p_prev[0] = pb[0];
+        p_prev[1] = pb[1];
     };
 
     // The body is straight-line for two tiles (tiles past the end repeat clamped loads and
     // are fully masked), which keeps the wait counts exact.  Every wave does the math of
     // every tile of the workgroup (a tile beyond a wave's own columns is fully masked
-    // there): the waves meet at the barrier anyway.
+    // there): the waves meet at the barrier anyway.  Tiles that every query of the
+    // workgroup sees in full come first and take the unmasked step.
     if (ntiles > 0) {
         PfRegs ra, rb;
-        // K waves start one tile ahead of V waves
+        // K is stored two tiles ahead of the step that multiplies it, V in the step that
+        // precedes its use
         {
             PfAddr a = next_addr();
             gload(a, ra);
@@ -971,42 +1065,39 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
                 lstore(1, rb);
                 a = next_addr();
                 gload(a, ra);  // K(2) in flight
-            } else {
-                lstore(0, ra);
-                a = next_addr();
-                gload(a, ra);  // V(1) in flight
             }
+            // V buffer 1 plays V(-1) in the first step (P(-1) = 0): finite values
+            unsigned* vz = reinterpret_cast<unsigned*>(Vt + kVtElems);
+            for (int i = tid; i < kVtElems / 2; i += 64 * kPfWaves) vz[i] = 0u;
         }
         PfAddr an = next_addr();
         __syncthreads();
-        float16_t s_cur = qk(0);
-        for (int tile = 0; tile < ntiles; tile += 2) {
-            // ---- tile (K(tile+1) in K buffer 1, V(tile) in V buffer 0)
+        s_cur = qk_first();
+        const int plain_tiles = min(ntiles, limit_of(i0) / kPfKeys) & ~1;
+        auto two_steps = [&](auto masked_c, int tile) {
+            // ---- tile: K(tile+3) / V(tile+1) requested, K(tile+2) / V(tile) to buffer 0
             PfAddr an2 = next_addr();
-            gload(an, rb);  // K(tile+3) / V(tile+2)
+            gload(an, rb);
             __builtin_amdgcn_sched_barrier(0);
-            float16_t s_nxt = qk(1);
-            VTile v;
-            vread(0, v);
-            half8_t pb[2];
-            softmax(tile, s_cur, pb);
-            pv(v, pb);
+            step(masked_c, ic<0>{}, tile);
             __builtin_amdgcn_sched_barrier(0);
-            // K(tile+2) -> K buffer 0, V(tile+1) -> V buffer 1
-            lstore(moves_v ? 1 : 0, ra);
+            lstore(0, ra);
             __syncthreads();
-            // ---- tile + 1 (K(tile+2) in K buffer 0, V(tile+1) in V buffer 1)
+            // ---- tile + 1: K(tile+4) / V(tile+2) requested, K(tile+3) / V(tile+1) to buffer 1
             an = next_addr();
-            gload(an2, ra);  // K(tile+4) / V(tile+3)
+            gload(an2, ra);
             __builtin_amdgcn_sched_barrier(0);
-            s_cur = qk(0);
-            vread(1, v);
-            softmax(tile + 1, s_nxt, pb);
-            pv(v, pb);
+            step(masked_c, ic<1>{}, tile + 1);
             __builtin_amdgcn_sched_barrier(0);
-            lstore(moves_v ? 0 : 1, rb);
+            lstore(1, rb);
             __syncthreads();
-        }
+        };
+        int tile = 0;
+        for (; tile < plain_tiles; tile += 2) two_steps(ic<0>{}, tile);
+        for (; tile < ntiles; tile += 2) two_steps(ic<1>{}, tile);
+        // the last tile's O: its V went to buffer 1 in the last step
+        pv_from(1, p_prev);
+        __syncthreads();  // the staging below reuses the K / V buffers
     }
 
     // ---- normalise, stage through this wave's LDS slice (16 columns at a time), write
