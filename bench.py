@@ -508,62 +508,64 @@ def bench_decode_step(args):
     stream.synchronize()
     del cal
 
-    # ---- the same step as a closed loop over token ids: embedding lookup in front, the
-    # vocabulary projection (151936 x 4096, Q4G128) with the greedy choice fused behind, the
-    # chosen tokens being the next step's input.  Reported beside the headline figure, which
-    # stays the 36 layers alone.
-    vocab = 151936
-    hq4 = (rng.integers(0, 256, size=(vocab, hidden // 2), dtype=np.uint8),
-           (rng.random((vocab, hidden // 128), np.float32) * 0.004 + 0.004).astype(np.float16),
-           (rng.random((vocab, hidden // 128), np.float32) * 2 + 6.5).astype(np.float16))
-    head_bufs = [hip.DeviceBuffer.from_numpy(hq4[0]),
-                 hip.DeviceBuffer.from_numpy(hq4[1].view(np.uint16)),
-                 hip.DeviceBuffer.from_numpy(hq4[2].view(np.uint16))]
-    head_bytes = sum(int(a.nbytes) for a in hq4)
-    del hq4
-    head = kernels.Q4Weight(*[hb.ptr.value for hb in head_bufs])
-    d_embed = hip.DeviceBuffer(vocab * hidden * 2)
-    d_embed.fill(0x3C)   # every entry the bf16 0x3C3C; the lookup's traffic does not depend on it
-    d_tok = hip.DeviceBuffer.from_numpy(rng.integers(0, vocab, size=S, dtype=np.uint32))
-    r.cfg.vocab = vocab
-    r.ws = hip.DeviceBuffer(kernels.decode_step_workspace_bytes(r.cfg, S, r.num_splits))
-    r.batch.token_ids = d_tok.ptr.value
-    r.batch.embed_table_bf16 = d_embed.ptr.value
-    r.batch.lm_head = C.pointer(head)
-    r.batch.out_tokens_u32 = d_tok.ptr.value   # fed back: read by the next step's lookup
-    g2 = hip.Graph(stream)
-    with g2:
-        kernels.launch_pack_ragged(d_ones, d_cur_prior, r.idx["block_tables"],
-                                   r.idx["cu_seqlens"], r.slots, r.idx["context_lens"], S, bs,
-                                   max_blocks, stream)
-        r.launch()
-    for i in range(warmup):
-        one_step(i, g2)
-    stream.synchronize()
-    e0.record(stream)
-    for i in range(steps):
-        one_step(warmup + i, g2)
-    e1.record(stream)
-    e1.synchronize()
-    ms_loop = e0.elapsed_ms(e1) / steps
-    toks = d_tok.to_numpy(np.uint32, (S,))
-    assert (toks < vocab).all()
-    # the vocabulary projection alone (its 330 MB exceed the 256 MB cache: every launch is cold)
-    d_xp = hip.DeviceBuffer(kernels.q4_xprep_bytes(S, hidden))
-    d_xp.fill(0x3C)
-    d_hws = hip.DeviceBuffer(kernels.qgemm_q4g128_greedy_workspace_bytes(S, vocab, hidden))
-    d_t2 = hip.DeviceBuffer(S * 4)
-    ms_head, _, _ = time_launches(
-        stream, [lambda: kernels.launch_qgemm_q4g128_greedy_xprep(
-            d_xp, head_bufs[0], head_bufs[1], head_bufs[2], d_t2, None, d_hws, S, vocab, hidden,
-            stream)], 40, 4)
-    closed_loop = {
-        "what": "token ids in, token ids out: embed_lookup + 36 layers + lm_head 151936x4096 "
-                "Q4G128 with greedy fused, chosen tokens fed back on the GPU",
-        "ms_per_step": round(ms_loop, 4), "tok_s": round(S / (ms_loop * 1e-3), 1),
-        "lm_head_bytes": head_bytes, "lm_head_greedy_us": round(ms_head * 1e3, 1),
-        "lm_head_GBps": round(head_bytes / (ms_head * 1e-3) / 1e9, 1)}
-    del d_embed, head_bufs
+    closed_loop = None
+    if not args.skip_closed_loop:
+        # ---- the same step as a closed loop over token ids: embedding lookup in front, the
+        # vocabulary projection (151936 x 4096, Q4G128) with the greedy choice fused behind, the
+        # chosen tokens being the next step's input.  Reported beside the headline figure, which
+        # stays the 36 layers alone.
+        vocab = 151936
+        hq4 = (rng.integers(0, 256, size=(vocab, hidden // 2), dtype=np.uint8),
+               (rng.random((vocab, hidden // 128), np.float32) * 0.004 + 0.004).astype(np.float16),
+               (rng.random((vocab, hidden // 128), np.float32) * 2 + 6.5).astype(np.float16))
+        head_bufs = [hip.DeviceBuffer.from_numpy(hq4[0]),
+                     hip.DeviceBuffer.from_numpy(hq4[1].view(np.uint16)),
+                     hip.DeviceBuffer.from_numpy(hq4[2].view(np.uint16))]
+        head_bytes = sum(int(a.nbytes) for a in hq4)
+        del hq4
+        head = kernels.Q4Weight(*[hb.ptr.value for hb in head_bufs])
+        d_embed = hip.DeviceBuffer(vocab * hidden * 2)
+        d_embed.fill(0x3C)   # every entry the bf16 0x3C3C; the lookup's traffic does not depend on it
+        d_tok = hip.DeviceBuffer.from_numpy(rng.integers(0, vocab, size=S, dtype=np.uint32))
+        r.cfg.vocab = vocab
+        r.ws = hip.DeviceBuffer(kernels.decode_step_workspace_bytes(r.cfg, S, r.num_splits))
+        r.batch.token_ids = d_tok.ptr.value
+        r.batch.embed_table_bf16 = d_embed.ptr.value
+        r.batch.lm_head = C.pointer(head)
+        r.batch.out_tokens_u32 = d_tok.ptr.value   # fed back: read by the next step's lookup
+        g2 = hip.Graph(stream)
+        with g2:
+            kernels.launch_pack_ragged(d_ones, d_cur_prior, r.idx["block_tables"],
+                                       r.idx["cu_seqlens"], r.slots, r.idx["context_lens"], S, bs,
+                                       max_blocks, stream)
+            r.launch()
+        for i in range(warmup):
+            one_step(i, g2)
+        stream.synchronize()
+        e0.record(stream)
+        for i in range(steps):
+            one_step(warmup + i, g2)
+        e1.record(stream)
+        e1.synchronize()
+        ms_loop = e0.elapsed_ms(e1) / steps
+        toks = d_tok.to_numpy(np.uint32, (S,))
+        assert (toks < vocab).all()
+        # the vocabulary projection alone (its 330 MB exceed the 256 MB cache: every launch is cold)
+        d_xp = hip.DeviceBuffer(kernels.q4_xprep_bytes(S, hidden))
+        d_xp.fill(0x3C)
+        d_hws = hip.DeviceBuffer(kernels.qgemm_q4g128_greedy_workspace_bytes(S, vocab, hidden))
+        d_t2 = hip.DeviceBuffer(S * 4)
+        ms_head, _, _ = time_launches(
+            stream, [lambda: kernels.launch_qgemm_q4g128_greedy_xprep(
+                d_xp, head_bufs[0], head_bufs[1], head_bufs[2], d_t2, None, d_hws, S, vocab, hidden,
+                stream)], 40, 4)
+        closed_loop = {
+            "what": "token ids in, token ids out: embed_lookup + 36 layers + lm_head 151936x4096 "
+                    "Q4G128 with greedy fused, chosen tokens fed back on the GPU",
+            "ms_per_step": round(ms_loop, 4), "tok_s": round(S / (ms_loop * 1e-3), 1),
+            "lm_head_bytes": head_bytes, "lm_head_greedy_us": round(ms_head * 1e3, 1),
+            "lm_head_GBps": round(head_bytes / (ms_head * 1e-3) / 1e9, 1)}
+        del d_embed, head_bufs
 
     per_layer_w = sum(int(np.asarray(t[0]).nbytes + np.asarray(t[1]).nbytes +
                           np.asarray(t[2]).nbytes)
@@ -615,6 +617,9 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=5.0)
     ap.add_argument("--skip-kernels", action="store_true",
                     help="only the decode-step line, without the per-kernel legs")
+    ap.add_argument("--skip-closed-loop", action="store_true",
+                    help="leave out the token-ids-in / token-ids-out leg of the decode step "
+                         "(embedding, lm_head + greedy); profiling runs use this")
     ap.add_argument("--workload", default="all",
                     choices=["all", "step", "config1", "config2", "config3", "config4"],
                     help="all: the decode-step line with every leg inside it (default); "

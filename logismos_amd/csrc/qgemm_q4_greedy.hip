@@ -232,18 +232,29 @@ __global__ __launch_bounds__(64 * kGreedyWaves) void qgemm_q4g128_greedy_kernel(
 }
 
 // token[r] = index of the best candidate over the workers; a row whose logits never exceeded
-// -inf (all -inf or NaN) gives 0, like the CPU loop that never updates.
-__global__ __launch_bounds__(64) void greedy_pick_kernel(const float* __restrict__ best_val,
-                                                         const int* __restrict__ best_idx,
-                                                         uint32_t* __restrict__ out, int b, int bp,
-                                                         int workers) {
-    const int r = threadIdx.x;
-    if (r >= b) return;
+// -inf (all -inf or NaN) gives 0, like the CPU loop that never updates.  One workgroup: thread
+// (g = t / bp, r = t % bp) folds workers g, g + groups, ...; the groups are folded through LDS.
+constexpr int kPickThreads = 1024;
+
+__global__ __launch_bounds__(kPickThreads) void greedy_pick_kernel(
+    const float* __restrict__ best_val, const int* __restrict__ best_idx,
+    uint32_t* __restrict__ out, int b, int bp, int workers) {
+    __shared__ float sv[kPickThreads];
+    __shared__ int si[kPickThreads];
+    const int r = threadIdx.x % bp;
+    const int g = threadIdx.x / bp;
+    const int groups = kPickThreads / bp;
     float v = -INFINITY;
     int i = kNoIndex;
-    for (int w = 0; w < workers; ++w)
+    for (int w = g; w < workers; w += groups)
         take_better(v, i, best_val[(int64_t)w * bp + r], best_idx[(int64_t)w * bp + r]);
-    out[r] = i == kNoIndex ? 0u : (uint32_t)i;
+    sv[threadIdx.x] = v;
+    si[threadIdx.x] = i;
+    __syncthreads();
+    if (g == 0 && r < b) {
+        for (int k = 1; k < groups; ++k) take_better(v, i, sv[k * bp + r], si[k * bp + r]);
+        out[r] = i == kNoIndex ? 0u : (uint32_t)i;
+    }
 }
 
 struct GreedyPlan {
@@ -288,7 +299,7 @@ static hipError_t launch_greedy(const void* xprep, const void* qw, const void* s
         static_cast<float*>(logits), best_val, best_idx, b, n, k, p.tiles_per_worker);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    greedy_pick_kernel<<<dim3(1), dim3(64), 0, stream>>>(
+    greedy_pick_kernel<<<dim3(1), dim3(kPickThreads), 0, stream>>>(
         best_val, best_idx, static_cast<uint32_t*>(out_tokens), b, BP, p.workers);
     return hipGetLastError();
 }
