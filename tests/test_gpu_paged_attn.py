@@ -219,3 +219,20 @@ def test_long_context_32k_single_sequence():
     rng = np.random.default_rng(6)
     c = workloads.paged_case(rng, [1, 1], [32767, 127], hq=32, hkv=8)
     _check(c, what="32k context")
+
+
+def test_chunked_prefill_sequence_order_ties_and_many_sequences():
+    # The prefill kernel takes sequences longest first (ranked inside the kernel): equal
+    # contexts must still give each workgroup a different sequence, decode rows and empty
+    # chunks rank last, and with more sequences than the ranking handles it falls back to
+    # grid order.
+    rng = np.random.default_rng(61)
+    new = [40] * 12 + [1, 1, 3, 3]
+    prior = [60] * 12 + [100, 5, 0, 0]
+    c = workloads.paged_case(rng, new, prior, hq=8, hkv=2)
+    _check(c, what="prefill, equal contexts")
+    n = 530
+    new = np.where(np.arange(n) % 3 == 0, 1, 2 + (np.arange(n) % 5)).astype(np.int32)
+    prior = (np.arange(n) * 7 % 40).astype(np.int32)
+    c = workloads.paged_case(rng, new, prior, hq=4, hkv=2)
+    _check(c, what="prefill, 530 sequences")
