@@ -566,6 +566,54 @@ def bench_decode_step(args):
             "lm_head_bytes": head_bytes, "lm_head_greedy_us": round(ms_head * 1e3, 1),
             "lm_head_GBps": round(head_bytes / (ms_head * 1e-3) / 1e9, 1)}
         del d_embed, head_bufs
+        # leave the runner as it was: 36 layers, hidden state in, hidden state out
+        r.cfg.vocab = 0
+        r.batch.token_ids = None
+        r.batch.lm_head = None
+
+    # ---- the 36 layers over TurboQuant 3-bit KV pools (the reference's KV codec): the fp16
+    # pools re-encoded on the device, new rows encoded as the step writes them, attention
+    # decoding inside its gather.  A different cache format, so a figure of its own.
+    turbo3_step = None
+    if not args.skip_closed_loop:
+        rows = r.pools[0][0].nbytes // (hkv * 128 * 2)
+        d_iota = hip.DeviceBuffer.from_numpy(np.arange(rows, dtype=np.int64))
+        t3_pools = []
+        for l in range(L):
+            kp, vp = r.pools[l]
+            k3, v3 = hip.DeviceBuffer(rows * hkv * 56), hip.DeviceBuffer(rows * hkv * 56)
+            kernels.launch_kv_write_turbo3(kp, vp, k3, v3, d_iota, rows, hkv, stream)
+            t3_pools.append((k3, v3))
+            r.layers[l].k_pool_f16, r.layers[l].v_pool_f16 = k3.ptr.value, v3.ptr.value
+        stream.synchronize()
+        r.cfg.kv_turbo3 = 1
+        g3 = hip.Graph(stream)
+        with g3:
+            kernels.launch_pack_ragged(d_ones, d_cur_prior, r.idx["block_tables"],
+                                       r.idx["cu_seqlens"], r.slots, r.idx["context_lens"], S, bs,
+                                       max_blocks, stream)
+            r.launch()
+        for i in range(warmup):
+            one_step(i, g3)
+        stream.synchronize()
+        e0.record(stream)
+        for i in range(steps):
+            one_step(warmup + i, g3)
+        e1.record(stream)
+        e1.synchronize()
+        ms_t3 = e0.elapsed_ms(e1) / steps
+        out3 = O.bf16_bits_to_f32(r.result_bits())
+        assert np.isfinite(out3).all()
+        turbo3_step = {
+            "what": "the same 36-layer step over TurboQuant 3-bit KV pools (56 bytes per head "
+                    "row instead of 256): rows encoded on write, decoded inside the attention",
+            "ms_per_step": round(ms_t3, 4), "tok_s": round(S / (ms_t3 * 1e-3), 1),
+            "kv_bytes_per_step": int(sum_ctx * L * 2 * hkv * 56)}
+        r.cfg.kv_turbo3 = 0
+        for l in range(L):
+            r.layers[l].k_pool_f16 = r.pools[l][0].ptr.value
+            r.layers[l].v_pool_f16 = r.pools[l][1].ptr.value
+        del t3_pools
 
     per_layer_w = sum(int(np.asarray(t[0]).nbytes + np.asarray(t[1]).nbytes +
                           np.asarray(t[2]).nbytes)
@@ -605,6 +653,7 @@ def bench_decode_step(args):
         "parity_rel_l2_vs_oracle_one_layer": rel_l2,
         "host_wall_ms_per_step": round(wall_ms, 4),
         "closed_loop_with_embedding_and_lm_head": closed_loop,
+        "step_over_turbo3_kv": turbo3_step,
     }
 
 
@@ -618,8 +667,9 @@ def main():
     ap.add_argument("--skip-kernels", action="store_true",
                     help="only the decode-step line, without the per-kernel legs")
     ap.add_argument("--skip-closed-loop", action="store_true",
-                    help="leave out the token-ids-in / token-ids-out leg of the decode step "
-                         "(embedding, lm_head + greedy); profiling runs use this")
+                    help="leave out the extra legs of the decode step (token ids in / token ids "
+                         "out with embedding, lm_head + greedy; the step over turbo3 KV pools); "
+                         "profiling runs use this")
     ap.add_argument("--workload", default="all",
                     choices=["all", "step", "config1", "config2", "config3", "config4"],
                     help="all: the decode-step line with every leg inside it (default); "

@@ -361,6 +361,15 @@ logismos_status_t logismos_launch_rope_kv_write_f32p(
     const void* sin_f32, const int64_t* slot_mapping, void* q_out_f16, void* k_pool_f16,
     void* v_pool_f16, int total_tokens, int num_q_heads, int num_kv_heads, int head_dim,
     int max_pos, logismos_stream_t stream);
+/* The same with turbo3 pools (see the TurboQuant section below): the rotated k and the v of
+ * every new token are rounded to fp16, as the fp16 pools would hold them, and encoded with
+ * `encode_turbo3_0_head` (crates/quant/src/lib.rs:316-353) into the 56-byte head rows at the
+ * token's slot. */
+logismos_status_t logismos_launch_rope_kv_write_f32p_turbo3(
+    const void* qkv_parts_f32, int num_parts, const int32_t* positions, const void* cos_f32,
+    const void* sin_f32, const int64_t* slot_mapping, void* q_out_f16, void* k_pool_t3,
+    void* v_pool_t3, int total_tokens, int num_q_heads, int num_kv_heads, int head_dim,
+    int max_pos, logismos_stream_t stream);
 logismos_status_t logismos_launch_silu_mul_f32p(const void* parts_f32, int num_parts,
                                                 void* out_bf16, int rows, int inter,
                                                 logismos_stream_t stream);
@@ -424,6 +433,10 @@ logismos_status_t logismos_launch_embed_lookup_bf16(const void* table_bf16, cons
  * `decode::greedy` per sequence (crates/decode/src/lib.rs:73-83) into `out_tokens_u32`
  * (and the fp32 logits into `logits_f32` if that is not NULL); `out_bf16` may then be NULL.
  *
+ * With cfg->kv_turbo3 the KV cache is TurboQuant 3-bit: new K/V rows are encoded as they
+ * are written and the attention decodes inside its gather (the entry points of the
+ * TurboQuant section below), everything else unchanged.
+ *
  * All launches are asynchronous on `stream`; `workspace` needs
  * logismos_decode_step_workspace_bytes() bytes, 256-byte aligned, contents don't matter.
  * ------------------------------------------------------------------------ */
@@ -437,14 +450,15 @@ typedef struct {
     int num_layers, hidden, num_q_heads, num_kv_heads, head_dim, intermediate;
     float rms_eps;
     int block_size, max_blocks_per_seq, max_pos;
-    int vocab; /* rows of the embedding table and of lm_head; 0 when neither is used */
+    int vocab;     /* rows of the embedding table and of lm_head; 0 when neither is used */
+    int kv_turbo3; /* != 0: the layers' pools are turbo3 pools (56 bytes per head row) */
 } logismos_decode_config_t;
 
 typedef struct {
     const void* norm1_w_f32; /* [hidden] */
     const void* norm2_w_f32; /* [hidden] */
     logismos_q4_weight_t qkv, o, gate_up, down;
-    void* k_pool_f16; /* this layer's paged pools */
+    void* k_pool_f16; /* this layer's paged pools (turbo3 pools with cfg->kv_turbo3) */
     void* v_pool_f16;
 } logismos_decode_layer_t;
 

@@ -114,16 +114,18 @@ extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_c
                                                        stream));
         LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk_xprep(
             w.xn, L.qkv.qw, L.qkv.scale, L.qkv.zero, w.qkv, b, qd + 2 * kvd, c.hidden, stream));
-        LG_TRY(logismos_launch_rope_kv_write_f32p(
-            w.qkv, w.j_qkv, batch->positions, batch->rope_cos_f32, batch->rope_sin_f32,
-            batch->slot_mapping, w.q, L.k_pool_f16, L.v_pool_f16, b, c.num_q_heads, c.num_kv_heads,
-            c.head_dim, c.max_pos, stream));
+        const auto rope_kv_write = c.kv_turbo3 ? logismos_launch_rope_kv_write_f32p_turbo3
+                                               : logismos_launch_rope_kv_write_f32p;
+        LG_TRY(rope_kv_write(w.qkv, w.j_qkv, batch->positions, batch->rope_cos_f32,
+                             batch->rope_sin_f32, batch->slot_mapping, w.q, L.k_pool_f16,
+                             L.v_pool_f16, b, c.num_q_heads, c.num_kv_heads, c.head_dim, c.max_pos,
+                             stream));
         // attention writes the prepared layout directly: its output only feeds the o projection
         LG_TRY(lg::paged_attn_launch(
             w.q, L.k_pool_f16, L.v_pool_f16, batch->block_tables, batch->cu_seqlens,
             batch->context_lens, w.attn_b, w.attn_ws, b, b, 1, c.num_q_heads, c.num_kv_heads,
             c.head_dim, c.block_size, c.max_blocks_per_seq, batch->num_splits, scale, 1,
-            LOGISMOS_ATTN_PHASE_ALL, 2, 0, stream));
+            LOGISMOS_ATTN_PHASE_ALL, 2, c.kv_turbo3 ? 1 : 0, stream));
         LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk_xprep(w.attn_b, L.o.qw, L.o.scale, L.o.zero,
                                                              w.proj, b, c.hidden, qd, stream));
         LG_TRY(logismos_launch_add_rms_norm_f32p_xprep(batch->hidden_f32, w.proj, w.j_o,

@@ -6,6 +6,7 @@
 #include "device_utils.hpp"
 #include "launch_common.hpp"
 #include "q4_common.hpp"
+#include "turbo3_device.hpp"
 
 #include <hip/hip_fp16.h>
 #include <math.h>
@@ -247,7 +248,10 @@ __global__ __launch_bounds__(256) void silu_mul_xprep_kernel(const float* __rest
 
 // grid (hq + 2*hkv, total_tokens), 64 threads: thread i rotates elements i and
 // i + d/2 (d = 128).  q heads go to q_out (fp16); k heads, rotated, and v heads,
-// as they are, go to the pools at the token's slot.
+// as they are, go to the pools at the token's slot: as fp16 rows, or (T3) rounded to fp16
+// like those and then encoded as turbo3 head rows -- the lane layout of the rotation is
+// the encoder's.
+template <bool T3>
 __global__ __launch_bounds__(64) void rope_kv_write_kernel(
     const uint16_t* __restrict__ qkv, const float* __restrict__ qkv_parts, int num_parts,
     int64_t part_stride, const int32_t* __restrict__ positions,
@@ -283,16 +287,30 @@ __global__ __launch_bounds__(64) void rope_kv_write_kernel(
         } else {
             const int64_t slot = slot_mapping[t];
             if (slot < 0) return;
-            __half* dst = k_pool + (slot * hkv + (head - hq)) * D;
-            dst[i] = __float2half_rn(y0);
-            dst[i + HALF] = __float2half_rn(y1);
+            if constexpr (T3) {
+                turbo3_encode_row(__half2float(__float2half_rn(y0)),
+                                  __half2float(__float2half_rn(y1)), i,
+                                  reinterpret_cast<uint8_t*>(k_pool) +
+                                      (slot * hkv + (head - hq)) * kTurbo3HeadBytes);
+            } else {
+                __half* dst = k_pool + (slot * hkv + (head - hq)) * D;
+                dst[i] = __float2half_rn(y0);
+                dst[i + HALF] = __float2half_rn(y1);
+            }
         }
     } else {
         const int64_t slot = slot_mapping[t];
         if (slot < 0) return;
-        __half* dst = v_pool + (slot * hkv + (head - hq - hkv)) * D;
-        dst[i] = __float2half_rn(x0);
-        dst[i + HALF] = __float2half_rn(x1);
+        if constexpr (T3) {
+            turbo3_encode_row(__half2float(__float2half_rn(x0)), __half2float(__float2half_rn(x1)),
+                              i,
+                              reinterpret_cast<uint8_t*>(v_pool) +
+                                  (slot * hkv + (head - hq - hkv)) * kTurbo3HeadBytes);
+        } else {
+            __half* dst = v_pool + (slot * hkv + (head - hq - hkv)) * D;
+            dst[i] = __float2half_rn(x0);
+            dst[i + HALF] = __float2half_rn(x1);
+        }
     }
 }
 
@@ -431,7 +449,7 @@ extern "C" logismos_status_t logismos_launch_rope_kv_write_fp16(
         !k_pool_f16 || !v_pool_f16)
         return hipErrorInvalidValue;
     dim3 grid(num_q_heads + 2 * num_kv_heads, total_tokens);
-    lg::rope_kv_write_kernel<<<grid, dim3(64), 0, static_cast<hipStream_t>(stream)>>>(
+    lg::rope_kv_write_kernel<false><<<grid, dim3(64), 0, static_cast<hipStream_t>(stream)>>>(
         static_cast<const uint16_t*>(qkv_bf16), nullptr, 0, 0, positions,
         static_cast<const float*>(cos_f32),
         static_cast<const float*>(sin_f32), slot_mapping, static_cast<__half*>(q_out_f16),
@@ -455,11 +473,34 @@ extern "C" logismos_status_t logismos_launch_rope_kv_write_f32p(
         !k_pool_f16 || !v_pool_f16)
         return hipErrorInvalidValue;
     dim3 grid(num_q_heads + 2 * num_kv_heads, total_tokens);
-    lg::rope_kv_write_kernel<<<grid, dim3(64), 0, static_cast<hipStream_t>(stream)>>>(
+    lg::rope_kv_write_kernel<false><<<grid, dim3(64), 0, static_cast<hipStream_t>(stream)>>>(
         nullptr, static_cast<const float*>(qkv_parts_f32), num_parts, (int64_t)total_tokens * width,
         positions, static_cast<const float*>(cos_f32), static_cast<const float*>(sin_f32),
         slot_mapping, static_cast<__half*>(q_out_f16), static_cast<__half*>(k_pool_f16),
         static_cast<__half*>(v_pool_f16), num_q_heads, num_kv_heads, max_pos);
+    return hipGetLastError();
+}
+
+extern "C" logismos_status_t logismos_launch_rope_kv_write_f32p_turbo3(
+    const void* qkv_parts_f32, int num_parts, const int32_t* positions, const void* cos_f32,
+    const void* sin_f32, const int64_t* slot_mapping, void* q_out_f16, void* k_pool_t3,
+    void* v_pool_t3, int total_tokens, int num_q_heads, int num_kv_heads, int head_dim,
+    int max_pos, logismos_stream_t stream) {
+    if (total_tokens < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || max_pos <= 0 || num_parts <= 0)
+        return hipErrorInvalidValue;
+    if (head_dim != 128 || total_tokens > 65535) return hipErrorInvalidValue;
+    const int64_t width = (int64_t)(num_q_heads + 2 * num_kv_heads) * head_dim;
+    if ((int64_t)total_tokens * width > (int64_t)INT32_MAX) return hipErrorInvalidValue;
+    if (total_tokens == 0) return hipSuccess;
+    if (!qkv_parts_f32 || !positions || !cos_f32 || !sin_f32 || !slot_mapping || !q_out_f16 ||
+        !k_pool_t3 || !v_pool_t3)
+        return hipErrorInvalidValue;
+    dim3 grid(num_q_heads + 2 * num_kv_heads, total_tokens);
+    lg::rope_kv_write_kernel<true><<<grid, dim3(64), 0, static_cast<hipStream_t>(stream)>>>(
+        nullptr, static_cast<const float*>(qkv_parts_f32), num_parts, (int64_t)total_tokens * width,
+        positions, static_cast<const float*>(cos_f32), static_cast<const float*>(sin_f32),
+        slot_mapping, static_cast<__half*>(q_out_f16), static_cast<__half*>(k_pool_t3),
+        static_cast<__half*>(v_pool_t3), num_q_heads, num_kv_heads, max_pos);
     return hipGetLastError();
 }
 

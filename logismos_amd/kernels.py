@@ -80,6 +80,8 @@ _SIGNATURES = {
     "logismos_launch_qgemm_q4g128_f32_splitk": (C.c_uint32, [_vp] * 5 + [_i, _i, _i, _vp]),
     "logismos_launch_add_rms_norm_f32p": (C.c_uint32, [_vp, _vp, _i, _vp, _vp, _i, _i, _f, _vp]),
     "logismos_launch_rope_kv_write_f32p": (C.c_uint32, [_vp, _i] + [_vp] * 7 + [_i] * 5 + [_vp]),
+    "logismos_launch_rope_kv_write_f32p_turbo3":
+        (C.c_uint32, [_vp, _i] + [_vp] * 7 + [_i] * 5 + [_vp]),
     "logismos_launch_silu_mul_f32p": (C.c_uint32, [_vp, _i, _vp, _i, _i, _vp]),
     "logismos_q4_xprep_bytes": (_sz, [_i, _i]),
     "logismos_launch_q4_prepare_x_bf16": (C.c_uint32, [_vp, _vp, _i, _i, _vp]),
@@ -128,7 +130,8 @@ class Q4Weight(C.Structure):
 class DecodeConfig(C.Structure):
     _fields_ = [("num_layers", _i), ("hidden", _i), ("num_q_heads", _i), ("num_kv_heads", _i),
                 ("head_dim", _i), ("intermediate", _i), ("rms_eps", _f), ("block_size", _i),
-                ("max_blocks_per_seq", _i), ("max_pos", _i), ("vocab", _i)]
+                ("max_blocks_per_seq", _i), ("max_pos", _i), ("vocab", _i),
+                ("kv_turbo3", _i)]
 
 
 class DecodeLayer(C.Structure):
@@ -419,8 +422,10 @@ def launch_add_rms_norm_f32p(h, parts, num_parts: int, w, out, rows: int, n: int
 
 def launch_rope_kv_write_f32p(parts, num_parts: int, positions, cos, sin, slot_mapping, q_out,
                               k_pool, v_pool, total_tokens: int, hq: int, hkv: int, head_dim: int,
-                              max_pos: int, stream=None) -> None:
-    _status("rope_kv_write_f32p", library().logismos_launch_rope_kv_write_f32p(
+                              max_pos: int, stream=None, turbo3: bool = False) -> None:
+    fn = (library().logismos_launch_rope_kv_write_f32p_turbo3 if turbo3
+          else library().logismos_launch_rope_kv_write_f32p)
+    _status("rope_kv_write_f32p", fn(
         _ptr(parts), num_parts, _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping),
         _ptr(q_out), _ptr(k_pool), _ptr(v_pool), total_tokens, hq, hkv, head_dim, max_pos,
         _raw(stream)))

@@ -497,6 +497,8 @@ _t3_kv_write = _sig("oracle_kv_write_turbo3", None, _vp, _vp, _vp, _vp, _vp, _sz
 _t3_gather = _sig("oracle_paged_gather_turbo3", None, _vp, _vp, _sz, _sz, _sz, _vp)
 _t3_attn = _sig("oracle_paged_attn_varlen_turbo3", None, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz,
                 _sz, _sz, _sz, _sz, C.c_float, C.c_int)
+_t3_attn_f32 = _sig("oracle_paged_attn_varlen_turbo3_f32out", None, _vp, _vp, _vp, _vp, _vp, _vp,
+                    _vp, _sz, _sz, _sz, _sz, _sz, C.c_float, C.c_int)
 TURBO3_BYTES_PER_HEAD = 56
 
 
@@ -567,7 +569,8 @@ def paged_gather_turbo3(pool, block_table_row, ctx, block_size, num_kv_heads):
 
 
 def paged_attn_varlen_turbo3(q, k_pool, v_pool, block_tables, cu_seqlens_q, context_lens,
-                             num_q_heads, num_kv_heads, block_size, scale, causal=True):
+                             num_q_heads, num_kv_heads, block_size, scale, causal=True,
+                             f32_out=False):
     q = _u16(q)
     k_pool = np.ascontiguousarray(k_pool, dtype=np.uint8)
     v_pool = np.ascontiguousarray(v_pool, dtype=np.uint8)
@@ -575,11 +578,12 @@ def paged_attn_varlen_turbo3(q, k_pool, v_pool, block_tables, cu_seqlens_q, cont
     cu = np.ascontiguousarray(cu_seqlens_q, dtype=np.int32)
     ctx = np.ascontiguousarray(context_lens, dtype=np.int32)
     num_seqs = ctx.size
-    out = np.zeros(q.shape, np.uint16)
-    _t3_attn(_p(q), _p(k_pool), _p(v_pool), _p(block_tables), _p(cu), _p(ctx), _p(out), num_seqs,
-             num_q_heads, num_kv_heads, block_size, block_tables.shape[1] if num_seqs else 0,
-             scale, 1 if causal else 0)
-    return out.view(np.float16)
+    out = np.zeros(q.shape, np.float32 if f32_out else np.uint16)
+    (_t3_attn_f32 if f32_out else _t3_attn)(
+        _p(q), _p(k_pool), _p(v_pool), _p(block_tables), _p(cu), _p(ctx), _p(out), num_seqs,
+        num_q_heads, num_kv_heads, block_size, block_tables.shape[1] if num_seqs else 0, scale,
+        1 if causal else 0)
+    return out if f32_out else out.view(np.float16)
 
 
 # ---------------------------------------------------------------- metric / threads

@@ -32,9 +32,10 @@ def add_rms_norm_bf16(h: np.ndarray, y, w, eps: float) -> np.ndarray:
     return O.f32_to_bf16_bits(O.rms_norm(h, w, rows, n, eps)).reshape(rows, n)
 
 
-def rope_kv_write(qkv, positions, cos, sin, slots, k_pool, v_pool, hq, hkv, d=128):
+def rope_kv_write(qkv, positions, cos, sin, slots, k_pool, v_pool, hq, hkv, d=128, turbo3=False):
     """qkv (bf16 bits or fp32) [T, (hq+2hkv)*d] -> q fp16 [T,hq,d]; roped k and v written into
-    the pools."""
+    the pools: as fp16 rows, or (turbo3: uint8 pools of 56-byte head rows) those fp16 rows
+    encoded with `encode_turbo3_0_head`."""
     qkv = np.asarray(qkv)
     t = qkv.shape[0]
     half = d // 2
@@ -53,7 +54,10 @@ def rope_kv_write(qkv, positions, cos, sin, slots, k_pool, v_pool, hq, hkv, d=12
     q16 = O.f32_to_f16_bits(q).view(np.float16).reshape(t, hq, d)
     k16 = O.f32_to_f16_bits(k).view(np.float16).reshape(t, hkv * d)
     v16 = O.f32_to_f16_bits(v).view(np.float16).reshape(t, hkv * d)
-    O.kv_write_fp16(k16, v16, k_pool, v_pool, slots, hkv * d)
+    if turbo3:
+        O.kv_write_turbo3(k16, v16, k_pool, v_pool, slots, hkv)
+    else:
+        O.kv_write_fp16(k16, v16, k_pool, v_pool, slots, hkv * d)
     return q16
 
 
@@ -79,7 +83,8 @@ def _gemm(x_bits, w, b):
 def decode_step(cfg, layers, batch, trace=None):
     """One decode step over `batch` (one new token per sequence).
 
-    cfg:    dict(hidden, hq, hkv, d, inter, eps, block_size)
+    cfg:    dict(hidden, hq, hkv, d, inter, eps, block_size[, kv_turbo3: the pools are uint8
+            turbo3 pools [rows][hkv*56]])
     layers: list of dict(norm1, qkv, o, norm2, gate_up, down, k_pool, v_pool); each weight a
             (qw, scale, zero) triple; pools are updated in place
     batch:  dict(h [B, hidden] fp32 (updated in place), block_tables, cu_seqlens, context_lens,
@@ -99,12 +104,22 @@ def decode_step(cfg, layers, batch, trace=None):
     for li, L in enumerate(layers):
         xn = add_rms_norm_bf16(h, y, L["norm1"], cfg["eps"])
         qkv = _gemm(xn, L["qkv"], b)
+        t3 = bool(cfg.get("kv_turbo3"))
         q16 = rope_kv_write(qkv, batch["positions"], batch["cos"], batch["sin"], batch["slots"],
-                            L["k_pool"], L["v_pool"], cfg["hq"], cfg["hkv"], cfg["d"])
-        attn = O.paged_attn_varlen_fp16(q16, L["k_pool"], L["v_pool"], batch["block_tables"],
-                                        batch["cu_seqlens"], batch["context_lens"], cfg["hq"],
-                                        cfg["hkv"], cfg["d"], cfg["block_size"],
-                                        1.0 / np.sqrt(np.float32(cfg["d"])), True, f32_out=True)
+                            L["k_pool"], L["v_pool"], cfg["hq"], cfg["hkv"], cfg["d"], turbo3=t3)
+        if t3:
+            attn = O.paged_attn_varlen_turbo3(q16, L["k_pool"], L["v_pool"],
+                                              batch["block_tables"], batch["cu_seqlens"],
+                                              batch["context_lens"], cfg["hq"], cfg["hkv"],
+                                              cfg["block_size"],
+                                              1.0 / np.sqrt(np.float32(cfg["d"])), True,
+                                              f32_out=True)
+        else:
+            attn = O.paged_attn_varlen_fp16(q16, L["k_pool"], L["v_pool"], batch["block_tables"],
+                                            batch["cu_seqlens"], batch["context_lens"], cfg["hq"],
+                                            cfg["hkv"], cfg["d"], cfg["block_size"],
+                                            1.0 / np.sqrt(np.float32(cfg["d"])), True,
+                                            f32_out=True)
         o = _gemm(O.f32_to_bf16_bits(attn.reshape(b, -1)), L["o"], b)
         xn2 = add_rms_norm_bf16(h, o, L["norm2"], cfg["eps"])
         gu = _gemm(xn2, L["gate_up"], b)

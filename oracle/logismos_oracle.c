@@ -1017,6 +1017,19 @@ void oracle_paged_attn_varlen_turbo3(const uint16_t* q, const uint8_t* k_pool,
                     scale, causal);
 }
 
+/* The same with the fp32 result (what the decode step rounds once to bf16). */
+void oracle_paged_attn_varlen_turbo3_f32out(const uint16_t* q, const uint8_t* k_pool,
+                                            const uint8_t* v_pool, const int32_t* block_tables,
+                                            const int32_t* cu_seqlens_q,
+                                            const int32_t* context_lens, float* out,
+                                            size_t num_seqs, size_t num_q_heads,
+                                            size_t num_kv_heads, size_t block_size,
+                                            size_t max_blocks_per_seq, float scale, int causal) {
+    paged_attn_core(q, k_pool, v_pool, 1, block_tables, cu_seqlens_q, context_lens, NULL, out,
+                    num_seqs, num_q_heads, num_kv_heads, 128, block_size, max_blocks_per_seq,
+                    scale, causal);
+}
+
 /* ------------------------------------------------------------------ metric / threads */
 
 /* crates/kernels/tests/matmul_parity.rs:83-99 -- max |g-c| and max |g-c| / max(|c|, 1e-3). */

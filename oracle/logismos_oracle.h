@@ -160,6 +160,12 @@ void oracle_paged_attn_varlen_turbo3(const uint16_t* q, const uint8_t* k_pool,
                                      uint16_t* out, size_t num_seqs, size_t num_q_heads,
                                      size_t num_kv_heads, size_t block_size,
                                      size_t max_blocks_per_seq, float scale, int causal);
+void oracle_paged_attn_varlen_turbo3_f32out(const uint16_t* q, const uint8_t* k_pool,
+                                     const uint8_t* v_pool, const int32_t* block_tables,
+                                     const int32_t* cu_seqlens_q, const int32_t* context_lens,
+                                     float* out, size_t num_seqs, size_t num_q_heads,
+                                     size_t num_kv_heads, size_t block_size,
+                                     size_t max_blocks_per_seq, float scale, int causal);
 
 /* ---- parity metric of the reference's GPU tests (crates/kernels/tests/matmul_parity.rs:83-99) */
 void oracle_parity_metric_f32(const float* got, const float* want, size_t n, float* max_abs,

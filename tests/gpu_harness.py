@@ -101,7 +101,8 @@ class DecodeStepRunner:
         self.cfg = kernels.DecodeConfig(len(layers), cfg["hidden"], cfg["hq"], cfg["hkv"], cfg["d"],
                                         cfg["inter"], cfg["eps"], cfg["block_size"], max_blocks,
                                         batch["cos"].size // half,
-                                        batch["lm_head"][0].shape[0] if "lm_head" in batch else 0)
+                                        batch["lm_head"][0].shape[0] if "lm_head" in batch else 0,
+                                        1 if cfg.get("kv_turbo3") else 0)
         up = hip.DeviceBuffer.from_numpy
         self.keep = []
 

@@ -107,3 +107,38 @@ def test_tokens_out_without_the_bf16_state_or_logits():
     lean.launch()
     got, _ = lean.result_tokens()
     assert np.array_equal(got, want)
+
+
+def test_step_over_turbo3_pools():
+    # TurboQuant 3-bit KV: new rows encoded as they are written, attention decoding in its
+    # gather; everything else as the fp16 step
+    rng = np.random.default_rng(36)
+    cfg, layers, batch = workloads.decode_step_problem(
+        rng, num_layers=2, hidden=1024, hq=8, hkv=2, inter=2048, ctx=[1, 17, 300, 64, 999, 5],
+        kv_turbo3=True)
+    r, got, want, lay, bat = _run_both(cfg, layers, batch)
+    # The encoder is a quantiser: a one-ulp difference in a new K/V row between the two paths
+    # can move a 3-bit index to the neighbouring centroid, which a one-token context (row 0:
+    # its output IS the decoded new V row) shows undamped.  Hence the wider bounds than for
+    # the fp16 step; the first layer's appended rows are compared byte for byte below.
+    assert _rel_l2(got, want) < 1e-2
+    assert np.all(np.abs(got - want) <= 5e-2 + 3e-2 * np.abs(want))
+    # the encoded rows the step appended: integer work, compared byte for byte wherever the
+    # fp16 row that went into the encoder was the same on both sides (first layer: its input
+    # does not depend on earlier GPU arithmetic beyond one GEMM; count the agreeing rows)
+    kp, vp = r.pools[0]
+    gk = kp.to_numpy(np.uint8, lay[0]["k_pool"].shape)
+    gv = vp.to_numpy(np.uint8, lay[0]["v_pool"].shape)
+    slots = np.asarray(batch["slots"])
+    untouched = np.setdiff1d(np.arange(gk.shape[0]), slots)
+    assert np.array_equal(gk[untouched], layers[0]["k_pool"][untouched])
+    assert np.array_equal(gv[untouched], layers[0]["v_pool"][untouched])
+    same = sum(np.array_equal(gk[s], lay[0]["k_pool"][s]) for s in slots)
+    assert same >= len(slots) // 2, same
+    # norms (fp16, first two bytes of every 14-byte block) agree to an fp16 ulp everywhere
+    def norms(p):
+        return p.reshape(p.shape[0], -1, 14)[:, :, :2].copy().view(np.float16).astype(np.float32)
+    assert_parity(norms(gk[slots]), norms(lay[0]["k_pool"][slots]), max_abs=1e-3, max_rel=2e-3,
+                  what="turbo3 K norms")
+    assert_parity(norms(gv[slots]), norms(lay[0]["v_pool"][slots]), max_abs=1e-3, max_rel=2e-3,
+                  what="turbo3 V norms")

@@ -154,6 +154,27 @@ def test_f32_parts_variants_add_the_parts_in_order():
     assert np.array_equal(d_vp.to_numpy(np.float16, v_pool.shape).view(np.uint16),
                           v_pool.view(np.uint16))
 
+    # the same into turbo3 pools: the encoder sees the fp16 rows the fp16 pools hold.  V is
+    # not rotated (its fp16 rows are exact above), so its encoded bytes must be identical;
+    # a rotated K row may differ from the oracle's in the last fp16 bit, and the byte-exact
+    # comparison is made against the encoding of the rows the GPU wrote above.
+    k3 = np.zeros((nblk * bs, hkv * 56), np.uint8)
+    v3 = np.zeros((nblk * bs, hkv * 56), np.uint8)
+    d_k3, d_v3 = hip.DeviceBuffer.from_numpy(k3), hip.DeviceBuffer.from_numpy(v3)
+    d_q3 = hip.DeviceBuffer(t * hq * d * 2)
+    kernels.launch_rope_kv_write_f32p(
+        hip.DeviceBuffer.from_numpy(qp), 2, hip.DeviceBuffer.from_numpy(positions),
+        hip.DeviceBuffer.from_numpy(cos), hip.DeviceBuffer.from_numpy(sin),
+        hip.DeviceBuffer.from_numpy(slots), d_q3, d_k3, d_v3, t, hq, hkv, d, max_pos, turbo3=True)
+    hip.synchronize()
+    assert np.array_equal(d_q3.to_numpy(np.uint16, (t, hq, d)), d_q.to_numpy(np.uint16, (t, hq, d)))
+    gpu_k16 = d_kp.to_numpy(np.float16, k_pool.shape)
+    gpu_v16 = d_vp.to_numpy(np.float16, v_pool.shape)
+    k3_want, v3_want = k3.copy(), v3.copy()
+    O.kv_write_turbo3(gpu_k16[slots], gpu_v16[slots], k3_want, v3_want, slots, hkv)
+    assert np.array_equal(d_k3.to_numpy(np.uint8, k3.shape), k3_want)
+    assert np.array_equal(d_v3.to_numpy(np.uint8, v3.shape), v3_want)
+
 
 def _unprepare(buf, b, k):
     """prepared layout -> (bf16 bits [b][k], group sums [b][k/128])"""

@@ -136,12 +136,14 @@ def qgemm_q4_algorithmic_bytes(b, n, k) -> int:
 
 
 def decode_step_problem(rng, num_layers, hidden, hq, hkv, inter, ctx, d=128, block_size=16,
-                        max_pos=None, eps=1e-6, theta=1e6, random_nibbles=False, vocab=0):
+                        max_pos=None, eps=1e-6, theta=1e6, random_nibbles=False, vocab=0,
+                        kv_turbo3=False):
     """A decode-step problem: `ctx[s]` is the context of sequence s INCLUDING the new token.
     Weights ~N(0,0.02) quantised to Q4G128 by the oracle (or raw random nibbles/scales when
     random_nibbles, for timing-only runs), RMSNorm gains 1+N(0,0.02), RoPE theta 1e6.
     With vocab > 0 the batch also carries token ids, a bf16 embedding table and a Q4G128
-    lm_head (tokens in, tokens out)."""
+    lm_head (tokens in, tokens out).  kv_turbo3: the pools are TurboQuant 3-bit pools
+    (uint8 [rows][hkv*56]) holding the encoded random rows."""
     import oracle as O
     ctx = np.asarray(ctx, np.int32)
     b = len(ctx)
@@ -176,6 +178,14 @@ def decode_step_problem(rng, num_layers, hidden, hq, hkv, inter, ctx, d=128, blo
                  positions=(ctx - 1).astype(np.int32), slots=slots, cos=cos, sin=sin,
                  final_norm=(1 + 0.02 * rng.standard_normal(hidden)).astype(np.float32))
     cfg = dict(hidden=hidden, hq=hq, hkv=hkv, d=d, inter=inter, eps=eps, block_size=block_size)
+    if kv_turbo3:
+        cfg["kv_turbo3"] = True
+        for L in layers:
+            rows = L["k_pool"].shape[0]
+            kp = np.zeros((rows, hkv * 56), np.uint8)
+            vp = np.zeros((rows, hkv * 56), np.uint8)
+            O.kv_write_turbo3(L["k_pool"], L["v_pool"], kp, vp, np.arange(rows), hkv)
+            L["k_pool"], L["v_pool"] = kp, vp
     if vocab:
         batch["token_ids"] = rng.integers(0, vocab, size=b, dtype=np.uint32)
         batch["embed_table"] = O.f32_to_bf16_bits(
