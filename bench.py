@@ -443,11 +443,15 @@ def bench_decode_step(args):
     O.set_num_threads(cores)
     import copy
     lay_cpu = copy.deepcopy(layers)
-    t0 = time.perf_counter()
     want = O.bf16_bits_to_f32(OS.decode_step(cfg, lay_cpu, dict(b0, h=batch["h"].copy())))
+    rel_l2 = float(np.linalg.norm(got - want) / np.linalg.norm(want))
+    # the baseline: one whole step (36 layers) on the oracle; the 36 layers share one layer's
+    # weights and pools (36 sets of pools would be 38 GB of host memory), which leaves the
+    # arithmetic and the bytes touched per layer as they are
+    t0 = time.perf_counter()
+    OS.decode_step(cfg, lay_cpu * L, dict(b0, h=batch["h"].copy()))
     cpu_s = time.perf_counter() - t0
     del lay_cpu
-    rel_l2 = float(np.linalg.norm(got - want) / np.linalg.norm(want))
 
     # ---- the 36-layer problem on the device (layer data replicated device-to-device)
     r = DecodeStepRunner(cfg, layers * L, b0, stream=stream, share_layer_data=True)
@@ -646,10 +650,11 @@ def bench_decode_step(args):
                                        "default steps, bytes per launch)",
                      "kernel": "paged_attn_balanced_kernel<4> (decode rows, one layer of the step)",
                      "ms_per_launch": round(ms_attn, 5), "algorithmic_bytes_per_launch": attn_bytes},
-        "cpu_baseline": {"value": round(S / (cpu_s * L), 3), "unit": "tok/s", "cores": cores,
+        "cpu_baseline": {"value": round(S / cpu_s, 3), "unit": "tok/s", "cores": cores,
                          "kind": "port",
-                         "sample": f"one of the 36 layers of step 0 ({cpu_s:.2f} s on the CPU "
-                                   "oracle), scaled by 36"},
+                         "sample": f"step 0 in full, 36 layers x 32 sequences, on the CPU oracle "
+                                   f"({cpu_s:.1f} s; one layer's weights and pools reused by "
+                                   "all 36)"},
         "parity_rel_l2_vs_oracle_one_layer": rel_l2,
         "host_wall_ms_per_step": round(wall_ms, 4),
         "closed_loop_with_embedding_and_lm_head": closed_loop,
