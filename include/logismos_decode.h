@@ -553,9 +553,13 @@ enum {
  * themselves (`logismos_launch_rope_kv_write_*`), and advance then records
  * those rows as written.  k_pool / v_pool / block_tables return the device
  * pointers the attention and packing entry points take (block table row of
- * sequence s at `block_tables + s * max_blocks_per_seq`; entries without a
- * block hold 0x3FFFFFFF).  Copies and launches go to `stream`; one caller
- * thread at a time per cache. */
+ * sequence s at `block_tables + s * max_blocks_per_seq`; entries that never
+ * had a block hold 0x3FFFFFFF, entries of a retired sequence keep their last
+ * value).  Copies and launches go to `stream`; one caller thread at a time per
+ * cache.  close_seq and reset do not wait for the device: on the stream that
+ * carried the sequence's copies and launches its blocks may be handed out
+ * again at once (what the next owner writes is ordered behind them); work on
+ * any other stream has to be ordered by the caller. */
 int logismos_paged_kv_cache_create(const logismos_paged_kv_layout_t* layout,
                                    logismos_paged_kv_cache_t** out);
 void logismos_paged_kv_cache_destroy(logismos_paged_kv_cache_t* cache);

@@ -72,12 +72,13 @@ int ensure_blocks(logismos_paged_kv_cache* c, int seq, int64_t rows, hipStream_t
     return e == hipSuccess ? LOGISMOS_KV_OK : LOGISMOS_KV_HIP_ERROR;
 }
 
+// The host row keeps its entries: a copy of them to the device that an earlier reserve or put
+// queued on a stream may not have run yet, and the launches queued behind it still need the
+// ids it carries.  (On one stream a freed block is safe to hand out at once: whatever the next
+// owner writes is ordered after those launches.)
 void release_blocks(logismos_paged_kv_cache* c, int seq) {
-    int32_t* r = c->row(seq);
-    for (int b = c->seq_blocks[(size_t)seq] - 1; b >= 0; --b) {
-        c->free_blocks.push_back(r[b]);
-        r[b] = kUnmapped;
-    }
+    const int32_t* r = c->row(seq);
+    for (int b = c->seq_blocks[(size_t)seq] - 1; b >= 0; --b) c->free_blocks.push_back(r[b]);
     c->seq_blocks[(size_t)seq] = 0;
     for (int l = 0; l < c->layout.num_layers; ++l) c->len(seq, l) = 0;
 }

@@ -14,6 +14,7 @@ __global__ __launch_bounds__(256) void pack_ragged_kernel(
     const int32_t* __restrict__ block_tables, int32_t* __restrict__ cu_seqlens,
     int64_t* __restrict__ slot_mapping, int32_t* __restrict__ context_lens, int num_seqs,
     int block_size, int max_blocks) {
+    (void)num_seqs;  // the grid has one workgroup per sequence
     const int s = blockIdx.x;
     __shared__ int partial[4];
     int sum = 0;

@@ -240,3 +240,20 @@ def test_reserve_and_advance_cover_rows_written_by_the_step_kernels():
     with pytest.raises(CacheError) as e:
         c.reserve(s, 33)         # beyond max_seq_len = 32
     assert e.value.kind == "LenOverflow"
+
+
+def test_retiring_a_sequence_does_not_disturb_a_queued_table_copy():
+    # reserve queues the copy of the new table entries on a stream; closing the sequence
+    # right away must not change what that copy delivers (the launches queued behind it
+    # still read through those entries)
+    c = small(num_blocks=6, max_blocks_per_seq=3)
+    st = hip.Stream()
+    s = c.open_seq()
+    c.reserve(s, 40, st)
+    want = c.block_tables_host()[s, :3].copy()
+    c.close_seq(s)
+    st.synchronize()
+    got = hip.DevicePtrView(c.block_tables(), 4 * c.layout.max_seqs * 3).to_numpy(np.int32)
+    assert sorted(want.tolist()) == sorted(set(want.tolist())) and (want < 6).all()
+    assert np.array_equal(got.reshape(-1, 3)[s], want)
+    assert c.free_blocks() == 6
