@@ -413,6 +413,43 @@ logismos_status_t logismos_launch_embed_lookup_bf16(const void* table_bf16, cons
                                                     long long vocab, logismos_stream_t stream);
 
 /* ------------------------------------------------------------------------
+ * The launchers the reference already has (built there for gfx1100), for gfx950
+ * ------------------------------------------------------------------------
+ * Same symbols, argument lists and meaning as the reference's own, so its private
+ * `extern "C"` blocks (crates/kernels/src/{rms_norm,softmax,rope,matmul}/mod.rs) link
+ * against this archive unchanged and `praxis::{rms_norm, softmax, rope_apply, matmul}` run
+ * on MI355X.  fp16 in and out, fp32 inside, one rounding at the output; results as the
+ * CPU references define them (crates/kernels/src/{rms_norm,softmax,rope,matmul}/cpu.rs). */
+
+/* crates/kernels/src/rms_norm/hip/rms_norm.hip:58-84: y[m][n] = x * inv_rms(row) * w[n]. */
+logismos_status_t logismos_launch_rms_norm_fp16(const void* x_fp16, const void* w_fp16,
+                                                void* y_fp16, int m, int n, float eps,
+                                                logismos_stream_t stream);
+/* crates/kernels/src/softmax/hip/softmax.hip:66-87: row softmax of x[m][n]; a row of -inf
+ * becomes uniform 1/n as in `softmax_fp16_ref` (crates/kernels/src/softmax/cpu.rs:40-59). */
+logismos_status_t logismos_launch_softmax_fp16(const void* x_fp16, void* y_fp16, int m, int n,
+                                               logismos_stream_t stream);
+/* crates/kernels/src/rope/hip/rope.hip:45-68: in place on (batch, seq, heads, head_dim),
+ * interleaved pairs (2i, 2i+1), table f32 `[seq][head_dim]` with cos at 2i and sin at 2i+1
+ * (`build_cos_sin_table`, crates/kernels/src/rope/cpu.rs:19-40).  Shape guard of
+ * `check_rope_shape` (crates/kernels/src/rope/mod.rs:79-130).  qk 4-byte, table 8-byte
+ * aligned. */
+logismos_status_t logismos_launch_rope_fp16(void* qk_fp16, const void* cos_sin_f32, int batch,
+                                            int seq, int heads, int head_dim,
+                                            logismos_stream_t stream);
+/* crates/kernels/src/matmul/hip/matmul_launchers.cpp:14-52: D[M,N] = A[M,K] . B[K,N],
+ * row-major, fp32 accumulation.  `naive`: one thread per element, ascending k, bit-identical
+ * to `matmul_fp16_ref` (crates/kernels/src/matmul/cpu.rs:12-30).  `wmma`: the matrix-core
+ * version (CDNA4 MFMA here; any M, N, K; a and b 16-byte aligned).  Shape guard of
+ * `check_matmul_shape` (crates/kernels/src/matmul/mod.rs:89-117). */
+logismos_status_t logismos_launch_matmul_naive_fp16(const void* a_fp16, const void* b_fp16,
+                                                    void* d_fp16, int m, int n, int k,
+                                                    logismos_stream_t stream);
+logismos_status_t logismos_launch_matmul_wmma_fp16(const void* a_fp16, const void* b_fp16,
+                                                   void* d_fp16, int m, int n, int k,
+                                                   logismos_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * Decode step: one new token for each of num_seqs <= 32 live sequences through
  * num_layers pre-norm layers (`StellaLayer::forward` order,
  * crates/encoders/src/stella.rs:190-206; attention and SwiGLU arithmetic of

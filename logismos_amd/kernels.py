@@ -69,6 +69,11 @@ _SIGNATURES = {
     "logismos_launch_silu_mul_bf16": (C.c_uint32, [_vp, _vp, _i, _i, _vp]),
     "logismos_launch_cast_f16_bf16": (C.c_uint32, [_vp, _vp, _sz, _vp]),
     "logismos_launch_greedy_f32": (C.c_uint32, [_vp, _vp, _i, _i, _vp]),
+    "logismos_launch_rms_norm_fp16": (C.c_uint32, [_vp, _vp, _vp, _i, _i, _f, _vp]),
+    "logismos_launch_softmax_fp16": (C.c_uint32, [_vp, _vp, _i, _i, _vp]),
+    "logismos_launch_rope_fp16": (C.c_uint32, [_vp, _vp, _i, _i, _i, _i, _vp]),
+    "logismos_launch_matmul_naive_fp16": (C.c_uint32, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "logismos_launch_matmul_wmma_fp16": (C.c_uint32, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "logismos_check_qgemm_q4g128_greedy_shape": (C.c_uint32, [_i, _i, _i, C.c_char_p, _sz]),
     "logismos_qgemm_q4g128_greedy_workspace_bytes": (_sz, [_i, _i, _i]),
     "logismos_launch_qgemm_q4g128_greedy_xprep": (C.c_uint32, [_vp] * 7 + [_i, _i, _i, _vp]),
@@ -354,6 +359,31 @@ def launch_cast_f16_bf16(src, dst, count: int, stream=None) -> None:
 def launch_greedy_f32(logits, out, rows: int, n: int, stream=None) -> None:
     _status("greedy_f32", library().logismos_launch_greedy_f32(
         _ptr(logits), _ptr(out), rows, n, _raw(stream)))
+
+
+# ---- the reference's existing launchers (same names as its Rust wrappers,
+# crates/kernels/src/{rms_norm,softmax,rope,matmul}/mod.rs)
+def launch_rms_norm_fp16(x, w, y, m: int, n: int, eps: float, stream=None) -> None:
+    _status("rms_norm_fp16", library().logismos_launch_rms_norm_fp16(
+        _ptr(x), _ptr(w), _ptr(y), m, n, eps, _raw(stream)))
+
+
+def launch_softmax_fp16(x, y, m: int, n: int, stream=None) -> None:
+    _status("softmax_fp16", library().logismos_launch_softmax_fp16(
+        _ptr(x), _ptr(y), m, n, _raw(stream)))
+
+
+def launch_rope_fp16_in_place(qk, cos_sin, batch: int, seq: int, heads: int, head_dim: int,
+                              stream=None) -> None:
+    _status("rope_fp16", library().logismos_launch_rope_fp16(
+        _ptr(qk), _ptr(cos_sin), batch, seq, heads, head_dim, _raw(stream)))
+
+
+def launch_matmul_fp16(variant: str, a, b, d, m: int, n: int, k: int, stream=None) -> None:
+    """variant: "naive" or "wmma" (`Variant`, crates/kernels/src/matmul/mod.rs:58-69)."""
+    fn = {"naive": library().logismos_launch_matmul_naive_fp16,
+          "wmma": library().logismos_launch_matmul_wmma_fp16}[variant]
+    _status(f"matmul_{variant}_fp16", fn(_ptr(a), _ptr(b), _ptr(d), m, n, k, _raw(stream)))
 
 
 def check_qgemm_q4g128_greedy_shape(b: int, n: int, k: int) -> None:

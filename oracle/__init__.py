@@ -222,6 +222,33 @@ def rms_norm_fp16_ref(x, w, m, n, eps):
     return y.view(np.float16)
 
 
+_cos_sin_table = _sig("oracle_build_cos_sin_table", None, _sz, _sz, C.c_float, _vp)
+_rope_fp16 = _sig("oracle_rope_apply_fp16_ref", None, _vp, _vp, _sz, _sz, _sz, _sz)
+
+
+def build_cos_sin_table(seq, head_dim, theta_base):
+    """`build_cos_sin_table` (crates/kernels/src/rope/cpu.rs:19-40): f32 [seq*head_dim]."""
+    assert head_dim % 2 == 0
+    t = np.empty(seq * head_dim, np.float32)
+    _cos_sin_table(seq, head_dim, theta_base, _p(t))
+    return t
+
+
+def rope_apply_fp16_ref(qk, cos_sin, batch, seq, heads, head_dim):
+    """`rope_apply_fp16_ref` (crates/kernels/src/rope/cpu.rs:56-127), returns the rotated copy;
+    length mismatches are refused as there (:63-84)."""
+    qk = _u16(qk).copy()
+    cos_sin = _f32(cos_sin)
+    if qk.size != batch * seq * heads * head_dim:
+        raise ValueError(f"rope_apply_fp16_ref: qk.len()={qk.size} != batch*seq*heads*head_dim="
+                         f"{batch * seq * heads * head_dim}")
+    if cos_sin.size != seq * head_dim:
+        raise ValueError(f"rope_apply_fp16_ref: cos_sin.len()={cos_sin.size} != seq*head_dim="
+                         f"{seq * head_dim}")
+    _rope_fp16(_p(qk), _p(cos_sin), batch, seq, heads, head_dim)
+    return qk.view(np.float16)
+
+
 # ---------------------------------------------------------------- attention pieces
 _transpose = _sig("oracle_transpose_seq_heads", None, _vp, _vp, _sz, _sz, _sz)
 _merge = _sig("oracle_merge_heads", None, _vp, _vp, _sz, _sz, _sz)

@@ -286,6 +286,42 @@ void oracle_rms_norm_fp16_ref(const uint16_t* x, const uint16_t* w, uint16_t* y,
     }
 }
 
+/* crates/kernels/src/rope/cpu.rs:19-40 -- `[seq][head_dim]` f32, cos at 2i and sin at 2i+1
+ * of row pos; frequency, angle, cos and sin all in f32 as there. */
+void oracle_build_cos_sin_table(size_t seq, size_t head_dim, float theta_base, float* table) {
+    size_t pairs = head_dim / 2;
+    for (size_t pos = 0; pos < seq; ++pos)
+        for (size_t i = 0; i < pairs; ++i) {
+            float e = -(2.0f * (float)i) / (float)head_dim;
+            float freq = powf(theta_base, e);
+            float angle = (float)pos * freq;
+            table[pos * head_dim + 2 * i] = cosf(angle);
+            table[pos * head_dim + 2 * i + 1] = sinf(angle);
+        }
+}
+
+/* crates/kernels/src/rope/cpu.rs:56-127 -- in place on fp16 (B, S, H, D), interleaved pairs. */
+void oracle_rope_apply_fp16_ref(uint16_t* qk, const float* cos_sin, size_t batch, size_t seq,
+                                size_t heads, size_t head_dim) {
+    size_t pairs = head_dim / 2;
+    for (size_t b = 0; b < batch; ++b)
+        for (size_t s = 0; s < seq; ++s) {
+            const float* row = cos_sin + s * head_dim;
+            for (size_t h = 0; h < heads; ++h) {
+                size_t base = ((b * seq + s) * heads + h) * head_dim;
+                for (size_t i = 0; i < pairs; ++i) {
+                    float c = row[2 * i], sn = row[2 * i + 1];
+                    float x0 = oracle_f16_to_f32(qk[base + 2 * i]);
+                    float x1 = oracle_f16_to_f32(qk[base + 2 * i + 1]);
+                    float y0 = x0 * c - x1 * sn;
+                    float y1 = x0 * sn + x1 * c;
+                    qk[base + 2 * i] = oracle_f32_to_f16(y0);
+                    qk[base + 2 * i + 1] = oracle_f32_to_f16(y1);
+                }
+            }
+        }
+}
+
 /* ------------------------------------------------------------------ attention pieces */
 
 /* crates/transformers/src/attention.rs:318-337 -- [seq,heads,d] -> [heads,seq,d] */

@@ -64,6 +64,9 @@ void oracle_matmul_fp16_ref(const uint16_t* a, const uint16_t* b, uint16_t* d, s
 void oracle_softmax_fp16_ref(const uint16_t* x, uint16_t* y, size_t m, size_t n);
 void oracle_rms_norm_fp16_ref(const uint16_t* x, const uint16_t* w, uint16_t* y, size_t m, size_t n,
                               float eps);
+void oracle_build_cos_sin_table(size_t seq, size_t head_dim, float theta_base, float* table);
+void oracle_rope_apply_fp16_ref(uint16_t* qk, const float* cos_sin, size_t batch, size_t seq,
+                                size_t heads, size_t head_dim);
 
 /* ---- attention pieces (crates/transformers/src/attention.rs) */
 void oracle_transpose_seq_heads(const float* x, float* out, size_t seq, size_t heads, size_t d);

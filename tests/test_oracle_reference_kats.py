@@ -273,3 +273,45 @@ def test_parity_metric_matches_reference_definition():
     ma, mr = O.parity_metric([1.0, 0.0005, -2.0], [1.1, 0.0, -2.0])
     assert abs(ma - 0.1) < 1e-6
     assert abs(mr - max(0.1 / 1.1, 0.0005 / 1e-3)) < 1e-5
+
+
+def test_rope_fp16_zero_positions_are_identity():
+    """crates/kernels/src/rope/cpu.rs:133-158"""
+    table = O.build_cos_sin_table(1, 4, 10_000.0)
+    for i, v in enumerate(table):
+        assert abs(v - (1.0 if i % 2 == 0 else 0.0)) < 1e-6
+    orig = np.array([1.0, 2.0, 3.0, 4.0], np.float16)
+    out = O.rope_apply_fp16_ref(orig, table, 1, 1, 1, 4)
+    assert np.array_equal(out.view(np.uint16), orig.view(np.uint16))
+
+
+def test_rope_fp16_table_length_mismatch_is_rejected():
+    """crates/kernels/src/rope/cpu.rs:160-183"""
+    short_table = np.zeros(4, np.float32)  # seq*head_dim = 8, only 4 present
+    qk = np.ones(1 * 2 * 1 * 4, np.float16)
+    with pytest.raises(ValueError, match="cos_sin.len"):
+        O.rope_apply_fp16_ref(qk, short_table, 1, 2, 1, 4)
+
+
+def test_rope_fp16_rotates_interleaved_pairs_by_the_table_angles():
+    # what the reference leaves open, fixed by the mathematics: pair (2i, 2i+1) at position
+    # pos is rotated by pos * theta^(-2i/d); a quarter turn maps (1, 0) to (0, 1); rotating
+    # by the table and by its transpose-in-sign (sin -> -sin) returns the input
+    d, seq = 8, 5
+    table = O.build_cos_sin_table(seq, d, 10_000.0).reshape(seq, d)
+    for pos in range(seq):
+        for i in range(d // 2):
+            ang = pos * 10_000.0 ** (-2.0 * i / d)
+            assert abs(table[pos, 2 * i] - math.cos(ang)) < 1e-5
+            assert abs(table[pos, 2 * i + 1] - math.sin(ang)) < 1e-5
+    quarter = np.zeros((1, 2), np.float32)
+    quarter[0] = [0.0, 1.0]  # cos = 0, sin = 1
+    out = O.rope_apply_fp16_ref(np.array([1.0, 0.0], np.float16), quarter, 1, 1, 1, 2)
+    assert out.tolist() == [0.0, 1.0]
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((2, seq, 3, d)).astype(np.float16)
+    fwd = O.rope_apply_fp16_ref(x, table, 2, seq, 3, d)
+    inv = table.copy()
+    inv[:, 1::2] *= -1
+    back = O.rope_apply_fp16_ref(fwd, inv, 2, seq, 3, d).astype(np.float32)
+    assert np.abs(back.ravel() - x.ravel().astype(np.float32)).max() < 4e-3
