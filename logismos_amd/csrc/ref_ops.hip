@@ -127,47 +127,56 @@ __global__ __launch_bounds__(256) void matmul_naive_fp16_kernel(const __half* __
     d[(int64_t)row * n + col] = __float2half_rn(acc);
 }
 
-// The matrix-core version: a workgroup of four waves owns a 64 x 64 tile of D, each wave a
-// 32 x 32 quarter (one v_mfma_f32_32x32x16_f16 accumulator).  Per 32-wide slab of K the
-// workgroup stages A[64 x 32] and B[32 x 64] in LDS -- B transposed to [n][k] on the way,
-// because the MFMA B operand wants eight consecutive k of one column and B is row-major --
-// and every wave issues two MFMAs.  Rows, columns and k beyond the matrix are zero-filled.
-constexpr int kMmTile = 64, kMmK = 32;
-constexpr int kMmAStride = kMmK + 8;  // halfs per LDS row: 80 bytes, 16-byte reads stay aligned
-constexpr int kMmBStride = kMmK + 8;
+// The matrix-core version: a workgroup of four waves owns a 128 x 128 tile of D, each wave a
+// 64 x 64 quarter (2 x 2 accumulators of v_mfma_f32_32x32x16_f16).  Per 32-wide slab of K the
+// workgroup stages A[128 x 32] and B[32 x 128] in LDS -- B transposed to [n][k] on the way,
+// because the MFMA B operand wants eight consecutive k of one column and B is row-major: two
+// k rows per thread, merged into (k, k+1) words, with the four 16-byte chunks of an LDS row
+// XOR-swizzled by (row / 16) % 4 so that these transposed 4-byte stores are two-way instead
+// of eight-way bank conflicts.  The LDS tiles are double buffered: slab s + 1 is fetched
+// from memory while slab s is multiplied, one barrier per slab.  Rows, columns and k beyond
+// the matrix are zero-filled.
+constexpr int kMmTile = 128, kMmK = 32;
+constexpr int kMmStride = kMmK + 8;  // halfs per LDS row: 80 bytes, 16-byte reads stay aligned
+constexpr int kMmBuf = kMmTile * kMmStride;
 
 __global__ __launch_bounds__(256) void matmul_mfma_fp16_kernel(const _Float16* __restrict__ a,
                                                                const _Float16* __restrict__ b,
                                                                _Float16* __restrict__ d, int m,
                                                                int n, int k) {
-    __shared__ __attribute__((aligned(16))) _Float16 as[kMmTile * kMmAStride];
-    __shared__ __attribute__((aligned(16))) _Float16 bs[kMmTile * kMmBStride];
+    __shared__ __attribute__((aligned(16))) _Float16 as[2 * kMmBuf];
+    __shared__ __attribute__((aligned(16))) _Float16 bs[2 * kMmBuf];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int row0 = blockIdx.y * kMmTile;
     const int col0 = blockIdx.x * kMmTile;
-    const int wr = (wave >> 1) * 32;  // this wave's quarter
-    const int wc = (wave & 1) * 32;
+    const int wr = (wave >> 1) * 64;  // this wave's quarter
+    const int wc = (wave & 1) * 64;
     const int r = lane & 31;
     const int h = lane >> 5;
 
-    float16_t acc;
+    float16_t acc[2][2];
 #pragma unroll
-    for (int e = 0; e < 16; ++e) acc[e] = 0.0f;
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-    // staging roles: A: thread -> (row tid / 4, 8 consecutive k at 8 * (tid % 4));
-    // B: thread -> (k row tid / 8, 8 consecutive columns at 8 * (tid % 8))
+    // staging roles.  A: thread -> rows tid / 4 and tid / 4 + 64, eight consecutive k at
+    // 8 * (tid % 4).  B: thread -> k rows 2 * (tid / 16) and + 1, eight consecutive columns at
+    // 8 * (tid % 16).
     const int a_row = tid >> 2, a_k = (tid & 3) * 8;
-    const int b_k = tid >> 3, b_col = (tid & 7) * 8;
+    const int b_kp = tid >> 4, b_col = (tid & 15) * 8;
     const bool a_vec = (k & 7) == 0, b_vec = (n & 7) == 0;
-
-    for (int k0 = 0; k0 < k; k0 += kMmK) {
-        // ---- A slab
-        {
+    half8_t ra[2], rb[2];
+    auto gload = [&](int k0) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
             half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-            const int gr = row0 + a_row, gk = k0 + a_k;
-            if (gr < m) {
+            const int gr = row0 + a_row + 64 * u, gk = k0 + a_k;
+            if (gr < m && gk < k) {
                 const _Float16* src = a + (int64_t)gr * k + gk;
                 if (a_vec && gk + 8 <= k) {
                     v = *reinterpret_cast<const half8_t*>(src);
@@ -177,13 +186,13 @@ __global__ __launch_bounds__(256) void matmul_mfma_fp16_kernel(const _Float16* _
                         if (gk + i < k) v[i] = src[i];
                 }
             }
-            *reinterpret_cast<half8_t*>(as + a_row * kMmAStride + a_k) = v;
+            ra[u] = v;
         }
-        // ---- B slab, transposed into [column][k]
-        {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
             half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-            const int gk = k0 + b_k, gc = col0 + b_col;
-            if (gk < k) {
+            const int gk = k0 + 2 * b_kp + u, gc = col0 + b_col;
+            if (gk < k && gc < n) {
                 const _Float16* src = b + (int64_t)gk * n + gc;
                 if (b_vec && gc + 8 <= n) {
                     v = *reinterpret_cast<const half8_t*>(src);
@@ -193,31 +202,73 @@ __global__ __launch_bounds__(256) void matmul_mfma_fp16_kernel(const _Float16* _
                         if (gc + i < n) v[i] = src[i];
                 }
             }
-#pragma unroll
-            for (int i = 0; i < 8; ++i) bs[(b_col + i) * kMmBStride + b_k] = v[i];
+            rb[u] = v;
         }
-        __syncthreads();
-        // ---- two MFMAs: k = 0..15 and 16..31 of the slab; operand: row / column r, eight
-        // consecutive k at 8h
+    };
+    // LDS column (halfs) of k pair b_kp in a B row whose swizzle key is `key`
+    auto lstore = [&](int buf) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+            *reinterpret_cast<half8_t*>(as + buf * kMmBuf + (a_row + 64 * u) * kMmStride + a_k) =
+                ra[u];
+        const uint4_t lo = __builtin_bit_cast(uint4_t, rb[0]);
+        const uint4_t hi = __builtin_bit_cast(uint4_t, rb[1]);
+        const int key = (b_col >> 4) & 3;  // (row / 16) % 4 of rows b_col .. b_col + 7
+        _Float16* dst =
+            bs + buf * kMmBuf + 8 * ((b_kp >> 2) ^ key) + 2 * (b_kp & 3);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const unsigned sel = (e & 1) ? 0x07060302u : 0x05040100u;
+            const unsigned pr = __builtin_amdgcn_perm(hi[e >> 1], lo[e >> 1], sel);
+            *reinterpret_cast<unsigned*>(dst + (b_col + e) * kMmStride) = pr;
+        }
+    };
+
+    const int slabs = (k + kMmK - 1) / kMmK;
+    gload(0);
+    lstore(0);
+    __syncthreads();
+    for (int sl = 0; sl < slabs; ++sl) {
+        const int buf = sl & 1;
+        if (sl + 1 < slabs) gload((sl + 1) * kMmK);
+        const _Float16* at = as + buf * kMmBuf;
+        const _Float16* bt = bs + buf * kMmBuf;
 #pragma unroll
         for (int kk = 0; kk < kMmK; kk += 16) {
-            const half8_t av =
-                *reinterpret_cast<const half8_t*>(as + (wr + r) * kMmAStride + kk + 8 * h);
-            const half8_t bv =
-                *reinterpret_cast<const half8_t*>(bs + (wc + r) * kMmBStride + kk + 8 * h);
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, bv, acc, 0, 0, 0);
+            half8_t av[2], bv[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+                av[i] = *reinterpret_cast<const half8_t*>(at + (wr + 32 * i + r) * kMmStride + kk +
+                                                          8 * h);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int row = wc + 32 * j + r;
+                bv[j] = *reinterpret_cast<const half8_t*>(
+                    bt + row * kMmStride + 8 * (((kk >> 3) + h) ^ ((row >> 4) & 3)));
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bv[j], acc[i][j], 0,
+                                                                       0, 0);
         }
+        if (sl + 1 < slabs) lstore(buf ^ 1);  // last read of that buffer: before the last barrier
         __syncthreads();
     }
-    // lane (h, r) holds column r, rows 8 * (e / 4) + 4h + e % 4 of its wave's quarter
-    const int gc = col0 + wc + r;
-    if (gc < n) {
+    // lane (h, r) holds column r, rows 8 * (e / 4) + 4h + e % 4 of each 32 x 32 block
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const int gr = row0 + wr + 8 * (e >> 2) + 4 * h + (e & 3);
-            if (gr < m) d[(int64_t)gr * n + gc] = (_Float16)acc[e];
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int gc = col0 + wc + 32 * j + r;
+            if (gc >= n) continue;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int gr = row0 + wr + 32 * i + 8 * (e >> 2) + 4 * h + (e & 3);
+                if (gr < m) d[(int64_t)gr * n + gc] = (_Float16)acc[i][j][e];
+            }
         }
-    }
 }
 
 // `check_matmul_shape` (crates/kernels/src/matmul/mod.rs:89-117)
