@@ -122,26 +122,31 @@ __global__ __launch_bounds__(kPrepThreads) void add_rms_norm_xprep_kernel(
     const int64_t row = blockIdx.x;
     float* hr = h + row * n;
     float v[kPrepMaxPasses][8];
+    float4_t wv[kPrepMaxPasses][2];  // the gains, requested with the first loads, not after the reduction
     float sum_sq = 0.0f;
 #pragma unroll
     for (int p = 0; p < kPrepMaxPasses; ++p) {
         const int j = (p * kPrepThreads + (int)threadIdx.x) * 8;
         if (j < n) {
+            wv[p][0] = *reinterpret_cast<const float4_t*>(w + j);
+            wv[p][1] = *reinterpret_cast<const float4_t*>(w + j + 4);
             const float4_t a = *reinterpret_cast<const float4_t*>(hr + j);
             const float4_t b = *reinterpret_cast<const float4_t*>(hr + j + 4);
             float4_t s0 = a, s1 = b;
-            // h + part 0 + part 1 + ... in this order; four loads in flight per round
-            for (int q0 = 0; q0 < num_parts; q0 += 4) {
-                float4_t t0[4], t1[4];
+            // h + part 0 + part 1 + ... in this order; the loads of six parts in flight per
+            // round (a round is one trip to memory: 4 parts take one, 12 take two)
+            constexpr int R = 6;
+            for (int q0 = 0; q0 < num_parts; q0 += R) {
+                float4_t t0[R], t1[R];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
+                for (int u = 0; u < R; ++u) {
                     const int q = (q0 + u) < num_parts ? (q0 + u) : q0;
                     const float* src = yp + (int64_t)q * part_stride + row * n + j;
                     t0[u] = *reinterpret_cast<const float4_t*>(src);
                     t1[u] = *reinterpret_cast<const float4_t*>(src + 4);
                 }
 #pragma unroll
-                for (int u = 0; u < 4; ++u)
+                for (int u = 0; u < R; ++u)
                     if (q0 + u < num_parts) {
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
@@ -182,8 +187,7 @@ __global__ __launch_bounds__(kPrepThreads) void add_rms_norm_xprep_kernel(
         const bool live = j < n;  // uniform over each group of 16 threads (n % 128 == 0)
         uint4_t o = {0u, 0u, 0u, 0u};
         if (live) {
-            const float4_t w0 = *reinterpret_cast<const float4_t*>(w + j);
-            const float4_t w1 = *reinterpret_cast<const float4_t*>(w + j + 4);
+            const float4_t w0 = wv[p][0], w1 = wv[p][1];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const float lo = v[p][2 * e] * inv * (2 * e < 4 ? w0[2 * e] : w1[2 * e - 4]);
@@ -215,19 +219,29 @@ __global__ __launch_bounds__(256) void silu_mul_xprep_kernel(const float* __rest
 #pragma unroll
         for (int e = 0; e < 8; ++e) g[e] = u[e] = 0.0f;
         const int64_t base = (int64_t)t * 2 * inter + (int64_t)c * 8;
-        for (int q = 0; q < num_parts; ++q) {
-            const float* src = parts + (int64_t)q * part_stride + base;
-            const float4_t g0 = *reinterpret_cast<const float4_t*>(src);
-            const float4_t g1 = *reinterpret_cast<const float4_t*>(src + 4);
-            const float4_t u0 = *reinterpret_cast<const float4_t*>(src + inter);
-            const float4_t u1 = *reinterpret_cast<const float4_t*>(src + inter + 4);
+        // parts are added in order; the loads of four parts are in flight per round
+        for (int q0 = 0; q0 < num_parts; q0 += 4) {
+            float4_t g0[4], g1[4], u0[4], u1[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                g[e] += g0[e];
-                g[4 + e] += g1[e];
-                u[e] += u0[e];
-                u[4 + e] += u1[e];
+            for (int r = 0; r < 4; ++r) {
+                const int q = (q0 + r) < num_parts ? (q0 + r) : q0;
+                const float* src = parts + (int64_t)q * part_stride + base;
+                g0[r] = *reinterpret_cast<const float4_t*>(src);
+                g1[r] = *reinterpret_cast<const float4_t*>(src + 4);
+                u0[r] = *reinterpret_cast<const float4_t*>(src + inter);
+                u1[r] = *reinterpret_cast<const float4_t*>(src + inter + 4);
             }
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (q0 + r < num_parts) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        g[e] += g0[r][e];
+                        g[4 + e] += g1[r][e];
+                        u[e] += u0[r][e];
+                        u[4 + e] += u1[r][e];
+                    }
+                }
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -268,9 +282,21 @@ __global__ __launch_bounds__(64) void rope_kv_write_kernel(
         x0 = bf16_to_f32(qkv[off + i]);
         x1 = bf16_to_f32(qkv[off + i + HALF]);
     } else {
-        for (int q = 0; q < num_parts; ++q) {
-            x0 += qkv_parts[(int64_t)q * part_stride + off + i];
-            x1 += qkv_parts[(int64_t)q * part_stride + off + i + HALF];
+        // parts are added in order; the loads of four parts are in flight per round
+        for (int q0 = 0; q0 < num_parts; q0 += 4) {
+            float a[4], b[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int q = (q0 + r) < num_parts ? (q0 + r) : q0;
+                a[r] = qkv_parts[(int64_t)q * part_stride + off + i];
+                b[r] = qkv_parts[(int64_t)q * part_stride + off + i + HALF];
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (q0 + r < num_parts) {
+                    x0 += a[r];
+                    x1 += b[r];
+                }
         }
     }
     if (head < hq + hkv) {
