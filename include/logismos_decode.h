@@ -650,14 +650,14 @@ logismos_status_t logismos_launch_kv_gather_turbo3_f32(const void* k_pool_t3,
                                                        int num_kv_heads, int block_size,
                                                        logismos_stream_t stream);
 
-/* `logismos_launch_paged_attn_varlen_fp16` over turbo3 pools, for decode rows
- * (every sequence has 0 or 1 new tokens: max_seqlen_q <= 1, else
- * hipErrorInvalidValue): out = softmax(q . K^T * scale) . V with K and V the rows
- * `decode_turbo3_0_head` (crates/quant/src/lib.rs:376-413) would return.  The decode is
- * fused into the gather: since a decoded row is norm * H c with H the orthonormal,
- * symmetric transform of `fwht_128` (:88-113), the kernel transforms each query once,
- * multiplies with the centroid values c (as fp16) and transforms each output once;
- * nothing is decoded to memory.  Same workspace, num_splits and block tables as the
+/* `logismos_launch_paged_attn_varlen_fp16` over turbo3 pools (decode rows and
+ * chunked-prefill rows of one packed batch): out = softmax(q . K^T * scale) . V with K and
+ * V the rows `decode_turbo3_0_head` (crates/quant/src/lib.rs:376-413) would return.  The
+ * decode is fused into the gather: since a decoded row is norm * H c with H the orthonormal,
+ * symmetric transform of `fwht_128` (:88-113), the kernels transform each query once,
+ * multiply with the centroid values c (as fp16) and transform each output once; nothing is
+ * decoded to memory.  The new tokens' rows must already be in the pools
+ * (`logismos_launch_kv_write_turbo3`).  Same workspace, num_splits and block tables as the
  * fp16 entry point; head_dim is 128; fp16 q and out. */
 logismos_status_t logismos_launch_paged_attn_varlen_turbo3(
     const void* q_f16, const void* k_pool_t3, const void* v_pool_t3, const int32_t* block_tables,

@@ -193,6 +193,87 @@ __device__ __forceinline__ void fwht_row(float (&x)[8]) {
     for (int i = 0; i < 8; ++i) x[i] *= 0.08838834764831844f;
 }
 
+// fwht_128 of a column held by the two lanes hl of a column pair (lanes c and c + 32) as
+// x[j][i] = element 16j + 8hl + i (the query layout of the prefill kernel)
+__device__ __forceinline__ void fwht_column_16j_8hl_i(float (&x)[8][8]) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int h = 1; h < 8; h <<= 1)
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if ((i & h) == 0) {
+                    const float a = x[j][i], b = x[j][i + h];
+                    x[j][i] = a + b;
+                    x[j][i + h] = a - b;
+                }
+    const bool hi = (threadIdx.x & 32) != 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float o = shfl_xor_f32(x[j][i], 32);
+            x[j][i] = hi ? o - x[j][i] : x[j][i] + o;
+        }
+#pragma unroll
+    for (int h = 1; h < 8; h <<= 1)
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            if ((j & h) == 0)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float a = x[j][i], b = x[j + h][i];
+                    x[j][i] = a + b;
+                    x[j + h][i] = a - b;
+                }
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[j][i] *= 0.08838834764831844f;
+}
+
+// fwht_128 of a column held by the two lanes hl of a column pair as acc[dt][r] = element
+// 32dt + 8(r / 4) + 4hl + r % 4 (the output layout of the prefill kernel)
+__device__ __forceinline__ void fwht_column_32dt_8rq_4hl_r(float16_t (&acc)[4]) {
+    // bits 0, 1 (r % 4) and 3, 4 (r / 4): slots of one accumulator
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int h = 1; h < 16; h <<= 1)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                if ((r & h) == 0) {
+                    const float a = acc[dt][r], b = acc[dt][r + h];
+                    acc[dt][r] = a + b;
+                    acc[dt][r + h] = a - b;
+                }
+    // bit 2: the lane half
+    const bool hi = (threadIdx.x & 32) != 0;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float o = shfl_xor_f32(acc[dt][r], 32);
+            acc[dt][r] = hi ? o - acc[dt][r] : acc[dt][r] + o;
+        }
+    // bits 5, 6: across the accumulators
+#pragma unroll
+    for (int h = 1; h < 4; h <<= 1)
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+            if ((dt & h) == 0)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float a = acc[dt][r], b = acc[dt + h][r];
+                    acc[dt][r] = a + b;
+                    acc[dt + h][r] = a - b;
+                }
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[dt][r] *= 0.08838834764831844f;
+}
+
 // Output row of a query with no visible key: zeros (softmax over zero columns).
 template <int G>
 __device__ __forceinline__ void attn_write_zero_row(const AttnParams& p, int t, int kvh, int lane) {
@@ -746,7 +827,12 @@ struct PfRegs {
     uint4_t x[2];  // the two keys of this thread's pair
 };
 
-template <int G>
+// T3: the pools are turbo3 pools.  A decoded row is norm * H c (H = fwht_128, orthonormal and
+// symmetric), so the kernel works in the transformed domain like the decode kernels: every
+// query column is transformed once when it is loaded, the movers put norm * centroid values
+// (fp16) into the K and V^T tiles instead of copying fp16 rows, and every output column is
+// transformed back once before it is written.  The tile loop is the same.
+template <int G, bool T3>
 __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const AttnParams p) {
     constexpr int TPW = 32 / G;  // query tokens per wave
     constexpr int QT = kPfWaves * TPW;
@@ -830,6 +916,20 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
 #pragma unroll
         for (int j = 0; j < 8; ++j)
             qreg[j] = col_valid ? *reinterpret_cast<const half8_t*>(qp + 16 * j) : z;
+        if constexpr (T3) {
+            // fwht_128 of the column: element d = 16j + 8hl + i lives in lane half hl,
+            // register j, slot i
+            float x[8][8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) x[j][i] = (float)qreg[j][i];
+            fwht_column_16j_8hl_i(x);
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) qreg[j][i] = (_Float16)x[j][i];
+        }
     }
 
     // ---- tile movement: thread (kp, piece) of a four-wave half carries the 16-byte piece
@@ -871,9 +971,26 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
     const int64_t blk_stride = (int64_t)p.block_size * row_stride;  // elements per block
     const unsigned lane_const = (unsigned)kvh * kHeadDim + 8u * piece;
     const _Float16* pool = moves_v ? p.v_pool : p.k_pool;
+    // turbo3: bytes; the thread's eight values are group piece % 4 of 14-byte block piece / 4
+    // of the 56-byte head row: 3 bytes of indices, read as the dword that starts one byte
+    // before them (it never leaves the block), and the block's fp16 norm
+    const unsigned row_bytes = (unsigned)p.hkv * 56u;
+    const int64_t blk_bytes = (int64_t)p.block_size * row_bytes;
+    const unsigned lane_bytes = (unsigned)kvh * 56u + 14u * (piece >> 2);
     auto gload = [&](const PfAddr& a, PfRegs& r) {
-        const _Float16* pb = pool + (int64_t)a.blk * blk_stride;   // wave-uniform
         const int rel_last = last_key - a.tile * kPfKeys + a.rel0;  // of key kmax - 1
+        if constexpr (T3) {
+            const uint8_t* pb = reinterpret_cast<const uint8_t*>(pool) + (int64_t)a.blk * blk_bytes;
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int rel = min(a.rel0 + 2 * kp + u, rel_last);
+                const uint8_t* src = pb + __umul24((unsigned)rel, row_bytes) + lane_bytes;
+                r.x[u][0] = load_u32_unaligned(src + 1 + 3 * (piece & 3));
+                r.x[u][1] = *reinterpret_cast<const unsigned short*>(src);
+            }
+            return;
+        }
+        const _Float16* pb = pool + (int64_t)a.blk * blk_stride;   // wave-uniform
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             // keys past the end re-read the last streamed key; they are masked below
@@ -882,11 +999,25 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
             r.x[u] = *reinterpret_cast<const uint4_t*>(pb + off);
         }
     };
+    // turbo3: the eight fp16 values norm * centroid of a loaded (indices, norm) pair
+    auto t3_values = [&](const uint4_t& raw) {
+        const half8_t cv = turbo3_decode8(raw[0]);
+        const _Float16 nh = __builtin_bit_cast(_Float16, (unsigned short)raw[1]);
+        half8_t o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = cv[i] * nh;
+        return __builtin_bit_cast(uint4_t, o);
+    };
     // column (in halfs) of this thread's key pair inside a V^T row (see lstore)
     const int vt_pos = ((2 * kp) & ~12) | (((2 * kp) & 4) << 1) | (((2 * kp) & 8) >> 1);
     const int vt_col = 8 * ((vt_pos >> 3) ^ ((piece >> 1) & 3)) + (vt_pos & 7);
     // K rows as they are; V transposed, (key 2kp, key 2kp+1) of element e as one word
-    auto lstore = [&](int buf, const PfRegs& r) {
+    auto lstore = [&](int buf, const PfRegs& raw) {
+        PfRegs r = raw;
+        if constexpr (T3) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u) r.x[u] = t3_values(raw.x[u]);
+        }
         if (!moves_v) {
             _Float16* ks = Ks + buf * kKsElems;
 #pragma unroll
@@ -1100,6 +1231,12 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
         __syncthreads();  // the staging below reuses the K / V buffers
     }
 
+    if constexpr (T3) {
+        // back from the transformed domain: fwht_128 of every output column; element
+        // d = 32dt + 8(r / 4) + 4hl + r % 4 lives in lane half hl, accumulator dt, slot r
+        fwht_column_32dt_8rq_4hl_r(oacc);
+    }
+
     // ---- normalise, stage through this wave's LDS slice (16 columns at a time), write
     // 16-byte pieces
     unsigned short* stage_u = reinterpret_cast<unsigned short*>(smem) + w * 16 * kStageStride;
@@ -1157,11 +1294,11 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
     }
 }
 
-template <int G>
+template <int G, bool T3>
 static void launch_prefill(const AttnParams& p, int max_seqlen_q, hipStream_t stream) {
     constexpr int QT = kPfWaves * (32 / G);
     dim3 grid(p.hkv, (max_seqlen_q + QT - 1) / QT, p.num_seqs);
-    paged_attn_prefill_kernel<G><<<grid, dim3(64 * kPfWaves), 0, stream>>>(p);
+    paged_attn_prefill_kernel<G, T3><<<grid, dim3(64 * kPfWaves), 0, stream>>>(p);
 }
 
 // Small batches stay on the static split: when every partition of every sequence is
@@ -1215,10 +1352,8 @@ static hipError_t launch_group(const AttnParams& p, int max_seqlen_q, int phases
             paged_attn_kernel<G, T3><<<grid_d, block, 0, stream>>>(p);
         }
     }
-    if constexpr (!T3) {
-        if ((phases & LOGISMOS_ATTN_PHASE_PREFILL) && max_seqlen_q > 1)
-            launch_prefill<G>(p, max_seqlen_q, stream);
-    }
+    if ((phases & LOGISMOS_ATTN_PHASE_PREFILL) && max_seqlen_q > 1)
+        launch_prefill<G, T3>(p, max_seqlen_q, stream);
     if ((phases & LOGISMOS_ATTN_PHASE_MERGE) && p.num_splits > 1) {
         dim3 grid_m(p.hq, p.num_seqs);
         paged_attn_merge_kernel<<<grid_m, dim3(256), 0, stream>>>(p);
@@ -1354,7 +1489,6 @@ logismos_status_t lg::paged_attn_launch(
     int num_seqs, int total_tokens, int max_seqlen_q, int num_q_heads, int num_kv_heads,
     int head_dim, int block_size, int max_blocks_per_seq, int num_splits, float scale, int causal,
     int phases, int out_bf16, int kv_turbo3, logismos_stream_t stream) {
-    if (kv_turbo3 && max_seqlen_q > 1) return hipErrorInvalidValue;  // decode rows only
     if (logismos_check_paged_attn_shape(num_seqs, total_tokens, max_seqlen_q, num_q_heads,
                                         num_kv_heads, head_dim, block_size, max_blocks_per_seq,
                                         num_splits, nullptr, 0) != 0)

@@ -185,12 +185,42 @@ def test_turbo3_attention_tracks_fp16_attention_over_the_same_rows():
     assert np.abs(got - ref).max() < 0.35 and np.corrcoef(got.ravel(), ref.ravel())[0, 1] > 0.8
 
 
-def test_turbo3_attention_rejects_prefill_rows():
-    rng = np.random.default_rng(73)
-    c = workloads.paged_case(rng, [1, 4], [10, 20], hq=4, hkv=2)
+@pytest.mark.parametrize("hq,hkv", [(4, 4), (8, 2), (12, 2), (32, 8), (14, 2)])
+def test_turbo3_chunked_prefill_rows(hq, hkv):
+    # chunks on both sides of the query-tile and key-tile edges, with and without prior
+    # context, next to decode rows: the movers decode turbo3 rows into the K / V^T tiles
+    rng = np.random.default_rng(75 + hq + hkv)
+    new = [31, 1, 32, 33, 2, 64, 65, 129, 7]
+    prior = [0, 77, 5, 100, 31, 0, 333, 17, 1]
+    c = workloads.paged_case(rng, new, prior, hq=hq, hkv=hkv)
     kp, vp = _turbo3_pools(c)
-    with pytest.raises(kernels.LaunchError):
-        _attn_turbo3(c, kp, vp)
+    want = _oracle_t3(c, kp, vp)
+    assert_parity(_attn_turbo3(c, kp, vp), want, what=f"turbo3 prefill {hq}/{hkv}")
+
+
+def test_turbo3_prefill_512_token_chunks_and_block_sizes():
+    rng = np.random.default_rng(76)
+    c = workloads.paged_case(rng, [512, 1, 200, 1], [0, 700, 1000, 12], hq=32, hkv=8)
+    kp, vp = _turbo3_pools(c)
+    assert_parity(_attn_turbo3(c, kp, vp), _oracle_t3(c, kp, vp), what="turbo3 512-token chunks")
+    for bs in (32, 128):
+        c = workloads.paged_case(rng, [100, 1, 40], [300, 50, 0], hq=8, hkv=2, block_size=bs)
+        kp, vp = _turbo3_pools(c)
+        assert_parity(_attn_turbo3(c, kp, vp), _oracle_t3(c, kp, vp),
+                      what=f"turbo3 prefill block {bs}")
+
+
+def test_turbo3_prefill_chunk_of_one_row_agrees_with_the_decode_kernel():
+    # the same (query, visible keys) through both kernels: a 2-token chunk's last row against
+    # a decode row over the same context
+    rng = np.random.default_rng(77)
+    c2 = workloads.paged_case(rng, [2], [300], hq=8, hkv=2)
+    kp, vp = _turbo3_pools(c2)
+    got2 = _attn_turbo3(c2, kp, vp).astype(np.float32)
+    c1 = dict(c2, new_tokens=np.array([1], np.int32), cu_seqlens=np.array([0, 1], np.int32),
+              q=np.ascontiguousarray(c2["q"][1:2]))
+    got1 = _attn_turbo3(c1, kp, vp).astype(np.float32)
+    assert_parity(got2[1:2], got1, what="turbo3 prefill row vs decode row")
 
 
 def test_put_encode_then_attend_round_trip_on_the_gpu():
