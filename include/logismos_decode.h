@@ -182,8 +182,12 @@ logismos_status_t logismos_launch_qgemm_q4g128_f32_splitk(const void* x_bf16, co
  *   float xg[K/128][BP]  sum of the bf16 values of each group of 128, after xp.
  * `logismos_q4_xprep_bytes` sizes the buffer, `logismos_launch_q4_prepare_x_bf16`
  * converts a plain bf16 `[b][K]` matrix, `..._splitk_xprep` consumes it.  The
- * step operators below can emit it directly (`out_prepared != 0`). */
+ * step operators below can emit it directly (`out_prepared != 0`).  With x
+ * prepared, other kernels become possible (x held in registers, a workgroup
+ * covering 2048 or 4096 columns of K), so the number of parts of this entry
+ * point is its own: `logismos_qgemm_q4g128_splitk_xprep_parts`. */
 size_t logismos_q4_xprep_bytes(int b, int k);
+int logismos_qgemm_q4g128_splitk_xprep_parts(int b, int n, int k);
 logismos_status_t logismos_launch_q4_prepare_x_bf16(const void* x_bf16, void* x_prepared, int b,
                                                     int k, logismos_stream_t stream);
 logismos_status_t logismos_launch_qgemm_q4g128_f32_splitk_xprep(

@@ -35,10 +35,10 @@ Workspace carve(const logismos_decode_config_t& c, int b, int num_splits, char* 
     };
     const size_t qd = (size_t)c.num_q_heads * c.head_dim;
     const size_t kvd = (size_t)c.num_kv_heads * c.head_dim;
-    w.j_qkv = logismos_qgemm_q4g128_splitk_parts(b, (int)(qd + 2 * kvd), c.hidden);
-    w.j_o = logismos_qgemm_q4g128_splitk_parts(b, c.hidden, (int)qd);
-    w.j_gu = logismos_qgemm_q4g128_splitk_parts(b, 2 * c.intermediate, c.hidden);
-    w.j_down = logismos_qgemm_q4g128_splitk_parts(b, c.hidden, c.intermediate);
+    w.j_qkv = logismos_qgemm_q4g128_splitk_xprep_parts(b, (int)(qd + 2 * kvd), c.hidden);
+    w.j_o = logismos_qgemm_q4g128_splitk_xprep_parts(b, c.hidden, (int)qd);
+    w.j_gu = logismos_qgemm_q4g128_splitk_xprep_parts(b, 2 * c.intermediate, c.hidden);
+    w.j_down = logismos_qgemm_q4g128_splitk_xprep_parts(b, c.hidden, c.intermediate);
     const int j_proj = w.j_o > w.j_down ? w.j_o : w.j_down;
     w.xn = take(logismos_q4_xprep_bytes(b, c.hidden));
     w.qkv = take((size_t)w.j_qkv * b * (qd + 2 * kvd) * 4);

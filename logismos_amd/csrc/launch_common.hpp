@@ -23,7 +23,7 @@ inline logismos_status_t reject(char* msg, size_t cap, const char* fmt, ...) {
 
 // Library-internal form of the paged-attention launcher: the public one with the
 // output element type selectable (fp16, or bf16 for the step executor) and the pools either
-// fp16 or turbo3 (kv_turbo3 != 0: decode rows only).
+// fp16 or turbo3 (kv_turbo3 != 0).
 logismos_status_t paged_attn_launch(
     const void* q_f16, const void* k_pool_f16, const void* v_pool_f16, const int32_t* block_tables,
     const int32_t* cu_seqlens_q, const int32_t* context_lens, void* out, void* workspace,
@@ -38,5 +38,19 @@ int stream_steps(int b, int n, int k);
 hipError_t qgemm_q4_stream_launch(const void* xprep, const void* qw, const void* scale,
                                   const void* zero, void* part, int b, int n, int k, int steps,
                                   hipStream_t stream);
+
+// Q4G128 GEMM with x in registers and the weights streamed through LDS
+// (qgemm_q4_regx.hip): the plan for a shape (parts == 0: not applicable) and the launch.
+struct RegxPlan {
+    int rows;   // weight rows per tile: 16 (up to 16 batch rows) or 32
+    int gs;     // groups per wave slice; a workgroup covers 8 * gs groups of K
+    int tpw;    // tiles per workgroup
+    int ring;   // tiles a wave keeps in flight
+    int parts;  // K parts = (K / 128) / (8 * gs)
+};
+RegxPlan regx_plan(int b, int n, int k);
+hipError_t qgemm_q4_regx_launch(const RegxPlan& plan, const void* xprep, const void* qw,
+                                const void* scale, const void* zero, void* part, int b, int n,
+                                int k, hipStream_t stream);
 
 }  // namespace lg

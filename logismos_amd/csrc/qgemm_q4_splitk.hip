@@ -311,6 +311,12 @@ extern "C" int logismos_qgemm_q4g128_splitk_parts(int b, int n, int k) {
     return lg::splitk_plan(b, n, k).parts;
 }
 
+extern "C" int logismos_qgemm_q4g128_splitk_xprep_parts(int b, int n, int k) {
+    if (logismos_check_qgemm_q4g128_shape(b, n, k, nullptr, 0) != 0) return 0;
+    if (const lg::RegxPlan rp = lg::regx_plan(b, n, k); rp.parts > 0) return rp.parts;
+    return lg::splitk_plan(b, n, k).parts;
+}
+
 static logismos_status_t splitk_dispatch(const void* x, bool prepared, const void* qw_u8,
                                          const void* scale_f16, const void* zero_f16,
                                          void* parts_f32, int b, int n, int k,
@@ -322,6 +328,8 @@ static logismos_status_t splitk_dispatch(const void* x, bool prepared, const voi
     const lg::SplitkPlan plan = lg::splitk_plan(b, n, k);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (prepared) {
+        if (const lg::RegxPlan rp = lg::regx_plan(b, n, k); rp.parts > 0)
+            return lg::qgemm_q4_regx_launch(rp, x, qw_u8, scale_f16, zero_f16, parts_f32, b, n, k, st);
         if (const int steps = lg::stream_steps(b, n, k))
             return lg::qgemm_q4_stream_launch(x, qw_u8, scale_f16, zero_f16, parts_f32, b, n, k,
                                               steps, st);

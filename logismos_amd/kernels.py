@@ -82,6 +82,7 @@ _SIGNATURES = {
     "logismos_decode_step_workspace_bytes": (_sz, [_vp, _i, _i]),
     "logismos_launch_decode_step": (C.c_uint32, [_vp, _vp, _vp, _vp, _vp]),
     "logismos_qgemm_q4g128_splitk_parts": (C.c_int, [_i, _i, _i]),
+    "logismos_qgemm_q4g128_splitk_xprep_parts": (C.c_int, [_i, _i, _i]),
     "logismos_launch_qgemm_q4g128_f32_splitk": (C.c_uint32, [_vp] * 5 + [_i, _i, _i, _vp]),
     "logismos_launch_add_rms_norm_f32p": (C.c_uint32, [_vp, _vp, _i, _vp, _vp, _i, _i, _f, _vp]),
     "logismos_launch_rope_kv_write_f32p": (C.c_uint32, [_vp, _i] + [_vp] * 7 + [_i] * 5 + [_vp]),
@@ -421,7 +422,9 @@ def launch_decode_step(cfg: DecodeConfig, layers, batch: DecodeBatch, workspace,
         C.byref(cfg), C.cast(layers, _vp), C.byref(batch), _ptr(workspace), _raw(stream)))
 
 
-def qgemm_q4g128_splitk_parts(b: int, n: int, k: int) -> int:
+def qgemm_q4g128_splitk_parts(b: int, n: int, k: int, prepared: bool = False) -> int:
+    if prepared:
+        return library().logismos_qgemm_q4g128_splitk_xprep_parts(b, n, k)
     return library().logismos_qgemm_q4g128_splitk_parts(b, n, k)
 
 

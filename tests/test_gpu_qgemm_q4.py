@@ -101,7 +101,7 @@ def test_batch_rows_are_independent():
 def _run_splitk(x_f32, qw, s, z, b, n, k, prepared=False):
     from logismos_amd import hip, kernels
     xb = O.f32_to_bf16_bits(x_f32[:b])
-    j = kernels.qgemm_q4g128_splitk_parts(b, n, k)
+    j = kernels.qgemm_q4g128_splitk_parts(b, n, k, prepared)
     assert j >= 1
     d_parts = hip.DeviceBuffer(j * b * n * 4)
     d_parts.fill(0xFF)
@@ -143,11 +143,13 @@ def test_splitk_ragged_shapes(b, n, k):
     assert_parity(got, want, max_abs=2e-4, max_rel=1e-3, what=f"split-K {b}x{n}x{k} (J={j})")
 
 
-@pytest.mark.parametrize("b,n,k", [(32, 6144, 4096), (5, 16, 128), (17, 33, 384),
-                                   (16, 1000, 1152), (31, 4100, 2048),
+@pytest.mark.parametrize("b,n,k", [(5, 16, 128), (17, 33, 384), (16, 1000, 1152), (2, 12288, 4096),
+                                   (32, 1000, 4096),
                                    # streaming kernel, one batch tile (same MFMA shape)
-                                   (16, 24576, 4096), (7, 45003, 1024), (3, 12288, 4096)])
+                                   (7, 45003, 1024), (16, 24576, 1024)])
 def test_splitk_with_prepared_x_is_bit_identical(b, n, k):
+    # shapes that stay on the split-K / streaming kernels (K not a multiple of 2048, fewer
+    # than 3 batch rows or fewer than 1024 weight rows): the same arithmetic in the same order
     rng = np.random.default_rng(b * 1000003 + n * 101 + k + 1)
     w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
     x = rng.standard_normal((b, k), np.float32)
@@ -158,11 +160,10 @@ def test_splitk_with_prepared_x_is_bit_identical(b, n, k):
     assert_parity(prep, want, max_abs=2e-4, max_rel=1e-3, what="split-K, prepared x")
 
 
-@pytest.mark.parametrize("b,n,k", [(32, 24576, 4096), (32, 4096, 12288), (32, 24570, 2048),
-                                   (17, 45003, 1024), (25, 12288, 4096)])
+@pytest.mark.parametrize("b,n,k", [(17, 45003, 1024), (32, 24576, 1024), (25, 16384, 3072)])
 def test_streaming_kernel_with_two_batch_tiles(b, n, k):
-    # batch 17..32 on the large shapes: against the oracle and the plain-x path, whole and
-    # ragged row tiles, one to twelve K parts
+    # batch 17..32 on large shapes whose K is a multiple of 1024 only: against the oracle and
+    # the plain-x path, whole and ragged row tiles
     rng = np.random.default_rng(b * 1000003 + n * 101 + k + 2)
     w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
     x = rng.standard_normal((b, k), np.float32)
@@ -172,3 +173,42 @@ def test_streaming_kernel_with_two_batch_tiles(b, n, k):
     assert j == k // 1024
     assert_parity(prep, want, max_abs=2e-4, max_rel=1e-3, what="streaming kernel vs oracle")
     assert_parity(prep, plain, max_abs=5e-5, max_rel=1e-4, what="streaming vs split-K kernel")
+
+
+@pytest.mark.parametrize("b,n,k,parts", [
+    # the step's four projections at batch 32: 32-row tiles, slices of two groups up to
+    # K = 4096 (two parts), of four beyond (three parts)
+    (32, 6144, 4096, 2), (32, 4096, 4096, 2), (32, 24576, 4096, 2), (32, 4096, 12288, 3),
+    # ragged: last tile short, batch rows short of the tile, one tile per workgroup
+    (31, 4100, 2048, 1), (17, 1030, 8192, 2), (25, 12289, 4096, 2), (20, 1024, 6144, 3),
+    # up to 16 batch rows: 16-row tiles
+    (16, 24576, 4096, 2), (3, 12288, 4096, 2), (9, 2001, 6144, 3), (12, 5000, 12288, 3),
+    (16, 70000, 2048, 1)])
+def test_register_x_kernels_match_oracle_and_split_k(b, n, k, parts):
+    # x in registers, weights through the LDS ring: against the oracle and the plain-x path.
+    # The zero-point term is summed apart from the products here (one fp32 MFMA per tile), so
+    # the two kernels agree to fp32 rounding, not bit for bit.
+    rng = np.random.default_rng(b * 1000003 + n * 101 + k + 3)
+    w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
+    x = rng.standard_normal((b, k), np.float32)
+    qw, s, z = O.quantize_q4g128(w, n, k)
+    plain, want, _ = _run_splitk(x, qw, s, z, b, n, k)
+    prep, _, j = _run_splitk(x, qw, s, z, b, n, k, prepared=True)
+    assert j == parts
+    assert_parity(prep, want, max_abs=2e-4, max_rel=1e-3, what="register-x kernel vs oracle")
+    assert_parity(prep, plain, max_abs=5e-5, max_rel=1e-4, what="register-x vs split-K kernel")
+
+
+def test_register_x_kernel_rows_do_not_depend_on_the_batch():
+    # a batch row's result is the same whatever its neighbours are and wherever it sits,
+    # within one kernel (32-row tiles) and across the two (16- and 32-row tiles)
+    b, n, k = 32, 4096, 4096
+    rng = np.random.default_rng(77)
+    w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
+    x = rng.standard_normal((b, k), np.float32)
+    qw, s, z = O.quantize_q4g128(w, n, k)
+    full, _, _ = _run_splitk(x, qw, s, z, 32, n, k, prepared=True)
+    part, _, _ = _run_splitk(x[5:25], qw, s, z, 20, n, k, prepared=True)
+    assert np.array_equal(full[5:25], part)
+    small, _, _ = _run_splitk(x[8:20], qw, s, z, 12, n, k, prepared=True)
+    assert_parity(small, full[8:20], max_abs=5e-5, max_rel=1e-4, what="16-row vs 32-row tiles")
