@@ -384,7 +384,7 @@ def bench_q4(args):
         ms, _, _ = time_launches(stream, [(lambda q=q: r.launch(qw=q)) for q in qws], args.steps,
                                  args.warmup)
         out[f"b{b}"] = {"us": round(ms * 1e3, 2), "GBps": round(algo / ms / 1e6, 1),
-                        "kernel": "gemv" if b <= 2 else "mfma"}
+                        "kernel": "gemv (VALU dot2)" if b <= 2 else "mfma, x in registers, weights through an LDS ring"}
         del r, qws
     # the same matrix size as ggml Q4_0 weights through the Q4G32 GEMV (x fp32, batch 1)
     qw32 = hip.DeviceBuffer.from_numpy(qw)

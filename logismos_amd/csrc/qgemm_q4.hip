@@ -438,8 +438,12 @@ static logismos_status_t qgemm_q4_dispatch(const void* x_bf16, const void* qw_u8
         switch (b) {
             case 1: return lg::launch_gemv_b<1>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, n, k, st);
             case 2: return lg::launch_gemv_b<2>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, n, k, st);
-            default: break;  // batch 3 and 4: the MFMA kernel is faster (measured crossover)
+            default: break;  // batch 3 and 4: the MFMA kernels are faster (measured crossover)
         }
+        // K = 2048 / 4096: x in registers, weights through the LDS ring, one workgroup per K
+        if (const lg::RegxPlan rp = lg::regx_plain_plan(b, n, k); rp.parts == 1)
+            return lg::qgemm_q4_regx_plain_launch(rp, x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, b, n,
+                                                  k, st);
     }
     if (b <= 16)
         return lg::launch_mfma<1, 2>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, b, n, k, st);

@@ -67,7 +67,7 @@ __host__ __device__ constexpr int regx_lds_bytes(int bt, int gs, int ring) {
     return kRegxWaves * ring * regx_tile_bytes(gs) + (regx_batch_tiles(gs) / 2) * kRegxWaves * bt * 1024;
 }
 
-template <int BT, int GS>
+template <int BT, int GS, bool PLAIN>
 __global__ __launch_bounds__(64 * kRegxWaves) void qgemm_q4g128_regx_kernel(
     const uint4_t* __restrict__ xprep, const uint8_t* __restrict__ qw,
     const __half* __restrict__ scale, const __half* __restrict__ zero, float* __restrict__ part,
@@ -143,14 +143,29 @@ __global__ __launch_bounds__(64 * kRegxWaves) void qgemm_q4g128_regx_kernel(
     // the zero-point term, are the A operand of one fp32 MFMA per tile (K = 4 = groups).
     uint4_t xr[GS][4][BT];
     float xs[BT];
+    if constexpr (PLAIN) {
+        // x as a plain bf16 [b][K] matrix: the 16 bytes of a chunk are contiguous there
+        const uint16_t* xp = reinterpret_cast<const uint16_t*>(xprep);
 #pragma unroll
-    for (int i = 0; i < GS; ++i)
+        for (int bt = 0; bt < BT; ++bt) {
+            const int row = bt * 16 + col;
+            const uint16_t* xrow = xp + (int64_t)min(row, b - 1) * k;
 #pragma unroll
-        for (int s4 = 0; s4 < 4; ++s4)
+            for (int i = 0; i < GS; ++i)
 #pragma unroll
-            for (int bt = 0; bt < BT; ++bt)
-                xr[i][s4][bt] = xprep[(16 * (g0 + i) + 4 * kc + s4) * BP + bt * 16 + col];
-    {
+                for (int s4 = 0; s4 < 4; ++s4) {
+                    const uint4_t v = *reinterpret_cast<const uint4_t*>(xrow + 8 * (16 * (g0 + i) + 4 * kc + s4));
+                    xr[i][s4][bt] = row < b ? v : uint4_t{0u, 0u, 0u, 0u};
+                }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < GS; ++i)
+#pragma unroll
+            for (int s4 = 0; s4 < 4; ++s4)
+#pragma unroll
+                for (int bt = 0; bt < BT; ++bt)
+                    xr[i][s4][bt] = xprep[(16 * (g0 + i) + 4 * kc + s4) * BP + bt * 16 + col];
         const float* xg_src = reinterpret_cast<const float*>(
             reinterpret_cast<const char*>(xprep) + xprep_xg_offset(b, k));
 #pragma unroll
@@ -165,6 +180,26 @@ __global__ __launch_bounds__(64 * kRegxWaves) void qgemm_q4g128_regx_kernel(
         for (int s4 = 0; s4 < 4; ++s4)
 #pragma unroll
             for (int bt = 0; bt < BT; ++bt) asm volatile("" : "+v"(xr[i][s4][bt]));
+    if constexpr (PLAIN) {
+        // group sums: a lane holds a quarter of each group's chunks of its batch row, the
+        // lanes 16, 32 and 48 further on the rest; then pair order for the MFMA operand
+#pragma unroll
+        for (int bt = 0; bt < BT; ++bt) {
+            float mine = 0.0f;
+#pragma unroll
+            for (int i = 0; i < GS; ++i) {
+                float part_sum = 0.0f;
+#pragma unroll
+                for (int s4 = 0; s4 < 4; ++s4) part_sum += sum8_bf16(xr[i][s4][bt]);
+                part_sum += __shfl_xor(part_sum, 16);
+                part_sum += __shfl_xor(part_sum, 32);
+                if (kc == i) mine = part_sum;
+#pragma unroll
+                for (int s4 = 0; s4 < 4; ++s4) xr[i][s4][bt] = pair_order(xr[i][s4][bt]);
+            }
+            xs[bt] = mine;
+        }
+    }
 #pragma unroll
     for (int bt = 0; bt < BT; ++bt) asm volatile("" : "+v"(xs[bt]));
     for (int s = 1; s < ahead; ++s) request_tile(t_begin + s, s);
@@ -333,7 +368,13 @@ __global__ __launch_bounds__(64 * kRegxWaves) void qgemm_q4g128_regx_kernel(
                             : "memory");
                     const float sum = ((((((v0 + v1) + v2) + v3) + v4) + v5) + v6) + v7;
                     const int row = (t_begin + s) * 16 + col;
-                    if (row < n && bi < b) pbase[(unsigned)bi * (unsigned)n + (unsigned)row] = sum;
+                    if (row < n && bi < b) {
+                        if constexpr (PLAIN)
+                            reinterpret_cast<unsigned short*>(part)[(unsigned)bi * (unsigned)n + (unsigned)row] =
+                                f32_to_bf16_rne(sum);
+                        else
+                            pbase[(unsigned)bi * (unsigned)n + (unsigned)row] = sum;
+                    }
                 }
             }
             // the next exchange writes the same buffers
@@ -355,7 +396,7 @@ __host__ __device__ constexpr int regx32_lds_bytes(int gs, int ring) {
 
 typedef float float2_t __attribute__((ext_vector_type(2)));
 
-template <int GS>
+template <int GS, bool PLAIN>
 __global__ __launch_bounds__(64 * kRegxWaves) void qgemm_q4g128_regx32_kernel(
     const uint4_t* __restrict__ xprep, const uint8_t* __restrict__ qw,
     const __half* __restrict__ scale, const __half* __restrict__ zero, float* __restrict__ part,
@@ -431,14 +472,25 @@ __global__ __launch_bounds__(64 * kRegxWaves) void qgemm_q4g128_regx32_kernel(
     // ---- x: A operand of MFMA (group i, half h2, dword d) = chunk 16 (g0 + i) + 8 h2 + 4 kh + d
     uint4_t xr[GS][2][4];
     float xs[GS / 2];
+    if constexpr (PLAIN) {
+        const uint16_t* xrow = reinterpret_cast<const uint16_t*>(xprep) + (int64_t)min(r32, b - 1) * k;
 #pragma unroll
-    for (int i = 0; i < GS; ++i)
+        for (int i = 0; i < GS; ++i)
 #pragma unroll
-        for (int h2 = 0; h2 < 2; ++h2)
+            for (int h2 = 0; h2 < 2; ++h2)
 #pragma unroll
-            for (int d = 0; d < 4; ++d)
-                xr[i][h2][d] = xprep[(16 * (g0 + i) + 8 * h2 + 4 * kh + d) * BP + r32];
-    {
+                for (int d = 0; d < 4; ++d) {
+                    const uint4_t v = *reinterpret_cast<const uint4_t*>(xrow + 8 * (16 * (g0 + i) + 8 * h2 + 4 * kh + d));
+                    xr[i][h2][d] = r32 < b ? v : uint4_t{0u, 0u, 0u, 0u};
+                }
+    } else {
+#pragma unroll
+        for (int i = 0; i < GS; ++i)
+#pragma unroll
+            for (int h2 = 0; h2 < 2; ++h2)
+#pragma unroll
+                for (int d = 0; d < 4; ++d)
+                    xr[i][h2][d] = xprep[(16 * (g0 + i) + 8 * h2 + 4 * kh + d) * BP + r32];
         const float* xg_src = reinterpret_cast<const float*>(
             reinterpret_cast<const char*>(xprep) + xprep_xg_offset(b, k));
 #pragma unroll
@@ -450,6 +502,23 @@ __global__ __launch_bounds__(64 * kRegxWaves) void qgemm_q4g128_regx32_kernel(
         for (int h2 = 0; h2 < 2; ++h2)
 #pragma unroll
             for (int d = 0; d < 4; ++d) asm volatile("" : "+v"(xr[i][h2][d]));
+    if constexpr (PLAIN) {
+        // group sums: this lane holds half of each group's chunks, the lane 32 on the rest
+#pragma unroll
+        for (int i = 0; i < GS; ++i) {
+            float part_sum = 0.0f;
+#pragma unroll
+            for (int h2 = 0; h2 < 2; ++h2)
+#pragma unroll
+                for (int d = 0; d < 4; ++d) part_sum += sum8_bf16(xr[i][h2][d]);
+            part_sum += __shfl_xor(part_sum, 32);
+            if ((i & 1) == kh) xs[i >> 1] = part_sum;
+#pragma unroll
+            for (int h2 = 0; h2 < 2; ++h2)
+#pragma unroll
+                for (int d = 0; d < 4; ++d) xr[i][h2][d] = pair_order(xr[i][h2][d]);
+        }
+    }
 #pragma unroll
     for (int e = 0; e < GS / 2; ++e) asm volatile("" : "+v"(xs[e]));
     for (int s = 1; s < ahead; ++s) request_tile(t_begin + s, s);
@@ -602,8 +671,15 @@ __global__ __launch_bounds__(64 * kRegxWaves) void qgemm_q4g128_regx32_kernel(
                 const float2_t sum = ((((((v0 + v1) + v2) + v3) + v4) + v5) + v6) + v7;
                 const int row = (t_begin + s) * 32 + r32;
                 if (row < n) {
-                    if (m0 < b) pbase[(unsigned)m0 * (unsigned)n + (unsigned)row] = sum[0];
-                    if (m0 + 1 < b) pbase[(unsigned)(m0 + 1) * (unsigned)n + (unsigned)row] = sum[1];
+                    if constexpr (PLAIN) {
+                        unsigned short* y = reinterpret_cast<unsigned short*>(part);
+                        if (m0 < b) y[(unsigned)m0 * (unsigned)n + (unsigned)row] = f32_to_bf16_rne(sum[0]);
+                        if (m0 + 1 < b)
+                            y[(unsigned)(m0 + 1) * (unsigned)n + (unsigned)row] = f32_to_bf16_rne(sum[1]);
+                    } else {
+                        if (m0 < b) pbase[(unsigned)m0 * (unsigned)n + (unsigned)row] = sum[0];
+                        if (m0 + 1 < b) pbase[(unsigned)(m0 + 1) * (unsigned)n + (unsigned)row] = sum[1];
+                    }
                 }
             }
             // the next exchange writes the same buffers
@@ -612,13 +688,13 @@ __global__ __launch_bounds__(64 * kRegxWaves) void qgemm_q4g128_regx32_kernel(
     }
 }
 
-template <int GS>
+template <int GS, bool PLAIN>
 static hipError_t launch_regx32(const void* xprep, const void* qw, const void* scale,
                                 const void* zero, void* part, int b, int n, int k, int tpw,
                                 int ring, hipStream_t stream) {
     const int tiles = (n + 31) / 32;
     const size_t lds = (size_t)regx32_lds_bytes(GS, ring);
-    auto kern = qgemm_q4g128_regx32_kernel<GS>;
+    auto kern = qgemm_q4g128_regx32_kernel<GS, PLAIN>;
     static const hipError_t opt = hipFuncSetAttribute(
         reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
         160 * 1024);
@@ -632,24 +708,28 @@ static hipError_t launch_regx32(const void* xprep, const void* qw, const void* s
 }
 
 static hipError_t qgemm_q4_regx32_launch(const void* xprep, const void* qw, const void* scale,
-                                  const void* zero, void* part, int b, int n, int k, int gs,
-                                  int tpw, int ring, hipStream_t stream) {
+                                         const void* zero, void* part, int b, int n, int k, int gs,
+                                         int tpw, int ring, bool plain, hipStream_t stream) {
     if (gs != 2 && gs != 4) return hipErrorInvalidValue;
     if (b <= 16 || b > 32) return hipErrorInvalidValue;
     if ((k / 128) % (kRegxWaves * gs) != 0 || tpw < 1 || ring < 1 || ring > kRegxMaxRing)
         return hipErrorInvalidValue;
     if (regx32_lds_bytes(gs, ring) > 160 * 1024) return hipErrorInvalidValue;
-    if (gs == 2) return launch_regx32<2>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
-    return launch_regx32<4>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
+    if (plain) {
+        if (gs == 2) return launch_regx32<2, true>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
+        return launch_regx32<4, true>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
+    }
+    if (gs == 2) return launch_regx32<2, false>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
+    return launch_regx32<4, false>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
 }
 
-template <int BT, int GS>
+template <int BT, int GS, bool PLAIN>
 static hipError_t launch_regx(const void* xprep, const void* qw, const void* scale,
                               const void* zero, void* part, int b, int n, int k, int tpw, int ring,
                               hipStream_t stream) {
     const int tiles = (n + 15) / 16;
     const size_t lds = (size_t)regx_lds_bytes(BT, GS, ring);
-    auto kern = qgemm_q4g128_regx_kernel<BT, GS>;
+    auto kern = qgemm_q4g128_regx_kernel<BT, GS, PLAIN>;
     static const hipError_t opt = hipFuncSetAttribute(
         reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
         160 * 1024);
@@ -664,18 +744,18 @@ static hipError_t launch_regx(const void* xprep, const void* qw, const void* sca
 
 static hipError_t qgemm_q4_regx16_launch(const void* xprep, const void* qw, const void* scale,
                                          const void* zero, void* part, int b, int n, int k, int gs,
-                                         int tpw, int ring, hipStream_t stream) {
+                                         int tpw, int ring, bool plain, hipStream_t stream) {
     if (gs != 2 && gs != 4) return hipErrorInvalidValue;
+    if (b < 1 || b > 16) return hipErrorInvalidValue;
     if ((k / 128) % (kRegxWaves * gs) != 0 || tpw < 1 || ring < 1 || ring > kRegxMaxRing)
         return hipErrorInvalidValue;
-    const int bt = b <= 16 ? 1 : 2;
-    if (regx_lds_bytes(bt, gs, ring) > 160 * 1024) return hipErrorInvalidValue;
-    if (b <= 16) {
-        if (gs == 2) return launch_regx<1, 2>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
-        return launch_regx<1, 4>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
+    if (regx_lds_bytes(1, gs, ring) > 160 * 1024) return hipErrorInvalidValue;
+    if (plain) {
+        if (gs == 2) return launch_regx<1, 2, true>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
+        return launch_regx<1, 4, true>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
     }
-    if (gs == 2) return launch_regx<2, 2>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
-    return launch_regx<2, 4>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
+    if (gs == 2) return launch_regx<1, 2, false>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
+    return launch_regx<1, 4, false>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
 }
 
 // Shapes the kernels above take, and how: K a multiple of 2048 (slices of two groups, two
@@ -703,13 +783,41 @@ RegxPlan regx_plan(int b, int n, int k) {
     return p;
 }
 
+// The same kernels reading x as a plain bf16 matrix and writing the bf16 product: possible
+// where one workgroup covers all of K (K = 2048 or 4096), so that there is a single part.
+RegxPlan regx_plain_plan(int b, int n, int k) {
+    RegxPlan p{0, 0, 0, 0, 0};
+    if (k != 2048 && k != 4096) return p;
+    if (b < 3 || b > 32 || n < 1024) return p;
+    p.gs = k / 1024;
+    p.parts = 1;
+    p.rows = b <= 16 ? 16 : 32;
+    p.ring = (p.rows == 16 && p.gs == 2) ? 2 : 1;
+    const int tiles = (n + p.rows - 1) / p.rows;
+    const int columns = device_cu_count();
+    p.tpw = (tiles + columns - 1) / columns;
+    return p;
+}
+
 hipError_t qgemm_q4_regx_launch(const RegxPlan& p, const void* xprep, const void* qw,
                                 const void* scale, const void* zero, void* part, int b, int n,
                                 int k, hipStream_t stream) {
     if (p.rows == 32)
         return qgemm_q4_regx32_launch(xprep, qw, scale, zero, part, b, n, k, p.gs, p.tpw, p.ring,
-                                      stream);
-    return qgemm_q4_regx16_launch(xprep, qw, scale, zero, part, b, n, k, p.gs, p.tpw, p.ring, stream);
+                                      false, stream);
+    return qgemm_q4_regx16_launch(xprep, qw, scale, zero, part, b, n, k, p.gs, p.tpw, p.ring, false,
+                                  stream);
+}
+
+hipError_t qgemm_q4_regx_plain_launch(const RegxPlan& p, const void* x_bf16, const void* qw,
+                                      const void* scale, const void* zero, void* y_bf16, int b,
+                                      int n, int k, hipStream_t stream) {
+    if (p.parts != 1) return hipErrorInvalidValue;
+    if (p.rows == 32)
+        return qgemm_q4_regx32_launch(x_bf16, qw, scale, zero, y_bf16, b, n, k, p.gs, p.tpw, p.ring,
+                                      true, stream);
+    return qgemm_q4_regx16_launch(x_bf16, qw, scale, zero, y_bf16, b, n, k, p.gs, p.tpw, p.ring, true,
+                                  stream);
 }
 
 }  // namespace lg
