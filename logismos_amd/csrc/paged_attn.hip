@@ -315,11 +315,15 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
     half8_t qreg[4];
     {
         const half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
-        const _Float16* qp =
-            p.q + ((int64_t)t * p.hq + kvh * G + (c < G ? c : 0)) * kHeadDim + 8 * tg;
+        // contraction slot j of a lane row tg: piece tg + 4j (turbo3), or piece
+        // 2tg + (j & 1) + 8 (j >> 1) for fp16 pools, where K arrives as whole 128-byte lines
+        const _Float16* qp = p.q + ((int64_t)t * p.hq + kvh * G + (c < G ? c : 0)) * kHeadDim +
+                             (T3 ? 8 * tg : 16 * tg);
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            qreg[j] = (c < G) ? *reinterpret_cast<const half8_t*>(qp + 32 * j) : z;
+            qreg[j] = (c < G) ? *reinterpret_cast<const half8_t*>(
+                                    qp + (T3 ? 32 * j : 8 * (j & 1) + 64 * (j >> 1)))
+                              : z;
         if constexpr (T3) {
             float x[4][8];
 #pragma unroll
@@ -340,7 +344,8 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
 
     // lane-constant element offsets inside a tile (row stride = hkv * 128)
     const unsigned row_stride = (unsigned)p.hkv * kHeadDim;
-    const unsigned k_lane_off = (unsigned)c * row_stride;
+    const unsigned k_half_off[2] = {(unsigned)(c & 7) * row_stride,
+                                    (unsigned)(8 + (c & 7)) * row_stride};
     unsigned v_lane_off[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) v_lane_off[i] = (unsigned)(4 * tg + i) * row_stride;
@@ -382,12 +387,19 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
         // Non-temporal loads: a decode step reads every K/V byte exactly once, and streaming
         // loads measured 7.0 against 6.3 TB/s for plain ones on a read-only sweep
         const unsigned last_off = (unsigned)(tok_end - 1 - tok_base) * row_stride;
-        const unsigned ko = min(k_lane_off, last_off) + 8u * tg;
         if constexpr (!T3) {
+            // K: request j covers keys 8 (j & 1) .. + 7, 128 contiguous bytes each (pieces
+            // 8 (j >> 1) .. + 7): lane (tg, c) fetches piece 2tg + c / 8 + 8 (j >> 1) of key
+            // 8 (j & 1) + c % 8.  Whole cache lines per request, where one request per
+            // 16 keys x 64 bytes touched every line twice; compute_tile swaps halves between
+            // the lanes c and c + 8 to get each key's four pieces into one lane.
+            const unsigned e0 = 16u * tg + 8u * (c >> 3);
+            const unsigned ko0 = min(k_half_off[0], last_off) + e0;
+            const unsigned ko1 = min(k_half_off[1], last_off) + e0;
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                kv.k[j] = __builtin_nontemporal_load(
-                    reinterpret_cast<const half8_t*>(kb + ko + 32 * j));
+                kv.k[j] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(
+                    kb + ((j & 1) ? ko1 : ko0) + 64 * (j >> 1)));
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const unsigned vo = min(v_lane_off[i], last_off) + 8u * c;
@@ -417,6 +429,22 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
             }
         } else {
             kv = raw;
+            // lanes c < 8 keep key c (requests 0, 2) and take its odd pieces from lane c + 8;
+            // lanes c >= 8 keep key c (requests 1, 3) and take its even pieces from lane c - 8
+            constexpr int kRor8 = 0x128;  // row_ror:8
+#pragma unroll
+            for (int x = 0; x < 2; ++x) {
+                uint4_t r0 = __builtin_bit_cast(uint4_t, raw.k[2 * x]);
+                uint4_t r1 = __builtin_bit_cast(uint4_t, raw.k[2 * x + 1]);
+                uint4_t k0, k1;
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    k0[d] = (unsigned)__builtin_amdgcn_update_dpp((int)r0[d], (int)r1[d], kRor8, 0xf, 0xc, false);
+                    k1[d] = (unsigned)__builtin_amdgcn_update_dpp((int)r1[d], (int)r0[d], kRor8, 0xf, 0x3, false);
+                }
+                kv.k[2 * x] = __builtin_bit_cast(half8_t, k0);
+                kv.k[2 * x + 1] = __builtin_bit_cast(half8_t, k1);
+            }
         }
         float4_t sacc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
