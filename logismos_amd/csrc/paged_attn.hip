@@ -5,12 +5,15 @@
 // per group.  Work inside the wave, per tile of 16 keys (a tile never
 // straddles a KV block because block_size % 16 == 0):
 //
-//   * K: lane (tg = lane/16, c = lane%16) loads key c of the tile, 16-byte
-//     pieces tg, tg+4, tg+8, tg+12 of its 256-byte row, straight into the
-//     A-operand layout of v_mfma_f32_16x16x32_f16 (row = key, 8 consecutive
-//     contraction elements per lane).  The query group sits in registers as
-//     the B operand (column = head, same piece order), so four MFMAs give the
-//     16 keys x 16 heads score tile; lane (tg, c) ends up with the scores of
+//   * K: the A operand of v_mfma_f32_16x16x32_f16 wants lane (tg = lane/16, c = lane%16)
+//     to hold key c of the tile, 8 consecutive contraction elements per slot.  fp16 pools:
+//     a request covers 8 keys x 128 contiguous bytes (lane (tg, c): piece 2tg + c/8 of key
+//     c%8, keys 8..15 and the second half of the rows in the other three requests), whole
+//     cache lines, and the lanes c and c + 8 then swap halves (DPP row_ror:8), which leaves
+//     lane (tg, c) with the pieces 2tg, 2tg+1, 2tg+8, 2tg+9 of key c.  turbo3 pools: lane
+//     (tg, c) loads the codes of pieces tg, tg+4, tg+8, tg+12 of key c directly.  The query
+//     group sits in registers as the B operand (column = head, same piece order), so four
+//     MFMAs give the 16 keys x 16 heads score tile; lane (tg, c) ends up with the scores of
 //     head c for keys 4*tg..4*tg+3.
 //   * V: lane (tg, c) loads the 16-byte piece c of keys 4*tg..4*tg+3: each
 //     wave instruction covers four whole 256-byte rows.
