@@ -636,8 +636,9 @@ const int32_t* logismos_paged_kv_cache_block_tables_host(const logismos_paged_kv
  * head_dim is 128 (`TURBOQUANT_HEAD_DIM`). */
 
 /* `encode_turbo3_0_head` (crates/quant/src/lib.rs:316-353) of every head of row t of
- * k_new / v_new (fp16 `[total_tokens][num_kv_heads][128]`, widened to f32), written to pool
- * row slot_mapping[t] (negative: skipped).  Bytes identical to the reference function's. */
+ * k_new / v_new (fp16 `[total_tokens][num_kv_heads][128]`, 16-byte aligned, widened to f32),
+ * written to pool row slot_mapping[t] (negative: skipped).  Bytes identical to the reference
+ * function's. */
 logismos_status_t logismos_launch_kv_write_turbo3(const void* k_new_f16, const void* v_new_f16,
                                                   void* k_pool_t3, void* v_pool_t3,
                                                   const int64_t* slot_mapping, int total_tokens,

@@ -83,6 +83,36 @@ __device__ __forceinline__ float shfl_xor_f32(float v, int mask) {
     return __shfl_xor(v, mask, kWave);
 }
 
+// Value of lane (lane ^ M) for a power of two M, without the LDS crossbar that __shfl_xor
+// goes through: quad permutes (1, 2), two masked row rotations (4: the banks of four lanes
+// with bit 2 clear read four lanes up, the others four lanes down), a row rotation (8), and
+// the gfx950 row / half-wave swaps (16, 32), whose two results hold the upper and the lower
+// partner's values.
+template <int M>
+__device__ __forceinline__ int lane_xor_i32(int v) {
+    static_assert(M == 1 || M == 2 || M == 4 || M == 8 || M == 16 || M == 32, "one bit");
+    if constexpr (M == 1) {
+        return __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, false);  // quad_perm [1,0,3,2]
+    } else if constexpr (M == 2) {
+        return __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, false);  // quad_perm [2,3,0,1]
+    } else if constexpr (M == 4) {
+        const int up = __builtin_amdgcn_update_dpp(0, v, kDppRowRor + 12, 0xf, 0x5, false);
+        return __builtin_amdgcn_update_dpp(up, v, kDppRowRor + 4, 0xf, 0xa, false);
+    } else if constexpr (M == 8) {
+        return __builtin_amdgcn_update_dpp(0, v, kDppRowRor + 8, 0xf, 0xf, false);
+    } else if constexpr (M == 16) {
+        const auto r = __builtin_amdgcn_permlane16_swap((unsigned)v, (unsigned)v, false, false);
+        return (int)((threadIdx.x & 16) ? r[0] : r[1]);
+    } else {
+        const auto r = __builtin_amdgcn_permlane32_swap((unsigned)v, (unsigned)v, false, false);
+        return (int)((threadIdx.x & 32) ? r[0] : r[1]);
+    }
+}
+template <int M>
+__device__ __forceinline__ float lane_xor_f32(float v) {
+    return __int_as_float(lane_xor_i32<M>(__float_as_int(v)));
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 }  // namespace lg

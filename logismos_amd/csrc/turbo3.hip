@@ -21,26 +21,48 @@
 
 namespace lg {
 
-// one wave per (token, kv head, K|V); block = 4 waves
+// One wave per kT3RowsPerWave rows, a row being one (token, kv head, K|V): first a lane per
+// row computes that row's norm on its own (the reference adds the 128 squares one after the
+// other; done across a wave that chain costs 256 dependent instructions per row), then the
+// wave encodes the rows one at a time, lane l holding elements l and l + 64, the next row's
+// elements already requested.  block = 4 waves
+constexpr int kT3RowsPerWave = 16;
+
 __global__ __launch_bounds__(256) void kv_write_turbo3_kernel(
     const _Float16* __restrict__ k_new, const _Float16* __restrict__ v_new,
     uint8_t* __restrict__ k_pool, uint8_t* __restrict__ v_pool,
     const int64_t* __restrict__ slot_mapping, int total_tokens, int hkv) {
+    constexpr int RW = kT3RowsPerWave;
     const int lane = threadIdx.x & 63;
-    const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (item >= (int64_t)total_tokens * hkv * 2) return;
-    const int which = (int)(item & 1);
-    const int64_t th = item >> 1;
-    const int t = (int)(th / hkv);
-    const int h = (int)(th - (int64_t)t * hkv);
-    const int64_t slot = slot_mapping[t];
-    if (slot < 0) return;
-    const _Float16* src = (which ? v_new : k_new) + ((int64_t)t * hkv + h) * 128;
-    float a = (float)src[lane];
-    float b = (float)src[lane + 64];
-
-    uint8_t* dst = (which ? v_pool : k_pool) + (slot * hkv + h) * kTurbo3HeadBytes;
-    turbo3_encode_row(a, b, lane, dst);
+    const int64_t items = (int64_t)total_tokens * hkv * 2;
+    const int64_t first = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * RW;
+    if (first >= items) return;
+    auto source = [&](int64_t item) {
+        const int64_t th = item >> 1;
+        return ((item & 1) ? v_new : k_new) + th * 128;
+    };
+    const int rows = (int)(items - first < RW ? items - first : RW);
+    float my_norm = 0.0f;
+    if (lane < rows) my_norm = turbo3_row_norm_serial(source(first + lane));
+    const _Float16* src = source(first);
+    float a = (float)src[lane], b = (float)src[lane + 64];
+    for (int r = 0; r < rows; ++r) {
+        const int64_t item = first + r;
+        const float norm = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_norm), r));
+        const float ca = a, cb = b;
+        if (r + 1 < rows) {
+            const _Float16* nxt = source(item + 1);
+            a = (float)nxt[lane];
+            b = (float)nxt[lane + 64];
+        }
+        const int64_t th = item >> 1;
+        const int t = (int)(th / hkv);
+        const int h = (int)(th - (int64_t)t * hkv);
+        const int64_t slot = slot_mapping[t];
+        if (slot < 0) continue;  // uniform
+        uint8_t* dst = ((item & 1) ? v_pool : k_pool) + (slot * hkv + h) * kTurbo3HeadBytes;
+        turbo3_encode_row_normed(ca, cb, norm, lane, dst);
+    }
 }
 
 __device__ __forceinline__ unsigned turbo3_index_at(const uint8_t* head, int e) {
@@ -90,8 +112,11 @@ extern "C" logismos_status_t logismos_launch_kv_write_turbo3(
         return hipErrorInvalidValue;
     if ((reinterpret_cast<uintptr_t>(k_pool_t3) | reinterpret_cast<uintptr_t>(v_pool_t3)) & 1u)
         return hipErrorInvalidValue;
+    if ((reinterpret_cast<uintptr_t>(k_new_f16) | reinterpret_cast<uintptr_t>(v_new_f16)) & 15u)
+        return hipErrorInvalidValue;
     const int64_t items = (int64_t)total_tokens * num_kv_heads * 2;
-    lg::kv_write_turbo3_kernel<<<dim3((unsigned)((items + 3) / 4)), dim3(256), 0,
+    const int64_t per_block = 4 * lg::kT3RowsPerWave;
+    lg::kv_write_turbo3_kernel<<<dim3((unsigned)((items + per_block - 1) / per_block)), dim3(256), 0,
                                  static_cast<hipStream_t>(stream)>>>(
         static_cast<const _Float16*>(k_new_f16), static_cast<const _Float16*>(v_new_f16),
         static_cast<uint8_t*>(k_pool_t3), static_cast<uint8_t*>(v_pool_t3), slot_mapping,

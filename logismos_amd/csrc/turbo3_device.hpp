@@ -21,15 +21,22 @@ static __device__ __constant__ const float kTurbo3Codebook[8] = {
 };
 
 // fwht_128 over elements (a = element lane, b = element lane + 64) of a wave
+template <int H>
+__device__ __forceinline__ void wave_fwht_stage(float& a, float& b, int lane) {
+    const float pa = lane_xor_f32<H>(a);
+    const float pb = lane_xor_f32<H>(b);
+    const bool hi = (lane & H) != 0;
+    a = hi ? __fsub_rn(pa, a) : __fadd_rn(a, pa);
+    b = hi ? __fsub_rn(pb, b) : __fadd_rn(b, pb);
+}
+
 __device__ __forceinline__ void wave_fwht_128(float& a, float& b, int lane) {
-#pragma unroll
-    for (int h = 1; h < 64; h <<= 1) {
-        const float pa = shfl_xor_f32(a, h);
-        const float pb = shfl_xor_f32(b, h);
-        const bool hi = (lane & h) != 0;
-        a = hi ? __fsub_rn(pa, a) : __fadd_rn(a, pa);
-        b = hi ? __fsub_rn(pb, b) : __fadd_rn(b, pb);
-    }
+    wave_fwht_stage<1>(a, b, lane);
+    wave_fwht_stage<2>(a, b, lane);
+    wave_fwht_stage<4>(a, b, lane);
+    wave_fwht_stage<8>(a, b, lane);
+    wave_fwht_stage<16>(a, b, lane);
+    wave_fwht_stage<32>(a, b, lane);
     const float x = a, y = b;
     a = __fadd_rn(x, y);
     b = __fsub_rn(x, y);
@@ -52,19 +59,10 @@ __device__ __forceinline__ unsigned turbo3_nearest(float v) {
     return best;
 }
 
-// Encodes the row held as (a, b) by the 64 lanes of a wave into the 56 bytes at dst.
-__device__ __forceinline__ void turbo3_encode_row(float a, float b, int lane, uint8_t* dst) {
-    // L2 norm: squares summed in element order, as the reference's loop does
-    const int asq = __float_as_int(__fmul_rn(a, a));
-    const int bsq = __float_as_int(__fmul_rn(b, b));
-    float sum_sq = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 64; ++i)
-        sum_sq = __fadd_rn(sum_sq, __int_as_float(__builtin_amdgcn_readlane(asq, i)));
-#pragma unroll
-    for (int i = 0; i < 64; ++i)
-        sum_sq = __fadd_rn(sum_sq, __int_as_float(__builtin_amdgcn_readlane(bsq, i)));
-    const float norm = __fsqrt_rn(sum_sq);
+// Encodes the row held as (a, b) by the 64 lanes of a wave into the 56 bytes at dst; `norm`
+// is the row's L2 norm as turbo3_row_norm / turbo3_row_norm_serial compute it.
+__device__ __forceinline__ void turbo3_encode_row_normed(float a, float b, float norm, int lane,
+                                                         uint8_t* dst) {
     const bool live = norm > 1e-12f;
     a = live ? __fdiv_rn(a, norm) : 0.0f;
     b = live ? __fdiv_rn(b, norm) : 0.0f;
@@ -91,12 +89,18 @@ __device__ __forceinline__ void turbo3_encode_row(float a, float b, int lane, ui
         }
     }
 #pragma unroll
-    for (int m = 1; m < 32; m <<= 1)
-#pragma unroll
-        for (int w = 0; w < 3; ++w) {
-            wa[w] |= (unsigned)__shfl_xor((int)wa[w], m, 64);
-            wb[w] |= (unsigned)__shfl_xor((int)wb[w], m, 64);
-        }
+    for (int w = 0; w < 3; ++w) {
+        wa[w] |= (unsigned)lane_xor_i32<1>((int)wa[w]);
+        wb[w] |= (unsigned)lane_xor_i32<1>((int)wb[w]);
+        wa[w] |= (unsigned)lane_xor_i32<2>((int)wa[w]);
+        wb[w] |= (unsigned)lane_xor_i32<2>((int)wb[w]);
+        wa[w] |= (unsigned)lane_xor_i32<4>((int)wa[w]);
+        wb[w] |= (unsigned)lane_xor_i32<4>((int)wb[w]);
+        wa[w] |= (unsigned)lane_xor_i32<8>((int)wa[w]);
+        wb[w] |= (unsigned)lane_xor_i32<8>((int)wb[w]);
+        wa[w] |= (unsigned)lane_xor_i32<16>((int)wa[w]);
+        wb[w] |= (unsigned)lane_xor_i32<16>((int)wb[w]);
+    }
     // halfword p (< 7) of the two 14-byte blocks this half-wave owns: the norm, then the
     // six halfwords of the payload
     if (p < 7) {
@@ -110,6 +114,42 @@ __device__ __forceinline__ void turbo3_encode_row(float a, float b, int lane, ui
         reinterpret_cast<unsigned short*>(dst + kTurbo3BlockBytes * blk_a)[p] = ha;
         reinterpret_cast<unsigned short*>(dst + kTurbo3BlockBytes * blk_b)[p] = hb;
     }
+}
+
+// L2 norm of the row held as (a, b) by a wave: squares summed in element order, as the
+// reference's loop does (128 dependent additions)
+__device__ __forceinline__ float turbo3_row_norm(float a, float b) {
+    const int asq = __float_as_int(__fmul_rn(a, a));
+    const int bsq = __float_as_int(__fmul_rn(b, b));
+    float sum_sq = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 64; ++i)
+        sum_sq = __fadd_rn(sum_sq, __int_as_float(__builtin_amdgcn_readlane(asq, i)));
+#pragma unroll
+    for (int i = 0; i < 64; ++i)
+        sum_sq = __fadd_rn(sum_sq, __int_as_float(__builtin_amdgcn_readlane(bsq, i)));
+    return __fsqrt_rn(sum_sq);
+}
+
+// The same norm computed by ONE lane from the row's 128 fp16 values in memory: 64 lanes do
+// 64 rows at once, which is what makes the dependent chain affordable when many rows are
+// encoded.  `row` is 16-byte aligned.
+__device__ __forceinline__ float turbo3_row_norm_serial(const _Float16* row) {
+    float sum_sq = 0.0f;
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+        const half8_t v = *reinterpret_cast<const half8_t*>(row + 8 * c);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float x = (float)v[e];
+            sum_sq = __fadd_rn(sum_sq, __fmul_rn(x, x));
+        }
+    }
+    return __fsqrt_rn(sum_sq);
+}
+
+__device__ __forceinline__ void turbo3_encode_row(float a, float b, int lane, uint8_t* dst) {
+    turbo3_encode_row_normed(a, b, turbo3_row_norm(a, b), lane, dst);
 }
 
 }  // namespace lg
