@@ -79,9 +79,6 @@ __device__ __forceinline__ float wave_sum(float v) {
            __int_as_float(__builtin_amdgcn_readlane(b, 48));
 }
 
-__device__ __forceinline__ float shfl_xor_f32(float v, int mask) {
-    return __shfl_xor(v, mask, kWave);
-}
 
 // Value of lane (lane ^ M) for a power of two M, without the LDS crossbar that __shfl_xor
 // goes through: quad permutes (1, 2), two masked row rotations (4: the banks of four lanes
@@ -111,6 +108,24 @@ __device__ __forceinline__ int lane_xor_i32(int v) {
 template <int M>
 __device__ __forceinline__ float lane_xor_f32(float v) {
     return __int_as_float(lane_xor_i32<M>(__float_as_int(v)));
+}
+
+// through the LDS crossbar: one instruction and no temporaries, for register-tight kernels
+__device__ __forceinline__ float shfl_xor_lds_f32(float v, int mask) {
+    return __shfl_xor(v, mask, kWave);
+}
+
+// the same for a mask that is a constant once the caller's loop is unrolled
+__device__ __forceinline__ float shfl_xor_f32(float v, int mask) {
+    switch (mask) {
+        case 1: return lane_xor_f32<1>(v);
+        case 2: return lane_xor_f32<2>(v);
+        case 4: return lane_xor_f32<4>(v);
+        case 8: return lane_xor_f32<8>(v);
+        case 16: return lane_xor_f32<16>(v);
+        case 32: return lane_xor_f32<32>(v);
+        default: return __shfl_xor(v, mask, kWave);
+    }
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }

@@ -150,7 +150,7 @@ __device__ __forceinline__ void fwht_pieces(float (&x)[4][8]) {
         for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const float o = shfl_xor_f32(x[j][i], mask);
+                const float o = shfl_xor_lds_f32(x[j][i], mask);
                 x[j][i] = hi ? o - x[j][i] : x[j][i] + o;
             }
     }
@@ -188,7 +188,7 @@ __device__ __forceinline__ void fwht_row(float (&x)[8]) {
         const bool hi = (lane & mask) != 0;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const float o = shfl_xor_f32(x[i], mask);
+            const float o = shfl_xor_lds_f32(x[i], mask);
             x[i] = hi ? o - x[i] : x[i] + o;
         }
     }
@@ -215,7 +215,7 @@ __device__ __forceinline__ void fwht_column_16j_8hl_i(float (&x)[8][8]) {
     for (int j = 0; j < 8; ++j)
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const float o = shfl_xor_f32(x[j][i], 32);
+            const float o = shfl_xor_lds_f32(x[j][i], 32);
             x[j][i] = hi ? o - x[j][i] : x[j][i] + o;
         }
 #pragma unroll
@@ -256,7 +256,7 @@ __device__ __forceinline__ void fwht_column_32dt_8rq_4hl_r(float16_t (&acc)[4]) 
     for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const float o = shfl_xor_f32(acc[dt][r], 32);
+            const float o = shfl_xor_lds_f32(acc[dt][r], 32);
             acc[dt][r] = hi ? o - acc[dt][r] : acc[dt][r] + o;
         }
     // bits 5, 6: across the accumulators
@@ -523,16 +523,16 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
         float lh = row_bcast<h>(l);
 #pragma unroll
         for (int mask = 16; mask <= 32; mask <<= 1) {
-            const float mo = shfl_xor_f32(mh, mask);
+            const float mo = shfl_xor_lds_f32(mh, mask);
             const float mn = fmaxf(mh, mo);
             const float msafe = (mn == -INFINITY) ? 0.0f : mn;
             const float f = fast_exp2(mh - msafe);
             lh *= f;
-            lh += shfl_xor_f32(lh, mask);
+            lh += shfl_xor_lds_f32(lh, mask);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const float v = acc[h][e] * f;
-                acc[h][e] = v + shfl_xor_f32(v, mask);
+                acc[h][e] = v + shfl_xor_lds_f32(v, mask);
             }
             mh = mn;
         }
@@ -1151,7 +1151,7 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
                 tm = fmaxf(tm, sc[r]);
             }
         }
-        tm = fmaxf(tm, shfl_xor_f32(tm, 32)) * p.scale_log2e;
+        tm = fmaxf(tm, lane_xor_f32<32>(tm)) * p.scale_log2e;
         // Lazy reference maximum: the column's exponentials stay relative to m until a
         // tile maximum exceeds it by more than 2^kLazyLog2 (probabilities are then at most
         // 2^kLazyLog2, well inside fp16 and fp32 range), so the accumulators are rescaled
@@ -1271,7 +1271,7 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
     // ---- normalise, stage through this wave's LDS slice (16 columns at a time), write
     // 16-byte pieces
     unsigned short* stage_u = reinterpret_cast<unsigned short*>(smem) + w * 16 * kStageStride;
-    const float lt = l + shfl_xor_f32(l, 32);
+    const float lt = l + lane_xor_f32<32>(l);
     const float inv = lt > 0.0f ? 1.0f / lt : 0.0f;
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf) {
