@@ -601,11 +601,17 @@ __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_kernel(const At
                           num_parts == 1, (int64_t)s * p.num_splits + split);
 }
 
-// 16-key tiles sequence s contributes to the decode stream
+// Units sequence s contributes to the decode stream: its 16-key tiles plus kSeqStartUnits for
+// starting it.  A worker that finishes one sequence and starts the next pays for a second
+// prologue (queries, first tiles with nothing in flight) and epilogue (row merge, partial
+// write): with equal tile counts such workers ended 3 us after the others and set the
+// duration of the launch.  With that cost in the stream they get fewer tiles (a tile takes
+// about 2.3 us); 3 to 5 units measured alike, 0 and 1 worse.
+constexpr int kSeqStartUnits = 4;
 __device__ __forceinline__ int decode_tiles(const AttnParams& p, int s) {
     const int n_new = p.cu_seqlens_q[s + 1] - p.cu_seqlens_q[s];
     const int ctx = p.context_lens[s];
-    return (n_new == 1 && ctx > 0) ? (ctx + kTileKeys - 1) / kTileKeys : 0;
+    return (n_new == 1 && ctx > 0) ? (ctx + kTileKeys - 1) / kTileKeys + kSeqStartUnits : 0;
 }
 
 constexpr int kMaxBalancedSeqs = 2048;  // prefix table held in LDS
@@ -617,14 +623,14 @@ __device__ __forceinline__ int worker_tiles(int total_tiles, int num_workers) {
 }
 
 // Decode rows, balanced: the key tiles of all decode sequences form one stream (sequence
-// after sequence); worker w (a workgroup, grid.x = num_workers, one per CU's worth of
-// waves) takes tiles [w*R, (w+1)*R) of it, R = ceil(total / num_workers), whichever
-// sequences they belong to.  Every worker therefore reads the same number of bytes,
-// whatever the context lengths are: with static partitions 288 equal workgroups on 256
-// CUs take two rounds, and the measured rate drops from 5.6 to 4.3 TB/s.  A worker's
-// piece of sequence s is written to workspace slot w + s (the pieces of one sequence get
-// consecutive slots since both w and s only grow along the stream); a sequence that lies
-// inside one worker is finished there.
+// after sequence, each preceded by kSeqStartUnits units of start-up cost); worker w (a
+// workgroup, grid.x = num_workers, one per CU's worth of waves) takes units [w*R, (w+1)*R) of
+// it, R = ceil(total / num_workers), whichever sequences they belong to.  Every worker
+// therefore does the same amount of work, whatever the context lengths are: with static
+// partitions 288 equal workgroups on 256 CUs take two rounds, and the measured rate drops
+// from 5.6 to 4.3 TB/s.  A worker's piece of sequence s is written to workspace slot w + s
+// (the pieces of one sequence get consecutive slots since both w and s only grow along the
+// stream); a sequence that lies inside one worker is finished there.
 template <int G, bool T3>
 __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_balanced_kernel(const AttnParams p) {
     __shared__ int pt[kMaxBalancedSeqs + 1];  // exclusive prefix of decode tiles
@@ -678,10 +684,15 @@ __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_balanced_kernel
         const int seq_end = __builtin_amdgcn_readfirstlane(pt[s + 1]);
         if (seq_end <= tcur) continue;  // a sequence without decode tiles
         const int seg_end = min(te, seq_end);
-        const int ctx = p.context_lens[s];
-        const bool single = tcur == seq_begin && seg_end == seq_end;
-        attn_partition<G, T3>(p, s, p.cu_seqlens_q[s], kvh, (tcur - seq_begin) * kTileKeys,
-                              min(ctx, (seg_end - seq_begin) * kTileKeys), single, (int64_t)w + s);
+        // units -> tiles of the sequence: the first kSeqStartUnits units are its start-up cost
+        const int tile_lo = max(tcur - seq_begin - kSeqStartUnits, 0);
+        const int tile_hi = seg_end - seq_begin - kSeqStartUnits;
+        if (tile_hi > tile_lo) {
+            const int ctx = p.context_lens[s];
+            const bool single = tile_lo == 0 && seg_end == seq_end;
+            attn_partition<G, T3>(p, s, p.cu_seqlens_q[s], kvh, tile_lo * kTileKeys,
+                                  min(ctx, tile_hi * kTileKeys), single, (int64_t)w + s);
+        }
         tcur = seg_end;
     }
 }
@@ -724,14 +735,16 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams 
         __syncthreads();
         total = red[0][0] + red[0][1] + red[0][2] + red[0][3];
         before = red[1][0] + red[1][1] + red[1][2] + red[1][3];
-        const int nt = ctx > 0 ? (ctx + kTileKeys - 1) / kTileKeys : 0;
+        // units of this row in the stream (as decode_tiles counts them)
+        const int nt = ctx > 0 ? (ctx + kTileKeys - 1) / kTileKeys + kSeqStartUnits : 0;
         if (nt == 0) {
             zero_row = true;  // the stream has no tile of this row: nobody wrote it
             np = 0;
             first_slot = 0;
         } else {
+            // its tiles are the units [before + kSeqStartUnits, before + nt)
             const int R = worker_tiles(total, p.num_workers);
-            const int w_first = before / R;
+            const int w_first = (before + kSeqStartUnits) / R;
             np = (before + nt - 1) / R - w_first + 1;
             first_slot = (int64_t)w_first + s;
             if (np <= 1) return;
