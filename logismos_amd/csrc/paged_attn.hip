@@ -506,10 +506,10 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
     Tile buf0, buf1;
     load_tile(0, buf0);
     for (int tile = 0; tile < ntiles; tile += 2) {
-        // the two waves of a SIMD (w and w + 4) take turns at the higher issue priority, 16
-        // tiles each: left alone the older wave wins every tie and the younger one finishes
-        // microseconds after it
-        if ((tile & 15) == 0) {
+        // balanced kernel (long partitions): the two waves of a SIMD (w and w + 4) take turns
+        // at the higher issue priority, 16 tiles each: left alone the older wave wins every
+        // tie and the younger one finishes microseconds after it
+        if (p.num_workers > 0 && (tile & 15) == 0) {
             if ((((tile >> 4) ^ (threadIdx.x >> 8)) & 1) != 0) __builtin_amdgcn_s_setprio(1);
             else __builtin_amdgcn_s_setprio(0);
         }
