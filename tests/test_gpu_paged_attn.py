@@ -201,6 +201,20 @@ def test_balanced_decode_kernel_many_short_sequences():
     _check(c, num_splits=2, what="300 short sequences, 2 splits")
 
 
+@pytest.mark.parametrize("seed", [70, 71, 72, 73, 74, 75])
+def test_balanced_decode_kernel_random_batches(seed):
+    # The balanced kernel splits a stream in which every sequence is preceded by a few units of
+    # start-up cost: random batches (2..40 sequences, 1..5000 visible keys) put worker edges on
+    # start-up units, on first and last tiles and inside sequences, and give sequences one, two
+    # or many pieces to merge
+    rng = np.random.default_rng(seed)
+    n = int(rng.integers(2, 41))
+    prior = np.where(rng.random(n) < 0.3, rng.integers(0, 48, size=n), rng.integers(0, 5000, size=n))
+    c = workloads.paged_case(rng, np.ones(n, np.int32), prior, hq=8, hkv=2, min_max_blocks=2048)
+    _check(c, what=f"random batch, seed {seed}")
+    _check(c, num_splits=3, what=f"random batch, seed {seed}, 3 splits")
+
+
 def test_zero_context_and_empty_sequences():
     rng = np.random.default_rng(5)
     c = workloads.paged_case(rng, [1, 0, 1, 3], [0, 5, 40, 0], hq=4, hkv=2)
