@@ -409,6 +409,17 @@ def bench_q4(args):
     out["q4g32_b1"] = {"us": round(ms * 1e3, 2), "GBps": round(algo32 / ms / 1e6, 1),
                        "GBps_warm_cache": round(algo32 / ms_warm / 1e6, 1),
                        "kernel": "qgemv_q4g32 (ggml Q4_0/Q4_1 arithmetic, x fp32)"}
+    # ... and as a batch of 16 bf16 rows through the matrix-core kernel
+    for b in (4, 16):
+        xb = hip.DeviceBuffer.from_numpy(O.f32_to_bf16_bits(rng.standard_normal((b, k), np.float32)))
+        yb = hip.DeviceBuffer(b * n * 2)
+        algo = n * k // 2 + n * (k // 32) * 4 + 2 * b * k + 2 * b * n
+        ms, _, _ = time_launches(
+            stream, [(lambda q=q: kernels.launch_qgemm_q4g32_bf16(xb, q, sc32, mn32, yb, b, n, k,
+                                                                  stream)) for q in qws],
+            args.steps, args.warmup)
+        out[f"q4g32_b{b}"] = {"us": round(ms * 1e3, 2), "GBps": round(algo / ms / 1e6, 1),
+                              "kernel": "qgemm_q4g32 (mfma, one group per 16x16x32 product)"}
     return {"workload": "config 3: Q4G128 GEMV/GEMM 12288x4096, x bf16, cold weights", **out}
 
 

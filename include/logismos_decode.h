@@ -203,6 +203,16 @@ logismos_status_t logismos_launch_qgemv_q4g32_f32(const void* x_f32, const void*
                                                   void* y_f32, int n, int k,
                                                   logismos_stream_t stream);
 
+/* y[b][n] = bf16(sum_k x[b][k] * (q[n][k] * scale[n][k/32] + min[n][k/32])): `linear_t` at
+ * m = batch (crates/kernels/src/cpu_f32/mod.rs:271-345) over the same Q4G32 weights, x and y
+ * bf16 like those of the Q4G128 GEMM, fp32 accumulation on the matrix cores.  batch 1..32,
+ * K % 128 == 0, N*K <= i32::MAX; qw and x 16-byte aligned, scale and min 8-byte aligned. */
+logismos_status_t logismos_check_qgemm_q4g32_shape(int b, int n, int k, char* msg, size_t msg_cap);
+logismos_status_t logismos_launch_qgemm_q4g32_bf16(const void* x_bf16, const void* qw_u8,
+                                                   const void* scale_f16, const void* min_f16,
+                                                   void* y_bf16, int b, int n, int k,
+                                                   logismos_stream_t stream);
+
 /* ggml Q4_0 / Q4_1 block streams `[N][K/32]` (the tensors the loader rejects today,
  * crates/loader/src/gguf.rs:127-145,397-406) -> planar Q4G32.  blocks 2-byte aligned. */
 logismos_status_t logismos_launch_repack_q4_0(const void* blocks_q4_0, void* qw_u8,

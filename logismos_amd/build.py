@@ -42,6 +42,7 @@ EXTRA_FLAGS = {
     "qgemm_q4_splitk.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "qgemm_q4_stream.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "qgemm_q4_greedy.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "qgemm_q4g32.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
 }
 
 

@@ -53,6 +53,8 @@ _SIGNATURES = {
     "logismos_launch_repack_q8_0": (C.c_uint32, [_vp, _vp, _vp, _i, _i, _vp]),
     "logismos_check_qgemv_q4g32_shape": (C.c_uint32, [_i, _i, C.c_char_p, _sz]),
     "logismos_launch_qgemv_q4g32_f32": (C.c_uint32, [_vp] * 5 + [_i, _i, _vp]),
+    "logismos_check_qgemm_q4g32_shape": (C.c_uint32, [_i, _i, _i, C.c_char_p, _sz]),
+    "logismos_launch_qgemm_q4g32_bf16": (C.c_uint32, [_vp] * 5 + [_i, _i, _i, _vp]),
     "logismos_launch_repack_q4_0": (C.c_uint32, [_vp] * 4 + [_i, _i, _vp]),
     "logismos_launch_repack_q4_1": (C.c_uint32, [_vp] * 4 + [_i, _i, _vp]),
     "logismos_paged_attn_num_splits": (C.c_int, [_i, _i, _i, _i]),
@@ -202,6 +204,17 @@ def launch_qgemv_q4g32_f32(x, qw, scale, minv, y, n: int, k: int, stream=None) -
     check_qgemv_q4g32_shape(n, k)
     _status("qgemv_q4g32_f32", library().logismos_launch_qgemv_q4g32_f32(
         _ptr(x), _ptr(qw), _ptr(scale), _ptr(minv), _ptr(y), n, k, _raw(stream)))
+
+
+def check_qgemm_q4g32_shape(b: int, n: int, k: int) -> None:
+    _guard("qgemm_q4g32_bf16", library().logismos_check_qgemm_q4g32_shape, b, n, k)
+
+
+def launch_qgemm_q4g32_bf16(x, qw, scale, minv, y, b: int, n: int, k: int, stream=None) -> None:
+    """Batched (1..32 rows) product over planar Q4G32 weights; x and y bf16."""
+    check_qgemm_q4g32_shape(b, n, k)
+    _status("qgemm_q4g32_bf16", library().logismos_launch_qgemm_q4g32_bf16(
+        _ptr(x), _ptr(qw), _ptr(scale), _ptr(minv), _ptr(y), b, n, k, _raw(stream)))
 
 
 def launch_repack_q4_blocks(blocks, qw, scale, minv, n: int, k: int, has_min: bool,

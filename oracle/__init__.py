@@ -372,6 +372,18 @@ def qgemv_q4g32_f32(x, qw, scale, minv, n, k):
     return y
 
 
+def qgemm_q4g32_f32(x_bf16_bits, qw, scale, minv, b, n, k):
+    """`linear_t` (crates/kernels/src/cpu_f32/mod.rs:271-345) at m = b over the dequantised Q4G32
+    matrix: the GEMV above once per batch row, x given as bf16 bits; fp32 result."""
+    x = bf16_bits_to_f32(np.asarray(x_bf16_bits).reshape(b, k))
+    return np.stack([qgemv_q4g32_f32(x[i], qw, scale, minv, n, k) for i in range(b)])
+
+
+def qgemm_q4g32_bf16(x_bf16_bits, qw, scale, minv, b, n, k):
+    """The same, rounded once to bf16 (round to nearest even) like the Q4G128 GEMM's output."""
+    return f32_to_bf16_bits(qgemm_q4g32_f32(x_bf16_bits, qw, scale, minv, b, n, k))
+
+
 def quantize_q8g32(w, n, k):
     w = _f32(w)
     assert w.size == n * k and k % 32 == 0

@@ -117,3 +117,99 @@ def test_shape_guards():
         kernels.check_qgemv_q4g32_shape(4, 48)
     with pytest.raises(kernels.UnsupportedShape):
         kernels.check_qgemv_q4g32_shape(0, 64)
+
+
+# ---------------------------------------------------------------- batched (matrix-core) product
+def _gemm(xbits, qw, sc, mn, b, n, k):
+    y = hip.DeviceBuffer(b * n * 2)
+    y.fill(0xFF)
+    kernels.launch_qgemm_q4g32_bf16(_dev(xbits), qw, sc, mn, y, b, n, k)
+    hip.synchronize()
+    return y.to_numpy(np.uint16, (b, n))
+
+
+def _batched_case(b, n, k, has_min, seed, wscale=0.02):
+    rng = np.random.default_rng(seed)
+    xbits = O.f32_to_bf16_bits(rng.standard_normal((b, k), np.float32))
+    w = rng.standard_normal((n, k), np.float32) * np.float32(wscale)
+    blocks = O.quantize_q4_blocks(w, n, k, has_min)
+    return xbits, blocks
+
+
+@pytest.mark.parametrize("has_min", [False, True])
+@pytest.mark.parametrize("b,n,k", [
+    (1, 1, 128), (2, 17, 256), (3, 16, 896),      # fewer 128-column chunks than waves
+    (5, 33, 1024), (16, 130, 2176),               # 17 chunks: an odd share per wave
+    (17, 47, 1152), (32, 257, 4096),              # two batch tiles
+    (9, 4096 + 48, 1024),                         # two row tiles per workgroup + a ragged last
+    (32, 12288, 4096), (16, 12288 + 16, 2048),    # three row tiles per workgroup
+])
+def test_batched_product_matches_oracle(b, n, k, has_min):
+    xbits, blocks = _batched_case(b, n, k, has_min, b * 104729 + n * 31 + k + has_min)
+    qw, sc, mn = _repack_gpu(blocks, n, k, has_min)
+    got = _gemm(xbits, qw, sc, mn, b, n, k)
+    pq, ps, pm = O.q4_blocks_to_q4g32(blocks, n, k, has_min)
+    want32 = O.qgemm_q4g32_f32(xbits, pq, ps, pm, b, n, k)
+    # bf16 output of an fp32 accumulation: the tolerance of the decode path
+    assert_parity(O.bf16_bits_to_f32(got), want32, max_abs=2e-3, max_rel=1e-2,
+                  what=f"qgemm_q4g32 b={b} {n}x{k}")
+    # and nearly always the very same bf16 value as the oracle's rounding of its own sum
+    want = O.qgemm_q4g32_bf16(xbits, pq, ps, pm, b, n, k)
+    assert (got == want).mean() > 0.97
+
+
+def test_batched_rows_do_not_depend_on_the_batch():
+    # row i of a batch of 32 equals the same x sent alone, bit for bit: the matrix-core
+    # product never mixes batch rows and the summation order does not depend on b
+    b, n, k = 32, 1000, 2048
+    xbits, blocks = _batched_case(b, n, k, True, 77)
+    qw, sc, mn = _repack_gpu(blocks, n, k, True)
+    full = _gemm(xbits, qw, sc, mn, b, n, k)
+    for i in (0, 15, 16, 31):
+        one = _gemm(xbits[i:i + 1], qw, sc, mn, 1, n, k)
+        assert np.array_equal(one[0], full[i])
+    part = _gemm(xbits[:7], qw, sc, mn, 7, n, k)
+    assert np.array_equal(part, full[:7])
+
+
+def test_batched_product_agrees_with_the_gemv():
+    # the same weights through the fp32 GEMV: x is bf16-exact, so only the output rounding
+    # and the summation order differ
+    b, n, k = 4, 512, 1024
+    xbits, blocks = _batched_case(b, n, k, False, 78)
+    qw, sc, mn = _repack_gpu(blocks, n, k, False)
+    got = O.bf16_bits_to_f32(_gemm(xbits, qw, sc, mn, b, n, k))
+    x = O.bf16_bits_to_f32(xbits)
+    for i in range(b):
+        y = _gemv(x[i], qw, sc, mn, n, k)
+        assert_parity(got[i], y, max_abs=2e-3, max_rel=1e-2, what="gemm row vs gemv")
+
+
+def test_batched_one_hot_reads_back_columns_of_every_group_position():
+    # one-hot x in batch row r selects column c_r: pins the lane / dword transpose of the
+    # weight tile (a wrong dword would return another column's value)
+    n, k = 48, 512
+    rng = np.random.default_rng(79)
+    w = rng.standard_normal((n, k), np.float32)
+    blocks = O.quantize_q4_blocks(w, n, k, True)
+    qw, sc, mn = _repack_gpu(blocks, n, k, True)
+    pq, ps, pm = O.q4_blocks_to_q4g32(blocks, n, k, True)
+    deq = O.dequantize_q4g32(pq, ps, pm, n, k)
+    cols = np.array([(37 * r + 5) % k for r in range(32)])
+    assert len(set(cols % 32)) == 32                       # every position inside a group
+    x = np.zeros((32, k), np.float32)
+    x[np.arange(32), cols] = 1.0
+    got = O.bf16_bits_to_f32(_gemm(O.f32_to_bf16_bits(x), qw, sc, mn, 32, n, k))
+    want = O.bf16_bits_to_f32(O.f32_to_bf16_bits(deq[:, cols].T.copy()))
+    assert np.array_equal(got, want)
+
+
+def test_batched_shape_guards():
+    with pytest.raises(kernels.UnsupportedShape):
+        kernels.check_qgemm_q4g32_shape(4, 64, 96)          # K not a multiple of 128
+    with pytest.raises(kernels.UnsupportedShape):
+        kernels.check_qgemm_q4g32_shape(33, 64, 128)
+    with pytest.raises(kernels.UnsupportedShape):
+        kernels.check_qgemm_q4g32_shape(0, 64, 128)
+    with pytest.raises(kernels.UnsupportedShape):
+        kernels.check_qgemm_q4g32_shape(2, 65536, 65536)

@@ -146,3 +146,24 @@ def test_qgemv_q4g32_matches_float64_bruteforce_and_orientation(has_min):
     e = np.zeros(k, np.float32)
     e[45] = 1.0
     assert np.array_equal(O.qgemv_q4g32_f32(e, qw, scale, minv, n, k), deq[:, 45].astype(np.float32))
+
+
+@pytest.mark.parametrize("has_min", [False, True])
+def test_qgemm_q4g32_is_the_float64_product_row_by_row(has_min):
+    rng = np.random.default_rng(12)
+    b, n, k = 5, 19, 256
+    w = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+    xbits = O.f32_to_bf16_bits(rng.standard_normal((b, k)).astype(np.float32))
+    x = O.bf16_bits_to_f32(xbits).astype(np.float64)
+    blocks = O.quantize_q4_blocks(w, n, k, has_min)
+    qw, scale, minv = O.q4_blocks_to_q4g32(blocks, n, k, has_min)
+    deq = O.dequantize_q4_blocks(blocks, n, k, has_min).astype(np.float64)
+    want = x @ deq.T                                            # [b, n]: weight is [out, in]
+    got = O.qgemm_q4g32_f32(xbits, qw, scale, minv, b, n, k)
+    assert got.shape == (b, n)
+    assert np.abs(got - want).max() <= 1e-5 * np.abs(deq).sum(axis=1).max() * np.abs(x).max()
+    # the bf16 form is that sum rounded once, to nearest even
+    bits = O.qgemm_q4g32_bf16(xbits, qw, scale, minv, b, n, k)
+    back = O.bf16_bits_to_f32(bits)
+    assert np.abs(back - got).max() <= np.abs(got).max() * 2.0 ** -8
+    assert np.array_equal(bits, O.f32_to_bf16_bits(got))
