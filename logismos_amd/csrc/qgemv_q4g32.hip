@@ -12,6 +12,7 @@
 // Algorithmic bytes per call: n*k/2 (nibbles) + n*(k/32)*4 (scale, min) + 4k + 4n.
 #include "device_utils.hpp"
 #include "launch_common.hpp"
+#include "q4_common.hpp"
 
 #include <hip/hip_fp16.h>
 
@@ -87,6 +88,126 @@ __global__ __launch_bounds__(256) void qgemv_q4g32_kernel(const float* __restric
     }
 }
 
+// The same product for rows of 32 .. 512 groups (K = 1024 .. 16384), with every load of a
+// wave issued at once.  A wave's R consecutive rows are one contiguous run of R*K/2 bytes (and
+// of R*K/32 scales / mins): lane l takes the groups l, l + 64, ... of that run, NP of them,
+// whichever row they fall into, so that the wave pays the memory latency once.  x is staged
+// in LDS in eight planes (quarter j of group c at xl[j * K/32 + c]) with the group sums of x
+// beside them; a group's result goes to the accumulator of its row by comparison.
+template <int R, int NP>
+__global__ __launch_bounds__(256) void qgemv_q4g32_flat_kernel(const float* __restrict__ x,
+                                                               const uint8_t* __restrict__ qw,
+                                                               const __half* __restrict__ scale,
+                                                               const __half* __restrict__ minv,
+                                                               float* __restrict__ y, int n, int k) {
+    extern __shared__ float4_t xl[];
+    const int groups = k >> 5;
+    float* xs = reinterpret_cast<float*>(xl + (size_t)8 * groups);
+    const int lane = threadIdx.x & 63;
+    const int64_t row0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * R;
+    const int rows = row0 < n ? (int)min((int64_t)R, (int64_t)n - row0) : 0;
+    const int valid = rows * groups;
+    // a wave past the end, and groups past a wave's rows, re-read a group that exists
+    const uint8_t* wbase = rows > 0 ? qw + row0 * (int64_t)(k >> 1) : qw;
+    const int64_t g0 = rows > 0 ? row0 * groups : 0;
+
+    uint4_t w[NP];
+    __half sc[NP], mn[NP];
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+        const int p = lane + 64 * i;
+        const int pc = p < valid ? p : 0;
+        w[i] = *reinterpret_cast<const uint4_t*>(wbase + (int64_t)pc * 16);
+        sc[i] = scale[g0 + pc];
+        mn[i] = minv[g0 + pc];
+    }
+    for (int c = threadIdx.x; c < groups; c += 256) {
+        float s = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float4_t v = reinterpret_cast<const float4_t*>(x)[c * 8 + j];
+            xl[j * groups + c] = v;
+            s += (v[0] + v[1]) + (v[2] + v[3]);
+        }
+        xs[c] = s;
+    }
+    __syncthreads();
+
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+        const int p = lane + 64 * i;
+        int r = 0;
+#pragma unroll
+        for (int j = 1; j < R; ++j) r += (p >= j * groups) ? 1 : 0;
+        const bool live = p < valid;
+        const int c = live ? p - r * groups : 0;
+        float s = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            // word j: nibbles of elements 8j .. 8j+7; even elements in the low nibbles
+            const unsigned v = w[i][j];
+            const unsigned ev = v & 0x0F0F0F0Fu;
+            const unsigned od = (v >> 4) & 0x0F0F0F0Fu;
+            const float4_t xa = xl[(2 * j) * groups + c];
+            const float4_t xb = xl[(2 * j + 1) * groups + c];
+            s = fmaf(xa[0], (float)(ev & 0xffu), s);
+            s = fmaf(xa[1], (float)(od & 0xffu), s);
+            s = fmaf(xa[2], (float)((ev >> 8) & 0xffu), s);
+            s = fmaf(xa[3], (float)((od >> 8) & 0xffu), s);
+            s = fmaf(xb[0], (float)((ev >> 16) & 0xffu), s);
+            s = fmaf(xb[1], (float)((od >> 16) & 0xffu), s);
+            s = fmaf(xb[2], (float)(ev >> 24), s);
+            s = fmaf(xb[3], (float)(od >> 24), s);
+        }
+        float v = fmaf(s, __half2float(sc[i]), xs[c] * __half2float(mn[i]));
+        v = live ? v : 0.0f;
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) acc[rr] += (r == rr) ? v : 0.0f;
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const float total = wave_sum(acc[r]);
+        if (lane == 0 && r < rows) y[row0 + r] = total;
+    }
+}
+
+template <int R, int NP = 1>
+static hipError_t launch_q4g32_flat(int np, const float* x, const uint8_t* qw, const __half* scale,
+                                    const __half* minv, float* y, int n, int k,
+                                    hipStream_t stream) {
+    if constexpr (NP > (R == 1 ? 8 : 4)) {
+        return hipErrorInvalidValue;
+    } else {
+        if (np != NP) return launch_q4g32_flat<R, NP + 1>(np, x, qw, scale, minv, y, n, k, stream);
+        const size_t lds = (size_t)(k / 32) * (8 * 16 + 4);  // at most 66 KiB (K = 16384)
+        auto kern = qgemv_q4g32_flat_kernel<R, NP>;
+        if (lds > 64 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return e;
+        }
+        const int64_t waves = ((int64_t)n + R - 1) / R;
+        kern<<<dim3((unsigned)((waves + 3) / 4)), dim3(256), lds, stream>>>(x, qw, scale, minv, y, n,
+                                                                          k);
+        return hipGetLastError();
+    }
+}
+
+// Rows per wave of the flat kernel, 0 when it does not apply.  At most 256 groups (four per
+// lane) per wave unless a single row is longer; fewer rows per wave while that leaves fewer
+// than four waves per CU.
+static int q4g32_flat_rows(int n, int k, int cus) {
+    const int groups = k / 32;
+    if (groups < 32 || groups > 512) return 0;
+    int r = 8;
+    while (r > 1 && r * groups > 256) r >>= 1;
+    while (r > 1 && (n + r - 1) / r < 4 * cus) r >>= 1;
+    return r;
+}
+
 // ggml Q4_0 (18-byte blocks: f16 d, 16 bytes) or Q4_1 (20-byte blocks: f16 d, f16 m, 16
 // bytes) stream -> planar Q4G32.  ggml keeps value j in the low and value j + 16 in the
 // high nibble of byte j; the planar form is in k order.  One thread per block.
@@ -151,14 +272,26 @@ extern "C" logismos_status_t logismos_launch_qgemv_q4g32_f32(const void* x_f32, 
     if (!x_f32 || !qw_u8 || !scale_f16 || !min_f16 || !y_f32) return hipErrorInvalidValue;
     if ((reinterpret_cast<uintptr_t>(qw_u8) & 15u) || (reinterpret_cast<uintptr_t>(x_f32) & 15u))
         return hipErrorInvalidValue;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    auto* xp = static_cast<const float*>(x_f32);
+    auto* qp = static_cast<const uint8_t*>(qw_u8);
+    auto* sp = static_cast<const __half*>(scale_f16);
+    auto* mp = static_cast<const __half*>(min_f16);
+    auto* yp = static_cast<float*>(y_f32);
+    if (const int fr = lg::q4g32_flat_rows(n, k, lg::device_cu_count()); fr > 0) {
+        const int np = (fr * (k / 32) + 63) / 64;
+        switch (fr) {
+            case 8: return lg::launch_q4g32_flat<8>(np, xp, qp, sp, mp, yp, n, k, st);
+            case 4: return lg::launch_q4g32_flat<4>(np, xp, qp, sp, mp, yp, n, k, st);
+            case 2: return lg::launch_q4g32_flat<2>(np, xp, qp, sp, mp, yp, n, k, st);
+            default: return lg::launch_q4g32_flat<1>(np, xp, qp, sp, mp, yp, n, k, st);
+        }
+    }
     constexpr int R = 4;
     const int waves = (n + R - 1) / R;
     const int wpb = 4;
     dim3 grid((waves + wpb - 1) / wpb), block(wpb * 64);
-    lg::qgemv_q4g32_kernel<R><<<grid, block, 0, static_cast<hipStream_t>(stream)>>>(
-        static_cast<const float*>(x_f32), static_cast<const uint8_t*>(qw_u8),
-        static_cast<const __half*>(scale_f16), static_cast<const __half*>(min_f16),
-        static_cast<float*>(y_f32), n, k);
+    lg::qgemv_q4g32_kernel<R><<<grid, block, 0, st>>>(xp, qp, sp, mp, yp, n, k);
     return hipGetLastError();
 }
 

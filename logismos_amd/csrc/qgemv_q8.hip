@@ -12,6 +12,7 @@
 // Algorithmic bytes per call: n*k (int8) + n*(k/32)*2 (scales) + 4k + 4n.
 #include "device_utils.hpp"
 #include "launch_common.hpp"
+#include "q4_common.hpp"
 
 #include <hip/hip_fp16.h>
 
@@ -73,6 +74,102 @@ __global__ __launch_bounds__(256) void qgemv_q8g32_kernel(const float* __restric
     }
 }
 
+// The same product for rows of 512 .. 8192 bytes, with every load of a wave issued at once.
+// A wave's R consecutive rows are one contiguous run of R*K bytes (and of R*K/32 scales):
+// lane l takes the 16-byte pieces l, l + 64, ... of that run, NP of them, whatever row they
+// fall into, so that no lane idles when K is not a multiple of 1024 and the wave pays the
+// memory latency once instead of once per 1024 columns.  x is staged in LDS in four planes
+// (quarter j of piece c at xl[j * K/16 + c]) so that neighbouring lanes read neighbouring
+// 16-byte words.  A piece's partial sum goes to the accumulator of its row by comparison.
+template <int R, int NP>
+__global__ __launch_bounds__(256) void qgemv_q8g32_flat_kernel(const float* __restrict__ x,
+                                                               const int8_t* __restrict__ qs,
+                                                               const __half* __restrict__ d,
+                                                               float* __restrict__ y, int n, int k) {
+    extern __shared__ float4_t xl[];
+    const int lane = threadIdx.x & 63;
+    const int ppr = k >> 4;  // pieces per row
+    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t row0 = wave * R;
+    const int rows = row0 < n ? (int)min((int64_t)R, (int64_t)n - row0) : 0;
+    const int valid = rows * ppr;
+    // a wave past the end, and pieces past a wave's rows, re-read a piece that exists
+    const int8_t* wbase = rows > 0 ? qs + row0 * k : qs;
+    const __half* dbase = rows > 0 ? d + row0 * (k >> 5) : d;
+
+    int4_t w[NP];
+    __half sc[NP];
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+        const int p = lane + 64 * i;
+        const int pc = p < valid ? p : 0;
+        w[i] = *reinterpret_cast<const int4_t*>(wbase + (int64_t)pc * 16);
+        sc[i] = dbase[pc >> 1];
+    }
+    for (int f = threadIdx.x; f < (k >> 2); f += 256)
+        xl[(f & 3) * ppr + (f >> 2)] = reinterpret_cast<const float4_t*>(x)[f];
+    __syncthreads();
+
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+        const int p = lane + 64 * i;
+        int r = 0;
+#pragma unroll
+        for (int j = 1; j < R; ++j) r += (p >= j * ppr) ? 1 : 0;
+        const bool live = p < valid;
+        const int c = live ? p - r * ppr : 0;
+        float s = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float4_t xv = xl[j * ppr + c];
+            const int v = w[i][j];
+            s = fmaf(xv[0], (float)(int8_t)(v), s);
+            s = fmaf(xv[1], (float)(int8_t)(v >> 8), s);
+            s = fmaf(xv[2], (float)(int8_t)(v >> 16), s);
+            s = fmaf(xv[3], (float)(int8_t)(v >> 24), s);
+        }
+        const float v = live ? s * __half2float(sc[i]) : 0.0f;
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) acc[rr] += (r == rr) ? v : 0.0f;
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const float total = wave_sum(acc[r]);
+        if (lane == 0 && r < rows) y[row0 + r] = total;
+    }
+}
+
+template <int R, int NP = 1>
+static hipError_t launch_flat(int np, const float* x, const int8_t* qs, const __half* d, float* y,
+                              int n, int k, hipStream_t stream) {
+    if constexpr (NP > 8) {
+        return hipErrorInvalidValue;
+    } else {
+        if (np != NP) return launch_flat<R, NP + 1>(np, x, qs, d, y, n, k, stream);
+        const int64_t waves = ((int64_t)n + R - 1) / R;
+        qgemv_q8g32_flat_kernel<R, NP><<<dim3((unsigned)((waves + 3) / 4)), dim3(256),
+                                         (size_t)k * 4, stream>>>(x, qs, d, y, n, k);
+        return hipGetLastError();
+    }
+}
+
+// Rows per wave of the flat kernel for this shape, 0 when it does not apply (rows shorter than
+// 512 or longer than 8192 bytes).  At most 256 pieces (four per lane) per wave unless a
+// single row is longer: on config-1 and 4096 x 4096 matrices two to four pieces per lane
+// measured 8 % faster than six or eight; fewer rows per wave while that leaves fewer than
+// four waves per CU.
+static int flat_rows(int n, int k) {
+    const int ppr = k / 16;
+    if (k % 16 != 0 || ppr < 32 || ppr > 512) return 0;
+    int r = 8;
+    while (r > 1 && r * ppr > 256) r >>= 1;
+    while (r > 1 && (n + r - 1) / r < 4 * device_cu_count()) r >>= 1;
+    return r;
+}
+
 // ggml Q8_0 block stream -> planar.  One thread per 34-byte block.
 __global__ __launch_bounds__(256) void repack_q8_0_kernel(const uint8_t* __restrict__ blocks,
                                                           int8_t* __restrict__ qs,
@@ -108,13 +205,25 @@ extern "C" logismos_status_t logismos_launch_qgemv_q8g32_f32(const void* x_f32, 
     if (!x_f32 || !qs_i8 || !d_f16 || !y_f32) return hipErrorInvalidValue;
     if ((reinterpret_cast<uintptr_t>(qs_i8) & 15u) || (reinterpret_cast<uintptr_t>(x_f32) & 15u))
         return hipErrorInvalidValue;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    auto* xp = static_cast<const float*>(x_f32);
+    auto* qp = static_cast<const int8_t*>(qs_i8);
+    auto* dp = static_cast<const __half*>(d_f16);
+    auto* yp = static_cast<float*>(y_f32);
+    if (const int fr = lg::flat_rows(n, k); fr > 0) {
+        const int np = (fr * (k / 16) + 63) / 64;
+        switch (fr) {
+            case 8: return lg::launch_flat<8>(np, xp, qp, dp, yp, n, k, st);
+            case 4: return lg::launch_flat<4>(np, xp, qp, dp, yp, n, k, st);
+            case 2: return lg::launch_flat<2>(np, xp, qp, dp, yp, n, k, st);
+            default: return lg::launch_flat<1>(np, xp, qp, dp, yp, n, k, st);
+        }
+    }
     constexpr int R = 4;
     const int waves = (n + R - 1) / R;
     const int wpb = 4;
     dim3 grid((waves + wpb - 1) / wpb), block(wpb * 64);
-    lg::qgemv_q8g32_kernel<R><<<grid, block, 0, static_cast<hipStream_t>(stream)>>>(
-        static_cast<const float*>(x_f32), static_cast<const int8_t*>(qs_i8),
-        static_cast<const __half*>(d_f16), static_cast<float*>(y_f32), n, k);
+    lg::qgemv_q8g32_kernel<R><<<grid, block, 0, st>>>(xp, qp, dp, yp, n, k);
     return hipGetLastError();
 }
 

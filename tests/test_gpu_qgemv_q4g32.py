@@ -63,7 +63,9 @@ def _gemv(x, qw, sc, mn, n, k):
 
 @pytest.mark.parametrize("has_min", [False, True])
 @pytest.mark.parametrize("n,k", [(1, 32), (3, 64), (5, 1024), (7, 1056), (257, 8960),
-                                 (12288, 4096)])
+                                 (12288, 4096),
+                                 # several rows per wave with a ragged last wave: 8, 4 and 2 rows
+                                 (8203, 1024), (4099, 1024), (2051, 2048), (700, 16384)])
 def test_block_stream_to_gemv_matches_oracle(n, k, has_min):
     # the whole row f3 describes: ggml blocks -> device repack -> dequant-fused GEMV
     rng = np.random.default_rng(n * 7919 + k + has_min)

@@ -25,7 +25,9 @@ def test_config1_up_proj_matches_oracle():
 
 
 @pytest.mark.parametrize("n,k", [(1, 32), (3, 64), (5, 1024), (7, 1056), (130, 2048), (257, 8960),
-                                 (4096, 4096)])
+                                 (4096, 4096),
+                                 # several rows per wave with a ragged last wave: 8, 4 and 2 rows
+                                 (8195, 512), (4099, 1024), (2051, 1536), (1500, 8192)])
 def test_ragged_shapes(n, k):
     rng = np.random.default_rng(n * 7919 + k)
     x = rng.standard_normal(k, np.float32)
