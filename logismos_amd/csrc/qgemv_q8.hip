@@ -158,7 +158,7 @@ static hipError_t launch_flat(int np, const float* x, const int8_t* qs, const __
 
 // Rows per wave of the flat kernel for this shape, 0 when it does not apply (rows shorter than
 // 512 or longer than 8192 bytes).  At most 256 pieces (four per lane) per wave unless a
-// single row is longer: on config-1 and 4096 x 4096 matrices two to four pieces per lane
+// single row is longer: on 8960 x 1536 and 4096 x 4096 matrices two to four pieces per lane
 // measured 8 % faster than six or eight; fewer rows per wave while that leaves fewer than
 // four waves per CU.
 static int flat_rows(int n, int k) {
