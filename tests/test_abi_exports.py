@@ -109,3 +109,23 @@ def test_qgemm_q4_shape_guard(b, n, k, frag):
         kernels.check_qgemm_q4g128_shape(b, n, k)
     assert frag in str(e.value)
     kernels.check_qgemm_q4g128_shape(1, 12288, 4096)
+
+
+@pytest.mark.parametrize("b,n,k,frag", [
+    (0, 8, 128, "batch must be positive"), (33, 8, 128, "exceeds the supported maximum of 32"),
+    (1, 0, 128, "N must be positive"), (1, 8, 96, "multiple of 128"),
+    (1, 1 << 20, 1 << 12, "exceeds i32::MAX"),
+])
+def test_qgemm_q4g32_shape_guard(b, n, k, frag):
+    with pytest.raises(kernels.UnsupportedShape) as e:
+        kernels.check_qgemm_q4g32_shape(b, n, k)
+    assert frag in str(e.value)
+    kernels.check_qgemm_q4g32_shape(16, 12288, 4096)
+
+
+def test_q4g32_launchers_reject_bad_arguments_without_touching_the_device():
+    lib = kernels.library()
+    # null pointers, then a K that is not a multiple of the group size
+    assert lib.logismos_launch_qgemm_q4g32_bf16(None, None, None, None, None, 4, 64, 128, None) == 1
+    assert lib.logismos_launch_qgemm_q4g32_bf16(None, None, None, None, None, 4, 64, 96, None) == 1
+    assert lib.logismos_launch_qgemv_q4g32_f32(None, None, None, None, None, 64, 48, None) == 1
