@@ -387,7 +387,7 @@ def bench_q4(args):
         ms_warm, _, _ = time_launches(stream, [lambda: r.launch()], args.steps, args.warmup)
         out[f"b{b}"] = {"us": round(ms * 1e3, 2), "GBps": round(algo / ms / 1e6, 1),
                         "GBps_warm_cache": round(algo / ms_warm / 1e6, 1),
-                        "kernel": ("gemv (VALU dot2)" if b <= 2
+                        "kernel": ("gemv (VALU dot2)" if b <= 1
                                    else "mfma, x in registers, weights through an LDS ring")}
         del r, qws
     # the same matrix size as ggml Q4_0 weights through the Q4G32 GEMV (x fp32, batch 1)

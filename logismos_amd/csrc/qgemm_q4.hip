@@ -10,11 +10,12 @@
 // x is staged once per workgroup in LDS, already permuted to the (s, s+4)
 // pair order, next to the per-chunk / per-group sums of x.
 //
-// Batch <= 4 (bandwidth-bound GEMV): VALU path.  One wave owns R rows; a lane
+// Batch 1 and 2 (bandwidth-bound GEMV): VALU path.  One wave owns R rows; a lane
 // reads 16 bytes (32 nibbles) of each row per step, unpacks them once and
 // feeds v_dot2_f32_bf16 for every batch row.
 //
-// Batch >= 5: MFMA path (see qgemm_q4g128_mfma_kernel below).
+// Batch >= 3, and batch 2 on large matrices: MFMA paths (the register-x kernel of
+// qgemm_q4_regx.hip for K = 2048 / 4096, else qgemm_q4g128_mfma_kernel below).
 //
 // Algorithmic bytes per call: n*k/2 (nibbles) + n*(k/128)*4 (scale, zero)
 // + b*k*2 (x) + b*n*2 (y).
@@ -437,7 +438,9 @@ static logismos_status_t qgemm_q4_dispatch(const void* x_bf16, const void* qw_u8
     if (!force_mfma) {
         switch (b) {
             case 1: return lg::launch_gemv_b<1>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, n, k, st);
-            case 2: return lg::launch_gemv_b<2>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, n, k, st);
+            case 2:
+                if (lg::regx_plain_plan(b, n, k).parts == 1) break;  // large matrices, see there
+                return lg::launch_gemv_b<2>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, n, k, st);
             default: break;  // batch 3 and 4: the MFMA kernels are faster (measured crossover)
         }
         // K = 2048 / 4096: x in registers, weights through the LDS ring, one workgroup per K

@@ -788,7 +788,10 @@ RegxPlan regx_plan(int b, int n, int k) {
 RegxPlan regx_plain_plan(int b, int n, int k) {
     RegxPlan p{0, 0, 0, 0, 0};
     if (k != 2048 && k != 4096) return p;
-    if (b < 3 || b > 32 || n < 1024) return p;
+    if (b < 2 || b > 32 || n < 1024) return p;
+    // batch 2: the VALU GEMV stays ahead on small matrices (4096 x 4096: 5.5 vs 6.2 us), this
+    // kernel on large ones (12288 x 4096: 8.6 vs 9.6 us, 24576 x 4096: 13.0 vs 16.3 us)
+    if (b == 2 && (int64_t)n * k < 40000000) return p;
     p.gs = k / 1024;
     p.parts = 1;
     p.rows = b <= 16 ? 16 : 32;

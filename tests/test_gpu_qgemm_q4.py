@@ -90,11 +90,18 @@ def test_batch_rows_are_independent():
     got4, _ = _run(c["x"], qw, s, z, 4, n, k)                 # MFMA kernel
     got3, _ = _run(c["x"][[2, 0, 1]], qw, s, z, 3, n, k)      # MFMA kernel, row 2 first
     assert np.array_equal(got4[2], got3[0])
-    got2, _ = _run(c["x"], qw, s, z, 2, n, k)                 # VALU GEMV
+    # batch 2 of a matrix this large takes the same MFMA kernel: its rows are those of batch 4
+    got2, _ = _run(c["x"], qw, s, z, 2, n, k)
+    assert np.array_equal(got2, got4[:2])
+    # the VALU GEMV (batch 1, and batch 2 of smaller matrices): same property
     got1, _ = _run(c["x"][1:2], qw, s, z, 1, n, k)
-    assert np.array_equal(got2[1], got1[0])
+    ns = 2048                                                  # 2048 x 4096: batch 2 stays on the GEMV
+    small2, _ = _run(c["x"], qw[:ns], s[:ns], z[:ns], 2, ns, k)
+    small1, _ = _run(c["x"][1:2], qw[:ns], s[:ns], z[:ns], 1, ns, k)
+    assert np.array_equal(small2[1], small1[0])
+    assert np.array_equal(small1[0], got1[0][:ns])             # and of the matrix height
     # the two kernels agree to bf16 rounding
-    assert_parity(got4[1], got2[1], what="mfma vs gemv")
+    assert_parity(got4[1], got1[0], what="mfma vs gemv")
 
 
 # ------------------------------------------------------------------ split-K form (fp32 parts)
