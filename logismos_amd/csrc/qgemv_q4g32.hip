@@ -93,9 +93,11 @@ __global__ __launch_bounds__(256) void qgemv_q4g32_kernel(const float* __restric
 // of R*K/32 scales / mins): lane l takes the groups l, l + 64, ... of that run, NP of them,
 // whichever row they fall into, so that the wave pays the memory latency once.  x is staged
 // in LDS in eight planes (quarter j of group c at xl[j * K/32 + c]) with the group sums of x
-// beside them; a group's result goes to the accumulator of its row by comparison.
+// beside them; a group's result goes to the accumulator of its row by comparison.  Eight
+// waves per workgroup share one copy of x.
+constexpr int kFlatWaves = 8;
 template <int R, int NP>
-__global__ __launch_bounds__(256) void qgemv_q4g32_flat_kernel(const float* __restrict__ x,
+__global__ __launch_bounds__(64 * kFlatWaves) void qgemv_q4g32_flat_kernel(const float* __restrict__ x,
                                                                const uint8_t* __restrict__ qw,
                                                                const __half* __restrict__ scale,
                                                                const __half* __restrict__ minv,
@@ -104,7 +106,7 @@ __global__ __launch_bounds__(256) void qgemv_q4g32_flat_kernel(const float* __re
     const int groups = k >> 5;
     float* xs = reinterpret_cast<float*>(xl + (size_t)8 * groups);
     const int lane = threadIdx.x & 63;
-    const int64_t row0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * R;
+    const int64_t row0 = ((int64_t)blockIdx.x * kFlatWaves + (threadIdx.x >> 6)) * R;
     const int rows = row0 < n ? (int)min((int64_t)R, (int64_t)n - row0) : 0;
     const int valid = rows * groups;
     // a wave past the end, and groups past a wave's rows, re-read a group that exists
@@ -121,7 +123,7 @@ __global__ __launch_bounds__(256) void qgemv_q4g32_flat_kernel(const float* __re
         sc[i] = scale[g0 + pc];
         mn[i] = minv[g0 + pc];
     }
-    for (int c = threadIdx.x; c < groups; c += 256) {
+    for (int c = threadIdx.x; c < groups; c += 64 * kFlatWaves) {
         float s = 0.0f;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -190,8 +192,8 @@ static hipError_t launch_q4g32_flat(int np, const float* x, const uint8_t* qw, c
             if (e != hipSuccess) return e;
         }
         const int64_t waves = ((int64_t)n + R - 1) / R;
-        kern<<<dim3((unsigned)((waves + 3) / 4)), dim3(256), lds, stream>>>(x, qw, scale, minv, y, n,
-                                                                          k);
+        kern<<<dim3((unsigned)((waves + kFlatWaves - 1) / kFlatWaves)), dim3(64 * kFlatWaves), lds,
+               stream>>>(x, qw, scale, minv, y, n, k);
         return hipGetLastError();
     }
 }

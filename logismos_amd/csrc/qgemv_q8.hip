@@ -81,15 +81,17 @@ __global__ __launch_bounds__(256) void qgemv_q8g32_kernel(const float* __restric
 // memory latency once instead of once per 1024 columns.  x is staged in LDS in four planes
 // (quarter j of piece c at xl[j * K/16 + c]) so that neighbouring lanes read neighbouring
 // 16-byte words.  A piece's partial sum goes to the accumulator of its row by comparison.
+// Eight waves per workgroup share one copy of x (8960 x 1536: 5.5 us against 5.75 with four).
+constexpr int kFlatWaves = 8;
 template <int R, int NP>
-__global__ __launch_bounds__(256) void qgemv_q8g32_flat_kernel(const float* __restrict__ x,
+__global__ __launch_bounds__(64 * kFlatWaves) void qgemv_q8g32_flat_kernel(const float* __restrict__ x,
                                                                const int8_t* __restrict__ qs,
                                                                const __half* __restrict__ d,
                                                                float* __restrict__ y, int n, int k) {
     extern __shared__ float4_t xl[];
     const int lane = threadIdx.x & 63;
     const int ppr = k >> 4;  // pieces per row
-    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t wave = (int64_t)blockIdx.x * kFlatWaves + (threadIdx.x >> 6);
     const int64_t row0 = wave * R;
     const int rows = row0 < n ? (int)min((int64_t)R, (int64_t)n - row0) : 0;
     const int valid = rows * ppr;
@@ -106,7 +108,7 @@ __global__ __launch_bounds__(256) void qgemv_q8g32_flat_kernel(const float* __re
         w[i] = *reinterpret_cast<const int4_t*>(wbase + (int64_t)pc * 16);
         sc[i] = dbase[pc >> 1];
     }
-    for (int f = threadIdx.x; f < (k >> 2); f += 256)
+    for (int f = threadIdx.x; f < (k >> 2); f += 64 * kFlatWaves)
         xl[(f & 3) * ppr + (f >> 2)] = reinterpret_cast<const float4_t*>(x)[f];
     __syncthreads();
 
@@ -150,8 +152,9 @@ static hipError_t launch_flat(int np, const float* x, const int8_t* qs, const __
     } else {
         if (np != NP) return launch_flat<R, NP + 1>(np, x, qs, d, y, n, k, stream);
         const int64_t waves = ((int64_t)n + R - 1) / R;
-        qgemv_q8g32_flat_kernel<R, NP><<<dim3((unsigned)((waves + 3) / 4)), dim3(256),
-                                         (size_t)k * 4, stream>>>(x, qs, d, y, n, k);
+        qgemv_q8g32_flat_kernel<R, NP>
+            <<<dim3((unsigned)((waves + kFlatWaves - 1) / kFlatWaves)), dim3(64 * kFlatWaves),
+               (size_t)k * 4, stream>>>(x, qs, d, y, n, k);
         return hipGetLastError();
     }
 }
