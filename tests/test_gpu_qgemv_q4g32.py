@@ -145,6 +145,7 @@ def _batched_case(b, n, k, has_min, seed, wscale=0.02):
     (17, 47, 1152), (32, 257, 4096),              # two batch tiles
     (9, 4096 + 48, 1024),                         # two row tiles per workgroup + a ragged last
     (32, 12288, 4096), (16, 12288 + 16, 2048),    # three row tiles per workgroup
+    (8, 1040, 12288),                             # 96 chunks: twelve per wave
 ])
 def test_batched_product_matches_oracle(b, n, k, has_min):
     xbits, blocks = _batched_case(b, n, k, has_min, b * 104729 + n * 31 + k + has_min)
