@@ -37,6 +37,7 @@ from tests.gpu_harness import PagedAttnRunner, QgemvQ8Runner  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
 PMC_CAL_BYTES = 256 << 20  # bytes the calibration copy reads (and writes)
+PARITY_REL_L2_BOUND = 4e-3  # one layer of the step vs the oracle (bf16 intermediates)
 COLD_BYTES = 640 << 20  # replicas together exceed 2x the 256 MiB Infinity Cache
 
 
@@ -67,13 +68,13 @@ def physical_cores() -> int:
     return max(1, n)
 
 
-def measured_traffic(summary: str):
+def measured_traffic(summary: str, key: str = "traffic_bytes_per_launch:"):
     """HBM bytes per launch from a committed hardware-counter summary under profiles/ (the
     counters cannot be read from inside this process); None when there is none."""
     try:
         with open(os.path.join(ROOT, "profiles", summary)) as f:
             for ln in f:
-                if ln.strip().startswith("traffic_bytes_per_launch:"):
+                if ln.strip().startswith(key):
                     return int(ln.split(":")[1])
     except OSError:
         pass
@@ -464,6 +465,10 @@ def bench_decode_step(args):
     lay_cpu = copy.deepcopy(layers)
     want = O.bf16_bits_to_f32(OS.decode_step(cfg, lay_cpu, dict(b0, h=batch["h"].copy())))
     rel_l2 = float(np.linalg.norm(got - want) / np.linalg.norm(want))
+    if not (rel_l2 < PARITY_REL_L2_BOUND):
+        sys.exit(f"bench.py: the one-layer step differs from the CPU oracle by relative L2 "
+                 f"{rel_l2:.3e} (bound {PARITY_REL_L2_BOUND:.0e}); a throughput of wrong results "
+                 "is not reported")
     # the baseline: one whole step (36 layers) on the oracle; the 36 layers share one layer's
     # weights and pools (36 sets of pools would be 38 GB of host memory), which leaves the
     # arithmetic and the bytes touched per layer as they are
@@ -519,7 +524,14 @@ def bench_decode_step(args):
             d_q, kp, vp, r.idx["block_tables"], r.idx["cu_seqlens"], r.idx["context_lens"], d_o,
             d_ws, S, S, 1, hq, hkv, 128, bs, max_blocks, ns, c_attn["scale"], True, stream,
             kernels.ATTN_PHASE_DECODE)
+    # ... at the contexts of step 0, so that the bytes per launch do not depend on how many
+    # steps were timed before
+    d_cur_prior.copy_from_device_async(d_prior, 4 * S, stream)
+    kernels.launch_pack_ragged(d_ones, d_cur_prior, r.idx["block_tables"], r.idx["cu_seqlens"],
+                               r.slots, r.idx["context_lens"], S, bs, max_blocks, stream)
+    stream.synchronize()
     ctx_now = r.idx["context_lens"].to_numpy(np.int32, (S,)).astype(np.int64)
+    assert np.array_equal(ctx_now, ctx_steps[0])
     attn_bytes = int(ctx_now.sum()) * 2 * hkv * 128 * 2 + 2 * S * hq * 128 * 2 + \
         4 * int(((ctx_now + bs - 1) // bs).sum()) + 4 * (2 * S + 1)
     ms_attn, _, _ = time_launches(stream, [attn(l) for l in range(L)], 72, 8)
@@ -532,7 +544,7 @@ def bench_decode_step(args):
     del cal
 
     closed_loop = None
-    if not args.skip_closed_loop:
+    if args.extras:
         # ---- the same step as a closed loop over token ids: embedding lookup in front, the
         # vocabulary projection (151936 x 4096, Q4G128) with the greedy choice fused behind, the
         # chosen tokens being the next step's input.  Reported beside the headline figure, which
@@ -598,7 +610,7 @@ def bench_decode_step(args):
     # pools re-encoded on the device, new rows encoded as the step writes them, attention
     # decoding inside its gather.  A different cache format, so a figure of its own.
     turbo3_step = None
-    if not args.skip_closed_loop:
+    if args.extras:
         rows = r.pools[0][0].nbytes // (hkv * 128 * 2)
         d_iota = hip.DeviceBuffer.from_numpy(np.arange(rows, dtype=np.int64))
         t3_pools = []
@@ -644,6 +656,14 @@ def bench_decode_step(args):
     algo_step = L * per_layer_w + sum_ctx * L * 2 * hkv * 128 * 2
     tok_s = S / (ms_step * 1e-3)
     achieved = attn_bytes / (ms_attn * 1e-3) / 1e9
+    # hardware-counter traffic of the dominant kernel: the counters cannot be read from inside
+    # this process, so the committed summary carries the measured bytes per launch together
+    # with the algorithmic bytes of the launches they were measured on (the roofline leg runs
+    # at step 0's contexts whatever --steps / --warmup are, so the two agree for this seed)
+    traffic = measured_traffic("paged_attn_decode_config5_pmc.txt")
+    if measured_traffic("paged_attn_decode_config5_pmc.txt",
+                        "algorithmic_bytes_per_launch:") != attn_bytes:
+        traffic = None
     return {
         "metric": "decode tok/s @ batch 32 (paged-attn + quant GEMV path)",
         "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
@@ -662,11 +682,12 @@ def bench_decode_step(args):
                    "hip_graph": True, "gpu_side_packing": True},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": measured_traffic("paged_attn_decode_config5_pmc.txt")
-                     if (steps, warmup) == (20, 3) else None,
-                     "traffic_source": "profiles/paged_attn_decode_config5_pmc.txt (rocprofv3 "
-                                       "--pmc FETCH_SIZE / WRITE_SIZE of this command at its "
-                                       "default steps, bytes per launch)",
+                     "traffic": traffic,
+                     "traffic_source": "profiles/paged_attn_decode_config5_pmc.txt: rocprofv3 "
+                                       "--pmc FETCH_SIZE, then WRITE_SIZE, of `bench.py "
+                                       "--skip-kernels`, each scaled by what the same counter "
+                                       "reads for that command's 256 MiB calibration copy; null "
+                                       "when the summary was taken at other bytes per launch",
                      "kernel": "paged_attn_balanced_kernel<4> (decode rows, one layer of the step)",
                      "ms_per_launch": round(ms_attn, 5), "algorithmic_bytes_per_launch": attn_bytes},
         "cpu_baseline": {"value": round(S / cpu_s, 3), "unit": "tok/s", "cores": cores,
@@ -690,10 +711,10 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=5.0)
     ap.add_argument("--skip-kernels", action="store_true",
                     help="only the decode-step line, without the per-kernel legs")
-    ap.add_argument("--skip-closed-loop", action="store_true",
-                    help="leave out the extra legs of the decode step (token ids in / token ids "
-                         "out with embedding, lm_head + greedy; the step over turbo3 KV pools); "
-                         "profiling runs use this")
+    ap.add_argument("--extras", action="store_true",
+                    help="add the extra legs of the decode step (token ids in / token ids out "
+                         "with embedding, lm_head + greedy; the step over turbo3 KV pools); not "
+                         "part of the metric, and not for runs under a profiler")
     ap.add_argument("--workload", default="all",
                     choices=["all", "step", "config1", "config2", "config3", "config4"],
                     help="all: the decode-step line with every leg inside it (default); "

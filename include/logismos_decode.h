@@ -300,17 +300,39 @@ logismos_status_t logismos_launch_paged_attn_varlen_fp16_phases(
     int head_dim, int block_size, int max_blocks_per_seq, int num_splits, float scale, int causal,
     int phases, logismos_stream_t stream);
 
+/* Decode rows only (one new token per sequence: total_tokens == num_seqs,
+ * cu_seqlens_q = 0,1,2,...), the bf16-rounded result written in the prepared
+ * layout of a following Q4G128 GEMM over K = num_q_heads*head_dim
+ * (`logismos_q4_xprep_bytes(num_seqs, num_q_heads*head_dim)` bytes; rows
+ * num_seqs..BP-1 of the layout are left as they are): what the step executor
+ * launches in front of its o projection (`merge_heads` then `wo`,
+ * crates/transformers/src/attention.rs:296-302).  num_seqs <= 32. */
+logismos_status_t logismos_launch_paged_attn_decode_fp16_xprep(
+    const void* q_f16, const void* k_pool_f16, const void* v_pool_f16, const int32_t* block_tables,
+    const int32_t* cu_seqlens_q, const int32_t* context_lens, void* out_prepared, void* workspace,
+    int num_seqs, int num_q_heads, int num_kv_heads, int head_dim, int block_size,
+    int max_blocks_per_seq, int num_splits, float scale, logismos_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Ragged packing and KV writes
  * ------------------------------------------------------------------------ */
 
 /* From per-sequence counts to the packed-batch index buffers, on the GPU:
  *   cu_seqlens[0] = 0, cu_seqlens[s+1] = cu_seqlens[s] + new_tokens[s]
- *   context_lens[s] = prior_ctx[s] + new_tokens[s]
- *   slot_mapping[cu_seqlens[s] + i] = slot of position prior_ctx[s] + i of sequence s
- *                                     (-1 when that position lies past max_blocks)
+ *   context_lens[s] = min(prior_ctx[s] + new_tokens[s], block_size * max_blocks)
+ *   slot_mapping[cu_seqlens[s] + i] = slot of position prior_ctx[s] + i of sequence s, or
+ *                                     -1 when that position lies past max_blocks or its
+ *                                     table entry names no block (negative, or
+ *                                     >= LOGISMOS_BLOCK_ID_LIMIT: the mark of an entry
+ *                                     that never had one)
  * new_tokens, prior_ctx int32 `[num_seqs]` (negative values count as 0);
- * slot_mapping int64 `[sum new_tokens]`.  The host never needs the total. */
+ * slot_mapping int64 `[sum new_tokens]`.  The host never needs the total.
+ * A sequence that outgrows its table row is the reference cache's
+ * `Error::LenOverflow` (crates/cache/src/flat.rs:180-255); a kernel cannot
+ * refuse, so the rows past the capacity get slot -1 (every writer skips them)
+ * and the context stops at the capacity (the attention never walks past the
+ * row); the scheduler is expected to have checked the length on the host. */
+#define LOGISMOS_BLOCK_ID_LIMIT 0x3FFFFFF
 logismos_status_t logismos_check_pack_ragged_shape(int num_seqs, int block_size, int max_blocks,
                                                    char* msg, size_t msg_cap);
 logismos_status_t logismos_launch_pack_ragged(const int32_t* new_tokens, const int32_t* prior_ctx,
@@ -345,9 +367,12 @@ logismos_status_t logismos_launch_add_rms_norm_bf16(void* h_f32, const void* y_b
 /* Splits qkv (bf16 `[T][(hq+2*hkv)*128]`, q heads, then k heads, then v heads),
  * applies RoPE in the halves convention (`rope_halves_in_place`,
  * crates/kernels/src/cpu_f32/mod.rs:502-547) to q and k with the token's
- * position (clamped to [0, max_pos)), and writes q as fp16 `[T][hq][128]`, k and
+ * position, and writes q as fp16 `[T][hq][128]`, k and
  * v as fp16 rows of the paged pools at slot_mapping[t] (negative: skipped).
- * cos / sin: fp32 `[max_pos][64]` (`build_rope_table_f32`, :599-619). */
+ * cos / sin: fp32 `[max_pos][64]` (`build_rope_table_f32`, :599-619).  The caller
+ * guarantees 0 <= positions[t] < max_pos (`RopeTable::gather` fails on a position past the
+ * table); the kernel only keeps an out-of-range position from reading outside the tables
+ * (it uses the nearest table row) and the result for such a token is unspecified. */
 logismos_status_t logismos_launch_rope_kv_write_fp16(
     const void* qkv_bf16, const int32_t* positions, const void* cos_f32, const void* sin_f32,
     const int64_t* slot_mapping, void* q_out_f16, void* k_pool_f16, void* v_pool_f16,
@@ -500,7 +525,9 @@ typedef struct {
 typedef struct {
     int num_layers, hidden, num_q_heads, num_kv_heads, head_dim, intermediate;
     float rms_eps;
-    int block_size, max_blocks_per_seq, max_pos;
+    int block_size, max_blocks_per_seq;
+    int max_pos; /* rows of the RoPE tables; >= block_size * max_blocks_per_seq, so that no
+                    position a block table can hold lies past the table (else rejected) */
     int vocab;     /* rows of the embedding table and of lm_head; 0 when neither is used */
     int kv_turbo3; /* != 0: the layers' pools are turbo3 pools (56 bytes per head row) */
 } logismos_decode_config_t;
@@ -610,7 +637,12 @@ enum {
  * cache.  close_seq and reset do not wait for the device: on the stream that
  * carried the sequence's copies and launches its blocks may be handed out
  * again at once (what the next owner writes is ordered behind them); work on
- * any other stream has to be ordered by the caller. */
+ * any other stream has to be ordered by the caller.  Table updates are copied
+ * to the device from staging memory that is not reused before the copy has
+ * run, never from the host table itself, so closing a sequence and reopening
+ * and growing its slot cannot change what an earlier, still queued update
+ * delivers (a reserve or put waits only if 32 such updates are all still
+ * queued). */
 int logismos_paged_kv_cache_create(const logismos_paged_kv_layout_t* layout,
                                    logismos_paged_kv_cache_t** out);
 void logismos_paged_kv_cache_destroy(logismos_paged_kv_cache_t* cache);

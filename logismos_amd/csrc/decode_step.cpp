@@ -62,6 +62,10 @@ bool config_ok(const logismos_decode_config_t* c, int b) {
     if (c->head_dim != 128 || c->num_q_heads <= 0 || c->num_kv_heads <= 0) return false;
     if (c->hidden % 128 != 0 || c->intermediate % 128 != 0) return false;
     if (((int64_t)c->num_q_heads * c->head_dim) % 128 != 0) return false;
+    // every position a block table can hold must have a row in the RoPE tables
+    if (c->block_size <= 0 || c->max_blocks_per_seq <= 0 ||
+        (int64_t)c->max_pos < (int64_t)c->block_size * c->max_blocks_per_seq)
+        return false;
     if (c->vocab < 0) return false;
     if (c->vocab > 0 && logismos_check_qgemm_q4g128_greedy_shape(b, c->vocab, c->hidden, nullptr, 0))
         return false;

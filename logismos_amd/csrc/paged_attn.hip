@@ -1520,6 +1520,20 @@ extern "C" logismos_status_t logismos_launch_paged_attn_varlen_fp16_phases(
                                  stream);
 }
 
+extern "C" logismos_status_t logismos_launch_paged_attn_decode_fp16_xprep(
+    const void* q_f16, const void* k_pool_f16, const void* v_pool_f16, const int32_t* block_tables,
+    const int32_t* cu_seqlens_q, const int32_t* context_lens, void* out_prepared, void* workspace,
+    int num_seqs, int num_q_heads, int num_kv_heads, int head_dim, int block_size,
+    int max_blocks_per_seq, int num_splits, float scale, logismos_stream_t stream) {
+    // the prepared layout holds at most 32 rows
+    if (num_seqs > 32) return hipErrorInvalidValue;
+    return lg::paged_attn_launch(q_f16, k_pool_f16, v_pool_f16, block_tables, cu_seqlens_q,
+                                 context_lens, out_prepared, workspace, num_seqs, num_seqs, 1,
+                                 num_q_heads, num_kv_heads, head_dim, block_size,
+                                 max_blocks_per_seq, num_splits, scale, 1,
+                                 LOGISMOS_ATTN_PHASE_ALL, 2, 0, stream);
+}
+
 extern "C" logismos_status_t logismos_launch_paged_attn_varlen_turbo3(
     const void* q_f16, const void* k_pool_t3, const void* v_pool_t3, const int32_t* block_tables,
     const int32_t* cu_seqlens_q, const int32_t* context_lens, void* out_f16, void* workspace,

@@ -11,11 +11,16 @@
 // fp16 `[num_kv_heads][head_dim]`, little-endian, in token order inside a block
 // (`CacheLayout`, crates/cache/src/flat.rs:36-69).
 //
-// Blocks come from a free list (most recently freed first).  The block tables live in
-// pinned host memory and are mirrored to the device with asynchronous copies on the
-// caller's stream whenever a sequence gains blocks, so a put or a reserve followed by a
-// launch on the same stream sees the new entries.  One thread at a time per cache.
+// Blocks come from a free list (most recently freed first).  The host keeps the block
+// tables as bookkeeping; whenever a sequence gains blocks the new entries are mirrored to
+// the device with an asynchronous copy on the caller's stream, so a put or a reserve
+// followed by a launch on the same stream sees them.  The source of such a copy is never
+// the bookkeeping row itself (a row is rewritten when its sequence slot is closed, reopened
+// and grown again, possibly before an earlier copy of it has run) but a slot of a ring of
+// pinned staging rows, reused only after an event recorded behind its copy has completed.
+// One thread at a time per cache.
 #include "launch_common.hpp"
+#include "staging_ring.hpp"
 
 #include <hip/hip_runtime.h>
 
@@ -24,12 +29,29 @@
 #include <new>
 #include <vector>
 
+namespace {
+
+constexpr int kStagingSlots = 32;
+
+// Fence of the staging ring: one HIP event per slot, recorded behind the slot's copy.
+struct EventFence {
+    hipEvent_t* events = nullptr;
+    void record(int slot, hipStream_t stream) { (void)hipEventRecord(events[slot], stream); }
+    void wait(int slot) { (void)hipEventSynchronize(events[slot]); }
+};
+
+}  // namespace
+
 struct logismos_paged_kv_cache {
     logismos_paged_kv_layout_t layout{};
     int device = 0;
     std::vector<void*> k_pools, v_pools;  // per layer, device
-    int32_t* bt_host = nullptr;           // pinned, [max_seqs][max_blocks_per_seq]
+    int32_t* bt_host = nullptr;           // pinned, [max_seqs][max_blocks_per_seq]; bookkeeping
     int32_t* bt_dev = nullptr;
+    int32_t* staging_mem = nullptr;       // pinned, [kStagingSlots][max_blocks_per_seq]
+    hipEvent_t staging_events[kStagingSlots] = {};
+    int staging_events_made = 0;
+    lg::StagingRing<EventFence, hipStream_t> staging;
     std::vector<int32_t> free_blocks;     // stack of physical block ids
     std::vector<uint8_t> seq_open;
     std::vector<int32_t> seq_blocks;      // blocks held by each sequence
@@ -66,16 +88,20 @@ int ensure_blocks(logismos_paged_kv_cache* c, int seq, int64_t rows, hipStream_t
         c->free_blocks.pop_back();
     }
     c->seq_blocks[(size_t)seq] = need;
+    // the copy reads its source when it runs: stage the entries, never copy from `r`
+    int32_t* staged = nullptr;
+    const int slot = c->staging.stage(r + have, need - have, &staged);
     const hipError_t e =
-        hipMemcpyAsync(c->bt_dev + (size_t)seq * c->layout.max_blocks_per_seq + have, r + have,
+        hipMemcpyAsync(c->bt_dev + (size_t)seq * c->layout.max_blocks_per_seq + have, staged,
                        sizeof(int32_t) * (size_t)(need - have), hipMemcpyHostToDevice, stream);
+    c->staging.queued(slot, stream);
     return e == hipSuccess ? LOGISMOS_KV_OK : LOGISMOS_KV_HIP_ERROR;
 }
 
-// The host row keeps its entries: a copy of them to the device that an earlier reserve or put
-// queued on a stream may not have run yet, and the launches queued behind it still need the
-// ids it carries.  (On one stream a freed block is safe to hand out at once: whatever the next
-// owner writes is ordered after those launches.)
+// Copies to the device that an earlier reserve or put queued may not have run yet; they read
+// their staging slots, so the bookkeeping row is free to be rewritten by the next owner of
+// this sequence slot.  (On one stream a freed block is safe to hand out at once: whatever the
+// next owner writes is ordered after the launches that still use it.)
 void release_blocks(logismos_paged_kv_cache* c, int seq) {
     const int32_t* r = c->row(seq);
     for (int b = c->seq_blocks[(size_t)seq] - 1; b >= 0; --b) c->free_blocks.push_back(r[b]);
@@ -97,7 +123,7 @@ extern "C" int logismos_paged_kv_cache_create(const logismos_paged_kv_layout_t* 
     if (row_elems % 8 != 0 || L.block_size % 16 != 0) return LOGISMOS_KV_SHAPE_MISMATCH;
     if ((int64_t)L.block_size * L.max_blocks_per_seq > INT32_MAX ||
         (int64_t)L.max_seqs * L.max_blocks_per_seq > INT32_MAX ||
-        (int64_t)L.block_size * row_elems > INT32_MAX || L.num_blocks >= kUnmapped)
+        (int64_t)L.block_size * row_elems > INT32_MAX || L.num_blocks > LOGISMOS_BLOCK_ID_LIMIT)
         return LOGISMOS_KV_SHAPE_MISMATCH;
 
     auto* c = new (std::nothrow) logismos_paged_kv_cache;
@@ -120,6 +146,16 @@ extern "C" int logismos_paged_kv_cache_create(const logismos_paged_kv_layout_t* 
     ok = ok && hipHostMalloc(reinterpret_cast<void**>(&c->bt_host), bt_bytes, hipHostMallocDefault) ==
                    hipSuccess;
     ok = ok && hipMalloc(reinterpret_cast<void**>(&c->bt_dev), bt_bytes) == hipSuccess;
+    ok = ok && hipHostMalloc(reinterpret_cast<void**>(&c->staging_mem),
+                             sizeof(int32_t) * (size_t)kStagingSlots * L.max_blocks_per_seq,
+                             hipHostMallocDefault) == hipSuccess;
+    for (int i = 0; ok && i < kStagingSlots; ++i) {
+        ok = hipEventCreateWithFlags(&c->staging_events[i], hipEventDisableTiming) == hipSuccess;
+        if (ok) c->staging_events_made = i + 1;
+    }
+    if (ok)
+        c->staging.init(c->staging_mem, kStagingSlots, L.max_blocks_per_seq,
+                        EventFence{c->staging_events});
     if (ok) {
         for (size_t i = 0; i < bt_bytes / sizeof(int32_t); ++i) c->bt_host[i] = kUnmapped;
         ok = hipMemcpy(c->bt_dev, c->bt_host, bt_bytes, hipMemcpyHostToDevice) == hipSuccess;
@@ -142,6 +178,9 @@ extern "C" int logismos_paged_kv_cache_create(const logismos_paged_kv_layout_t* 
 
 extern "C" void logismos_paged_kv_cache_destroy(logismos_paged_kv_cache_t* c) {
     if (!c) return;
+    if (c->staging.slots() > 0) c->staging.drain();
+    for (int i = 0; i < c->staging_events_made; ++i) (void)hipEventDestroy(c->staging_events[i]);
+    if (c->staging_mem) (void)hipHostFree(c->staging_mem);
     for (void* p : c->k_pools) (void)hipFree(p);
     for (void* p : c->v_pools) (void)hipFree(p);
     if (c->bt_dev) (void)hipFree(c->bt_dev);

@@ -368,6 +368,23 @@ __global__ __launch_bounds__(1024) void qgemm_q4g128_mfma_kernel(
     }
 }
 
+constexpr size_t kMaxLds = 160 * 1024;
+
+// LDS bytes of the MFMA path (per-wave partial slots + staged scales and zeros) for the
+// template form launch_mfma picks; the shape check and the launcher share it.
+static size_t mfma_lds_bytes(int b, int n, int k) {
+    const int groups = k / 128;
+    const int bt = b <= 16 ? 1 : 2;
+    const int gw = b <= 16 ? 2 : 1;
+    int waves = (groups + gw - 1) / gw;
+    if (waves > 16) waves = 16;
+    const int tiles = (n + 15) / 16;
+    const int cus = device_cu_count();
+    int t = (tiles + cus - 1) / cus;
+    if (t > 3) t = 3;
+    return (size_t)waves * t * bt * 16 * 16 * 4 + (size_t)2 * t * 16 * groups * 2;
+}
+
 template <int BT, int GW, int T>
 static hipError_t launch_mfma_t(const void* x, const void* qw, const void* scale, const void* zero,
                                 void* y, int b, int n, int k, hipStream_t stream) {
@@ -378,11 +395,13 @@ static hipError_t launch_mfma_t(const void* x, const void* qw, const void* scale
     const size_t lds =
         (size_t)waves * T * BT * 16 * 16 * 4 + (size_t)2 * T * 16 * groups * 2;
     auto kern = qgemm_q4g128_mfma_kernel<BT, GW, T>;
-    if (lds > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-    }
+    if (lds > kMaxLds) return hipErrorInvalidValue;  // the shape check refuses these shapes
+    // opt in to the full LDS once per instantiation (the attribute is per function and device;
+    // one device per process here)
+    static const hipError_t attr =
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds);
+    if (attr != hipSuccess) return attr;
     kern<<<dim3((tiles + T - 1) / T), dim3(64 * waves), lds, stream>>>(
         static_cast<const uint16_t*>(x), static_cast<const uint8_t*>(qw),
         static_cast<const __half*>(scale), static_cast<const __half*>(zero),
@@ -400,8 +419,6 @@ static hipError_t launch_mfma(const void* x, const void* qw, const void* scale, 
     if (t == 2) return launch_mfma_t<BT, GW, 2>(x, qw, scale, zero, y, b, n, k, stream);
     return launch_mfma_t<BT, GW, 1>(x, qw, scale, zero, y, b, n, k, stream);
 }
-
-constexpr size_t kMaxLds = 160 * 1024;
 
 }  // namespace lg
 
@@ -423,6 +440,12 @@ extern "C" logismos_status_t logismos_check_qgemm_q4g128_shape(int b, int n, int
     if (b <= 4 && (size_t)b * (k / 32) * 68 > lg::kMaxLds)
         return lg::reject(msg, msg_cap, "%s: batch*K = %lld does not fit the LDS staging of x", kn,
                           (long long)((int64_t)b * k));
+    // the matrix-core path (batch >= 3; ..._bf16_mfma refuses such a shape at any batch) stages a
+    // workgroup's scales and zeros for all of K next to its partial sums
+    if (b >= 3 && lg::mfma_lds_bytes(b, n, k) > lg::kMaxLds)
+        return lg::reject(msg, msg_cap,
+                          "%s: K = %d needs %zu bytes of LDS on the matrix-core path (limit %zu)",
+                          kn, k, lg::mfma_lds_bytes(b, n, k), lg::kMaxLds);
     return 0;
 }
 

@@ -35,14 +35,24 @@ __global__ __launch_bounds__(256) void pack_ragged_kernel(
     if (threadIdx.x == 0) {
         if (s == 0) cu_seqlens[0] = 0;
         cu_seqlens[s + 1] = start + n_new;
-        context_lens[s] = prior + n_new;
+        // a context never exceeds what the block table can hold: the attention kernels walk
+        // the table row by context_lens
+        const int64_t cap = (int64_t)block_size * max_blocks;
+        const int64_t ctx = (int64_t)prior + n_new;
+        context_lens[s] = (int32_t)(ctx < cap ? ctx : cap);
     }
     const int32_t* bt = block_tables + (int64_t)s * max_blocks;
     for (int i = threadIdx.x; i < n_new; i += 256) {
-        const int pos = prior + i;
-        const int blk = pos / block_size;
+        const int64_t pos = (int64_t)prior + i;
+        const int64_t blk = pos / block_size;
         int64_t slot = -1;
-        if (blk < max_blocks) slot = (int64_t)bt[blk] * block_size + (pos - blk * block_size);
+        if (blk < max_blocks) {
+            // an entry that names no block (negative, or the "unmapped" mark and above) gives
+            // no slot: the row is skipped by the writers instead of landing outside the pool
+            const int32_t id = bt[blk];
+            if (id >= 0 && id < LOGISMOS_BLOCK_ID_LIMIT)
+                slot = (int64_t)id * block_size + (pos - blk * block_size);
+        }
         slot_mapping[(int64_t)start + i] = slot;
     }
 }

@@ -63,6 +63,8 @@ _SIGNATURES = {
         (C.c_uint32, [_vp] * 8 + [_i] * 9 + [_f, _i, _vp]),
     "logismos_launch_paged_attn_varlen_fp16_phases":
         (C.c_uint32, [_vp] * 8 + [_i] * 9 + [_f, _i, _i, _vp]),
+    "logismos_launch_paged_attn_decode_fp16_xprep":
+        (C.c_uint32, [_vp] * 8 + [_i] * 7 + [_f, _vp]),
     "logismos_check_pack_ragged_shape": (C.c_uint32, [_i, _i, _i, C.c_char_p, _sz]),
     "logismos_launch_pack_ragged": (C.c_uint32, [_vp] * 6 + [_i, _i, _i, _vp]),
     "logismos_launch_kv_write_fp16": (C.c_uint32, [_vp] * 5 + [_i, _i, _i, _vp]),
@@ -290,6 +292,21 @@ def launch_paged_attn_varlen_fp16(q, k_pool, v_pool, block_tables, cu_seqlens_q,
         code = library().logismos_launch_paged_attn_varlen_fp16_phases(*args, int(phases),
                                                                        _raw(stream))
     _status("paged_attn_varlen_fp16", code)
+
+
+def launch_paged_attn_decode_fp16_xprep(q, k_pool, v_pool, block_tables, cu_seqlens_q,
+                                        context_lens, out_prepared, workspace, num_seqs,
+                                        num_q_heads, num_kv_heads, head_dim, block_size,
+                                        max_blocks_per_seq, num_splits, scale,
+                                        stream=None) -> None:
+    """Decode rows only, result in the prepared layout of the o projection."""
+    check_paged_attn_shape(num_seqs, num_seqs, 1, num_q_heads, num_kv_heads, head_dim, block_size,
+                           max_blocks_per_seq, num_splits)
+    _status("paged_attn_decode_fp16_xprep", library().logismos_launch_paged_attn_decode_fp16_xprep(
+        _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables), _ptr(cu_seqlens_q),
+        _ptr(context_lens), _ptr(out_prepared),
+        _ptr(workspace) if workspace is not None else None, num_seqs, num_q_heads, num_kv_heads,
+        head_dim, block_size, max_blocks_per_seq, num_splits, float(scale), _raw(stream)))
 
 
 def launch_probe_copy(src, dst, nbytes: int, stream=None) -> None:

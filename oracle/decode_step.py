@@ -44,7 +44,11 @@ def rope_kv_write(qkv, positions, cos, sin, slots, k_pool, v_pool, hq, hkv, d=12
     k = np.ascontiguousarray(x[:, hq:hq + hkv]).reshape(t * hkv, d)
     v = np.ascontiguousarray(x[:, hq + hkv:]).reshape(t, hkv * d)
     max_pos = cos.size // half
-    pos = np.clip(np.asarray(positions, np.int64), 0, max_pos - 1)
+    pos = np.asarray(positions, np.int64)
+    if pos.size and (pos.min() < 0 or pos.max() >= max_pos):
+        # `RopeTable::gather` (crates/transformers/src/rope.rs) fails on a position past the
+        # table; so does the oracle
+        raise ValueError(f"rope_kv_write: position outside the RoPE table of {max_pos} rows")
     cos2, sin2 = cos.reshape(max_pos, half), sin.reshape(max_pos, half)
     # `RopeTable::gather` (crates/transformers/src/rope.rs): one cos/sin row per (token, head)
     O.rope_halves_in_place(q, np.repeat(cos2[pos], hq, axis=0), np.repeat(sin2[pos], hq, axis=0),

@@ -752,6 +752,8 @@ void oracle_qgemm_q4g128_f32(const uint16_t* x_bf16, const uint8_t* qw, const ui
  *   block_tables[s][pos / block_size] * block_size + pos % block_size.
  * A position whose block index is >= max_blocks gets slot -1.  Returns the
  * number of such tokens, or -1 for a negative count. */
+#define ORACLE_BLOCK_ID_LIMIT 0x3FFFFFF /* entries from here up, and negative ones, name no block */
+
 int oracle_pack_ragged(const int32_t* new_tokens, const int32_t* prior_ctx,
                        const int32_t* block_tables, int32_t* cu_seqlens, int64_t* slot_mapping,
                        int32_t* context_lens, size_t num_seqs, size_t block_size,
@@ -761,17 +763,22 @@ int oracle_pack_ragged(const int32_t* new_tokens, const int32_t* prior_ctx,
     for (size_t s = 0; s < num_seqs; ++s) {
         if (new_tokens[s] < 0 || prior_ctx[s] < 0) return -1;
         cu_seqlens[s + 1] = cu_seqlens[s] + new_tokens[s];
-        context_lens[s] = prior_ctx[s] + new_tokens[s];
+        /* the reference cache refuses to grow past its capacity (Error::LenOverflow,
+         * crates/cache/src/flat.rs:180-255); a packer cannot refuse, so the context stops at
+         * what the table row can hold and the tokens past it get no slot */
+        int64_t cap = (int64_t)block_size * (int64_t)max_blocks;
+        int64_t ctx = (int64_t)prior_ctx[s] + (int64_t)new_tokens[s];
+        context_lens[s] = (int32_t)(ctx < cap ? ctx : cap);
         for (int32_t i = 0; i < new_tokens[s]; ++i) {
             size_t pos = (size_t)prior_ctx[s] + (size_t)i;
             size_t blk = pos / block_size;
             int64_t slot;
-            if (blk >= max_blocks) {
-                slot = -1;
+            int32_t id = blk < max_blocks ? block_tables[s * max_blocks + blk] : -1;
+            if (blk >= max_blocks || id < 0 || id >= ORACLE_BLOCK_ID_LIMIT) {
+                slot = -1; /* past the table, or an entry that names no block */
                 bad++;
             } else {
-                slot = (int64_t)block_tables[s * max_blocks + blk] * (int64_t)block_size +
-                       (int64_t)(pos % block_size);
+                slot = (int64_t)id * (int64_t)block_size + (int64_t)(pos % block_size);
             }
             slot_mapping[(size_t)cu_seqlens[s] + (size_t)i] = slot;
         }

@@ -103,6 +103,8 @@ def test_num_splits_and_workspace_are_pure_functions():
 @pytest.mark.parametrize("b,n,k,frag", [
     (0, 8, 128, "batch must be positive"), (1, 0, 128, "N must be positive"),
     (1, 8, 64, "multiple of the group size 128"), (1, 1 << 20, 1 << 12, "exceeds i32::MAX"),
+    # scales and zeros of all of K next to the partial sums exceed 160 KiB on the MFMA path
+    (32, 12288, 45056, "bytes of LDS"),
 ])
 def test_qgemm_q4_shape_guard(b, n, k, frag):
     with pytest.raises(kernels.UnsupportedShape) as e:

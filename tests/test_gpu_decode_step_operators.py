@@ -1,0 +1,226 @@
+"""Config 5's decode step operator by operator, at its own contexts (32 live sequences,
+contexts U[256,8192], Qwen3-8B-style geometry, one layer), through the C ABI.
+
+Every GPU operator of the step is fed the CPU oracle's input for that operator (the
+`trace=` hook of oracle/decode_step.py) and held to the decode path's tolerance, 2e-3
+absolute or 1e-2 relative, so an operator's error is judged on its own and not after it has
+been amplified by the ones behind it.  The whole step, which at these contexts runs the
+balanced decode-attention kernel writing the prepared layout of the o projection, is then
+checked end to end.
+"""
+import copy
+
+import numpy as np
+import pytest
+
+import oracle as O
+from oracle import decode_step as OS
+from logismos_amd import hip, kernels
+from tests import workloads
+from tests.gpu_harness import DecodeStepRunner, assert_parity
+
+pytestmark = pytest.mark.gpu
+
+S, HIDDEN, HQ, HKV, D, INTER, BS = 32, 4096, 32, 8, 128, 12288, 16
+
+
+class _Case:
+    pass
+
+
+@pytest.fixture(scope="module")
+def case():
+    c = _Case()
+    rng = np.random.default_rng(workloads.SEED + 5)
+    c.ctx = rng.integers(256, 8193, size=S)  # the benchmark's first draw of live contexts
+    c.cfg, c.layers, c.batch = workloads.decode_step_problem(
+        rng, num_layers=1, hidden=HIDDEN, hq=HQ, hkv=HKV, inter=INTER, ctx=c.ctx)
+    c.lay = copy.deepcopy(c.layers)
+    c.bat = dict(c.batch, h=c.batch["h"].copy())
+    c.trace = []
+    c.out = OS.decode_step(c.cfg, c.lay, c.bat, trace=c.trace)
+    c.t = c.trace[0]
+    c.max_blocks = c.batch["block_tables"].shape[1]
+    return c
+
+
+def unprepare(buf, b, k):
+    """prepared layout -> (bf16 bits [b][k], group sums [b][k/128])"""
+    bp = 16 if b <= 16 else 32
+    chunks = k // 8
+    xp = buf[: chunks * bp * 16].view(np.uint16).reshape(chunks, bp, 8)
+    nat = np.empty_like(xp)
+    nat[..., [0, 4, 1, 5, 2, 6, 3, 7]] = xp  # pairs (x0,x4)(x1,x5)(x2,x6)(x3,x7) -> natural
+    x = nat.transpose(1, 0, 2).reshape(bp, k)[:b]
+    xg = buf[chunks * bp * 16:].view(np.float32).reshape(k // 128, bp).T[:b]
+    return x, xg
+
+
+def gemm_prepared(x_bits, w, b):
+    """The step's GEMM: prepared x -> fp32 K parts, added in ascending order as the
+    consumers do."""
+    qw, s, z = w
+    n, k = qw.shape[0], qw.shape[1] * 2
+    d_x = hip.DeviceBuffer.from_numpy(np.ascontiguousarray(x_bits, np.uint16))
+    d_xp = hip.DeviceBuffer(kernels.q4_xprep_bytes(b, k))
+    kernels.launch_q4_prepare_x_bf16(d_x, d_xp, b, k)
+    j = kernels.qgemm_q4g128_splitk_parts(b, n, k, prepared=True)
+    assert j > 0
+    d_parts = hip.DeviceBuffer(j * b * n * 4)
+    d_parts.fill(0xFF)
+    kernels.launch_qgemm_q4g128_f32_splitk(
+        d_xp, hip.DeviceBuffer.from_numpy(qw), hip.DeviceBuffer.from_numpy(s.view(np.uint16)),
+        hip.DeviceBuffer.from_numpy(z.view(np.uint16)), d_parts, b, n, k, prepared=True)
+    hip.synchronize()
+    parts = d_parts.to_numpy(np.float32, (j, b, n))
+    acc = parts[0].copy()
+    for i in range(1, j):
+        acc += parts[i]
+    return acc
+
+
+def test_norm1_into_the_prepared_layout(case):
+    h = case.batch["h"]
+    d_h = hip.DeviceBuffer.from_numpy(h)
+    d_xp = hip.DeviceBuffer(kernels.q4_xprep_bytes(S, HIDDEN))
+    kernels.launch_add_rms_norm_f32p_xprep(
+        d_h, None, 0, hip.DeviceBuffer.from_numpy(case.layers[0]["norm1"]), d_xp, S, HIDDEN,
+        case.cfg["eps"])
+    hip.synchronize()
+    assert np.array_equal(d_h.to_numpy(np.float32, h.shape), h)  # nothing to add: h untouched
+    x, xg = unprepare(d_xp.to_numpy(np.uint8, (d_xp.nbytes,)), S, HIDDEN)
+    assert_parity(O.bf16_bits_to_f32(x), O.bf16_bits_to_f32(case.t["xn"]), what="norm1")
+    sums = O.bf16_bits_to_f32(x).reshape(S, HIDDEN // 128, 128).sum(axis=2)
+    assert np.abs(xg - sums).max() < 1e-3
+
+
+@pytest.mark.parametrize("name,src", [("qkv", "xn"), ("gate_up", "xn2"), ("down", "act")])
+def test_projection(case, name, src):
+    got = gemm_prepared(case.t[src], case.layers[0][name], S)
+    want = case.t[{"qkv": "qkv", "gate_up": "gu", "down": "down"}[name]]
+    assert_parity(got, want, what=f"{name} projection")
+
+
+def test_o_projection(case):
+    x = O.f32_to_bf16_bits(case.t["attn"].reshape(S, HQ * D))
+    got = gemm_prepared(x, case.layers[0]["o"], S)
+    assert_parity(got, case.t["o"], what="o projection")
+
+
+def test_rope_and_kv_append(case):
+    b, L0 = case.batch, case.layers[0]
+    max_pos = b["cos"].size // (D // 2)
+    d_kp = hip.DeviceBuffer.from_numpy(L0["k_pool"])
+    d_vp = hip.DeviceBuffer.from_numpy(L0["v_pool"])
+    d_q = hip.DeviceBuffer(S * HQ * D * 2)
+    kernels.launch_rope_kv_write_f32p(
+        hip.DeviceBuffer.from_numpy(case.t["qkv"]), 1,
+        hip.DeviceBuffer.from_numpy(np.ascontiguousarray(b["positions"], np.int32)),
+        hip.DeviceBuffer.from_numpy(b["cos"]), hip.DeviceBuffer.from_numpy(b["sin"]),
+        hip.DeviceBuffer.from_numpy(np.ascontiguousarray(b["slots"], np.int64)), d_q, d_kp, d_vp,
+        S, HQ, HKV, D, max_pos)
+    hip.synchronize()
+    assert_parity(d_q.to_numpy(np.float16, (S, HQ, D)), case.t["q"], max_abs=1e-3, max_rel=2e-3,
+                  what="roped q")
+    slots = np.asarray(b["slots"])
+    kp = d_kp.to_numpy(np.float16, L0["k_pool"].shape)
+    vp = d_vp.to_numpy(np.float16, L0["v_pool"].shape)
+    assert_parity(kp[slots], case.lay[0]["k_pool"][slots], max_abs=1e-3, max_rel=2e-3,
+                  what="appended K rows")
+    # V is not rotated: one fp16 rounding of the same fp32 number on both sides
+    assert np.array_equal(vp[slots].view(np.uint16), case.lay[0]["v_pool"][slots].view(np.uint16))
+    # every other row of the pools is untouched: integer work, bit-exact
+    rest = np.ones(kp.shape[0], bool)
+    rest[slots] = False
+    assert np.array_equal(kp[rest].view(np.uint16), L0["k_pool"][rest].view(np.uint16))
+    assert np.array_equal(vp[rest].view(np.uint16), L0["v_pool"][rest].view(np.uint16))
+
+
+def test_decode_attention_into_the_prepared_layout(case):
+    """The launch the step makes: decode rows at config 5's contexts go to the balanced
+    kernel (the block tables are far wider than the static-split bound), whose merge writes
+    the bf16 result in the prepared layout of the o projection."""
+    b = case.batch
+    ns = kernels.paged_attn_num_splits(S, HKV, BS, case.max_blocks)
+    assert S * HKV * BS * case.max_blocks > 200000 and ns > 2  # not the small-batch kernel
+    d_ws = hip.DeviceBuffer(kernels.paged_attn_workspace_bytes(S, HQ, D, ns))
+    d_ws.fill(0xFF)
+    d_out = hip.DeviceBuffer(kernels.q4_xprep_bytes(S, HQ * D))
+    d_out.fill(0xFF)
+    kernels.launch_paged_attn_decode_fp16_xprep(
+        hip.DeviceBuffer.from_numpy(case.t["q"]), hip.DeviceBuffer.from_numpy(case.lay[0]["k_pool"]),
+        hip.DeviceBuffer.from_numpy(case.lay[0]["v_pool"]),
+        hip.DeviceBuffer.from_numpy(b["block_tables"]),
+        hip.DeviceBuffer.from_numpy(np.ascontiguousarray(b["cu_seqlens"], np.int32)),
+        hip.DeviceBuffer.from_numpy(np.ascontiguousarray(b["context_lens"], np.int32)),
+        d_out, d_ws, S, HQ, HKV, D, BS, case.max_blocks, ns, 1.0 / np.sqrt(128.0))
+    hip.synchronize()
+    x, xg = unprepare(d_out.to_numpy(np.uint8, (d_out.nbytes,)), S, HQ * D)
+    got = O.bf16_bits_to_f32(x)
+    assert_parity(got, case.t["attn"].reshape(S, HQ * D), what="decode attention (prepared)")
+    assert np.abs(xg - got.reshape(S, HQ, 128).sum(axis=2)).max() < 1e-3
+    # the same rows as plain fp16 through the public launcher
+    d_o16 = hip.DeviceBuffer(S * HQ * D * 2)
+    kernels.launch_paged_attn_varlen_fp16(
+        hip.DeviceBuffer.from_numpy(case.t["q"]), hip.DeviceBuffer.from_numpy(case.lay[0]["k_pool"]),
+        hip.DeviceBuffer.from_numpy(case.lay[0]["v_pool"]),
+        hip.DeviceBuffer.from_numpy(b["block_tables"]),
+        hip.DeviceBuffer.from_numpy(np.ascontiguousarray(b["cu_seqlens"], np.int32)),
+        hip.DeviceBuffer.from_numpy(np.ascontiguousarray(b["context_lens"], np.int32)),
+        d_o16, d_ws, S, S, 1, HQ, HKV, D, BS, case.max_blocks, ns, 1.0 / np.sqrt(128.0))
+    hip.synchronize()
+    assert_parity(d_o16.to_numpy(np.float16, (S, HQ * D)), case.t["attn"].reshape(S, HQ * D),
+                  what="decode attention (fp16)")
+
+
+def test_residual_add_and_norm2(case):
+    h0 = case.batch["h"]
+    d_h = hip.DeviceBuffer.from_numpy(h0)
+    d_xp = hip.DeviceBuffer(kernels.q4_xprep_bytes(S, HIDDEN))
+    kernels.launch_add_rms_norm_f32p_xprep(
+        d_h, hip.DeviceBuffer.from_numpy(case.t["o"]), 1,
+        hip.DeviceBuffer.from_numpy(case.layers[0]["norm2"]), d_xp, S, HIDDEN, case.cfg["eps"])
+    hip.synchronize()
+    # the residual add is one fp32 add per element: bit-exact
+    assert np.array_equal(d_h.to_numpy(np.float32, h0.shape), case.t["h"])
+    x, _ = unprepare(d_xp.to_numpy(np.uint8, (d_xp.nbytes,)), S, HIDDEN)
+    assert_parity(O.bf16_bits_to_f32(x), O.bf16_bits_to_f32(case.t["xn2"]), what="norm2")
+
+
+def test_silu_mul_into_the_prepared_layout(case):
+    d_xp = hip.DeviceBuffer(kernels.q4_xprep_bytes(S, INTER))
+    kernels.launch_silu_mul_f32p_xprep(hip.DeviceBuffer.from_numpy(case.t["gu"]), 1, d_xp, S, INTER)
+    hip.synchronize()
+    x, _ = unprepare(d_xp.to_numpy(np.uint8, (d_xp.nbytes,)), S, INTER)
+    assert_parity(O.bf16_bits_to_f32(x), O.bf16_bits_to_f32(case.t["act"]), what="silu * up")
+
+
+def test_final_add_and_norm(case):
+    d_h = hip.DeviceBuffer.from_numpy(case.t["h"])
+    d_out = hip.DeviceBuffer(S * HIDDEN * 2)
+    kernels.launch_add_rms_norm_f32p(
+        d_h, hip.DeviceBuffer.from_numpy(case.t["down"]), 1,
+        hip.DeviceBuffer.from_numpy(case.batch["final_norm"]), d_out, S, HIDDEN, case.cfg["eps"])
+    hip.synchronize()
+    assert np.array_equal(d_h.to_numpy(np.float32, (S, HIDDEN)), case.bat["h"])
+    assert_parity(O.bf16_bits_to_f32(d_out.to_numpy(np.uint16, (S, HIDDEN))),
+                  O.bf16_bits_to_f32(case.out), what="final norm")
+
+
+def test_whole_step_at_config5_contexts(case):
+    """logismos_launch_decode_step on the same problem: the operators above chained on the
+    device.  One-ulp bf16 differences of an intermediate are carried through the layer, so the
+    end-to-end bound is wider than an operator's: relative L2 and two bf16 ulps per element."""
+    r = DecodeStepRunner(case.cfg, case.layers, case.batch)
+    r.launch()
+    got = O.bf16_bits_to_f32(r.result_bits())
+    want = O.bf16_bits_to_f32(case.out)
+    rel = float(np.linalg.norm(got - want) / np.linalg.norm(want))
+    assert rel < 4e-3, rel
+    assert np.all(np.abs(got - want) <= 4e-3 + 1.6e-2 * np.abs(want))
+    h_gpu = r.h.to_numpy(np.float32, case.bat["h"].shape)
+    assert float(np.linalg.norm(h_gpu - case.bat["h"]) / np.linalg.norm(case.bat["h"])) < 2e-3
+    kp, vp = r.pools[0]
+    slots = np.asarray(case.batch["slots"])
+    assert_parity(kp.to_numpy(np.float16, case.lay[0]["k_pool"].shape)[slots],
+                  case.lay[0]["k_pool"][slots], what="K rows appended by the step")

@@ -257,3 +257,49 @@ def test_retiring_a_sequence_does_not_disturb_a_queued_table_copy():
     assert sorted(want.tolist()) == sorted(set(want.tolist())) and (want < 6).all()
     assert np.array_equal(got.reshape(-1, 3)[s], want)
     assert c.free_blocks() == 6
+
+
+def test_reopened_slot_does_not_change_a_queued_table_update():
+    """A sequence retires and its slot is reopened and grown while the stream is still busy:
+    the table update queued for the first owner must deliver the first owner's block ids (the
+    cache stages every update; it does not copy from the host table, which the second owner
+    rewrites).  The gather queued between the two owners reads the device table when it runs."""
+    c = small(num_layers=1, num_kv_heads=1, head_dim=8, num_blocks=8, max_seqs=2,
+              max_blocks_per_seq=4)
+    row = 8
+    nrows = 8 * 16
+    # pool row r holds the value r in every element
+    pool = np.repeat(np.arange(nrows, dtype=np.float16)[:, None], row, axis=1)
+    d_pool = hip.DeviceBuffer.from_numpy(pool)
+    view_k = hip.DevicePtrView(c.k_pool(0), pool.nbytes)
+    view_v = hip.DevicePtrView(c.v_pool(0), pool.nbytes)
+    for view in (view_k, view_v):
+        hip.check(hip._runtime().hipMemcpy(view.ptr, d_pool.ptr, pool.nbytes, 3), "hipMemcpy")
+    stream = hip.Stream()
+    busy = hip.DeviceBuffer(1 << 30)
+    a = c.open_seq()
+    other = c.open_seq()
+    # keep the stream busy so that the copies below are still queued while the host goes on
+    for _ in range(4):
+        kernels.launch_probe_copy(busy, busy.offset(1 << 29), 1 << 29, stream)
+    c.reserve(a, 32, stream)
+    first_owner = c.block_tables_host()[a, :2].copy()
+    c.advance(a, 0, 32)
+    k_out = hip.DeviceBuffer(32 * row * 2)
+    v_out = hip.DeviceBuffer(32 * row * 2)
+    _check = c._lib.logismos_paged_kv_cache_get(c._h, a, 0, 32, k_out.ptr, v_out.ptr, stream.raw)
+    assert _check == 0
+    c.close_seq(a)
+    c.reserve(other, 16, stream)           # takes the block the first owner freed last
+    b = c.open_seq()
+    assert b == a                          # the slot is handed out again
+    c.reserve(b, 48, stream)
+    second_owner = c.block_tables_host()[b, :3].copy()
+    assert not np.array_equal(second_owner[:2], first_owner)
+    stream.synchronize()
+    want = np.concatenate([np.arange(16) + 16 * int(blk) for blk in first_owner])
+    got = k_out.to_numpy(np.float16, (32, row))
+    assert np.array_equal(got[:, 0].astype(np.int64), want)
+    # and the device table ends up with the second owner's ids
+    bt = hip.DevicePtrView(c.block_tables(), 2 * 4 * 4).to_numpy(np.int32, (2, 4))
+    assert np.array_equal(bt[b, :3], second_owner)

@@ -50,6 +50,19 @@ def test_config4_mixed_batch_packing_is_bit_exact():
     _check_pack(new, prior, bt, 16)
 
 
+def test_overflowing_and_unmapped_positions_get_no_slot():
+    # past the table row: slot -1 and the context capped; entries that name no block
+    # (negative, the cache's 0x3FFFFFFF mark, anything from LOGISMOS_BLOCK_ID_LIMIT up): -1
+    bt = np.array([[1, 0, 7, 7, 7], [5, 0x3FFFFFFF, -3, 0x3FFFFFF, 0x3FFFFFE]], np.int32)
+    new, prior = [60, 80], [30, 0]
+    cu, slots, ctx = _pack_gpu(new, prior, bt, 16)
+    cu_o, slots_o, ctx_o, bad = O.pack_ragged(new, prior, bt, 16)
+    assert np.array_equal(cu, cu_o) and np.array_equal(ctx, ctx_o)
+    assert np.array_equal(slots, slots_o)
+    assert ctx.tolist() == [80, 80] and bad == 10 + 48
+    assert (slots[50:60] == -1).all() and (slots[60 + 16:60 + 64] == -1).all()
+
+
 @pytest.mark.parametrize("s", [1, 2, 63, 64, 65, 257, 1000, 5000])
 def test_sequence_counts(s):
     rng = np.random.default_rng(s)

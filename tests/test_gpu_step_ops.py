@@ -34,7 +34,7 @@ def test_rope_kv_write_matches_oracle_and_reference_table():
     rng = np.random.default_rng(21)
     t, hq, hkv, d, bs, nblk, max_pos = 7, 8, 2, 128, 16, 12, 4096
     qkv = O.f32_to_bf16_bits(rng.standard_normal((t, (hq + 2 * hkv) * d), np.float32))
-    positions = np.array([0, 1, 17, 4095, 300, 5000, 2], np.int32)  # 5000 clamps to 4095
+    positions = np.array([0, 1, 17, 4095, 300, 4094, 2], np.int32)
     slots = rng.permutation(nblk * bs)[:t].astype(np.int64)
     slots[3] = -1
     cos, sin = O.build_rope_table_f32(max_pos, d, 1_000_000.0)

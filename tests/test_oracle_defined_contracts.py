@@ -205,8 +205,20 @@ def test_pack_ragged_overflowing_position_gets_minus_one():
     bt = np.arange(2, dtype=np.int32).reshape(1, 2)
     cu, slots, ctx, bad = O.pack_ragged([3], [30], bt, 16)
     assert bad == 1 and slots.tolist() == [1 * 16 + 14, 1 * 16 + 15, -1]
+    assert ctx.tolist() == [32]  # capped at what the table row holds (LenOverflow upstream)
     with pytest.raises(ValueError):
         O.pack_ragged([-1], [0], bt, 16)
+
+
+def test_pack_ragged_entries_that_name_no_block_give_no_slot():
+    # the cache marks never-mapped entries 0x3FFFFFFF; the workloads poison with 0x3FFFFFF;
+    # a negative id is no block either
+    bt = np.array([[5, 0x3FFFFFFF, -3, 0x3FFFFFF, 0x3FFFFFE]], np.int32)
+    cu, slots, ctx, bad = O.pack_ragged([80], [0], bt, 16)
+    assert bad == 48 and ctx.tolist() == [80]
+    assert slots[:16].tolist() == [5 * 16 + i for i in range(16)]
+    assert (slots[16:64] == -1).all()
+    assert slots[64:].tolist() == [0x3FFFFFE * 16 + i for i in range(16)]
 
 
 def test_kv_write_then_gather_is_identity_through_a_permutation():

@@ -1,6 +1,8 @@
 """Host-side checks of the paged KV cache that need no GPU: layouts are validated before
 any HIP call, and null handles are tolerated by the accessors."""
 import ctypes as C
+import os
+import subprocess
 
 import pytest
 
@@ -48,3 +50,19 @@ def test_append_and_gather_reject_bad_arguments_on_the_host():
                                               None) == 0   # nothing to do
     assert lib.logismos_launch_kv_gather_fp16(None, None, None, None, None, 0, 3, 2, 8, 16,
                                               None) == 1   # null pointers
+
+
+def test_block_table_updates_are_staged_until_their_copy_has_run(tmp_path):
+    """The deferral rule of the cache's block-table mirror (lg::StagingRing): a queued copy
+    delivers what the table row held when it was queued, whatever the host writes to the row
+    afterwards, and a staging slot is reused only behind its fence.  Exercised with a
+    simulated stream (tests/cpp/staging_ring_test.cpp, plain g++, no device)."""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = tmp_path / "staging_ring_test"
+    subprocess.run(["g++", "-std=c++17", "-O1", "-Wall", "-Werror",
+                    "-I", os.path.join(root, "logismos_amd", "csrc"),
+                    os.path.join(root, "tests", "cpp", "staging_ring_test.cpp"), "-o", str(exe)],
+                   check=True)
+    r = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "staging ring ok" in r.stdout

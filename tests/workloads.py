@@ -170,6 +170,8 @@ def decode_step_problem(rng, num_layers, hidden, hq, hkv, inter, ctx, d=128, blo
             gate_up=q4(2 * inter, hidden), down=q4(hidden, inter),
             k_pool=rng.standard_normal((rows, hkv * d), np.float32).astype(np.float16),
             v_pool=rng.standard_normal((rows, hkv * d), np.float32).astype(np.float16)))
+    # the RoPE tables cover every position the block tables can hold
+    max_pos = max(max_pos, block_size * base["block_tables"].shape[1])
     cos, sin = O.build_rope_table_f32(max_pos, d, theta)
     cu, slots, ctx_lens, _ = O.pack_ragged(np.ones(b, np.int32), ctx - 1, base["block_tables"],
                                            block_size)
