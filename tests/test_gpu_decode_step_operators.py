@@ -209,15 +209,20 @@ def test_final_add_and_norm(case):
 
 def test_whole_step_at_config5_contexts(case):
     """logismos_launch_decode_step on the same problem: the operators above chained on the
-    device.  One-ulp bf16 differences of an intermediate are carried through the layer, so the
-    end-to-end bound is wider than an operator's: relative L2 and two bf16 ulps per element."""
+    device.  Each operator alone agrees with the oracle far inside its tolerance (the GEMMs to
+    3e-6 relative), but every bf16 rounding point turns a pre-rounding difference d into one-ulp
+    flips of a fraction d / ulp of the elements, i.e. an error of about sqrt(d * ulp): measured
+    stage by stage on this problem, 8e-5 after the first norm and GEMM grows to 3e-4 after the
+    second norm and 1.3e-3 after silu * up and the down projection.  The end-to-end bound is
+    therefore a relative L2 plus, per element, what a 2e-3 rms error distribution reaches over
+    131072 outputs and one ulp of the bf16 result itself."""
     r = DecodeStepRunner(case.cfg, case.layers, case.batch)
     r.launch()
     got = O.bf16_bits_to_f32(r.result_bits())
     want = O.bf16_bits_to_f32(case.out)
     rel = float(np.linalg.norm(got - want) / np.linalg.norm(want))
     assert rel < 4e-3, rel
-    assert np.all(np.abs(got - want) <= 4e-3 + 1.6e-2 * np.abs(want))
+    assert np.all(np.abs(got - want) <= 1.2e-2 + 1.6e-2 * np.abs(want))
     h_gpu = r.h.to_numpy(np.float32, case.bat["h"].shape)
     assert float(np.linalg.norm(h_gpu - case.bat["h"]) / np.linalg.norm(case.bat["h"])) < 2e-3
     kp, vp = r.pools[0]
