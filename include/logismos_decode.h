@@ -20,9 +20,13 @@
  *   - index arithmetic inside the kernels is 64-bit
  *     (crates/kernels/src/matmul/hip/matmul_naive.hip:26-41).
  *
- * The library keeps no global mutable state and is re-entrant across
- * streams (the reference's `Stream` is Send but not Sync,
- * crates/hipcore/src/stream.rs:21-25: one caller thread per stream).
+ * The library is re-entrant across streams (the reference's `Stream` is Send
+ * but not Sync, crates/hipcore/src/stream.rs:21-25: one caller thread per
+ * stream): no launch changes library state.  What it keeps are values computed
+ * once per process and the same from whichever thread computes them first (the
+ * device's CU count, kernel attribute opt-ins, the address of the static
+ * workspace of the `_noalloc` entry point), for the device that is current at
+ * that moment: one device per process.
  *
  * The reference defines none of the data contracts below (its `sched`,
  * paged `cache` and weight-`quant` crates are scaffolds); they extend the
@@ -299,6 +303,27 @@ logismos_status_t logismos_launch_paged_attn_varlen_fp16_phases(
     int num_seqs, int total_tokens, int max_seqlen_q, int num_q_heads, int num_kv_heads,
     int head_dim, int block_size, int max_blocks_per_seq, int num_splits, float scale, int causal,
     int phases, logismos_stream_t stream);
+
+/* The full launch above without a workspace argument and without any allocation.
+ * No counterpart in the reference: it is for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * it).  The split-K partials go to a static device array of
+ * LOGISMOS_PAGED_ATTN_STATIC_WORKSPACE_BYTES bytes that every device the library
+ * runs on holds until the process ends; a launch whose
+ * `logismos_paged_attn_workspace_bytes(...)` exceeds it is refused with
+ * hipErrorInvalidValue (choose a smaller num_splits).  All calls on a device share
+ * that device's array: launches that can overlap in time (two streams, two
+ * threads) race on it and must be ordered by the caller.  The array needs no
+ * clearing between calls (its contents never matter on entry).  Results are
+ * identical to `logismos_launch_paged_attn_varlen_fp16` with the same arguments. */
+#define LOGISMOS_PAGED_ATTN_STATIC_WORKSPACE_BYTES (16u << 20)
+size_t logismos_paged_attn_static_workspace_bytes(void);
+logismos_status_t logismos_launch_paged_attn_varlen_fp16_noalloc(
+    const void* q_f16, const void* k_pool_f16, const void* v_pool_f16, const int32_t* block_tables,
+    const int32_t* cu_seqlens_q, const int32_t* context_lens, void* out_f16, int num_seqs,
+    int total_tokens, int max_seqlen_q, int num_q_heads, int num_kv_heads, int head_dim,
+    int block_size, int max_blocks_per_seq, int num_splits, float scale, int causal,
+    logismos_stream_t stream);
 
 /* Decode rows only (one new token per sequence: total_tokens == num_seqs,
  * cu_seqlens_q = 0,1,2,...), the bf16-rounded result written in the prepared

@@ -39,6 +39,8 @@
 #include <hip/hip_fp16.h>
 #include <math.h>
 
+#include <atomic>
+
 namespace lg {
 
 constexpr int kHeadDim = 128;
@@ -1547,6 +1549,62 @@ extern "C" logismos_status_t logismos_launch_paged_attn_varlen_turbo3(
                                  max_seqlen_q, num_q_heads, num_kv_heads, 128, block_size,
                                  max_blocks_per_seq, num_splits, scale, 1,
                                  LOGISMOS_ATTN_PHASE_ALL, 0, 1, stream);
+}
+
+// ---- the entry point that allocates nothing -------------------------------------------
+// Split-K partials live in a file-scope device array instead of a caller workspace.  In host
+// code the array's name is only a handle for the symbol: the device address is looked up once
+// per device with hipGetSymbolAddress and kept; kernels receive that address as an argument,
+// exactly as they receive a caller's workspace.
+namespace {
+constexpr size_t kStaticWorkspaceBytes = (size_t)LOGISMOS_PAGED_ATTN_STATIC_WORKSPACE_BYTES;
+constexpr int kMaxDevices = 64;
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[kStaticWorkspaceBytes];
+static std::atomic<void*> scratch_ptr[kMaxDevices];
+
+// Device address of this device's copy of `scratch` (each device holds its own), resolved on
+// the first call with that device current.
+static hipError_t static_workspace(void** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    void* p = scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!p) return hipErrorInvalidSymbol;
+        scratch_ptr[dev].store(p, std::memory_order_release);  // same value from any thread
+    }
+    *out = p;
+    return hipSuccess;
+}
+
+extern "C" size_t logismos_paged_attn_static_workspace_bytes(void) { return kStaticWorkspaceBytes; }
+
+extern "C" logismos_status_t logismos_launch_paged_attn_varlen_fp16_noalloc(
+    const void* q_f16, const void* k_pool_f16, const void* v_pool_f16, const int32_t* block_tables,
+    const int32_t* cu_seqlens_q, const int32_t* context_lens, void* out_f16, int num_seqs,
+    int total_tokens, int max_seqlen_q, int num_q_heads, int num_kv_heads, int head_dim,
+    int block_size, int max_blocks_per_seq, int num_splits, float scale, int causal,
+    logismos_stream_t stream) {
+    if (logismos_check_paged_attn_shape(num_seqs, total_tokens, max_seqlen_q, num_q_heads,
+                                        num_kv_heads, head_dim, block_size, max_blocks_per_seq,
+                                        num_splits, nullptr, 0) != 0)
+        return hipErrorInvalidValue;
+    // the partials of this launch must fit the array: a clear refusal, never a smaller split
+    if (logismos_paged_attn_workspace_bytes(num_seqs, num_q_heads, head_dim, num_splits) >
+        kStaticWorkspaceBytes)
+        return hipErrorInvalidValue;
+    void* ws = nullptr;
+    const hipError_t e = static_workspace(&ws);
+    if (e != hipSuccess) return e;
+    return lg::paged_attn_launch(q_f16, k_pool_f16, v_pool_f16, block_tables, cu_seqlens_q,
+                                 context_lens, out_f16, ws, num_seqs, total_tokens, max_seqlen_q,
+                                 num_q_heads, num_kv_heads, head_dim, block_size,
+                                 max_blocks_per_seq, num_splits, scale, causal,
+                                 LOGISMOS_ATTN_PHASE_ALL, 0, 0, stream);
 }
 
 logismos_status_t lg::paged_attn_launch(

@@ -63,6 +63,9 @@ _SIGNATURES = {
         (C.c_uint32, [_vp] * 8 + [_i] * 9 + [_f, _i, _vp]),
     "logismos_launch_paged_attn_varlen_fp16_phases":
         (C.c_uint32, [_vp] * 8 + [_i] * 9 + [_f, _i, _i, _vp]),
+    "logismos_paged_attn_static_workspace_bytes": (_sz, []),
+    "logismos_launch_paged_attn_varlen_fp16_noalloc":
+        (C.c_uint32, [_vp] * 7 + [_i] * 9 + [_f, _i, _vp]),
     "logismos_launch_paged_attn_decode_fp16_xprep":
         (C.c_uint32, [_vp] * 8 + [_i] * 7 + [_f, _vp]),
     "logismos_check_pack_ragged_shape": (C.c_uint32, [_i, _i, _i, C.c_char_p, _sz]),
@@ -292,6 +295,28 @@ def launch_paged_attn_varlen_fp16(q, k_pool, v_pool, block_tables, cu_seqlens_q,
         code = library().logismos_launch_paged_attn_varlen_fp16_phases(*args, int(phases),
                                                                        _raw(stream))
     _status("paged_attn_varlen_fp16", code)
+
+
+def launch_paged_attn_varlen_fp16_noalloc(q, k_pool, v_pool, block_tables, cu_seqlens_q,
+                                          context_lens, out, num_seqs, total_tokens, max_seqlen_q,
+                                          num_q_heads, num_kv_heads, head_dim, block_size,
+                                          max_blocks_per_seq, num_splits, scale, causal=True,
+                                          stream=None) -> None:
+    """The paged-attention launch over the library's static workspace: allocates nothing."""
+    check_paged_attn_shape(num_seqs, total_tokens, max_seqlen_q, num_q_heads, num_kv_heads,
+                           head_dim, block_size, max_blocks_per_seq, num_splits)
+    need = paged_attn_workspace_bytes(num_seqs, num_q_heads, head_dim, num_splits)
+    cap = library().logismos_paged_attn_static_workspace_bytes()
+    if need > cap:
+        raise UnsupportedShape("paged_attn_varlen_fp16_noalloc",
+                               f"split-K partials need {need} bytes, the static workspace "
+                               f"holds {cap}")
+    _status("paged_attn_varlen_fp16_noalloc",
+            library().logismos_launch_paged_attn_varlen_fp16_noalloc(
+                _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables), _ptr(cu_seqlens_q),
+                _ptr(context_lens), _ptr(out), num_seqs, total_tokens, max_seqlen_q, num_q_heads,
+                num_kv_heads, head_dim, block_size, max_blocks_per_seq, num_splits, float(scale),
+                1 if causal else 0, _raw(stream)))
 
 
 def launch_paged_attn_decode_fp16_xprep(q, k_pool, v_pool, block_tables, cu_seqlens_q,
