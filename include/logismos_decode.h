@@ -143,17 +143,34 @@ logismos_status_t logismos_check_paged_attn_shape(int num_seqs, int total_tokens
 logismos_status_t logismos_launch_qgemv_q8g32_f32(const void* x_f32, const void* qs_i8,
                                                   const void* d_f16, void* y_f32, int n, int k,
                                                   logismos_stream_t stream);
+/* ... `+ bias[n]` (fp32 `[N]`, NULL: none), added to the finished fp32 sum as
+ * `linear_t` adds it (crates/kernels/src/cpu_f32/mod.rs:336-343; the q/k/v
+ * projections of Qwen2 carry one, crates/transformers/src/attention.rs:49-57). */
+logismos_status_t logismos_launch_qgemv_q8g32_f32_bias(const void* x_f32, const void* qs_i8,
+                                                       const void* d_f16, const void* bias_f32,
+                                                       void* y_f32, int n, int k,
+                                                       logismos_stream_t stream);
 
 /* y[b][n] = sum_k x[b][k] * w[n][k], w in Q4G128.  x bf16 `[B][K]`, y bf16
  * `[B][N]`, fp32 accumulation, one rounding at the end: `cpu_f32::linear_t`
  * (crates/kernels/src/cpu_f32/mod.rs:271-345) over the dequantised matrix with
- * m = B <= 32.  Batch 1..2 runs the bandwidth-bound VALU GEMV (in-register nibble
- * unpack, v_dot2), batch >= 3 the MFMA kernel (measured crossover on MI355X).  Requires k % 128 == 0; x and qw 16-byte aligned. */
+ * m = B.  Batch 1..2 runs the bandwidth-bound VALU GEMV (in-register nibble
+ * unpack, v_dot2), batch >= 3 the MFMA kernels (measured crossover on MI355X);
+ * more than 32 rows (the prefill chunks of a mixed batch) are taken 32 at a
+ * time, each pass streaming the weights once.  Requires k % 128 == 0; x and qw
+ * 16-byte aligned. */
 logismos_status_t logismos_check_qgemm_q4g128_shape(int b, int n, int k, char* msg, size_t msg_cap);
 logismos_status_t logismos_launch_qgemm_q4g128_bf16(const void* x_bf16, const void* qw_u8,
                                                     const void* scale_f16, const void* zero_f16,
                                                     void* y_bf16, int b, int n, int k,
                                                     logismos_stream_t stream);
+/* ... `+ bias[n]` (fp32 `[N]`, NULL: none) on the fp32 sum before the one
+ * rounding to bf16 (`linear_t`'s bias, crates/kernels/src/cpu_f32/mod.rs:336-343). */
+logismos_status_t logismos_launch_qgemm_q4g128_bf16_bias(const void* x_bf16, const void* qw_u8,
+                                                         const void* scale_f16,
+                                                         const void* zero_f16,
+                                                         const void* bias_f32, void* y_bf16, int b,
+                                                         int n, int k, logismos_stream_t stream);
 
 /* The same product forced onto the MFMA kernel for any batch 1..32 (the default
  * launcher uses it from batch 3): lets a caller or a benchmark compare the two
@@ -206,16 +223,24 @@ logismos_status_t logismos_launch_qgemv_q4g32_f32(const void* x_f32, const void*
                                                   const void* scale_f16, const void* min_f16,
                                                   void* y_f32, int n, int k,
                                                   logismos_stream_t stream);
+logismos_status_t logismos_launch_qgemv_q4g32_f32_bias(const void* x_f32, const void* qw_u8,
+                                                       const void* scale_f16, const void* min_f16,
+                                                       const void* bias_f32, void* y_f32, int n,
+                                                       int k, logismos_stream_t stream);
 
 /* y[b][n] = bf16(sum_k x[b][k] * (q[n][k] * scale[n][k/32] + min[n][k/32])): `linear_t` at
  * m = batch (crates/kernels/src/cpu_f32/mod.rs:271-345) over the same Q4G32 weights, x and y
- * bf16 like those of the Q4G128 GEMM, fp32 accumulation on the matrix cores.  batch 1..32,
- * K % 128 == 0, N*K <= i32::MAX; qw and x 16-byte aligned, scale and min 8-byte aligned. */
+ * bf16 like those of the Q4G128 GEMM, fp32 accumulation on the matrix cores.  More than 32
+ * rows are taken 32 at a time.  K % 128 == 0, N*K <= i32::MAX; qw and x 16-byte aligned, scale and min 8-byte aligned. */
 logismos_status_t logismos_check_qgemm_q4g32_shape(int b, int n, int k, char* msg, size_t msg_cap);
 logismos_status_t logismos_launch_qgemm_q4g32_bf16(const void* x_bf16, const void* qw_u8,
                                                    const void* scale_f16, const void* min_f16,
                                                    void* y_bf16, int b, int n, int k,
                                                    logismos_stream_t stream);
+logismos_status_t logismos_launch_qgemm_q4g32_bf16_bias(const void* x_bf16, const void* qw_u8,
+                                                        const void* scale_f16, const void* min_f16,
+                                                        const void* bias_f32, void* y_bf16, int b,
+                                                        int n, int k, logismos_stream_t stream);
 
 /* ggml Q4_0 / Q4_1 block streams `[N][K/32]` (the tensors the loader rejects today,
  * crates/loader/src/gguf.rs:127-145,397-406) -> planar Q4G32.  blocks 2-byte aligned. */
@@ -434,6 +459,20 @@ logismos_status_t logismos_launch_rope_kv_write_f32p_turbo3(
     const void* sin_f32, const int64_t* slot_mapping, void* q_out_f16, void* k_pool_t3,
     void* v_pool_t3, int total_tokens, int num_q_heads, int num_kv_heads, int head_dim,
     int max_pos, logismos_stream_t stream);
+/* The two launchers above with the projection's bias (fp32 `[(hq+2*hkv)*128]`, NULL: none)
+ * added to the summed parts before the rotation: `linear_t`'s bias
+ * (crates/kernels/src/cpu_f32/mod.rs:336-343) of the q/k/v projections
+ * (crates/transformers/src/attention.rs:49-57). */
+logismos_status_t logismos_launch_rope_kv_write_f32p_bias(
+    const void* qkv_parts_f32, int num_parts, const void* bias_f32, const int32_t* positions,
+    const void* cos_f32, const void* sin_f32, const int64_t* slot_mapping, void* q_out_f16,
+    void* k_pool_f16, void* v_pool_f16, int total_tokens, int num_q_heads, int num_kv_heads,
+    int head_dim, int max_pos, logismos_stream_t stream);
+logismos_status_t logismos_launch_rope_kv_write_f32p_turbo3_bias(
+    const void* qkv_parts_f32, int num_parts, const void* bias_f32, const int32_t* positions,
+    const void* cos_f32, const void* sin_f32, const int64_t* slot_mapping, void* q_out_f16,
+    void* k_pool_t3, void* v_pool_t3, int total_tokens, int num_q_heads, int num_kv_heads,
+    int head_dim, int max_pos, logismos_stream_t stream);
 logismos_status_t logismos_launch_silu_mul_f32p(const void* parts_f32, int num_parts,
                                                 void* out_bf16, int rows, int inter,
                                                 logismos_stream_t stream);
@@ -563,6 +602,9 @@ typedef struct {
     logismos_q4_weight_t qkv, o, gate_up, down;
     void* k_pool_f16; /* this layer's paged pools (turbo3 pools with cfg->kv_turbo3) */
     void* v_pool_f16;
+    const void* qkv_bias_f32; /* [(hq+2*hkv)*head_dim] or NULL: the q/k/v projection's bias
+                                 (crates/transformers/src/attention.rs:49-57), added to the
+                                 projection's fp32 result before RoPE */
 } logismos_decode_layer_t;
 
 typedef struct {
@@ -583,10 +625,22 @@ typedef struct {
     const logismos_q4_weight_t* lm_head; /* [vocab][hidden] Q4G128 (host pointer) or NULL */
     void* out_tokens_u32;                /* [num_seqs], with lm_head */
     void* logits_f32;                    /* [num_seqs][vocab] or NULL */
+    /* A mixed batch (chunked prefill + decode): total_tokens = cu_seqlens[num_seqs] packed
+     * rows and the largest number of new tokens of a sequence; 0 / 0 means one new token per
+     * sequence.  Every per-row array above (hidden_f32, out_bf16, positions, slot_mapping) then
+     * has total_tokens rows, in packed order.  Rows go through the projections 32 at a time,
+     * every pass streaming the layer's weights once (`linear_t` over `seq` rows,
+     * crates/transformers/src/mlp.rs:104-111); the attention takes the whole ragged batch in
+     * one launch.  token_ids / lm_head need total_tokens <= 32. */
+    int total_tokens;
+    int max_seqlen_q;
 } logismos_decode_batch_t;
 
 size_t logismos_decode_step_workspace_bytes(const logismos_decode_config_t* cfg, int num_seqs,
                                             int num_splits);
+/* ... for a mixed batch of total_tokens packed rows */
+size_t logismos_decode_step_workspace_bytes_tokens(const logismos_decode_config_t* cfg,
+                                                   int num_seqs, int total_tokens, int num_splits);
 logismos_status_t logismos_launch_decode_step(const logismos_decode_config_t* cfg,
                                               const logismos_decode_layer_t* layers,
                                               const logismos_decode_batch_t* batch, void* workspace,

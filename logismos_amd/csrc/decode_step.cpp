@@ -9,23 +9,32 @@
 
 namespace {
 
+constexpr int kChunkRows = 32;  // rows the prepared layout and the decode GEMMs hold
+
 struct Workspace {
-    char* xn;        // prepared activations of width hidden (input of qkv / gate_up)
-    char* qkv;       // f32  [Jqkv][B][(hq+2hkv)*d]   split-K parts
-    char* q;         // f16  [B][hq*d]
-    char* attn_b;    // prepared activations of width hq*d (input of the o projection)
-    char* proj;      // f32  [max(Jo,Jdown)][B][hidden]  (o projection, then down projection)
-    char* gate_up;   // f32  [Jgu][B][2*inter]
+    char* xn;        // prepared activations of width hidden, one per 32-row chunk (input of qkv /
+                     // gate_up; a chunk's buffer carries its normed rows from the end of one
+                     // layer to the start of the next)
+    char* qkv;       // f32  [Jqkv][rows][(hq+2hkv)*d]   split-K parts of one chunk
+    char* q;         // f16  [T][hq*d]
+    char* attn_b;    // prepared activations of width hq*d of one chunk (input of the o projection)
+    char* attn_out;  // bf16 [T][hq*d]: attention output of a step that is not one chunk of
+                     // decode rows (those go straight into attn_b)
+    char* proj;      // f32  [max(Jo,Jdown)][rows][hidden]  (o projection, then down projection)
+    char* gate_up;   // f32  [Jgu][rows][2*inter]
     char* act;       // prepared activations of width inter (input of the down projection)
     char* attn_ws;   // split-K workspace of the attention
     char* head_ws;   // per-workgroup candidates of the token selection (vocab > 0)
+    size_t xn_stride;
+    int chunks, rows;  // rows: rows of a full chunk (= T when there is one chunk)
     int j_qkv, j_o, j_gu, j_down;
     size_t total;
 };
 
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
-Workspace carve(const logismos_decode_config_t& c, int b, int num_splits, char* base) {
+Workspace carve(const logismos_decode_config_t& c, int num_seqs, int t, int num_splits,
+                char* base) {
     Workspace w{};
     size_t off = 0;
     auto take = [&](size_t bytes) {
@@ -35,19 +44,34 @@ Workspace carve(const logismos_decode_config_t& c, int b, int num_splits, char* 
     };
     const size_t qd = (size_t)c.num_q_heads * c.head_dim;
     const size_t kvd = (size_t)c.num_kv_heads * c.head_dim;
-    w.j_qkv = logismos_qgemm_q4g128_splitk_xprep_parts(b, (int)(qd + 2 * kvd), c.hidden);
-    w.j_o = logismos_qgemm_q4g128_splitk_xprep_parts(b, c.hidden, (int)qd);
-    w.j_gu = logismos_qgemm_q4g128_splitk_xprep_parts(b, 2 * c.intermediate, c.hidden);
-    w.j_down = logismos_qgemm_q4g128_splitk_xprep_parts(b, c.hidden, c.intermediate);
+    w.chunks = (t + kChunkRows - 1) / kChunkRows;
+    w.rows = t < kChunkRows ? t : kChunkRows;
+    const int b = w.rows;
+    // the number of K parts depends on the batch only through its tile height (<= 16 rows or
+    // more), so a ragged last chunk of a long step may plan fewer parts than a full one: size
+    // for the larger and let every launch use its own count
+    auto parts = [&](int n, int k) {
+        int j = logismos_qgemm_q4g128_splitk_xprep_parts(b, n, k);
+        const int last = t - (w.chunks - 1) * kChunkRows;
+        const int jl = logismos_qgemm_q4g128_splitk_xprep_parts(last, n, k);
+        return j > jl ? j : jl;
+    };
+    w.j_qkv = parts((int)(qd + 2 * kvd), c.hidden);
+    w.j_o = parts(c.hidden, (int)qd);
+    w.j_gu = parts(2 * c.intermediate, c.hidden);
+    w.j_down = parts(c.hidden, c.intermediate);
     const int j_proj = w.j_o > w.j_down ? w.j_o : w.j_down;
-    w.xn = take(logismos_q4_xprep_bytes(b, c.hidden));
+    w.xn_stride = align256(logismos_q4_xprep_bytes(b, c.hidden));
+    w.xn = take(w.xn_stride * w.chunks);
     w.qkv = take((size_t)w.j_qkv * b * (qd + 2 * kvd) * 4);
-    w.q = take((size_t)b * qd * 2);
+    w.q = take((size_t)t * qd * 2);
     w.attn_b = take(logismos_q4_xprep_bytes(b, (int)qd));
+    w.attn_out = take((size_t)t * qd * 2);
     w.proj = take((size_t)j_proj * b * c.hidden * 4);
     w.gate_up = take((size_t)w.j_gu * b * 2 * c.intermediate * 4);
     w.act = take(logismos_q4_xprep_bytes(b, c.intermediate));
-    w.attn_ws = take(logismos_paged_attn_workspace_bytes(b, c.num_q_heads, c.head_dim, num_splits));
+    w.attn_ws =
+        take(logismos_paged_attn_workspace_bytes(num_seqs, c.num_q_heads, c.head_dim, num_splits));
     w.head_ws = c.vocab > 0
                     ? take(logismos_qgemm_q4g128_greedy_workspace_bytes(b, c.vocab, c.hidden))
                     : nullptr;
@@ -55,8 +79,9 @@ Workspace carve(const logismos_decode_config_t& c, int b, int num_splits, char* 
     return w;
 }
 
-bool config_ok(const logismos_decode_config_t* c, int b) {
-    if (!c || b <= 0 || b > 32) return false;
+bool config_ok(const logismos_decode_config_t* c, int num_seqs, int t, int max_seqlen_q) {
+    if (!c || num_seqs <= 0 || t < num_seqs || max_seqlen_q < 1 || max_seqlen_q > t) return false;
+    if (num_seqs > 65535 || t > 65535) return false;
     if (c->num_layers <= 0 || c->hidden <= 0 || c->intermediate <= 0 || c->max_pos <= 0)
         return false;
     if (c->head_dim != 128 || c->num_q_heads <= 0 || c->num_kv_heads <= 0) return false;
@@ -66,18 +91,45 @@ bool config_ok(const logismos_decode_config_t* c, int b) {
     if (c->block_size <= 0 || c->max_blocks_per_seq <= 0 ||
         (int64_t)c->max_pos < (int64_t)c->block_size * c->max_blocks_per_seq)
         return false;
+    if ((int64_t)t * (c->num_q_heads + 2 * c->num_kv_heads) * c->head_dim > (int64_t)INT32_MAX ||
+        (int64_t)t * c->hidden > (int64_t)INT32_MAX)
+        return false;
     if (c->vocab < 0) return false;
-    if (c->vocab > 0 && logismos_check_qgemm_q4g128_greedy_shape(b, c->vocab, c->hidden, nullptr, 0))
+    // tokens in / tokens out is a decode-step feature: one chunk
+    if (c->vocab > 0 && t <= kChunkRows &&
+        logismos_check_qgemm_q4g128_greedy_shape(t, c->vocab, c->hidden, nullptr, 0))
+        return false;
+    const int b = t < kChunkRows ? t : kChunkRows;
+    const int qd = c->num_q_heads * c->head_dim;
+    const int kvd = c->num_kv_heads * c->head_dim;
+    if (logismos_qgemm_q4g128_splitk_xprep_parts(b, qd + 2 * kvd, c->hidden) <= 0 ||
+        logismos_qgemm_q4g128_splitk_xprep_parts(b, c->hidden, qd) <= 0 ||
+        logismos_qgemm_q4g128_splitk_xprep_parts(b, 2 * c->intermediate, c->hidden) <= 0 ||
+        logismos_qgemm_q4g128_splitk_xprep_parts(b, c->hidden, c->intermediate) <= 0)
         return false;
     return true;
+}
+
+// total_tokens / max_seqlen_q of a batch: 0 means "one new token per sequence"
+int batch_tokens(const logismos_decode_batch_t* b) {
+    return b->total_tokens > 0 ? b->total_tokens : b->num_seqs;
+}
+int batch_max_q(const logismos_decode_batch_t* b) {
+    return b->max_seqlen_q > 0 ? b->max_seqlen_q : 1;
 }
 
 }  // namespace
 
 extern "C" size_t logismos_decode_step_workspace_bytes(const logismos_decode_config_t* cfg,
                                                        int num_seqs, int num_splits) {
-    if (!config_ok(cfg, num_seqs) || num_splits <= 0) return 0;
-    return carve(*cfg, num_seqs, num_splits, nullptr).total;
+    return logismos_decode_step_workspace_bytes_tokens(cfg, num_seqs, num_seqs, num_splits);
+}
+
+extern "C" size_t logismos_decode_step_workspace_bytes_tokens(const logismos_decode_config_t* cfg,
+                                                              int num_seqs, int total_tokens,
+                                                              int num_splits) {
+    if (!config_ok(cfg, num_seqs, total_tokens, 1) || num_splits <= 0) return 0;
+    return carve(*cfg, num_seqs, total_tokens, num_splits, nullptr).total;
 }
 
 #define LG_TRY(call)                                  \
@@ -92,8 +144,10 @@ extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_c
                                                          void* workspace,
                                                          logismos_stream_t stream) {
     if (!cfg || !layers || !batch || !workspace) return hipErrorInvalidValue;
-    const int b = batch->num_seqs;
-    if (!config_ok(cfg, b) || batch->num_splits <= 0) return hipErrorInvalidValue;
+    const int num_seqs = batch->num_seqs;
+    const int t = batch_tokens(batch);
+    const int max_q = batch_max_q(batch);
+    if (!config_ok(cfg, num_seqs, t, max_q) || batch->num_splits <= 0) return hipErrorInvalidValue;
     if (reinterpret_cast<uintptr_t>(workspace) & 255u) return hipErrorInvalidValue;
     const logismos_decode_config_t& c = *cfg;
     const bool tokens_in = batch->token_ids != nullptr;
@@ -102,64 +156,115 @@ extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_c
     if (tokens_in && !batch->embed_table_bf16) return hipErrorInvalidValue;
     if (tokens_out && !batch->out_tokens_u32) return hipErrorInvalidValue;
     if (!tokens_out && !batch->out_bf16) return hipErrorInvalidValue;
-    const Workspace w = carve(c, b, batch->num_splits, static_cast<char*>(workspace));
+    // the vocabulary projection with its token choice takes one chunk of rows
+    if (tokens_out && t > kChunkRows) return hipErrorInvalidValue;
+    const Workspace w = carve(c, num_seqs, t, batch->num_splits, static_cast<char*>(workspace));
     const int qd = c.num_q_heads * c.head_dim;
     const int kvd = c.num_kv_heads * c.head_dim;
+    const int width = qd + 2 * kvd;
     const float scale = 1.0f / sqrtf((float)c.head_dim);
+    const bool one_chunk = w.chunks == 1;
+    const bool direct = one_chunk && max_q == 1;  // attention writes the o projection's input
+    float* const h = static_cast<float*>(batch->hidden_f32);
+    auto rows_of = [&](int ch) {
+        const int r0 = ch * kChunkRows;
+        return t - r0 < kChunkRows ? t - r0 : kChunkRows;
+    };
 
     if (tokens_in)
         LG_TRY(logismos_launch_embed_lookup_bf16(batch->embed_table_bf16, batch->token_ids,
-                                                 batch->hidden_f32, b, c.hidden, c.vocab, stream));
-    int res_parts = 0;  // split-K parts of the projection the next add_rms_norm folds into h
+                                                 batch->hidden_f32, t, c.hidden, c.vocab, stream));
+    // The normed input of a layer's first half is produced where the residual stream is
+    // completed: before layer 0 here, afterwards by the add + norm that folds a chunk's down
+    // projection into h (with the NEXT layer's gains).
+    for (int ch = 0; ch < w.chunks; ++ch)
+        LG_TRY(logismos_launch_add_rms_norm_f32p_xprep(
+            h + (int64_t)ch * kChunkRows * c.hidden, nullptr, 0, layers[0].norm1_w_f32,
+            w.xn + ch * w.xn_stride, rows_of(ch), c.hidden, c.rms_eps, stream));
+    int res_parts = 0;  // split-K parts of the last down projection not yet folded into h
     for (int l = 0; l < c.num_layers; ++l) {
         const logismos_decode_layer_t& L = layers[l];
-        LG_TRY(logismos_launch_add_rms_norm_f32p_xprep(batch->hidden_f32, w.proj, res_parts,
-                                                       L.norm1_w_f32, w.xn, b, c.hidden, c.rms_eps,
-                                                       stream));
-        LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk_xprep(
-            w.xn, L.qkv.qw, L.qkv.scale, L.qkv.zero, w.qkv, b, qd + 2 * kvd, c.hidden, stream));
-        const auto rope_kv_write = c.kv_turbo3 ? logismos_launch_rope_kv_write_f32p_turbo3
-                                               : logismos_launch_rope_kv_write_f32p;
-        LG_TRY(rope_kv_write(w.qkv, w.j_qkv, batch->positions, batch->rope_cos_f32,
-                             batch->rope_sin_f32, batch->slot_mapping, w.q, L.k_pool_f16,
-                             L.v_pool_f16, b, c.num_q_heads, c.num_kv_heads, c.head_dim, c.max_pos,
-                             stream));
-        // attention writes the prepared layout directly: its output only feeds the o projection
+        const bool last_layer = l + 1 == c.num_layers;
+        // ---- first half, chunk by chunk: q/k/v projection, RoPE, K/V rows into the pools
+        for (int ch = 0; ch < w.chunks; ++ch) {
+            const int r0 = ch * kChunkRows, rows = rows_of(ch);
+            LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk_xprep(
+                w.xn + ch * w.xn_stride, L.qkv.qw, L.qkv.scale, L.qkv.zero, w.qkv, rows, width,
+                c.hidden, stream));
+            const int j = logismos_qgemm_q4g128_splitk_xprep_parts(rows, width, c.hidden);
+            const auto rope_kv_write = c.kv_turbo3 ? logismos_launch_rope_kv_write_f32p_turbo3_bias
+                                                   : logismos_launch_rope_kv_write_f32p_bias;
+            LG_TRY(rope_kv_write(w.qkv, j, L.qkv_bias_f32, batch->positions + r0,
+                                 batch->rope_cos_f32, batch->rope_sin_f32,
+                                 batch->slot_mapping + r0, w.q + (size_t)r0 * qd * 2, L.k_pool_f16,
+                                 L.v_pool_f16, rows, c.num_q_heads, c.num_kv_heads, c.head_dim,
+                                 c.max_pos, stream));
+        }
+        // ---- attention over the whole ragged batch.  One chunk of decode rows: the result
+        // goes straight into the prepared layout of the o projection; otherwise bf16 rows that
+        // each chunk prepares for itself.
         LG_TRY(lg::paged_attn_launch(
             w.q, L.k_pool_f16, L.v_pool_f16, batch->block_tables, batch->cu_seqlens,
-            batch->context_lens, w.attn_b, w.attn_ws, b, b, 1, c.num_q_heads, c.num_kv_heads,
-            c.head_dim, c.block_size, c.max_blocks_per_seq, batch->num_splits, scale, 1,
-            LOGISMOS_ATTN_PHASE_ALL, 2, c.kv_turbo3 ? 1 : 0, stream));
-        LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk_xprep(w.attn_b, L.o.qw, L.o.scale, L.o.zero,
-                                                             w.proj, b, c.hidden, qd, stream));
-        LG_TRY(logismos_launch_add_rms_norm_f32p_xprep(batch->hidden_f32, w.proj, w.j_o,
-                                                       L.norm2_w_f32, w.xn, b, c.hidden, c.rms_eps,
-                                                       stream));
-        LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk_xprep(w.xn, L.gate_up.qw, L.gate_up.scale,
-                                                             L.gate_up.zero, w.gate_up, b,
-                                                             2 * c.intermediate, c.hidden, stream));
-        LG_TRY(logismos_launch_silu_mul_f32p_xprep(w.gate_up, w.j_gu, w.act, b, c.intermediate,
-                                                   stream));
-        LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk_xprep(w.act, L.down.qw, L.down.scale,
-                                                             L.down.zero, w.proj, b, c.hidden,
-                                                             c.intermediate, stream));
-        res_parts = w.j_down;
+            batch->context_lens, direct ? w.attn_b : w.attn_out,
+            w.attn_ws, num_seqs, t, max_q, c.num_q_heads, c.num_kv_heads, c.head_dim, c.block_size,
+            c.max_blocks_per_seq, batch->num_splits, scale, 1, LOGISMOS_ATTN_PHASE_ALL,
+            direct ? 2 : 1, c.kv_turbo3 ? 1 : 0, stream));
+        // ---- second half, chunk by chunk
+        for (int ch = 0; ch < w.chunks; ++ch) {
+            const int r0 = ch * kChunkRows, rows = rows_of(ch);
+            float* hc = h + (int64_t)r0 * c.hidden;
+            if (!direct)
+                LG_TRY(logismos_launch_q4_prepare_x_bf16(w.attn_out + (size_t)r0 * qd * 2, w.attn_b,
+                                                         rows, qd, stream));
+            LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk_xprep(
+                w.attn_b, L.o.qw, L.o.scale, L.o.zero, w.proj, rows, c.hidden, qd, stream));
+            LG_TRY(logismos_launch_add_rms_norm_f32p_xprep(
+                hc, w.proj, logismos_qgemm_q4g128_splitk_xprep_parts(rows, c.hidden, qd),
+                L.norm2_w_f32, w.xn + ch * w.xn_stride, rows, c.hidden, c.rms_eps, stream));
+            LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk_xprep(
+                w.xn + ch * w.xn_stride, L.gate_up.qw, L.gate_up.scale, L.gate_up.zero, w.gate_up,
+                rows, 2 * c.intermediate, c.hidden, stream));
+            LG_TRY(logismos_launch_silu_mul_f32p_xprep(
+                w.gate_up,
+                logismos_qgemm_q4g128_splitk_xprep_parts(rows, 2 * c.intermediate, c.hidden), w.act,
+                rows, c.intermediate, stream));
+            LG_TRY(logismos_launch_qgemm_q4g128_f32_splitk_xprep(
+                w.act, L.down.qw, L.down.scale, L.down.zero, w.proj, rows, c.hidden, c.intermediate,
+                stream));
+            const int j_down =
+                logismos_qgemm_q4g128_splitk_xprep_parts(rows, c.hidden, c.intermediate);
+            if (!last_layer) {
+                // fold the down projection into h and norm for the next layer's first half
+                LG_TRY(logismos_launch_add_rms_norm_f32p_xprep(
+                    hc, w.proj, j_down, layers[l + 1].norm1_w_f32, w.xn + ch * w.xn_stride, rows,
+                    c.hidden, c.rms_eps, stream));
+            } else if (!one_chunk) {
+                // last layer of a multi-chunk step: the final norm of this chunk's rows
+                LG_TRY(logismos_launch_add_rms_norm_f32p(
+                    hc, w.proj, j_down, batch->final_norm_w_f32,
+                    static_cast<char*>(batch->out_bf16) + (size_t)r0 * c.hidden * 2, rows, c.hidden,
+                    c.rms_eps, stream));
+            } else {
+                res_parts = j_down;
+            }
+        }
     }
+    if (!one_chunk) return 0;
     if (tokens_out) {
         // the normed state in the layout of the vocabulary projection, then the projection
         // with the token choice fused into it
         LG_TRY(logismos_launch_add_rms_norm_f32p_xprep(batch->hidden_f32, w.proj, res_parts,
-                                                       batch->final_norm_w_f32, w.xn, b, c.hidden,
+                                                       batch->final_norm_w_f32, w.xn, t, c.hidden,
                                                        c.rms_eps, stream));
         res_parts = 0;  // folded into h by the call above
         const logismos_q4_weight_t& H = *batch->lm_head;
         LG_TRY(logismos_launch_qgemm_q4g128_greedy_xprep(w.xn, H.qw, H.scale, H.zero,
                                                          batch->out_tokens_u32, batch->logits_f32,
-                                                         w.head_ws, b, c.vocab, c.hidden, stream));
+                                                         w.head_ws, t, c.vocab, c.hidden, stream));
     }
     if (batch->out_bf16)
         LG_TRY(logismos_launch_add_rms_norm_f32p(batch->hidden_f32, w.proj, res_parts,
-                                                 batch->final_norm_w_f32, batch->out_bf16, b,
+                                                 batch->final_norm_w_f32, batch->out_bf16, t,
                                                  c.hidden, c.rms_eps, stream));
     return 0;
 }

@@ -52,8 +52,9 @@ RegxPlan regx_plan(int b, int n, int k);
 // ... and for x as a plain bf16 [b][K] matrix with the bf16 product as output (one part)
 RegxPlan regx_plain_plan(int b, int n, int k);
 hipError_t qgemm_q4_regx_plain_launch(const RegxPlan& plan, const void* x_bf16, const void* qw,
-                                      const void* scale, const void* zero, void* y_bf16, int b,
-                                      int n, int k, hipStream_t stream);
+                                      const void* scale, const void* zero, void* y_bf16,
+                                      const float* bias, int b, int n, int k,
+                                      hipStream_t stream);
 hipError_t qgemm_q4_regx_launch(const RegxPlan& plan, const void* xprep, const void* qw,
                                 const void* scale, const void* zero, void* part, int b, int n,
                                 int k, hipStream_t stream);

@@ -38,7 +38,8 @@ __global__ __launch_bounds__(256) void qgemv_q4g128_kernel(const uint16_t* __res
                                                            const uint8_t* __restrict__ qw,
                                                            const __half* __restrict__ scale,
                                                            const __half* __restrict__ zero,
-                                                           uint16_t* __restrict__ y, int n, int k) {
+                                                           uint16_t* __restrict__ y,
+                                                           const float* __restrict__ bias, int n, int k) {
     extern __shared__ uint4_t lds[];
     const int nchunks = k >> 5;  // 32 elements = 16 bytes of nibbles
     const int groups = k >> 7;
@@ -149,13 +150,15 @@ __global__ __launch_bounds__(256) void qgemv_q4g128_kernel(const uint16_t* __res
 #pragma unroll
         for (int b = 0; b < B; ++b) {
             const float total = wave_sum(acc[r][b]);
-            if (lane == 0 && row0 + r < n) y[(int64_t)b * n + row0 + r] = f32_to_bf16_rne(total);
+            if (lane == 0 && row0 + r < n)
+                y[(int64_t)b * n + row0 + r] =
+                    f32_to_bf16_rne(bias ? total + bias[row0 + r] : total);
         }
 }
 
 template <int B, int R>
 static hipError_t launch_gemv(const void* x, const void* qw, const void* scale, const void* zero,
-                              void* y, int n, int k, hipStream_t stream) {
+                              void* y, const float* bias, int n, int k, hipStream_t stream) {
     const int nchunks = k / 32;
     const size_t lds = (size_t)B * nchunks * (4 * 16 + 4);
     auto kern = qgemv_q4g128_kernel<B, R>;
@@ -170,17 +173,17 @@ static hipError_t launch_gemv(const void* x, const void* qw, const void* scale, 
                                        static_cast<const uint8_t*>(qw),
                                        static_cast<const __half*>(scale),
                                        static_cast<const __half*>(zero),
-                                       static_cast<uint16_t*>(y), n, k);
+                                       static_cast<uint16_t*>(y), bias, n, k);
     return hipGetLastError();
 }
 
 template <int B>
 static hipError_t launch_gemv_b(const void* x, const void* qw, const void* scale, const void* zero,
-                                void* y, int n, int k, hipStream_t stream) {
+                                void* y, const float* bias, int n, int k, hipStream_t stream) {
     // rows per wave: enough waves to cover the chip several times over
-    if (n >= 8192) return launch_gemv<B, 4>(x, qw, scale, zero, y, n, k, stream);
-    if (n >= 4096) return launch_gemv<B, 2>(x, qw, scale, zero, y, n, k, stream);
-    return launch_gemv<B, 1>(x, qw, scale, zero, y, n, k, stream);
+    if (n >= 8192) return launch_gemv<B, 4>(x, qw, scale, zero, y, bias, n, k, stream);
+    if (n >= 4096) return launch_gemv<B, 2>(x, qw, scale, zero, y, bias, n, k, stream);
+    return launch_gemv<B, 1>(x, qw, scale, zero, y, bias, n, k, stream);
 }
 
 
@@ -210,7 +213,7 @@ template <int BT, int GW, int T>
 __global__ __launch_bounds__(1024) void qgemm_q4g128_mfma_kernel(
     const uint16_t* __restrict__ x, const uint8_t* __restrict__ qw,
     const __half* __restrict__ scale, const __half* __restrict__ zero, uint16_t* __restrict__ y,
-    int b, int n, int k) {
+    const float* __restrict__ bias, int b, int n, int k) {
     extern __shared__ uint4_t lds[];
     constexpr int BP = BT * 16;
     const int groups = k >> 7;
@@ -364,7 +367,8 @@ __global__ __launch_bounds__(1024) void qgemm_q4g128_mfma_kernel(
         const int r = ti * 16 + c;
         float sum = 0.0f;
         for (int w = 0; w < nwaves; ++w) sum += yl[(size_t)w * T * BP * 16 + i];
-        if (r < rows_here && bi < b) y[(int64_t)bi * n + row0 + r] = f32_to_bf16_rne(sum);
+        if (r < rows_here && bi < b)
+            y[(int64_t)bi * n + row0 + r] = f32_to_bf16_rne(bias ? sum + bias[row0 + r] : sum);
     }
 }
 
@@ -387,7 +391,8 @@ static size_t mfma_lds_bytes(int b, int n, int k) {
 
 template <int BT, int GW, int T>
 static hipError_t launch_mfma_t(const void* x, const void* qw, const void* scale, const void* zero,
-                                void* y, int b, int n, int k, hipStream_t stream) {
+                                void* y, const float* bias, int b, int n, int k,
+                                hipStream_t stream) {
     const int groups = k / 128;
     const int tiles = (n + 15) / 16;
     int waves = (groups + GW - 1) / GW;
@@ -405,19 +410,20 @@ static hipError_t launch_mfma_t(const void* x, const void* qw, const void* scale
     kern<<<dim3((tiles + T - 1) / T), dim3(64 * waves), lds, stream>>>(
         static_cast<const uint16_t*>(x), static_cast<const uint8_t*>(qw),
         static_cast<const __half*>(scale), static_cast<const __half*>(zero),
-        static_cast<uint16_t*>(y), b, n, k);
+        static_cast<uint16_t*>(y), bias, b, n, k);
     return hipGetLastError();
 }
 
 template <int BT, int GW>
 static hipError_t launch_mfma(const void* x, const void* qw, const void* scale, const void* zero,
-                              void* y, int b, int n, int k, hipStream_t stream) {
+                              void* y, const float* bias, int b, int n, int k,
+                              hipStream_t stream) {
     const int tiles = (n + 15) / 16;
     const int cus = device_cu_count();
     const int t = (tiles + cus - 1) / cus;  // row tiles per workgroup (LDS slots cap it at 3)
-    if (t >= 3) return launch_mfma_t<BT, GW, 3>(x, qw, scale, zero, y, b, n, k, stream);
-    if (t == 2) return launch_mfma_t<BT, GW, 2>(x, qw, scale, zero, y, b, n, k, stream);
-    return launch_mfma_t<BT, GW, 1>(x, qw, scale, zero, y, b, n, k, stream);
+    if (t >= 3) return launch_mfma_t<BT, GW, 3>(x, qw, scale, zero, y, bias, b, n, k, stream);
+    if (t == 2) return launch_mfma_t<BT, GW, 2>(x, qw, scale, zero, y, bias, b, n, k, stream);
+    return launch_mfma_t<BT, GW, 1>(x, qw, scale, zero, y, bias, b, n, k, stream);
 }
 
 }  // namespace lg
@@ -430,60 +436,89 @@ extern "C" logismos_status_t logismos_check_qgemm_q4g128_shape(int b, int n, int
     if (k <= 0) return lg::reject(msg, msg_cap, "%s: K must be positive, got %d", kn, k);
     if (k % 128 != 0)
         return lg::reject(msg, msg_cap, "%s: K = %d is not a multiple of the group size 128", kn, k);
-    if (b > 32)
-        return lg::reject(msg, msg_cap, "%s: batch %d exceeds the supported maximum of 32", kn, b);
     if ((int64_t)n * k > (int64_t)INT32_MAX)
         return lg::reject(msg, msg_cap, "%s: N*K = %lld exceeds i32::MAX", kn,
                           (long long)((int64_t)n * k));
     if ((int64_t)b * n > (int64_t)INT32_MAX || (int64_t)b * k > (int64_t)INT32_MAX)
         return lg::reject(msg, msg_cap, "%s: batch*N or batch*K exceeds i32::MAX", kn);
+    // (rows beyond 32 are taken 32 at a time: the per-launch bounds below use min(b, 32))
     if (b <= 4 && (size_t)b * (k / 32) * 68 > lg::kMaxLds)
         return lg::reject(msg, msg_cap, "%s: batch*K = %lld does not fit the LDS staging of x", kn,
                           (long long)((int64_t)b * k));
     // the matrix-core path (batch >= 3; ..._bf16_mfma refuses such a shape at any batch) stages a
     // workgroup's scales and zeros for all of K next to its partial sums
-    if (b >= 3 && lg::mfma_lds_bytes(b, n, k) > lg::kMaxLds)
+    if (b >= 3 && lg::mfma_lds_bytes(b < 32 ? b : 32, n, k) > lg::kMaxLds)
         return lg::reject(msg, msg_cap,
                           "%s: K = %d needs %zu bytes of LDS on the matrix-core path (limit %zu)",
-                          kn, k, lg::mfma_lds_bytes(b, n, k), lg::kMaxLds);
+                          kn, k, lg::mfma_lds_bytes(b < 32 ? b : 32, n, k), lg::kMaxLds);
     return 0;
 }
 
+// One launch for up to 32 activation rows.
+static logismos_status_t qgemm_q4_dispatch32(const void* x_bf16, const void* qw_u8,
+                                             const void* scale_f16, const void* zero_f16,
+                                             const float* bias, void* y_bf16, int b, int n, int k,
+                                             bool force_mfma, hipStream_t st) {
+    if (!force_mfma) {
+        switch (b) {
+            case 1:
+                return lg::launch_gemv_b<1>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, bias, n, k, st);
+            case 2:
+                if (lg::regx_plain_plan(b, n, k).parts == 1) break;  // large matrices, see there
+                return lg::launch_gemv_b<2>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, bias, n, k, st);
+            default: break;  // batch 3 and 4: the MFMA kernels are faster (measured crossover)
+        }
+        // K = 2048 / 4096: x in registers, weights through the LDS ring, one workgroup per K
+        if (const lg::RegxPlan rp = lg::regx_plain_plan(b, n, k); rp.parts == 1)
+            return lg::qgemm_q4_regx_plain_launch(rp, x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, bias,
+                                                  b, n, k, st);
+    }
+    if (b <= 16)
+        return lg::launch_mfma<1, 2>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, bias, b, n, k, st);
+    return lg::launch_mfma<2, 1>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, bias, b, n, k, st);
+}
+
+// `linear_t` takes any m (crates/kernels/src/cpu_f32/mod.rs:271-345).  The kernels hold at
+// most 32 activation rows per workgroup, so a taller x is taken 32 rows at a time: every
+// launch streams the weights once (the prefill chunks of a mixed batch pass through the
+// quantized projections this way).
 static logismos_status_t qgemm_q4_dispatch(const void* x_bf16, const void* qw_u8,
                                            const void* scale_f16, const void* zero_f16,
-                                           void* y_bf16, int b, int n, int k, bool force_mfma,
-                                           logismos_stream_t stream) {
+                                           const void* bias_f32, void* y_bf16, int b, int n, int k,
+                                           bool force_mfma, logismos_stream_t stream) {
     if (logismos_check_qgemm_q4g128_shape(b, n, k, nullptr, 0) != 0) return hipErrorInvalidValue;
     if (!x_bf16 || !qw_u8 || !scale_f16 || !zero_f16 || !y_bf16) return hipErrorInvalidValue;
     if ((reinterpret_cast<uintptr_t>(qw_u8) & 15u) || (reinterpret_cast<uintptr_t>(x_bf16) & 15u))
         return hipErrorInvalidValue;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (!force_mfma) {
-        switch (b) {
-            case 1: return lg::launch_gemv_b<1>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, n, k, st);
-            case 2:
-                if (lg::regx_plain_plan(b, n, k).parts == 1) break;  // large matrices, see there
-                return lg::launch_gemv_b<2>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, n, k, st);
-            default: break;  // batch 3 and 4: the MFMA kernels are faster (measured crossover)
-        }
-        // K = 2048 / 4096: x in registers, weights through the LDS ring, one workgroup per K
-        if (const lg::RegxPlan rp = lg::regx_plain_plan(b, n, k); rp.parts == 1)
-            return lg::qgemm_q4_regx_plain_launch(rp, x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, b, n,
-                                                  k, st);
+    const float* bias = static_cast<const float*>(bias_f32);
+    for (int m0 = 0; m0 < b; m0 += 32) {
+        const int rows = b - m0 < 32 ? b - m0 : 32;
+        const logismos_status_t e = qgemm_q4_dispatch32(
+            static_cast<const uint16_t*>(x_bf16) + (int64_t)m0 * k, qw_u8, scale_f16, zero_f16, bias,
+            static_cast<uint16_t*>(y_bf16) + (int64_t)m0 * n, rows, n, k, force_mfma, st);
+        if (e != 0) return e;
     }
-    if (b <= 16)
-        return lg::launch_mfma<1, 2>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, b, n, k, st);
-    return lg::launch_mfma<2, 1>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, b, n, k, st);
+    return 0;
 }
 
 extern "C" logismos_status_t logismos_launch_qgemm_q4g128_bf16(
     const void* x_bf16, const void* qw_u8, const void* scale_f16, const void* zero_f16,
     void* y_bf16, int b, int n, int k, logismos_stream_t stream) {
-    return qgemm_q4_dispatch(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, b, n, k, false, stream);
+    return qgemm_q4_dispatch(x_bf16, qw_u8, scale_f16, zero_f16, nullptr, y_bf16, b, n, k, false,
+                             stream);
+}
+
+extern "C" logismos_status_t logismos_launch_qgemm_q4g128_bf16_bias(
+    const void* x_bf16, const void* qw_u8, const void* scale_f16, const void* zero_f16,
+    const void* bias_f32, void* y_bf16, int b, int n, int k, logismos_stream_t stream) {
+    return qgemm_q4_dispatch(x_bf16, qw_u8, scale_f16, zero_f16, bias_f32, y_bf16, b, n, k, false,
+                             stream);
 }
 
 extern "C" logismos_status_t logismos_launch_qgemm_q4g128_bf16_mfma(
     const void* x_bf16, const void* qw_u8, const void* scale_f16, const void* zero_f16,
     void* y_bf16, int b, int n, int k, logismos_stream_t stream) {
-    return qgemm_q4_dispatch(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, b, n, k, true, stream);
+    return qgemm_q4_dispatch(x_bf16, qw_u8, scale_f16, zero_f16, nullptr, y_bf16, b, n, k, true,
+                             stream);
 }

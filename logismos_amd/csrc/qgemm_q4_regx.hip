@@ -71,7 +71,7 @@ template <int BT, int GS, bool PLAIN>
 __global__ __launch_bounds__(64 * kRegxWaves) void qgemm_q4g128_regx_kernel(
     const uint4_t* __restrict__ xprep, const uint8_t* __restrict__ qw,
     const __half* __restrict__ scale, const __half* __restrict__ zero, float* __restrict__ part,
-    int b, int n, int k, int tiles_per_worker, int ring) {
+    int b, int n, int k, int tiles_per_worker, int ring, const float* __restrict__ bias) {
     static_assert(GS == 2 || GS == 4, "slices of 2 or 4 groups");
     constexpr int BP = BT * 16;
     constexpr int W = kRegxWaves;
@@ -371,7 +371,7 @@ __global__ __launch_bounds__(64 * kRegxWaves) void qgemm_q4g128_regx_kernel(
                     if (row < n && bi < b) {
                         if constexpr (PLAIN)
                             reinterpret_cast<unsigned short*>(part)[(unsigned)bi * (unsigned)n + (unsigned)row] =
-                                f32_to_bf16_rne(sum);
+                                f32_to_bf16_rne(bias ? sum + bias[row] : sum);
                         else
                             pbase[(unsigned)bi * (unsigned)n + (unsigned)row] = sum;
                     }
@@ -400,7 +400,7 @@ template <int GS, bool PLAIN>
 __global__ __launch_bounds__(64 * kRegxWaves) void qgemm_q4g128_regx32_kernel(
     const uint4_t* __restrict__ xprep, const uint8_t* __restrict__ qw,
     const __half* __restrict__ scale, const __half* __restrict__ zero, float* __restrict__ part,
-    int b, int n, int k, int tiles_per_worker, int ring) {
+    int b, int n, int k, int tiles_per_worker, int ring, const float* __restrict__ bias) {
     static_assert(GS == 2 || GS == 4, "slices of 2 or 4 groups");
     constexpr int BP = 32;
     constexpr int W = kRegxWaves;
@@ -673,9 +673,12 @@ __global__ __launch_bounds__(64 * kRegxWaves) void qgemm_q4g128_regx32_kernel(
                 if (row < n) {
                     if constexpr (PLAIN) {
                         unsigned short* y = reinterpret_cast<unsigned short*>(part);
-                        if (m0 < b) y[(unsigned)m0 * (unsigned)n + (unsigned)row] = f32_to_bf16_rne(sum[0]);
+                        const float bv = bias ? bias[row] : 0.0f;
+                        if (m0 < b)
+                            y[(unsigned)m0 * (unsigned)n + (unsigned)row] = f32_to_bf16_rne(sum[0] + bv);
                         if (m0 + 1 < b)
-                            y[(unsigned)(m0 + 1) * (unsigned)n + (unsigned)row] = f32_to_bf16_rne(sum[1]);
+                            y[(unsigned)(m0 + 1) * (unsigned)n + (unsigned)row] =
+                                f32_to_bf16_rne(sum[1] + bv);
                     } else {
                         if (m0 < b) pbase[(unsigned)m0 * (unsigned)n + (unsigned)row] = sum[0];
                         if (m0 + 1 < b) pbase[(unsigned)(m0 + 1) * (unsigned)n + (unsigned)row] = sum[1];
@@ -690,8 +693,8 @@ __global__ __launch_bounds__(64 * kRegxWaves) void qgemm_q4g128_regx32_kernel(
 
 template <int GS, bool PLAIN>
 static hipError_t launch_regx32(const void* xprep, const void* qw, const void* scale,
-                                const void* zero, void* part, int b, int n, int k, int tpw,
-                                int ring, hipStream_t stream) {
+                                const void* zero, void* part, const float* bias, int b, int n, int k,
+                                int tpw, int ring, hipStream_t stream) {
     const int tiles = (n + 31) / 32;
     const size_t lds = (size_t)regx32_lds_bytes(GS, ring);
     auto kern = qgemm_q4g128_regx32_kernel<GS, PLAIN>;
@@ -703,30 +706,31 @@ static hipError_t launch_regx32(const void* xprep, const void* qw, const void* s
     kern<<<grid, dim3(64 * kRegxWaves), lds, stream>>>(
         static_cast<const uint4_t*>(xprep), static_cast<const uint8_t*>(qw),
         static_cast<const __half*>(scale), static_cast<const __half*>(zero),
-        static_cast<float*>(part), b, n, k, tpw, ring);
+        static_cast<float*>(part), b, n, k, tpw, ring, bias);
     return hipGetLastError();
 }
 
 static hipError_t qgemm_q4_regx32_launch(const void* xprep, const void* qw, const void* scale,
-                                         const void* zero, void* part, int b, int n, int k, int gs,
-                                         int tpw, int ring, bool plain, hipStream_t stream) {
+                                         const void* zero, void* part, const float* bias, int b, int n,
+                                         int k, int gs, int tpw, int ring, bool plain,
+                                         hipStream_t stream) {
     if (gs != 2 && gs != 4) return hipErrorInvalidValue;
     if (b <= 16 || b > 32) return hipErrorInvalidValue;
     if ((k / 128) % (kRegxWaves * gs) != 0 || tpw < 1 || ring < 1 || ring > kRegxMaxRing)
         return hipErrorInvalidValue;
     if (regx32_lds_bytes(gs, ring) > 160 * 1024) return hipErrorInvalidValue;
     if (plain) {
-        if (gs == 2) return launch_regx32<2, true>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
-        return launch_regx32<4, true>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
+        if (gs == 2) return launch_regx32<2, true>(xprep, qw, scale, zero, part, bias, b, n, k, tpw, ring, stream);
+        return launch_regx32<4, true>(xprep, qw, scale, zero, part, bias, b, n, k, tpw, ring, stream);
     }
-    if (gs == 2) return launch_regx32<2, false>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
-    return launch_regx32<4, false>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
+    if (gs == 2) return launch_regx32<2, false>(xprep, qw, scale, zero, part, bias, b, n, k, tpw, ring, stream);
+    return launch_regx32<4, false>(xprep, qw, scale, zero, part, bias, b, n, k, tpw, ring, stream);
 }
 
 template <int BT, int GS, bool PLAIN>
 static hipError_t launch_regx(const void* xprep, const void* qw, const void* scale,
-                              const void* zero, void* part, int b, int n, int k, int tpw, int ring,
-                              hipStream_t stream) {
+                              const void* zero, void* part, const float* bias, int b, int n, int k,
+                              int tpw, int ring, hipStream_t stream) {
     const int tiles = (n + 15) / 16;
     const size_t lds = (size_t)regx_lds_bytes(BT, GS, ring);
     auto kern = qgemm_q4g128_regx_kernel<BT, GS, PLAIN>;
@@ -738,24 +742,25 @@ static hipError_t launch_regx(const void* xprep, const void* qw, const void* sca
     kern<<<grid, dim3(64 * kRegxWaves), lds, stream>>>(
         static_cast<const uint4_t*>(xprep), static_cast<const uint8_t*>(qw),
         static_cast<const __half*>(scale), static_cast<const __half*>(zero),
-        static_cast<float*>(part), b, n, k, tpw, ring);
+        static_cast<float*>(part), b, n, k, tpw, ring, bias);
     return hipGetLastError();
 }
 
 static hipError_t qgemm_q4_regx16_launch(const void* xprep, const void* qw, const void* scale,
-                                         const void* zero, void* part, int b, int n, int k, int gs,
-                                         int tpw, int ring, bool plain, hipStream_t stream) {
+                                         const void* zero, void* part, const float* bias, int b, int n,
+                                         int k, int gs, int tpw, int ring, bool plain,
+                                         hipStream_t stream) {
     if (gs != 2 && gs != 4) return hipErrorInvalidValue;
     if (b < 1 || b > 16) return hipErrorInvalidValue;
     if ((k / 128) % (kRegxWaves * gs) != 0 || tpw < 1 || ring < 1 || ring > kRegxMaxRing)
         return hipErrorInvalidValue;
     if (regx_lds_bytes(1, gs, ring) > 160 * 1024) return hipErrorInvalidValue;
     if (plain) {
-        if (gs == 2) return launch_regx<1, 2, true>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
-        return launch_regx<1, 4, true>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
+        if (gs == 2) return launch_regx<1, 2, true>(xprep, qw, scale, zero, part, bias, b, n, k, tpw, ring, stream);
+        return launch_regx<1, 4, true>(xprep, qw, scale, zero, part, bias, b, n, k, tpw, ring, stream);
     }
-    if (gs == 2) return launch_regx<1, 2, false>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
-    return launch_regx<1, 4, false>(xprep, qw, scale, zero, part, b, n, k, tpw, ring, stream);
+    if (gs == 2) return launch_regx<1, 2, false>(xprep, qw, scale, zero, part, bias, b, n, k, tpw, ring, stream);
+    return launch_regx<1, 4, false>(xprep, qw, scale, zero, part, bias, b, n, k, tpw, ring, stream);
 }
 
 // Shapes the kernels above take, and how: K a multiple of 2048 (slices of two groups, two
@@ -806,21 +811,22 @@ hipError_t qgemm_q4_regx_launch(const RegxPlan& p, const void* xprep, const void
                                 const void* scale, const void* zero, void* part, int b, int n,
                                 int k, hipStream_t stream) {
     if (p.rows == 32)
-        return qgemm_q4_regx32_launch(xprep, qw, scale, zero, part, b, n, k, p.gs, p.tpw, p.ring,
-                                      false, stream);
-    return qgemm_q4_regx16_launch(xprep, qw, scale, zero, part, b, n, k, p.gs, p.tpw, p.ring, false,
-                                  stream);
+        return qgemm_q4_regx32_launch(xprep, qw, scale, zero, part, nullptr, b, n, k, p.gs, p.tpw,
+                                      p.ring, false, stream);
+    return qgemm_q4_regx16_launch(xprep, qw, scale, zero, part, nullptr, b, n, k, p.gs, p.tpw, p.ring,
+                                  false, stream);
 }
 
 hipError_t qgemm_q4_regx_plain_launch(const RegxPlan& p, const void* x_bf16, const void* qw,
-                                      const void* scale, const void* zero, void* y_bf16, int b,
-                                      int n, int k, hipStream_t stream) {
+                                      const void* scale, const void* zero, void* y_bf16,
+                                      const float* bias, int b, int n, int k,
+                                      hipStream_t stream) {
     if (p.parts != 1) return hipErrorInvalidValue;
     if (p.rows == 32)
-        return qgemm_q4_regx32_launch(x_bf16, qw, scale, zero, y_bf16, b, n, k, p.gs, p.tpw, p.ring,
-                                      true, stream);
-    return qgemm_q4_regx16_launch(x_bf16, qw, scale, zero, y_bf16, b, n, k, p.gs, p.tpw, p.ring, true,
-                                  stream);
+        return qgemm_q4_regx32_launch(x_bf16, qw, scale, zero, y_bf16, bias, b, n, k, p.gs, p.tpw,
+                                      p.ring, true, stream);
+    return qgemm_q4_regx16_launch(x_bf16, qw, scale, zero, y_bf16, bias, b, n, k, p.gs, p.tpw, p.ring,
+                                  true, stream);
 }
 
 }  // namespace lg

@@ -306,13 +306,14 @@ static hipError_t launch_splitk_bt(const void* x, const void* qw, const void* sc
 
 }  // namespace lg
 
+// The split-K forms hold the whole batch in one launch (and the prepared layout has 32 rows).
 extern "C" int logismos_qgemm_q4g128_splitk_parts(int b, int n, int k) {
-    if (logismos_check_qgemm_q4g128_shape(b, n, k, nullptr, 0) != 0) return 0;
+    if (b > 32 || logismos_check_qgemm_q4g128_shape(b, n, k, nullptr, 0) != 0) return 0;
     return lg::splitk_plan(b, n, k).parts;
 }
 
 extern "C" int logismos_qgemm_q4g128_splitk_xprep_parts(int b, int n, int k) {
-    if (logismos_check_qgemm_q4g128_shape(b, n, k, nullptr, 0) != 0) return 0;
+    if (b > 32 || logismos_check_qgemm_q4g128_shape(b, n, k, nullptr, 0) != 0) return 0;
     if (const lg::RegxPlan rp = lg::regx_plan(b, n, k); rp.parts > 0) return rp.parts;
     return lg::splitk_plan(b, n, k).parts;
 }
@@ -321,7 +322,8 @@ static logismos_status_t splitk_dispatch(const void* x, bool prepared, const voi
                                          const void* scale_f16, const void* zero_f16,
                                          void* parts_f32, int b, int n, int k,
                                          logismos_stream_t stream) {
-    if (logismos_check_qgemm_q4g128_shape(b, n, k, nullptr, 0) != 0) return hipErrorInvalidValue;
+    if (b > 32 || logismos_check_qgemm_q4g128_shape(b, n, k, nullptr, 0) != 0)
+        return hipErrorInvalidValue;
     if (!x || !qw_u8 || !scale_f16 || !zero_f16 || !parts_f32) return hipErrorInvalidValue;
     if ((reinterpret_cast<uintptr_t>(qw_u8) & 15u) || (reinterpret_cast<uintptr_t>(x) & 15u))
         return hipErrorInvalidValue;

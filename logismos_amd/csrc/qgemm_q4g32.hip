@@ -53,7 +53,7 @@ template <int BT, int T>
 __global__ __launch_bounds__(64 * kG32Waves) void qgemm_q4g32_mfma_kernel(
     const uint16_t* __restrict__ x, const uint8_t* __restrict__ qw,
     const __half* __restrict__ scale, const __half* __restrict__ minv, uint16_t* __restrict__ y,
-    int b, int n, int k) {
+    const float* __restrict__ bias, int b, int n, int k) {
     extern __shared__ float yl[];  // [waves][T][BP][16] partial results
     constexpr int BP = BT * 16;
     const int nchunks = k >> 7;
@@ -187,31 +187,33 @@ __global__ __launch_bounds__(64 * kG32Waves) void qgemm_q4g32_mfma_kernel(
         float sum = 0.0f;
 #pragma unroll
         for (int w = 0; w < kG32Waves; ++w) sum += yl[(size_t)w * T * BP * 16 + i];
-        if (r < rows_here && bi < b) y[(int64_t)bi * n + row0 + r] = f32_to_bf16_rne(sum);
+        if (r < rows_here && bi < b)
+            y[(int64_t)bi * n + row0 + r] = f32_to_bf16_rne(bias ? sum + bias[row0 + r] : sum);
     }
 }
 
 template <int BT, int T>
 static hipError_t launch_g32(const void* x, const void* qw, const void* scale, const void* minv,
-                             void* y, int b, int n, int k, hipStream_t stream) {
+                             void* y, const float* bias, int b, int n, int k, hipStream_t stream) {
     const int tiles = (n + 15) / 16;
     const size_t lds = (size_t)kG32Waves * T * BT * 16 * 16 * 4;  // at most 48 KiB
     qgemm_q4g32_mfma_kernel<BT, T><<<dim3((tiles + T - 1) / T), dim3(64 * kG32Waves), lds, stream>>>(
         static_cast<const uint16_t*>(x), static_cast<const uint8_t*>(qw),
         static_cast<const __half*>(scale), static_cast<const __half*>(minv),
-        static_cast<uint16_t*>(y), b, n, k);
+        static_cast<uint16_t*>(y), bias, b, n, k);
     return hipGetLastError();
 }
 
 template <int BT>
 static hipError_t launch_g32_b(const void* x, const void* qw, const void* scale, const void* minv,
-                               void* y, int b, int n, int k, hipStream_t stream) {
+                               void* y, const float* bias, int b, int n, int k,
+                               hipStream_t stream) {
     // row tiles per workgroup: one workgroup per CU where the matrix allows it
     const int tiles = (n + 15) / 16;
     const int t = (tiles + device_cu_count() - 1) / device_cu_count();
-    if (t >= 3) return launch_g32<BT, 3>(x, qw, scale, minv, y, b, n, k, stream);
-    if (t == 2) return launch_g32<BT, 2>(x, qw, scale, minv, y, b, n, k, stream);
-    return launch_g32<BT, 1>(x, qw, scale, minv, y, b, n, k, stream);
+    if (t >= 3) return launch_g32<BT, 3>(x, qw, scale, minv, y, bias, b, n, k, stream);
+    if (t == 2) return launch_g32<BT, 2>(x, qw, scale, minv, y, bias, b, n, k, stream);
+    return launch_g32<BT, 1>(x, qw, scale, minv, y, bias, b, n, k, stream);
 }
 
 }  // namespace lg
@@ -225,8 +227,6 @@ extern "C" logismos_status_t logismos_check_qgemm_q4g32_shape(int b, int n, int 
     if (k % 128 != 0)
         return lg::reject(msg, msg_cap, "%s: K = %d is not a multiple of 128 (four groups of 32)",
                           kn, k);
-    if (b > 32)
-        return lg::reject(msg, msg_cap, "%s: batch %d exceeds the supported maximum of 32", kn, b);
     if ((int64_t)n * k > (int64_t)INT32_MAX)
         return lg::reject(msg, msg_cap, "%s: N*K = %lld exceeds i32::MAX", kn,
                           (long long)((int64_t)n * k));
@@ -235,15 +235,32 @@ extern "C" logismos_status_t logismos_check_qgemm_q4g32_shape(int b, int n, int 
     return 0;
 }
 
-extern "C" logismos_status_t logismos_launch_qgemm_q4g32_bf16(
+extern "C" logismos_status_t logismos_launch_qgemm_q4g32_bf16_bias(
     const void* x_bf16, const void* qw_u8, const void* scale_f16, const void* min_f16,
-    void* y_bf16, int b, int n, int k, logismos_stream_t stream) {
+    const void* bias_f32, void* y_bf16, int b, int n, int k, logismos_stream_t stream) {
     if (logismos_check_qgemm_q4g32_shape(b, n, k, nullptr, 0) != 0) return hipErrorInvalidValue;
     if (!x_bf16 || !qw_u8 || !scale_f16 || !min_f16 || !y_bf16) return hipErrorInvalidValue;
     if ((reinterpret_cast<uintptr_t>(qw_u8) & 15u) || (reinterpret_cast<uintptr_t>(x_bf16) & 15u) ||
         (reinterpret_cast<uintptr_t>(scale_f16) & 7u) || (reinterpret_cast<uintptr_t>(min_f16) & 7u))
         return hipErrorInvalidValue;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (b <= 16) return lg::launch_g32_b<1>(x_bf16, qw_u8, scale_f16, min_f16, y_bf16, b, n, k, st);
-    return lg::launch_g32_b<2>(x_bf16, qw_u8, scale_f16, min_f16, y_bf16, b, n, k, st);
+    const float* bias = static_cast<const float*>(bias_f32);  // may be null: no bias
+    // a taller x is taken 32 rows at a time (`linear_t` takes any m)
+    for (int m0 = 0; m0 < b; m0 += 32) {
+        const int rows = b - m0 < 32 ? b - m0 : 32;
+        const uint16_t* xs = static_cast<const uint16_t*>(x_bf16) + (int64_t)m0 * k;
+        uint16_t* ys = static_cast<uint16_t*>(y_bf16) + (int64_t)m0 * n;
+        const hipError_t e =
+            rows <= 16 ? lg::launch_g32_b<1>(xs, qw_u8, scale_f16, min_f16, ys, bias, rows, n, k, st)
+                       : lg::launch_g32_b<2>(xs, qw_u8, scale_f16, min_f16, ys, bias, rows, n, k, st);
+        if (e != hipSuccess) return e;
+    }
+    return 0;
+}
+
+extern "C" logismos_status_t logismos_launch_qgemm_q4g32_bf16(
+    const void* x_bf16, const void* qw_u8, const void* scale_f16, const void* min_f16,
+    void* y_bf16, int b, int n, int k, logismos_stream_t stream) {
+    return logismos_launch_qgemm_q4g32_bf16_bias(x_bf16, qw_u8, scale_f16, min_f16, nullptr, y_bf16,
+                                                 b, n, k, stream);
 }

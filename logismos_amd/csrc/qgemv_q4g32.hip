@@ -23,7 +23,8 @@ __global__ __launch_bounds__(256) void qgemv_q4g32_kernel(const float* __restric
                                                           const uint8_t* __restrict__ qw,
                                                           const __half* __restrict__ scale,
                                                           const __half* __restrict__ minv,
-                                                          float* __restrict__ y, int n, int k) {
+                                                          float* __restrict__ y,
+        const float* __restrict__ bias, int n, int k) {
     const int lane = threadIdx.x & 63;
     const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     const int64_t row0 = wave * R;
@@ -84,7 +85,7 @@ __global__ __launch_bounds__(256) void qgemv_q4g32_kernel(const float* __restric
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const float total = wave_sum(acc[r]);
-        if (lane == 0 && row0 + r < n) y[row0 + r] = total;
+        if (lane == 0 && row0 + r < n) y[row0 + r] = bias ? total + bias[row0 + r] : total;
     }
 }
 
@@ -101,7 +102,8 @@ __global__ __launch_bounds__(64 * kFlatWaves) void qgemv_q4g32_flat_kernel(const
                                                                const uint8_t* __restrict__ qw,
                                                                const __half* __restrict__ scale,
                                                                const __half* __restrict__ minv,
-                                                               float* __restrict__ y, int n, int k) {
+                                                               float* __restrict__ y,
+        const float* __restrict__ bias, int n, int k) {
     extern __shared__ float4_t xl[];
     const int groups = k >> 5;
     float* xs = reinterpret_cast<float*>(xl + (size_t)8 * groups);
@@ -172,18 +174,18 @@ __global__ __launch_bounds__(64 * kFlatWaves) void qgemv_q4g32_flat_kernel(const
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const float total = wave_sum(acc[r]);
-        if (lane == 0 && r < rows) y[row0 + r] = total;
+        if (lane == 0 && r < rows) y[row0 + r] = bias ? total + bias[row0 + r] : total;
     }
 }
 
 template <int R, int NP = 1>
 static hipError_t launch_q4g32_flat(int np, const float* x, const uint8_t* qw, const __half* scale,
-                                    const __half* minv, float* y, int n, int k,
+                                    const __half* minv, float* y, const float* bias, int n, int k,
                                     hipStream_t stream) {
     if constexpr (NP > (R == 1 ? 8 : 4)) {
         return hipErrorInvalidValue;
     } else {
-        if (np != NP) return launch_q4g32_flat<R, NP + 1>(np, x, qw, scale, minv, y, n, k, stream);
+        if (np != NP) return launch_q4g32_flat<R, NP + 1>(np, x, qw, scale, minv, y, bias, n, k, stream);
         const size_t lds = (size_t)(k / 32) * (8 * 16 + 4);  // at most 66 KiB (K = 16384)
         auto kern = qgemv_q4g32_flat_kernel<R, NP>;
         if (lds > 64 * 1024) {
@@ -193,7 +195,7 @@ static hipError_t launch_q4g32_flat(int np, const float* x, const uint8_t* qw, c
         }
         const int64_t waves = ((int64_t)n + R - 1) / R;
         kern<<<dim3((unsigned)((waves + kFlatWaves - 1) / kFlatWaves)), dim3(64 * kFlatWaves), lds,
-               stream>>>(x, qw, scale, minv, y, n, k);
+               stream>>>(x, qw, scale, minv, y, bias, n, k);
         return hipGetLastError();
     }
 }
@@ -265,11 +267,9 @@ extern "C" logismos_status_t logismos_check_qgemv_q4g32_shape(int n, int k, char
     return 0;
 }
 
-extern "C" logismos_status_t logismos_launch_qgemv_q4g32_f32(const void* x_f32, const void* qw_u8,
-                                                             const void* scale_f16,
-                                                             const void* min_f16, void* y_f32,
-                                                             int n, int k,
-                                                             logismos_stream_t stream) {
+extern "C" logismos_status_t logismos_launch_qgemv_q4g32_f32_bias(
+    const void* x_f32, const void* qw_u8, const void* scale_f16, const void* min_f16,
+    const void* bias_f32, void* y_f32, int n, int k, logismos_stream_t stream) {
     if (logismos_check_qgemv_q4g32_shape(n, k, nullptr, 0) != 0) return hipErrorInvalidValue;
     if (!x_f32 || !qw_u8 || !scale_f16 || !min_f16 || !y_f32) return hipErrorInvalidValue;
     if ((reinterpret_cast<uintptr_t>(qw_u8) & 15u) || (reinterpret_cast<uintptr_t>(x_f32) & 15u))
@@ -280,21 +280,31 @@ extern "C" logismos_status_t logismos_launch_qgemv_q4g32_f32(const void* x_f32, 
     auto* sp = static_cast<const __half*>(scale_f16);
     auto* mp = static_cast<const __half*>(min_f16);
     auto* yp = static_cast<float*>(y_f32);
+    auto* bp = static_cast<const float*>(bias_f32);  // may be null: no bias
     if (const int fr = lg::q4g32_flat_rows(n, k, lg::device_cu_count()); fr > 0) {
         const int np = (fr * (k / 32) + 63) / 64;
         switch (fr) {
-            case 8: return lg::launch_q4g32_flat<8>(np, xp, qp, sp, mp, yp, n, k, st);
-            case 4: return lg::launch_q4g32_flat<4>(np, xp, qp, sp, mp, yp, n, k, st);
-            case 2: return lg::launch_q4g32_flat<2>(np, xp, qp, sp, mp, yp, n, k, st);
-            default: return lg::launch_q4g32_flat<1>(np, xp, qp, sp, mp, yp, n, k, st);
+            case 8: return lg::launch_q4g32_flat<8>(np, xp, qp, sp, mp, yp, bp, n, k, st);
+            case 4: return lg::launch_q4g32_flat<4>(np, xp, qp, sp, mp, yp, bp, n, k, st);
+            case 2: return lg::launch_q4g32_flat<2>(np, xp, qp, sp, mp, yp, bp, n, k, st);
+            default: return lg::launch_q4g32_flat<1>(np, xp, qp, sp, mp, yp, bp, n, k, st);
         }
     }
     constexpr int R = 4;
     const int waves = (n + R - 1) / R;
     const int wpb = 4;
     dim3 grid((waves + wpb - 1) / wpb), block(wpb * 64);
-    lg::qgemv_q4g32_kernel<R><<<grid, block, 0, st>>>(xp, qp, sp, mp, yp, n, k);
+    lg::qgemv_q4g32_kernel<R><<<grid, block, 0, st>>>(xp, qp, sp, mp, yp, bp, n, k);
     return hipGetLastError();
+}
+
+extern "C" logismos_status_t logismos_launch_qgemv_q4g32_f32(const void* x_f32, const void* qw_u8,
+                                                             const void* scale_f16,
+                                                             const void* min_f16, void* y_f32,
+                                                             int n, int k,
+                                                             logismos_stream_t stream) {
+    return logismos_launch_qgemv_q4g32_f32_bias(x_f32, qw_u8, scale_f16, min_f16, nullptr, y_f32, n,
+                                                k, stream);
 }
 
 static logismos_status_t repack_q4(bool has_min, const void* blocks, void* qw_u8, void* scale_f16,

@@ -22,7 +22,8 @@ template <int R>
 __global__ __launch_bounds__(256) void qgemv_q8g32_kernel(const float* __restrict__ x,
                                                           const int8_t* __restrict__ qs,
                                                           const __half* __restrict__ d,
-                                                          float* __restrict__ y, int n, int k) {
+                                                          float* __restrict__ y,
+        const float* __restrict__ bias, int n, int k) {
     const int lane = threadIdx.x & 63;
     const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     const int64_t row0 = wave * R;
@@ -70,7 +71,7 @@ __global__ __launch_bounds__(256) void qgemv_q8g32_kernel(const float* __restric
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const float total = wave_sum(acc[r]);
-        if (lane == 0 && row0 + r < n) y[row0 + r] = total;
+        if (lane == 0 && row0 + r < n) y[row0 + r] = bias ? total + bias[row0 + r] : total;
     }
 }
 
@@ -87,7 +88,8 @@ template <int R, int NP>
 __global__ __launch_bounds__(64 * kFlatWaves) void qgemv_q8g32_flat_kernel(const float* __restrict__ x,
                                                                const int8_t* __restrict__ qs,
                                                                const __half* __restrict__ d,
-                                                               float* __restrict__ y, int n, int k) {
+                                                               float* __restrict__ y,
+        const float* __restrict__ bias, int n, int k) {
     extern __shared__ float4_t xl[];
     const int lane = threadIdx.x & 63;
     const int ppr = k >> 4;  // pieces per row
@@ -140,21 +142,21 @@ __global__ __launch_bounds__(64 * kFlatWaves) void qgemv_q8g32_flat_kernel(const
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const float total = wave_sum(acc[r]);
-        if (lane == 0 && r < rows) y[row0 + r] = total;
+        if (lane == 0 && r < rows) y[row0 + r] = bias ? total + bias[row0 + r] : total;
     }
 }
 
 template <int R, int NP = 1>
 static hipError_t launch_flat(int np, const float* x, const int8_t* qs, const __half* d, float* y,
-                              int n, int k, hipStream_t stream) {
+                              const float* bias, int n, int k, hipStream_t stream) {
     if constexpr (NP > 8) {
         return hipErrorInvalidValue;
     } else {
-        if (np != NP) return launch_flat<R, NP + 1>(np, x, qs, d, y, n, k, stream);
+        if (np != NP) return launch_flat<R, NP + 1>(np, x, qs, d, y, bias, n, k, stream);
         const int64_t waves = ((int64_t)n + R - 1) / R;
         qgemv_q8g32_flat_kernel<R, NP>
             <<<dim3((unsigned)((waves + kFlatWaves - 1) / kFlatWaves)), dim3(64 * kFlatWaves),
-               (size_t)k * 4, stream>>>(x, qs, d, y, n, k);
+               (size_t)k * 4, stream>>>(x, qs, d, y, bias, n, k);
         return hipGetLastError();
     }
 }
@@ -201,9 +203,9 @@ extern "C" logismos_status_t logismos_check_qgemv_q8g32_shape(int n, int k, char
     return 0;
 }
 
-extern "C" logismos_status_t logismos_launch_qgemv_q8g32_f32(const void* x_f32, const void* qs_i8,
-                                                             const void* d_f16, void* y_f32, int n,
-                                                             int k, logismos_stream_t stream) {
+extern "C" logismos_status_t logismos_launch_qgemv_q8g32_f32_bias(
+    const void* x_f32, const void* qs_i8, const void* d_f16, const void* bias_f32, void* y_f32,
+    int n, int k, logismos_stream_t stream) {
     if (logismos_check_qgemv_q8g32_shape(n, k, nullptr, 0) != 0) return hipErrorInvalidValue;
     if (!x_f32 || !qs_i8 || !d_f16 || !y_f32) return hipErrorInvalidValue;
     if ((reinterpret_cast<uintptr_t>(qs_i8) & 15u) || (reinterpret_cast<uintptr_t>(x_f32) & 15u))
@@ -213,21 +215,28 @@ extern "C" logismos_status_t logismos_launch_qgemv_q8g32_f32(const void* x_f32, 
     auto* qp = static_cast<const int8_t*>(qs_i8);
     auto* dp = static_cast<const __half*>(d_f16);
     auto* yp = static_cast<float*>(y_f32);
+    auto* bp = static_cast<const float*>(bias_f32);  // may be null: no bias
     if (const int fr = lg::flat_rows(n, k); fr > 0) {
         const int np = (fr * (k / 16) + 63) / 64;
         switch (fr) {
-            case 8: return lg::launch_flat<8>(np, xp, qp, dp, yp, n, k, st);
-            case 4: return lg::launch_flat<4>(np, xp, qp, dp, yp, n, k, st);
-            case 2: return lg::launch_flat<2>(np, xp, qp, dp, yp, n, k, st);
-            default: return lg::launch_flat<1>(np, xp, qp, dp, yp, n, k, st);
+            case 8: return lg::launch_flat<8>(np, xp, qp, dp, yp, bp, n, k, st);
+            case 4: return lg::launch_flat<4>(np, xp, qp, dp, yp, bp, n, k, st);
+            case 2: return lg::launch_flat<2>(np, xp, qp, dp, yp, bp, n, k, st);
+            default: return lg::launch_flat<1>(np, xp, qp, dp, yp, bp, n, k, st);
         }
     }
     constexpr int R = 4;
     const int waves = (n + R - 1) / R;
     const int wpb = 4;
     dim3 grid((waves + wpb - 1) / wpb), block(wpb * 64);
-    lg::qgemv_q8g32_kernel<R><<<grid, block, 0, st>>>(xp, qp, dp, yp, n, k);
+    lg::qgemv_q8g32_kernel<R><<<grid, block, 0, st>>>(xp, qp, dp, yp, bp, n, k);
     return hipGetLastError();
+}
+
+extern "C" logismos_status_t logismos_launch_qgemv_q8g32_f32(const void* x_f32, const void* qs_i8,
+                                                             const void* d_f16, void* y_f32, int n,
+                                                             int k, logismos_stream_t stream) {
+    return logismos_launch_qgemv_q8g32_f32_bias(x_f32, qs_i8, d_f16, nullptr, y_f32, n, k, stream);
 }
 
 extern "C" logismos_status_t logismos_launch_repack_q8_0(const void* blocks_q8_0, void* qs_i8,

@@ -271,7 +271,8 @@ __global__ __launch_bounds__(64) void rope_kv_write_kernel(
     int64_t part_stride, const int32_t* __restrict__ positions,
     const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     const int64_t* __restrict__ slot_mapping, __half* __restrict__ q_out,
-    __half* __restrict__ k_pool, __half* __restrict__ v_pool, int hq, int hkv, int max_pos) {
+    __half* __restrict__ k_pool, __half* __restrict__ v_pool, int hq, int hkv, int max_pos,
+    const float* __restrict__ bias) {
     constexpr int D = 128, HALF = 64;
     const int head = blockIdx.x;
     const int64_t t = blockIdx.y;
@@ -298,6 +299,11 @@ __global__ __launch_bounds__(64) void rope_kv_write_kernel(
                     x1 += b[r];
                 }
         }
+    }
+    if (bias) {
+        // the projection's bias (`linear_t`, one fp32 add on the finished sum), column head*D + i
+        x0 += bias[head * D + i];
+        x1 += bias[head * D + i + HALF];
     }
     if (head < hq + hkv) {
         int pos = positions[t];
@@ -480,15 +486,15 @@ extern "C" logismos_status_t logismos_launch_rope_kv_write_fp16(
         static_cast<const float*>(cos_f32),
         static_cast<const float*>(sin_f32), slot_mapping, static_cast<__half*>(q_out_f16),
         static_cast<__half*>(k_pool_f16), static_cast<__half*>(v_pool_f16), num_q_heads,
-        num_kv_heads, max_pos);
+        num_kv_heads, max_pos, nullptr);
     return hipGetLastError();
 }
 
-extern "C" logismos_status_t logismos_launch_rope_kv_write_f32p(
-    const void* qkv_parts_f32, int num_parts, const int32_t* positions, const void* cos_f32,
-    const void* sin_f32, const int64_t* slot_mapping, void* q_out_f16, void* k_pool_f16,
-    void* v_pool_f16, int total_tokens, int num_q_heads, int num_kv_heads, int head_dim,
-    int max_pos, logismos_stream_t stream) {
+extern "C" logismos_status_t logismos_launch_rope_kv_write_f32p_bias(
+    const void* qkv_parts_f32, int num_parts, const void* bias_f32, const int32_t* positions,
+    const void* cos_f32, const void* sin_f32, const int64_t* slot_mapping, void* q_out_f16,
+    void* k_pool_f16, void* v_pool_f16, int total_tokens, int num_q_heads, int num_kv_heads,
+    int head_dim, int max_pos, logismos_stream_t stream) {
     if (total_tokens < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || max_pos <= 0 || num_parts <= 0)
         return hipErrorInvalidValue;
     if (head_dim != 128 || total_tokens > 65535) return hipErrorInvalidValue;
@@ -503,15 +509,28 @@ extern "C" logismos_status_t logismos_launch_rope_kv_write_f32p(
         nullptr, static_cast<const float*>(qkv_parts_f32), num_parts, (int64_t)total_tokens * width,
         positions, static_cast<const float*>(cos_f32), static_cast<const float*>(sin_f32),
         slot_mapping, static_cast<__half*>(q_out_f16), static_cast<__half*>(k_pool_f16),
-        static_cast<__half*>(v_pool_f16), num_q_heads, num_kv_heads, max_pos);
+        static_cast<__half*>(v_pool_f16), num_q_heads, num_kv_heads, max_pos,
+        static_cast<const float*>(bias_f32));
     return hipGetLastError();
 }
 
-extern "C" logismos_status_t logismos_launch_rope_kv_write_f32p_turbo3(
+extern "C" logismos_status_t logismos_launch_rope_kv_write_f32p(
     const void* qkv_parts_f32, int num_parts, const int32_t* positions, const void* cos_f32,
-    const void* sin_f32, const int64_t* slot_mapping, void* q_out_f16, void* k_pool_t3,
-    void* v_pool_t3, int total_tokens, int num_q_heads, int num_kv_heads, int head_dim,
+    const void* sin_f32, const int64_t* slot_mapping, void* q_out_f16, void* k_pool_f16,
+    void* v_pool_f16, int total_tokens, int num_q_heads, int num_kv_heads, int head_dim,
     int max_pos, logismos_stream_t stream) {
+    return logismos_launch_rope_kv_write_f32p_bias(qkv_parts_f32, num_parts, nullptr, positions,
+                                                   cos_f32, sin_f32, slot_mapping, q_out_f16,
+                                                   k_pool_f16, v_pool_f16, total_tokens,
+                                                   num_q_heads, num_kv_heads, head_dim, max_pos,
+                                                   stream);
+}
+
+extern "C" logismos_status_t logismos_launch_rope_kv_write_f32p_turbo3_bias(
+    const void* qkv_parts_f32, int num_parts, const void* bias_f32, const int32_t* positions,
+    const void* cos_f32, const void* sin_f32, const int64_t* slot_mapping, void* q_out_f16,
+    void* k_pool_t3, void* v_pool_t3, int total_tokens, int num_q_heads, int num_kv_heads,
+    int head_dim, int max_pos, logismos_stream_t stream) {
     if (total_tokens < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || max_pos <= 0 || num_parts <= 0)
         return hipErrorInvalidValue;
     if (head_dim != 128 || total_tokens > 65535) return hipErrorInvalidValue;
@@ -526,8 +545,19 @@ extern "C" logismos_status_t logismos_launch_rope_kv_write_f32p_turbo3(
         nullptr, static_cast<const float*>(qkv_parts_f32), num_parts, (int64_t)total_tokens * width,
         positions, static_cast<const float*>(cos_f32), static_cast<const float*>(sin_f32),
         slot_mapping, static_cast<__half*>(q_out_f16), static_cast<__half*>(k_pool_t3),
-        static_cast<__half*>(v_pool_t3), num_q_heads, num_kv_heads, max_pos);
+        static_cast<__half*>(v_pool_t3), num_q_heads, num_kv_heads, max_pos,
+        static_cast<const float*>(bias_f32));
     return hipGetLastError();
+}
+
+extern "C" logismos_status_t logismos_launch_rope_kv_write_f32p_turbo3(
+    const void* qkv_parts_f32, int num_parts, const int32_t* positions, const void* cos_f32,
+    const void* sin_f32, const int64_t* slot_mapping, void* q_out_f16, void* k_pool_t3,
+    void* v_pool_t3, int total_tokens, int num_q_heads, int num_kv_heads, int head_dim,
+    int max_pos, logismos_stream_t stream) {
+    return logismos_launch_rope_kv_write_f32p_turbo3_bias(
+        qkv_parts_f32, num_parts, nullptr, positions, cos_f32, sin_f32, slot_mapping, q_out_f16,
+        k_pool_t3, v_pool_t3, total_tokens, num_q_heads, num_kv_heads, head_dim, max_pos, stream);
 }
 
 extern "C" logismos_status_t logismos_launch_silu_mul_f32p(const void* parts_f32, int num_parts,

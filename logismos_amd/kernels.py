@@ -47,6 +47,10 @@ _SIGNATURES = {
     "logismos_check_qgemv_q8g32_shape": (C.c_uint32, [_i, _i, C.c_char_p, _sz]),
     "logismos_check_paged_attn_shape": (C.c_uint32, [_i] * 9 + [C.c_char_p, _sz]),
     "logismos_launch_qgemv_q8g32_f32": (C.c_uint32, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
+    "logismos_launch_qgemv_q8g32_f32_bias": (C.c_uint32, [_vp] * 5 + [_i, _i, _vp]),
+    "logismos_launch_qgemm_q4g128_bf16_bias": (C.c_uint32, [_vp] * 6 + [_i, _i, _i, _vp]),
+    "logismos_launch_qgemv_q4g32_f32_bias": (C.c_uint32, [_vp] * 6 + [_i, _i, _vp]),
+    "logismos_launch_qgemm_q4g32_bf16_bias": (C.c_uint32, [_vp] * 6 + [_i, _i, _i, _vp]),
     "logismos_check_qgemm_q4g128_shape": (C.c_uint32, [_i, _i, _i, C.c_char_p, _sz]),
     "logismos_launch_qgemm_q4g128_bf16": (C.c_uint32, [_vp] * 5 + [_i, _i, _i, _vp]),
     "logismos_launch_qgemm_q4g128_bf16_mfma": (C.c_uint32, [_vp] * 5 + [_i, _i, _i, _vp]),
@@ -87,6 +91,11 @@ _SIGNATURES = {
     "logismos_launch_embed_lookup_f32": (C.c_uint32, [_vp, _vp, _vp, _i, _i, C.c_longlong, _vp]),
     "logismos_launch_embed_lookup_bf16": (C.c_uint32, [_vp, _vp, _vp, _i, _i, C.c_longlong, _vp]),
     "logismos_decode_step_workspace_bytes": (_sz, [_vp, _i, _i]),
+    "logismos_decode_step_workspace_bytes_tokens": (_sz, [_vp, _i, _i, _i]),
+    "logismos_launch_rope_kv_write_f32p_bias":
+        (C.c_uint32, [_vp, _i] + [_vp] * 8 + [_i] * 5 + [_vp]),
+    "logismos_launch_rope_kv_write_f32p_turbo3_bias":
+        (C.c_uint32, [_vp, _i] + [_vp] * 8 + [_i] * 5 + [_vp]),
     "logismos_launch_decode_step": (C.c_uint32, [_vp, _vp, _vp, _vp, _vp]),
     "logismos_qgemm_q4g128_splitk_parts": (C.c_int, [_i, _i, _i]),
     "logismos_qgemm_q4g128_splitk_xprep_parts": (C.c_int, [_i, _i, _i]),
@@ -150,7 +159,7 @@ class DecodeConfig(C.Structure):
 class DecodeLayer(C.Structure):
     _fields_ = [("norm1_w_f32", _vp), ("norm2_w_f32", _vp), ("qkv", Q4Weight), ("o", Q4Weight),
                 ("gate_up", Q4Weight), ("down", Q4Weight), ("k_pool_f16", _vp),
-                ("v_pool_f16", _vp)]
+                ("v_pool_f16", _vp), ("qkv_bias_f32", _vp)]
 
 
 class DecodeBatch(C.Structure):
@@ -159,7 +168,8 @@ class DecodeBatch(C.Structure):
                 ("positions", _vp), ("slot_mapping", _vp), ("rope_cos_f32", _vp),
                 ("rope_sin_f32", _vp), ("num_seqs", _i), ("num_splits", _i),
                 ("token_ids", _vp), ("embed_table_bf16", _vp), ("lm_head", C.POINTER(Q4Weight)),
-                ("out_tokens_u32", _vp), ("logits_f32", _vp)]
+                ("out_tokens_u32", _vp), ("logits_f32", _vp), ("total_tokens", _i),
+                ("max_seqlen_q", _i)]
 
 
 def library() -> C.CDLL:
@@ -205,21 +215,26 @@ def check_qgemv_q4g32_shape(n: int, k: int) -> None:
     _guard("qgemv_q4g32_f32", library().logismos_check_qgemv_q4g32_shape, n, k)
 
 
-def launch_qgemv_q4g32_f32(x, qw, scale, minv, y, n: int, k: int, stream=None) -> None:
+def launch_qgemv_q4g32_f32(x, qw, scale, minv, y, n: int, k: int, stream=None,
+                           bias=None) -> None:
+    """`bias`: fp32 [n] on the device or None, as `linear_t`'s `bias: Option<&[f32]>`."""
     check_qgemv_q4g32_shape(n, k)
-    _status("qgemv_q4g32_f32", library().logismos_launch_qgemv_q4g32_f32(
-        _ptr(x), _ptr(qw), _ptr(scale), _ptr(minv), _ptr(y), n, k, _raw(stream)))
+    _status("qgemv_q4g32_f32", library().logismos_launch_qgemv_q4g32_f32_bias(
+        _ptr(x), _ptr(qw), _ptr(scale), _ptr(minv), _ptr(bias) if bias is not None else None,
+        _ptr(y), n, k, _raw(stream)))
 
 
 def check_qgemm_q4g32_shape(b: int, n: int, k: int) -> None:
     _guard("qgemm_q4g32_bf16", library().logismos_check_qgemm_q4g32_shape, b, n, k)
 
 
-def launch_qgemm_q4g32_bf16(x, qw, scale, minv, y, b: int, n: int, k: int, stream=None) -> None:
-    """Batched (1..32 rows) product over planar Q4G32 weights; x and y bf16."""
+def launch_qgemm_q4g32_bf16(x, qw, scale, minv, y, b: int, n: int, k: int, stream=None,
+                            bias=None) -> None:
+    """Batched product over planar Q4G32 weights; x and y bf16; optional fp32 bias [n]."""
     check_qgemm_q4g32_shape(b, n, k)
-    _status("qgemm_q4g32_bf16", library().logismos_launch_qgemm_q4g32_bf16(
-        _ptr(x), _ptr(qw), _ptr(scale), _ptr(minv), _ptr(y), b, n, k, _raw(stream)))
+    _status("qgemm_q4g32_bf16", library().logismos_launch_qgemm_q4g32_bf16_bias(
+        _ptr(x), _ptr(qw), _ptr(scale), _ptr(minv), _ptr(bias) if bias is not None else None,
+        _ptr(y), b, n, k, _raw(stream)))
 
 
 def launch_repack_q4_blocks(blocks, qw, scale, minv, n: int, k: int, has_min: bool,
@@ -236,10 +251,16 @@ def check_qgemv_q8g32_shape(n: int, k: int) -> None:
     _guard("qgemv_q8g32_f32", library().logismos_check_qgemv_q8g32_shape, n, k)
 
 
-def launch_qgemv_q8g32_f32(x, qs, d, y, n: int, k: int, stream=None) -> None:
+def launch_qgemv_q8g32_f32(x, qs, d, y, n: int, k: int, stream=None, bias=None) -> None:
+    """`bias`: fp32 [n] on the device or None, as `linear_t`'s `bias: Option<&[f32]>`."""
     check_qgemv_q8g32_shape(n, k)
-    _status("qgemv_q8g32_f32", library().logismos_launch_qgemv_q8g32_f32(
-        _ptr(x), _ptr(qs), _ptr(d), _ptr(y), n, k, _raw(stream)))
+    if bias is None:
+        code = library().logismos_launch_qgemv_q8g32_f32(
+            _ptr(x), _ptr(qs), _ptr(d), _ptr(y), n, k, _raw(stream))
+    else:
+        code = library().logismos_launch_qgemv_q8g32_f32_bias(
+            _ptr(x), _ptr(qs), _ptr(d), _ptr(bias), _ptr(y), n, k, _raw(stream))
+    _status("qgemv_q8g32_f32", code)
 
 
 def check_qgemm_q4g128_shape(b: int, n: int, k: int) -> None:
@@ -247,8 +268,15 @@ def check_qgemm_q4g128_shape(b: int, n: int, k: int) -> None:
 
 
 def launch_qgemm_q4g128_bf16(x, qw, scale, zero, y, b: int, n: int, k: int, stream=None,
-                             force_mfma: bool = False) -> None:
+                             force_mfma: bool = False, bias=None) -> None:
     check_qgemm_q4g128_shape(b, n, k)
+    if bias is not None:
+        if force_mfma:
+            raise ValueError("the forced matrix-core entry point takes no bias")
+        _status("qgemm_q4g128_bf16", library().logismos_launch_qgemm_q4g128_bf16_bias(
+            _ptr(x), _ptr(qw), _ptr(scale), _ptr(zero), _ptr(bias), _ptr(y), b, n, k,
+            _raw(stream)))
+        return
     fn = (library().logismos_launch_qgemm_q4g128_bf16_mfma if force_mfma
           else library().logismos_launch_qgemm_q4g128_bf16)
     _status("qgemm_q4g128_bf16", fn(_ptr(x), _ptr(qw), _ptr(scale), _ptr(zero), _ptr(y), b, n, k,
@@ -467,6 +495,12 @@ def launch_embed_lookup(table, ids, out, rows: int, hidden: int, vocab: int, bf1
                                _raw(stream)))
 
 
+def decode_step_workspace_bytes_tokens(cfg: DecodeConfig, num_seqs: int, total_tokens: int,
+                                       num_splits: int) -> int:
+    return library().logismos_decode_step_workspace_bytes_tokens(C.byref(cfg), num_seqs,
+                                                                 total_tokens, num_splits)
+
+
 def decode_step_workspace_bytes(cfg: DecodeConfig, num_seqs: int, num_splits: int) -> int:
     return library().logismos_decode_step_workspace_bytes(C.byref(cfg), num_seqs, num_splits)
 
@@ -510,13 +544,13 @@ def launch_add_rms_norm_f32p(h, parts, num_parts: int, w, out, rows: int, n: int
 
 def launch_rope_kv_write_f32p(parts, num_parts: int, positions, cos, sin, slot_mapping, q_out,
                               k_pool, v_pool, total_tokens: int, hq: int, hkv: int, head_dim: int,
-                              max_pos: int, stream=None, turbo3: bool = False) -> None:
-    fn = (library().logismos_launch_rope_kv_write_f32p_turbo3 if turbo3
-          else library().logismos_launch_rope_kv_write_f32p)
+                              max_pos: int, stream=None, turbo3: bool = False, bias=None) -> None:
+    fn = (library().logismos_launch_rope_kv_write_f32p_turbo3_bias if turbo3
+          else library().logismos_launch_rope_kv_write_f32p_bias)
     _status("rope_kv_write_f32p", fn(
-        _ptr(parts), num_parts, _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping),
-        _ptr(q_out), _ptr(k_pool), _ptr(v_pool), total_tokens, hq, hkv, head_dim, max_pos,
-        _raw(stream)))
+        _ptr(parts), num_parts, _ptr(bias) if bias is not None else None, _ptr(positions),
+        _ptr(cos), _ptr(sin), _ptr(slot_mapping), _ptr(q_out), _ptr(k_pool), _ptr(v_pool),
+        total_tokens, hq, hkv, head_dim, max_pos, _raw(stream)))
 
 
 def launch_silu_mul_f32p(parts, num_parts: int, out, rows: int, inter: int, stream=None) -> None:

@@ -363,25 +363,36 @@ def dequantize_q4g32(qw, scale, minv, n, k):
     return w
 
 
-def qgemv_q4g32_f32(x, qw, scale, minv, n, k):
+
+def _add_bias(y, bias):
+    """`linear_t`'s bias (crates/kernels/src/cpu_f32/mod.rs:336-343): one fp32 add per output,
+    after the accumulation, broadcast over the rows."""
+    if bias is None:
+        return y
+    bias = _f32(bias)
+    assert bias.shape == (y.shape[-1],)
+    return (y + bias).astype(np.float32)
+
+
+def qgemv_q4g32_f32(x, qw, scale, minv, n, k, bias=None):
     x = _f32(x)
     qw = np.ascontiguousarray(qw, dtype=np.uint8)
     scale, minv = _u16(scale), _u16(minv)
     y = np.empty(n, np.float32)
     _qgemv_q4g32(_p(x), _p(qw), _p(scale), _p(minv), _p(y), n, k)
-    return y
+    return _add_bias(y, bias)
 
 
-def qgemm_q4g32_f32(x_bf16_bits, qw, scale, minv, b, n, k):
+def qgemm_q4g32_f32(x_bf16_bits, qw, scale, minv, b, n, k, bias=None):
     """`linear_t` (crates/kernels/src/cpu_f32/mod.rs:271-345) at m = b over the dequantised Q4G32
     matrix: the GEMV above once per batch row, x given as bf16 bits; fp32 result."""
     x = bf16_bits_to_f32(np.asarray(x_bf16_bits).reshape(b, k))
-    return np.stack([qgemv_q4g32_f32(x[i], qw, scale, minv, n, k) for i in range(b)])
+    return np.stack([qgemv_q4g32_f32(x[i], qw, scale, minv, n, k, bias) for i in range(b)])
 
 
-def qgemm_q4g32_bf16(x_bf16_bits, qw, scale, minv, b, n, k):
+def qgemm_q4g32_bf16(x_bf16_bits, qw, scale, minv, b, n, k, bias=None):
     """The same, rounded once to bf16 (round to nearest even) like the Q4G128 GEMM's output."""
-    return f32_to_bf16_bits(qgemm_q4g32_f32(x_bf16_bits, qw, scale, minv, b, n, k))
+    return f32_to_bf16_bits(qgemm_q4g32_f32(x_bf16_bits, qw, scale, minv, b, n, k, bias))
 
 
 def quantize_q8g32(w, n, k):
@@ -417,13 +428,13 @@ def q8_0_blocks_to_q8g32(blocks, n, k):
     return qs, d.view(np.float16)
 
 
-def qgemv_q8g32_f32(x, qs, d, n, k):
+def qgemv_q8g32_f32(x, qs, d, n, k, bias=None):
     x = _f32(x)
     qs = np.ascontiguousarray(qs, dtype=np.int8)
     d = _u16(d)
     y = np.empty(n, np.float32)
     _qgemv_q8(_p(x), _p(qs), _p(d), _p(y), n, k)
-    return y
+    return _add_bias(y, bias)
 
 
 def quantize_q4g128(w, n, k):
@@ -447,16 +458,18 @@ def dequantize_q4g128(qw, scale, zero, n, k):
 _qgemm_q4_f32 = _sig("oracle_qgemm_q4g128_f32", None, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz)
 
 
-def qgemm_q4g128_f32(x_bf16_bits, qw, scale, zero, b, n, k):
+def qgemm_q4g128_f32(x_bf16_bits, qw, scale, zero, b, n, k, bias=None):
     x = _u16(x_bf16_bits)
     qw = np.ascontiguousarray(qw, dtype=np.uint8)
     scale, zero = _u16(scale), _u16(zero)
     y = np.empty((b, n), np.float32)
     _qgemm_q4_f32(_p(x), _p(qw), _p(scale), _p(zero), _p(y), b, n, k)
-    return y
+    return _add_bias(y, bias)
 
 
-def qgemm_q4g128_bf16(x_bf16_bits, qw, scale, zero, b, n, k):
+def qgemm_q4g128_bf16(x_bf16_bits, qw, scale, zero, b, n, k, bias=None):
+    if bias is not None:  # the bias goes onto the fp32 sum, before the one rounding
+        return f32_to_bf16_bits(qgemm_q4g128_f32(x_bf16_bits, qw, scale, zero, b, n, k, bias))
     x = _u16(x_bf16_bits)
     qw = np.ascontiguousarray(qw, dtype=np.uint8)
     scale, zero = _u16(scale), _u16(zero)

@@ -78,19 +78,23 @@ def cast_f16_bf16(a16):
     return O.f32_to_bf16_bits(O.f16_bits_to_f32(np.ascontiguousarray(a16).view(np.uint16)))
 
 
-def _gemm(x_bits, w, b):
+def _gemm(x_bits, w, b, bias=None):
     qw, s, z = w
     n, k = qw.shape[0], qw.shape[1] * 2
-    return O.qgemm_q4g128_f32(np.ascontiguousarray(x_bits), qw, s, z, b, n, k)
+    return O.qgemm_q4g128_f32(np.ascontiguousarray(x_bits), qw, s, z, b, n, k, bias)
 
 
 def decode_step(cfg, layers, batch, trace=None):
-    """One decode step over `batch` (one new token per sequence).
+    """One step over `batch`: one row per new token, in packed order -- one token per sequence
+    for a decode step, `cu_seqlens[s+1] - cu_seqlens[s]` tokens of sequence s for a mixed batch
+    (chunked prefill + decode; causal inside a chunk).
 
     cfg:    dict(hidden, hq, hkv, d, inter, eps, block_size[, kv_turbo3: the pools are uint8
             turbo3 pools [rows][hkv*56]])
-    layers: list of dict(norm1, qkv, o, norm2, gate_up, down, k_pool, v_pool); each weight a
-            (qw, scale, zero) triple; pools are updated in place
+    layers: list of dict(norm1, qkv, o, norm2, gate_up, down, k_pool, v_pool[, qkv_bias]); each
+            weight a (qw, scale, zero) triple; qkv_bias fp32 [(hq+2hkv)*d] is the bias of the
+            q/k/v projections (crates/transformers/src/attention.rs:49-57), added as `linear_t`
+            adds it; pools are updated in place
     batch:  dict(h [B, hidden] fp32 (updated in place), block_tables, cu_seqlens, context_lens,
             positions, slots, cos, sin, final_norm); optionally token_ids (uint32 [B]) with
             embed_table (bf16 bits [vocab, hidden]): h is first filled by `embed_lookup`; and
@@ -107,7 +111,7 @@ def decode_step(cfg, layers, batch, trace=None):
     y = None
     for li, L in enumerate(layers):
         xn = add_rms_norm_bf16(h, y, L["norm1"], cfg["eps"])
-        qkv = _gemm(xn, L["qkv"], b)
+        qkv = _gemm(xn, L["qkv"], b, L.get("qkv_bias"))
         t3 = bool(cfg.get("kv_turbo3"))
         q16 = rope_kv_write(qkv, batch["positions"], batch["cos"], batch["sin"], batch["slots"],
                             L["k_pool"], L["v_pool"], cfg["hq"], cfg["hkv"], cfg["d"], turbo3=t3)

@@ -92,10 +92,12 @@ class DecodeStepRunner:
 
     def __init__(self, cfg, layers, batch, num_splits=None, stream=None, share_layer_data=False):
         self.cfg_d, self.stream = cfg, stream
-        b = batch["h"].shape[0]
+        b = batch["h"].shape[0]  # packed rows (= sequences for a decode step)
         self.b = b
+        nseq = len(batch["context_lens"])
+        self.num_seqs = nseq
         max_blocks = batch["block_tables"].shape[1]
-        self.num_splits = num_splits or kernels.paged_attn_num_splits(b, cfg["hkv"],
+        self.num_splits = num_splits or kernels.paged_attn_num_splits(nseq, cfg["hkv"],
                                                                       cfg["block_size"], max_blocks)
         half = cfg["d"] // 2
         self.cfg = kernels.DecodeConfig(len(layers), cfg["hidden"], cfg["hq"], cfg["hkv"], cfg["d"],
@@ -149,6 +151,10 @@ class DecodeStepRunner:
             for name, trio in zip(("qkv", "o", "gate_up", "down"), q4):
                 setattr(lay, name, kernels.Q4Weight(*[_val(x) for x in trio]))
             lay.k_pool_f16, lay.v_pool_f16 = _val(kp), _val(vp)
+            if L.get("qkv_bias") is not None:
+                bb = up(np.ascontiguousarray(L["qkv_bias"], np.float32))
+                self.keep.append(bb)
+                lay.qkv_bias_f32 = _val(bb)
 
         self.h = up(batch["h"].astype(np.float32))
         self.out = hip.DeviceBuffer(b * cfg["hidden"] * 2)
@@ -161,8 +167,12 @@ class DecodeStepRunner:
         self.batch = kernels.DecodeBatch(
             _val(self.h), _val(self.out), _val(self.fnorm), _val(self.idx["block_tables"]),
             _val(self.idx["cu_seqlens"]), _val(self.idx["context_lens"]),
-            _val(self.idx["positions"]), _val(self.slots), _val(self.cos), _val(self.sin), b,
+            _val(self.idx["positions"]), _val(self.slots), _val(self.cos), _val(self.sin), nseq,
             self.num_splits)
+        if b != nseq:
+            cu = np.asarray(batch["cu_seqlens"])
+            self.batch.total_tokens = b
+            self.batch.max_seqlen_q = int(np.diff(cu).max())
         self.vocab = self.cfg.vocab
         if self.vocab:
             # tokens in (embedding lookup) and tokens out (vocabulary projection + greedy)
@@ -178,7 +188,7 @@ class DecodeStepRunner:
             self.batch.lm_head = C.pointer(self.head)
             self.batch.out_tokens_u32 = _val(self.tokens)
             self.batch.logits_f32 = _val(self.logits)
-        ws = kernels.decode_step_workspace_bytes(self.cfg, b, self.num_splits)
+        ws = kernels.decode_step_workspace_bytes_tokens(self.cfg, nseq, b, self.num_splits)
         assert ws > 0
         self.ws = hip.DeviceBuffer(ws)
         self.ws.fill(0xFF)

@@ -31,7 +31,7 @@ def test_binding_covers_exactly_the_header():
 
 def test_identity():
     lib = kernels.library()
-    assert lib.logismos_decode_abi_version() == 3
+    assert lib.logismos_decode_abi_version() == 4
     assert lib.logismos_decode_offload_arch() == b"gfx950"
 
 
@@ -111,10 +111,14 @@ def test_qgemm_q4_shape_guard(b, n, k, frag):
         kernels.check_qgemm_q4g128_shape(b, n, k)
     assert frag in str(e.value)
     kernels.check_qgemm_q4g128_shape(1, 12288, 4096)
+    kernels.check_qgemm_q4g128_shape(8240, 4096, 4096)  # any m, as linear_t; 32 rows per pass
+    # the split-K forms hold the whole batch in one launch: at most 32 rows
+    assert kernels.qgemm_q4g128_splitk_parts(33, 4096, 4096) == 0
+    assert kernels.qgemm_q4g128_splitk_parts(33, 4096, 4096, prepared=True) == 0
 
 
 @pytest.mark.parametrize("b,n,k,frag", [
-    (0, 8, 128, "batch must be positive"), (33, 8, 128, "exceeds the supported maximum of 32"),
+    (0, 8, 128, "batch must be positive"),
     (1, 0, 128, "N must be positive"), (1, 8, 96, "multiple of 128"),
     (1, 1 << 20, 1 << 12, "exceeds i32::MAX"),
 ])
@@ -123,6 +127,7 @@ def test_qgemm_q4g32_shape_guard(b, n, k, frag):
         kernels.check_qgemm_q4g32_shape(b, n, k)
     assert frag in str(e.value)
     kernels.check_qgemm_q4g32_shape(16, 12288, 4096)
+    kernels.check_qgemm_q4g32_shape(8240, 4096, 4096)  # any m, as linear_t; 32 rows per pass
 
 
 def test_q4g32_launchers_reject_bad_arguments_without_touching_the_device():

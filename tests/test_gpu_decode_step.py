@@ -7,6 +7,7 @@ import pytest
 import oracle as O
 from oracle import decode_step as OS
 from tests import workloads
+from logismos_amd import hip, kernels
 from tests.gpu_harness import DecodeStepRunner, assert_parity
 
 pytestmark = pytest.mark.gpu
@@ -142,3 +143,88 @@ def test_step_over_turbo3_pools():
                   what="turbo3 K norms")
     assert_parity(norms(gv[slots]), norms(lay[0]["v_pool"][slots]), max_abs=1e-3, max_rel=2e-3,
                   what="turbo3 V norms")
+
+
+def _check_step(cfg, layers, batch, what, layers_n):
+    r, got, want, lay, bat = _run_both(cfg, layers, batch)
+    assert _rel_l2(got, want) < 5e-3, what
+    assert np.all(np.abs(got - want) <= 2e-2 + 3e-2 * np.abs(want)), what
+    h_gpu = r.h.to_numpy(np.float32, bat["h"].shape)
+    assert _rel_l2(h_gpu, bat["h"]) < 5e-3, what
+    slots = np.asarray(batch["slots"])
+    for (kp, vp), L in zip(r.pools, lay):
+        gk = kp.to_numpy(np.float16, L["k_pool"].shape)
+        assert_parity(gk[slots], L["k_pool"][slots], max_abs=4e-3, max_rel=1e-2,
+                      what=f"{what}: appended K rows")
+        rest = np.ones(gk.shape[0], bool)
+        rest[slots] = False
+        assert np.array_equal(gk[rest].view(np.uint16), L["k_pool"][rest].view(np.uint16))
+    return r
+
+
+def test_mixed_batch_in_one_chunk_with_qkv_bias():
+    # a decode row, a 7-token chunk with prior context, a whole 3-token prompt, a 5-token
+    # chunk: 16 packed rows, causal inside each chunk; the q/k/v projections carry a bias
+    rng = np.random.default_rng(37)
+    cfg, layers, batch = workloads.decode_step_problem(
+        rng, num_layers=2, hidden=512, hq=4, hkv=2, inter=1024, ctx=[90, 400, 3, 21],
+        new_tokens=[1, 7, 3, 5], qkv_bias=True)
+    _check_step(cfg, layers, batch, "mixed batch, one chunk", 2)
+
+
+def test_mixed_batch_over_several_chunks_of_rows():
+    # 1 + 40 + 3 + 1 + 37 = 82 packed rows: three passes of 32, 32 and 18 rows through the
+    # projections, one attention launch over the ragged batch per layer
+    rng = np.random.default_rng(38)
+    cfg, layers, batch = workloads.decode_step_problem(
+        rng, num_layers=2, hidden=512, hq=4, hkv=2, inter=1024, ctx=[700, 140, 3, 33, 37],
+        new_tokens=[1, 40, 3, 1, 37], qkv_bias=True)
+    assert batch["h"].shape[0] == 82
+    _check_step(cfg, layers, batch, "mixed batch, three chunks", 2)
+
+
+def test_more_than_32_decode_sequences():
+    rng = np.random.default_rng(39)
+    ctx = rng.integers(1, 300, size=45)
+    cfg, layers, batch = workloads.decode_step_problem(
+        rng, num_layers=2, hidden=512, hq=4, hkv=2, inter=1024, ctx=ctx)
+    _check_step(cfg, layers, batch, "45 decode sequences", 2)
+
+
+def test_full_layer_mixed_batch_at_qwen3_8b_geometry():
+    # one layer at config 5's geometry over a mixed batch: 6 decode rows and two prefill chunks
+    # (130 and 64 tokens, prior contexts 200 and 0) = 200 packed rows, 7 passes of rows
+    rng = np.random.default_rng(40)
+    ctx = [300, 17, 1024, 330, 2000, 64, 5, 77]
+    new = [1, 1, 1, 130, 1, 64, 1, 1]
+    cfg, layers, batch = workloads.decode_step_problem(
+        rng, num_layers=1, hidden=4096, hq=32, hkv=8, inter=12288, ctx=ctx, new_tokens=new)
+    assert batch["h"].shape[0] == 200
+    r, got, want, lay, bat = _run_both(cfg, layers, batch)
+    assert _rel_l2(got, want) < 4e-3
+    assert np.all(np.abs(got - want) <= 1.2e-2 + 1.6e-2 * np.abs(want))
+
+
+def test_step_rejects_what_it_cannot_run():
+    import ctypes as C
+    rng = np.random.default_rng(41)
+    cfg, layers, batch = workloads.decode_step_problem(
+        rng, num_layers=1, hidden=512, hq=4, hkv=2, inter=1024, ctx=[5, 9])
+    r = DecodeStepRunner(cfg, layers, batch)
+    lib = kernels.library()
+    call = lambda: lib.logismos_launch_decode_step(C.byref(r.cfg), r.layers, C.byref(r.batch),
+                                                   r.ws.ptr, None)
+    assert call() == 0
+    # RoPE tables shorter than what the block tables can hold
+    keep = r.cfg.max_pos
+    r.cfg.max_pos = r.cfg.block_size * r.cfg.max_blocks_per_seq - 1
+    assert call() == 1
+    r.cfg.max_pos = keep
+    # fewer packed rows than sequences, or a chunk longer than the batch
+    r.batch.total_tokens, r.batch.max_seqlen_q = 1, 1
+    assert call() == 1
+    r.batch.total_tokens, r.batch.max_seqlen_q = 2, 3
+    assert call() == 1
+    r.batch.total_tokens, r.batch.max_seqlen_q = 0, 0
+    assert call() == 0
+    hip.synchronize()

@@ -1,0 +1,141 @@
+"""GPU parity of what `cpu_f32::linear_t` is beyond a bare decode GEMV
+(crates/kernels/src/cpu_f32/mod.rs:271-345): the optional bias (the q/k/v projections of
+Qwen2 carry one, crates/transformers/src/attention.rs:49-57) and any number of activation
+rows m (`seq` rows of a prefill chunk, crates/transformers/src/mlp.rs:104-111), through the
+C ABI, against the CPU oracle.  bf16 / fp32 outputs with fp32 accumulation: 2e-3 absolute or
+1e-2 relative (fp32 GEMV outputs: 2e-5 / 1e-4)."""
+import numpy as np
+import pytest
+
+import oracle as O
+from logismos_amd import hip, kernels
+from tests.gpu_harness import assert_parity
+
+pytestmark = pytest.mark.gpu
+
+up = hip.DeviceBuffer.from_numpy
+
+
+def _q4(rng, n, k):
+    w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
+    return O.quantize_q4g128(w, n, k)
+
+
+def _gemm_q4(xb, qw, s, z, b, n, k, bias):
+    d_y = hip.DeviceBuffer(b * n * 2)
+    d_y.fill(0xFF)
+    kernels.launch_qgemm_q4g128_bf16(up(xb), up(qw), up(s.view(np.uint16)), up(z.view(np.uint16)),
+                                     d_y, b, n, k, bias=up(bias) if bias is not None else None)
+    hip.synchronize()
+    return O.bf16_bits_to_f32(d_y.to_numpy(np.uint16, (b, n)))
+
+
+# every kernel behind the Q4G128 entry point: VALU GEMV (b = 1, 2), x-in-registers kernels
+# for 16- and 32-row tiles (K = 4096 / 2048, N >= 1024), the MFMA kernel (other K)
+@pytest.mark.parametrize("b,n,k", [(1, 2048, 1536), (2, 300, 1536), (2, 12288, 4096),
+                                   (4, 1100, 4096), (16, 4096, 2048), (32, 6144, 4096),
+                                   (5, 2048, 1536), (24, 777, 1152)])
+def test_q4g128_bias_epilogue(b, n, k):
+    rng = np.random.default_rng(1000 * b + n + k)
+    qw, s, z = _q4(rng, n, k)
+    xb = O.f32_to_bf16_bits(rng.standard_normal((b, k), np.float32))
+    bias = (rng.standard_normal(n) * 2).astype(np.float32)
+    got = _gemm_q4(xb, qw, s, z, b, n, k, bias)
+    want = O.bf16_bits_to_f32(O.qgemm_q4g128_bf16(xb, qw, s, z, b, n, k, bias))
+    assert_parity(got, want, what=f"q4g128 + bias {b}x{n}x{k}")
+    # the bias really is in there (outputs without it differ by about |bias|)
+    plain = O.bf16_bits_to_f32(O.qgemm_q4g128_bf16(xb, qw, s, z, b, n, k))
+    assert np.abs(got - plain).max() > 1.0
+
+
+def test_q8g32_gemv_bias_qwen2_qkv_shape():
+    # Qwen2-1.5B q/k/v projection with its bias: 1536 -> (12 + 2 * 2) * 128
+    rng = np.random.default_rng(5)
+    n, k = 2048, 1536
+    w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
+    qs, d = O.quantize_q8g32(w, n, k)
+    x = rng.standard_normal(k, np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    d_y = hip.DeviceBuffer(n * 4)
+    for shape_n in (n, 37):  # the flat kernel and the short-matrix kernel
+        kernels.launch_qgemv_q8g32_f32(up(x), up(qs[:shape_n]), up(d[:shape_n].view(np.uint16)), d_y,
+                                       shape_n, k, bias=up(bias[:shape_n]))
+        hip.synchronize()
+        got = d_y.to_numpy(np.float32, (shape_n,))
+        want = O.qgemv_q8g32_f32(x, qs[:shape_n], d[:shape_n], shape_n, k, bias[:shape_n])
+        assert_parity(got, want, max_abs=2e-5, max_rel=1e-4, what="q8g32 gemv + bias")
+
+
+def test_q4g32_gemv_and_gemm_bias():
+    rng = np.random.default_rng(6)
+    n, k, b = 1500, 1024, 7
+    w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
+    q32, s32, m32 = O.q4_blocks_to_q4g32(O.quantize_q4_blocks(w, n, k, True), n, k, True)
+    bias = rng.standard_normal(n).astype(np.float32)
+    x = rng.standard_normal((b, k), np.float32)
+    d_q, d_s, d_m = up(q32), up(s32.view(np.uint16)), up(m32.view(np.uint16))
+    d_y = hip.DeviceBuffer(n * 4)
+    kernels.launch_qgemv_q4g32_f32(up(x[0]), d_q, d_s, d_m, d_y, n, k, bias=up(bias))
+    hip.synchronize()
+    assert_parity(d_y.to_numpy(np.float32, (n,)), O.qgemv_q4g32_f32(x[0], q32, s32, m32, n, k, bias),
+                  max_abs=2e-5, max_rel=1e-4, what="q4g32 gemv + bias")
+    xb = O.f32_to_bf16_bits(x)
+    d_yb = hip.DeviceBuffer(b * n * 2)
+    kernels.launch_qgemm_q4g32_bf16(up(xb), d_q, d_s, d_m, d_yb, b, n, k, bias=up(bias))
+    hip.synchronize()
+    assert_parity(O.bf16_bits_to_f32(d_yb.to_numpy(np.uint16, (b, n))),
+                  O.bf16_bits_to_f32(O.qgemm_q4g32_bf16(xb, q32, s32, m32, b, n, k, bias)),
+                  what="q4g32 gemm + bias")
+
+
+def test_q4g128_512_rows_through_the_mlp_up_projection():
+    # one 512-token prefill chunk through gate/up-sized weights: m = 512, 12288 x 4096
+    rng = np.random.default_rng(7)
+    b, n, k = 512, 12288, 4096
+    qw = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+    s = (rng.random((n, k // 128), np.float32) * 0.004 + 0.004).astype(np.float16)
+    z = (rng.random((n, k // 128), np.float32) * 2 + 6.5).astype(np.float16)
+    xb = O.f32_to_bf16_bits(rng.standard_normal((b, k), np.float32))
+    got = _gemm_q4(xb, qw, s, z, b, n, k, None)
+    # the oracle on a sample of rows that straddles the 32-row passes (each row of the product
+    # depends on its own row of x only)
+    rows = np.r_[0:34, 250:262, 480:512]
+    want = O.bf16_bits_to_f32(O.qgemm_q4g128_bf16(xb[rows], qw, s, z, len(rows), n, k))
+    assert_parity(got[rows], want, what="q4g128 m = 512")
+    assert np.isfinite(got).all()
+    # every row was written by its own pass: a row of x repeated gives the same output row
+    xb2 = xb.copy()
+    xb2[300] = xb2[3]
+    xb2[511] = xb2[3]
+    got2 = _gemm_q4(xb2, qw, s, z, b, n, k, None)
+    assert np.array_equal(got2[300], got2[3]) and np.array_equal(got2[511], got2[3])
+
+
+def test_q4g128_packed_mixed_batch_rows_with_a_ragged_tail_and_bias():
+    # config 4's packed token buffer (48 decode rows + 16 x 512 prefill rows = 8240 = 257 * 32
+    # + 16) through an attention-output-sized projection, with a bias
+    rng = np.random.default_rng(8)
+    b, n, k = 8240, 4096, 4096
+    qw, s, z = _q4(rng, n, k)
+    xb = O.f32_to_bf16_bits(rng.standard_normal((b, k), np.float32))
+    bias = rng.standard_normal(n).astype(np.float32)
+    got = _gemm_q4(xb, qw, s, z, b, n, k, bias)
+    rows = np.r_[0:3, 30:35, 4111:4114, 8222:8240]
+    want = O.bf16_bits_to_f32(O.qgemm_q4g128_bf16(xb[rows], qw, s, z, len(rows), n, k, bias))
+    assert_parity(got[rows], want, what="q4g128 m = 8240 + bias")
+    assert np.isfinite(got).all()
+
+
+def test_q4g32_tall_x():
+    rng = np.random.default_rng(9)
+    b, n, k = 83, 1024, 512
+    w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
+    q32, s32, m32 = O.q4_blocks_to_q4g32(O.quantize_q4_blocks(w, n, k, False), n, k, False)
+    xb = O.f32_to_bf16_bits(rng.standard_normal((b, k), np.float32))
+    d_yb = hip.DeviceBuffer(b * n * 2)
+    kernels.launch_qgemm_q4g32_bf16(up(xb), up(q32), up(s32.view(np.uint16)),
+                                    up(m32.view(np.uint16)), d_yb, b, n, k)
+    hip.synchronize()
+    assert_parity(O.bf16_bits_to_f32(d_yb.to_numpy(np.uint16, (b, n))),
+                  O.bf16_bits_to_f32(O.qgemm_q4g32_bf16(xb, q32, s32, m32, b, n, k)),
+                  what="q4g32 gemm m = 83")

@@ -71,7 +71,9 @@ def rope_halves(x, pos, theta, d):
 
 
 class DenseStep:
-    """Float64 dense restatement of one decode step for ONE new token per sequence."""
+    """Float64 dense restatement of one step: row t of the packed batch is new token
+    t - cu[s] of its sequence s, at position ctx[s] - new[s] + (t - cu[s]), and sees the keys
+    up to its own position."""
 
     def __init__(self, cfg, layers, batch, theta, rounding):
         self.cfg, self.rounding, self.theta = cfg, rounding, theta
@@ -81,11 +83,13 @@ class DenseStep:
             norm1=L["norm1"].astype(np.float64), norm2=L["norm2"].astype(np.float64),
             qkv=dequant_q4g128(L["qkv"]), o=dequant_q4g128(L["o"]),
             gate_up=dequant_q4g128(L["gate_up"]), down=dequant_q4g128(L["down"]),
-            k_pool=L["k_pool"].astype(np.float64), v_pool=L["v_pool"].astype(np.float64))
+            k_pool=L["k_pool"].astype(np.float64), v_pool=L["v_pool"].astype(np.float64),
+            qkv_bias=None if L.get("qkv_bias") is None else L["qkv_bias"].astype(np.float64))
             for L in layers]
         self.h = batch["h"].astype(np.float64)
         self.bt = batch["block_tables"]
         self.ctx = np.asarray(batch["context_lens"], np.int64)
+        self.cu = np.asarray(batch["cu_seqlens"], np.int64)
         self.final_norm = batch["final_norm"].astype(np.float64)
         self.trace = []
 
@@ -100,31 +104,40 @@ class DenseStep:
         c = self.cfg
         hq, hkv, d, inter = c["hq"], c["hkv"], c["d"], c["inter"]
         groups = hq // hkv
-        nseq = self.h.shape[0]
+        rows = self.h.shape[0]
+        nseq = len(self.ctx)
         for L in self.layers:
             xn = self.rb(self.norm(self.h, L["norm1"]))
             qkv = xn @ L["qkv"].T
-            attn = np.zeros((nseq, hq, d))
-            qs = np.zeros((nseq, hq, d))
+            if L.get("qkv_bias") is not None:
+                qkv = qkv + L["qkv_bias"]
+            attn = np.zeros((rows, hq, d))
+            qs = np.zeros((rows, hq, d))
             for s in range(nseq):
                 n_ctx = int(self.ctx[s])
-                pos = n_ctx - 1  # the new token is the last of its context
-                q = self.r16(rope_halves(qkv[s, :hq * d].reshape(hq, d), pos, self.theta, d))
-                k = self.r16(rope_halves(qkv[s, hq * d:(hq + hkv) * d].reshape(hkv, d), pos,
-                                         self.theta, d))
-                v = self.r16(qkv[s, (hq + hkv) * d:].reshape(hkv, d))
-                L["k_pool"][self.slot(s, pos)] = k.reshape(-1)
-                L["v_pool"][self.slot(s, pos)] = v.reshape(-1)
-                rows = [self.slot(s, p) for p in range(n_ctx)]
-                kc = L["k_pool"][rows].reshape(n_ctx, hkv, d)
-                vc = L["v_pool"][rows].reshape(n_ctx, hkv, d)
-                qs[s] = q
-                for hh in range(hq):
-                    g = hh // groups
-                    sc = (kc[:, g] @ q[hh]) / np.sqrt(np.float64(d))
-                    p = np.exp(sc - sc.max())
-                    attn[s, hh] = (p / p.sum()) @ vc[:, g]
-            o = self.rb(attn.reshape(nseq, hq * d)) @ L["o"].T
+                r0, r1 = int(self.cu[s]), int(self.cu[s + 1])
+                n_new = r1 - r0  # the new tokens are the last n_new of the context
+                # RoPE on q and k by position, then K / V into the cache
+                # (attention.rs:199-216), for every new token of the sequence
+                for i in range(n_new):
+                    t, pos = r0 + i, n_ctx - n_new + i
+                    qs[t] = self.r16(rope_halves(qkv[t, :hq * d].reshape(hq, d), pos, self.theta, d))
+                    k = self.r16(rope_halves(qkv[t, hq * d:(hq + hkv) * d].reshape(hkv, d), pos,
+                                             self.theta, d))
+                    v = self.r16(qkv[t, (hq + hkv) * d:].reshape(hkv, d))
+                    L["k_pool"][self.slot(s, pos)] = k.reshape(-1)
+                    L["v_pool"][self.slot(s, pos)] = v.reshape(-1)
+                for i in range(n_new):
+                    t, pos = r0 + i, n_ctx - n_new + i
+                    slots = [self.slot(s, p) for p in range(pos + 1)]  # causal: keys 0..pos
+                    kc = L["k_pool"][slots].reshape(pos + 1, hkv, d)
+                    vc = L["v_pool"][slots].reshape(pos + 1, hkv, d)
+                    for hh in range(hq):
+                        g = hh // groups
+                        sc = (kc[:, g] @ qs[t, hh]) / np.sqrt(np.float64(d))
+                        p = np.exp(sc - sc.max())
+                        attn[t, hh] = (p / p.sum()) @ vc[:, g]
+            o = self.rb(attn.reshape(rows, hq * d)) @ L["o"].T
             self.h = self.h + o
             xn2 = self.rb(self.norm(self.h, L["norm2"]))
             gu = xn2 @ L["gate_up"].T
@@ -132,7 +145,7 @@ class DenseStep:
             act = self.rb(gate / (1.0 + np.exp(-gate)) * up)
             down = act @ L["down"].T
             self.h = self.h + down
-            self.trace.append(dict(xn=xn, qkv=qkv, q=qs, attn=attn.reshape(nseq, -1), o=o,
+            self.trace.append(dict(xn=xn, qkv=qkv, q=qs, attn=attn.reshape(rows, -1), o=o,
                                    xn2=xn2, gu=gu, act=act, down=down, h=self.h.copy()))
         return self.rb(self.norm(self.h, self.final_norm))
 
@@ -140,10 +153,10 @@ class DenseStep:
 THETA = 1e6
 
 
-def _problem(seed, ctx, num_layers=2, hidden=256, hq=4, hkv=2, inter=384):
+def _problem(seed, ctx, num_layers=2, hidden=256, hq=4, hkv=2, inter=384, **kw):
     rng = np.random.default_rng(seed)
     return workloads.decode_step_problem(rng, num_layers=num_layers, hidden=hidden, hq=hq,
-                                         hkv=hkv, inter=inter, ctx=ctx, theta=THETA)
+                                         hkv=hkv, inter=inter, ctx=ctx, theta=THETA, **kw)
 
 
 def _oracle(cfg, layers, batch, trace=None):
@@ -198,6 +211,38 @@ def test_step_matches_float64_dense_composition_stage_by_stage():
     for L, R in zip(lay, ref.layers):
         _close(L["k_pool"].astype(np.float64), R["k_pool"], 2e-3, 1e-3, "K pool after the step")
         _close(L["v_pool"].astype(np.float64), R["v_pool"], 2e-3, 1e-3, "V pool after the step")
+
+
+def test_mixed_batch_with_qkv_bias_matches_float64_dense_composition():
+    """A mixed chunked-prefill + decode batch (packed rows, causal inside a chunk) whose
+    q/k/v projections carry a bias (attention.rs:49-57): the same stage-by-stage check."""
+    ctx = [9, 40, 3, 21]
+    new = [1, 7, 3, 5]  # decode row, a chunk with prior context, a whole short prompt, a chunk
+    cfg, layers, batch = _problem(111, ctx=ctx, new_tokens=new, qkv_bias=True)
+    assert batch["h"].shape[0] == 16 and list(batch["cu_seqlens"]) == [0, 1, 8, 11, 16]
+    assert list(batch["positions"][1:8]) == list(range(33, 40))
+    trace = []
+    out, lay, bat = _oracle(cfg, layers, batch, trace=trace)
+    ref = DenseStep(cfg, layers, batch, THETA, rounding=True)
+    want = ref.run()
+    for li, (t, r) in enumerate(zip(trace, ref.trace)):
+        _close(t["qkv"], r["qkv"], 2e-4, 2e-4, f"layer {li} qkv + bias")
+        _close(t["q"].astype(np.float64), r["q"], 4e-3, 1e-3, f"layer {li} roped q")
+        _close(t["attn"].reshape(r["attn"].shape), r["attn"], 1e-3, 1e-3, f"layer {li} attn")
+        _close(t["down"], r["down"], 2e-4, 1e-3, f"layer {li} down projection")
+    assert np.linalg.norm(out - want) / np.linalg.norm(want) < 1e-3
+    for L, R in zip(lay, ref.layers):
+        _close(L["k_pool"].astype(np.float64), R["k_pool"], 4e-3, 1e-3, "K pool after the step")
+    # the bias is in the projection (not dropped, not added twice): without it the result moves
+    nb = [dict(L, qkv_bias=None) for L in layers]
+    out_nb, _, _ = _oracle(cfg, nb, batch)
+    assert np.abs(out_nb - out).max() > 1e-2
+    # causal inside a chunk: the first token of the 7-token chunk does not see the later six;
+    # changing the LAST token's hidden row leaves the earlier rows of the chunk untouched
+    b2 = dict(batch, h=batch["h"].copy())
+    b2["h"][7] += 1.0
+    out2, _, _ = _oracle(cfg, layers, b2)
+    assert np.array_equal(out2[1:7], out[1:7]) and not np.array_equal(out2[7], out[7])
 
 
 def test_step_rounding_points_cost_what_bf16_and_fp16_cost():

@@ -173,6 +173,52 @@ def test_qgemm_q4_matches_float64_bruteforce():
     assert (np.abs(y - y64) <= np.abs(y64) * 2.0**-8 + 1e-6).all()
 
 
+def test_quantized_products_with_bias_equal_linear_t_with_bias():
+    """`linear_t(a, b, Some(bias), m, n, k)` (crates/kernels/src/cpu_f32/mod.rs:271-345, pinned
+    by cpu_f32/tests.rs:46-63,84-92 on the oracle's linear_t): the quantized products with a
+    bias are that function over the dequantised matrix -- the bias is added to the finished
+    fp32 sum, once per output, the same vector for every row."""
+    rng = np.random.default_rng(23)
+    b, n, k = 3, 19, 256
+    w = rng.normal(0, 0.02, size=(n, k)).astype(np.float32)
+    bias = rng.normal(size=n).astype(np.float32)
+    x = rng.normal(size=(b, k)).astype(np.float32)
+    # Q8G32, m = 1: bit-identical to linear_t with the bias (same ascending-k sum, one add)
+    qs, d = O.quantize_q8g32(w, n, k)
+    wd8 = O.dequantize_q8g32(qs, d, n, k)
+    assert np.array_equal(O.qgemv_q8g32_f32(x[0], qs, d, n, k, bias),
+                          O.linear_t(x[0], wd8, bias, 1, n, k))
+    # the reference's hand-computed case (tests.rs:84-92) through the quantized path: weights
+    # that Q8G32 holds exactly
+    w_exact = np.zeros((2, 32), np.float32)
+    w_exact[0, 0] = 1.0
+    w_exact[1, 1] = w_exact[1, 2] = 1.0
+    qe, de = O.quantize_q8g32(w_exact, 2, 32)
+    xe = np.zeros(32, np.float32)
+    xe[:3] = [1.0, 2.0, 3.0]
+    ye = O.qgemv_q8g32_f32(xe, qe, de, 2, 32, [10.0, 20.0])
+    assert abs(ye[0] - 11.0) < 1e-2 and abs(ye[1] - 25.0) < 1e-2  # d = 1/127 in fp16
+    # Q4G128 and Q4G32, m = 3: float64 brute force, bias before the bf16 rounding
+    x_bits = O.f32_to_bf16_bits(x)
+    xb = O.bf16_bits_to_f32(x_bits).astype(np.float64)
+    qw, s, z = O.quantize_q4g128(w, n, k)
+    wd4 = O.dequantize_q4g128(qw, s, z, n, k).astype(np.float64)
+    y64 = xb @ wd4.T + bias.astype(np.float64)
+    yf = O.qgemm_q4g128_f32(x_bits, qw, s, z, b, n, k, bias)
+    assert np.abs(yf - y64).max() < 2e-5
+    yb = O.bf16_bits_to_f32(O.qgemm_q4g128_bf16(x_bits, qw, s, z, b, n, k, bias))
+    assert (np.abs(yb - y64) <= np.abs(y64) * 2.0**-8 + 1e-6).all()
+    # without a bias nothing changes, and the bias is not applied twice or per group
+    assert np.array_equal(O.qgemm_q4g128_f32(x_bits, qw, s, z, b, n, k, None),
+                          O.qgemm_q4g128_f32(x_bits, qw, s, z, b, n, k))
+    assert np.abs((yf - O.qgemm_q4g128_f32(x_bits, qw, s, z, b, n, k)) - bias).max() < 1e-6
+    blocks = O.quantize_q4_blocks(w, n, k, True)
+    q32, s32, m32 = O.q4_blocks_to_q4g32(blocks, n, k, True)
+    wd32 = O.dequantize_q4g32(q32, s32, m32, n, k).astype(np.float64)
+    y32 = O.qgemm_q4g32_f32(x_bits, q32, s32, m32, b, n, k, bias)
+    assert np.abs(y32 - (xb @ wd32.T + bias)).max() < 2e-5
+
+
 # ------------------------------------------------------------------ ragged packing
 def test_pack_ragged_closed_forms():
     rng = np.random.default_rng(31)

@@ -137,8 +137,11 @@ def qgemm_q4_algorithmic_bytes(b, n, k) -> int:
 
 def decode_step_problem(rng, num_layers, hidden, hq, hkv, inter, ctx, d=128, block_size=16,
                         max_pos=None, eps=1e-6, theta=1e6, random_nibbles=False, vocab=0,
-                        kv_turbo3=False):
-    """A decode-step problem: `ctx[s]` is the context of sequence s INCLUDING the new token.
+                        kv_turbo3=False, new_tokens=None, qkv_bias=False):
+    """A decode-step problem: `ctx[s]` is the context of sequence s INCLUDING its new tokens
+    (one per sequence, or `new_tokens[s]` for a mixed chunked-prefill + decode batch: the batch
+    then has sum(new_tokens) packed rows).  qkv_bias: every layer's q/k/v projection carries a
+    bias ~N(0,1).
     Weights ~N(0,0.02) quantised to Q4G128 by the oracle (or raw random nibbles/scales when
     random_nibbles, for timing-only runs), RMSNorm gains 1+N(0,0.02), RoPE theta 1e6.
     With vocab > 0 the batch also carries token ids, a bf16 embedding table and a Q4G128
@@ -146,7 +149,9 @@ def decode_step_problem(rng, num_layers, hidden, hq, hkv, inter, ctx, d=128, blo
     (uint8 [rows][hkv*56]) holding the encoded random rows."""
     import oracle as O
     ctx = np.asarray(ctx, np.int32)
-    b = len(ctx)
+    new = np.ones(len(ctx), np.int32) if new_tokens is None else np.asarray(new_tokens, np.int32)
+    assert len(new) == len(ctx) and (new >= 1).all() and (new <= ctx).all()
+    b = int(new.sum())  # packed rows
     max_pos = max_pos or int(ctx.max()) + 1
 
     def q4(n, k):
@@ -158,8 +163,8 @@ def decode_step_problem(rng, num_layers, hidden, hq, hkv, inter, ctx, d=128, blo
         w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
         return O.quantize_q4g128(w, n, k)
 
-    base = paged_case(rng, np.ones(b, np.int32), ctx - 1, hq=hq, hkv=hkv, d=d,
-                      block_size=block_size, spare_frac=0.05)
+    base = paged_case(rng, new, ctx - new, hq=hq, hkv=hkv, d=d, block_size=block_size,
+                      spare_frac=0.05)
     layers = []
     for _ in range(num_layers):
         rows = base["k_pool"].shape[0]
@@ -170,14 +175,17 @@ def decode_step_problem(rng, num_layers, hidden, hq, hkv, inter, ctx, d=128, blo
             gate_up=q4(2 * inter, hidden), down=q4(hidden, inter),
             k_pool=rng.standard_normal((rows, hkv * d), np.float32).astype(np.float16),
             v_pool=rng.standard_normal((rows, hkv * d), np.float32).astype(np.float16)))
+        if qkv_bias:
+            layers[-1]["qkv_bias"] = rng.standard_normal((hq + 2 * hkv) * d).astype(np.float32)
     # the RoPE tables cover every position the block tables can hold
     max_pos = max(max_pos, block_size * base["block_tables"].shape[1])
     cos, sin = O.build_rope_table_f32(max_pos, d, theta)
-    cu, slots, ctx_lens, _ = O.pack_ragged(np.ones(b, np.int32), ctx - 1, base["block_tables"],
-                                           block_size)
+    cu, slots, ctx_lens, _ = O.pack_ragged(new, ctx - new, base["block_tables"], block_size)
+    # position of packed row t: prior context of its sequence + its index inside the chunk
+    positions = np.concatenate([np.arange(c - n, c) for c, n in zip(ctx, new)]).astype(np.int32)
     batch = dict(h=rng.standard_normal((b, hidden), np.float32),
                  block_tables=base["block_tables"], cu_seqlens=cu, context_lens=ctx_lens,
-                 positions=(ctx - 1).astype(np.int32), slots=slots, cos=cos, sin=sin,
+                 positions=positions, slots=slots, cos=cos, sin=sin,
                  final_norm=(1 + 0.02 * rng.standard_normal(hidden)).astype(np.float32))
     cfg = dict(hidden=hidden, hq=hq, hkv=hkv, d=d, inter=inter, eps=eps, block_size=block_size)
     if kv_turbo3:
