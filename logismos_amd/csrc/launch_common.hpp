@@ -59,4 +59,11 @@ hipError_t qgemm_q4_regx_launch(const RegxPlan& plan, const void* xprep, const v
                                 const void* scale, const void* zero, void* part, int b, int n,
                                 int k, hipStream_t stream);
 
+// Q4G128 GEMM for a tall x (qgemm_q4_tall.hip): 128 x 128 output tiles, x through LDS, the
+// matrix cores as the bound.  x bf16 [b][K], y bf16 [b][N], bias fp32 [N] or null.
+bool qgemm_q4_tall_applies(int b, int n, int k);
+hipError_t qgemm_q4_tall_launch(const void* x_bf16, const void* qw, const void* scale,
+                                const void* zero, const float* bias, void* y_bf16, int b, int n,
+                                int k, hipStream_t stream);
+
 }  // namespace lg

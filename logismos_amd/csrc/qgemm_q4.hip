@@ -478,10 +478,10 @@ static logismos_status_t qgemm_q4_dispatch32(const void* x_bf16, const void* qw_
     return lg::launch_mfma<2, 1>(x_bf16, qw_u8, scale_f16, zero_f16, y_bf16, bias, b, n, k, st);
 }
 
-// `linear_t` takes any m (crates/kernels/src/cpu_f32/mod.rs:271-345).  The kernels hold at
-// most 32 activation rows per workgroup, so a taller x is taken 32 rows at a time: every
-// launch streams the weights once (the prefill chunks of a mixed batch pass through the
-// quantized projections this way).
+// `linear_t` takes any m (crates/kernels/src/cpu_f32/mod.rs:271-345).  The decode kernels hold
+// at most 32 activation rows per workgroup, so a somewhat taller x is taken 32 rows at a time
+// (every launch streams the weights once); from about a hundred rows on (the prefill chunks
+// of a mixed batch) the tiled kernel of qgemm_q4_tall.hip takes over.
 static logismos_status_t qgemm_q4_dispatch(const void* x_bf16, const void* qw_u8,
                                            const void* scale_f16, const void* zero_f16,
                                            const void* bias_f32, void* y_bf16, int b, int n, int k,
@@ -492,6 +492,11 @@ static logismos_status_t qgemm_q4_dispatch(const void* x_bf16, const void* qw_u8
         return hipErrorInvalidValue;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const float* bias = static_cast<const float*>(bias_f32);
+    // many rows: the tiled kernel, one pass over the weights per 128 rows of x and the matrix
+    // cores as its bound
+    if (!force_mfma && lg::qgemm_q4_tall_applies(b, n, k))
+        return lg::qgemm_q4_tall_launch(x_bf16, qw_u8, scale_f16, zero_f16, bias, y_bf16, b, n, k,
+                                        st);
     for (int m0 = 0; m0 < b; m0 += 32) {
         const int rows = b - m0 < 32 ? b - m0 : 32;
         const logismos_status_t e = qgemm_q4_dispatch32(

@@ -139,3 +139,37 @@ def test_q4g32_tall_x():
     assert_parity(O.bf16_bits_to_f32(d_yb.to_numpy(np.uint16, (b, n))),
                   O.bf16_bits_to_f32(O.qgemm_q4g32_bf16(xb, q32, s32, m32, b, n, k)),
                   what="q4g32 gemm m = 83")
+
+
+@pytest.mark.parametrize("b,n,k,with_bias", [(97, 128, 128, False), (130, 200, 256, True),
+                                             (257, 1000, 1152, True), (300, 4100, 4096, False),
+                                             (1000, 333, 2048, True)])
+def test_q4g128_tiled_kernel_ragged_shapes(b, n, k, with_bias):
+    # the 128 x 128-tile kernel that serves tall x: partial tiles in rows and in weight rows,
+    # K of one group and of an odd number of groups, with and without a bias
+    rng = np.random.default_rng(b + 7 * n + 13 * k)
+    qw, s, z = _q4(rng, n, k)
+    xb = O.f32_to_bf16_bits(rng.standard_normal((b, k), np.float32))
+    bias = rng.standard_normal(n).astype(np.float32) if with_bias else None
+    got = _gemm_q4(xb, qw, s, z, b, n, k, bias)
+    want = O.bf16_bits_to_f32(O.qgemm_q4g128_bf16(xb, qw, s, z, b, n, k, bias))
+    assert_parity(got, want, what=f"q4g128 tiled {b}x{n}x{k}")
+
+
+def test_q4g128_tiled_kernel_one_hot_rows_read_back_dequantised_columns():
+    # orientation, nibble order, pair order of x and the zero-point term in one exact check:
+    # row i of x is the unit vector of column c_i, so row i of y is column c_i of the
+    # dequantised matrix (one product, one rounding)
+    rng = np.random.default_rng(10)
+    b, n, k = 256, 160, 384
+    w = rng.standard_normal((n, k), np.float32)
+    qw, s, z = O.quantize_q4g128(w, n, k)
+    wd = O.dequantize_q4g128(qw, s, z, n, k)
+    cols = rng.integers(0, k, size=b)
+    cols[:8] = [0, 1, 4, 7, 8, 63, 64, 127]
+    x = np.zeros((b, k), np.float32)
+    x[np.arange(b), cols] = 1.0
+    got = _gemm_q4(O.f32_to_bf16_bits(x), qw, s, z, b, n, k, None)
+    want = O.bf16_bits_to_f32(O.f32_to_bf16_bits(wd[:, cols].T.copy()))
+    # (128 + q) - (128 + zero) in fp32, times scale: the same value the oracle rounds
+    assert_parity(got, want, max_abs=1e-6, max_rel=4e-3, what="one-hot rows")
