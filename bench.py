@@ -424,6 +424,51 @@ def bench_q4(args):
     return {"workload": "config 3: Q4G128 GEMV/GEMM 12288x4096, x bf16, cold weights", **out}
 
 
+def bench_q4_tall(args):
+    """Config 4's packed token buffer (48 decode rows + 16 x 512 prefill rows = 8240 rows) through
+    one layer's four Q4G128 projections at Qwen3-8B geometry: `linear_t` at m = 8240 on the
+    tiled matrix-core kernel.  MFMA-bound by construction (arithmetic intensity ~4000 flop per
+    weight byte); reported against the dense bf16 peak."""
+    import oracle as O
+    stream = hip.Stream()
+    rng = np.random.default_rng(workloads.SEED + 40)
+    b = 8240
+    shapes = [("qkv", 6144, 4096), ("o", 4096, 4096), ("gate_up", 24576, 4096),
+              ("down", 4096, 12288)]
+    out, flops_all, ms_all = {}, 0.0, 0.0
+    parity = None
+    for name, n, k in shapes:
+        qw = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+        s = (rng.random((n, k // 128), np.float32) * 0.004 + 0.004).astype(np.float16)
+        z = (rng.random((n, k // 128), np.float32) * 2 + 6.5).astype(np.float16)
+        xb = O.f32_to_bf16_bits(rng.standard_normal((b, k), np.float32))
+        d = [hip.DeviceBuffer.from_numpy(a) for a in (xb, qw, s.view(np.uint16), z.view(np.uint16))]
+        dy = hip.DeviceBuffer(b * n * 2)
+        fn = lambda: kernels.launch_qgemm_q4g128_bf16(d[0], d[1], d[2], d[3], dy, b, n, k, stream)  # noqa: E731
+        ms, _, _ = time_launches(stream, [fn], 10, 2)
+        if name == "o":
+            # parity of what is being timed: a sample of rows against the oracle
+            rows = np.r_[0:4, 4111:4115, 8236:8240]
+            got = O.bf16_bits_to_f32(dy.to_numpy(np.uint16, (b, n))[rows])
+            want = O.bf16_bits_to_f32(O.qgemm_q4g128_bf16(xb[rows], qw, s, z, len(rows), n, k))
+            parity = float(np.abs(got - want).max())
+        flops = 2.0 * b * n * k
+        flops_all += flops
+        ms_all += ms
+        out[name] = {"n": n, "k": k, "us": round(ms * 1e3, 1),
+                     "TFLOPs": round(flops / ms / 1e9, 1)}
+        del d, dy
+    return {"workload": "config 4's 8240 packed rows through one layer's Q4G128 projections "
+                        "(qkv 6144x4096, o 4096x4096, gate_up 24576x4096, down 4096x12288)",
+            "kernel": "qgemm_q4g128_tall_kernel (128x128 tiles, v_mfma_f32_32x32x16_bf16)",
+            "projections": out, "ms_per_layer": round(ms_all, 4),
+            "roofline": {"bound": "mfma", "achieved": round(flops_all / ms_all / 1e9, 1),
+                         "peak": 2500.0, "unit": "TFLOP/s",
+                         "frac": round(flops_all / ms_all / 1e9 / 2500.0, 4), "traffic": None,
+                         "flops_per_layer": flops_all},
+            "parity_max_abs_vs_oracle_sample": parity}
+
+
 def bench_decode_step(args):
     """Config 5: full decode step, Qwen3-8B-style geometry, 32 live sequences."""
     import oracle as O
@@ -716,7 +761,8 @@ def main():
                          "with embedding, lm_head + greedy; the step over turbo3 KV pools); not "
                          "part of the metric, and not for runs under a profiler")
     ap.add_argument("--workload", default="all",
-                    choices=["all", "step", "config1", "config2", "config3", "config4"],
+                    choices=["all", "step", "config1", "config2", "config3", "config4",
+                             "config4_gemm"],
                     help="all: the decode-step line with every leg inside it (default); "
                          "otherwise only that workload's own JSON line")
     args = ap.parse_args()
@@ -729,11 +775,11 @@ def main():
     kernels.library()
     args.steps_c5 = args.steps if args.steps is not None else 20
     args.warmup_c5 = args.warmup if args.warmup is not None else 3
-    if args.workload in ("config1", "config2", "config3", "config4"):
+    if args.workload in ("config1", "config2", "config3", "config4", "config4_gemm"):
         args.steps = args.steps if args.steps is not None else 200
         args.warmup = args.warmup if args.warmup is not None else 20
         leg = {"config1": bench_qgemv_q8, "config2": bench_paged_decode, "config3": bench_q4,
-               "config4": bench_mixed_config4}[args.workload]
+               "config4": bench_mixed_config4, "config4_gemm": bench_q4_tall}[args.workload]
         print(json.dumps(leg(args)))
         return
     line = bench_decode_step(args)
@@ -747,6 +793,7 @@ def main():
         line["paged_attn_turbo3_config5"] = bench_turbo3(args)
         line["qgemv_q8_config1"] = bench_qgemv_q8(args)
         line["qgemm_q4_config3"] = bench_q4(args)
+        line["qgemm_q4_tall_config4_rows"] = bench_q4_tall(args)
     print(json.dumps(line))
 
 

@@ -628,10 +628,11 @@ typedef struct {
     /* A mixed batch (chunked prefill + decode): total_tokens = cu_seqlens[num_seqs] packed
      * rows and the largest number of new tokens of a sequence; 0 / 0 means one new token per
      * sequence.  Every per-row array above (hidden_f32, out_bf16, positions, slot_mapping) then
-     * has total_tokens rows, in packed order.  Rows go through the projections 32 at a time,
-     * every pass streaming the layer's weights once (`linear_t` over `seq` rows,
-     * crates/transformers/src/mlp.rs:104-111); the attention takes the whole ragged batch in
-     * one launch.  token_ids / lm_head need total_tokens <= 32. */
+     * has total_tokens rows, in packed order.  Up to 96 rows go through the projections 32 at
+     * a time, every pass streaming the layer's weights once; from 97 rows on every projection
+     * is one launch of the tiled matrix-core GEMM over all rows (`linear_t` over `seq` rows,
+     * crates/transformers/src/mlp.rs:104-111).  The attention takes the whole ragged batch in
+     * one launch either way.  token_ids / lm_head need total_tokens <= 32. */
     int total_tokens;
     int max_seqlen_q;
 } logismos_decode_batch_t;

@@ -11,6 +11,10 @@ namespace {
 
 constexpr int kChunkRows = 32;  // rows the prepared layout and the decode GEMMs hold
 
+// A step with this many packed rows or more takes the projections on the tiled GEMM (plain bf16
+// activations, fp32 products for the whole batch at once) instead of 32-row chunks.
+constexpr int kTallRows = 97;
+
 struct Workspace {
     char* xn;        // prepared activations of width hidden, one per 32-row chunk (input of qkv /
                      // gate_up; a chunk's buffer carries its normed rows from the end of one
@@ -25,6 +29,13 @@ struct Workspace {
     char* act;       // prepared activations of width inter (input of the down projection)
     char* attn_ws;   // split-K workspace of the attention
     char* head_ws;   // per-workgroup candidates of the token selection (vocab > 0)
+    // many-row steps (tall): plain buffers for all T rows
+    char* t_xn;    // bf16 [T][hidden]
+    char* t_qkv;   // f32  [T][(hq+2hkv)*d]
+    char* t_proj;  // f32  [T][hidden]
+    char* t_gu;    // f32  [T][2*inter]
+    char* t_act;   // bf16 [T][inter]
+    bool tall;
     size_t xn_stride;
     int chunks, rows;  // rows: rows of a full chunk (= T when there is one chunk)
     int j_qkv, j_o, j_gu, j_down;
@@ -44,6 +55,20 @@ Workspace carve(const logismos_decode_config_t& c, int num_seqs, int t, int num_
     };
     const size_t qd = (size_t)c.num_q_heads * c.head_dim;
     const size_t kvd = (size_t)c.num_kv_heads * c.head_dim;
+    w.tall = t >= kTallRows;
+    if (w.tall) {
+        w.attn_ws = take(
+            logismos_paged_attn_workspace_bytes(num_seqs, c.num_q_heads, c.head_dim, num_splits));
+        w.t_xn = take((size_t)t * c.hidden * 2);
+        w.t_qkv = take((size_t)t * (qd + 2 * kvd) * 4);
+        w.q = take((size_t)t * qd * 2);
+        w.attn_out = take((size_t)t * qd * 2);
+        w.t_proj = take((size_t)t * c.hidden * 4);
+        w.t_gu = take((size_t)t * 2 * c.intermediate * 4);
+        w.t_act = take((size_t)t * c.intermediate * 2);
+        w.total = off;
+        return w;
+    }
     w.chunks = (t + kChunkRows - 1) / kChunkRows;
     w.rows = t < kChunkRows ? t : kChunkRows;
     const int b = w.rows;
@@ -102,6 +127,15 @@ bool config_ok(const logismos_decode_config_t* c, int num_seqs, int t, int max_s
     const int b = t < kChunkRows ? t : kChunkRows;
     const int qd = c->num_q_heads * c->head_dim;
     const int kvd = c->num_kv_heads * c->head_dim;
+    if (t >= kTallRows) {
+        // the tiled GEMM's own limits (the products of the whole batch are held in fp32)
+        const int64_t lim = INT32_MAX;
+        const int64_t widest = 2 * (int64_t)c->intermediate > qd + 2 * kvd
+                                   ? 2 * (int64_t)c->intermediate
+                                   : (int64_t)qd + 2 * kvd;
+        return (int64_t)t * widest <= lim && (int64_t)widest * c->hidden <= lim &&
+               (int64_t)c->hidden * c->intermediate <= lim && c->hidden >= 128 && qd >= 128;
+    }
     if (logismos_qgemm_q4g128_splitk_xprep_parts(b, qd + 2 * kvd, c->hidden) <= 0 ||
         logismos_qgemm_q4g128_splitk_xprep_parts(b, c->hidden, qd) <= 0 ||
         logismos_qgemm_q4g128_splitk_xprep_parts(b, 2 * c->intermediate, c->hidden) <= 0 ||
@@ -174,6 +208,46 @@ extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_c
     if (tokens_in)
         LG_TRY(logismos_launch_embed_lookup_bf16(batch->embed_table_bf16, batch->token_ids,
                                                  batch->hidden_f32, t, c.hidden, c.vocab, stream));
+    if (w.tall) {
+        // ---- many rows: every projection is one launch of the tiled GEMM over all T rows
+        // (fp32 products, consumed un-rounded by the next operator as in the chunked path), the
+        // small operators run over all rows at once
+        hipStream_t st = static_cast<hipStream_t>(stream);
+        auto gemm = [&](const void* x_bf16, const logismos_q4_weight_t& W, const void* bias,
+                        void* y_f32, int n, int k) -> logismos_status_t {
+            return lg::qgemm_q4_tall_f32_launch(x_bf16, W.qw, W.scale, W.zero,
+                                                static_cast<const float*>(bias), y_f32, t, n, k, st);
+        };
+        int res_parts = 0;
+        for (int l = 0; l < c.num_layers; ++l) {
+            const logismos_decode_layer_t& L = layers[l];
+            LG_TRY(logismos_launch_add_rms_norm_f32p(batch->hidden_f32, w.t_proj, res_parts,
+                                                     L.norm1_w_f32, w.t_xn, t, c.hidden, c.rms_eps,
+                                                     stream));
+            LG_TRY(gemm(w.t_xn, L.qkv, nullptr, w.t_qkv, width, c.hidden));
+            const auto rope_kv_write = c.kv_turbo3 ? logismos_launch_rope_kv_write_f32p_turbo3_bias
+                                                   : logismos_launch_rope_kv_write_f32p_bias;
+            LG_TRY(rope_kv_write(w.t_qkv, 1, L.qkv_bias_f32, batch->positions, batch->rope_cos_f32,
+                                 batch->rope_sin_f32, batch->slot_mapping, w.q, L.k_pool_f16,
+                                 L.v_pool_f16, t, c.num_q_heads, c.num_kv_heads, c.head_dim,
+                                 c.max_pos, stream));
+            LG_TRY(lg::paged_attn_launch(
+                w.q, L.k_pool_f16, L.v_pool_f16, batch->block_tables, batch->cu_seqlens,
+                batch->context_lens, w.attn_out, w.attn_ws, num_seqs, t, max_q, c.num_q_heads,
+                c.num_kv_heads, c.head_dim, c.block_size, c.max_blocks_per_seq, batch->num_splits,
+                scale, 1, LOGISMOS_ATTN_PHASE_ALL, 1, c.kv_turbo3 ? 1 : 0, stream));
+            LG_TRY(gemm(w.attn_out, L.o, nullptr, w.t_proj, c.hidden, qd));
+            LG_TRY(logismos_launch_add_rms_norm_f32p(batch->hidden_f32, w.t_proj, 1, L.norm2_w_f32,
+                                                     w.t_xn, t, c.hidden, c.rms_eps, stream));
+            LG_TRY(gemm(w.t_xn, L.gate_up, nullptr, w.t_gu, 2 * c.intermediate, c.hidden));
+            LG_TRY(logismos_launch_silu_mul_f32p(w.t_gu, 1, w.t_act, t, c.intermediate, stream));
+            LG_TRY(gemm(w.t_act, L.down, nullptr, w.t_proj, c.hidden, c.intermediate));
+            res_parts = 1;
+        }
+        return logismos_launch_add_rms_norm_f32p(batch->hidden_f32, w.t_proj, res_parts,
+                                                 batch->final_norm_w_f32, batch->out_bf16, t,
+                                                 c.hidden, c.rms_eps, stream);
+    }
     // The normed input of a layer's first half is produced where the residual stream is
     // completed: before layer 0 here, afterwards by the add + norm that folds a chunk's down
     // projection into h (with the NEXT layer's gains).

@@ -65,5 +65,9 @@ bool qgemm_q4_tall_applies(int b, int n, int k);
 hipError_t qgemm_q4_tall_launch(const void* x_bf16, const void* qw, const void* scale,
                                 const void* zero, const float* bias, void* y_bf16, int b, int n,
                                 int k, hipStream_t stream);
+// ... with the fp32 product as output (the step executor keeps projections un-rounded)
+hipError_t qgemm_q4_tall_f32_launch(const void* x_bf16, const void* qw, const void* scale,
+                                    const void* zero, const float* bias, void* y_f32, int b,
+                                    int n, int k, hipStream_t stream);
 
 }  // namespace lg

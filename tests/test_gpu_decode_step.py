@@ -183,6 +183,17 @@ def test_mixed_batch_over_several_chunks_of_rows():
     _check_step(cfg, layers, batch, "mixed batch, three chunks", 2)
 
 
+def test_mixed_batch_with_many_rows_on_the_tiled_gemm():
+    # 1 + 100 + 3 + 1 + 37 = 142 packed rows: from 97 rows on every projection is one launch of
+    # the tiled GEMM over all rows; two layers, q/k/v bias, a ragged last tile (142 = 128 + 14)
+    rng = np.random.default_rng(42)
+    cfg, layers, batch = workloads.decode_step_problem(
+        rng, num_layers=2, hidden=512, hq=4, hkv=2, inter=1024, ctx=[700, 140, 3, 33, 37],
+        new_tokens=[1, 100, 3, 1, 37], qkv_bias=True)
+    assert batch["h"].shape[0] == 142
+    _check_step(cfg, layers, batch, "mixed batch, tiled GEMM", 2)
+
+
 def test_more_than_32_decode_sequences():
     rng = np.random.default_rng(39)
     ctx = rng.integers(1, 300, size=45)
