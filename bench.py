@@ -762,7 +762,7 @@ def main():
                          "part of the metric, and not for runs under a profiler")
     ap.add_argument("--workload", default="all",
                     choices=["all", "step", "config1", "config2", "config3", "config4",
-                             "config4_gemm"],
+                             "config4_gemm", "turbo3"],
                     help="all: the decode-step line with every leg inside it (default); "
                          "otherwise only that workload's own JSON line")
     args = ap.parse_args()
@@ -775,11 +775,12 @@ def main():
     kernels.library()
     args.steps_c5 = args.steps if args.steps is not None else 20
     args.warmup_c5 = args.warmup if args.warmup is not None else 3
-    if args.workload in ("config1", "config2", "config3", "config4", "config4_gemm"):
+    if args.workload in ("config1", "config2", "config3", "config4", "config4_gemm", "turbo3"):
         args.steps = args.steps if args.steps is not None else 200
         args.warmup = args.warmup if args.warmup is not None else 20
         leg = {"config1": bench_qgemv_q8, "config2": bench_paged_decode, "config3": bench_q4,
-               "config4": bench_mixed_config4, "config4_gemm": bench_q4_tall}[args.workload]
+               "config4": bench_mixed_config4, "config4_gemm": bench_q4_tall,
+               "turbo3": bench_turbo3}[args.workload]
         print(json.dumps(leg(args)))
         return
     line = bench_decode_step(args)

@@ -53,6 +53,12 @@ __device__ __forceinline__ float row_bcast(float v) {
     return dpp_f32<kDppRowNewBcast + N>(v);
 }
 
+// value held by lane N of each group of four lanes, broadcast to the four (quad_perm)
+template <int N>
+__device__ __forceinline__ float quad_bcast(float v) {
+    return dpp_f32<N | (N << 2) | (N << 4) | (N << 6)>(v);
+}
+
 // sum over each row of 16 lanes; every lane of the row gets the row total
 __device__ __forceinline__ float row16_sum(float v) {
     v += dpp_f32<kDppRowRor + 8>(v);

@@ -96,8 +96,9 @@ __device__ __forceinline__ unsigned short attn_out_elem(float v, int out_bf16) {
 // sum_j p_j v_j = H sum_j (p_j norm_j) c_j: the kernel transforms q once, works on the
 // centroid values themselves and transforms the result once.
 struct KvTileT3 {
-    unsigned k[4], v[4];  // 24 index bits (8 values) each, in bits 8..31
-    unsigned short kn[4], vn[4];
+    unsigned k[3];  // the 96 index bits of one 32-value block of a key
+    unsigned v[4];  // 24 index bits (8 values) each, in bits 8..31
+    unsigned short kn, vn;
 };
 
 // fp16 bits of `TURBO3_CODEBOOK` (RNE): b207 af90 ac43 a588 2588 2c43 2f90 3207; tables of
@@ -125,13 +126,40 @@ __device__ __forceinline__ half8_t turbo3_decode8(unsigned dword) {
     return __builtin_bit_cast(half8_t, o);
 }
 
+// The same through a 64-entry table in LDS: entry (i0 | i1 << 3) holds the fp16 pair
+// (centroid i0, centroid i1).  64 dwords are one per bank, so two lanes on one bank read one
+// address (a broadcast) and the lookup never conflicts; it costs two vector instructions per
+// pair where the byte permutes above cost 4.5.
+__device__ __forceinline__ unsigned turbo3_pair_entry(int i) {
+    constexpr unsigned long long lo = ((unsigned long long)kT3LoHi << 32) | kT3LoLo;
+    constexpr unsigned long long hi = ((unsigned long long)kT3HiHi << 32) | kT3HiLo;
+    const int i0 = i & 7, i1 = (i >> 3) & 7;
+    const unsigned h0 = (unsigned)((lo >> (8 * i0)) & 0xff) | ((unsigned)((hi >> (8 * i0)) & 0xff) << 8);
+    const unsigned h1 = (unsigned)((lo >> (8 * i1)) & 0xff) | ((unsigned)((hi >> (8 * i1)) & 0xff) << 8);
+    return h0 | (h1 << 16);
+}
+
+// FIRST = bit of `word` where the 24 index bits start (bits outside them are ignored)
+template <int FIRST>
+__device__ __forceinline__ half8_t turbo3_decode8_lds(unsigned word, const unsigned* table) {
+    uint4_t o;
+#pragma unroll
+    for (int pr = 0; pr < 4; ++pr) {
+        constexpr int kToByteOffset = 2;  // entry index -> byte offset
+        const int sh = FIRST + 6 * pr - kToByteOffset;
+        const unsigned off = (sh >= 0 ? word >> sh : word << -sh) & 0xFCu;
+        o[pr] = *reinterpret_cast<const unsigned*>(reinterpret_cast<const char*>(table) + off);
+    }
+    return __builtin_bit_cast(half8_t, o);
+}
+
 __device__ __forceinline__ unsigned load_u32_unaligned(const uint8_t* ptr) {
     unsigned v;
     __builtin_memcpy(&v, ptr, 4);
     return v;
 }
 
-// fwht_128 of a head held by the 4 lanes tg of a column as x[j][i] = element 8*(tg + 4j) + i
+// fwht_128 of a head held by the 4 lanes tg of a column as x[j][i] = element 8*(j + 4tg) + i
 __device__ __forceinline__ void fwht_pieces(float (&x)[4][8]) {
 #pragma unroll
     for (int j = 0; j < 4; ++j)
@@ -143,6 +171,17 @@ __device__ __forceinline__ void fwht_pieces(float (&x)[4][8]) {
                     const float a = x[j][i], b = x[j][i + h];
                     x[j][i] = a + b;
                     x[j][i + h] = a - b;
+                }
+#pragma unroll
+    for (int h = 1; h < 4; h <<= 1)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if ((j & h) == 0)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float a = x[j][i], b = x[j + h][i];
+                    x[j][i] = a + b;
+                    x[j + h][i] = a - b;
                 }
     const int lane = threadIdx.x & 63;
 #pragma unroll
@@ -156,17 +195,6 @@ __device__ __forceinline__ void fwht_pieces(float (&x)[4][8]) {
                 x[j][i] = hi ? o - x[j][i] : x[j][i] + o;
             }
     }
-#pragma unroll
-    for (int h = 1; h < 4; h <<= 1)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            if ((j & h) == 0)
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const float a = x[j][i], b = x[j + h][i];
-                    x[j][i] = a + b;
-                    x[j + h][i] = a - b;
-                }
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -316,18 +344,19 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
     const int c = lane & 15;
     const int ntiles = (tok_end - tok_begin + kTileKeys - 1) / kTileKeys;
 
-    // ---- query group as the MFMA B operand: column = head c, piece tg + 4j
+    // ---- query group as the MFMA B operand: column = head c
     half8_t qreg[4];
     {
         const half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
-        // contraction slot j of a lane row tg: piece tg + 4j (turbo3), or piece
-        // 2tg + (j & 1) + 8 (j >> 1) for fp16 pools, where K arrives as whole 128-byte lines
+        // contraction slot j of a lane row tg: piece 4tg + j for turbo3 pools (a lane row
+        // takes one 32-value block of every key), or piece 2tg + (j & 1) + 8 (j >> 1) for
+        // fp16 pools, where K arrives as whole 128-byte lines
         const _Float16* qp = p.q + ((int64_t)t * p.hq + kvh * G + (c < G ? c : 0)) * kHeadDim +
-                             (T3 ? 8 * tg : 16 * tg);
+                             (T3 ? 32 * tg : 16 * tg);
 #pragma unroll
         for (int j = 0; j < 4; ++j)
             qreg[j] = (c < G) ? *reinterpret_cast<const half8_t*>(
-                                    qp + (T3 ? 32 * j : 8 * (j & 1) + 64 * (j >> 1)))
+                                    qp + (T3 ? 8 * j : 8 * (j & 1) + 64 * (j >> 1)))
                               : z;
         if constexpr (T3) {
             float x[4][8];
@@ -356,10 +385,12 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
     for (int i = 0; i < 4; ++i) v_lane_off[i] = (unsigned)(4 * tg + i) * row_stride;
 
     using Tile = typename std::conditional<T3, KvTileT3, KvTile>::type;
-    // turbo3: byte offsets inside a tile (row stride = hkv * 56); a lane reads the dword
-    // that starts one byte before its 3-byte group, which never leaves the head row
+    // turbo3: byte offsets inside a tile (row stride = hkv * 56).  K: lane (tg, c) takes the
+    // 12 index bytes of block tg of key c in one request.  V: the dword that starts one byte
+    // before the lane's 3-byte group (it never leaves the head row).  Norms: lane (tg, c)
+    // fetches those of key 4tg + c % 4; compute_tile spreads them over the quad.
     const unsigned row_bytes = (unsigned)p.hkv * 56u;
-    const unsigned k3_piece = 14u * 0u + 1u + 3u * tg;                 // + 14 * j
+    const unsigned k3_piece = 14u * tg + 2u;
     const unsigned v3_piece = 14u * (c >> 2) + 1u + 3u * (c & 3);
     auto load_tile = [&](int tile, Tile& kv) {
         const int tok_base = __builtin_amdgcn_readfirstlane(tok_begin + tile * kTileKeys);
@@ -373,15 +404,15 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
             const uint8_t* vb = reinterpret_cast<const uint8_t*>(p.v_pool) + base;
             const unsigned last_off = (unsigned)(tok_end - 1 - tok_base) * row_bytes;
             const unsigned ko = min((unsigned)c * row_bytes, last_off) + k3_piece;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) kv.k[j] = load_u32_unaligned(kb + ko + 14u * j);
+            __builtin_memcpy(kv.k, kb + ko, 12);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const unsigned ro = min((unsigned)(4 * tg + i) * row_bytes, last_off);
                 kv.v[i] = load_u32_unaligned(vb + ro + v3_piece);
-                kv.kn[i] = *reinterpret_cast<const unsigned short*>(kb + ro);
-                kv.vn[i] = *reinterpret_cast<const unsigned short*>(vb + ro);
             }
+            const unsigned no = min((unsigned)(4 * tg + (c & 3)) * row_bytes, last_off);
+            kv.kn = *reinterpret_cast<const unsigned short*>(kb + no);
+            kv.vn = *reinterpret_cast<const unsigned short*>(vb + no);
             return;
         }
         const int64_t base = (row_base * p.hkv + kvh) * kHeadDim;
@@ -420,18 +451,38 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
     for (int h = 0; h < G; ++h)
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[h][e] = 0.0f;
+    // turbo3 pools: P.V on the matrix cores (the tile is bound by its vector instructions, and
+    // the 128 multiply-adds of P.V are the largest single item).  accp[e][r] = element 8c + e of
+    // head 4 tg + r: the C layout of v_mfma_f32_16x16x16_f16 with A = P (row = head, the four
+    // keys of this lane row), B_e = element e of the lane's eight values of each of its four
+    // keys (column = c).  The sum over all 16 keys of a tile is the MFMA's, so the four lane
+    // rows share one running maximum per head (m) and only the sums l are per row.
+    float4_t accp[T3 ? 8 : 1];
+    // centroid pairs for the decode: every wave writes all 64 entries (the same values), so a
+    // wave's reads are ordered behind its own writes and need no barrier
+    __shared__ unsigned t3_pairs[T3 ? 64 : 1];
+    if constexpr (T3) t3_pairs[lane] = turbo3_pair_entry(lane);
+#pragma unroll
+    for (int e = 0; e < (T3 ? 8 : 1); ++e) accp[e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
     auto compute_tile = [&](int tile, const Tile& raw) {
         KvTile kv;
         float kn[4], vn[4];
         if constexpr (T3) {
+            // groups 0..3 of the block start at bits 0, 24, 48 and 72 of its 96
+            kv.k[0] = turbo3_decode8_lds<0>(raw.k[0], t3_pairs);
+            kv.k[1] = turbo3_decode8_lds<0>(__builtin_amdgcn_alignbit(raw.k[1], raw.k[0], 24), t3_pairs);
+            kv.k[2] = turbo3_decode8_lds<0>(__builtin_amdgcn_alignbit(raw.k[2], raw.k[1], 16), t3_pairs);
+            kv.k[3] = turbo3_decode8_lds<8>(raw.k[2], t3_pairs);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                kv.k[j] = turbo3_decode8(raw.k[j]);
-                kv.v[j] = turbo3_decode8(raw.v[j]);
-                kn[j] = __half2float(__builtin_bit_cast(__half, raw.kn[j])) * p.scale_log2e;
-                vn[j] = __half2float(__builtin_bit_cast(__half, raw.vn[j]));
-            }
+            for (int j = 0; j < 4; ++j) kv.v[j] = turbo3_decode8_lds<8>(raw.v[j], t3_pairs);
+            const float kq = __half2float(__builtin_bit_cast(__half, raw.kn)) * p.scale_log2e;
+            const float vq = __half2float(__builtin_bit_cast(__half, raw.vn));
+            static_for<4>([&](auto rc) {
+                constexpr int r = decltype(rc)::value;
+                kn[r] = quad_bcast<r>(kq);
+                vn[r] = quad_bcast<r>(vq);
+            });
         } else {
             kv = raw;
             // lanes c < 8 keep key c (requests 0, 2) and take its odd pieces from lane c + 8;
@@ -461,8 +512,14 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const float sv = T3 ? sacc[r] * kn[r] : sacc[r] * p.scale_log2e;
-            sc[r] = (tok0 + r < tok_end) ? sv : -INFINITY;
+            // (turbo3: lanes beyond the group carry no head and must contribute P = 0)
+            sc[r] = (tok0 + r < tok_end && (!T3 || c < G)) ? sv : -INFINITY;
             mx = fmaxf(mx, sc[r]);
+        }
+        if constexpr (T3) {
+            // one maximum per head for all 16 keys: the lane rows hold four keys each
+            mx = fmaxf(mx, lane_xor_f32<16>(mx));
+            mx = fmaxf(mx, lane_xor_f32<32>(mx));
         }
         const float msafe = (mx == -INFINITY) ? 0.0f : mx;
         const float alpha = fast_exp2(m - msafe);
@@ -477,8 +534,38 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
         m = mx;
         if constexpr (T3) {
             // the value rows are unit-scale centroids: their norms ride on the probabilities
+            half4_t pa;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) pr[r] *= vn[r];
+            for (int r = 0; r < 4; ++r) pa[r] = (_Float16)(pr[r] * vn[r]);
+            // rescale: row r of the accumulators is head 4 tg + r, whose factor sits in lane
+            // c = 4 tg + r of every lane row
+            float ar[4];
+            static_for<4>([&](auto rc) {
+                constexpr int r = decltype(rc)::value;
+                if constexpr (G <= 4) {
+                    ar[r] = row_bcast<r>(alpha);  // rows tg > 0 hold no head: their P is zero
+                } else {
+                    const float lo = row_bcast<r>(alpha), hi = row_bcast<4 + r>(alpha);
+                    ar[r] = tg == 0 ? lo : hi;
+                }
+            });
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) accp[e][r] *= ar[r];
+                // B operand: element e of the eight values this lane holds of its four keys
+                const unsigned sel = (e & 1) ? 0x07060302u : 0x05040100u;
+                const uint4_t v0 = __builtin_bit_cast(uint4_t, kv.v[0]);
+                const uint4_t v1 = __builtin_bit_cast(uint4_t, kv.v[1]);
+                const uint4_t v2 = __builtin_bit_cast(uint4_t, kv.v[2]);
+                const uint4_t v3 = __builtin_bit_cast(uint4_t, kv.v[3]);
+                uint2_t bw;
+                bw[0] = __builtin_amdgcn_perm(v1[e >> 1], v0[e >> 1], sel);
+                bw[1] = __builtin_amdgcn_perm(v3[e >> 1], v2[e >> 1], sel);
+                accp[e] = __builtin_amdgcn_mfma_f32_16x16x16f16(
+                    pa, __builtin_bit_cast(half4_t, bw), accp[e], 0, 0, 0);
+            }
+            return;
         }
         static_for<G>([&](auto hc) {
             constexpr int h = decltype(hc)::value;
@@ -527,6 +614,17 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
     __builtin_amdgcn_s_setprio(0);
 
     // ---- merge the four rows of the wave, then write
+    if constexpr (T3) {
+        // the matrix cores have summed over all 16 keys of every tile: head h's row is complete
+        // in lane row h / 4, and the lane rows share m.  Put it in the form the merge below
+        // expects (every lane row a partial with its own sum): the row in lane row h / 4,
+        // zeros elsewhere; the per-row sums l add up to the full sum.
+        static_for<G>([&](auto hc) {
+            constexpr int h = decltype(hc)::value;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[h][e] = (tg == (h >> 2)) ? accp[e][h & 3] : 0.0f;
+        });
+    }
     static_for<G>([&](auto hc) {
         constexpr int h = decltype(hc)::value;
         float mh = row_bcast<h>(m);
