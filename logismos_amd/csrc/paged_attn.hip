@@ -96,8 +96,7 @@ __device__ __forceinline__ unsigned short attn_out_elem(float v, int out_bf16) {
 // sum_j p_j v_j = H sum_j (p_j norm_j) c_j: the kernel transforms q once, works on the
 // centroid values themselves and transforms the result once.
 struct KvTileT3 {
-    unsigned k[3];  // the 96 index bits of one 32-value block of a key
-    unsigned v[4];  // 24 index bits (8 values) each, in bits 8..31
+    unsigned k[3], v[3];  // the 96 index bits of one 32-value block of a key
     unsigned short kn, vn;
 };
 
@@ -386,12 +385,14 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
 
     using Tile = typename std::conditional<T3, KvTileT3, KvTile>::type;
     // turbo3: byte offsets inside a tile (row stride = hkv * 56).  K: lane (tg, c) takes the
-    // 12 index bytes of block tg of key c in one request.  V: the dword that starts one byte
-    // before the lane's 3-byte group (it never leaves the head row).  Norms: lane (tg, c)
-    // fetches those of key 4tg + c % 4; compute_tile spreads them over the quad.
+    // 12 index bytes of block tg of key c in one request.  V and the norms: lane (tg, c)
+    // fetches block c / 4 and the norms of key 4tg + c % 4; compute_tile spreads the norms
+    // over the four lanes c / 4 = const and transposes the block's four groups against the
+    // four keys there, which leaves group c % 4 of block c / 4 (values 8c .. 8c + 7) of the
+    // keys 4tg .. 4tg + 3 in the lane: the B operand of P.V.
     const unsigned row_bytes = (unsigned)p.hkv * 56u;
     const unsigned k3_piece = 14u * tg + 2u;
-    const unsigned v3_piece = 14u * (c >> 2) + 1u + 3u * (c & 3);
+    const unsigned v3_piece = 14u * (c >> 2) + 2u;
     auto load_tile = [&](int tile, Tile& kv) {
         const int tok_base = __builtin_amdgcn_readfirstlane(tok_begin + tile * kTileKeys);
         const int blk_idx = tok_base / p.block_size;
@@ -405,12 +406,8 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
             const unsigned last_off = (unsigned)(tok_end - 1 - tok_base) * row_bytes;
             const unsigned ko = min((unsigned)c * row_bytes, last_off) + k3_piece;
             __builtin_memcpy(kv.k, kb + ko, 12);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const unsigned ro = min((unsigned)(4 * tg + i) * row_bytes, last_off);
-                kv.v[i] = load_u32_unaligned(vb + ro + v3_piece);
-            }
             const unsigned no = min((unsigned)(4 * tg + (c & 3)) * row_bytes, last_off);
+            __builtin_memcpy(kv.v, vb + no + v3_piece, 12);
             kv.kn = *reinterpret_cast<const unsigned short*>(kb + no);
             kv.vn = *reinterpret_cast<const unsigned short*>(vb + no);
             return;
@@ -465,26 +462,9 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
 #pragma unroll
     for (int e = 0; e < (T3 ? 8 : 1); ++e) accp[e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-    auto compute_tile = [&](int tile, const Tile& raw) {
-        KvTile kv;
-        float kn[4], vn[4];
-        if constexpr (T3) {
-            // groups 0..3 of the block start at bits 0, 24, 48 and 72 of its 96
-            kv.k[0] = turbo3_decode8_lds<0>(raw.k[0], t3_pairs);
-            kv.k[1] = turbo3_decode8_lds<0>(__builtin_amdgcn_alignbit(raw.k[1], raw.k[0], 24), t3_pairs);
-            kv.k[2] = turbo3_decode8_lds<0>(__builtin_amdgcn_alignbit(raw.k[2], raw.k[1], 16), t3_pairs);
-            kv.k[3] = turbo3_decode8_lds<8>(raw.k[2], t3_pairs);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) kv.v[j] = turbo3_decode8_lds<8>(raw.v[j], t3_pairs);
-            const float kq = __half2float(__builtin_bit_cast(__half, raw.kn)) * p.scale_log2e;
-            const float vq = __half2float(__builtin_bit_cast(__half, raw.vn));
-            static_for<4>([&](auto rc) {
-                constexpr int r = decltype(rc)::value;
-                kn[r] = quad_bcast<r>(kq);
-                vn[r] = quad_bcast<r>(vq);
-            });
-        } else {
-            kv = raw;
+    auto compute_tile = [&](int tile, const KvTile& raw) {
+        KvTile kv = raw;
+        {
             // lanes c < 8 keep key c (requests 0, 2) and take its odd pieces from lane c + 8;
             // lanes c >= 8 keep key c (requests 1, 3) and take its even pieces from lane c - 8
             constexpr int kRor8 = 0x128;  // row_ror:8
@@ -511,15 +491,8 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
         float mx = m;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const float sv = T3 ? sacc[r] * kn[r] : sacc[r] * p.scale_log2e;
-            // (turbo3: lanes beyond the group carry no head and must contribute P = 0)
-            sc[r] = (tok0 + r < tok_end && (!T3 || c < G)) ? sv : -INFINITY;
+            sc[r] = (tok0 + r < tok_end) ? sacc[r] * p.scale_log2e : -INFINITY;
             mx = fmaxf(mx, sc[r]);
-        }
-        if constexpr (T3) {
-            // one maximum per head for all 16 keys: the lane rows hold four keys each
-            mx = fmaxf(mx, lane_xor_f32<16>(mx));
-            mx = fmaxf(mx, lane_xor_f32<32>(mx));
         }
         const float msafe = (mx == -INFINITY) ? 0.0f : mx;
         const float alpha = fast_exp2(m - msafe);
@@ -532,41 +505,6 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
         }
         l = l * alpha + psum;
         m = mx;
-        if constexpr (T3) {
-            // the value rows are unit-scale centroids: their norms ride on the probabilities
-            half4_t pa;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) pa[r] = (_Float16)(pr[r] * vn[r]);
-            // rescale: row r of the accumulators is head 4 tg + r, whose factor sits in lane
-            // c = 4 tg + r of every lane row
-            float ar[4];
-            static_for<4>([&](auto rc) {
-                constexpr int r = decltype(rc)::value;
-                if constexpr (G <= 4) {
-                    ar[r] = row_bcast<r>(alpha);  // rows tg > 0 hold no head: their P is zero
-                } else {
-                    const float lo = row_bcast<r>(alpha), hi = row_bcast<4 + r>(alpha);
-                    ar[r] = tg == 0 ? lo : hi;
-                }
-            });
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) accp[e][r] *= ar[r];
-                // B operand: element e of the eight values this lane holds of its four keys
-                const unsigned sel = (e & 1) ? 0x07060302u : 0x05040100u;
-                const uint4_t v0 = __builtin_bit_cast(uint4_t, kv.v[0]);
-                const uint4_t v1 = __builtin_bit_cast(uint4_t, kv.v[1]);
-                const uint4_t v2 = __builtin_bit_cast(uint4_t, kv.v[2]);
-                const uint4_t v3 = __builtin_bit_cast(uint4_t, kv.v[3]);
-                uint2_t bw;
-                bw[0] = __builtin_amdgcn_perm(v1[e >> 1], v0[e >> 1], sel);
-                bw[1] = __builtin_amdgcn_perm(v3[e >> 1], v2[e >> 1], sel);
-                accp[e] = __builtin_amdgcn_mfma_f32_16x16x16f16(
-                    pa, __builtin_bit_cast(half4_t, bw), accp[e], 0, 0, 0);
-            }
-            return;
-        }
         static_for<G>([&](auto hc) {
             constexpr int h = decltype(hc)::value;
             const float a = row_bcast<h>(alpha);
@@ -586,45 +524,226 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
         });
     };
 
+    // turbo3 pools, two tiles (32 keys) at a time: one running-maximum update and one rescale
+    // of the accumulators for both, and the two tiles' independent decode -> score chains are
+    // there for the scheduler to interleave.
+    struct T3Decoded {
+        half8_t k[4], v[4];
+        float kn[4], vn[4];
+    };
+    auto t3_decode = [&](const KvTileT3& raw, T3Decoded& d) {
+        // groups 0..3 of a block start at bits 0, 24, 48 and 72 of its 96
+        d.k[0] = turbo3_decode8_lds<0>(raw.k[0], t3_pairs);
+        d.k[1] = turbo3_decode8_lds<0>(__builtin_amdgcn_alignbit(raw.k[1], raw.k[0], 24), t3_pairs);
+        d.k[2] = turbo3_decode8_lds<0>(__builtin_amdgcn_alignbit(raw.k[2], raw.k[1], 16), t3_pairs);
+        d.k[3] = turbo3_decode8_lds<8>(raw.k[2], t3_pairs);
+        // a[i] = group i of this lane's key; after the transpose, group c % 4 of key 4tg + i.
+        // Two butterfly steps (lanes c ^ 1, then c ^ 2): a lane keeps the registers whose
+        // index bit equals its own and trades the others.
+        const unsigned a[4] = {raw.v[0], __builtin_amdgcn_alignbit(raw.v[1], raw.v[0], 24),
+                               __builtin_amdgcn_alignbit(raw.v[2], raw.v[1], 16), raw.v[2] >> 8};
+        const bool o1 = (c & 1) != 0, o2 = (c & 2) != 0;
+        constexpr int kQuadXor1 = 0xB1, kQuadXor2 = 0x4E;  // quad_perm [1,0,3,2], [2,3,0,1]
+        const unsigned r0 = (unsigned)dpp_i32<kQuadXor1>((int)(o1 ? a[0] : a[1]));
+        const unsigned r1 = (unsigned)dpp_i32<kQuadXor1>((int)(o1 ? a[2] : a[3]));
+        const unsigned c0 = o1 ? r0 : a[0], c1 = o1 ? a[1] : r0;
+        const unsigned c2 = o1 ? r1 : a[2], c3 = o1 ? a[3] : r1;
+        const unsigned u0 = (unsigned)dpp_i32<kQuadXor2>((int)(o2 ? c0 : c2));
+        const unsigned u1 = (unsigned)dpp_i32<kQuadXor2>((int)(o2 ? c1 : c3));
+        d.v[0] = turbo3_decode8_lds<0>(o2 ? u0 : c0, t3_pairs);
+        d.v[1] = turbo3_decode8_lds<0>(o2 ? u1 : c1, t3_pairs);
+        d.v[2] = turbo3_decode8_lds<0>(o2 ? c2 : u0, t3_pairs);
+        d.v[3] = turbo3_decode8_lds<0>(o2 ? c3 : u1, t3_pairs);
+        const float kq = __half2float(__builtin_bit_cast(__half, raw.kn)) * p.scale_log2e;
+        const float vq = __half2float(__builtin_bit_cast(__half, raw.vn));
+        static_for<4>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            d.kn[r] = quad_bcast<r>(kq);
+            d.vn[r] = quad_bcast<r>(vq);
+        });
+    };
+    auto t3_compute_pair = [&](int tile, const KvTileT3& raw0, const KvTileT3& raw1) {
+        T3Decoded d[2];
+        t3_decode(raw0, d[0]);
+        t3_decode(raw1, d[1]);
+        float4_t sacc[2] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int x = 0; x < 2; ++x)
+                sacc[x] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d[x].k[j], qreg[j], sacc[x], 0, 0, 0);
+        const int tok0 = tok_begin + tile * kTileKeys + 4 * tg;
+        float sc[2][4];
+        float mx = m;
+#pragma unroll
+        for (int x = 0; x < 2; ++x)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                // lanes beyond the group carry no head and must contribute P = 0
+                sc[x][r] = (tok0 + kTileKeys * x + r < tok_end && c < G) ? sacc[x][r] * d[x].kn[r]
+                                                                          : -INFINITY;
+                mx = fmaxf(mx, sc[x][r]);
+            }
+        // one maximum per head for all 32 keys: the lane rows hold eight keys each
+        mx = fmaxf(mx, lane_xor_f32<16>(mx));
+        mx = fmaxf(mx, lane_xor_f32<32>(mx));
+        const float msafe = (mx == -INFINITY) ? 0.0f : mx;
+        const float alpha = fast_exp2(m - msafe);
+        float psum = 0.0f;
+        half4_t pa[2];
+#pragma unroll
+        for (int x = 0; x < 2; ++x)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float pr = fast_exp2(sc[x][r] - msafe);
+                psum += pr;
+                // the value rows are unit-scale centroids: their norms ride on the probabilities
+                pa[x][r] = (_Float16)(pr * d[x].vn[r]);
+            }
+        l = l * alpha + psum;
+        m = mx;
+        // rescale: row r of the accumulators is head 4 tg + r, whose factor sits in lane
+        // c = 4 tg + r of every lane row
+        float ar[4];
+        static_for<4>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            if constexpr (G <= 4) {
+                ar[r] = row_bcast<r>(alpha);  // rows tg > 0 hold no head: their P is zero
+            } else {
+                const float lo = row_bcast<r>(alpha), hi = row_bcast<4 + r>(alpha);
+                ar[r] = tg == 0 ? lo : hi;
+            }
+        });
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) accp[e][r] *= ar[r];
+#pragma unroll
+            for (int x = 0; x < 2; ++x) {
+                // B operand: element e of the eight values this lane holds of its four keys
+                const unsigned sel = (e & 1) ? 0x07060302u : 0x05040100u;
+                const uint4_t v0 = __builtin_bit_cast(uint4_t, d[x].v[0]);
+                const uint4_t v1 = __builtin_bit_cast(uint4_t, d[x].v[1]);
+                const uint4_t v2 = __builtin_bit_cast(uint4_t, d[x].v[2]);
+                const uint4_t v3 = __builtin_bit_cast(uint4_t, d[x].v[3]);
+                uint2_t bw;
+                bw[0] = __builtin_amdgcn_perm(v1[e >> 1], v0[e >> 1], sel);
+                bw[1] = __builtin_amdgcn_perm(v3[e >> 1], v2[e >> 1], sel);
+                accp[e] = __builtin_amdgcn_mfma_f32_16x16x16f16(
+                    pa[x], __builtin_bit_cast(half4_t, bw), accp[e], 0, 0, 0);
+            }
+        }
+    };
+
     // Register double buffer, two tiles per iteration in one straight-line
     // body: every iteration issues the same loads (the tile index is clamped;
     // a tile past the end re-reads the last one and is fully masked in
     // compute_tile), so the loads of the next tile stay in flight while the
     // current one is consumed and the wait counts stay exact.
     const int last_tile = ntiles - 1;
-    Tile buf0, buf1;
-    load_tile(0, buf0);
-    for (int tile = 0; tile < ntiles; tile += 2) {
-        // balanced kernel (long partitions): the two waves of a SIMD (w and w + 4) take turns
-        // at the higher issue priority, 16 tiles each: left alone the older wave wins every
-        // tie and the younger one finishes microseconds after it
+    // balanced kernel (long partitions): the two waves of a SIMD (w and w + 4) take turns
+    // at the higher issue priority, 16 tiles each: left alone the older wave wins every
+    // tie and the younger one finishes microseconds after it
+    auto take_turns = [&](int tile) {
         if (p.num_workers > 0 && (tile & 15) == 0) {
             if ((((tile >> 4) ^ (threadIdx.x >> 8)) & 1) != 0) __builtin_amdgcn_s_setprio(1);
             else __builtin_amdgcn_s_setprio(0);
         }
-        load_tile(min(tile + 1, last_tile), buf1);
-        __builtin_amdgcn_sched_barrier(0);  // keep the prefetch above the math
-        compute_tile(tile, buf0);
-        __builtin_amdgcn_sched_barrier(0);
-        load_tile(min(tile + 2, last_tile), buf0);
-        __builtin_amdgcn_sched_barrier(0);
-        compute_tile(tile + 1, buf1);
-        __builtin_amdgcn_sched_barrier(0);
+    };
+    if constexpr (T3) {
+        // the same with pairs of tiles
+        KvTileT3 a0, a1, b0, b1;
+        load_tile(0, a0);
+        load_tile(min(1, last_tile), a1);
+        for (int tile = 0; tile < ntiles; tile += 4) {
+            take_turns(tile);
+            load_tile(min(tile + 2, last_tile), b0);
+            load_tile(min(tile + 3, last_tile), b1);
+            __builtin_amdgcn_sched_barrier(0);
+            t3_compute_pair(tile, a0, a1);
+            __builtin_amdgcn_sched_barrier(0);
+            load_tile(min(tile + 4, last_tile), a0);
+            load_tile(min(tile + 5, last_tile), a1);
+            __builtin_amdgcn_sched_barrier(0);
+            if (tile + 2 < ntiles) t3_compute_pair(tile + 2, b0, b1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    } else {
+        KvTile buf0, buf1;
+        load_tile(0, buf0);
+        for (int tile = 0; tile < ntiles; tile += 2) {
+            take_turns(tile);
+            load_tile(min(tile + 1, last_tile), buf1);
+            __builtin_amdgcn_sched_barrier(0);  // keep the prefetch above the math
+            compute_tile(tile, buf0);
+            __builtin_amdgcn_sched_barrier(0);
+            load_tile(min(tile + 2, last_tile), buf0);
+            __builtin_amdgcn_sched_barrier(0);
+            compute_tile(tile + 1, buf1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
     __builtin_amdgcn_s_setprio(0);
 
-    // ---- merge the four rows of the wave, then write
-    if constexpr (T3) {
-        // the matrix cores have summed over all 16 keys of every tile: head h's row is complete
-        // in lane row h / 4, and the lane rows share m.  Put it in the form the merge below
-        // expects (every lane row a partial with its own sum): the row in lane row h / 4,
-        // zeros elsewhere; the per-row sums l add up to the full sum.
-        static_for<G>([&](auto hc) {
-            constexpr int h = decltype(hc)::value;
+    // ---- write head `h` (elements 8c .. 8c + 7 of it in x, running maximum mh, sum lh)
+    auto write_head = [&](int h, const float (&x)[8], float mh, float lh) {
+        const int head = kvh * G + h;
+        if (single) {
+            const float inv = 1.0f / lh;
+            uint4_t o;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[h][e] = (tg == (h >> 2)) ? accp[e][h & 3] : 0.0f;
+            for (int e = 0; e < 4; ++e)
+                o[e] = (unsigned)attn_out_elem(x[2 * e] * inv, p.out_bf16) |
+                       ((unsigned)attn_out_elem(x[2 * e + 1] * inv, p.out_bf16) << 16);
+            if (p.out_bf16 == 2) {
+                // a head is one group of 128: the 16 lanes of this row hold its 16 chunks
+                const float gs = row16_sum(sum8_bf16(o));
+                const int bp = xprep_bp(p.out_rows);
+                reinterpret_cast<uint4_t*>(p.out)[(int64_t)(head * 16 + c) * bp + t] = pair_order(o);
+                if (c == 0)
+                    reinterpret_cast<float*>(
+                        reinterpret_cast<char*>(p.out) +
+                        xprep_xg_offset(p.out_rows, p.hq * kHeadDim))[(int64_t)head * bp + t] = gs;
+            } else {
+                *reinterpret_cast<uint4_t*>(p.out + ((int64_t)t * p.hq + head) * kHeadDim + 8 * c) = o;
+            }
+        } else {
+            const int64_t idx = slot * p.hq + head;
+            float4_t a0 = {x[0], x[1], x[2], x[3]};
+            float4_t a1 = {x[4], x[5], x[6], x[7]};
+            float* dst = p.ws_acc + idx * kHeadDim + 8 * c;
+            *reinterpret_cast<float4_t*>(dst) = a0;
+            *reinterpret_cast<float4_t*>(dst + 4) = a1;
+            if (c == 0) {
+                p.ws_ml[idx * 2] = mh;
+                p.ws_ml[idx * 2 + 1] = lh;
+            }
+        }
+    };
+    if constexpr (T3) {
+        // the matrix cores have summed over all the keys: head 4tg + r is complete in row r of
+        // the accumulators of lane row tg, the lane rows share m, and the sums l of the four
+        // lane rows (four keys of every tile each) add up to the whole
+        float lsum = l + lane_xor_f32<16>(l);
+        lsum += lane_xor_f32<32>(lsum);
+        static_for<(G < 4 ? G : 4)>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            float x[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = accp[e][r];
+            fwht_row(x);  // back from the centroid domain
+            float mh = row_bcast<r>(m), lh = row_bcast<r>(lsum);
+            if constexpr (G > 4) {
+                const float mhi = row_bcast<4 + (r < G - 4 ? r : 0)>(m);
+                const float lhi = row_bcast<4 + (r < G - 4 ? r : 0)>(lsum);
+                mh = tg == 0 ? mh : mhi;
+                lh = tg == 0 ? lh : lhi;
+            }
+            if (4 * tg + r < G) write_head(4 * tg + r, x, mh, lh);
         });
+        return;
     }
+    // ---- fp16 pools: merge the four rows of the wave, then write
     static_for<G>([&](auto hc) {
         constexpr int h = decltype(hc)::value;
         float mh = row_bcast<h>(m);
@@ -644,43 +763,7 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
             }
             mh = mn;
         }
-        if constexpr (T3) fwht_row(acc[h]);  // back from the centroid domain (all rows alike)
-        if (tg == (h & 3)) {
-            const int head = kvh * G + h;
-            if (single) {
-                const float inv = 1.0f / lh;
-                uint4_t o;
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    o[e] = (unsigned)attn_out_elem(acc[h][2 * e] * inv, p.out_bf16) |
-                           ((unsigned)attn_out_elem(acc[h][2 * e + 1] * inv, p.out_bf16) << 16);
-                if (p.out_bf16 == 2) {
-                    // a head is one group of 128: the 16 lanes of this row hold its 16 chunks
-                    const float gs = row16_sum(sum8_bf16(o));
-                    const int bp = xprep_bp(p.out_rows);
-                    reinterpret_cast<uint4_t*>(p.out)[(int64_t)(head * 16 + c) * bp + t] =
-                        pair_order(o);
-                    if (c == 0)
-                        reinterpret_cast<float*>(
-                            reinterpret_cast<char*>(p.out) +
-                            xprep_xg_offset(p.out_rows, p.hq * kHeadDim))[(int64_t)head * bp + t] = gs;
-                } else {
-                    *reinterpret_cast<uint4_t*>(p.out + ((int64_t)t * p.hq + head) * kHeadDim +
-                                                8 * c) = o;
-                }
-            } else {
-                const int64_t idx = slot * p.hq + head;
-                float4_t a0 = {acc[h][0], acc[h][1], acc[h][2], acc[h][3]};
-                float4_t a1 = {acc[h][4], acc[h][5], acc[h][6], acc[h][7]};
-                float* dst = p.ws_acc + idx * kHeadDim + 8 * c;
-                *reinterpret_cast<float4_t*>(dst) = a0;
-                *reinterpret_cast<float4_t*>(dst + 4) = a1;
-                if (c == 0) {
-                    p.ws_ml[idx * 2] = mh;
-                    p.ws_ml[idx * 2 + 1] = lh;
-                }
-            }
-        }
+        if (tg == (h & 3)) write_head(h, acc[h], mh, lh);
     });
 }
 
