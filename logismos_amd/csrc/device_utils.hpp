@@ -38,13 +38,16 @@ __device__ __forceinline__ void static_for(F&& f) {
 constexpr int kDppRowRor = 0x120;       // + n, rotate right within a row of 16
 constexpr int kDppRowNewBcast = 0x150;  // + n, lane n of each row of 16 to the whole row
 
+// (every control used here reads a live lane for every lane, so the value a disabled or
+// unfed lane would keep is never needed: with none given, the compiler has no register to
+// clear before each of these and can fold them into the instruction that uses the result)
 template <int CTRL>
 __device__ __forceinline__ float dpp_f32(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xf, 0xf, true));
 }
 template <int CTRL>
 __device__ __forceinline__ int dpp_i32(int v) {
-    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false);
+    return __builtin_amdgcn_mov_dpp(v, CTRL, 0xf, 0xf, true);
 }
 
 // value held by lane (row_base + N) broadcast to its row of 16 lanes
