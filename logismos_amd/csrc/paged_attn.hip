@@ -125,10 +125,7 @@ __device__ __forceinline__ half8_t turbo3_decode8(unsigned dword) {
     return __builtin_bit_cast(half8_t, o);
 }
 
-// The same through a 64-entry table in LDS: entry (i0 | i1 << 3) holds the fp16 pair
-// (centroid i0, centroid i1).  64 dwords are one per bank, so two lanes on one bank read one
-// address (a broadcast) and the lookup never conflicts; it costs two vector instructions per
-// pair where the byte permutes above cost 4.5.
+// the fp16 pair (centroid i & 7, centroid (i >> 3) & 7)
 __device__ __forceinline__ unsigned turbo3_pair_entry(int i) {
     constexpr unsigned long long lo = ((unsigned long long)kT3LoHi << 32) | kT3LoLo;
     constexpr unsigned long long hi = ((unsigned long long)kT3HiHi << 32) | kT3HiLo;
@@ -138,17 +135,29 @@ __device__ __forceinline__ unsigned turbo3_pair_entry(int i) {
     return h0 | (h1 << 16);
 }
 
+// ... and through a 4096-entry table: entry (i0 | i1 << 3 | i2 << 6 | i3 << 9) holds the four
+// fp16 centroids, so eight values cost two lookups of two vector instructions each (the
+// byte permutes above: 18).  32 KB of LDS per workgroup, filled by all its threads; the
+// caller puts a barrier between the fill and the first lookup.
+constexpr int kT3QuadEntries = 4096;
+__device__ __forceinline__ void turbo3_fill_quads(uint2_t* table) {
+    for (int i = threadIdx.x; i < kT3QuadEntries; i += blockDim.x) {
+        uint2_t e;
+        e[0] = turbo3_pair_entry(i & 63);
+        e[1] = turbo3_pair_entry(i >> 6);
+        table[i] = e;
+    }
+}
 // FIRST = bit of `word` where the 24 index bits start (bits outside them are ignored)
 template <int FIRST>
-__device__ __forceinline__ half8_t turbo3_decode8_lds(unsigned word, const unsigned* table) {
-    uint4_t o;
-#pragma unroll
-    for (int pr = 0; pr < 4; ++pr) {
-        constexpr int kToByteOffset = 2;  // entry index -> byte offset
-        const int sh = FIRST + 6 * pr - kToByteOffset;
-        const unsigned off = (sh >= 0 ? word >> sh : word << -sh) & 0xFCu;
-        o[pr] = *reinterpret_cast<const unsigned*>(reinterpret_cast<const char*>(table) + off);
-    }
+__device__ __forceinline__ half8_t turbo3_decode8_lds(unsigned word, const uint2_t* table) {
+    constexpr int kToByteOffset = 3;  // entry index -> byte offset
+    constexpr int s0 = FIRST - kToByteOffset, s1 = FIRST + 12 - kToByteOffset;
+    const unsigned o0 = (s0 >= 0 ? word >> (s0 >= 0 ? s0 : 0) : word << (s0 < 0 ? -s0 : 0)) & 0x7FF8u;
+    const unsigned o1 = (word >> s1) & 0x7FF8u;
+    const uint2_t lo = *reinterpret_cast<const uint2_t*>(reinterpret_cast<const char*>(table) + o0);
+    const uint2_t hi = *reinterpret_cast<const uint2_t*>(reinterpret_cast<const char*>(table) + o1);
+    const uint4_t o = {lo[0], lo[1], hi[0], hi[1]};
     return __builtin_bit_cast(half8_t, o);
 }
 
@@ -337,7 +346,7 @@ __device__ __forceinline__ void attn_write_zero_row(const AttnParams& p, int t, 
 template <int G, bool T3>
 __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t, int kvh,
                                                int tok_begin, int tok_end, bool single,
-                                               int64_t slot) {
+                                               int64_t slot, const uint2_t* t3_quads) {
     const int lane = threadIdx.x & 63;
     const int tg = lane >> 4;
     const int c = lane & 15;
@@ -455,10 +464,6 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
     // keys (column = c).  The sum over all 16 keys of a tile is the MFMA's, so the four lane
     // rows share one running maximum per head (m) and only the sums l are per row.
     float4_t accp[T3 ? 8 : 1];
-    // centroid pairs for the decode: every wave writes all 64 entries (the same values), so a
-    // wave's reads are ordered behind its own writes and need no barrier
-    __shared__ unsigned t3_pairs[T3 ? 64 : 1];
-    if constexpr (T3) t3_pairs[lane] = turbo3_pair_entry(lane);
 #pragma unroll
     for (int e = 0; e < (T3 ? 8 : 1); ++e) accp[e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
@@ -533,10 +538,10 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
     };
     auto t3_decode = [&](const KvTileT3& raw, T3Decoded& d) {
         // groups 0..3 of a block start at bits 0, 24, 48 and 72 of its 96
-        d.k[0] = turbo3_decode8_lds<0>(raw.k[0], t3_pairs);
-        d.k[1] = turbo3_decode8_lds<0>(__builtin_amdgcn_alignbit(raw.k[1], raw.k[0], 24), t3_pairs);
-        d.k[2] = turbo3_decode8_lds<0>(__builtin_amdgcn_alignbit(raw.k[2], raw.k[1], 16), t3_pairs);
-        d.k[3] = turbo3_decode8_lds<8>(raw.k[2], t3_pairs);
+        d.k[0] = turbo3_decode8_lds<0>(raw.k[0], t3_quads);
+        d.k[1] = turbo3_decode8_lds<0>(__builtin_amdgcn_alignbit(raw.k[1], raw.k[0], 24), t3_quads);
+        d.k[2] = turbo3_decode8_lds<0>(__builtin_amdgcn_alignbit(raw.k[2], raw.k[1], 16), t3_quads);
+        d.k[3] = turbo3_decode8_lds<8>(raw.k[2], t3_quads);
         // a[i] = group i of this lane's key; after the transpose, group c % 4 of key 4tg + i.
         // Two butterfly steps (lanes c ^ 1, then c ^ 2): a lane keeps the registers whose
         // index bit equals its own and trades the others.
@@ -550,10 +555,10 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
         const unsigned c2 = o1 ? r1 : a[2], c3 = o1 ? a[3] : r1;
         const unsigned u0 = (unsigned)dpp_i32<kQuadXor2>((int)(o2 ? c0 : c2));
         const unsigned u1 = (unsigned)dpp_i32<kQuadXor2>((int)(o2 ? c1 : c3));
-        d.v[0] = turbo3_decode8_lds<0>(o2 ? u0 : c0, t3_pairs);
-        d.v[1] = turbo3_decode8_lds<0>(o2 ? u1 : c1, t3_pairs);
-        d.v[2] = turbo3_decode8_lds<0>(o2 ? c2 : u0, t3_pairs);
-        d.v[3] = turbo3_decode8_lds<0>(o2 ? c3 : u1, t3_pairs);
+        d.v[0] = turbo3_decode8_lds<0>(o2 ? u0 : c0, t3_quads);
+        d.v[1] = turbo3_decode8_lds<0>(o2 ? u1 : c1, t3_quads);
+        d.v[2] = turbo3_decode8_lds<0>(o2 ? c2 : u0, t3_quads);
+        d.v[3] = turbo3_decode8_lds<0>(o2 ? c3 : u1, t3_quads);
         const float kq = __half2float(__builtin_bit_cast(__half, raw.kn)) * p.scale_log2e;
         const float vq = __half2float(__builtin_bit_cast(__half, raw.vn));
         static_for<4>([&](auto rc) {
@@ -774,6 +779,11 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
 // paged_attn_prefill_kernel below.
 template <int G, bool T3>
 __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_kernel(const AttnParams p) {
+    __shared__ uint2_t t3_quads[T3 ? kT3QuadEntries : 1];
+    if constexpr (T3) {
+        turbo3_fill_quads(t3_quads);
+        __syncthreads();  // (every exit below is taken by the whole workgroup)
+    }
     const int lane = threadIdx.x & 63;
     const int kvh = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);
     const int s = blockIdx.z;
@@ -789,7 +799,7 @@ __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_kernel(const At
     if (tok_begin >= ctx) return;
     const int num_parts = (ctx + p.part_tokens - 1) / p.part_tokens;
     attn_partition<G, T3>(p, s, t, kvh, tok_begin, min(ctx, tok_begin + p.part_tokens),
-                          num_parts == 1, (int64_t)s * p.num_splits + split);
+                          num_parts == 1, (int64_t)s * p.num_splits + split, t3_quads);
 }
 
 // Units sequence s contributes to the decode stream: its 16-key tiles plus kSeqStartUnits for
@@ -825,6 +835,8 @@ __device__ __forceinline__ int worker_tiles(int total_tiles, int num_workers) {
 template <int G, bool T3>
 __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_balanced_kernel(const AttnParams p) {
     __shared__ int pt[kMaxBalancedSeqs + 1];  // exclusive prefix of decode tiles
+    __shared__ uint2_t t3_quads[T3 ? kT3QuadEntries : 1];
+    if constexpr (T3) turbo3_fill_quads(t3_quads);  // (the barrier below covers it)
     const int lane = threadIdx.x & 63;
     const int kvh = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);
     const int S = p.num_seqs;
@@ -882,7 +894,7 @@ __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_balanced_kernel
             const int ctx = p.context_lens[s];
             const bool single = tile_lo == 0 && seg_end == seq_end;
             attn_partition<G, T3>(p, s, p.cu_seqlens_q[s], kvh, tile_lo * kTileKeys,
-                                  min(ctx, tile_hi * kTileKeys), single, (int64_t)w + s);
+                                  min(ctx, tile_hi * kTileKeys), single, (int64_t)w + s, t3_quads);
         }
         tcur = seg_end;
     }
