@@ -42,19 +42,35 @@ __device__ __forceinline__ uint4_t transpose_groups(uint4_t w) {
     return uint4_t{c[0], d[0], c[1], d[1]};
 }
 
+// What a wave has in flight for one chunk of 128 columns, in the layout it is LOADED in:
+// four consecutive lanes read 64 consecutive bytes (of x: sixteen lanes read a row's 256), so
+// a request touches each cache line once.  Loading straight into the MFMA operand layout
+// (lane = row % 16 + 16 * piece) put the four lanes of every quad on four different rows, a
+// tag look-up per lane: the texture addresser was busy 75 % of the launch and set its pace.
 template <int BT, int T>
 struct G32Chunk {
-    uint4_t xa[4][BT];  // x of group t, columns 8 kc .. 8 kc + 7, batch row bt * 16 + col
-    uint4_t w[T];       // group kc of weight row ti * 16 + col
-    uint2_t sc[T], mn[T];  // the row's four scales / mins of the chunk
+    uint4_t x[4][BT];  // batch row bt * 16 + 4 i + lane / 16, columns 8 (lane % 16) .. + 7
+    uint4_t w[T];      // group lane % 4 of weight row ti * 16 + lane / 4
+    unsigned short sc[T], mn[T];  // that group's scale and min
 };
+
+// per-wave LDS staging: the loaded layout goes in, the operand layout comes out (the LDS
+// queue of a wave is in order, so no wait sits between the write and the read)
+constexpr int kG32XRow = 272;                     // bytes per staged x row (256 + 16: no conflicts)
+constexpr int kG32WRow = 80;                      // bytes per staged weight row (64 + 16)
+constexpr int kG32StageX = 16 * kG32XRow;         // one 16-row x block
+constexpr int kG32StageW = 16 * kG32WRow;
+constexpr int kG32StageS = 16 * 8;                // four fp16 per row
+constexpr int kG32Stage = kG32StageX + kG32StageW + 2 * kG32StageS;
 
 template <int BT, int T>
 __global__ __launch_bounds__(64 * kG32Waves) void qgemm_q4g32_mfma_kernel(
     const uint16_t* __restrict__ x, const uint8_t* __restrict__ qw,
     const __half* __restrict__ scale, const __half* __restrict__ minv, uint16_t* __restrict__ y,
     const float* __restrict__ bias, int b, int n, int k) {
-    extern __shared__ float yl[];  // [waves][T][BP][16] partial results
+    // the staging areas of the eight waves; afterwards [waves][T][BP][16] partial results
+    extern __shared__ __attribute__((aligned(16))) unsigned char g32_lds[];
+    float* yl = reinterpret_cast<float*>(g32_lds);
     constexpr int BP = BT * 16;
     const int nchunks = k >> 7;
     const int groups = k >> 5;
@@ -76,29 +92,31 @@ __global__ __launch_bounds__(64 * kG32Waves) void qgemm_q4g32_mfma_kernel(
     const __half* mrow[T];
 #pragma unroll
     for (int ti = 0; ti < T; ++ti) {
-        const int r = ti * 16 + col;
+        const int r = ti * 16 + (lane >> 2);
         const int64_t row = row0 + (r < rows_here ? r : rows_here - 1);
-        wrow[ti] = qw + row * (int64_t)(k >> 1) + kc * 16;
-        srow[ti] = scale + row * groups;
-        mrow[ti] = minv + row * groups;
+        wrow[ti] = qw + row * (int64_t)(k >> 1) + (lane & 3) * 16;
+        srow[ti] = scale + row * groups + (lane & 3);
+        mrow[ti] = minv + row * groups + (lane & 3);
     }
-    const uint16_t* xrow[BT];
+    const uint16_t* xrow[4][BT];
 #pragma unroll
-    for (int bt = 0; bt < BT; ++bt) {
-        const int bi = bt * 16 + col;
-        xrow[bt] = x + (int64_t)(bi < b ? bi : b - 1) * k + kc * 8;
-    }
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int bt = 0; bt < BT; ++bt) {
+            const int bi = bt * 16 + 4 * i + kc;
+            xrow[i][bt] = x + (int64_t)(bi < b ? bi : b - 1) * k + col * 8;
+        }
     auto load_chunk = [&](int c, G32Chunk<BT, T>& ch) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
             for (int bt = 0; bt < BT; ++bt)
-                ch.xa[t][bt] = *reinterpret_cast<const uint4_t*>(xrow[bt] + c * 128 + t * 32);
+                ch.x[i][bt] = *reinterpret_cast<const uint4_t*>(xrow[i][bt] + c * 128);
 #pragma unroll
         for (int ti = 0; ti < T; ++ti) {
             ch.w[ti] = *reinterpret_cast<const uint4_t*>(wrow[ti] + c * 64);
-            ch.sc[ti] = *reinterpret_cast<const uint2_t*>(srow[ti] + c * 4);
-            ch.mn[ti] = *reinterpret_cast<const uint2_t*>(mrow[ti] + c * 4);
+            ch.sc[ti] = *reinterpret_cast<const unsigned short*>(srow[ti] + c * 4);
+            ch.mn[ti] = *reinterpret_cast<const unsigned short*>(mrow[ti] + c * 4);
         }
     };
 
@@ -108,25 +126,59 @@ __global__ __launch_bounds__(64 * kG32Waves) void qgemm_q4g32_mfma_kernel(
 #pragma unroll
         for (int bt = 0; bt < BT; ++bt) ysum[ti][bt] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-    auto compute_chunk = [&](G32Chunk<BT, T>& ch) {
+    unsigned char* stage = g32_lds + (size_t)wave * kG32Stage;
+    unsigned char* st_x = stage;
+    unsigned char* st_w = stage + kG32StageX;
+    unsigned char* st_s = st_w + kG32StageW;
+    unsigned char* st_m = st_s + kG32StageS;
+    // a wave's LDS accesses execute in program order; this only keeps the compiler from
+    // moving one across (another lane's data is not a dependence it sees)
+    auto in_order = [&]() {
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("" ::: "memory");
+    };
+
+    auto compute_chunk = [&](const G32Chunk<BT, T>& ch) {
+        // x in operand layout: xa[t][bt] = group t, columns 8 kc .. 8 kc + 7, batch row
+        // bt * 16 + col
+        uint4_t xa[4][BT];
         // sums of x over each group, in result layout: xs[t][bt][e] belongs to batch row
         // bt * 16 + 4 kc + e (the same for every column)
         float4_t xs[4][BT];
+#pragma unroll
+        for (int bt = 0; bt < BT; ++bt) {
+            in_order();
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                *reinterpret_cast<uint4_t*>(st_x + (4 * i + kc) * kG32XRow + col * 16) = ch.x[i][bt];
+            in_order();
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                xa[t][bt] = *reinterpret_cast<const uint4_t*>(st_x + col * kG32XRow + t * 64 + kc * 16);
+        }
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
             for (int bt = 0; bt < BT; ++bt) {
                 xs[t][bt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                    __builtin_bit_cast(bf16x8_t, ch.xa[t][bt]), one_op,
+                    __builtin_bit_cast(bf16x8_t, xa[t][bt]), one_op,
                     float4_t{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
-                ch.xa[t][bt] = pair_order(ch.xa[t][bt]);
+                xa[t][bt] = pair_order(xa[t][bt]);
             }
 #pragma unroll
         for (int ti = 0; ti < T; ++ti) {
-            const uint4_t wt = transpose_groups(ch.w[ti]);
+            in_order();
+            *reinterpret_cast<uint4_t*>(st_w + (lane >> 2) * kG32WRow + (lane & 3) * 16) = ch.w[ti];
+            *reinterpret_cast<unsigned short*>(st_s + (lane >> 2) * 8 + (lane & 3) * 2) = ch.sc[ti];
+            *reinterpret_cast<unsigned short*>(st_m + (lane >> 2) * 8 + (lane & 3) * 2) = ch.mn[ti];
+            in_order();
+            const uint4_t wl = *reinterpret_cast<const uint4_t*>(st_w + col * kG32WRow + kc * 16);
+            const uint2_t sc4 = *reinterpret_cast<const uint2_t*>(st_s + col * 8);
+            const uint2_t mn4 = *reinterpret_cast<const uint2_t*>(st_m + col * 8);
+            const uint4_t wt = transpose_groups(wl);
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                const unsigned sw = ch.sc[ti][t >> 1], mw = ch.mn[ti][t >> 1];
+                const unsigned sw = sc4[t >> 1], mw = mn4[t >> 1];
                 const unsigned short sh = (unsigned short)((t & 1) ? (sw >> 16) : (sw & 0xffffu));
                 const unsigned short mh = (unsigned short)((t & 1) ? (mw >> 16) : (mw & 0xffffu));
                 const float d = __half2float(__builtin_bit_cast(__half, sh));
@@ -139,7 +191,7 @@ __global__ __launch_bounds__(64 * kG32Waves) void qgemm_q4g32_mfma_kernel(
 #pragma unroll
                 for (int bt = 0; bt < BT; ++bt) {
                     const float4_t acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                        __builtin_bit_cast(bf16x8_t, ch.xa[t][bt]), bop,
+                        __builtin_bit_cast(bf16x8_t, xa[t][bt]), bop,
                         float4_t{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
@@ -169,6 +221,7 @@ __global__ __launch_bounds__(64 * kG32Waves) void qgemm_q4g32_mfma_kernel(
             __builtin_amdgcn_sched_barrier(0);
         }
     }
+    __syncthreads();  // the partial results reuse the staging areas
 
     float* yw = yl + (size_t)wave * T * BP * 16;
 #pragma unroll
@@ -196,7 +249,9 @@ template <int BT, int T>
 static hipError_t launch_g32(const void* x, const void* qw, const void* scale, const void* minv,
                              void* y, const float* bias, int b, int n, int k, hipStream_t stream) {
     const int tiles = (n + 15) / 16;
-    const size_t lds = (size_t)kG32Waves * T * BT * 16 * 16 * 4;  // at most 48 KiB
+    const size_t parts = (size_t)kG32Waves * T * BT * 16 * 16 * 4;  // at most 48 KiB
+    const size_t staging = (size_t)kG32Waves * kG32Stage;           // 46 KiB
+    const size_t lds = parts > staging ? parts : staging;
     qgemm_q4g32_mfma_kernel<BT, T><<<dim3((tiles + T - 1) / T), dim3(64 * kG32Waves), lds, stream>>>(
         static_cast<const uint16_t*>(x), static_cast<const uint8_t*>(qw),
         static_cast<const __half*>(scale), static_cast<const __half*>(minv),
