@@ -655,7 +655,7 @@ def bench_decode_step(args):
     # pools re-encoded on the device, new rows encoded as the step writes them, attention
     # decoding inside its gather.  A different cache format, so a figure of its own.
     turbo3_step = None
-    if args.extras:
+    if args.extras or (not args.skip_kernels and args.workload == "all"):
         rows = r.pools[0][0].nbytes // (hkv * 128 * 2)
         d_iota = hip.DeviceBuffer.from_numpy(np.arange(rows, dtype=np.int64))
         t3_pools = []
@@ -758,8 +758,9 @@ def main():
                     help="only the decode-step line, without the per-kernel legs")
     ap.add_argument("--extras", action="store_true",
                     help="add the extra legs of the decode step (token ids in / token ids out "
-                         "with embedding, lm_head + greedy; the step over turbo3 KV pools); not "
-                         "part of the metric, and not for runs under a profiler")
+                         "with embedding, lm_head + greedy; the step over turbo3 KV pools, which "
+                         "the full default run includes anyway); not part of the metric, and "
+                         "not for runs under a profiler")
     ap.add_argument("--workload", default="all",
                     choices=["all", "step", "config1", "config2", "config3", "config4",
                              "config4_gemm", "turbo3"],
