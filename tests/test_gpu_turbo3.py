@@ -158,11 +158,14 @@ def test_turbo3_attention_gqa_group_sizes(hq, hkv):
         assert_parity(_attn_turbo3(c, kp, vp, ns), want, what=f"turbo3 {hq}/{hkv} splits {ns}")
 
 
-def test_turbo3_attention_balanced_kernel_and_zero_context():
-    rng = np.random.default_rng(71)
+@pytest.mark.parametrize("hq,hkv", [(8, 2), (16, 2), (32, 8), (7, 1), (3, 1)])
+def test_turbo3_attention_balanced_kernel_and_zero_context(hq, hkv):
+    # group sizes on both sides of four (a lane row of the P.V accumulators holds four heads),
+    # one to eight waves sharing the workgroup's centroid table, odd and even tile counts
+    rng = np.random.default_rng(71 + hq)
     new = np.ones(12, np.int32)
     prior = [0, 40, 2047, 16, 511, 300, 1, 999, 64, 65, 129, 700]
-    c = workloads.paged_case(rng, new, prior, hq=8, hkv=2, min_max_blocks=8192)
+    c = workloads.paged_case(rng, new, prior, hq=hq, hkv=hkv, min_max_blocks=8192)
     c["context_lens"][3] = 0
     kp, vp = _turbo3_pools(c)
     want = _oracle_t3(c, kp, vp)
