@@ -56,6 +56,23 @@ __device__ __forceinline__ float row_bcast(float v) {
     return dpp_f32<kDppRowNewBcast + N>(v);
 }
 
+// Split-K parts are added in part order, several loads in flight per round: body(ic<N>{}, q0)
+// is called for the parts q0 .. q0 + N - 1, N = MAXR for full rounds and exactly what is left
+// for the last one (a round padded with repeated loads of its first part costs the
+// workgroup's L1 bandwidth as if they were real).
+template <int N, class F>
+__device__ __forceinline__ void part_round_of(int left, int q0, F&& body) {
+    if (left == N) body(ic<N>{}, q0);
+    else if constexpr (N > 1) part_round_of<N - 1>(left, q0, body);
+}
+template <int MAXR, class F>
+__device__ __forceinline__ void for_part_rounds(int num_parts, F&& body) {
+    for (int q0 = 0; q0 < num_parts; q0 += MAXR) {
+        const int left = num_parts - q0;
+        part_round_of<MAXR>(left < MAXR ? left : MAXR, q0, body);
+    }
+}
+
 // value held by lane N of each group of four lanes, broadcast to the four (quad_perm)
 template <int N>
 __device__ __forceinline__ float quad_bcast(float v) {

@@ -55,14 +55,18 @@ __global__ __launch_bounds__(kNormThreads) void add_rms_norm_kernel(
                     *reinterpret_cast<float4_t*>(hr + j) = v[p];
                 } else if (yp) {
                     // fp32 partial sums of a split-K projection, added in part order
-                    for (int q = 0; q < num_parts; ++q) {
-                        const float4_t t4 = *reinterpret_cast<const float4_t*>(
-                            yp + (int64_t)q * part_stride + row * n + j);
-                        v[p][0] += t4[0];
-                        v[p][1] += t4[1];
-                        v[p][2] += t4[2];
-                        v[p][3] += t4[3];
-                    }
+                    for_part_rounds<4>(num_parts, [&](auto nc, int q0) {
+                        constexpr int N = decltype(nc)::value;
+                        float4_t t4[N];
+#pragma unroll
+                        for (int u = 0; u < N; ++u)
+                            t4[u] = *reinterpret_cast<const float4_t*>(
+                                yp + (int64_t)(q0 + u) * part_stride + row * n + j);
+#pragma unroll
+                        for (int u = 0; u < N; ++u)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[p][e] += t4[u][e];
+                    });
                     *reinterpret_cast<float4_t*>(hr + j) = v[p];
                 }
 #pragma unroll
@@ -133,28 +137,25 @@ __global__ __launch_bounds__(kPrepThreads) void add_rms_norm_xprep_kernel(
             const float4_t a = *reinterpret_cast<const float4_t*>(hr + j);
             const float4_t b = *reinterpret_cast<const float4_t*>(hr + j + 4);
             float4_t s0 = a, s1 = b;
-            // h + part 0 + part 1 + ... in this order; the loads of six parts in flight per
-            // round (a round is one trip to memory: 4 parts take one, 12 take two)
-            constexpr int R = 6;
-            for (int q0 = 0; q0 < num_parts; q0 += R) {
-                float4_t t0[R], t1[R];
+            // h + part 0 + part 1 + ... in this order; the loads of up to six parts in flight
+            // per round (a round is one trip to memory: 4 parts take one, 12 take two)
+            for_part_rounds<6>(num_parts, [&](auto nc, int q0) {
+                constexpr int N = decltype(nc)::value;
+                float4_t t0[N], t1[N];
 #pragma unroll
-                for (int u = 0; u < R; ++u) {
-                    const int q = (q0 + u) < num_parts ? (q0 + u) : q0;
-                    const float* src = yp + (int64_t)q * part_stride + row * n + j;
+                for (int u = 0; u < N; ++u) {
+                    const float* src = yp + (int64_t)(q0 + u) * part_stride + row * n + j;
                     t0[u] = *reinterpret_cast<const float4_t*>(src);
                     t1[u] = *reinterpret_cast<const float4_t*>(src + 4);
                 }
 #pragma unroll
-                for (int u = 0; u < R; ++u)
-                    if (q0 + u < num_parts) {
+                for (int u = 0; u < N; ++u)
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            s0[e] += t0[u][e];
-                            s1[e] += t1[u][e];
-                        }
+                    for (int e = 0; e < 4; ++e) {
+                        s0[e] += t0[u][e];
+                        s1[e] += t1[u][e];
                     }
-            }
+            });
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 v[p][e] = s0[e];
@@ -219,30 +220,28 @@ __global__ __launch_bounds__(256) void silu_mul_xprep_kernel(const float* __rest
 #pragma unroll
         for (int e = 0; e < 8; ++e) g[e] = u[e] = 0.0f;
         const int64_t base = (int64_t)t * 2 * inter + (int64_t)c * 8;
-        // parts are added in order; the loads of four parts are in flight per round
-        for (int q0 = 0; q0 < num_parts; q0 += 4) {
-            float4_t g0[4], g1[4], u0[4], u1[4];
+        // parts are added in order; the loads of up to four parts are in flight per round
+        for_part_rounds<4>(num_parts, [&](auto nc, int q0) {
+            constexpr int N = decltype(nc)::value;
+            float4_t g0[N], g1[N], u0[N], u1[N];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int q = (q0 + r) < num_parts ? (q0 + r) : q0;
-                const float* src = parts + (int64_t)q * part_stride + base;
+            for (int r = 0; r < N; ++r) {
+                const float* src = parts + (int64_t)(q0 + r) * part_stride + base;
                 g0[r] = *reinterpret_cast<const float4_t*>(src);
                 g1[r] = *reinterpret_cast<const float4_t*>(src + 4);
                 u0[r] = *reinterpret_cast<const float4_t*>(src + inter);
                 u1[r] = *reinterpret_cast<const float4_t*>(src + inter + 4);
             }
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-                if (q0 + r < num_parts) {
+            for (int r = 0; r < N; ++r)
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        g[e] += g0[r][e];
-                        g[4 + e] += g1[r][e];
-                        u[e] += u0[r][e];
-                        u[4 + e] += u1[r][e];
-                    }
+                for (int e = 0; e < 4; ++e) {
+                    g[e] += g0[r][e];
+                    g[4 + e] += g1[r][e];
+                    u[e] += u0[r][e];
+                    u[4 + e] += u1[r][e];
                 }
-        }
+        });
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const float a = g[2 * e] / (1.0f + expf(-g[2 * e])) * u[2 * e];
@@ -283,22 +282,21 @@ __global__ __launch_bounds__(64) void rope_kv_write_kernel(
         x0 = bf16_to_f32(qkv[off + i]);
         x1 = bf16_to_f32(qkv[off + i + HALF]);
     } else {
-        // parts are added in order; the loads of four parts are in flight per round
-        for (int q0 = 0; q0 < num_parts; q0 += 4) {
-            float a[4], b[4];
+        // parts are added in order; the loads of up to four parts are in flight per round
+        for_part_rounds<4>(num_parts, [&](auto nc, int q0) {
+            constexpr int N = decltype(nc)::value;
+            float a[N], b[N];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int q = (q0 + r) < num_parts ? (q0 + r) : q0;
-                a[r] = qkv_parts[(int64_t)q * part_stride + off + i];
-                b[r] = qkv_parts[(int64_t)q * part_stride + off + i + HALF];
+            for (int r = 0; r < N; ++r) {
+                a[r] = qkv_parts[(int64_t)(q0 + r) * part_stride + off + i];
+                b[r] = qkv_parts[(int64_t)(q0 + r) * part_stride + off + i + HALF];
             }
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-                if (q0 + r < num_parts) {
-                    x0 += a[r];
-                    x1 += b[r];
-                }
-        }
+            for (int r = 0; r < N; ++r) {
+                x0 += a[r];
+                x1 += b[r];
+            }
+        });
     }
     if (bias) {
         // the projection's bias (`linear_t`, one fp32 add on the finished sum), column head*D + i
