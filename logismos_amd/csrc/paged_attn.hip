@@ -96,9 +96,10 @@ __device__ __forceinline__ unsigned short attn_out_elem(float v, int out_bf16) {
 // sum_j p_j v_j = H sum_j (p_j norm_j) c_j: the kernel transforms q once, works on the
 // centroid values themselves and transforms the result once.
 struct KvTileT3 {
-    unsigned k[3], v[3];  // the 96 index bits of one 32-value block of a key
-    unsigned short kn, vn;
+    // 16 dword-aligned bytes around one 14-byte block {norm, 96 index bits} of a key each
+    uint4_t k, v;
 };
+typedef uint4_t __attribute__((aligned(4))) uint4_a4_t;
 
 // fp16 bits of `TURBO3_CODEBOOK` (RNE): b207 af90 ac43 a588 2588 2c43 2f90 3207; tables of
 // their low and high bytes for v_perm_b32
@@ -399,9 +400,14 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
     // over the four lanes c / 4 = const and transposes the block's four groups against the
     // four keys there, which leaves group c % 4 of block c / 4 (values 8c .. 8c + 7) of the
     // keys 4tg .. 4tg + 3 in the lane: the B operand of P.V.
+    // Requests are 16 bytes at a multiple of 4 (the 12 index bytes of block b start at byte
+    // 14b + 2: the request starts 2 bytes before them for even b, 4 bytes for odd b, i.e. at
+    // 0, 12, 28, 40, and ends inside the 56-byte head row), two per tile; the block-0 requests
+    // bring the row's norm along.  Unaligned 12-byte and 2-byte requests, five per tile, kept
+    // the CU's texture addresser busy two thirds of the launch.
     const unsigned row_bytes = (unsigned)p.hkv * 56u;
-    const unsigned k3_piece = 14u * tg + 2u;
-    const unsigned v3_piece = 14u * (c >> 2) + 2u;
+    const unsigned k3_piece = 14u * tg + 2u - ((tg & 1) ? 4u : 2u);
+    const unsigned v3_piece = 14u * (c >> 2) + 2u - (((c >> 2) & 1) ? 4u : 2u);
     auto load_tile = [&](int tile, Tile& kv) {
         const int tok_base = __builtin_amdgcn_readfirstlane(tok_begin + tile * kTileKeys);
         const int blk_idx = tok_base / p.block_size;
@@ -414,11 +420,9 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
             const uint8_t* vb = reinterpret_cast<const uint8_t*>(p.v_pool) + base;
             const unsigned last_off = (unsigned)(tok_end - 1 - tok_base) * row_bytes;
             const unsigned ko = min((unsigned)c * row_bytes, last_off) + k3_piece;
-            __builtin_memcpy(kv.k, kb + ko, 12);
+            kv.k = *reinterpret_cast<const uint4_a4_t*>(kb + ko);
             const unsigned no = min((unsigned)(4 * tg + (c & 3)) * row_bytes, last_off);
-            __builtin_memcpy(kv.v, vb + no + v3_piece, 12);
-            kv.kn = *reinterpret_cast<const unsigned short*>(kb + no);
-            kv.vn = *reinterpret_cast<const unsigned short*>(vb + no);
+            kv.v = *reinterpret_cast<const uint4_a4_t*>(vb + no + v3_piece);
             return;
         }
         const int64_t base = (row_base * p.hkv + kvh) * kHeadDim;
@@ -537,16 +541,25 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
         float kn[4], vn[4];
     };
     auto t3_decode = [&](const KvTileT3& raw, T3Decoded& d) {
+        // the 96 index bits out of the 16 loaded bytes: they start at byte 2 (even block) or 4
+        const unsigned ksel = (tg & 1) ? 0x07060504u : 0x05040302u;
+        const unsigned k0 = __builtin_amdgcn_perm(raw.k[1], raw.k[0], ksel);
+        const unsigned k1 = __builtin_amdgcn_perm(raw.k[2], raw.k[1], ksel);
+        const unsigned k2 = __builtin_amdgcn_perm(raw.k[3], raw.k[2], ksel);
         // groups 0..3 of a block start at bits 0, 24, 48 and 72 of its 96
-        d.k[0] = turbo3_decode8_lds<0>(raw.k[0], t3_quads);
-        d.k[1] = turbo3_decode8_lds<0>(__builtin_amdgcn_alignbit(raw.k[1], raw.k[0], 24), t3_quads);
-        d.k[2] = turbo3_decode8_lds<0>(__builtin_amdgcn_alignbit(raw.k[2], raw.k[1], 16), t3_quads);
-        d.k[3] = turbo3_decode8_lds<8>(raw.k[2], t3_quads);
+        d.k[0] = turbo3_decode8_lds<0>(k0, t3_quads);
+        d.k[1] = turbo3_decode8_lds<0>(__builtin_amdgcn_alignbit(k1, k0, 24), t3_quads);
+        d.k[2] = turbo3_decode8_lds<0>(__builtin_amdgcn_alignbit(k2, k1, 16), t3_quads);
+        d.k[3] = turbo3_decode8_lds<8>(k2, t3_quads);
+        const unsigned vsel = (c & 4) ? 0x07060504u : 0x05040302u;
+        const unsigned v0 = __builtin_amdgcn_perm(raw.v[1], raw.v[0], vsel);
+        const unsigned v1 = __builtin_amdgcn_perm(raw.v[2], raw.v[1], vsel);
+        const unsigned v2 = __builtin_amdgcn_perm(raw.v[3], raw.v[2], vsel);
         // a[i] = group i of this lane's key; after the transpose, group c % 4 of key 4tg + i.
         // Two butterfly steps (lanes c ^ 1, then c ^ 2): a lane keeps the registers whose
         // index bit equals its own and trades the others.
-        const unsigned a[4] = {raw.v[0], __builtin_amdgcn_alignbit(raw.v[1], raw.v[0], 24),
-                               __builtin_amdgcn_alignbit(raw.v[2], raw.v[1], 16), raw.v[2] >> 8};
+        const unsigned a[4] = {v0, __builtin_amdgcn_alignbit(v1, v0, 24),
+                               __builtin_amdgcn_alignbit(v2, v1, 16), v2 >> 8};
         const bool o1 = (c & 1) != 0, o2 = (c & 2) != 0;
         constexpr int kQuadXor1 = 0xB1, kQuadXor2 = 0x4E;  // quad_perm [1,0,3,2], [2,3,0,1]
         const unsigned r0 = (unsigned)dpp_i32<kQuadXor1>((int)(o1 ? a[0] : a[1]));
@@ -559,12 +572,18 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
         d.v[1] = turbo3_decode8_lds<0>(o2 ? u1 : c1, t3_quads);
         d.v[2] = turbo3_decode8_lds<0>(o2 ? c2 : u0, t3_quads);
         d.v[3] = turbo3_decode8_lds<0>(o2 ? c3 : u1, t3_quads);
-        const float kq = __half2float(__builtin_bit_cast(__half, raw.kn)) * p.scale_log2e;
-        const float vq = __half2float(__builtin_bit_cast(__half, raw.vn));
+        // norms (the first block's, as the reference decoder takes them): key c's K norm came
+        // with the block-0 request of lane (0, c), key 4tg + c % 4's V norm with that of lane
+        // (tg, c % 4).  A lane row needs those of its keys 4tg .. 4tg + 3.
+        const unsigned kn_bits = (unsigned)__builtin_amdgcn_ds_bpermute(
+            (int)((4 * tg + (c & 3)) * 4), (int)raw.k[0]);
+        const float kq = __half2float(__builtin_bit_cast(__half, (unsigned short)kn_bits)) *
+                         p.scale_log2e;
+        const float vq = __half2float(__builtin_bit_cast(__half, (unsigned short)raw.v[0]));
         static_for<4>([&](auto rc) {
             constexpr int r = decltype(rc)::value;
             d.kn[r] = quad_bcast<r>(kq);
-            d.vn[r] = quad_bcast<r>(vq);
+            d.vn[r] = row_bcast<r>(vq);
         });
     };
     auto t3_compute_pair = [&](int tile, const KvTileT3& raw0, const KvTileT3& raw1) {
