@@ -456,20 +456,18 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
 
     float m = -INFINITY;  // running max (log2 domain), meaningful in lanes c < G
     float l = 0.0f;       // running sum
-    float acc[G][8];
+    // P.V on the matrix cores (fp32 accumulation, probabilities rounded to fp16 like the values
+    // they multiply).  accp[e][r] = element 8c + e of head 4 tg + r: the C layout of
+    // v_mfma_f32_16x16x16_f16 with A = P (row = head, the four keys of this lane row), B_e =
+    // element e of the lane's eight values of each of its four keys (column = c).  The sum over
+    // all 16 keys of a tile is the MFMA's, so the four lane rows share one running maximum per
+    // head (m), only the sums l are per row, and the epilogue has no partial rows to merge.
+    // For turbo3 pools the 128 multiply-adds of P.V were the largest item of a tile bound by its
+    // vector instructions; for fp16 pools a long stream runs at the same rate either way and a
+    // short one (16 sequences of at most 2048 keys) is 20 % faster for the shorter epilogue.
+    float4_t accp[8];
 #pragma unroll
-    for (int h = 0; h < G; ++h)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[h][e] = 0.0f;
-    // turbo3 pools: P.V on the matrix cores (the tile is bound by its vector instructions, and
-    // the 128 multiply-adds of P.V are the largest single item).  accp[e][r] = element 8c + e of
-    // head 4 tg + r: the C layout of v_mfma_f32_16x16x16_f16 with A = P (row = head, the four
-    // keys of this lane row), B_e = element e of the lane's eight values of each of its four
-    // keys (column = c).  The sum over all 16 keys of a tile is the MFMA's, so the four lane
-    // rows share one running maximum per head (m) and only the sums l are per row.
-    float4_t accp[T3 ? 8 : 1];
-#pragma unroll
-    for (int e = 0; e < (T3 ? 8 : 1); ++e) accp[e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int e = 0; e < 8; ++e) accp[e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
     auto compute_tile = [&](int tile, const KvTile& raw) {
         KvTile kv = raw;
@@ -503,34 +501,50 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
             sc[r] = (tok0 + r < tok_end) ? sacc[r] * p.scale_log2e : -INFINITY;
             mx = fmaxf(mx, sc[r]);
         }
+        // one maximum per head for all 16 keys (the lane rows hold four keys each): the matrix
+        // cores sum P.V over the whole tile
+        mx = fmaxf(mx, lane_xor_f32<16>(mx));
+        mx = fmaxf(mx, lane_xor_f32<32>(mx));
         const float msafe = (mx == -INFINITY) ? 0.0f : mx;
         const float alpha = fast_exp2(m - msafe);
-        float pr[4];
+        half4_t pa;
         float psum = 0.0f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            pr[r] = fast_exp2(sc[r] - msafe);
-            psum += pr[r];
+            const float pr = fast_exp2(sc[r] - msafe);
+            psum += pr;
+            pa[r] = (_Float16)pr;
         }
         l = l * alpha + psum;
         m = mx;
-        static_for<G>([&](auto hc) {
-            constexpr int h = decltype(hc)::value;
-            const float a = row_bcast<h>(alpha);
-            const float p0 = row_bcast<h>(pr[0]);
-            const float p1 = row_bcast<h>(pr[1]);
-            const float p2 = row_bcast<h>(pr[2]);
-            const float p3 = row_bcast<h>(pr[3]);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                float v = acc[h][e] * a;
-                v = fmaf(p0, (float)kv.v[0][e], v);
-                v = fmaf(p1, (float)kv.v[1][e], v);
-                v = fmaf(p2, (float)kv.v[2][e], v);
-                v = fmaf(p3, (float)kv.v[3][e], v);
-                acc[h][e] = v;
+        // rescale: row r of the accumulators is head 4 tg + r, whose factor sits in lane
+        // c = 4 tg + r of every lane row
+        float ar[4];
+        static_for<4>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            if constexpr (G <= 4) {
+                ar[r] = row_bcast<r>(alpha);
+            } else {
+                const float lo = row_bcast<r>(alpha), hi = row_bcast<4 + r>(alpha);
+                ar[r] = tg == 0 ? lo : hi;
             }
         });
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) accp[e][r] *= ar[r];
+            // B operand: element e of the eight values this lane holds of its four keys
+            const unsigned sel = (e & 1) ? 0x07060302u : 0x05040100u;
+            const uint4_t v0 = __builtin_bit_cast(uint4_t, kv.v[0]);
+            const uint4_t v1 = __builtin_bit_cast(uint4_t, kv.v[1]);
+            const uint4_t v2 = __builtin_bit_cast(uint4_t, kv.v[2]);
+            const uint4_t v3 = __builtin_bit_cast(uint4_t, kv.v[3]);
+            uint2_t bw;
+            bw[0] = __builtin_amdgcn_perm(v1[e >> 1], v0[e >> 1], sel);
+            bw[1] = __builtin_amdgcn_perm(v3[e >> 1], v2[e >> 1], sel);
+            accp[e] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa, __builtin_bit_cast(half4_t, bw),
+                                                            accp[e], 0, 0, 0);
+        }
     };
 
     // turbo3 pools, two tiles (32 keys) at a time: one running-maximum update and one rescale
@@ -744,7 +758,7 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
             }
         }
     };
-    if constexpr (T3) {
+    {
         // the matrix cores have summed over all the keys: head 4tg + r is complete in row r of
         // the accumulators of lane row tg, the lane rows share m, and the sums l of the four
         // lane rows (four keys of every tile each) add up to the whole
@@ -755,7 +769,7 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
             float x[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) x[e] = accp[e][r];
-            fwht_row(x);  // back from the centroid domain
+            if constexpr (T3) fwht_row(x);  // back from the centroid domain
             float mh = row_bcast<r>(m), lh = row_bcast<r>(lsum);
             if constexpr (G > 4) {
                 const float mhi = row_bcast<4 + (r < G - 4 ? r : 0)>(m);
@@ -765,30 +779,7 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
             }
             if (4 * tg + r < G) write_head(4 * tg + r, x, mh, lh);
         });
-        return;
     }
-    // ---- fp16 pools: merge the four rows of the wave, then write
-    static_for<G>([&](auto hc) {
-        constexpr int h = decltype(hc)::value;
-        float mh = row_bcast<h>(m);
-        float lh = row_bcast<h>(l);
-#pragma unroll
-        for (int mask = 16; mask <= 32; mask <<= 1) {
-            const float mo = shfl_xor_lds_f32(mh, mask);
-            const float mn = fmaxf(mh, mo);
-            const float msafe = (mn == -INFINITY) ? 0.0f : mn;
-            const float f = fast_exp2(mh - msafe);
-            lh *= f;
-            lh += shfl_xor_lds_f32(lh, mask);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float v = acc[h][e] * f;
-                acc[h][e] = v + shfl_xor_lds_f32(v, mask);
-            }
-            mh = mn;
-        }
-        if (tg == (h & 3)) write_head(h, acc[h], mh, lh);
-    });
 }
 
 // Decode rows, static split: grid (num_splits, hkv / waves, num_seqs); sequences with
