@@ -237,3 +237,17 @@ def test_put_encode_then_attend_round_trip_on_the_gpu():
     assert np.array_equal(kp.to_numpy(np.uint8, kp_h.shape), kp_h)
     got = _attn_turbo3(c, kp_h, vp_h)
     assert_parity(got, _oracle_t3(c, kp_h, vp_h), what="turbo3 put -> attend")
+
+
+def test_turbo3_attention_at_config5_contexts():
+    """The decode step's own attention shape (32 sequences, contexts U{256..8192}, 32 query /
+    8 KV heads: the balanced kernel, eight waves per workgroup, partitions that start and end
+    inside sequences) over turbo3 pools, every row against the oracle."""
+    rng = np.random.default_rng(workloads.SEED + 5)
+    ctx = rng.integers(256, 8193, size=32)
+    # (pools that repeat 4099 random rows: drawing 150 k distinct rows takes a quarter minute)
+    c = workloads.paged_case(rng, np.ones(32, np.int32), ctx - 1, hq=32, hkv=8, spare_frac=0.05,
+                             pool_period_rows=4099)
+    kp, vp = _turbo3_pools(c)
+    want = _oracle_t3(c, kp, vp)
+    assert_parity(_attn_turbo3(c, kp, vp), want, what="turbo3 attention, config-5 contexts")
