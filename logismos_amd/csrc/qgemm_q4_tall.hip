@@ -111,17 +111,24 @@ __global__ __launch_bounds__(128 * NW, NW == 2 ? 2 : 1) void qgemm_q4g128_tall_k
     // the 32 bytes of a group are consumed 16 at a time (MFMAs 0-3, then 4-7); each half is
     // requested again, for the next group, as soon as its last MFMA has been issued
     uint4_t wcur[2][2];
-    __half scur[2], zcur[2], snext[2], znext[2];
+    // scales and zeros of two consecutive groups per request (one dword: a 2-byte request per
+    // lane costs the texture addresser as much as a 16-byte one)
+    unsigned scur[2], zcur[2], snext[2], znext[2];
     auto gload_w_half = [&](int g, int half) {
 #pragma unroll
         for (int j = 0; j < 2; ++j)
             wcur[j][half] = reinterpret_cast<const uint4_t*>(qw + (woff[j] + (unsigned)g * 64u))[half];
     };
-    auto gload_sz = [&](int g, __half (&s)[2], __half (&z)[2]) {
+    auto gload_sz = [&](int g, unsigned (&s)[2], unsigned (&z)[2]) {  // g even: groups g, g + 1
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            s[j] = scale[soff[j] + (unsigned)g];
-            z[j] = zero[soff[j] + (unsigned)g];
+            if (g + 1 < groups) {
+                __builtin_memcpy(&s[j], scale + soff[j] + (unsigned)g, 4);
+                __builtin_memcpy(&z[j], zero + soff[j] + (unsigned)g, 4);
+            } else {  // an odd number of groups: the last one alone
+                s[j] = __builtin_bit_cast(unsigned short, scale[soff[j] + (unsigned)g]);
+                z[j] = __builtin_bit_cast(unsigned short, zero[soff[j] + (unsigned)g]);
+            }
         }
     };
 
@@ -146,7 +153,7 @@ __global__ __launch_bounds__(128 * NW, NW == 2 ? 2 : 1) void qgemm_q4g128_tall_k
         const bool more = g + 1 < groups;
         if (more) {
             gload_x(g + 1, 0);
-            gload_sz(g + 1, snext, znext);
+            if (((g + 1) & 1) == 0) gload_sz(g + 1, snext, znext);
         }
         const uint16_t* xt = xs_lds + buf * kTallSlab;
         float16_t acc[2][2];
@@ -198,8 +205,10 @@ __global__ __launch_bounds__(128 * NW, NW == 2 ? 2 : 1) void qgemm_q4g128_tall_k
             }
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                const float sf = __half2float(scur[j]);
-                const float off = 128.0f + __half2float(zcur[j]);
+                const unsigned short sb = (unsigned short)((g & 1) ? (scur[j] >> 16) : scur[j]);
+                const unsigned short zb = (unsigned short)((g & 1) ? (zcur[j] >> 16) : zcur[j]);
+                const float sf = __half2float(__builtin_bit_cast(__half, sb));
+                const float off = 128.0f + __half2float(__builtin_bit_cast(__half, zb));
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
                     yacc[i][j][e] = fmaf(sf, fmaf(-off, sx[e], acc[i][j][e]), yacc[i][j][e]);
@@ -208,10 +217,11 @@ __global__ __launch_bounds__(128 * NW, NW == 2 ? 2 : 1) void qgemm_q4g128_tall_k
         if (more) {
             lstore_x(buf ^ 1, 1);
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                scur[j] = snext[j];
-                zcur[j] = znext[j];
-            }
+            for (int j = 0; j < 2; ++j)
+                if (((g + 1) & 1) == 0) {
+                    scur[j] = snext[j];
+                    zcur[j] = znext[j];
+                }
         }
         __syncthreads();
     }
