@@ -919,6 +919,25 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams 
     const int h = blockIdx.x;
     const int lane = threadIdx.x & 63;
     const int w = threadIdx.x >> 6;
+    // Static split: where a sequence's partials sit does not depend on its lengths, so this
+    // wave's first round of partials (w, w + 4, w + 8, w + 12) is requested before the lengths
+    // are back: one trip to memory instead of two in a launch that is little else.  (Slots
+    // past the sequence's partitions are inside the workspace; what they hold is not used.)
+    float pm[4], pl[4], pa0[4], pa1[4];
+    const bool prefetched = p.num_workers == 0 && p.num_splits > 1;
+    if (prefetched) {
+        const int64_t base0 = (int64_t)s * p.num_splits * p.hq + h;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = min(w + 4 * j, p.num_splits - 1);
+            const int64_t idx = base0 + (int64_t)i * p.hq;
+            pm[j] = p.ws_ml[idx * 2];
+            pl[j] = p.ws_ml[idx * 2 + 1];
+            const float* a = p.ws_acc + idx * kHeadDim + 2 * lane;
+            pa0[j] = a[0];
+            pa1[j] = a[1];
+        }
+    }
     const int t0 = p.cu_seqlens_q[s];
     if (p.cu_seqlens_q[s + 1] - t0 != 1) return;
     const int ctx = p.context_lens[s];
@@ -976,11 +995,20 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams 
         for (int j = 0; j < 4; ++j) {
             const int i = i0 + 4 * j;
             const bool valid = i < np;
-            const int64_t idx = base + (int64_t)(valid ? i : i0) * p.hq;
-            const float mv = p.ws_ml[idx * 2];
-            const float lv = p.ws_ml[idx * 2 + 1];
-            const float* a = p.ws_acc + idx * kHeadDim + 2 * lane;
-            const float av0 = a[0], av1 = a[1];
+            float mv, lv, av0, av1;
+            if (prefetched && i0 == w) {
+                mv = pm[j];
+                lv = pl[j];
+                av0 = pa0[j];
+                av1 = pa1[j];
+            } else {
+                const int64_t idx = base + (int64_t)(valid ? i : i0) * p.hq;
+                mv = p.ws_ml[idx * 2];
+                lv = p.ws_ml[idx * 2 + 1];
+                const float* a = p.ws_acc + idx * kHeadDim + 2 * lane;
+                av0 = a[0];
+                av1 = a[1];
+            }
             mj[j] = valid ? mv : -INFINITY;
             lj[j] = valid ? lv : 0.0f;
             a0[j] = valid ? av0 : 0.0f;
