@@ -507,13 +507,16 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
         mx = fmaxf(mx, lane_xor_f32<32>(mx));
         const float msafe = (mx == -INFINITY) ? 0.0f : mx;
         const float alpha = fast_exp2(m - msafe);
-        half4_t pa;
+        // the probabilities as two fp16 terms (the matrix cores have time to spare here, and
+        // one term alone costs three decimal digits of the result)
+        half4_t pa, pb;
         float psum = 0.0f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const float pr = fast_exp2(sc[r] - msafe);
             psum += pr;
             pa[r] = (_Float16)pr;
+            pb[r] = (_Float16)(pr - (float)pa[r]);
         }
         l = l * alpha + psum;
         m = mx;
@@ -543,6 +546,8 @@ __device__ __forceinline__ void attn_partition(const AttnParams& p, int s, int t
             bw[0] = __builtin_amdgcn_perm(v1[e >> 1], v0[e >> 1], sel);
             bw[1] = __builtin_amdgcn_perm(v3[e >> 1], v2[e >> 1], sel);
             accp[e] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa, __builtin_bit_cast(half4_t, bw),
+                                                            accp[e], 0, 0, 0);
+            accp[e] = __builtin_amdgcn_mfma_f32_16x16x16f16(pb, __builtin_bit_cast(half4_t, bw),
                                                             accp[e], 0, 0, 0);
         }
     };
