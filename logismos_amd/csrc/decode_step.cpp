@@ -109,7 +109,11 @@ bool config_ok(const logismos_decode_config_t* c, int num_seqs, int t, int max_s
     if (num_seqs > 65535 || t > 65535) return false;
     if (c->num_layers <= 0 || c->hidden <= 0 || c->intermediate <= 0 || c->max_pos <= 0)
         return false;
-    if (c->head_dim != 128 || c->num_q_heads <= 0 || c->num_kv_heads <= 0) return false;
+    if (c->num_q_heads <= 0 || c->num_kv_heads <= 0) return false;
+    // heads of 128 on the kernels built for them; other multiples of 32 up to 256 on the general
+    // attention kernel (fp16 pools only: a turbo3 head row is 128 wide)
+    if (c->head_dim <= 0 || c->head_dim % 32 != 0 || c->head_dim > 256) return false;
+    if (c->head_dim != 128 && c->kv_turbo3) return false;
     if (c->hidden % 128 != 0 || c->intermediate % 128 != 0) return false;
     if (((int64_t)c->num_q_heads * c->head_dim) % 128 != 0) return false;
     // every position a block table can hold must have a row in the RoPE tables
@@ -198,7 +202,9 @@ extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_c
     const int width = qd + 2 * kvd;
     const float scale = 1.0f / sqrtf((float)c.head_dim);
     const bool one_chunk = w.chunks == 1;
-    const bool direct = one_chunk && max_q == 1;  // attention writes the o projection's input
+    // attention writes the o projection's input (the prepared layout's groups of 128 are whole
+    // heads only at head_dim 128)
+    const bool direct = one_chunk && max_q == 1 && c.head_dim == 128;
     float* const h = static_cast<float*>(batch->hidden_f32);
     auto rows_of = [&](int ch) {
         const int r0 = ch * kChunkRows;

@@ -34,6 +34,7 @@
 // + G * 256 * 2 (q, out) + 4 * ceil(ctx/block_size) (block table).
 #include "device_utils.hpp"
 #include "launch_common.hpp"
+#include "paged_attn_params.hpp"
 #include "q4_common.hpp"
 
 #include <hip/hip_fp16.h>
@@ -52,43 +53,6 @@ struct KvTile {
     half8_t k[4];
     half8_t v[4];
 };
-
-struct AttnParams {
-    const _Float16* q;
-    const _Float16* k_pool;
-    const _Float16* v_pool;
-    const int32_t* block_tables;
-    const int32_t* cu_seqlens_q;
-    const int32_t* context_lens;
-    _Float16* out;
-    float* ws_acc;  // [slot][hq][128], slot < num_seqs * num_splits
-    float* ws_ml;   // [slot][hq][2]
-    int num_seqs;
-    int hq;
-    int hkv;
-    int block_size;
-    int max_blocks_per_seq;
-    int num_splits;
-    int part_tokens;  // keys per partition (multiple of 16), static split only
-    int num_workers;  // > 0: balanced decode (see paged_attn_balanced_kernel), else static split
-    float scale_log2e;
-    int causal;
-    // 0: fp16 [T][hq][128]; 1: bf16, same shape; 2: the prepared layout of the following
-    // Q4G128 GEMM (x = [out_rows][hq*128], see q4_common.hpp) -- what the step executor uses
-    int out_bf16;
-    int out_rows;
-};
-
-__device__ __forceinline__ unsigned short attn_out_elem(float v, int out_bf16) {
-    if (out_bf16) {
-        unsigned u = __float_as_uint(v);
-        if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40u);
-        u += 0x7fffu + ((u >> 16) & 1u);
-        return (unsigned short)(u >> 16);
-    }
-    const _Float16 hv = (_Float16)v;
-    return __builtin_bit_cast(unsigned short, hv);
-}
 
 // ---- TurboQuant 3-bit pools (crates/quant/src/lib.rs): a head row is four 14-byte blocks
 // {fp16 norm, 32 x 3-bit centroid indices}.  With H the (orthonormal, symmetric) transform of
@@ -1674,16 +1638,22 @@ extern "C" logismos_status_t logismos_check_paged_attn_shape(int num_seqs, int t
     if (max_seqlen_q > total_tokens)
         return lg::reject(msg, msg_cap, "%s: max_seqlen_q = %d exceeds total_tokens = %d", k,
                           max_seqlen_q, total_tokens);
-    if (head_dim != lg::kHeadDim)
-        return lg::reject(msg, msg_cap, "%s: head_dim must be 128, got %d", k, head_dim);
+    if (head_dim % 32 != 0 || head_dim > 256)
+        return lg::reject(msg, msg_cap, "%s: head_dim must be a multiple of 32 up to 256, got %d", k,
+                          head_dim);
     if (block_size % 16 != 0)
         return lg::reject(msg, msg_cap, "%s: block_size = %d is not a multiple of 16", k, block_size);
     if (num_q_heads % num_kv_heads != 0)
         return lg::reject(msg, msg_cap, "%s: num_q_heads = %d is not a multiple of num_kv_heads = %d",
                           k, num_q_heads, num_kv_heads);
-    if (num_q_heads / num_kv_heads > 8)
-        return lg::reject(msg, msg_cap, "%s: GQA group size %d exceeds 8", k,
-                          num_q_heads / num_kv_heads);
+    // the head_dim-128 kernels keep a group of up to 8 heads in registers, the kernel for the
+    // other widths takes up to the 16 columns of a score tile
+    if (num_q_heads / num_kv_heads > (head_dim == lg::kHeadDim ? 8 : 16))
+        return lg::reject(msg, msg_cap, "%s: GQA group size %d exceeds %d at head_dim %d", k,
+                          num_q_heads / num_kv_heads, head_dim == lg::kHeadDim ? 8 : 16, head_dim);
+    if (head_dim != lg::kHeadDim && total_tokens > 65535)
+        return lg::reject(msg, msg_cap, "%s: total_tokens must be <= 65535 at head_dim %d", k,
+                          head_dim);
     if (num_seqs > 65535 || num_kv_heads > 65535)
         return lg::reject(msg, msg_cap, "%s: num_seqs and num_kv_heads must be <= 65535", k);
     const int64_t i32max = INT32_MAX;
@@ -1695,7 +1665,7 @@ extern "C" logismos_status_t logismos_check_paged_attn_shape(int num_seqs, int t
         return lg::reject(msg, msg_cap, "%s: block_size*num_kv_heads*head_dim exceeds i32::MAX", k);
     if ((int64_t)num_seqs * max_blocks_per_seq > i32max)
         return lg::reject(msg, msg_cap, "%s: num_seqs*max_blocks_per_seq exceeds i32::MAX", k);
-    if ((int64_t)num_seqs * num_splits * num_q_heads > i32max / 130)
+    if ((int64_t)num_seqs * num_splits * num_q_heads > i32max / (head_dim + 2))
         return lg::reject(msg, msg_cap, "%s: split-K workspace index exceeds i32::MAX", k);
     return 0;
 }
@@ -1869,7 +1839,7 @@ logismos_status_t lg::paged_attn_launch(
     p.context_lens = context_lens;
     p.out = static_cast<_Float16*>(out_f16);
     p.ws_acc = static_cast<float*>(workspace);
-    p.ws_ml = p.ws_acc ? p.ws_acc + (size_t)num_seqs * num_splits * num_q_heads * lg::kHeadDim
+    p.ws_ml = p.ws_acc ? p.ws_acc + (size_t)num_seqs * num_splits * num_q_heads * head_dim
                        : nullptr;
     p.num_seqs = num_seqs;
     p.hq = num_q_heads;
@@ -1886,6 +1856,12 @@ logismos_status_t lg::paged_attn_launch(
     p.out_rows = total_tokens;
 
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (head_dim != lg::kHeadDim) {
+        // turbo3 head rows and the prepared output layout are defined for 128-wide heads
+        if (kv_turbo3 || out_bf16 == 2) return hipErrorInvalidValue;
+        p.num_workers = 0;
+        return lg::paged_attn_anydim_launch(p, head_dim, total_tokens, max_seqlen_q, phases, st);
+    }
     switch (num_q_heads / num_kv_heads) {
         case 1:
             return kv_turbo3 ? lg::launch_group<1, true>(p, max_seqlen_q, phases, st)

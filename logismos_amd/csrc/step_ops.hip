@@ -264,82 +264,86 @@ __global__ __launch_bounds__(256) void silu_mul_xprep_kernel(const float* __rest
 // as they are, go to the pools at the token's slot: as fp16 rows, or (T3) rounded to fp16
 // like those and then encoded as turbo3 head rows -- the lane layout of the rotation is
 // the encoder's.
-template <bool T3>
+template <bool T3, bool D128>
 __global__ __launch_bounds__(64) void rope_kv_write_kernel(
     const uint16_t* __restrict__ qkv, const float* __restrict__ qkv_parts, int num_parts,
     int64_t part_stride, const int32_t* __restrict__ positions,
     const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     const int64_t* __restrict__ slot_mapping, __half* __restrict__ q_out,
     __half* __restrict__ k_pool, __half* __restrict__ v_pool, int hq, int hkv, int max_pos,
-    const float* __restrict__ bias) {
-    constexpr int D = 128, HALF = 64;
+    const float* __restrict__ bias, int head_dim) {
+    // 128-wide heads: one pair (i, i + 64) per lane; other widths walk their pairs 64 at a time
+    static_assert(D128 || !T3, "turbo3 head rows are 128 wide");
+    const int D = D128 ? 128 : head_dim, HALF = D / 2;
     const int head = blockIdx.x;
     const int64_t t = blockIdx.y;
-    const int i = threadIdx.x;
     const int64_t off = (t * (hq + 2 * hkv) + head) * D;
-    float x0 = 0.0f, x1 = 0.0f;
-    if (qkv) {
-        x0 = bf16_to_f32(qkv[off + i]);
-        x1 = bf16_to_f32(qkv[off + i + HALF]);
-    } else {
-        // parts are added in order; the loads of up to four parts are in flight per round
-        for_part_rounds<4>(num_parts, [&](auto nc, int q0) {
-            constexpr int N = decltype(nc)::value;
-            float a[N], b[N];
+    for (int i = threadIdx.x; i < HALF; i += 64) {
+        float x0 = 0.0f, x1 = 0.0f;
+        if (qkv) {
+            x0 = bf16_to_f32(qkv[off + i]);
+            x1 = bf16_to_f32(qkv[off + i + HALF]);
+        } else {
+            // parts are added in order; the loads of up to four parts are in flight per round
+            for_part_rounds<4>(num_parts, [&](auto nc, int q0) {
+                constexpr int N = decltype(nc)::value;
+                float a[N], b[N];
 #pragma unroll
-            for (int r = 0; r < N; ++r) {
-                a[r] = qkv_parts[(int64_t)(q0 + r) * part_stride + off + i];
-                b[r] = qkv_parts[(int64_t)(q0 + r) * part_stride + off + i + HALF];
-            }
+                for (int r = 0; r < N; ++r) {
+                    a[r] = qkv_parts[(int64_t)(q0 + r) * part_stride + off + i];
+                    b[r] = qkv_parts[(int64_t)(q0 + r) * part_stride + off + i + HALF];
+                }
 #pragma unroll
-            for (int r = 0; r < N; ++r) {
-                x0 += a[r];
-                x1 += b[r];
+                for (int r = 0; r < N; ++r) {
+                    x0 += a[r];
+                    x1 += b[r];
+                }
+            });
+        }
+        if (bias) {
+            // the projection's bias (`linear_t`, one fp32 add on the finished sum), column
+            // head*D + i
+            x0 += bias[head * D + i];
+            x1 += bias[head * D + i + HALF];
+        }
+        if (head < hq + hkv) {
+            int pos = positions[t];
+            pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
+            const float c = cos_t[(int64_t)pos * HALF + i];
+            const float s = sin_t[(int64_t)pos * HALF + i];
+            const float y0 = x0 * c - x1 * s;
+            const float y1 = x0 * s + x1 * c;
+            if (head < hq) {
+                __half* dst = q_out + (t * hq + head) * D;
+                dst[i] = __float2half_rn(y0);
+                dst[i + HALF] = __float2half_rn(y1);
+            } else {
+                const int64_t slot = slot_mapping[t];
+                if (slot < 0) return;
+                if constexpr (T3) {
+                    turbo3_encode_row(__half2float(__float2half_rn(y0)),
+                                      __half2float(__float2half_rn(y1)), i,
+                                      reinterpret_cast<uint8_t*>(k_pool) +
+                                          (slot * hkv + (head - hq)) * kTurbo3HeadBytes);
+                } else {
+                    __half* dst = k_pool + (slot * hkv + (head - hq)) * D;
+                    dst[i] = __float2half_rn(y0);
+                    dst[i + HALF] = __float2half_rn(y1);
+                }
             }
-        });
-    }
-    if (bias) {
-        // the projection's bias (`linear_t`, one fp32 add on the finished sum), column head*D + i
-        x0 += bias[head * D + i];
-        x1 += bias[head * D + i + HALF];
-    }
-    if (head < hq + hkv) {
-        int pos = positions[t];
-        pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
-        const float c = cos_t[(int64_t)pos * HALF + i];
-        const float s = sin_t[(int64_t)pos * HALF + i];
-        const float y0 = x0 * c - x1 * s;
-        const float y1 = x0 * s + x1 * c;
-        if (head < hq) {
-            __half* dst = q_out + (t * hq + head) * D;
-            dst[i] = __float2half_rn(y0);
-            dst[i + HALF] = __float2half_rn(y1);
         } else {
             const int64_t slot = slot_mapping[t];
             if (slot < 0) return;
             if constexpr (T3) {
-                turbo3_encode_row(__half2float(__float2half_rn(y0)),
-                                  __half2float(__float2half_rn(y1)), i,
-                                  reinterpret_cast<uint8_t*>(k_pool) +
-                                      (slot * hkv + (head - hq)) * kTurbo3HeadBytes);
+                turbo3_encode_row(__half2float(__float2half_rn(x0)),
+                                  __half2float(__float2half_rn(x1)), i,
+                                  reinterpret_cast<uint8_t*>(v_pool) +
+                                      (slot * hkv + (head - hq - hkv)) * kTurbo3HeadBytes);
             } else {
-                __half* dst = k_pool + (slot * hkv + (head - hq)) * D;
-                dst[i] = __float2half_rn(y0);
-                dst[i + HALF] = __float2half_rn(y1);
+                __half* dst = v_pool + (slot * hkv + (head - hq - hkv)) * D;
+                dst[i] = __float2half_rn(x0);
+                dst[i + HALF] = __float2half_rn(x1);
             }
-        }
-    } else {
-        const int64_t slot = slot_mapping[t];
-        if (slot < 0) return;
-        if constexpr (T3) {
-            turbo3_encode_row(__half2float(__float2half_rn(x0)), __half2float(__float2half_rn(x1)),
-                              i,
-                              reinterpret_cast<uint8_t*>(v_pool) +
-                                  (slot * hkv + (head - hq - hkv)) * kTurbo3HeadBytes);
-        } else {
-            __half* dst = v_pool + (slot * hkv + (head - hq - hkv)) * D;
-            dst[i] = __float2half_rn(x0);
-            dst[i + HALF] = __float2half_rn(x1);
         }
     }
 }
@@ -471,7 +475,9 @@ extern "C" logismos_status_t logismos_launch_rope_kv_write_fp16(
     logismos_stream_t stream) {
     if (total_tokens < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || max_pos <= 0)
         return hipErrorInvalidValue;
-    if (head_dim != 128 || total_tokens > 65535) return hipErrorInvalidValue;
+    // an even number of elements per head (a rotation pair is (i, i + head_dim / 2))
+    if (head_dim <= 0 || head_dim % 2 != 0 || head_dim > 1024 || total_tokens > 65535)
+        return hipErrorInvalidValue;
     if ((int64_t)total_tokens * (num_q_heads + 2 * num_kv_heads) * head_dim > (int64_t)INT32_MAX)
         return hipErrorInvalidValue;
     if (total_tokens == 0) return hipSuccess;
@@ -479,12 +485,14 @@ extern "C" logismos_status_t logismos_launch_rope_kv_write_fp16(
         !k_pool_f16 || !v_pool_f16)
         return hipErrorInvalidValue;
     dim3 grid(num_q_heads + 2 * num_kv_heads, total_tokens);
-    lg::rope_kv_write_kernel<false><<<grid, dim3(64), 0, static_cast<hipStream_t>(stream)>>>(
+    const auto kernel = head_dim == 128 ? lg::rope_kv_write_kernel<false, true>
+                                        : lg::rope_kv_write_kernel<false, false>;
+    kernel<<<grid, dim3(64), 0, static_cast<hipStream_t>(stream)>>>(
         static_cast<const uint16_t*>(qkv_bf16), nullptr, 0, 0, positions,
         static_cast<const float*>(cos_f32),
         static_cast<const float*>(sin_f32), slot_mapping, static_cast<__half*>(q_out_f16),
         static_cast<__half*>(k_pool_f16), static_cast<__half*>(v_pool_f16), num_q_heads,
-        num_kv_heads, max_pos, nullptr);
+        num_kv_heads, max_pos, nullptr, head_dim);
     return hipGetLastError();
 }
 
@@ -495,7 +503,9 @@ extern "C" logismos_status_t logismos_launch_rope_kv_write_f32p_bias(
     int head_dim, int max_pos, logismos_stream_t stream) {
     if (total_tokens < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || max_pos <= 0 || num_parts <= 0)
         return hipErrorInvalidValue;
-    if (head_dim != 128 || total_tokens > 65535) return hipErrorInvalidValue;
+    // an even number of elements per head (a rotation pair is (i, i + head_dim / 2))
+    if (head_dim <= 0 || head_dim % 2 != 0 || head_dim > 1024 || total_tokens > 65535)
+        return hipErrorInvalidValue;
     const int64_t width = (int64_t)(num_q_heads + 2 * num_kv_heads) * head_dim;
     if ((int64_t)total_tokens * width > (int64_t)INT32_MAX) return hipErrorInvalidValue;
     if (total_tokens == 0) return hipSuccess;
@@ -503,12 +513,14 @@ extern "C" logismos_status_t logismos_launch_rope_kv_write_f32p_bias(
         !k_pool_f16 || !v_pool_f16)
         return hipErrorInvalidValue;
     dim3 grid(num_q_heads + 2 * num_kv_heads, total_tokens);
-    lg::rope_kv_write_kernel<false><<<grid, dim3(64), 0, static_cast<hipStream_t>(stream)>>>(
+    const auto kernel = head_dim == 128 ? lg::rope_kv_write_kernel<false, true>
+                                        : lg::rope_kv_write_kernel<false, false>;
+    kernel<<<grid, dim3(64), 0, static_cast<hipStream_t>(stream)>>>(
         nullptr, static_cast<const float*>(qkv_parts_f32), num_parts, (int64_t)total_tokens * width,
         positions, static_cast<const float*>(cos_f32), static_cast<const float*>(sin_f32),
         slot_mapping, static_cast<__half*>(q_out_f16), static_cast<__half*>(k_pool_f16),
         static_cast<__half*>(v_pool_f16), num_q_heads, num_kv_heads, max_pos,
-        static_cast<const float*>(bias_f32));
+        static_cast<const float*>(bias_f32), head_dim);
     return hipGetLastError();
 }
 
@@ -539,12 +551,12 @@ extern "C" logismos_status_t logismos_launch_rope_kv_write_f32p_turbo3_bias(
         !k_pool_t3 || !v_pool_t3)
         return hipErrorInvalidValue;
     dim3 grid(num_q_heads + 2 * num_kv_heads, total_tokens);
-    lg::rope_kv_write_kernel<true><<<grid, dim3(64), 0, static_cast<hipStream_t>(stream)>>>(
+    lg::rope_kv_write_kernel<true, true><<<grid, dim3(64), 0, static_cast<hipStream_t>(stream)>>>(
         nullptr, static_cast<const float*>(qkv_parts_f32), num_parts, (int64_t)total_tokens * width,
         positions, static_cast<const float*>(cos_f32), static_cast<const float*>(sin_f32),
         slot_mapping, static_cast<__half*>(q_out_f16), static_cast<__half*>(k_pool_t3),
         static_cast<__half*>(v_pool_t3), num_q_heads, num_kv_heads, max_pos,
-        static_cast<const float*>(bias_f32));
+        static_cast<const float*>(bias_f32), 128);
     return hipGetLastError();
 }
 

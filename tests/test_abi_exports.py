@@ -66,7 +66,10 @@ def test_qgemv_q8_shape_guard_accepts_config1():
 
 @pytest.mark.parametrize("args,frag", [
     (dict(num_seqs=0), "num_seqs must be positive"),
-    (dict(head_dim=64), "head_dim must be 128"),
+    (dict(head_dim=80), "head_dim must be a multiple of 32 up to 256"),
+    (dict(head_dim=288), "head_dim must be a multiple of 32 up to 256"),
+    (dict(head_dim=64, num_q_heads=34, num_kv_heads=2), "group size 17 exceeds 16"),
+    (dict(head_dim=64, num_seqs=2, total_tokens=70000, max_seqlen_q=40000), "<= 65535"),
     (dict(block_size=24), "multiple of 16"),
     (dict(num_q_heads=12, num_kv_heads=5), "not a multiple of num_kv_heads"),
     (dict(num_q_heads=32, num_kv_heads=2), "group size 16 exceeds 8"),
@@ -88,7 +91,7 @@ def test_launchers_reject_bad_shapes_with_invalid_value_and_do_not_touch_the_dev
     lib = kernels.library()
     assert lib.logismos_launch_qgemv_q8g32_f32(None, None, None, None, 8, 48, None) == 1
     assert lib.logismos_launch_paged_attn_varlen_fp16(
-        None, None, None, None, None, None, None, None, 16, 16, 1, 12, 2, 64, 16, 8, 1, 0.1, 1,
+        None, None, None, None, None, None, None, None, 16, 16, 1, 12, 2, 80, 16, 8, 1, 0.1, 1,
         None) == 1
 
 

@@ -216,6 +216,31 @@ def test_full_layer_mixed_batch_at_qwen3_8b_geometry():
     assert np.all(np.abs(got - want) <= 1.2e-2 + 1.6e-2 * np.abs(want))
 
 
+def test_step_at_qwen2_05b_geometry_head_dim_64():
+    # Qwen2-0.5B's layer geometry: hidden 896, 14 query / 2 KV heads of 64, MLP 4864, q/k/v
+    # biases (crates/transformers/src/attention.rs:49-57); decode rows only, two layers
+    rng = np.random.default_rng(64)
+    ctx = rng.integers(1, 700, size=12)
+    cfg, layers, batch = workloads.decode_step_problem(
+        rng, num_layers=2, hidden=896, hq=14, hkv=2, inter=4864, ctx=ctx, d=64, qkv_bias=True,
+        theta=1e4)
+    _check_step(cfg, layers, batch, "head_dim 64, decode rows", 2)
+
+
+@pytest.mark.parametrize("d,hq,hkv,hidden", [(64, 8, 2, 512), (96, 4, 4, 384), (256, 2, 1, 512)])
+def test_mixed_batch_at_other_head_dims(d, hq, hkv, hidden):
+    # decode rows and chunks in one chunk of rows, then over three chunks of rows
+    rng = np.random.default_rng(640 + d)
+    cfg, layers, batch = workloads.decode_step_problem(
+        rng, num_layers=2, hidden=hidden, hq=hq, hkv=hkv, inter=1024, ctx=[90, 400, 3, 21],
+        new_tokens=[1, 7, 3, 5], d=d, qkv_bias=True)
+    _check_step(cfg, layers, batch, f"head_dim {d}, one chunk", 2)
+    cfg, layers, batch = workloads.decode_step_problem(
+        rng, num_layers=1, hidden=hidden, hq=hq, hkv=hkv, inter=1024, ctx=[300, 40, 70, 9, 33],
+        new_tokens=[1, 40, 30, 1, 8], d=d)
+    _check_step(cfg, layers, batch, f"head_dim {d}, three chunks", 1)
+
+
 def test_step_rejects_what_it_cannot_run():
     import ctypes as C
     rng = np.random.default_rng(41)

@@ -61,6 +61,56 @@ def test_rope_kv_write_matches_oracle_and_reference_table():
     assert np.array_equal(q_got[0], x0.astype(np.float16))
 
 
+@pytest.mark.parametrize("d", [32, 64, 96, 256])
+def test_rope_kv_write_at_other_head_dims(d):
+    # the rotation pairs (i, i + d/2) of `rope_halves_in_place`
+    # (crates/kernels/src/cpu_f32/mod.rs:599-619) at head widths other than 128, from bf16
+    # rows and from fp32 split-K parts with a bias
+    rng = np.random.default_rng(210 + d)
+    t, hq, hkv, bs, nblk, max_pos = 9, 6, 2, 16, 12, 2048
+    width = (hq + 2 * hkv) * d
+    positions = np.array([0, 1, 17, 2047, 300, 2046, 2, 5, 1000], np.int32)
+    slots = rng.permutation(nblk * bs)[:t].astype(np.int64)
+    slots[3] = -1
+    cos, sin = O.build_rope_table_f32(max_pos, d, 10_000.0)
+    k0 = rng.standard_normal((nblk * bs, hkv * d), np.float32).astype(np.float16)
+    v0 = rng.standard_normal((nblk * bs, hkv * d), np.float32).astype(np.float16)
+    dev = hip.DeviceBuffer.from_numpy
+
+    qkv = O.f32_to_bf16_bits(rng.standard_normal((t, width), np.float32))
+    k_pool, v_pool = k0.copy(), v0.copy()
+    d_kp, d_vp, d_q = dev(k_pool), dev(v_pool), hip.DeviceBuffer(t * hq * d * 2)
+    kernels.launch_rope_kv_write_fp16(dev(qkv), dev(positions), dev(cos), dev(sin), dev(slots),
+                                      d_q, d_kp, d_vp, t, hq, hkv, d, max_pos)
+    hip.synchronize()
+    q_want = OS.rope_kv_write(qkv, positions, cos, sin, slots, k_pool, v_pool, hq, hkv, d)
+    q_got = d_q.to_numpy(np.float16, (t, hq, d))
+    assert_parity(q_got, q_want, max_abs=1e-3, max_rel=2e-3, what=f"rope q d={d}")
+    assert_parity(d_kp.to_numpy(np.float16, k_pool.shape), k_pool, max_abs=1e-3, max_rel=2e-3,
+                  what=f"rope k pool d={d}")
+    assert np.array_equal(d_vp.to_numpy(np.float16, v_pool.shape).view(np.uint16),
+                          v_pool.view(np.uint16))
+    x0 = O.bf16_bits_to_f32(qkv[0]).reshape(hq + 2 * hkv, d)[:hq]
+    assert np.array_equal(q_got[0], x0.astype(np.float16))  # position 0: identity
+
+    parts = rng.standard_normal((3, t, width), np.float32)
+    bias = rng.standard_normal(width).astype(np.float32)
+    k_pool, v_pool = k0.copy(), v0.copy()
+    d_kp, d_vp, d_q = dev(k_pool), dev(v_pool), hip.DeviceBuffer(t * hq * d * 2)
+    kernels.launch_rope_kv_write_f32p(dev(parts), 3, dev(positions), dev(cos), dev(sin),
+                                      dev(slots), d_q, d_kp, d_vp, t, hq, hkv, d, max_pos,
+                                      bias=dev(bias))
+    hip.synchronize()
+    q_want = OS.rope_kv_write(parts[0] + parts[1] + parts[2] + bias, positions, cos, sin, slots,
+                              k_pool, v_pool, hq, hkv, d)
+    assert_parity(d_q.to_numpy(np.float16, (t, hq, d)), q_want, max_abs=1e-3, max_rel=2e-3,
+                  what=f"rope_f32p q d={d}")
+    assert_parity(d_kp.to_numpy(np.float16, k_pool.shape), k_pool, max_abs=1e-3, max_rel=2e-3,
+                  what=f"rope_f32p k d={d}")
+    assert_parity(d_vp.to_numpy(np.float16, v_pool.shape), v_pool, max_abs=1e-3, max_rel=2e-3,
+                  what=f"rope_f32p v d={d}")
+
+
 def test_silu_mul_and_cast():
     rng = np.random.default_rng(22)
     rows, inter = 5, 1000
