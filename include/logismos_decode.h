@@ -265,6 +265,13 @@ logismos_status_t logismos_launch_repack_q8_0(const void* blocks_q8_0, void* qs_
 int logismos_paged_attn_num_splits(int num_seqs, int num_kv_heads, int block_size,
                                    int max_blocks_per_seq);
 
+/* The same for a given head width.  head_dim 128: what the function above returns.  Other
+ * widths (multiples of 32 up to 256, `crates/transformers/src/attention.rs:97-127` is
+ * generic in head_dim) run on a general kernel with a static split, whose partition count
+ * this sizes for its workgroups (one per partition and group of up to 8 KV heads). */
+int logismos_paged_attn_num_splits_hd(int num_seqs, int num_kv_heads, int head_dim,
+                                      int block_size, int max_blocks_per_seq);
+
 /* Bytes of split-K workspace the launcher needs for these arguments. */
 size_t logismos_paged_attn_workspace_bytes(int num_seqs, int num_q_heads, int head_dim,
                                            int num_splits);

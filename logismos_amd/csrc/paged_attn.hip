@@ -1696,6 +1696,15 @@ extern "C" int logismos_paged_attn_num_splits(int num_seqs, int num_kv_heads, in
     return (int)splits;
 }
 
+extern "C" int logismos_paged_attn_num_splits_hd(int num_seqs, int num_kv_heads, int head_dim,
+                                                 int block_size, int max_blocks_per_seq) {
+    if (head_dim == lg::kHeadDim)
+        return logismos_paged_attn_num_splits(num_seqs, num_kv_heads, block_size,
+                                              max_blocks_per_seq);
+    return lg::paged_attn_anydim_num_splits(num_seqs, num_kv_heads, head_dim, block_size,
+                                            max_blocks_per_seq);
+}
+
 extern "C" size_t logismos_paged_attn_workspace_bytes(int num_seqs, int num_q_heads, int head_dim,
                                                       int num_splits) {
     if (num_seqs <= 0 || num_q_heads <= 0 || head_dim <= 0 || num_splits <= 1) return 0;

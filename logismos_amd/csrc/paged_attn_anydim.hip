@@ -4,13 +4,24 @@
 // of crates/transformers/src/attention.rs:233-260), not tuned to their degree: one kernel for
 // every row of the ragged batch.
 //
-// One wave64 owns one (query token, KV head, KV partition) and serves the whole GQA group.
+// One wave64 serves the whole GQA group of one KV head over 16-key tiles of one (query
+// token, KV partition).  A workgroup of up to eight waves is (KV heads) x (tile phases): its
+// waves of different heads read the same token rows, so the workgroup streams runs of whole
+// rows (a wave alone reads one head's 2 * head_dim bytes out of every row); with fewer than
+// eight KV heads the waves of a head take the partition's tiles in turn (phase f the tiles
+// f, f + F, ...) and their (m, l, acc) states are combined through LDS at the end.
 // Per tile of 16 keys (a tile never straddles a KV block: block_size % 16 == 0), with
 // lane = (tg = lane / 16, c = lane % 16):
-//   * scores on v_mfma_f32_16x16x32_f16: A = K (lane: key c, elements 32j + 8tg .. + 8 of
-//     piece j, one 16-byte load per piece), B = the query group (column c = head c, same
-//     pieces, kept in registers); head_dim / 32 MFMAs give 16 keys x 16 heads, lane (tg, c)
-//     holding head c for the keys 4tg .. 4tg + 3.
+//   * scores on v_mfma_f32_16x16x32_f16: A = K (lane: key c, 8 elements per MFMA), B = the
+//     query group (column c = head c, the same elements, kept in registers); head_dim / 32
+//     MFMAs give 16 keys x 16 heads, lane (tg, c) holding head c for the keys 4tg .. 4tg + 3.
+//     Which elements a lane contributes to which MFMA is free as long as K and q agree.
+//     head_dim a multiple of 64 (head rows are whole 128-byte lines): a request covers 8 keys
+//     x one line (lane (tg, c): 16-byte piece 2tg + c/8 of key c%8; keys 8..15 in a second
+//     request), and the lanes c and c + 8 then swap halves (DPP row_ror:8), which leaves lane
+//     (tg, c) with the pieces 2tg, 2tg + 1 of key c per line -- requests whose neighbouring
+//     lanes read neighbouring bytes.  Other widths: lane (tg, c) loads the elements
+//     32j + 8tg .. + 8 of key c directly (neighbouring lanes on different rows).
 //   * one running maximum per head shared by the four lane rows, sums per lane row.
 //   * P.V on v_mfma_f32_16x16x16_f16: A = the probabilities as two fp16 terms (head c, keys
 //     4tg + r: the layout the scores arrive in), B = V (lane: E = head_dim / 16 consecutive
@@ -26,6 +37,7 @@
 #include "device_utils.hpp"
 #include "launch_common.hpp"
 #include "paged_attn_params.hpp"
+#include "q4_common.hpp"
 
 #include <math.h>
 
@@ -34,38 +46,43 @@ namespace lg {
 namespace {
 
 constexpr int kAnyTileKeys = 16;
+constexpr int kAnyWaves = 8;           // waves of a workgroup: KV heads x tile phases
+constexpr int kAnyLdsBytes = 48 * 1024;  // for the accumulators of the phases beyond the first
+constexpr int kAnyWgHeads = 8;           // KV heads per workgroup at most
+constexpr int kAnyPhases = 8;            // tile phases per head at most
+
+// KV heads per workgroup: the largest divisor of hkv up to kAnyWgHeads
+int anydim_wg_heads(int hkv) {
+    for (int w = kAnyWgHeads; w > 1; --w)
+        if (hkv % w == 0) return w;
+    return 1;
+}
 
 template <int NJ>
 struct AnyTile {
     half8_t k[NJ];
-    _Float16 v[4][2 * NJ];
+    unsigned v[4][NJ];  // key 4tg + r: the lane's 2 NJ elements, two per dword
 };
 
-// E consecutive fp16 values; 2E bytes, aligned to 4 (E is even)
-template <int E>
-__device__ __forceinline__ void load_halves(const _Float16* src, _Float16 (&dst)[E]) {
-    if constexpr (E % 8 == 0) {
+typedef unsigned __attribute__((ext_vector_type(4), aligned(4))) uint4_a4_t;
+typedef unsigned __attribute__((ext_vector_type(2), aligned(4))) uint2_a4_t;
+
+// N consecutive dwords, aligned to 4 bytes, in as few requests as N allows
+template <int N>
+__device__ __forceinline__ void load_dwords(const void* src, unsigned (&dst)[N]) {
+    const unsigned* sp = static_cast<const unsigned*>(src);
+    int i = 0;
 #pragma unroll
-        for (int i = 0; i < E / 8; ++i) {
-            const half8_t x = *reinterpret_cast<const half8_t*>(src + 8 * i);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) dst[8 * i + e] = x[e];
-        }
-    } else if constexpr (E % 4 == 0) {
-#pragma unroll
-        for (int i = 0; i < E / 4; ++i) {
-            const half4_t x = *reinterpret_cast<const half4_t*>(src + 4 * i);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) dst[4 * i + e] = x[e];
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < E / 2; ++i) {
-            const half2_t x = *reinterpret_cast<const half2_t*>(src + 2 * i);
-            dst[2 * i] = x[0];
-            dst[2 * i + 1] = x[1];
-        }
+    for (; i + 4 <= N; i += 4) {
+        const uint4_a4_t x = *reinterpret_cast<const uint4_a4_t*>(sp + i);
+        dst[i] = x[0], dst[i + 1] = x[1], dst[i + 2] = x[2], dst[i + 3] = x[3];
     }
+    if (N - i >= 2) {
+        const uint2_a4_t x = *reinterpret_cast<const uint2_a4_t*>(sp + i);
+        dst[i] = x[0], dst[i + 1] = x[1];
+        i += 2;
+    }
+    if (N - i == 1) dst[i] = sp[i];
 }
 
 __device__ __forceinline__ float lane_read_f32(float v, int src_lane) {
@@ -84,14 +101,23 @@ __device__ __forceinline__ int seq_of_row(const int32_t* cu, int num_seqs, int t
 }
 
 template <int NJ>
-__global__ __launch_bounds__(64) void paged_attn_anydim_kernel(const AttnParams p, int G,
-                                                               int decode_rows) {
+__global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_kernel(const AttnParams p,
+                                                                           int G,
+                                                                           int decode_rows,
+                                                                           int wg_heads,
+                                                                           int phases) {
     constexpr int D = 32 * NJ;
     constexpr int E = 2 * NJ;
-    const int lane = threadIdx.x;
+    constexpr bool kLines = NJ % 2 == 0;  // head rows are whole 128-byte lines
+    __shared__ float sm_m[kAnyWaves][16], sm_l[kAnyWaves][16];  // [phase * wg_heads + head]
+    extern __shared__ float sm_acc[];  // [phases - 1][wg_heads][G][D]
+    // (the wave index as a scalar: tile positions and block ids stay in scalar registers, the
+    // block table is read with scalar loads)
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int c = lane & 15, tg = lane >> 4;
     const int split = blockIdx.x;
-    const int kvh = blockIdx.y;
+    const int wg_head = wave % wg_heads, phase = wave / wg_heads;
+    const int kvh = blockIdx.y * wg_heads + wg_head;
     // decode launch: grid.z walks the sequences and takes those with one new token;
     // the other launch walks the packed rows and takes those of the other sequences
     const int s = decode_rows ? (int)blockIdx.z : seq_of_row(p.cu_seqlens_q, p.num_seqs, blockIdx.z);
@@ -116,7 +142,7 @@ __global__ __launch_bounds__(64) void paged_attn_anydim_kernel(const AttnParams 
     if (visible <= 0) {
         // no visible key: a row of zeros (written once)
         if (split == 0)
-            for (int i = lane; i < G * D; i += 64) out_row[i] = (_Float16)0.0f;
+            for (int i = lane + 64 * phase; i < G * D; i += 64 * phases) out_row[i] = (_Float16)0.0f;
         return;
     }
     if (key_begin >= key_end) return;
@@ -124,10 +150,12 @@ __global__ __launch_bounds__(64) void paged_attn_anydim_kernel(const AttnParams 
     // the query group as the B operand: column c = head c (zero beyond the group)
     half8_t qb[NJ];
     {
-        const _Float16* qp = p.q + ((int64_t)t * p.hq + (int64_t)kvh * G + (c < G ? c : 0)) * D + 8 * tg;
+        const _Float16* qp = p.q + ((int64_t)t * p.hq + (int64_t)kvh * G + (c < G ? c : 0)) * D;
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
-            qb[j] = *reinterpret_cast<const half8_t*>(qp + 32 * j);
+            // (the element order of the K operand, see load_tile / k_operand)
+            const int off = kLines ? 64 * (j >> 1) + 16 * tg + 8 * (j & 1) : 32 * j + 8 * tg;
+            qb[j] = *reinterpret_cast<const half8_t*>(qp + off);
             if (c >= G) qb[j] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
         }
     }
@@ -135,20 +163,33 @@ __global__ __launch_bounds__(64) void paged_attn_anydim_kernel(const AttnParams 
     const int64_t row_halves = (int64_t)p.hkv * D;
     const int last_key = key_end - 1;
 
-    auto load_tile = [&](int tile_begin, AnyTile<NJ>& tl) {
-        const int block = table[tile_begin / p.block_size];
-        const int64_t base = (int64_t)block * p.block_size + tile_begin % p.block_size;
+    auto load_tile = [&](int tile_begin, int block, int off_in_block, AnyTile<NJ>& tl) {
+        const int64_t base = (int64_t)block * p.block_size + off_in_block;
         // keys past the end of the range read the last key of the range and are masked
         const int over = tile_begin + 15 - last_key;  // > 0: the tile runs past the range
-        const int kk = (over > 0 && c > 15 - over) ? 15 - over : c;
-        const _Float16* kp = p.k_pool + (base + kk) * row_halves + (int64_t)kvh * D + 8 * tg;
+        if constexpr (kLines) {
+            // k[2u + kh]: piece 2tg + c/8 of line u of key 8kh + c%8
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) tl.k[j] = *reinterpret_cast<const half8_t*>(kp + 32 * j);
+            for (int kh = 0; kh < 2; ++kh) {
+                const int key = 8 * kh + (c & 7);
+                const int kk = (over > 0 && key > 15 - over) ? 15 - over : key;
+                const _Float16* kp = p.k_pool + (base + kk) * row_halves + (int64_t)kvh * D +
+                                     16 * tg + 8 * (c >> 3);
+#pragma unroll
+                for (int u = 0; u < NJ / 2; ++u)
+                    tl.k[2 * u + kh] = *reinterpret_cast<const half8_t*>(kp + 64 * u);
+            }
+        } else {
+            const int kk = (over > 0 && c > 15 - over) ? 15 - over : c;
+            const _Float16* kp = p.k_pool + (base + kk) * row_halves + (int64_t)kvh * D + 8 * tg;
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) tl.k[j] = *reinterpret_cast<const half8_t*>(kp + 32 * j);
+        }
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int key = 4 * tg + r;
             const int vk = (over > 0 && key > 15 - over) ? 15 - over : key;
-            load_halves<E>(p.v_pool + (base + vk) * row_halves + (int64_t)kvh * D + E * c, tl.v[r]);
+            load_dwords<NJ>(p.v_pool + (base + vk) * row_halves + (int64_t)kvh * D + E * c, tl.v[r]);
         }
     };
 
@@ -159,9 +200,27 @@ __global__ __launch_bounds__(64) void paged_attn_anydim_kernel(const AttnParams 
 
     auto compute_tile = [&](int tile_begin, const AnyTile<NJ>& tl) {
         float4_t sacc = {0.0f, 0.0f, 0.0f, 0.0f};
+        if constexpr (kLines) {
+            // lane c < 8 holds (key c, key c + 8), lane c >= 8 (key c - 8, key c) of its
+            // piece: each sends the one its partner c ^ 8 needs and keeps its own key's
 #pragma unroll
-        for (int j = 0; j < NJ; ++j)
-            sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(tl.k[j], qb[j], sacc, 0, 0, 0);
+            for (int u = 0; u < NJ / 2; ++u) {
+                const uint4_t r0 = __builtin_bit_cast(uint4_t, tl.k[2 * u]);
+                const uint4_t r1 = __builtin_bit_cast(uint4_t, tl.k[2 * u + 1]);
+                uint4_t recv;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    recv[i] = (unsigned)lane_xor_i32<8>((int)(c < 8 ? r1[i] : r0[i]));
+                const half8_t a0 = __builtin_bit_cast(half8_t, c < 8 ? r0 : recv);
+                const half8_t a1 = __builtin_bit_cast(half8_t, c < 8 ? recv : r1);
+                sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, qb[2 * u], sacc, 0, 0, 0);
+                sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, qb[2 * u + 1], sacc, 0, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+                sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(tl.k[j], qb[j], sacc, 0, 0, 0);
+        }
         float sc[4];
         float tmax = -INFINITY;
 #pragma unroll
@@ -193,29 +252,99 @@ __global__ __launch_bounds__(64) void paged_attn_anydim_kernel(const AttnParams 
         for (int e = 0; e < E; ++e) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[e][r] *= ar[r];
-            const half4_t vb = {tl.v[0][e], tl.v[1][e], tl.v[2][e], tl.v[3][e]};
+            // B = element e of the lane's four keys: the low or high halves of their dwords e/2
+            const unsigned sel = (e & 1) ? 0x07060302u : 0x05040100u;
+            const uint2_t bw = {__builtin_amdgcn_perm(tl.v[1][e >> 1], tl.v[0][e >> 1], sel),
+                                __builtin_amdgcn_perm(tl.v[3][e >> 1], tl.v[2][e >> 1], sel)};
+            const half4_t vb = __builtin_bit_cast(half4_t, bw);
             acc[e] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa, vb, acc[e], 0, 0, 0);
             acc[e] = __builtin_amdgcn_mfma_f32_16x16x16f16(pb, vb, acc[e], 0, 0, 0);
         }
     };
 
-    AnyTile<NJ> cur, nxt;
-    load_tile(key_begin, cur);
-    for (int tb = key_begin; tb < key_end; tb += kAnyTileKeys) {
-        const bool more = tb + kAnyTileKeys < key_end;
-        if (more) load_tile(tb + kAnyTileKeys, nxt);
-        compute_tile(tb, cur);
-        if (more) cur = nxt;
+    {
+        // Two tile buffers in turn, straight-line: the requests of one tile are in flight while
+        // the other is consumed, and the block id of a tile is read (a scalar load) a tile
+        // before its requests.  A position past the wave's last tile stays on the last tile:
+        // every request is unconditional and reads memory the range owns; what was read twice
+        // is not consumed.
+        const int kStep = kAnyTileKeys * phases;
+        const int tb0 = key_begin + kAnyTileKeys * phase;
+        if (tb0 < key_end) {
+            const int n_tiles = (key_end - tb0 + kStep - 1) / kStep;
+            int tb = tb0, bi = tb0 / p.block_size, bo = tb0 - bi * p.block_size;
+            auto advance = [&]() {
+                if (tb + kStep < key_end) {
+                    tb += kStep;
+                    bo += kStep;
+                    while (bo >= p.block_size) {
+                        bo -= p.block_size;
+                        ++bi;
+                    }
+                }
+            };
+            AnyTile<NJ> ta, tc;
+            int tb_a = tb, bo_a = bo, id_a = table[bi];
+            advance();
+            int tb_c = tb, bo_c = bo, id_c = table[bi];
+            load_tile(tb_a, id_a, bo_a, ta);
+            for (int i = 0; i < n_tiles; i += 2) {
+                load_tile(tb_c, id_c, bo_c, tc);
+                advance();
+                const int tb_a2 = tb, bo_a2 = bo, id_a2 = table[bi];
+                compute_tile(tb_a, ta);
+                load_tile(tb_a2, id_a2, bo_a2, ta);
+                tb_a = tb_a2;
+                advance();
+                const int tb_c2 = tb, bo_c2 = bo, id_c2 = table[bi];
+                if (i + 1 < n_tiles) compute_tile(tb_c, tc);
+                tb_c = tb_c2, bo_c = bo_c2, id_c = id_c2;
+            }
+        }
     }
 
+    // ---- the states of a head's phases into its phase 0: M = max m_f, factors 2^(m_f - M).
+    // A wave without a tile has m = -inf, l = 0, acc = 0 and factor 0; phase 0 always has one.
     float lsum = l + lane_xor_f32<16>(l);
     lsum += lane_xor_f32<32>(lsum);
+    if (tg == 0) {
+        sm_m[wave][c] = m;
+        sm_l[wave][c] = lsum;
+    }
+    __syncthreads();
+    float mall = m, lall = 0.0f;
+    for (int f = 0; f < phases; ++f) mall = fmaxf(mall, sm_m[f * wg_heads + wg_head][c]);
+    for (int f = 0; f < phases; ++f)
+        lall += fast_exp2(sm_m[f * wg_heads + wg_head][c] - mall) * sm_l[f * wg_heads + wg_head][c];
+    const float fown = fast_exp2(m - mall);
+    float fr[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) fr[r] = lane_read_f32(fown, (lane & 48) | (4 * tg + r));
+    if (phase > 0) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int h = 4 * tg + r;
+            if (h >= G) continue;
+            float* dst = sm_acc + (((phase - 1) * wg_heads + wg_head) * G + h) * D + E * c;
+#pragma unroll
+            for (int e = 0; e < E; ++e) dst[e] = acc[e][r] * fr[r];
+        }
+    }
+    __syncthreads();
+    if (phase > 0) return;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int h = 4 * tg + r;
-        const float mh = lane_read_f32(m, (lane & 48) | h);
-        const float lh = lane_read_f32(lsum, (lane & 48) | h);
+        const float mh = lane_read_f32(mall, (lane & 48) | h);
+        const float lh = lane_read_f32(lall, (lane & 48) | h);
         if (h >= G) continue;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            float a = acc[e][r] * fr[r];
+            for (int f = 0; f < phases - 1; ++f)
+                a += sm_acc[((f * wg_heads + wg_head) * G + h) * D + E * c + e];
+            acc[e][r] = a;
+        }
         const int head = kvh * G + h;
         if (single) {
             const float inv = 1.0f / lh;
@@ -241,8 +370,12 @@ __global__ __launch_bounds__(64) void paged_attn_anydim_kernel(const AttnParams 
 }
 
 // Decode rows with more than one partition: out = sum_p w_p acc_p / sum_p w_p l_p,
-// w_p = 2^(m_p - max m).  grid (hq, num_seqs), one thread per element pair.
-__global__ __launch_bounds__(128) void paged_attn_anydim_merge_kernel(const AttnParams p, int D) {
+// w_p = 2^(m_p - max m).  grid (hq, num_seqs), 256 threads: thread = (stripe, element pair),
+// stripe j sums the partitions j, j + S, ...; the stripes are added through LDS.
+__global__ __launch_bounds__(256) void paged_attn_anydim_merge_kernel(const AttnParams p, int D) {
+    __shared__ float sm_red[4];
+    __shared__ float sm_a[256][2];
+    __shared__ float sm_lt[128];
     const int head = blockIdx.x;
     const int s = blockIdx.y;
     const int t = p.cu_seqlens_q[s];
@@ -251,39 +384,93 @@ __global__ __launch_bounds__(128) void paged_attn_anydim_merge_kernel(const Attn
     if (ctx <= p.part_tokens) return;  // zero or one partition: already final
     const int parts = (ctx + p.part_tokens - 1) / p.part_tokens;
     const int64_t slot0 = (int64_t)s * p.num_splits;
+    const int tid = threadIdx.x;
     float mmax = -INFINITY;
-    for (int q = 0; q < parts; ++q) mmax = fmaxf(mmax, p.ws_ml[((slot0 + q) * p.hq + head) * 2]);
-    const int d = 2 * threadIdx.x;
-    if (d >= D) return;
+    for (int q = tid; q < parts; q += 256)
+        mmax = fmaxf(mmax, p.ws_ml[((slot0 + q) * p.hq + head) * 2]);
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) mmax = fmaxf(mmax, shfl_xor_f32(mmax, o));
+    if ((tid & 63) == 0) sm_red[tid >> 6] = mmax;
+    __syncthreads();
+    mmax = fmaxf(fmaxf(sm_red[0], sm_red[1]), fmaxf(sm_red[2], sm_red[3]));
+
+    const int d2 = D / 2;
+    const int stripes = 256 / d2;  // >= 2
+    const int stripe = tid / d2, pair = tid - stripe * d2;
     float a0 = 0.0f, a1 = 0.0f, lt = 0.0f;
-    for (int q = 0; q < parts; ++q) {
-        const int64_t idx = (slot0 + q) * p.hq + head;
-        const float w = fast_exp2(p.ws_ml[idx * 2] - mmax);
-        lt += w * p.ws_ml[idx * 2 + 1];
-        a0 += w * p.ws_acc[idx * D + d];
-        a1 += w * p.ws_acc[idx * D + d + 1];
+    if (stripe < stripes) {
+        for (int q = stripe; q < parts; q += stripes) {
+            const int64_t idx = (slot0 + q) * p.hq + head;
+            const float w = fast_exp2(p.ws_ml[idx * 2] - mmax);
+            lt += w * p.ws_ml[idx * 2 + 1];
+            const float2 a = *reinterpret_cast<const float2*>(p.ws_acc + idx * D + 2 * pair);
+            a0 += w * a.x;
+            a1 += w * a.y;
+        }
+        sm_a[tid][0] = a0;
+        sm_a[tid][1] = a1;
+        if (pair == 0) sm_lt[stripe] = lt;
+    }
+    __syncthreads();
+    if (stripe != 0) return;
+    for (int j = 1; j < stripes; ++j) {
+        a0 += sm_a[j * d2 + pair][0];
+        a1 += sm_a[j * d2 + pair][1];
+        lt += sm_lt[j];
     }
     const float inv = 1.0f / lt;
     const unsigned w = (unsigned)attn_out_elem(a0 * inv, p.out_bf16) |
                        ((unsigned)attn_out_elem(a1 * inv, p.out_bf16) << 16);
     *reinterpret_cast<unsigned*>(reinterpret_cast<unsigned short*>(p.out) +
-                                 ((int64_t)t * p.hq + head) * D + d) = w;
+                                 ((int64_t)t * p.hq + head) * D + 2 * pair) = w;
 }
 
 template <int NJ>
 void launch_rows(const AttnParams& p, int total_tokens, int max_seqlen_q, int phases,
                  hipStream_t stream) {
+    const int g = p.hq / p.hkv;
+    // waves of a workgroup: KV heads first, the rest as tile phases (a power of two) as far as
+    // their accumulators fit the LDS budget
+    const int wg_heads = anydim_wg_heads(p.hkv);
+    const size_t phase_bytes = (size_t)wg_heads * g * (32 * NJ) * sizeof(float);
+    int tile_phases = 1;
+    while (tile_phases * 2 <= kAnyPhases && tile_phases * 2 * wg_heads <= kAnyWaves &&
+           (size_t)(tile_phases * 2 - 1) * phase_bytes <= (size_t)kAnyLdsBytes)
+        tile_phases *= 2;
+    const size_t lds = (size_t)(tile_phases - 1) * phase_bytes;
+    dim3 block(64 * wg_heads * tile_phases);
     if (phases & LOGISMOS_ATTN_PHASE_DECODE) {
-        dim3 grid(p.num_splits, p.hkv, p.num_seqs);
-        paged_attn_anydim_kernel<NJ><<<grid, dim3(64), 0, stream>>>(p, p.hq / p.hkv, 1);
+        dim3 grid(p.num_splits, p.hkv / wg_heads, p.num_seqs);
+        paged_attn_anydim_kernel<NJ><<<grid, block, lds, stream>>>(p, g, 1, wg_heads, tile_phases);
     }
     if ((phases & LOGISMOS_ATTN_PHASE_PREFILL) && max_seqlen_q > 1) {
-        dim3 grid(1, p.hkv, total_tokens);
-        paged_attn_anydim_kernel<NJ><<<grid, dim3(64), 0, stream>>>(p, p.hq / p.hkv, 0);
+        dim3 grid(1, p.hkv / wg_heads, total_tokens);
+        paged_attn_anydim_kernel<NJ><<<grid, block, lds, stream>>>(p, g, 0, wg_heads, tile_phases);
     }
 }
 
 }  // namespace
+
+// Workgroups = partitions x groups of KV heads.  Narrow heads (two workgroups fit a CU) aim at
+// two per CU, wide ones at half the CUs (one workgroup per CU and no second round even when
+// the contexts run long), for contexts of half the longest on average; a partition keeps at
+// least 128 keys.
+int paged_attn_anydim_num_splits(int num_seqs, int num_kv_heads, int head_dim, int block_size,
+                                 int max_blocks_per_seq) {
+    if (num_seqs <= 0 || num_kv_heads <= 0 || head_dim <= 0 || block_size <= 0 ||
+        max_blocks_per_seq <= 0)
+        return 1;
+    const int64_t max_ctx = (int64_t)block_size * max_blocks_per_seq;
+    const int64_t cus = device_cu_count();
+    const int64_t target = head_dim <= 64 ? 2 * cus : cus / 2;
+    const int64_t groups = (int64_t)num_seqs * (num_kv_heads / anydim_wg_heads(num_kv_heads));
+    int64_t splits = (2 * target + groups - 1) / groups;
+    const int64_t most = (max_ctx + 127) / 128;
+    if (splits > most) splits = most;
+    if (splits > 4096) splits = 4096;
+    if (splits < 1) splits = 1;
+    return (int)splits;
+}
 
 hipError_t paged_attn_anydim_launch(const AttnParams& p, int head_dim, int total_tokens,
                                     int max_seqlen_q, int phases, hipStream_t stream) {
@@ -305,7 +492,7 @@ hipError_t paged_attn_anydim_launch(const AttnParams& p, int head_dim, int total
     }
     if ((phases & LOGISMOS_ATTN_PHASE_MERGE) && p.num_splits > 1) {
         dim3 grid(p.hq, p.num_seqs);
-        paged_attn_anydim_merge_kernel<<<grid, dim3(128), 0, stream>>>(p, head_dim);
+        paged_attn_anydim_merge_kernel<<<grid, dim3(256), 0, stream>>>(p, head_dim);
     }
     return hipGetLastError();
 }

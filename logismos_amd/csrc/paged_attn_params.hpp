@@ -51,4 +51,8 @@ __device__ __forceinline__ unsigned short attn_out_elem(float v, int out_bf16) {
 hipError_t paged_attn_anydim_launch(const AttnParams& p, int head_dim, int total_tokens,
                                     int max_seqlen_q, int phases, hipStream_t stream);
 
+// Partition count for that kernel (pure host arithmetic).
+int paged_attn_anydim_num_splits(int num_seqs, int num_kv_heads, int head_dim, int block_size,
+                                 int max_blocks_per_seq);
+
 }  // namespace lg

@@ -62,6 +62,7 @@ _SIGNATURES = {
     "logismos_launch_repack_q4_0": (C.c_uint32, [_vp] * 4 + [_i, _i, _vp]),
     "logismos_launch_repack_q4_1": (C.c_uint32, [_vp] * 4 + [_i, _i, _vp]),
     "logismos_paged_attn_num_splits": (C.c_int, [_i, _i, _i, _i]),
+    "logismos_paged_attn_num_splits_hd": (C.c_int, [_i, _i, _i, _i, _i]),
     "logismos_paged_attn_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "logismos_launch_paged_attn_varlen_fp16":
         (C.c_uint32, [_vp] * 8 + [_i] * 9 + [_f, _i, _vp]),
@@ -289,9 +290,10 @@ def launch_repack_q8_0(blocks, qs, d, n: int, k: int, stream=None) -> None:
         _ptr(blocks), _ptr(qs), _ptr(d), n, k, _raw(stream)))
 
 
-def paged_attn_num_splits(num_seqs, num_kv_heads, block_size, max_blocks_per_seq) -> int:
-    return library().logismos_paged_attn_num_splits(num_seqs, num_kv_heads, block_size,
-                                                    max_blocks_per_seq)
+def paged_attn_num_splits(num_seqs, num_kv_heads, block_size, max_blocks_per_seq,
+                          head_dim: int = 128) -> int:
+    return library().logismos_paged_attn_num_splits_hd(num_seqs, num_kv_heads, head_dim,
+                                                       block_size, max_blocks_per_seq)
 
 
 def paged_attn_workspace_bytes(num_seqs, num_q_heads, head_dim, num_splits) -> int:

@@ -19,7 +19,7 @@ class PagedAttnRunner:
         self.total_tokens = int(c["cu_seqlens"][-1])
         self.max_seqlen_q = int(c["new_tokens"].max()) if self.num_seqs else 0
         self.num_splits = num_splits or kernels.paged_attn_num_splits(
-            self.num_seqs, c["hkv"], c["block_size"], c["max_blocks"])
+            self.num_seqs, c["hkv"], c["block_size"], c["max_blocks"], c["d"])
         self.q = hip.DeviceBuffer.from_numpy(c["q"])
         self.k_pool = hip.DeviceBuffer.from_numpy(c["k_pool"])
         self.v_pool = hip.DeviceBuffer.from_numpy(c["v_pool"])
@@ -97,8 +97,8 @@ class DecodeStepRunner:
         nseq = len(batch["context_lens"])
         self.num_seqs = nseq
         max_blocks = batch["block_tables"].shape[1]
-        self.num_splits = num_splits or kernels.paged_attn_num_splits(nseq, cfg["hkv"],
-                                                                      cfg["block_size"], max_blocks)
+        self.num_splits = num_splits or kernels.paged_attn_num_splits(
+            nseq, cfg["hkv"], cfg["block_size"], max_blocks, cfg["d"])
         half = cfg["d"] // 2
         self.cfg = kernels.DecodeConfig(len(layers), cfg["hidden"], cfg["hq"], cfg["hkv"], cfg["d"],
                                         cfg["inter"], cfg["eps"], cfg["block_size"], max_blocks,

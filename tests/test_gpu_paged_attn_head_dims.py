@@ -41,7 +41,8 @@ def test_ragged_decode_at_every_head_dim(d):
     _check(c, num_splits=63, what=f"d={d}, 63 splits")
 
 
-@pytest.mark.parametrize("hq,hkv", [(1, 1), (2, 2), (14, 2), (9, 1), (16, 1), (32, 2), (12, 4)])
+@pytest.mark.parametrize("hq,hkv", [(1, 1), (2, 2), (14, 2), (9, 1), (16, 1), (32, 2), (12, 4),
+                                    (16, 8), (12, 6), (9, 3), (20, 10), (7, 7)])
 def test_gqa_group_sizes_at_head_dim_64(hq, hkv):
     rng = np.random.default_rng(hq * 100 + hkv)
     ctx = np.array([1, 16, 17, 63, 64, 65, 200, 511])
