@@ -309,9 +309,14 @@ size_t logismos_paged_attn_workspace_bytes(int num_seqs, int num_q_heads, int he
  * the softmax is fp32 and max-subtracted
  * (`softmax_last_dim`, crates/kernels/src/cpu_f32/mod.rs:380-433); a query
  * with no visible key yields zeros.  `scale` must be finite and > 0 (else
- * hipErrorInvalidValue).  Requires head_dim == 128,
- * block_size % 16 == 0, num_q_heads % num_kv_heads == 0 and a group size
- * num_q_heads/num_kv_heads <= 8. */
+ * hipErrorInvalidValue).  Requires block_size % 16 == 0,
+ * num_q_heads % num_kv_heads == 0 and head_dim == 128 with a group size
+ * num_q_heads/num_kv_heads <= 8 (the kernels the decode step of the headline
+ * configuration runs on), or any other head_dim that is a multiple of 32 up to
+ * 256 with a group size <= 16 and total_tokens <= 65535 (a general kernel:
+ * decode rows on a static split, every row of a chunk over its whole visible
+ * context; `QwenAttention` is generic in head_dim,
+ * crates/transformers/src/attention.rs:97-127). */
 logismos_status_t logismos_launch_paged_attn_varlen_fp16(
     const void* q_f16, const void* k_pool_f16, const void* v_pool_f16, const int32_t* block_tables,
     const int32_t* cu_seqlens_q, const int32_t* context_lens, void* out_f16, void* workspace,
@@ -363,7 +368,8 @@ logismos_status_t logismos_launch_paged_attn_varlen_fp16_noalloc(
  * (`logismos_q4_xprep_bytes(num_seqs, num_q_heads*head_dim)` bytes; rows
  * num_seqs..BP-1 of the layout are left as they are): what the step executor
  * launches in front of its o projection (`merge_heads` then `wo`,
- * crates/transformers/src/attention.rs:296-302).  num_seqs <= 32. */
+ * crates/transformers/src/attention.rs:296-302).  num_seqs <= 32, head_dim 128 (a group
+ * of 128 of the layout is one head). */
 logismos_status_t logismos_launch_paged_attn_decode_fp16_xprep(
     const void* q_f16, const void* k_pool_f16, const void* v_pool_f16, const int32_t* block_tables,
     const int32_t* cu_seqlens_q, const int32_t* context_lens, void* out_prepared, void* workspace,
@@ -424,9 +430,10 @@ logismos_status_t logismos_launch_add_rms_norm_bf16(void* h_f32, const void* y_b
 /* Splits qkv (bf16 `[T][(hq+2*hkv)*128]`, q heads, then k heads, then v heads),
  * applies RoPE in the halves convention (`rope_halves_in_place`,
  * crates/kernels/src/cpu_f32/mod.rs:502-547) to q and k with the token's
- * position, and writes q as fp16 `[T][hq][128]`, k and
+ * position, and writes q as fp16 `[T][hq][head_dim]`, k and
  * v as fp16 rows of the paged pools at slot_mapping[t] (negative: skipped).
- * cos / sin: fp32 `[max_pos][64]` (`build_rope_table_f32`, :599-619).  The caller
+ * cos / sin: fp32 `[max_pos][head_dim/2]` (`build_rope_table_f32`, :599-619);
+ * head_dim even, at most 1024 (the turbo3 forms below: 128).  The caller
  * guarantees 0 <= positions[t] < max_pos (`RopeTable::gather` fails on a position past the
  * table); the kernel only keeps an out-of-range position from reading outside the tables
  * (it uses the nearest table row) and the result for such a token is unspecified. */
@@ -595,6 +602,8 @@ typedef struct {
 
 typedef struct {
     int num_layers, hidden, num_q_heads, num_kv_heads, head_dim, intermediate;
+    /* head_dim: 128, or (fp16 pools only) another multiple of 32 up to 256;
+       hidden, intermediate and num_q_heads*head_dim multiples of 128 */
     float rms_eps;
     int block_size, max_blocks_per_seq;
     int max_pos; /* rows of the RoPE tables; >= block_size * max_blocks_per_seq, so that no
@@ -623,7 +632,7 @@ typedef struct {
     const int32_t* context_lens;  /* [num_seqs], including the new token */
     const int32_t* positions;     /* [num_seqs] = context_lens - 1 */
     const int64_t* slot_mapping;  /* [num_seqs] */
-    const void* rope_cos_f32;     /* [max_pos][64] */
+    const void* rope_cos_f32;     /* [max_pos][head_dim/2] */
     const void* rope_sin_f32;
     int num_seqs;
     int num_splits;
