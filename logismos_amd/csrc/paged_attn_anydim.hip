@@ -160,36 +160,40 @@ __global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_kernel(const
         }
     }
     const int32_t* table = p.block_tables + (int64_t)s * p.max_blocks_per_seq;
-    const int64_t row_halves = (int64_t)p.hkv * D;
     const int last_key = key_end - 1;
+    // A tile's addresses: a scalar base (block, offset in the block, KV head) plus a 32-bit
+    // lane offset (key of the tile x row bytes + the lane's bytes inside the head row).
+    const unsigned row_bytes = (unsigned)p.hkv * D * 2;  // (hkv <= 65535: 16 rows < 2^31)
+    const unsigned k_lane = kLines ? 32 * tg + 16 * (c >> 3) : 16 * tg;
+    const unsigned v_lane = 2 * E * c;
 
     auto load_tile = [&](int tile_begin, int block, int off_in_block, AnyTile<NJ>& tl) {
-        const int64_t base = (int64_t)block * p.block_size + off_in_block;
+        const int64_t row0_bytes =
+            ((int64_t)block * p.block_size + off_in_block) * row_bytes + (int64_t)kvh * (D * 2);
+        const char* kb = reinterpret_cast<const char*>(p.k_pool) + row0_bytes;
+        const char* vb = reinterpret_cast<const char*>(p.v_pool) + row0_bytes;
         // keys past the end of the range read the last key of the range and are masked
         const int over = tile_begin + 15 - last_key;  // > 0: the tile runs past the range
+        const int lim = over > 0 ? 15 - over : 15;
         if constexpr (kLines) {
             // k[2u + kh]: piece 2tg + c/8 of line u of key 8kh + c%8
 #pragma unroll
             for (int kh = 0; kh < 2; ++kh) {
-                const int key = 8 * kh + (c & 7);
-                const int kk = (over > 0 && key > 15 - over) ? 15 - over : key;
-                const _Float16* kp = p.k_pool + (base + kk) * row_halves + (int64_t)kvh * D +
-                                     16 * tg + 8 * (c >> 3);
+                const unsigned koff = (unsigned)min(8 * kh + (c & 7), lim) * row_bytes + k_lane;
 #pragma unroll
                 for (int u = 0; u < NJ / 2; ++u)
-                    tl.k[2 * u + kh] = *reinterpret_cast<const half8_t*>(kp + 64 * u);
+                    tl.k[2 * u + kh] = *reinterpret_cast<const half8_t*>(kb + koff + 128 * u);
             }
         } else {
-            const int kk = (over > 0 && c > 15 - over) ? 15 - over : c;
-            const _Float16* kp = p.k_pool + (base + kk) * row_halves + (int64_t)kvh * D + 8 * tg;
+            const unsigned koff = (unsigned)min(c, lim) * row_bytes + k_lane;
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) tl.k[j] = *reinterpret_cast<const half8_t*>(kp + 32 * j);
+            for (int j = 0; j < NJ; ++j)
+                tl.k[j] = *reinterpret_cast<const half8_t*>(kb + koff + 64 * j);
         }
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int key = 4 * tg + r;
-            const int vk = (over > 0 && key > 15 - over) ? 15 - over : key;
-            load_dwords<NJ>(p.v_pool + (base + vk) * row_halves + (int64_t)kvh * D + E * c, tl.v[r]);
+            const unsigned voff = (unsigned)min(4 * tg + r, lim) * row_bytes + v_lane;
+            load_dwords<NJ>(vb + voff, tl.v[r]);
         }
     };
 
@@ -207,12 +211,17 @@ __global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_kernel(const
             for (int u = 0; u < NJ / 2; ++u) {
                 const uint4_t r0 = __builtin_bit_cast(uint4_t, tl.k[2 * u]);
                 const uint4_t r1 = __builtin_bit_cast(uint4_t, tl.k[2 * u + 1]);
-                uint4_t recv;
+                uint4_t x0, x1;
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    recv[i] = (unsigned)lane_xor_i32<8>((int)(c < 8 ? r1[i] : r0[i]));
-                const half8_t a0 = __builtin_bit_cast(half8_t, c < 8 ? r0 : recv);
-                const half8_t a1 = __builtin_bit_cast(half8_t, c < 8 ? recv : r1);
+                for (int i = 0; i < 4; ++i) {
+                    // row_ror:8 written to the upper (lower) eight lanes of each row only
+                    x0[i] = (unsigned)__builtin_amdgcn_update_dpp((int)r0[i], (int)r1[i],
+                                                                  kDppRowRor + 8, 0xf, 0xc, false);
+                    x1[i] = (unsigned)__builtin_amdgcn_update_dpp((int)r1[i], (int)r0[i],
+                                                                  kDppRowRor + 8, 0xf, 0x3, false);
+                }
+                const half8_t a0 = __builtin_bit_cast(half8_t, x0);
+                const half8_t a1 = __builtin_bit_cast(half8_t, x1);
                 sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, qb[2 * u], sacc, 0, 0, 0);
                 sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, qb[2 * u + 1], sacc, 0, 0, 0);
             }
@@ -222,36 +231,44 @@ __global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_kernel(const
                 sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(tl.k[j], qb[j], sacc, 0, 0, 0);
         }
         float sc[4];
-        float tmax = -INFINITY;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            sc[r] = tile_begin + 4 * tg + r <= last_key ? sacc[r] * p.scale_log2e : -INFINITY;
-            tmax = fmaxf(tmax, sc[r]);
+        for (int r = 0; r < 4; ++r) sc[r] = sacc[r] * p.scale_log2e;
+        if (tile_begin + 15 > last_key) {  // (a whole-wave branch) the range ends inside the tile
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                sc[r] = tile_begin + 4 * tg + r <= last_key ? sc[r] : -INFINITY;
         }
+        float tmax = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
         tmax = fmaxf(tmax, lane_xor_f32<16>(tmax));
         tmax = fmaxf(tmax, lane_xor_f32<32>(tmax));
-        const float m_new = fmaxf(m, tmax);  // finite: the first key of every tile is in range
-        const float alpha = fast_exp2(m - m_new);
-        m = m_new;
+        // Only when some head's maximum grows (a whole-wave branch; rare once a few tiles are
+        // in) are the sums and accumulators rescaled.  The accumulators of lane row tg belong
+        // to the heads 4tg + r: their factors sit in the lanes c = 4tg + r of this row.
+        if (NJ > 4 || __builtin_amdgcn_ballot_w64(tmax > m) != 0) {
+            const float m_new = fmaxf(m, tmax);  // finite: a tile's first key is in range
+            const float alpha = fast_exp2(m - m_new);
+            m = m_new;
+            l *= alpha;
+            float ar[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) ar[r] = lane_read_f32(alpha, (lane & 48) | (4 * tg + r));
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[e][r] *= ar[r];
+        }
         half4_t pa, pb;
         float psum = 0.0f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const float pr = fast_exp2(sc[r] - m_new);
+            const float pr = fast_exp2(sc[r] - m);
             psum += pr;
             pa[r] = (_Float16)pr;
             pb[r] = (_Float16)(pr - (float)pa[r]);
         }
-        l = l * alpha + psum;
-        // the accumulators of lane row tg belong to the heads 4tg + r: their factors sit in
-        // the lanes c = 4tg + r of this row
-        float ar[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) ar[r] = lane_read_f32(alpha, (lane & 48) | (4 * tg + r));
+        l += psum;
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) acc[e][r] *= ar[r];
             // B = element e of the lane's four keys: the low or high halves of their dwords e/2
             const unsigned sel = (e & 1) ? 0x07060302u : 0x05040100u;
             const uint2_t bw = {__builtin_amdgcn_perm(tl.v[1][e >> 1], tl.v[0][e >> 1], sel),
