@@ -112,3 +112,31 @@ def test_phases_and_rejections():
         kernels.check_paged_attn_shape(3, 22, 20, 34, 2, 64, 16, 64, 4)
     with pytest.raises(kernels.UnsupportedShape):
         kernels.check_paged_attn_shape(3, 22, 20, 4, 2, 80, 16, 64, 4)
+
+
+def _random_case(rng, d, max_group):
+    hkv = int(rng.choice([1, 2, 3, 4, 8]))
+    g = int(rng.integers(1, max_group + 1))
+    block_size = int(rng.choice([16, 32, 48, 64]))
+    n = int(rng.integers(1, 10))
+    # a mix of decode rows, chunks and (sometimes) empty sequences
+    kind = rng.integers(0, 4, size=n)
+    new = np.where(kind == 0, 0, np.where(kind == 1, 1, rng.integers(2, 45, size=n)))
+    prior = rng.integers(0, 500, size=n) * (rng.random(n) < 0.8)
+    if new.sum() == 0:
+        new[0] = 1
+    c = workloads.paged_case(rng, new.astype(np.int32), prior.astype(np.int32), hq=g * hkv,
+                             hkv=hkv, d=d, block_size=block_size)
+    return c, f"d={d} heads {g * hkv}/{hkv} block {block_size} new {new.tolist()} prior {prior.tolist()}"
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_randomized_ragged_batches(seed):
+    # random geometry, batch mix and partition count, every supported width in turn (128:
+    # the kernels built for it, groups up to 8)
+    rng = np.random.default_rng(9000 + seed)
+    d = [32, 64, 96, 128, 160, 192, 224, 256][seed % 8]
+    c, what = _random_case(rng, d, 8 if d == 128 else 16)
+    causal = bool(rng.integers(0, 2))
+    ns = [None, 1, int(rng.integers(2, 40))][seed % 3]
+    _check(c, num_splits=ns, causal=causal, what=f"{what} causal={causal} splits={ns}")
