@@ -29,8 +29,10 @@
 //     takes element e, so its output column c is element E c + e); lane (tg, c) ends up with
 //     the heads 4tg + r at its E elements.
 // Decode rows (one new token) are split into partitions of part_tokens keys whose partials
-// (m, l, acc) the merge kernel combines; rows of sequences with several new tokens take their
-// whole visible context in one wave.
+// (m, l, acc) the merge kernel combines.  Rows of sequences with several new tokens: the 16
+// columns of a score tile are (query token, head) pairs, 16 / G consecutive tokens of a chunk
+// per wave, each column masked at its own token's visible length; such a wave takes the whole
+// context its last token sees.
 //
 // Algorithmic HBM bytes per (decode sequence, KV head): ctx * 4 * head_dim (K and V rows)
 // + G * 4 * head_dim (q, out) + 4 * ceil(ctx / block_size).
@@ -105,12 +107,12 @@ __global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_kernel(const
                                                                            int G,
                                                                            int decode_rows,
                                                                            int wg_heads,
-                                                                           int phases) {
+                                                                           int phases, int cols) {
     constexpr int D = 32 * NJ;
     constexpr int E = 2 * NJ;
     constexpr bool kLines = NJ % 2 == 0;  // head rows are whole 128-byte lines
     __shared__ float sm_m[kAnyWaves][16], sm_l[kAnyWaves][16];  // [phase * wg_heads + head]
-    extern __shared__ float sm_acc[];  // [phases - 1][wg_heads][G][D]
+    extern __shared__ float sm_acc[];  // [phases - 1][wg_heads][cols][D]
     // (the wave index as a scalar: tile positions and block ids stay in scalar registers, the
     // block table is read with scalar loads)
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -119,15 +121,36 @@ __global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_kernel(const
     const int wg_head = wave % wg_heads, phase = wave / wg_heads;
     const int kvh = blockIdx.y * wg_heads + wg_head;
     // decode launch: grid.z walks the sequences and takes those with one new token;
-    // the other launch walks the packed rows and takes those of the other sequences
-    const int s = decode_rows ? (int)blockIdx.z : seq_of_row(p.cu_seqlens_q, p.num_seqs, blockIdx.z);
+    // the other launch walks the packed rows and takes those of the other sequences.  There a
+    // workgroup serves 16 / G consecutive rows of a chunk and the workgroups of the other rows
+    // leave at once: grid.z walks the rows with that stride (0, n, 2n, .., then 1, n + 1, ..),
+    // so that the workgroups that stay are neighbours in launch order and spread over all
+    // XCDs (walking row by row, every n-th workgroup stays: with n = 4, two XCDs of eight).
+    const int tpw = decode_rows ? 1 : 16 / G;
+    int row = blockIdx.z;
+    if (!decode_rows) {
+        const int nq = (p.out_rows + tpw - 1) / tpw;
+        row = (row % nq) * tpw + row / nq;
+        if (row >= p.out_rows) return;
+    }
+    const int s = decode_rows ? (int)blockIdx.z : seq_of_row(p.cu_seqlens_q, p.num_seqs, row);
     const int row0 = p.cu_seqlens_q[s];
     const int n_new = p.cu_seqlens_q[s + 1] - row0;
-    const int t = decode_rows ? row0 : (int)blockIdx.z;
+    const int t = decode_rows ? row0 : row;
     const int ctx = p.context_lens[s];
     const bool decode_row = n_new == 1;
     if (decode_row != (decode_rows != 0)) return;
-    const int visible = p.causal ? ctx - n_new + (t - row0) + 1 : ctx;
+    // columns of the score tile: (query token, head).  A decode row: its G heads.  A chunk:
+    // 16 / G consecutive tokens, taken by the workgroup of the first of them.
+    const int i0 = t - row0;
+    if (i0 % tpw != 0) return;
+    const int ntok = min(tpw, n_new - i0);
+    const int ncols = ntok * G;
+    const int ctok = c / G, chead = c - ctok * G;
+    // visible keys of the first and the last token of the group, and of this lane's column
+    const int vis_first = p.causal ? ctx - n_new + i0 + 1 : ctx;
+    const int visible = p.causal ? vis_first + ntok - 1 : ctx;
+    const int vis_c = (p.causal && c < ncols) ? vis_first + ctok : visible;
 
     int key_begin = 0, key_end = visible;
     bool single = true;
@@ -138,29 +161,37 @@ __global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_kernel(const
     } else if (split != 0) {
         return;
     }
-    _Float16* out_row = p.out + ((int64_t)t * p.hq + (int64_t)kvh * G) * D;
     if (visible <= 0) {
-        // no visible key: a row of zeros (written once)
+        // no visible key for any of the tokens: rows of zeros (written once)
         if (split == 0)
-            for (int i = lane + 64 * phase; i < G * D; i += 64 * phases) out_row[i] = (_Float16)0.0f;
+            for (int tq = 0; tq < ntok; ++tq) {
+                _Float16* out_row = p.out + ((int64_t)(t + tq) * p.hq + (int64_t)kvh * G) * D;
+                for (int i = lane + 64 * phase; i < G * D; i += 64 * phases)
+                    out_row[i] = (_Float16)0.0f;
+            }
         return;
     }
     if (key_begin >= key_end) return;
 
-    // the query group as the B operand: column c = head c (zero beyond the group)
+    // the queries as the B operand: column c = (token ctok, head chead), zero beyond ncols
     half8_t qb[NJ];
     {
-        const _Float16* qp = p.q + ((int64_t)t * p.hq + (int64_t)kvh * G + (c < G ? c : 0)) * D;
+        const bool cvalid = c < ncols;
+        const _Float16* qp = p.q + ((int64_t)(t + (cvalid ? ctok : 0)) * p.hq + (int64_t)kvh * G +
+                                    (cvalid ? chead : 0)) * D;
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
             // (the element order of the K operand, see load_tile / k_operand)
             const int off = kLines ? 64 * (j >> 1) + 16 * tg + 8 * (j & 1) : 32 * j + 8 * tg;
             qb[j] = *reinterpret_cast<const half8_t*>(qp + off);
-            if (c >= G) qb[j] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            if (!cvalid) qb[j] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
         }
     }
     const int32_t* table = p.block_tables + (int64_t)s * p.max_blocks_per_seq;
     const int last_key = key_end - 1;
+    // a column's keys end at lim_c; tiles that reach past the shortest column are masked
+    const int lim_c = min(vis_c, key_end);
+    const int mask_from = min(vis_first, key_end);
     // A tile's addresses: a scalar base (block, offset in the block, KV head) plus a 32-bit
     // lane offset (key of the tile x row bytes + the lane's bytes inside the head row).
     const unsigned row_bytes = (unsigned)p.hkv * D * 2;  // (hkv <= 65535: 16 rows < 2^31)
@@ -233,10 +264,10 @@ __global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_kernel(const
         float sc[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) sc[r] = sacc[r] * p.scale_log2e;
-        if (tile_begin + 15 > last_key) {  // (a whole-wave branch) the range ends inside the tile
+        if (tile_begin + 16 > mask_from) {  // (a whole-wave branch) some column ends in the tile
 #pragma unroll
             for (int r = 0; r < 4; ++r)
-                sc[r] = tile_begin + 4 * tg + r <= last_key ? sc[r] : -INFINITY;
+                sc[r] = tile_begin + 4 * tg + r < lim_c ? sc[r] : -INFINITY;
         }
         float tmax = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
         tmax = fmaxf(tmax, lane_xor_f32<16>(tmax));
@@ -244,9 +275,11 @@ __global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_kernel(const
         // Only when some head's maximum grows (a whole-wave branch; rare once a few tiles are
         // in) are the sums and accumulators rescaled.  The accumulators of lane row tg belong
         // to the heads 4tg + r: their factors sit in the lanes c = 4tg + r of this row.
+        // (A column none of whose keys has come yet -- a token of a chunk that sees nothing --
+        // keeps m = -inf, l = 0: factors and probabilities are taken against 0 there.)
         if (NJ > 4 || __builtin_amdgcn_ballot_w64(tmax > m) != 0) {
-            const float m_new = fmaxf(m, tmax);  // finite: a tile's first key is in range
-            const float alpha = fast_exp2(m - m_new);
+            const float m_new = fmaxf(m, tmax);
+            const float alpha = m_new == -INFINITY ? 1.0f : fast_exp2(m - m_new);
             m = m_new;
             l *= alpha;
             float ar[4];
@@ -259,9 +292,10 @@ __global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_kernel(const
         }
         half4_t pa, pb;
         float psum = 0.0f;
+        const float mref = m == -INFINITY ? 0.0f : m;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const float pr = fast_exp2(sc[r] - m);
+            const float pr = fast_exp2(sc[r] - mref);
             psum += pr;
             pa[r] = (_Float16)pr;
             pb[r] = (_Float16)(pr - (float)pa[r]);
@@ -331,18 +365,20 @@ __global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_kernel(const
     __syncthreads();
     float mall = m, lall = 0.0f;
     for (int f = 0; f < phases; ++f) mall = fmaxf(mall, sm_m[f * wg_heads + wg_head][c]);
+    const float mall_ref = mall == -INFINITY ? 0.0f : mall;
     for (int f = 0; f < phases; ++f)
-        lall += fast_exp2(sm_m[f * wg_heads + wg_head][c] - mall) * sm_l[f * wg_heads + wg_head][c];
-    const float fown = fast_exp2(m - mall);
+        lall += fast_exp2(sm_m[f * wg_heads + wg_head][c] - mall_ref) *
+                sm_l[f * wg_heads + wg_head][c];
+    const float fown = fast_exp2(m - mall_ref);
     float fr[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) fr[r] = lane_read_f32(fown, (lane & 48) | (4 * tg + r));
     if (phase > 0) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int h = 4 * tg + r;
-            if (h >= G) continue;
-            float* dst = sm_acc + (((phase - 1) * wg_heads + wg_head) * G + h) * D + E * c;
+            const int h = 4 * tg + r;  // the column these accumulator rows belong to
+            if (h >= ncols) continue;
+            float* dst = sm_acc + (((phase - 1) * wg_heads + wg_head) * cols + h) * D + E * c;
 #pragma unroll
             for (int e = 0; e < E; ++e) dst[e] = acc[e][r] * fr[r];
         }
@@ -354,19 +390,20 @@ __global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_kernel(const
         const int h = 4 * tg + r;
         const float mh = lane_read_f32(mall, (lane & 48) | h);
         const float lh = lane_read_f32(lall, (lane & 48) | h);
-        if (h >= G) continue;
+        if (h >= ncols) continue;
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             float a = acc[e][r] * fr[r];
             for (int f = 0; f < phases - 1; ++f)
-                a += sm_acc[((f * wg_heads + wg_head) * G + h) * D + E * c + e];
+                a += sm_acc[((f * wg_heads + wg_head) * cols + h) * D + E * c + e];
             acc[e][r] = a;
         }
-        const int head = kvh * G + h;
+        const int htok = h / G;
+        const int head = kvh * G + (h - htok * G);
         if (single) {
-            const float inv = 1.0f / lh;
-            unsigned short* dst =
-                reinterpret_cast<unsigned short*>(p.out) + ((int64_t)t * p.hq + head) * D + E * c;
+            const float inv = lh > 0.0f ? 1.0f / lh : 0.0f;  // a token that sees no key: zeros
+            unsigned short* dst = reinterpret_cast<unsigned short*>(p.out) +
+                                  ((int64_t)(t + htok) * p.hq + head) * D + E * c;
 #pragma unroll
             for (int e = 0; e < E; e += 2) {
                 const unsigned w = (unsigned)attn_out_elem(acc[e][r] * inv, p.out_bf16) |
@@ -449,21 +486,26 @@ void launch_rows(const AttnParams& p, int total_tokens, int max_seqlen_q, int ph
     // waves of a workgroup: KV heads first, the rest as tile phases (a power of two) as far as
     // their accumulators fit the LDS budget
     const int wg_heads = anydim_wg_heads(p.hkv);
-    const size_t phase_bytes = (size_t)wg_heads * g * (32 * NJ) * sizeof(float);
-    int tile_phases = 1;
-    while (tile_phases * 2 <= kAnyPhases && tile_phases * 2 * wg_heads <= kAnyWaves &&
-           (size_t)(tile_phases * 2 - 1) * phase_bytes <= (size_t)kAnyLdsBytes)
-        tile_phases *= 2;
-    const size_t lds = (size_t)(tile_phases - 1) * phase_bytes;
-    dim3 block(64 * wg_heads * tile_phases);
-    if (phases & LOGISMOS_ATTN_PHASE_DECODE) {
-        dim3 grid(p.num_splits, p.hkv / wg_heads, p.num_seqs);
-        paged_attn_anydim_kernel<NJ><<<grid, block, lds, stream>>>(p, g, 1, wg_heads, tile_phases);
-    }
-    if ((phases & LOGISMOS_ATTN_PHASE_PREFILL) && max_seqlen_q > 1) {
-        dim3 grid(1, p.hkv / wg_heads, total_tokens);
-        paged_attn_anydim_kernel<NJ><<<grid, block, lds, stream>>>(p, g, 0, wg_heads, tile_phases);
-    }
+    // (cols: the columns a wave's accumulators cover -- a decode row's group, or the
+    // 16 / G tokens of a chunk times the group)
+    auto launch = [&](int grid_x, int grid_z, int decode_rows, int cols, int wg_heads) {
+        const size_t phase_bytes = (size_t)wg_heads * cols * (32 * NJ) * sizeof(float);
+        int tile_phases = 1;
+        while (tile_phases * 2 <= kAnyPhases && tile_phases * 2 * wg_heads <= kAnyWaves &&
+               (size_t)(tile_phases * 2 - 1) * phase_bytes <= (size_t)kAnyLdsBytes)
+            tile_phases *= 2;
+        const size_t lds = (size_t)(tile_phases - 1) * phase_bytes;
+        paged_attn_anydim_kernel<NJ>
+            <<<dim3(grid_x, p.hkv / wg_heads, grid_z), dim3(64 * wg_heads * tile_phases), lds,
+               stream>>>(p, g, decode_rows, wg_heads, tile_phases, cols);
+    };
+    if (phases & LOGISMOS_ATTN_PHASE_DECODE)
+        launch(p.num_splits, p.num_seqs, 1, g, wg_heads);
+    // rows of chunks: a workgroup walks a whole context, most of it out of L2, and the longest
+    // walk sets the time of the launch -- more tile phases per head, fewer heads together
+    if ((phases & LOGISMOS_ATTN_PHASE_PREFILL) && max_seqlen_q > 1)
+        launch(1, (total_tokens + 16 / g - 1) / (16 / g) * (16 / g), 0, (16 / g) * g,
+               wg_heads % 2 == 0 ? 2 : 1);
 }
 
 }  // namespace
