@@ -747,6 +747,70 @@ def bench_decode_step(args):
     }
 
 
+def bench_head_dim64(args):
+    """The general-head-width kernel at head_dim 64: config 5's batch at 32 / 8 heads (the
+    roofline figure), config 2's batch at Qwen2-0.5B's 14 / 2 heads (checked against the
+    oracle), and a mixed batch of two 512-token chunks and six decode rows."""
+    import oracle as O
+    stream = hip.Stream()
+
+    def timed(case, phases=None):
+        r = PagedAttnRunner(case, stream=stream)
+        kv_bytes = case["k_pool"].nbytes + case["v_pool"].nbytes
+        copies = max(2, min(16, -(-COLD_BYTES // kv_bytes)))
+        kps, vps = replicate(r.k_pool, copies), replicate(r.v_pool, copies)
+        fns = [lambda k=k, v=v: r.launch(phases=phases, k_pool=k, v_pool=v)
+               for k, v in zip(kps, vps)]
+        return r, time_launches(stream, fns, args.steps, args.warmup)[0]
+
+    rng = np.random.default_rng(workloads.SEED + 64)
+    ctx = rng.integers(256, 8193, size=32)
+    big = workloads.paged_case(rng, np.ones(32, np.int32), ctx - 1, hq=32, hkv=8, d=64,
+                               pool_period_rows=4099)
+    algo = workloads.paged_attn_algorithmic_bytes(big)
+    r_big, ms_full = timed(big)
+    _, ms_dec = timed(big, kernels.ATTN_PHASE_DECODE)
+
+    ctx = rng.integers(64, 2049, size=16)
+    small = workloads.paged_case(rng, np.ones(16, np.int32), ctx - 1, hq=14, hkv=2, d=64)
+    r_small, ms_small = timed(small)
+    r_small.launch()
+    got = r_small.result().astype(np.float32)
+    want = O.paged_attn_varlen_fp16(small["q"], small["k_pool"], small["v_pool"],
+                                    small["block_tables"], small["cu_seqlens"],
+                                    small["context_lens"], 14, 2, 64, small["block_size"],
+                                    small["scale"], True).astype(np.float32)
+    mixed = workloads.paged_case(rng, [512, 1, 512, 1, 1, 1, 1, 1],
+                                 [1000, 3000, 0, 500, 7000, 100, 2000, 4000], hq=32, hkv=8, d=64,
+                                 pool_period_rows=4099)
+    _, ms_mixed = timed(mixed)
+    _, ms_mixed_chunks = timed(mixed, kernels.ATTN_PHASE_PREFILL)
+    achieved = algo / (ms_dec * 1e-3) / 1e9
+    return {
+        "metric": "paged-attn decode achieved HBM GB/s (head_dim 64)",
+        "value": round(algo / (ms_full * 1e-3) / 1e9, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_full, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "config 5's batch (32 seqs, ctx U[256,8192]) at 32 q / 8 kv heads "
+                               "of 64, block 16, fp16 KV: decode + merge",
+                   "sum_ctx": int(big["context_lens"].sum()), "num_splits": r_big.num_splits,
+                   "algorithmic_bytes_per_step": algo},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "paged_attn_anydim_kernel<2> (decode launch)",
+                     "ms_per_launch": round(ms_dec, 5)},
+        "config2_batch_14q_2kv_heads": {"ms_per_step": round(ms_small, 5),
+                                        "num_splits": r_small.num_splits,
+                                        "algorithmic_bytes_per_step":
+                                            workloads.paged_attn_algorithmic_bytes(small),
+                                        "parity_max_abs_vs_oracle":
+                                            float(np.abs(got - want).max())},
+        "mixed_2x512_token_chunks_6_decode_rows": {"ms_per_step": round(ms_mixed, 5),
+                                                   "ms_chunk_rows": round(ms_mixed_chunks, 5)},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -763,7 +827,7 @@ def main():
                          "not for runs under a profiler")
     ap.add_argument("--workload", default="all",
                     choices=["all", "step", "config1", "config2", "config3", "config4",
-                             "config4_gemm", "turbo3"],
+                             "config4_gemm", "turbo3", "headdim64"],
                     help="all: the decode-step line with every leg inside it (default); "
                          "otherwise only that workload's own JSON line")
     args = ap.parse_args()
@@ -776,12 +840,13 @@ def main():
     kernels.library()
     args.steps_c5 = args.steps if args.steps is not None else 20
     args.warmup_c5 = args.warmup if args.warmup is not None else 3
-    if args.workload in ("config1", "config2", "config3", "config4", "config4_gemm", "turbo3"):
+    if args.workload in ("config1", "config2", "config3", "config4", "config4_gemm", "turbo3",
+                         "headdim64"):
         args.steps = args.steps if args.steps is not None else 200
         args.warmup = args.warmup if args.warmup is not None else 20
         leg = {"config1": bench_qgemv_q8, "config2": bench_paged_decode, "config3": bench_q4,
                "config4": bench_mixed_config4, "config4_gemm": bench_q4_tall,
-               "turbo3": bench_turbo3}[args.workload]
+               "turbo3": bench_turbo3, "headdim64": bench_head_dim64}[args.workload]
         print(json.dumps(leg(args)))
         return
     line = bench_decode_step(args)

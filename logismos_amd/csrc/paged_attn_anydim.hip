@@ -45,8 +45,6 @@
 
 namespace lg {
 
-namespace {
-
 constexpr int kAnyTileKeys = 16;
 constexpr int kAnyWaves = 8;           // waves of a workgroup: KV heads x tile phases
 constexpr int kAnyLdsBytes = 48 * 1024;  // for the accumulators of the phases beyond the first
@@ -54,7 +52,7 @@ constexpr int kAnyWgHeads = 8;           // KV heads per workgroup at most
 constexpr int kAnyPhases = 8;            // tile phases per head at most
 
 // KV heads per workgroup: the largest divisor of hkv up to kAnyWgHeads
-int anydim_wg_heads(int hkv) {
+static int anydim_wg_heads(int hkv) {
     for (int w = kAnyWgHeads; w > 1; --w)
         if (hkv % w == 0) return w;
     return 1;
@@ -117,7 +115,6 @@ __global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_kernel(const
     // block table is read with scalar loads)
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int c = lane & 15, tg = lane >> 4;
-    const int split = blockIdx.x;
     const int wg_head = wave % wg_heads, phase = wave / wg_heads;
     const int kvh = blockIdx.y * wg_heads + wg_head;
     // decode launch: grid.z walks the sequences and takes those with one new token;
@@ -134,6 +131,11 @@ __global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_kernel(const
         if (row >= p.out_rows) return;
     }
     const int s = decode_rows ? (int)blockIdx.z : seq_of_row(p.cu_seqlens_q, p.num_seqs, row);
+    // Partition of this workgroup: rotated by the sequence index.  Workgroups are dealt to the
+    // eight XCDs in launch order; with partition p of every sequence at x = p and a partition
+    // count that is a multiple of 8, the first partitions (which every sequence has) would all
+    // land on the same XCDs and the last ones (which only long sequences have) on others.
+    const int split = decode_rows ? (int)((blockIdx.x + 5u * (unsigned)s) % gridDim.x) : 0;
     const int row0 = p.cu_seqlens_q[s];
     const int n_new = p.cu_seqlens_q[s + 1] - row0;
     const int t = decode_rows ? row0 : row;
@@ -480,7 +482,7 @@ __global__ __launch_bounds__(256) void paged_attn_anydim_merge_kernel(const Attn
 }
 
 template <int NJ>
-void launch_rows(const AttnParams& p, int total_tokens, int max_seqlen_q, int phases,
+static void launch_rows(const AttnParams& p, int total_tokens, int max_seqlen_q, int phases,
                  hipStream_t stream) {
     const int g = p.hq / p.hkv;
     // waves of a workgroup: KV heads first, the rest as tile phases (a power of two) as far as
@@ -508,7 +510,6 @@ void launch_rows(const AttnParams& p, int total_tokens, int max_seqlen_q, int ph
                wg_heads % 2 == 0 ? 2 : 1);
 }
 
-}  // namespace
 
 // Workgroups = partitions x groups of KV heads.  Narrow heads (two workgroups fit a CU) aim at
 // two per CU, wide ones at half the CUs (one workgroup per CU and no second round even when
