@@ -798,7 +798,7 @@ def bench_head_dim64(args):
                    "algorithmic_bytes_per_step": algo},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "paged_attn_anydim_kernel<2> (decode launch)",
+                     "kernel": "paged_attn_anydim_balanced_kernel<2>",
                      "ms_per_launch": round(ms_dec, 5)},
         "config2_batch_14q_2kv_heads": {"ms_per_step": round(ms_small, 5),
                                         "num_splits": r_small.num_splits,

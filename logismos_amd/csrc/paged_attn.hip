@@ -45,7 +45,6 @@
 namespace lg {
 
 constexpr int kHeadDim = 128;
-constexpr int kTileKeys = 16;
 constexpr int kMaxHeadWaves = 8;  // waves (KV heads) per workgroup
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -779,27 +778,6 @@ __global__ __launch_bounds__(64 * kMaxHeadWaves) void paged_attn_kernel(const At
     const int num_parts = (ctx + p.part_tokens - 1) / p.part_tokens;
     attn_partition<G, T3>(p, s, t, kvh, tok_begin, min(ctx, tok_begin + p.part_tokens),
                           num_parts == 1, (int64_t)s * p.num_splits + split, t3_quads);
-}
-
-// Units sequence s contributes to the decode stream: its 16-key tiles plus kSeqStartUnits for
-// starting it.  A worker that finishes one sequence and starts the next pays for a second
-// prologue (queries, first tiles with nothing in flight) and epilogue (row merge, partial
-// write): with equal tile counts such workers ended 3 us after the others and set the
-// duration of the launch.  With that cost in the stream they get fewer tiles (a tile takes
-// about 2.3 us); 3 to 5 units measured alike, 0 and 1 worse.
-constexpr int kSeqStartUnits = 4;
-__device__ __forceinline__ int decode_tiles(const AttnParams& p, int s) {
-    const int n_new = p.cu_seqlens_q[s + 1] - p.cu_seqlens_q[s];
-    const int ctx = p.context_lens[s];
-    return (n_new == 1 && ctx > 0) ? (ctx + kTileKeys - 1) / kTileKeys + kSeqStartUnits : 0;
-}
-
-constexpr int kMaxBalancedSeqs = 2048;  // prefix table held in LDS
-constexpr int kMinWorkerTiles = 8;      // a worker streams at least 128 keys
-
-__device__ __forceinline__ int worker_tiles(int total_tiles, int num_workers) {
-    const int r = (total_tiles + num_workers - 1) / num_workers;
-    return r < kMinWorkerTiles ? kMinWorkerTiles : r;
 }
 
 // Decode rows, balanced: the key tiles of all decode sequences form one stream (sequence
@@ -1553,15 +1531,6 @@ static void launch_prefill(const AttnParams& p, int max_seqlen_q, hipStream_t st
     constexpr int QT = kPfWaves * (32 / G);
     dim3 grid(p.hkv, (max_seqlen_q + QT - 1) / QT, p.num_seqs);
     paged_attn_prefill_kernel<G, T3><<<grid, dim3(64 * kPfWaves), 0, stream>>>(p);
-}
-
-// Small batches stay on the static split: when every partition of every sequence is
-// resident at once there is no second round to balance away, and the balanced kernel's
-// prologue (prefix table, search) costs more than it saves (config 2: 12.7 vs 18 us).
-// The bound is on what the block tables could hold, the only size the host knows.
-static bool small_decode_batch(int num_seqs, int num_kv_heads, int block_size,
-                               int max_blocks_per_seq) {
-    return (int64_t)num_seqs * num_kv_heads * block_size * max_blocks_per_seq <= 200000;
 }
 
 // Workers of the balanced decode kernel: eight waves per CU (one wave = one KV head of one

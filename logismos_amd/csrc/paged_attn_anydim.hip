@@ -45,7 +45,6 @@
 
 namespace lg {
 
-constexpr int kAnyTileKeys = 16;
 constexpr int kAnyWaves = 8;           // waves of a workgroup: KV heads x tile phases
 constexpr int kAnyLdsBytes = 48 * 1024;  // for the accumulators of the phases beyond the first
 constexpr int kAnyWgHeads = 8;           // KV heads per workgroup at most
@@ -100,80 +99,29 @@ __device__ __forceinline__ int seq_of_row(const int32_t* cu, int num_seqs, int t
     return lo;
 }
 
+// The work of one workgroup on the keys [key_begin, key_end) (not empty) of sequence s for the
+// ntok query tokens from packed row t on: scores, softmax, P.V, the merge of the tile phases,
+// and either the finished rows (single) or the partial (m, l, acc) at workspace slot `slot`.
+// Called by every wave of the workgroup (it holds two barriers).
 template <int NJ>
-__global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_kernel(const AttnParams p,
-                                                                           int G,
-                                                                           int decode_rows,
-                                                                           int wg_heads,
-                                                                           int phases, int cols) {
+__device__ __forceinline__ void anydim_range(const AttnParams& p, int G, int wg_heads, int phases,
+                                             int cols, int s, int t, int ntok, int vis_first,
+                                             int visible, int key_begin, int key_end, bool single,
+                                             int64_t slot, float (*sm_m)[16], float (*sm_l)[16],
+                                             float* sm_acc) {
     constexpr int D = 32 * NJ;
     constexpr int E = 2 * NJ;
     constexpr bool kLines = NJ % 2 == 0;  // head rows are whole 128-byte lines
-    __shared__ float sm_m[kAnyWaves][16], sm_l[kAnyWaves][16];  // [phase * wg_heads + head]
-    extern __shared__ float sm_acc[];  // [phases - 1][wg_heads][cols][D]
     // (the wave index as a scalar: tile positions and block ids stay in scalar registers, the
     // block table is read with scalar loads)
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int c = lane & 15, tg = lane >> 4;
     const int wg_head = wave % wg_heads, phase = wave / wg_heads;
     const int kvh = blockIdx.y * wg_heads + wg_head;
-    // decode launch: grid.z walks the sequences and takes those with one new token;
-    // the other launch walks the packed rows and takes those of the other sequences.  There a
-    // workgroup serves 16 / G consecutive rows of a chunk and the workgroups of the other rows
-    // leave at once: grid.z walks the rows with that stride (0, n, 2n, .., then 1, n + 1, ..),
-    // so that the workgroups that stay are neighbours in launch order and spread over all
-    // XCDs (walking row by row, every n-th workgroup stays: with n = 4, two XCDs of eight).
-    const int tpw = decode_rows ? 1 : 16 / G;
-    int row = blockIdx.z;
-    if (!decode_rows) {
-        const int nq = (p.out_rows + tpw - 1) / tpw;
-        row = (row % nq) * tpw + row / nq;
-        if (row >= p.out_rows) return;
-    }
-    const int s = decode_rows ? (int)blockIdx.z : seq_of_row(p.cu_seqlens_q, p.num_seqs, row);
-    // Partition of this workgroup: rotated by the sequence index.  Workgroups are dealt to the
-    // eight XCDs in launch order; with partition p of every sequence at x = p and a partition
-    // count that is a multiple of 8, the first partitions (which every sequence has) would all
-    // land on the same XCDs and the last ones (which only long sequences have) on others.
-    const int split = decode_rows ? (int)((blockIdx.x + 5u * (unsigned)s) % gridDim.x) : 0;
-    const int row0 = p.cu_seqlens_q[s];
-    const int n_new = p.cu_seqlens_q[s + 1] - row0;
-    const int t = decode_rows ? row0 : row;
-    const int ctx = p.context_lens[s];
-    const bool decode_row = n_new == 1;
-    if (decode_row != (decode_rows != 0)) return;
-    // columns of the score tile: (query token, head).  A decode row: its G heads.  A chunk:
-    // 16 / G consecutive tokens, taken by the workgroup of the first of them.
-    const int i0 = t - row0;
-    if (i0 % tpw != 0) return;
-    const int ntok = min(tpw, n_new - i0);
+    // columns of the score tile: (query token, head)
     const int ncols = ntok * G;
     const int ctok = c / G, chead = c - ctok * G;
-    // visible keys of the first and the last token of the group, and of this lane's column
-    const int vis_first = p.causal ? ctx - n_new + i0 + 1 : ctx;
-    const int visible = p.causal ? vis_first + ntok - 1 : ctx;
     const int vis_c = (p.causal && c < ncols) ? vis_first + ctok : visible;
-
-    int key_begin = 0, key_end = visible;
-    bool single = true;
-    if (decode_row && p.num_splits > 1) {
-        key_begin = split * p.part_tokens;
-        key_end = min(visible, key_begin + p.part_tokens);
-        single = visible <= p.part_tokens;
-    } else if (split != 0) {
-        return;
-    }
-    if (visible <= 0) {
-        // no visible key for any of the tokens: rows of zeros (written once)
-        if (split == 0)
-            for (int tq = 0; tq < ntok; ++tq) {
-                _Float16* out_row = p.out + ((int64_t)(t + tq) * p.hq + (int64_t)kvh * G) * D;
-                for (int i = lane + 64 * phase; i < G * D; i += 64 * phases)
-                    out_row[i] = (_Float16)0.0f;
-            }
-        return;
-    }
-    if (key_begin >= key_end) return;
 
     // the queries as the B operand: column c = (token ctok, head chead), zero beyond ncols
     half8_t qb[NJ];
@@ -321,8 +269,8 @@ __global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_kernel(const
         // before its requests.  A position past the wave's last tile stays on the last tile:
         // every request is unconditional and reads memory the range owns; what was read twice
         // is not consumed.
-        const int kStep = kAnyTileKeys * phases;
-        const int tb0 = key_begin + kAnyTileKeys * phase;
+        const int kStep = kTileKeys * phases;
+        const int tb0 = key_begin + kTileKeys * phase;
         if (tb0 < key_end) {
             const int n_tiles = (key_end - tb0 + kStep - 1) / kStep;
             int tb = tb0, bi = tb0 / p.block_size, bo = tb0 - bi * p.block_size;
@@ -413,7 +361,7 @@ __global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_kernel(const
                 *reinterpret_cast<unsigned*>(dst + e) = w;
             }
         } else {
-            const int64_t idx = ((int64_t)s * p.num_splits + split) * p.hq + head;
+            const int64_t idx = slot * p.hq + head;
             float* dst = p.ws_acc + idx * D + E * c;
 #pragma unroll
             for (int e = 0; e < E; ++e) dst[e] = acc[e][r];
@@ -422,6 +370,151 @@ __global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_kernel(const
                 p.ws_ml[idx * 2 + 1] = lh;
             }
         }
+    }
+}
+
+// Static split and rows of chunks: grid (partitions, KV-head groups, sequences or packed rows).
+template <int NJ>
+__global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_kernel(const AttnParams p,
+                                                                           int G,
+                                                                           int decode_rows,
+                                                                           int wg_heads,
+                                                                           int phases, int cols) {
+    constexpr int D = 32 * NJ;
+    __shared__ float sm_m[kAnyWaves][16], sm_l[kAnyWaves][16];  // [phase * wg_heads + head]
+    extern __shared__ float sm_acc[];  // [phases - 1][wg_heads][cols][D]
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wg_head = wave % wg_heads, phase = wave / wg_heads;
+    const int kvh = blockIdx.y * wg_heads + wg_head;
+    // decode launch: grid.z walks the sequences and takes those with one new token;
+    // the other launch walks the packed rows and takes those of the other sequences.  There a
+    // workgroup serves 16 / G consecutive rows of a chunk and the workgroups of the other rows
+    // leave at once: grid.z walks the rows with that stride (0, n, 2n, .., then 1, n + 1, ..),
+    // so that the workgroups that stay are neighbours in launch order and spread over all
+    // XCDs (walking row by row, every n-th workgroup stays: with n = 4, two XCDs of eight).
+    const int tpw = decode_rows ? 1 : 16 / G;
+    int row = blockIdx.z;
+    if (!decode_rows) {
+        const int nq = (p.out_rows + tpw - 1) / tpw;
+        row = (row % nq) * tpw + row / nq;
+        if (row >= p.out_rows) return;
+    }
+    const int s = decode_rows ? (int)blockIdx.z : seq_of_row(p.cu_seqlens_q, p.num_seqs, row);
+    // Partition of this workgroup: rotated by the sequence index.  Workgroups are dealt to the
+    // eight XCDs in launch order; with partition p of every sequence at x = p and a partition
+    // count that is a multiple of 8, the first partitions (which every sequence has) would all
+    // land on the same XCDs and the last ones (which only long sequences have) on others.
+    const int split = decode_rows ? (int)((blockIdx.x + 5u * (unsigned)s) % gridDim.x) : 0;
+    const int row0 = p.cu_seqlens_q[s];
+    const int n_new = p.cu_seqlens_q[s + 1] - row0;
+    const int t = decode_rows ? row0 : row;
+    const int ctx = p.context_lens[s];
+    const bool decode_row = n_new == 1;
+    if (decode_row != (decode_rows != 0)) return;
+    // columns of the score tile: (query token, head).  A decode row: its G heads.  A chunk:
+    // 16 / G consecutive tokens, taken by the workgroup of the first of them.
+    const int i0 = t - row0;
+    if (i0 % tpw != 0) return;
+    const int ntok = min(tpw, n_new - i0);
+    // visible keys of the first and the last token of the group
+    const int vis_first = p.causal ? ctx - n_new + i0 + 1 : ctx;
+    const int visible = p.causal ? vis_first + ntok - 1 : ctx;
+
+    int key_begin = 0, key_end = visible;
+    bool single = true;
+    if (decode_row && p.num_splits > 1) {
+        key_begin = split * p.part_tokens;
+        key_end = min(visible, key_begin + p.part_tokens);
+        single = visible <= p.part_tokens;
+    } else if (split != 0) {
+        return;
+    }
+    if (visible <= 0) {
+        // no visible key for any of the tokens: rows of zeros (written once)
+        if (split == 0)
+            for (int tq = 0; tq < ntok; ++tq) {
+                _Float16* out_row = p.out + ((int64_t)(t + tq) * p.hq + (int64_t)kvh * G) * D;
+                for (int i = lane + 64 * phase; i < G * D; i += 64 * phases)
+                    out_row[i] = (_Float16)0.0f;
+            }
+        return;
+    }
+    if (key_begin >= key_end) return;
+
+    anydim_range<NJ>(p, G, wg_heads, phases, cols, s, t, ntok, vis_first, visible, key_begin,
+                     key_end, single, (int64_t)s * p.num_splits + split, sm_m, sm_l, sm_acc);
+}
+
+// Decode rows, balanced: the 16-key tiles of all decode sequences form one stream (each
+// sequence preceded by kSeqStartUnits units for starting it); worker w (grid.x) takes the units
+// [wR, (w + 1)R), R = ceil(total / workers), whichever sequences they belong to, so every
+// workgroup does the same amount of work whatever the context lengths are.  Its piece of
+// sequence s goes to workspace slot w + s (the pieces of a sequence get consecutive slots); a
+// sequence inside one worker is finished there.  grid (workers, KV-head groups).
+template <int NJ>
+__global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_balanced_kernel(
+    const AttnParams p, int G, int wg_heads, int phases) {
+    __shared__ int pt[kMaxBalancedSeqs + 1];  // exclusive prefix of the sequences' units
+    __shared__ float sm_m[kAnyWaves][16], sm_l[kAnyWaves][16];
+    extern __shared__ float sm_acc[];  // [phases - 1][wg_heads][G][D]
+    const int lane = threadIdx.x & 63;
+    const int S = p.num_seqs;
+    if (threadIdx.x < 64) {
+        const int per = (S + 63) / 64;
+        int sum = 0;
+        for (int i = 0; i < per; ++i) {
+            const int s = lane * per + i;
+            if (s < S) sum += decode_tiles(p, s);
+        }
+        int incl = sum;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int v = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += v;
+        }
+        int run = incl - sum;
+        for (int i = 0; i < per; ++i) {
+            const int s = lane * per + i;
+            if (s < S) {
+                pt[s] = run;
+                run += decode_tiles(p, s);
+            }
+        }
+        if (lane == 63) pt[S] = incl;
+    }
+    __syncthreads();
+    // (LDS reads land in vector registers: wave-uniform values are made scalar again so that
+    // block ids keep coming through scalar loads)
+    const int total = __builtin_amdgcn_readfirstlane(pt[S]);
+    const int w = blockIdx.x;
+    const int R = worker_tiles(total, p.num_workers);
+    const int64_t ub64 = (int64_t)w * R;
+    if (ub64 >= total) return;
+    const int ub = (int)ub64;
+    const int ue = (int)min((int64_t)total, ub64 + R);
+    int lo = 0, hi = S;  // the sequence holding unit ub: the largest s with pt[s] <= ub
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (__builtin_amdgcn_readfirstlane(pt[mid]) <= ub) lo = mid;
+        else hi = mid;
+    }
+    int ucur = ub;
+    for (int s = lo; ucur < ue; ++s) {
+        const int seq_begin = __builtin_amdgcn_readfirstlane(pt[s]);
+        const int seq_end = __builtin_amdgcn_readfirstlane(pt[s + 1]);
+        if (seq_end <= ucur) continue;  // a sequence without decode tiles
+        const int seg_end = min(ue, seq_end);
+        // units -> tiles of the sequence: its first kSeqStartUnits units are the start-up cost
+        const int tile_lo = max(ucur - seq_begin - kSeqStartUnits, 0);
+        const int tile_hi = seg_end - seq_begin - kSeqStartUnits;
+        if (tile_hi > tile_lo) {
+            const int ctx = p.context_lens[s];
+            const bool single = tile_lo == 0 && seg_end == seq_end;
+            anydim_range<NJ>(p, G, wg_heads, phases, G, s, p.cu_seqlens_q[s], 1, ctx, ctx,
+                             tile_lo * kTileKeys, min(ctx, tile_hi * kTileKeys), single,
+                             (int64_t)w + s, sm_m, sm_l, sm_acc);
+        }
+        ucur = seg_end;
     }
 }
 
@@ -437,10 +530,48 @@ __global__ __launch_bounds__(256) void paged_attn_anydim_merge_kernel(const Attn
     const int t = p.cu_seqlens_q[s];
     if (p.cu_seqlens_q[s + 1] - t != 1) return;
     const int ctx = p.context_lens[s];
-    if (ctx <= p.part_tokens) return;  // zero or one partition: already final
-    const int parts = (ctx + p.part_tokens - 1) / p.part_tokens;
-    const int64_t slot0 = (int64_t)s * p.num_splits;
     const int tid = threadIdx.x;
+    int parts;      // partials of this sequence
+    int64_t slot0;  // of its first partial
+    if (p.num_workers > 0) {
+        // balanced split: where this sequence sits in the stream of units
+        __shared__ int red[2][4];
+        int before = 0, total = 0;
+        for (int i = tid; i < p.num_seqs; i += 256) {
+            const int nt = decode_tiles(p, i);
+            total += nt;
+            before += i < s ? nt : 0;
+        }
+#pragma unroll
+        for (int mask = 32; mask >= 1; mask >>= 1) {
+            total += __shfl_xor(total, mask, 64);
+            before += __shfl_xor(before, mask, 64);
+        }
+        if ((tid & 63) == 0) {
+            red[0][tid >> 6] = total;
+            red[1][tid >> 6] = before;
+        }
+        __syncthreads();
+        total = red[0][0] + red[0][1] + red[0][2] + red[0][3];
+        before = red[1][0] + red[1][1] + red[1][2] + red[1][3];
+        if (ctx <= 0) {
+            // the stream has no tile of this row and nobody wrote it: a row of zeros
+            if (2 * tid < D)
+                *reinterpret_cast<unsigned*>(reinterpret_cast<unsigned short*>(p.out) +
+                                             ((int64_t)t * p.hq + head) * D + 2 * tid) = 0u;
+            return;
+        }
+        // its tiles are the units [before + kSeqStartUnits, before + nt)
+        const int nt = (ctx + kTileKeys - 1) / kTileKeys + kSeqStartUnits;
+        const int R = worker_tiles(total, p.num_workers);
+        const int w_first = (before + kSeqStartUnits) / R;
+        parts = (before + nt - 1) / R - w_first + 1;
+        slot0 = (int64_t)w_first + s;
+    } else {
+        parts = ctx <= 0 ? 0 : (ctx + p.part_tokens - 1) / p.part_tokens;
+        slot0 = (int64_t)s * p.num_splits;
+    }
+    if (parts <= 1) return;  // zero or one partial: already final
     float mmax = -INFINITY;
     for (int q = tid; q < parts; q += 256)
         mmax = fmaxf(mmax, p.ws_ml[((slot0 + q) * p.hq + head) * 2]);
@@ -501,8 +632,20 @@ static void launch_rows(const AttnParams& p, int total_tokens, int max_seqlen_q,
             <<<dim3(grid_x, p.hkv / wg_heads, grid_z), dim3(64 * wg_heads * tile_phases), lds,
                stream>>>(p, g, decode_rows, wg_heads, tile_phases, cols);
     };
-    if (phases & LOGISMOS_ATTN_PHASE_DECODE)
-        launch(p.num_splits, p.num_seqs, 1, g, wg_heads);
+    if (phases & LOGISMOS_ATTN_PHASE_DECODE) {
+        if (p.num_workers > 0) {
+            const size_t phase_bytes = (size_t)wg_heads * g * (32 * NJ) * sizeof(float);
+            int tile_phases = 1;
+            while (tile_phases * 2 <= kAnyPhases && tile_phases * 2 * wg_heads <= kAnyWaves &&
+                   (size_t)(tile_phases * 2 - 1) * phase_bytes <= (size_t)kAnyLdsBytes)
+                tile_phases *= 2;
+            paged_attn_anydim_balanced_kernel<NJ>
+                <<<dim3(p.num_workers, p.hkv / wg_heads), dim3(64 * wg_heads * tile_phases),
+                   (size_t)(tile_phases - 1) * phase_bytes, stream>>>(p, g, wg_heads, tile_phases);
+        } else {
+            launch(p.num_splits, p.num_seqs, 1, g, wg_heads);
+        }
+    }
     // rows of chunks: a workgroup walks a whole context, most of it out of L2, and the longest
     // walk sets the time of the launch -- more tile phases per head, fewer heads together
     if ((phases & LOGISMOS_ATTN_PHASE_PREFILL) && max_seqlen_q > 1)
@@ -510,6 +653,24 @@ static void launch_rows(const AttnParams& p, int total_tokens, int max_seqlen_q,
                wg_heads % 2 == 0 ? 2 : 1);
 }
 
+
+// Workers of a balanced launch per group of KV heads: one workgroup per CU (narrow heads fit
+// two, and measured slower with two: 62 vs 56 us at head_dim 64 on config 5's batch).
+static int64_t anydim_resident_workgroups(int) { return (int64_t)device_cu_count(); }
+
+// Workers of the balanced decode launch (0: static split -- one partition, a small batch, or
+// more sequences than the prefix table holds): what is resident at once per group of KV heads,
+// limited by the workspace the caller sized for num_splits partials per sequence (slots used:
+// at most workers + num_seqs - 1).
+static int anydim_workers(const AttnParams& p, int head_dim) {
+    if (p.num_splits <= 1 || p.num_seqs > kMaxBalancedSeqs ||
+        small_decode_batch(p.num_seqs, p.hkv, p.block_size, p.max_blocks_per_seq))
+        return 0;
+    int64_t target = anydim_resident_workgroups(head_dim) / (p.hkv / anydim_wg_heads(p.hkv));
+    if (target < 1) target = 1;
+    const int64_t cap = (int64_t)p.num_seqs * (p.num_splits - 1);
+    return (int)(target < cap ? target : cap);
+}
 
 // Workgroups = partitions x groups of KV heads.  Narrow heads (two workgroups fit a CU) aim at
 // two per CU, wide ones at half the CUs (one workgroup per CU and no second round even when
@@ -527,13 +688,23 @@ int paged_attn_anydim_num_splits(int num_seqs, int num_kv_heads, int head_dim, i
     int64_t splits = (2 * target + groups - 1) / groups;
     const int64_t most = (max_ctx + 127) / 128;
     if (splits > most) splits = most;
+    if (num_seqs <= kMaxBalancedSeqs &&
+        !small_decode_batch(num_seqs, num_kv_heads, block_size, max_blocks_per_seq)) {
+        // the balanced launch: slots for every resident workgroup (workers + num_seqs - 1)
+        const int64_t workers =
+            anydim_resident_workgroups(head_dim) / (num_kv_heads / anydim_wg_heads(num_kv_heads));
+        const int64_t need = (workers + num_seqs - 1) / num_seqs + 1;
+        if (splits < need) splits = need;
+    }
     if (splits > 4096) splits = 4096;
     if (splits < 1) splits = 1;
     return (int)splits;
 }
 
-hipError_t paged_attn_anydim_launch(const AttnParams& p, int head_dim, int total_tokens,
+hipError_t paged_attn_anydim_launch(const AttnParams& params, int head_dim, int total_tokens,
                                     int max_seqlen_q, int phases, hipStream_t stream) {
+    AttnParams p = params;
+    p.num_workers = anydim_workers(p, head_dim);
     if (head_dim <= 0 || head_dim % 32 != 0 || head_dim > 256) return hipErrorInvalidValue;
     if (p.hq % p.hkv != 0 || p.hq / p.hkv > 16) return hipErrorInvalidValue;
     if (total_tokens > 65535 || p.num_seqs > 65535 || p.hkv > 65535) return hipErrorInvalidValue;

@@ -45,6 +45,39 @@ __device__ __forceinline__ unsigned short attn_out_elem(float v, int out_bf16) {
     return __builtin_bit_cast(unsigned short, hv);
 }
 
+// ---- the balanced split of decode rows (both kernel families) -------------------------
+constexpr int kTileKeys = 16;
+
+// Units sequence s contributes to the decode stream: its 16-key tiles plus kSeqStartUnits for
+// starting it.  A worker that finishes one sequence and starts the next pays for a second
+// prologue (queries, first tiles with nothing in flight) and epilogue (row merge, partial
+// write): with equal tile counts such workers ended 3 us after the others and set the
+// duration of the launch.  With that cost in the stream they get fewer tiles (a tile of the
+// head_dim-128 kernel takes about 2.3 us); 3 to 5 units measured alike, 0 and 1 worse.
+constexpr int kSeqStartUnits = 4;
+__device__ __forceinline__ int decode_tiles(const AttnParams& p, int s) {
+    const int n_new = p.cu_seqlens_q[s + 1] - p.cu_seqlens_q[s];
+    const int ctx = p.context_lens[s];
+    return (n_new == 1 && ctx > 0) ? (ctx + kTileKeys - 1) / kTileKeys + kSeqStartUnits : 0;
+}
+
+constexpr int kMaxBalancedSeqs = 2048;  // prefix table held in LDS
+constexpr int kMinWorkerTiles = 8;      // a worker streams at least 128 keys
+
+__device__ __forceinline__ int worker_tiles(int total_tiles, int num_workers) {
+    const int r = (total_tiles + num_workers - 1) / num_workers;
+    return r < kMinWorkerTiles ? kMinWorkerTiles : r;
+}
+
+// Small batches stay on the static split: when every partition of every sequence is
+// resident at once there is no second round to balance away, and the balanced kernel's
+// prologue (prefix table, search) costs more than it saves (config 2: 12.7 vs 18 us).
+// The bound is on what the block tables could hold, the only size the host knows.
+inline bool small_decode_batch(int num_seqs, int num_kv_heads, int block_size,
+                               int max_blocks_per_seq) {
+    return (int64_t)num_seqs * num_kv_heads * block_size * max_blocks_per_seq <= 200000;
+}
+
 // The kernel for head widths other than 128 (multiples of 32 up to 256, GQA groups up to 16):
 // decode rows on the static split, rows of sequences with several new tokens over their whole
 // visible context, then the merge of the decode partitions.  `phases` as in the public launcher.

@@ -140,3 +140,24 @@ def test_randomized_ragged_batches(seed):
     causal = bool(rng.integers(0, 2))
     ns = [None, 1, int(rng.integers(2, 40))][seed % 3]
     _check(c, num_splits=ns, causal=causal, what=f"{what} causal={causal} splits={ns}")
+
+
+@pytest.mark.parametrize("d,hq,hkv", [(64, 32, 8), (64, 14, 2), (96, 12, 4), (256, 8, 8), (32, 16, 1)])
+def test_balanced_split_of_large_batches(d, hq, hkv):
+    # block tables wide enough that the launch takes the balanced split (its size test looks at
+    # what the tables could hold): the tiles of all sequences dealt evenly to the workers,
+    # sequences that start and end inside a worker, a row without context, single keys
+    rng = np.random.default_rng(7000 + d + hq)
+    ctx = np.array([1, 3000, 17, 1, 640, 5000, 33, 2, 900, 128, 129, 4097, 16, 15, 700, 31])
+    c = workloads.paged_case(rng, np.ones(len(ctx), np.int32), ctx - 1, hq=hq, hkv=hkv, d=d,
+                             min_max_blocks=2048)
+    c["context_lens"][3] = 0
+    _check(c, what=f"balanced d={d} {hq}/{hkv}")
+    _check(c, num_splits=2, what=f"balanced d={d} {hq}/{hkv}, 2 splits (few workers)")
+    _check(c, num_splits=40, what=f"balanced d={d} {hq}/{hkv}, 40 splits")
+    # a mixed batch on the same wide tables: chunks beside balanced decode rows
+    new = [1, 40, 1, 1, 7, 1, 1, 130]
+    prior = [2000, 100, 0, 4000, 0, 777, 15, 300]
+    c = workloads.paged_case(rng, new, prior, hq=hq, hkv=hkv, d=d, min_max_blocks=2048)
+    _check(c, what=f"balanced mixed d={d} {hq}/{hkv}")
+    _check(c, causal=False, num_splits=9, what=f"balanced mixed non-causal d={d} {hq}/{hkv}")
