@@ -510,6 +510,8 @@ __global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_balanced_ker
         if (tile_hi > tile_lo) {
             const int ctx = p.context_lens[s];
             const bool single = tile_lo == 0 && seg_end == seq_end;
+            // (inlined: as a call the body needs its frame in scratch memory; four tile buffers
+            // instead of two measured no faster at head_dim 64, 46.8 vs 45.6 us)
             anydim_range<NJ>(p, G, wg_heads, phases, G, s, p.cu_seqlens_q[s], 1, ctx, ctx,
                              tile_lo * kTileKeys, min(ctx, tile_hi * kTileKeys), single,
                              (int64_t)w + s, sm_m, sm_l, sm_acc);
@@ -662,8 +664,14 @@ static int64_t anydim_resident_workgroups(int) { return (int64_t)device_cu_count
 // more sequences than the prefix table holds): what is resident at once per group of KV heads,
 // limited by the workspace the caller sized for num_splits partials per sequence (slots used:
 // at most workers + num_seqs - 1).
+static bool anydim_balanced_width(int head_dim) {
+    // above 192 the worker loop around the body runs out of registers (it spills at 256, and
+    // the static split measured faster there: 227 vs 240-248 us on config 5's batch)
+    return head_dim <= 192;
+}
+
 static int anydim_workers(const AttnParams& p, int head_dim) {
-    if (p.num_splits <= 1 || p.num_seqs > kMaxBalancedSeqs ||
+    if (!anydim_balanced_width(head_dim) || p.num_splits <= 1 || p.num_seqs > kMaxBalancedSeqs ||
         small_decode_batch(p.num_seqs, p.hkv, p.block_size, p.max_blocks_per_seq))
         return 0;
     int64_t target = anydim_resident_workgroups(head_dim) / (p.hkv / anydim_wg_heads(p.hkv));
@@ -688,7 +696,7 @@ int paged_attn_anydim_num_splits(int num_seqs, int num_kv_heads, int head_dim, i
     int64_t splits = (2 * target + groups - 1) / groups;
     const int64_t most = (max_ctx + 127) / 128;
     if (splits > most) splits = most;
-    if (num_seqs <= kMaxBalancedSeqs &&
+    if (anydim_balanced_width(head_dim) && num_seqs <= kMaxBalancedSeqs &&
         !small_decode_batch(num_seqs, num_kv_heads, block_size, max_blocks_per_seq)) {
         // the balanced launch: slots for every resident workgroup (workers + num_seqs - 1)
         const int64_t workers =
