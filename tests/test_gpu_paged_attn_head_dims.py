@@ -161,3 +161,17 @@ def test_balanced_split_of_large_batches(d, hq, hkv):
     c = workloads.paged_case(rng, new, prior, hq=hq, hkv=hkv, d=d, min_max_blocks=2048)
     _check(c, what=f"balanced mixed d={d} {hq}/{hkv}")
     _check(c, causal=False, num_splits=9, what=f"balanced mixed non-causal d={d} {hq}/{hkv}")
+
+
+@pytest.mark.parametrize("d", [64, 128])
+def test_more_decode_sequences_than_the_balanced_split_holds(d):
+    # 2100 decode sequences: past the prefix table of the balanced launches (2048 entries), so
+    # both kernel families fall back to the static split; also a batch of 2048, the last that
+    # takes the balanced one
+    for n in (2100, 2048):
+        rng = np.random.default_rng(d + n)
+        ctx = rng.integers(1, 60, size=n)
+        c = workloads.paged_case(rng, np.ones(n, np.int32), ctx - 1, hq=4, hkv=2, d=d,
+                                 min_max_blocks=8)
+        _check(c, what=f"{n} sequences, d={d}")
+        _check(c, num_splits=3, what=f"{n} sequences, d={d}, 3 splits")
