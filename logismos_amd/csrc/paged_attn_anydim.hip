@@ -66,22 +66,30 @@ struct AnyTile {
 typedef unsigned __attribute__((ext_vector_type(4), aligned(4))) uint4_a4_t;
 typedef unsigned __attribute__((ext_vector_type(2), aligned(4))) uint2_a4_t;
 
+// A load that is (NT) or is not marked non-temporal: decode rows use every K/V byte once per
+// launch, rows of chunks read theirs many times out of L2.
+template <bool NT, typename T>
+__device__ __forceinline__ T load_kv(const T* ptr) {
+    if constexpr (NT) return __builtin_nontemporal_load(ptr);
+    else return *ptr;
+}
+
 // N consecutive dwords, aligned to 4 bytes, in as few requests as N allows
-template <int N>
+template <int N, bool NT>
 __device__ __forceinline__ void load_dwords(const void* src, unsigned (&dst)[N]) {
     const unsigned* sp = static_cast<const unsigned*>(src);
     int i = 0;
 #pragma unroll
     for (; i + 4 <= N; i += 4) {
-        const uint4_a4_t x = *reinterpret_cast<const uint4_a4_t*>(sp + i);
+        const uint4_a4_t x = load_kv<NT>(reinterpret_cast<const uint4_a4_t*>(sp + i));
         dst[i] = x[0], dst[i + 1] = x[1], dst[i + 2] = x[2], dst[i + 3] = x[3];
     }
     if (N - i >= 2) {
-        const uint2_a4_t x = *reinterpret_cast<const uint2_a4_t*>(sp + i);
+        const uint2_a4_t x = load_kv<NT>(reinterpret_cast<const uint2_a4_t*>(sp + i));
         dst[i] = x[0], dst[i + 1] = x[1];
         i += 2;
     }
-    if (N - i == 1) dst[i] = sp[i];
+    if (N - i == 1) dst[i] = load_kv<NT>(sp + i);
 }
 
 __device__ __forceinline__ float lane_read_f32(float v, int src_lane) {
@@ -103,7 +111,7 @@ __device__ __forceinline__ int seq_of_row(const int32_t* cu, int num_seqs, int t
 // ntok query tokens from packed row t on: scores, softmax, P.V, the merge of the tile phases,
 // and either the finished rows (single) or the partial (m, l, acc) at workspace slot `slot`.
 // Called by every wave of the workgroup (it holds two barriers).
-template <int NJ>
+template <int NJ, bool NT>
 __device__ __forceinline__ void anydim_range(const AttnParams& p, int G, int wg_heads, int phases,
                                              int cols, int s, int t, int ntok, int vis_first,
                                              int visible, int key_begin, int key_end, bool single,
@@ -163,18 +171,19 @@ __device__ __forceinline__ void anydim_range(const AttnParams& p, int G, int wg_
                 const unsigned koff = (unsigned)min(8 * kh + (c & 7), lim) * row_bytes + k_lane;
 #pragma unroll
                 for (int u = 0; u < NJ / 2; ++u)
-                    tl.k[2 * u + kh] = *reinterpret_cast<const half8_t*>(kb + koff + 128 * u);
+                    tl.k[2 * u + kh] =
+                        load_kv<NT>(reinterpret_cast<const half8_t*>(kb + koff + 128 * u));
             }
         } else {
             const unsigned koff = (unsigned)min(c, lim) * row_bytes + k_lane;
 #pragma unroll
             for (int j = 0; j < NJ; ++j)
-                tl.k[j] = *reinterpret_cast<const half8_t*>(kb + koff + 64 * j);
+                tl.k[j] = load_kv<NT>(reinterpret_cast<const half8_t*>(kb + koff + 64 * j));
         }
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const unsigned voff = (unsigned)min(4 * tg + r, lim) * row_bytes + v_lane;
-            load_dwords<NJ>(vb + voff, tl.v[r]);
+            load_dwords<NJ, NT>(vb + voff, tl.v[r]);
         }
     };
 
@@ -441,8 +450,11 @@ __global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_kernel(const
     }
     if (key_begin >= key_end) return;
 
-    anydim_range<NJ>(p, G, wg_heads, phases, cols, s, t, ntok, vis_first, visible, key_begin,
-                     key_end, single, (int64_t)s * p.num_splits + split, sm_m, sm_l, sm_acc);
+    // (plain loads: rows of chunks read their keys many times out of L2, and the short
+    // partitions of a small decode batch measured slower with non-temporal ones, 10.2 vs 9.3 us)
+    anydim_range<NJ, false>(p, G, wg_heads, phases, cols, s, t, ntok, vis_first, visible,
+                            key_begin, key_end, single, (int64_t)s * p.num_splits + split, sm_m,
+                            sm_l, sm_acc);
 }
 
 // Decode rows, balanced: the 16-key tiles of all decode sequences form one stream (each
@@ -512,7 +524,11 @@ __global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_balanced_ker
             const bool single = tile_lo == 0 && seg_end == seq_end;
             // (inlined: as a call the body needs its frame in scratch memory; four tile buffers
             // instead of two measured no faster at head_dim 64, 46.8 vs 45.6 us)
-            anydim_range<NJ>(p, G, wg_heads, phases, G, s, p.cu_seqlens_q[s], 1, ctx, ctx,
+            // Non-temporal K/V loads where every request covers whole 128-byte lines, i.e. at
+            // head_dim 64 (41.9 vs 45.6 us on config 5's batch).  Wider heads split a line of V
+            // between two requests, and marked non-temporal the second one fetches it again
+            // (head_dim 256, static split: 273 vs 227 us).
+            anydim_range<NJ, NJ == 2>(p, G, wg_heads, phases, G, s, p.cu_seqlens_q[s], 1, ctx, ctx,
                              tile_lo * kTileKeys, min(ctx, tile_hi * kTileKeys), single,
                              (int64_t)w + s, sm_m, sm_l, sm_acc);
         }
