@@ -24,10 +24,11 @@
 //     32j + 8tg .. + 8 of key c directly (neighbouring lanes on different rows).
 //   * one running maximum per head shared by the four lane rows, sums per lane row.
 //   * P.V on v_mfma_f32_16x16x16_f16: A = the probabilities as two fp16 terms (head c, keys
-//     4tg + r: the layout the scores arrive in), B = V (lane: E = head_dim / 16 consecutive
-//     elements E c .. E c + E - 1 of its keys 4tg + r, one load of 2E bytes per key; MFMA e
-//     takes element e, so its output column c is element E c + e); lane (tg, c) ends up with
-//     the heads 4tg + r at its E elements.
+//     4tg + r: the layout the scores arrive in), B = V (lane: E = head_dim / 16 elements of
+//     its keys 4tg + r, in chunks of 8, 4 or 2 consecutive ones such that a request covers 16
+//     lanes x one chunk = a run of consecutive bytes of the row, see v_chunk_pos; MFMA e takes
+//     the lane's element e, so its output column c is that element's place in the row); lane
+//     (tg, c) ends up with the heads 4tg + r at its E elements.
 // Decode rows (one new token) are split into partitions of part_tokens keys whose partials
 // (m, l, acc) the merge kernel combines.  Rows of sequences with several new tokens: the 16
 // columns of a score tile are (query token, head) pairs, 16 / G consecutive tokens of a chunk
@@ -63,9 +64,6 @@ struct AnyTile {
     unsigned v[4][NJ];  // key 4tg + r: the lane's 2 NJ elements, two per dword
 };
 
-typedef unsigned __attribute__((ext_vector_type(4), aligned(4))) uint4_a4_t;
-typedef unsigned __attribute__((ext_vector_type(2), aligned(4))) uint2_a4_t;
-
 // A load that is (NT) or is not marked non-temporal: decode rows use every K/V byte once per
 // launch, rows of chunks read theirs many times out of L2.
 template <bool NT, typename T>
@@ -74,22 +72,34 @@ __device__ __forceinline__ T load_kv(const T* ptr) {
     else return *ptr;
 }
 
-// N consecutive dwords, aligned to 4 bytes, in as few requests as N allows
+// Which of a head row's elements a lane holds for P.V: its E = head_dim / 16 elements come in
+// chunks of 8, 4 or 2 (E = 14: 8 + 4 + 2), and chunk (eo, len) of lane c is the elements
+// 16 eo + c len .. + len - 1 of the row -- so a request for one chunk of one row covers
+// 16 lanes x len consecutive elements, whole 128-byte lines where len >= 4.
+constexpr int v_chunk_len(int E, int eo) { return E - eo >= 8 ? 8 : (E - eo >= 4 ? 4 : 2); }
+constexpr int v_chunk_start(int E, int e) {
+    int eo = 0;
+    while (e >= eo + v_chunk_len(E, eo)) eo += v_chunk_len(E, eo);
+    return eo;
+}
+// first element of the chunk that holds the lane's element e, as a position in the row
+__device__ __forceinline__ constexpr int v_chunk_pos(int E, int e, int c) {
+    return 16 * v_chunk_start(E, e) + c * v_chunk_len(E, v_chunk_start(E, e));
+}
+
+// N consecutive dwords (N = 1, 2, 4: a chunk of V, aligned to its own size)
 template <int N, bool NT>
-__device__ __forceinline__ void load_dwords(const void* src, unsigned (&dst)[N]) {
-    const unsigned* sp = static_cast<const unsigned*>(src);
-    int i = 0;
-#pragma unroll
-    for (; i + 4 <= N; i += 4) {
-        const uint4_a4_t x = load_kv<NT>(reinterpret_cast<const uint4_a4_t*>(sp + i));
-        dst[i] = x[0], dst[i + 1] = x[1], dst[i + 2] = x[2], dst[i + 3] = x[3];
+__device__ __forceinline__ void load_dwords(const void* src, unsigned* dst) {
+    static_assert(N == 1 || N == 2 || N == 4, "a chunk of 2, 4 or 8 elements");
+    if constexpr (N == 4) {
+        const uint4_t x = load_kv<NT>(static_cast<const uint4_t*>(src));
+        dst[0] = x[0], dst[1] = x[1], dst[2] = x[2], dst[3] = x[3];
+    } else if constexpr (N == 2) {
+        const uint2_t x = load_kv<NT>(static_cast<const uint2_t*>(src));
+        dst[0] = x[0], dst[1] = x[1];
+    } else {
+        dst[0] = load_kv<NT>(static_cast<const unsigned*>(src));
     }
-    if (N - i >= 2) {
-        const uint2_a4_t x = load_kv<NT>(reinterpret_cast<const uint2_a4_t*>(sp + i));
-        dst[i] = x[0], dst[i + 1] = x[1];
-        i += 2;
-    }
-    if (N - i == 1) dst[i] = load_kv<NT>(sp + i);
 }
 
 __device__ __forceinline__ float lane_read_f32(float v, int src_lane) {
@@ -154,7 +164,6 @@ __device__ __forceinline__ void anydim_range(const AttnParams& p, int G, int wg_
     // lane offset (key of the tile x row bytes + the lane's bytes inside the head row).
     const unsigned row_bytes = (unsigned)p.hkv * D * 2;  // (hkv <= 65535: 16 rows < 2^31)
     const unsigned k_lane = kLines ? 32 * tg + 16 * (c >> 3) : 16 * tg;
-    const unsigned v_lane = 2 * E * c;
 
     auto load_tile = [&](int tile_begin, int block, int off_in_block, AnyTile<NJ>& tl) {
         const int64_t row0_bytes =
@@ -182,8 +191,13 @@ __device__ __forceinline__ void anydim_range(const AttnParams& p, int G, int wg_
         }
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const unsigned voff = (unsigned)min(4 * tg + r, lim) * row_bytes + v_lane;
-            load_dwords<NJ, NT>(vb + voff, tl.v[r]);
+            const unsigned voff = (unsigned)min(4 * tg + r, lim) * row_bytes;
+            static_for<E>([&](auto ec) {
+                constexpr int e = decltype(ec)::value;
+                if constexpr (v_chunk_start(E, e) == e)  // one request per chunk
+                    load_dwords<v_chunk_len(E, e) / 2, NT>(vb + voff + 2 * v_chunk_pos(E, e, c),
+                                                           &tl.v[r][e / 2]);
+            });
         }
     };
 
@@ -362,18 +376,21 @@ __device__ __forceinline__ void anydim_range(const AttnParams& p, int G, int wg_
         if (single) {
             const float inv = lh > 0.0f ? 1.0f / lh : 0.0f;  // a token that sees no key: zeros
             unsigned short* dst = reinterpret_cast<unsigned short*>(p.out) +
-                                  ((int64_t)(t + htok) * p.hq + head) * D + E * c;
-#pragma unroll
-            for (int e = 0; e < E; e += 2) {
+                                  ((int64_t)(t + htok) * p.hq + head) * D;
+            static_for<E / 2>([&](auto ec) {
+                constexpr int e = 2 * decltype(ec)::value;
                 const unsigned w = (unsigned)attn_out_elem(acc[e][r] * inv, p.out_bf16) |
                                    ((unsigned)attn_out_elem(acc[e + 1][r] * inv, p.out_bf16) << 16);
-                *reinterpret_cast<unsigned*>(dst + e) = w;
-            }
+                *reinterpret_cast<unsigned*>(dst + v_chunk_pos(E, e, c) +
+                                             (e - v_chunk_start(E, e))) = w;
+            });
         } else {
             const int64_t idx = slot * p.hq + head;
-            float* dst = p.ws_acc + idx * D + E * c;
-#pragma unroll
-            for (int e = 0; e < E; ++e) dst[e] = acc[e][r];
+            float* dst = p.ws_acc + idx * D;
+            static_for<E>([&](auto ec) {
+                constexpr int e = decltype(ec)::value;
+                dst[v_chunk_pos(E, e, c) + (e - v_chunk_start(E, e))] = acc[e][r];
+            });
             if (c == 0) {
                 p.ws_ml[idx * 2] = mh;
                 p.ws_ml[idx * 2 + 1] = lh;
@@ -524,11 +541,12 @@ __global__ __launch_bounds__(64 * kAnyWaves) void paged_attn_anydim_balanced_ker
             const bool single = tile_lo == 0 && seg_end == seq_end;
             // (inlined: as a call the body needs its frame in scratch memory; four tile buffers
             // instead of two measured no faster at head_dim 64, 46.8 vs 45.6 us)
-            // Non-temporal K/V loads where every request covers whole 128-byte lines, i.e. at
-            // head_dim 64 (41.9 vs 45.6 us on config 5's batch).  Wider heads split a line of V
-            // between two requests, and marked non-temporal the second one fetches it again
-            // (head_dim 256, static split: 273 vs 227 us).
-            anydim_range<NJ, NJ == 2>(p, G, wg_heads, phases, G, s, p.cu_seqlens_q[s], 1, ctx, ctx,
+            // Non-temporal K/V loads where every request covers whole 128-byte lines: head_dim
+            // a multiple of 64 (K requested line-wise, V in chunks of 4 or 8 elements per lane).
+            // Config 5's batch: 41.9 vs 45.6 us at head_dim 64, 228-235 vs 240-248 us at 256.
+            // Otherwise a line is split between requests and the later one, marked non-temporal,
+            // fetches it again.
+            anydim_range<NJ, NJ % 2 == 0>(p, G, wg_heads, phases, G, s, p.cu_seqlens_q[s], 1, ctx, ctx,
                              tile_lo * kTileKeys, min(ctx, tile_hi * kTileKeys), single,
                              (int64_t)w + s, sm_m, sm_l, sm_acc);
         }
@@ -671,7 +689,6 @@ static void launch_rows(const AttnParams& p, int total_tokens, int max_seqlen_q,
                wg_heads % 2 == 0 ? 2 : 1);
 }
 
-
 // Workers of a balanced launch per group of KV heads: one workgroup per CU (narrow heads fit
 // two, and measured slower with two: 62 vs 56 us at head_dim 64 on config 5's batch).
 static int64_t anydim_resident_workgroups(int) { return (int64_t)device_cu_count(); }
@@ -680,14 +697,8 @@ static int64_t anydim_resident_workgroups(int) { return (int64_t)device_cu_count
 // more sequences than the prefix table holds): what is resident at once per group of KV heads,
 // limited by the workspace the caller sized for num_splits partials per sequence (slots used:
 // at most workers + num_seqs - 1).
-static bool anydim_balanced_width(int head_dim) {
-    // above 192 the worker loop around the body runs out of registers (it spills at 256, and
-    // the static split measured faster there: 227 vs 240-248 us on config 5's batch)
-    return head_dim <= 192;
-}
-
 static int anydim_workers(const AttnParams& p, int head_dim) {
-    if (!anydim_balanced_width(head_dim) || p.num_splits <= 1 || p.num_seqs > kMaxBalancedSeqs ||
+    if (p.num_splits <= 1 || p.num_seqs > kMaxBalancedSeqs ||
         small_decode_batch(p.num_seqs, p.hkv, p.block_size, p.max_blocks_per_seq))
         return 0;
     int64_t target = anydim_resident_workgroups(head_dim) / (p.hkv / anydim_wg_heads(p.hkv));
@@ -712,7 +723,7 @@ int paged_attn_anydim_num_splits(int num_seqs, int num_kv_heads, int head_dim, i
     int64_t splits = (2 * target + groups - 1) / groups;
     const int64_t most = (max_ctx + 127) / 128;
     if (splits > most) splits = most;
-    if (anydim_balanced_width(head_dim) && num_seqs <= kMaxBalancedSeqs &&
+    if (num_seqs <= kMaxBalancedSeqs &&
         !small_decode_batch(num_seqs, num_kv_heads, block_size, max_blocks_per_seq)) {
         // the balanced launch: slots for every resident workgroup (workers + num_seqs - 1)
         const int64_t workers =
