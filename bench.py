@@ -786,6 +786,21 @@ def bench_head_dim64(args):
     _, ms_mixed = timed(mixed)
     _, ms_mixed_chunks = timed(mixed, kernels.ATTN_PHASE_PREFILL)
     achieved = algo / (ms_dec * 1e-3) / 1e9
+
+    # a whole decode step at Qwen2-0.5B's geometry (24 layers, hidden 896, 14 q / 2 kv heads of
+    # 64, MLP 4864, q/k/v bias), 32 live sequences at fixed contexts U[256,8192]; the layers
+    # share one layer's weights (replicated on the device) as the headline step's do
+    from tests.gpu_harness import DecodeStepRunner
+    S, L = 32, 24
+    ctx = rng.integers(256, 8193, size=S)
+    cfg, layers, batch = workloads.decode_step_problem(
+        rng, num_layers=1, hidden=896, hq=14, hkv=2, inter=4864, ctx=ctx, d=64,
+        random_nibbles=True, qkv_bias=True, theta=1e4)
+    r = DecodeStepRunner(cfg, layers * L, batch, stream=stream, share_layer_data=True)
+    ms_model = time_launches(stream, [r.launch], 20, 3)[0]
+    kv_bytes_step = int(ctx.sum()) * 2 * 2 * 64 * 2 * L
+    w_bytes_layer = sum(w[0].nbytes + w[1].nbytes + w[2].nbytes
+                        for w in (layers[0][k] for k in ("qkv", "o", "gate_up", "down")))
     return {
         "metric": "paged-attn decode achieved HBM GB/s (head_dim 64)",
         "value": round(algo / (ms_full * 1e-3) / 1e9, 1), "unit": "GB/s", "n_gpus": 1,
@@ -808,6 +823,11 @@ def bench_head_dim64(args):
                                             float(np.abs(got - want).max())},
         "mixed_2x512_token_chunks_6_decode_rows": {"ms_per_step": round(ms_mixed, 5),
                                                    "ms_chunk_rows": round(ms_mixed_chunks, 5)},
+        "decode_step_qwen2_05b_geometry": {"ms_per_step": round(ms_model, 4),
+                                           "tok_s": round(S / (ms_model * 1e-3), 1),
+                                           "layers": L, "sum_ctx": int(ctx.sum()),
+                                           "num_splits": r.num_splits,
+                                           "bytes_per_step": kv_bytes_step + w_bytes_layer * L},
     }
 
 
