@@ -313,7 +313,7 @@ size_t logismos_paged_attn_workspace_bytes(int num_seqs, int num_q_heads, int he
  * num_q_heads % num_kv_heads == 0 and head_dim == 128 with a group size
  * num_q_heads/num_kv_heads <= 8 (the kernels the decode step of the headline
  * configuration runs on), or any other head_dim that is a multiple of 32 up to
- * 256 with a group size <= 16 and total_tokens <= 65535 (a general kernel:
+ * 256 with a group size <= 16 and total_tokens <= 65520 (a general kernel:
  * decode rows on a static split, every row of a chunk over its whole visible
  * context; `QwenAttention` is generic in head_dim,
  * crates/transformers/src/attention.rs:97-127). */

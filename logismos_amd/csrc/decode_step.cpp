@@ -114,6 +114,12 @@ bool config_ok(const logismos_decode_config_t* c, int num_seqs, int t, int max_s
     // attention kernel (fp16 pools only: a turbo3 head row is 128 wide)
     if (c->head_dim <= 0 || c->head_dim % 32 != 0 || c->head_dim > 256) return false;
     if (c->head_dim != 128 && c->kv_turbo3) return false;
+    // what the attention launcher accepts, checked here so that no step is launched in part:
+    // GQA groups up to 8 (16 on the general kernel), whose packed rows end at 65520
+    if (c->num_q_heads % c->num_kv_heads != 0 ||
+        c->num_q_heads / c->num_kv_heads > (c->head_dim == 128 ? 8 : 16))
+        return false;
+    if (c->head_dim != 128 && t > 65520) return false;
     if (c->hidden % 128 != 0 || c->intermediate % 128 != 0) return false;
     if (((int64_t)c->num_q_heads * c->head_dim) % 128 != 0) return false;
     // every position a block table can hold must have a row in the RoPE tables

@@ -1620,8 +1620,9 @@ extern "C" logismos_status_t logismos_check_paged_attn_shape(int num_seqs, int t
     if (num_q_heads / num_kv_heads > (head_dim == lg::kHeadDim ? 8 : 16))
         return lg::reject(msg, msg_cap, "%s: GQA group size %d exceeds %d at head_dim %d", k,
                           num_q_heads / num_kv_heads, head_dim == lg::kHeadDim ? 8 : 16, head_dim);
-    if (head_dim != lg::kHeadDim && total_tokens > 65535)
-        return lg::reject(msg, msg_cap, "%s: total_tokens must be <= 65535 at head_dim %d", k,
+    // (the general kernel walks the packed rows, padded to groups of up to 16, in grid.z)
+    if (head_dim != lg::kHeadDim && total_tokens > 65520)
+        return lg::reject(msg, msg_cap, "%s: total_tokens must be <= 65520 at head_dim %d", k,
                           head_dim);
     if (num_seqs > 65535 || num_kv_heads > 65535)
         return lg::reject(msg, msg_cap, "%s: num_seqs and num_kv_heads must be <= 65535", k);

@@ -742,7 +742,7 @@ hipError_t paged_attn_anydim_launch(const AttnParams& params, int head_dim, int 
     p.num_workers = anydim_workers(p, head_dim);
     if (head_dim <= 0 || head_dim % 32 != 0 || head_dim > 256) return hipErrorInvalidValue;
     if (p.hq % p.hkv != 0 || p.hq / p.hkv > 16) return hipErrorInvalidValue;
-    if (total_tokens > 65535 || p.num_seqs > 65535 || p.hkv > 65535) return hipErrorInvalidValue;
+    if (total_tokens > 65520 || p.num_seqs > 65535 || p.hkv > 65535) return hipErrorInvalidValue;
     if (p.out_bf16 != 0 && p.out_bf16 != 1) return hipErrorInvalidValue;
     if (phases & (LOGISMOS_ATTN_PHASE_DECODE | LOGISMOS_ATTN_PHASE_PREFILL)) {
         switch (head_dim / 32) {

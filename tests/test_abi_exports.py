@@ -69,7 +69,7 @@ def test_qgemv_q8_shape_guard_accepts_config1():
     (dict(head_dim=80), "head_dim must be a multiple of 32 up to 256"),
     (dict(head_dim=288), "head_dim must be a multiple of 32 up to 256"),
     (dict(head_dim=64, num_q_heads=34, num_kv_heads=2), "group size 17 exceeds 16"),
-    (dict(head_dim=64, num_seqs=2, total_tokens=70000, max_seqlen_q=40000), "<= 65535"),
+    (dict(head_dim=64, num_seqs=2, total_tokens=65530, max_seqlen_q=40000), "<= 65520"),
     (dict(block_size=24), "multiple of 16"),
     (dict(num_q_heads=12, num_kv_heads=5), "not a multiple of num_kv_heads"),
     (dict(num_q_heads=32, num_kv_heads=2), "group size 16 exceeds 8"),
