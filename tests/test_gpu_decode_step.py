@@ -264,3 +264,12 @@ def test_step_rejects_what_it_cannot_run():
     r.batch.total_tokens, r.batch.max_seqlen_q = 0, 0
     assert call() == 0
     hip.synchronize()
+    # head widths and GQA groups the attention launchers would refuse are refused up front
+    keep = (r.cfg.head_dim, r.cfg.num_q_heads, r.cfg.kv_turbo3)
+    for head_dim, hq_, t3 in ((80, 4, 0), (288, 4, 0), (64, 8, 1), (128, 18, 0), (64, 34, 0),
+                              (128, 5, 0)):
+        r.cfg.head_dim, r.cfg.num_q_heads, r.cfg.kv_turbo3 = head_dim, hq_, t3
+        assert call() == 1, (head_dim, hq_, t3)
+    r.cfg.head_dim, r.cfg.num_q_heads, r.cfg.kv_turbo3 = keep
+    assert call() == 0
+    hip.synchronize()
