@@ -1,8 +1,7 @@
 // Ragged paged attention for head widths other than 128 (fp16 KV, fp32 softmax): head_dim a
 // multiple of 32 up to 256, GQA groups up to 16 heads.  Same semantics as the head_dim-128
 // kernels (crates/kernels/src/cpu_f32/mod.rs:380-433 attention, :502-547 softmax; the GQA map
-// of crates/transformers/src/attention.rs:233-260), not tuned to their degree: one kernel for
-// every row of the ragged batch.
+// of crates/transformers/src/attention.rs:233-260); one body for every row of the ragged batch.
 //
 // One wave64 serves the whole GQA group of one KV head over 16-key tiles of one (query
 // token, KV partition).  A workgroup of up to eight waves is (KV heads) x (tile phases): its
@@ -29,8 +28,9 @@
 //     lanes x one chunk = a run of consecutive bytes of the row, see v_chunk_pos; MFMA e takes
 //     the lane's element e, so its output column c is that element's place in the row); lane
 //     (tg, c) ends up with the heads 4tg + r at its E elements.
-// Decode rows (one new token) are split into partitions of part_tokens keys whose partials
-// (m, l, acc) the merge kernel combines.  Rows of sequences with several new tokens: the 16
+// Decode rows (one new token): a small batch is split into partitions of part_tokens keys, a
+// large one evenly over one worker per CU (the balanced kernel below); the partials (m, l, acc)
+// are combined by the merge kernel.  Rows of sequences with several new tokens: the 16
 // columns of a score tile are (query token, head) pairs, 16 / G consecutive tokens of a chunk
 // per wave, each column masked at its own token's visible length; such a wave takes the whole
 // context its last token sees.
