@@ -815,11 +815,19 @@ logismos_status_t logismos_launch_paged_attn_varlen_turbo3(
  * crates/kernels/examples/gemm_bench.rs:120-128).  A plain copy and a plain
  * read of `bytes` bytes (multiple of 16, 16-byte aligned): the achievable HBM
  * ceiling of the box, and the calibration for FETCH_SIZE / WRITE_SIZE.
+ * `_read_ex` takes flags: non-temporal loads (what the decode attention reads
+ * K and V with), and 256 resident workgroups taking chunks in turn instead of
+ * 2048 workgroups with a slab each; the read ceiling at a size is the best of
+ * the four.
  * ------------------------------------------------------------------------ */
+#define LOGISMOS_PROBE_NON_TEMPORAL 1
+#define LOGISMOS_PROBE_STRIDED 2
 logismos_status_t logismos_launch_probe_copy(const void* src, void* dst, size_t bytes,
                                              logismos_stream_t stream);
 logismos_status_t logismos_launch_probe_read(const void* src, void* sink_u32, size_t bytes,
                                              logismos_stream_t stream);
+logismos_status_t logismos_launch_probe_read_ex(const void* src, void* sink_u32, size_t bytes,
+                                                int flags, logismos_stream_t stream);
 
 #ifdef __cplusplus
 }

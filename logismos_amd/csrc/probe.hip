@@ -1,5 +1,5 @@
 // Memory-system probes: a plain 16-byte-per-lane copy kernel and a read-only
-// sum kernel.  They give the box's achievable HBM ceiling next to the
+// sum kernel (plain or non-temporal loads).  They give the box's achievable HBM ceiling next to the
 // datasheet figure, and the calibration factor for the FETCH_SIZE /
 // WRITE_SIZE hardware counters (a copy of known size).
 #include "device_utils.hpp"
@@ -14,22 +14,31 @@ __global__ __launch_bounds__(256) void probe_copy_kernel(const uint4_t* __restri
         dst[i] = src[i];
 }
 
-// Each workgroup reads a contiguous slab, 4 x 16 bytes per lane in flight.
-__global__ __launch_bounds__(256) void probe_read_kernel(const uint4_t* __restrict__ src,
+// Read-only sum, 4 x 16 bytes per lane in flight.  NT: the loads are non-temporal, as the decode
+// attention reads K and V (every byte used once per step).  STRIDED: the workgroups take
+// chunks of blockDim.x * 4 pieces in turn (grid-stride) instead of one contiguous slab each.
+template <bool NT, bool STRIDED>
+__global__ __launch_bounds__(512) void probe_read_kernel(const uint4_t* __restrict__ src,
                                                          unsigned* __restrict__ sink, int64_t n16) {
-    const int64_t per_block = (n16 + gridDim.x - 1) / gridDim.x;
-    const int64_t begin = (int64_t)blockIdx.x * per_block;
-    const int64_t end = begin + per_block < n16 ? begin + per_block : n16;
-    unsigned acc = 0;
-    int64_t i = begin + threadIdx.x;
-    for (; i + 3 * 256 < end; i += 4 * 256) {
-        const uint4_t a = src[i], b = src[i + 256], c = src[i + 512], d = src[i + 768];
-        acc ^= a[0] ^ a[1] ^ a[2] ^ a[3] ^ b[0] ^ b[1] ^ b[2] ^ b[3];
-        acc ^= c[0] ^ c[1] ^ c[2] ^ c[3] ^ d[0] ^ d[1] ^ d[2] ^ d[3];
+    const int64_t T = blockDim.x;
+    const int64_t chunks = (n16 + 4 * T - 1) / (4 * T);
+    int64_t c0, c1, cs;
+    if (STRIDED) {
+        c0 = blockIdx.x, c1 = chunks, cs = gridDim.x;
+    } else {
+        const int64_t per = (chunks + gridDim.x - 1) / gridDim.x;
+        c0 = (int64_t)blockIdx.x * per, c1 = c0 + per < chunks ? c0 + per : chunks, cs = 1;
     }
-    for (; i < end; i += 256) {
-        const uint4_t a = src[i];
-        acc ^= a[0] ^ a[1] ^ a[2] ^ a[3];
+    auto ld = [&](int64_t j) {
+        j = j < n16 ? j : n16 - 1;  // the ragged tail re-reads the last piece
+        return NT ? __builtin_nontemporal_load(src + j) : src[j];
+    };
+    unsigned acc = 0;
+    for (int64_t c = c0; c < c1; c += cs) {
+        const int64_t i = c * 4 * T + threadIdx.x;
+        const uint4_t a = ld(i), b = ld(i + T), e = ld(i + 2 * T), d = ld(i + 3 * T);
+        acc ^= a[0] ^ a[1] ^ a[2] ^ a[3] ^ b[0] ^ b[1] ^ b[2] ^ b[3];
+        acc ^= e[0] ^ e[1] ^ e[2] ^ e[3] ^ d[0] ^ d[1] ^ d[2] ^ d[3];
     }
     if (acc == 0x9e3779b9u) sink[0] = acc;  // practically never; keeps the loads alive
 }
@@ -49,14 +58,40 @@ extern "C" logismos_status_t logismos_launch_probe_copy(const void* src, void* d
     return hipGetLastError();
 }
 
-extern "C" logismos_status_t logismos_launch_probe_read(const void* src, void* sink_u32,
-                                                        size_t bytes, logismos_stream_t stream) {
-    if (!src || !sink_u32 || bytes == 0 || (bytes & 15u)) return hipErrorInvalidValue;
+static logismos_status_t probe_read(const void* src, void* sink_u32, size_t bytes, int flags,
+                                    logismos_stream_t stream) {
+    if (!src || !sink_u32 || bytes == 0 || (bytes & 15u) || (flags & ~3)) return hipErrorInvalidValue;
     if (reinterpret_cast<uintptr_t>(src) & 15u) return hipErrorInvalidValue;
     const int64_t n16 = (int64_t)(bytes >> 4);
-    int64_t blocks = (n16 + 1023) / 1024;
-    if (blocks > 256 * 8) blocks = 256 * 8;
-    lg::probe_read_kernel<<<dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
-        static_cast<const lg::uint4_t*>(src), static_cast<unsigned*>(sink_u32), n16);
+    const lg::uint4_t* s = static_cast<const lg::uint4_t*>(src);
+    unsigned* sink = static_cast<unsigned*>(sink_u32);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (flags & LOGISMOS_PROBE_STRIDED) {
+        // one resident workgroup of 512 threads per CU's worth of the chip
+        const dim3 grid(256), block(512);
+        if (flags & LOGISMOS_PROBE_NON_TEMPORAL)
+            lg::probe_read_kernel<true, true><<<grid, block, 0, st>>>(s, sink, n16);
+        else
+            lg::probe_read_kernel<false, true><<<grid, block, 0, st>>>(s, sink, n16);
+    } else {
+        int64_t blocks = (n16 + 1023) / 1024;
+        if (blocks > 256 * 8) blocks = 256 * 8;
+        const dim3 grid((unsigned)blocks), block(256);
+        if (flags & LOGISMOS_PROBE_NON_TEMPORAL)
+            lg::probe_read_kernel<true, false><<<grid, block, 0, st>>>(s, sink, n16);
+        else
+            lg::probe_read_kernel<false, false><<<grid, block, 0, st>>>(s, sink, n16);
+    }
     return hipGetLastError();
+}
+
+extern "C" logismos_status_t logismos_launch_probe_read(const void* src, void* sink_u32,
+                                                        size_t bytes, logismos_stream_t stream) {
+    return probe_read(src, sink_u32, bytes, 0, stream);
+}
+
+extern "C" logismos_status_t logismos_launch_probe_read_ex(const void* src, void* sink_u32,
+                                                           size_t bytes, int flags,
+                                                           logismos_stream_t stream) {
+    return probe_read(src, sink_u32, bytes, flags, stream);
 }

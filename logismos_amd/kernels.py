@@ -136,6 +136,7 @@ _SIGNATURES = {
     "logismos_launch_kv_gather_turbo3_f32": (C.c_uint32, [_vp] * 5 + [_i] * 4 + [_vp]),
     "logismos_launch_probe_copy": (C.c_uint32, [_vp, _vp, _sz, _vp]),
     "logismos_launch_probe_read": (C.c_uint32, [_vp, _vp, _sz, _vp]),
+    "logismos_launch_probe_read_ex": (C.c_uint32, [_vp, _vp, _sz, _i, _vp]),
 }
 
 ATTN_PHASE_DECODE, ATTN_PHASE_PREFILL, ATTN_PHASE_MERGE, ATTN_PHASE_ALL = 1, 2, 4, 7
@@ -369,9 +370,12 @@ def launch_probe_copy(src, dst, nbytes: int, stream=None) -> None:
                                                                _raw(stream)))
 
 
-def launch_probe_read(src, sink, nbytes: int, stream=None) -> None:
-    _status("probe_read", library().logismos_launch_probe_read(_ptr(src), _ptr(sink), nbytes,
-                                                               _raw(stream)))
+PROBE_NON_TEMPORAL, PROBE_STRIDED = 1, 2
+
+
+def launch_probe_read(src, sink, nbytes: int, stream=None, flags: int = 0) -> None:
+    _status("probe_read", library().logismos_launch_probe_read_ex(_ptr(src), _ptr(sink), nbytes,
+                                                                  flags, _raw(stream)))
 
 
 def launch_pack_ragged(new_tokens, prior_ctx, block_tables, cu_seqlens, slot_mapping, context_lens,
