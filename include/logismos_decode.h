@@ -352,9 +352,16 @@ logismos_status_t logismos_launch_paged_attn_varlen_fp16_phases(
  * that device's array: launches that can overlap in time (two streams, two
  * threads) race on it and must be ordered by the caller.  The array needs no
  * clearing between calls (its contents never matter on entry).  Results are
- * identical to `logismos_launch_paged_attn_varlen_fp16` with the same arguments. */
+ * identical to `logismos_launch_paged_attn_varlen_fp16` with the same arguments.
+ * `logismos_paged_attn_noalloc_init()`: call it once per device at set-up, with that
+ * device current and outside any region that must not allocate: it resolves the
+ * array's device address (the look-up makes the runtime load the library's code
+ * object and place the array) and the device's CU count.  Without it the first
+ * launch on a device does that work itself, and only the later ones allocate
+ * nothing. */
 #define LOGISMOS_PAGED_ATTN_STATIC_WORKSPACE_BYTES (16u << 20)
 size_t logismos_paged_attn_static_workspace_bytes(void);
+logismos_status_t logismos_paged_attn_noalloc_init(void);
 logismos_status_t logismos_launch_paged_attn_varlen_fp16_noalloc(
     const void* q_f16, const void* k_pool_f16, const void* v_pool_f16, const int32_t* block_tables,
     const int32_t* cu_seqlens_q, const int32_t* context_lens, void* out_f16, int num_seqs,

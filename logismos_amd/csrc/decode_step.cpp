@@ -146,11 +146,15 @@ bool config_ok(const logismos_decode_config_t* c, int num_seqs, int t, int max_s
         return (int64_t)t * widest <= lim && (int64_t)widest * c->hidden <= lim &&
                (int64_t)c->hidden * c->intermediate <= lim && c->hidden >= 128 && qd >= 128;
     }
-    if (logismos_qgemm_q4g128_splitk_xprep_parts(b, qd + 2 * kvd, c->hidden) <= 0 ||
-        logismos_qgemm_q4g128_splitk_xprep_parts(b, c->hidden, qd) <= 0 ||
-        logismos_qgemm_q4g128_splitk_xprep_parts(b, 2 * c->intermediate, c->hidden) <= 0 ||
-        logismos_qgemm_q4g128_splitk_xprep_parts(b, c->hidden, c->intermediate) <= 0)
-        return false;
+    // every projection must have a plan for a full chunk of rows and for the ragged last chunk
+    const int last = t - (t - 1) / kChunkRows * kChunkRows;
+    for (const int rows : {b, last}) {
+        if (logismos_qgemm_q4g128_splitk_xprep_parts(rows, qd + 2 * kvd, c->hidden) <= 0 ||
+            logismos_qgemm_q4g128_splitk_xprep_parts(rows, c->hidden, qd) <= 0 ||
+            logismos_qgemm_q4g128_splitk_xprep_parts(rows, 2 * c->intermediate, c->hidden) <= 0 ||
+            logismos_qgemm_q4g128_splitk_xprep_parts(rows, c->hidden, c->intermediate) <= 0)
+            return false;
+    }
     return true;
 }
 

@@ -1768,6 +1768,16 @@ static hipError_t static_workspace(void** out) {
 
 extern "C" size_t logismos_paged_attn_static_workspace_bytes(void) { return kStaticWorkspaceBytes; }
 
+// Everything the `_noalloc` launch would otherwise do on its first call on a device: the
+// symbol look-up (which makes the runtime load the code object and place the array) and the
+// CU count the launch heuristics read.  After it the launch entry point touches no allocator.
+extern "C" logismos_status_t logismos_paged_attn_noalloc_init(void) {
+    void* ws = nullptr;
+    const hipError_t e = static_workspace(&ws);
+    if (e != hipSuccess) return e;
+    return lg::device_cu_count() > 0 ? hipSuccess : hipErrorInvalidDevice;
+}
+
 extern "C" logismos_status_t logismos_launch_paged_attn_varlen_fp16_noalloc(
     const void* q_f16, const void* k_pool_f16, const void* v_pool_f16, const int32_t* block_tables,
     const int32_t* cu_seqlens_q, const int32_t* context_lens, void* out_f16, int num_seqs,

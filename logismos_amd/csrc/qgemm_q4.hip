@@ -441,16 +441,22 @@ extern "C" logismos_status_t logismos_check_qgemm_q4g128_shape(int b, int n, int
                           (long long)((int64_t)n * k));
     if ((int64_t)b * n > (int64_t)INT32_MAX || (int64_t)b * k > (int64_t)INT32_MAX)
         return lg::reject(msg, msg_cap, "%s: batch*N or batch*K exceeds i32::MAX", kn);
-    // (rows beyond 32 are taken 32 at a time: the per-launch bounds below use min(b, 32))
-    if (b <= 4 && (size_t)b * (k / 32) * 68 > lg::kMaxLds)
-        return lg::reject(msg, msg_cap, "%s: batch*K = %lld does not fit the LDS staging of x", kn,
-                          (long long)((int64_t)b * k));
-    // the matrix-core path (batch >= 3; ..._bf16_mfma refuses such a shape at any batch) stages a
-    // workgroup's scales and zeros for all of K next to its partial sums
-    if (b >= 3 && lg::mfma_lds_bytes(b < 32 ? b : 32, n, k) > lg::kMaxLds)
-        return lg::reject(msg, msg_cap,
-                          "%s: K = %d needs %zu bytes of LDS on the matrix-core path (limit %zu)",
-                          kn, k, lg::mfma_lds_bytes(b < 32 ? b : 32, n, k), lg::kMaxLds);
+    // rows beyond 32 are taken 32 at a time: the per-launch bounds hold for a full pass and for
+    // the ragged last pass (which may fall to another kernel family), so that no launch of a
+    // call is refused after an earlier one has written its rows
+    const int passes[2] = {b < 32 ? b : 32, b > 32 ? b % 32 : 0};
+    for (const int rows : passes) {
+        if (rows == 0) continue;
+        if (rows <= 4 && (size_t)rows * (k / 32) * 68 > lg::kMaxLds)
+            return lg::reject(msg, msg_cap,
+                              "%s: %d rows x K = %d do not fit the LDS staging of x", kn, rows, k);
+        // the matrix-core path (3 rows or more; ..._bf16_mfma refuses such a shape at any batch)
+        // stages a workgroup's scales and zeros for all of K next to its partial sums
+        if (rows >= 3 && lg::mfma_lds_bytes(rows, n, k) > lg::kMaxLds)
+            return lg::reject(msg, msg_cap,
+                              "%s: K = %d needs %zu bytes of LDS on the matrix-core path (limit %zu)",
+                              kn, k, lg::mfma_lds_bytes(rows, n, k), lg::kMaxLds);
+    }
     return 0;
 }
 

@@ -69,6 +69,7 @@ _SIGNATURES = {
     "logismos_launch_paged_attn_varlen_fp16_phases":
         (C.c_uint32, [_vp] * 8 + [_i] * 9 + [_f, _i, _i, _vp]),
     "logismos_paged_attn_static_workspace_bytes": (_sz, []),
+    "logismos_paged_attn_noalloc_init": (C.c_uint32, []),
     "logismos_launch_paged_attn_varlen_fp16_noalloc":
         (C.c_uint32, [_vp] * 7 + [_i] * 9 + [_f, _i, _vp]),
     "logismos_launch_paged_attn_decode_fp16_xprep":
@@ -326,6 +327,11 @@ def launch_paged_attn_varlen_fp16(q, k_pool, v_pool, block_tables, cu_seqlens_q,
         code = library().logismos_launch_paged_attn_varlen_fp16_phases(*args, int(phases),
                                                                        _raw(stream))
     _status("paged_attn_varlen_fp16", code)
+
+
+def paged_attn_noalloc_init() -> None:
+    """Set-up of the entry point that allocates nothing, for the current device."""
+    _status("paged_attn_noalloc_init", library().logismos_paged_attn_noalloc_init())
 
 
 def launch_paged_attn_varlen_fp16_noalloc(q, k_pool, v_pool, block_tables, cu_seqlens_q,

@@ -108,6 +108,9 @@ def test_num_splits_and_workspace_are_pure_functions():
     (1, 8, 64, "multiple of the group size 128"), (1, 1 << 20, 1 << 12, "exceeds i32::MAX"),
     # scales and zeros of all of K next to the partial sums exceed 160 KiB on the MFMA path
     (32, 12288, 45056, "bytes of LDS"),
+    # a 33rd row is a second pass of one row on the GEMV path, whose x staging K = 77824 exceeds:
+    # refused as a whole, not after the first 32 rows were written
+    (33, 16, 77824, "do not fit the LDS staging"),
 ])
 def test_qgemm_q4_shape_guard(b, n, k, frag):
     with pytest.raises(kernels.UnsupportedShape) as e:
@@ -115,6 +118,8 @@ def test_qgemm_q4_shape_guard(b, n, k, frag):
     assert frag in str(e.value)
     kernels.check_qgemm_q4g128_shape(1, 12288, 4096)
     kernels.check_qgemm_q4g128_shape(8240, 4096, 4096)  # any m, as linear_t; 32 rows per pass
+    kernels.check_qgemm_q4g128_shape(32, 16, 77824)     # one full pass on the matrix cores
+    kernels.check_qgemm_q4g128_shape(37, 16, 77824)     # ... and a last pass of five rows
     # the split-K forms hold the whole batch in one launch: at most 32 rows
     assert kernels.qgemm_q4g128_splitk_parts(33, 4096, 4096) == 0
     assert kernels.qgemm_q4g128_splitk_parts(33, 4096, 4096, prepared=True) == 0

@@ -194,6 +194,39 @@ def test_mixed_batch_with_many_rows_on_the_tiled_gemm():
     _check_step(cfg, layers, batch, "mixed batch, tiled GEMM", 2)
 
 
+def test_many_rows_at_head_dim_64_with_a_projection_width_off_the_tile():
+    # the tiled-GEMM path (97 rows or more) at another head width: 8 query / 1 KV head of 64,
+    # so the q/k/v projection is 640 columns wide -- five 128-column tiles of which the last
+    # is half empty -- and the attention runs on the general kernel with a GQA group of 8
+    rng = np.random.default_rng(43)
+    cfg, layers, batch = workloads.decode_step_problem(
+        rng, num_layers=2, hidden=512, hq=8, hkv=1, inter=1024, ctx=[700, 140, 3, 33, 37],
+        new_tokens=[1, 100, 3, 1, 37], d=64, qkv_bias=True)
+    assert batch["h"].shape[0] == 142 and (8 + 2) * 64 % 128 != 0
+    _check_step(cfg, layers, batch, "142 rows, head_dim 64, width 640", 2)
+
+
+def test_many_rows_over_turbo3_pools():
+    # the same path over TurboQuant 3-bit pools: the chunk's new rows are rotated, rounded and
+    # encoded by one launch over all 142 rows, the prefill kernel decodes inside its gather
+    rng = np.random.default_rng(44)
+    cfg, layers, batch = workloads.decode_step_problem(
+        rng, num_layers=2, hidden=1024, hq=8, hkv=2, inter=2048, ctx=[700, 140, 3, 33, 37],
+        new_tokens=[1, 100, 3, 1, 37], kv_turbo3=True)
+    assert batch["h"].shape[0] == 142
+    r, got, want, lay, bat = _run_both(cfg, layers, batch)
+    assert _rel_l2(got, want) < 1e-2
+    assert np.all(np.abs(got - want) <= 5e-2 + 3e-2 * np.abs(want))
+    # rows of the pools the step did not write are untouched (integer work, bit-exact)
+    slots = np.asarray(batch["slots"])
+    for (kp, vp), L0 in zip(r.pools, layers):
+        gk = kp.to_numpy(np.uint8, L0["k_pool"].shape)
+        gv = vp.to_numpy(np.uint8, L0["v_pool"].shape)
+        rest = np.setdiff1d(np.arange(gk.shape[0]), slots)
+        assert np.array_equal(gk[rest], L0["k_pool"][rest])
+        assert np.array_equal(gv[rest], L0["v_pool"][rest])
+
+
 def test_more_than_32_decode_sequences():
     rng = np.random.default_rng(39)
     ctx = rng.integers(1, 300, size=45)
