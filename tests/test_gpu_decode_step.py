@@ -194,16 +194,16 @@ def test_mixed_batch_with_many_rows_on_the_tiled_gemm():
     _check_step(cfg, layers, batch, "mixed batch, tiled GEMM", 2)
 
 
-def test_many_rows_at_head_dim_64_with_a_projection_width_off_the_tile():
-    # the tiled-GEMM path (97 rows or more) at another head width: 8 query / 1 KV head of 64,
-    # so the q/k/v projection is 640 columns wide -- five 128-column tiles of which the last
-    # is half empty -- and the attention runs on the general kernel with a GQA group of 8
+def test_many_rows_at_head_dim_96_with_a_projection_width_off_the_tile():
+    # the tiled-GEMM path (97 rows or more) at another head width: 4 query / 1 KV head of 96,
+    # so the q/k/v projection is 576 columns wide -- four and a half 128-column tiles, the
+    # last one half empty -- and the attention runs on the general kernel
     rng = np.random.default_rng(43)
     cfg, layers, batch = workloads.decode_step_problem(
-        rng, num_layers=2, hidden=512, hq=8, hkv=1, inter=1024, ctx=[700, 140, 3, 33, 37],
-        new_tokens=[1, 100, 3, 1, 37], d=64, qkv_bias=True)
-    assert batch["h"].shape[0] == 142 and (8 + 2) * 64 % 128 != 0
-    _check_step(cfg, layers, batch, "142 rows, head_dim 64, width 640", 2)
+        rng, num_layers=2, hidden=512, hq=4, hkv=1, inter=1024, ctx=[700, 140, 3, 33, 37],
+        new_tokens=[1, 100, 3, 1, 37], d=96, qkv_bias=True)
+    assert batch["h"].shape[0] == 142 and ((4 + 2) * 96) % 128 != 0
+    _check_step(cfg, layers, batch, "142 rows, head_dim 96, width 576", 2)
 
 
 def test_many_rows_over_turbo3_pools():
