@@ -884,6 +884,147 @@ def bench_head_dim64(args):
     }
 
 
+def bench_two_streams(args):
+    """Config 5's step as two half-batches of 16 sequences on two equal-priority streams,
+    against the one batch of 32 on one stream that the headline times; and, per layer, the
+    decode attention of one half on stream A while the other half's chain of projections and
+    small operators runs on stream B (fork / join inside one captured graph), against each of
+    them alone.  The attention's workers are capped through num_splits (16 x (splits - 1)) to
+    leave CUs to the chain.  Weights and pools are shared by the halves."""
+    import oracle as O
+    from tests.gpu_harness import DecodeStepRunner
+    rng = np.random.default_rng(workloads.SEED + 5)
+    S, L, hidden, hq, hkv, inter, bs = 32, 36, 4096, 32, 8, 12288, 16
+    H = S // 2
+    ctx = rng.integers(256, 8193, size=S).astype(np.int64)
+    max_ctx = 8194
+    cfg, layers, batch = workloads.decode_step_problem(
+        rng, num_layers=1, hidden=hidden, hq=hq, hkv=hkv, inter=inter, ctx=np.full(S, max_ctx),
+        max_pos=max_ctx + 1, random_nibbles=True)
+    max_blocks = batch["block_tables"].shape[1]
+    sa, sb = hip.Stream(), hip.Stream()
+    prior = (ctx - 1).astype(np.int32)
+    cu, slots, ctx_l, _ = O.pack_ragged(np.ones(S, np.int32), prior, batch["block_tables"], bs)
+    b0 = dict(batch, h=batch["h"].copy())
+    b0.update(cu_seqlens=cu, slots=slots, context_lens=ctx_l, positions=prior)
+    r = DecodeStepRunner(cfg, layers * L, b0, stream=sa, share_layer_data=True)
+    ev_f, ev_j = hip.Event(), hip.Event()
+
+    def timed(build, n=10, w=3):
+        g = hip.Graph(sa)
+        with g:
+            build()
+        for _ in range(w):
+            g.launch()
+        sa.synchronize()
+        e0, e1 = hip.Event(), hip.Event()
+        e0.record(sa)
+        for _ in range(n):
+            g.launch()
+        e1.record(sa)
+        e1.synchronize()
+        return e0.elapsed_ms(e1) / n
+
+    def forked(on_a, on_b):
+        ev_f.record(sa)
+        sb.wait_event(ev_f)
+        on_a()
+        on_b()
+        ev_j.record(sb)
+        sa.wait_event(ev_j)
+
+    # ---- whole steps
+    d_cu16 = hip.DeviceBuffer.from_numpy(np.arange(H + 1, dtype=np.int32))
+
+    def half(lo, ns):
+        b = kernels.DecodeBatch()
+        C.memmove(C.byref(b), C.byref(r.batch), C.sizeof(b))
+        b.hidden_f32 = r.h.ptr.value + lo * hidden * 4
+        b.out_bf16 = r.out.ptr.value + lo * hidden * 2
+        b.block_tables = r.idx["block_tables"].ptr.value + lo * max_blocks * 4
+        b.cu_seqlens = d_cu16.ptr.value
+        b.context_lens = r.idx["context_lens"].ptr.value + lo * 4
+        b.positions = r.idx["positions"].ptr.value + lo * 4
+        b.slot_mapping = r.slots.ptr.value + lo * 8
+        b.num_seqs, b.num_splits = H, ns
+        return b, hip.DeviceBuffer(kernels.decode_step_workspace_bytes(r.cfg, H, ns))
+
+    ms32 = timed(r.launch)
+    steps = []
+    for ns in (17, 9):
+        (ba, wa), (bb, wb) = half(0, ns), half(H, ns)
+        step_a = lambda: kernels.launch_decode_step(r.cfg, r.layers, ba, wa, sa)  # noqa: E731
+        step_b_on_a = lambda: kernels.launch_decode_step(r.cfg, r.layers, bb, wb, sa)  # noqa: E731
+        step_b = lambda: kernels.launch_decode_step(r.cfg, r.layers, bb, wb, sb)  # noqa: E731
+        steps.append({"attention_workers": min(256, H * (ns - 1)),
+                      "half_alone_ms": round(timed(step_a), 4),
+                      "halves_one_after_the_other_ms": round(timed(lambda: (step_a(), step_b_on_a())), 4),
+                      "halves_on_two_streams_ms": round(timed(lambda: forked(step_a, step_b)), 4)})
+
+    # ---- per layer: attention of half A beside the chain of half B
+    qd, kvd = hq * 128, hkv * 128
+    width = qd + 2 * kvd
+    d_cu = hip.DeviceBuffer.from_numpy(np.arange(S + 1, dtype=np.int32))
+    d_q = hip.DeviceBuffer(S * qd * 2)
+    d_q.fill(0x3C)
+    xb = lambda k: hip.DeviceBuffer(kernels.q4_xprep_bytes(H, k))  # noqa: E731
+    d_attn_b, d_xn, d_act, d_attn_a = xb(qd), xb(hidden), xb(inter), xb(qd)
+    for d in (d_attn_b, d_xn, d_act):
+        d.fill(0x3C)
+    jp = lambda n, k: kernels.qgemm_q4g128_splitk_parts(H, n, k, prepared=True)  # noqa: E731
+    j_o, j_gu, j_dn, j_qkv = jp(hidden, qd), jp(2 * inter, hidden), jp(hidden, inter), jp(width, hidden)
+    d_proj = hip.DeviceBuffer(max(j_o, j_dn) * H * hidden * 4)
+    d_gu = hip.DeviceBuffer(j_gu * H * 2 * inter * 4)
+    d_qkv = hip.DeviceBuffer(j_qkv * H * width * 4)
+    d_h = hip.DeviceBuffer(H * hidden * 4)
+    d_h.fill(0)
+    d_q2 = hip.DeviceBuffer(H * qd * 2)
+    scale = 1.0 / np.sqrt(128.0)
+
+    def chain(l, stream):
+        lay = r.layers[l]
+        gemm = lambda x, w, parts, n, k: kernels.launch_qgemm_q4g128_f32_splitk(  # noqa: E731
+            x, w.qw, w.scale, w.zero, parts, H, n, k, stream, prepared=True)
+        gemm(d_attn_b, lay.o, d_proj, hidden, qd)
+        kernels.launch_add_rms_norm_f32p_xprep(d_h, d_proj, j_o, lay.norm2_w_f32, d_xn, H, hidden,
+                                               1e-6, stream)
+        gemm(d_xn, lay.gate_up, d_gu, 2 * inter, hidden)
+        kernels.launch_silu_mul_f32p_xprep(d_gu, j_gu, d_act, H, inter, stream)
+        gemm(d_act, lay.down, d_proj, hidden, inter)
+        kernels.launch_add_rms_norm_f32p_xprep(d_h, d_proj, j_dn, lay.norm1_w_f32, d_xn, H, hidden,
+                                               1e-6, stream)
+        gemm(d_xn, lay.qkv, d_qkv, width, hidden)
+        kernels.launch_rope_kv_write_f32p(
+            d_qkv, j_qkv, r.idx["positions"].ptr.value + H * 4, r.cos, r.sin,
+            r.slots.ptr.value + H * 8, d_q2, lay.k_pool_f16, lay.v_pool_f16, H, hq, hkv, 128,
+            r.cfg.max_pos, stream)
+
+    us_chain = timed(lambda: [chain(l, sa) for l in range(L)]) * 1e3 / L
+    layers_out = []
+    for ns in (17, 13, 9):
+        ws = hip.DeviceBuffer(kernels.paged_attn_workspace_bytes(H, hq, 128, ns))
+
+        def attn(l, stream):
+            lay = r.layers[l]
+            kernels.launch_paged_attn_decode_fp16_xprep(
+                d_q, lay.k_pool_f16, lay.v_pool_f16, r.idx["block_tables"], d_cu,
+                r.idx["context_lens"], d_attn_a, ws, H, hq, hkv, 128, bs, max_blocks, ns, scale,
+                stream)
+        us_attn = timed(lambda: [attn(l, sa) for l in range(L)]) * 1e3 / L
+        us_both = timed(lambda: [forked(lambda l=l: attn(l, sa), lambda l=l: chain(l, sb))
+                                 for l in range(L)]) * 1e3 / L
+        layers_out.append({"attention_workers": min(256, H * (ns - 1)),
+                           "attention_us": round(us_attn, 1), "chain_us": round(us_chain, 1),
+                           "both_us": round(us_both, 1),
+                           "both_over_sum": round(us_both / (us_attn + us_chain), 3),
+                           "both_over_max": round(us_both / max(us_attn, us_chain), 3)})
+    return {"workload": "config 5 as two half-batches of 16 sequences on two equal-priority "
+                        "streams (36 layers, same weights and pools as the headline step)",
+            "one_batch_of_32_on_one_stream_ms": round(ms32, 4), "whole_steps": steps,
+            "per_layer_attention_of_one_half_beside_the_chain_of_the_other": layers_out,
+            "sum_ctx_half_a": int(ctx[:H].sum()), "sum_ctx_half_b": int(ctx[H:].sum())}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -901,7 +1042,7 @@ def main():
                          "profiler leave them out (--skip-kernels without --extras)")
     ap.add_argument("--workload", default="all",
                     choices=["all", "step", "config1", "config2", "config3", "config4",
-                             "config4_gemm", "turbo3", "headdim64"],
+                             "config4_gemm", "turbo3", "headdim64", "two_streams"],
                     help="all: the decode-step line with every leg inside it (default); "
                          "otherwise only that workload's own JSON line")
     args = ap.parse_args()
@@ -915,12 +1056,13 @@ def main():
     args.steps_c5 = args.steps if args.steps is not None else 20
     args.warmup_c5 = args.warmup if args.warmup is not None else 3
     if args.workload in ("config1", "config2", "config3", "config4", "config4_gemm", "turbo3",
-                         "headdim64"):
+                         "headdim64", "two_streams"):
         args.steps = args.steps if args.steps is not None else 200
         args.warmup = args.warmup if args.warmup is not None else 20
         leg = {"config1": bench_qgemv_q8, "config2": bench_paged_decode, "config3": bench_q4,
                "config4": bench_mixed_config4, "config4_gemm": bench_q4_tall,
-               "turbo3": bench_turbo3, "headdim64": bench_head_dim64}[args.workload]
+               "turbo3": bench_turbo3, "headdim64": bench_head_dim64,
+               "two_streams": bench_two_streams}[args.workload]
         print(json.dumps(leg(args)))
         return
     line = bench_decode_step(args)

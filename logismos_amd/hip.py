@@ -101,6 +101,10 @@ class Stream:
     def synchronize(self) -> None:
         check(_runtime().hipStreamSynchronize(self._h), "hipStreamSynchronize")
 
+    def wait_event(self, event: "Event") -> None:
+        """Work enqueued on this stream from now on starts after `event` (as recorded so far)."""
+        check(_runtime().hipStreamWaitEvent(self._h, event._h, C.c_uint(0)), "hipStreamWaitEvent")
+
     def __del__(self):
         try:
             if self._h:
