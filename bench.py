@@ -487,7 +487,7 @@ def bench_q4_tall(args):
     b = 8240
     shapes = [("qkv", 6144, 4096), ("o", 4096, 4096), ("gate_up", 24576, 4096),
               ("down", 4096, 12288)]
-    out, flops_all, ms_all = {}, 0.0, 0.0
+    out, flops_all, ms_all, ms_noworkspace = {}, 0.0, 0.0, 0.0
     parity = None
     for name, n, k in shapes:
         qw = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
@@ -496,8 +496,15 @@ def bench_q4_tall(args):
         xb = O.f32_to_bf16_bits(rng.standard_normal((b, k), np.float32))
         d = [hip.DeviceBuffer.from_numpy(a) for a in (xb, qw, s.view(np.uint16), z.view(np.uint16))]
         dy = hip.DeviceBuffer(b * n * 2)
-        fn = lambda: kernels.launch_qgemm_q4g128_bf16(d[0], d[1], d[2], d[3], dy, b, n, k, stream)  # noqa: E731
+        ws = hip.DeviceBuffer(kernels.qgemm_q4g128_tall_workspace_bytes(b, k))
+        # the entry point with a workspace (first pass over x + the tiled kernel) ...
+        fn = lambda: kernels.launch_qgemm_q4g128_tall(d[0], d[1], d[2], d[3], dy, ws, b, n, k,  # noqa: E731
+                                                      stream)
+        # ... and the same product through the entry point without one
+        fn0 = lambda: kernels.launch_qgemm_q4g128_bf16(d[0], d[1], d[2], d[3], dy, b, n, k, stream)  # noqa: E731
+        ms0, _, _ = time_launches(stream, [fn0], 10, 2)
         ms, _, _ = time_launches(stream, [fn], 10, 2)
+        ms_noworkspace += ms0
         if name == "o":
             # parity of what is being timed: a sample of rows against the oracle
             rows = np.r_[0:4, 4111:4115, 8236:8240]
@@ -509,11 +516,13 @@ def bench_q4_tall(args):
         ms_all += ms
         out[name] = {"n": n, "k": k, "us": round(ms * 1e3, 1),
                      "TFLOPs": round(flops / ms / 1e9, 1)}
-        del d, dy
+        del d, dy, ws
     return {"workload": "config 4's 8240 packed rows through one layer's Q4G128 projections "
                         "(qkv 6144x4096, o 4096x4096, gate_up 24576x4096, down 4096x12288)",
-            "kernel": "qgemm_q4g128_tall_kernel (128x128 tiles, v_mfma_f32_32x32x16_bf16)",
+            "kernel": "q4_tall_prepare_kernel + qgemm_q4g128_tallp_kernel (128x128 tiles, x "
+                      "straight into LDS, v_mfma_f32_32x32x16_bf16)",
             "projections": out, "ms_per_layer": round(ms_all, 4),
+            "ms_per_layer_entry_point_without_workspace": round(ms_noworkspace, 4),
             "roofline": {"bound": "mfma", "achieved": round(flops_all / ms_all / 1e9, 1),
                          "peak": 2500.0, "unit": "TFLOP/s",
                          "frac": round(flops_all / ms_all / 1e9 / 2500.0, 4), "traffic": None,

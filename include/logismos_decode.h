@@ -180,6 +180,25 @@ logismos_status_t logismos_launch_qgemm_q4g128_bf16_mfma(const void* x_bf16, con
                                                          const void* zero_f16, void* y_bf16, int b,
                                                          int n, int k, logismos_stream_t stream);
 
+/* `linear_t` over many rows of x (the prefill chunks of a mixed batch: hundreds to thousands
+ * of rows, crates/transformers/src/mlp.rs:104-111) with a workspace: a first pass copies x
+ * into the element order the kernel's nibble unpack produces and takes every row's sum over
+ * each group of 128 columns, the tiled matrix-core kernel then moves that copy straight into
+ * LDS and takes the zero-point term as a small product of its own.  Any m >= 1 (built for
+ * m >= ~100), K a multiple of 256, y bf16 `[m][N]` or, with y_is_f32, fp32 (what the step
+ * executor keeps between operators); bias fp32 `[N]` or NULL.  The workspace
+ * (`..._workspace_bytes(m, k)`, 16-byte aligned, caller-owned) is scratch: nothing in it
+ * matters before or after the call.  The entry points above serve the same product without
+ * a workspace (slower from about a hundred rows on). */
+logismos_status_t logismos_check_qgemm_q4g128_tall_shape(int m, int n, int k, char* msg,
+                                                         size_t msg_cap);
+size_t logismos_qgemm_q4g128_tall_workspace_bytes(int m, int k);
+logismos_status_t logismos_launch_qgemm_q4g128_tall(const void* x_bf16, const void* qw_u8,
+                                                    const void* scale_f16, const void* zero_f16,
+                                                    const void* bias_f32, void* y, int y_is_f32,
+                                                    void* workspace, int m, int n, int k,
+                                                    logismos_stream_t stream);
+
 /* Split-K form for a decode batch (b <= 32): fp32 partial products
  *   parts[j][b][n] = sum over K part j of x[b][k] * w[n][k],  j < J,
  * whose sum over j is the product.  Workgroups are tall (up to 256 weight rows

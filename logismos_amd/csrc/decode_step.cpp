@@ -35,6 +35,7 @@ struct Workspace {
     char* t_proj;  // f32  [T][hidden]
     char* t_gu;    // f32  [T][2*inter]
     char* t_act;   // bf16 [T][inter]
+    char* t_gemm;  // workspace of the tiled GEMM (its copy of x in unpack order + group sums)
     bool tall;
     size_t xn_stride;
     int chunks, rows;  // rows: rows of a full chunk (= T when there is one chunk)
@@ -66,6 +67,9 @@ Workspace carve(const logismos_decode_config_t& c, int num_seqs, int t, int num_
         w.t_proj = take((size_t)t * c.hidden * 4);
         w.t_gu = take((size_t)t * 2 * c.intermediate * 4);
         w.t_act = take((size_t)t * c.intermediate * 2);
+        const int kmax = c.intermediate > (int)qd ? (c.intermediate > c.hidden ? c.intermediate : c.hidden)
+                                                  : ((int)qd > c.hidden ? (int)qd : c.hidden);
+        w.t_gemm = take(logismos_qgemm_q4g128_tall_workspace_bytes(t, kmax));
         w.total = off;
         return w;
     }
@@ -231,6 +235,11 @@ extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_c
         hipStream_t st = static_cast<hipStream_t>(stream);
         auto gemm = [&](const void* x_bf16, const logismos_q4_weight_t& W, const void* bias,
                         void* y_f32, int n, int k) -> logismos_status_t {
+            // K in pairs of groups: the kernel that takes x through a first pass into the
+            // workspace; otherwise the one that stages x itself
+            if (logismos_check_qgemm_q4g128_tall_shape(t, n, k, nullptr, 0) == 0)
+                return logismos_launch_qgemm_q4g128_tall(x_bf16, W.qw, W.scale, W.zero, bias, y_f32,
+                                                         1, w.t_gemm, t, n, k, stream);
             return lg::qgemm_q4_tall_f32_launch(x_bf16, W.qw, W.scale, W.zero,
                                                 static_cast<const float*>(bias), y_f32, t, n, k, st);
         };

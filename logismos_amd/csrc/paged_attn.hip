@@ -1,9 +1,11 @@
 // Ragged paged attention for gfx950 (head_dim 128, fp16 KV, fp32 softmax).
 //
-// One wave64 owns one (query token, KV head, KV partition) and serves the
-// whole GQA group of that KV head, so every K/V byte is fetched from HBM once
-// per group.  Work inside the wave, per tile of 16 keys (a tile never
-// straddles a KV block because block_size % 16 == 0):
+// Decode rows: one wave64 owns one (sequence, KV head, piece of the context) and serves the
+// whole GQA group of that KV head, so every K/V byte is fetched from HBM once per group; the
+// pieces are equal shares of all sequences' key tiles (balanced launch, one workgroup per
+// CU) or fixed partitions (small batches).  Rows of a chunk (more than one new token) go
+// to the MFMA prefill kernel further down.  Work inside a decode wave, per tile of 16 keys
+// (a tile never straddles a KV block because block_size % 16 == 0):
 //
 //   * K: the A operand of v_mfma_f32_16x16x32_f16 wants lane (tg = lane/16, c = lane%16)
 //     to hold key c of the tile, 8 consecutive contraction elements per slot.  fp16 pools:
@@ -17,14 +19,19 @@
 //     head c for keys 4*tg..4*tg+3.
 //   * V: lane (tg, c) loads the 16-byte piece c of keys 4*tg..4*tg+3: each
 //     wave instruction covers four whole 256-byte rows.
-//   * The 16 lanes of a row (fixed tg) therefore hold both the scores and the
-//     values of the same four keys per tile: each row runs its own online
-//     softmax (running max / sum in the lanes c < G) with no traffic between
-//     rows; probabilities reach the value lanes through DPP row broadcasts and
-//     are applied with mixed-precision FMAs (fp16 value, fp32 accumulator).
-//   * The four rows are merged once at the end (log-sum-exp merge over
-//     ds_bpermute), then either normalised and written as fp16 (single
-//     partition) or written as an fp32 partial (m, l, acc) that the merge
+//   * Softmax: the scaled scores of a tile give one running maximum PER HEAD for all 16
+//     keys (the four lane rows exchange their maxima with two cross-row moves), so the
+//     accumulators of a head are rescaled by one factor per tile; only the running sums stay
+//     per lane row and are added up once in the epilogue.
+//   * P.V on the matrix cores as well: v_mfma_f32_16x16x16_f16 with A = the probabilities of
+//     the lane row's four keys (row = head) as TWO fp16 terms, the rounded value and the
+//     remainder, in two MFMAs on the same B (one term alone costs three decimal digits), and
+//     B = element e of the eight values the lane holds of each of its four keys, picked with
+//     one v_perm_b32 per two keys; eight (e) x two MFMAs per tile, fp32 accumulation.  The
+//     MFMA sums over all 16 keys of the tile, so there are no per-row partial outputs.
+//   * Epilogue: the accumulators are already the whole partition's; they are normalised
+//     and written as fp16 / bf16 / the prepared layout of the o projection (a sequence
+//     handled in one piece), or written as an fp32 partial (m, l, acc) that the merge
 //     kernel combines across partitions.
 //
 // Tiles are double-buffered in registers: the loads of tile i+1 are in flight

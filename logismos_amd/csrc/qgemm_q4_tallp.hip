@@ -1,0 +1,414 @@
+// Q4G128 GEMM for a tall x over a workspace: the tiled kernel of qgemm_q4_tall.hip with the
+// work that does not belong in its inner loop taken out of it.
+//   y[m][n] = sum_k x[m][k] * (q[n][k] - zero[n][k/128]) * scale[n][k/128] (+ bias[n])
+// `cpu_f32::linear_t` (crates/kernels/src/cpu_f32/mod.rs:271-345) at m = hundreds to thousands
+// of rows over the dequantised matrix.
+//
+// Counters of the workspace-less kernel show its vector pipe, not its matrix pipe, setting the
+// pace: per 32 MFMAs a wave issues ~500 vector instructions -- the nibble unpack (112), the
+// staging of x through registers into LDS with the pair-order permute and the group sums
+// (~130), and two multiply-adds per result and group for scale and zero point (128).  Here:
+//
+// * a first pass (`q4_tall_prepare_kernel`, x read once, ~1 % of the product's time) writes x
+//   in the order the nibble unpack produces ("pair order": (x0,x4)(x1,x5)(x2,x6)(x3,x7) per
+//   16-byte chunk), rows padded with zeros to a multiple of 128, and every row's sum over each
+//   group of 128 columns;
+// * the product kernel moves a group's 128 x 128 slab of that copy from global memory
+//   STRAIGHT into LDS (global_load_lds, 16 bytes per lane, no registers, no vector
+//   instructions), double buffered, one barrier per group.  A request writes 1 KiB of
+//   consecutive LDS (four rows), so instead of padding rows the 16-byte chunks of a row are
+//   stored XOR-swizzled by the row index; a lane's eight read addresses per buffer are
+//   loop-invariant registers and the ds_read_b128 of the MFMA A operand stays conflict-free;
+// * the zero-point term -scale * (128 + zero) * sum_x is a rank-(K/128) product of its own:
+//   one v_mfma_f32_32x32x2_f32 per output tile and PAIR of groups, accumulating into the same
+//   registers, in place of a multiply-add per result and group;
+// * what is left per group and wave: the unpack (a lane of the v_mfma_f32_32x32x16_bf16 B
+//   operand is one weight row and one dword of nibbles, made bf16 `128 + q` with an and-or per
+//   pair, exact), one multiply-add per result for the group's scale, 32 MFMAs.
+//
+// LDS is only touched through inline assembly inside the loop: the compiler would order
+// every LDS access it can see behind all outstanding global_load_lds.
+#include "device_utils.hpp"
+#include "launch_common.hpp"
+#include "q4_common.hpp"
+
+#include <hip/hip_fp16.h>
+
+namespace lg {
+
+typedef __attribute__((address_space(3))) void* tp_lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* tp_glb_ptr_t;
+
+constexpr int kTpTileM = 128;             // rows of x per workgroup
+constexpr int kTpTileN = 256;             // weight rows per workgroup
+constexpr int kTpSlabBytes = 128 * 256;   // one group's slab of x: 128 rows x 128 bf16
+constexpr int kTpWBytes = 256 * 64;       // one group's tile of weights: 256 rows x 128 nibbles
+constexpr int kTpBufBytes = kTpSlabBytes + kTpWBytes;
+constexpr int kTpBufs = 3;                // groups in LDS: one in use, two on their way
+
+__host__ __device__ inline int tp_padded_rows(int m) { return (m + kTpTileM - 1) / kTpTileM * kTpTileM; }
+__host__ __device__ inline size_t tp_sums_offset(int m, int k) {
+    return ((size_t)tp_padded_rows(m) * k * 2 + 255) & ~(size_t)255;
+}
+
+// x [m][k] bf16 -> xp [m_pad][k] bf16 in pair order (rows >= m: zeros), xs [m_pad][k/128] fp32
+// sums of the bf16 values of each group.  One thread per 16-byte chunk; the 16 lanes of a row
+// of lanes hold one group of one row.
+__global__ __launch_bounds__(256) void q4_tall_prepare_kernel(const uint16_t* __restrict__ x,
+                                                             uint16_t* __restrict__ xp,
+                                                             float* __restrict__ xs, int m,
+                                                             int m_pad, int k) {
+    const int64_t chunks_per_row = k >> 3;
+    const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (id >= (int64_t)m_pad * chunks_per_row) return;  // (whole rows of 16 lanes: k % 128 == 0)
+    const int64_t row = id / chunks_per_row;
+    const int64_t c = id - row * chunks_per_row;
+    uint4_t v = {0u, 0u, 0u, 0u};
+    if (row < m) v = *reinterpret_cast<const uint4_t*>(x + row * k + c * 8);
+    const float gs = row16_sum(sum8_bf16(v));
+    *reinterpret_cast<uint4_t*>(xp + row * k + c * 8) = pair_order(v);
+    if ((threadIdx.x & 15) == 0) xs[row * (k >> 7) + (c >> 4)] = gs;
+}
+
+template <bool F32OUT>
+__global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
+    const uint16_t* __restrict__ xp, const float* __restrict__ xs, const uint8_t* __restrict__ qw,
+    const __half* __restrict__ scale, const __half* __restrict__ zero,
+    const float* __restrict__ bias, void* __restrict__ y_out, int m, int n, int k) {
+    extern __shared__ uint4_t tp_lds[];  // kTpBufs x {slab of x, tile of weights}
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 31;
+    const int h = lane >> 5;
+    const int row0 = blockIdx.y * kTpTileM;
+    const int col0 = blockIdx.x * kTpTileN;
+    const int wr = (wave >> 2) * 64;  // this wave's 64 x 64 part of the 128 x 256 tile
+    const int wc = (wave & 3) * 64;
+    const int groups = k >> 7;
+
+    unsigned magic;
+    asm volatile("v_mov_b32 %0, 0x43004300" : "=v"(magic));
+    const unsigned lds_base = (unsigned)(uintptr_t)(tp_lds_ptr_t)tp_lds;
+    char* const lds_c = reinterpret_cast<char*>(tp_lds);
+
+    // ---- requests of a group, straight into LDS (a request writes 1 KiB of consecutive LDS).
+    // x: request q of this wave covers rows 16 wave + 4 q .. + 3, lane -> row + lane / 16, LDS
+    // position lane % 16 of that row, which holds the row's chunk (position ^ row % 16).
+    // weights: request q covers rows 32 wave + 16 q .. + 15 of the tile, lane -> row + lane / 4,
+    // position lane % 4 of the row's 64 bytes, which holds piece (position ^ (row / 4) % 4).
+    // Byte offsets fit 32 bits (m_pad * K * 2 and N * K < 2^31 are checked on the host).
+    unsigned xoff[4], woff[2];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int row = 16 * wave + 4 * q + (lane >> 4);
+        const int c = (lane & 15) ^ (row & 15);
+        xoff[q] = ((unsigned)(row0 + row) * (unsigned)k + (unsigned)c * 8u) * 2u;
+    }
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        const int row = 32 * wave + 16 * q + (lane >> 2);
+        const int piece = (lane & 3) ^ ((row >> 2) & 3);
+        const int gn = min(col0 + row, n - 1);  // a row past n re-reads the last row
+        woff[q] = (unsigned)gn * (unsigned)(k >> 1) + (unsigned)piece * 16u;
+    }
+    auto request_group = [&](int g, int buf) {
+        char* dst = lds_c + buf * kTpBufBytes;
+        const char* xsrc = reinterpret_cast<const char*>(xp) + (size_t)g * 256;
+        const char* wsrc = reinterpret_cast<const char*>(qw) + (size_t)g * 64;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            __builtin_amdgcn_global_load_lds((tp_glb_ptr_t)(xsrc + xoff[q]),
+                                             (tp_lds_ptr_t)(dst + (wave * 4 + q) * 1024), 16, 0, 0);
+#pragma unroll
+        for (int q = 0; q < 2; ++q)
+            __builtin_amdgcn_global_load_lds(
+                (tp_glb_ptr_t)(wsrc + woff[q]),
+                (tp_lds_ptr_t)(dst + kTpSlabBytes + (wave * 2 + q) * 1024), 16, 0, 0);
+    };
+    constexpr int kReq = 6;  // requests per group and wave
+    // ---- A operand reads: lane (r, h) at step s8 wants chunk 8 h + s8 of row wr + 32 i + r,
+    // stored at position (8 h + s8) ^ (r % 16): a0 ^ (s8 << 4), the i-tile as an immediate
+    const unsigned a0 = lds_base + (unsigned)(wr + r) * 256u +
+                        (unsigned)(((8 * h) ^ (r & 8)) | (r & 7)) * 16u;
+    unsigned a_addr[8];
+#pragma unroll
+    for (int s8 = 0; s8 < 8; ++s8) a_addr[s8] = a0 ^ ((unsigned)s8 << 4);
+    // ---- B operand reads: lane (r, h) of n-tile j wants the pieces 2 h, 2 h + 1 of row
+    // wc + 32 j + r (dword s8 % 4 of piece 2 h + s8 / 4 feeds step s8); j as an immediate
+    unsigned b_addr[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+        b_addr[t] = lds_base + kTpSlabBytes + (unsigned)(wc + r) * 64u +
+                    (unsigned)((2 * h + t) ^ ((r >> 2) & 3)) * 16u;
+
+    // scales and zeros of a pair of groups g, g + 1 (g even) in one dword each, from global
+    // memory into registers (a lane's 16 results of a tile belong to one weight row)
+    unsigned soff[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+        soff[j] = (unsigned)min(col0 + wc + 32 * j + r, n - 1) * (unsigned)groups;
+    unsigned scur[2], zcur[2], snext[2], znext[2];
+    auto gload_sz = [&](int g, unsigned (&sv)[2], unsigned (&zv)[2]) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            __builtin_memcpy(&sv[j], scale + soff[j] + (unsigned)g, 4);
+            __builtin_memcpy(&zv[j], zero + soff[j] + (unsigned)g, 4);
+        }
+    };
+    // group sums of x for the zero-point product: lane (r, h) holds row wr + 32 i + r, group
+    // g + h of the pair
+    float xsum[2], xsum_next[2];
+    auto gload_xs = [&](int g, float (&v)[2]) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+            v[i] = xs[(size_t)(row0 + wr + 32 * i + r) * groups + g + h];
+    };
+
+    float16_t yacc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) yacc[i][j][e] = 0.0f;
+
+    gload_sz(0, scur, zcur);
+    gload_xs(0, xsum);
+    request_group(0, 0);
+    if (groups > 1) request_group(1, 1);
+
+    // One group of 128 columns out of buffer BUF (immediates in the LDS reads); PAR: the
+    // group's place in its pair.  A wave's requests complete in the order they were issued,
+    // so "at most the six youngest outstanding" means the group's own have landed while the
+    // next group's may still be on their way.
+    auto group = [&](auto buf_c, auto par_c, int g) {
+        constexpr int BUF = decltype(buf_c)::value;
+        constexpr int PAR = decltype(par_c)::value;
+        if (g + 1 < groups) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kReq) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // after the barrier everybody's requests for this group have landed, and everybody is
+        // done reading the buffer of the group before it, which the group after next reuses
+        __builtin_amdgcn_s_barrier();
+        if (g + 2 < groups) {
+            // (the small loads first: what waits for them need not wait for the requests)
+            if (PAR == 1) {
+                gload_sz(g + 1, snext, znext);
+                gload_xs(g + 1, xsum_next);
+            }
+            request_group(g + 2, (BUF + 2) % kTpBufs);
+        } else if (PAR == 1 && g + 1 < groups) {
+            gload_sz(g + 1, snext, znext);
+            gload_xs(g + 1, xsum_next);
+        }
+        float16_t acc[2][2];
+        bf16x8_t av[2][2];  // [step parity][i]
+        bf16x8_t bv[2][2];  // [step parity][j]
+        uint4_t wq[2][2];   // [j][half of the group]: the group's nibbles of this lane's rows
+        constexpr int kBufOff = BUF * kTpBufBytes;
+        // (the buffer's offset is added here, as a literal: LDS offsets of up to 144 KiB do not
+        // fit the 16-bit immediate of a read)
+        unsigned t0, t1;
+        asm volatile("v_add_u32 %4, %c8, %6\n\tv_add_u32 %5, %c8, %7\n\t"
+                     "ds_read_b128 %0, %4\n\tds_read_b128 %1, %5\n\t"
+                     "ds_read_b128 %2, %4 offset:2048\n\tds_read_b128 %3, %5 offset:2048"
+                     : "=&v"(wq[0][0]), "=&v"(wq[0][1]), "=&v"(wq[1][0]), "=&v"(wq[1][1]),
+                       "=&v"(t0), "=&v"(t1)
+                     : "v"(b_addr[0]), "v"(b_addr[1]), "n"(kBufOff)
+                     : "memory");
+        asm volatile("v_add_u32 %2, %c4, %3\n\t"
+                     "ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:8192"
+                     : "=&v"(av[0][0]), "=&v"(av[0][1]), "=&v"(t0)
+                     : "v"(a_addr[0]), "n"(kBufOff)
+                     : "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(wq[0][0]), "+v"(wq[0][1]), "+v"(wq[1][0]), "+v"(wq[1][1]),
+                       "+v"(av[0][0]), "+v"(av[0][1])::"memory");
+        auto unpack = [&](auto s8c, bf16x8_t (&b)[2]) {
+            constexpr int s8 = decltype(s8c)::value;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const unsigned wd = wq[j][s8 >> 2][s8 & 3];
+                uint4_t e4;
+#pragma unroll
+                for (int sft = 0; sft < 4; ++sft) e4[sft] = ((wd >> (4 * sft)) & kNibMask) | magic;
+                b[j] = __builtin_bit_cast(bf16x8_t, e4);
+            }
+        };
+        unpack(ic<0>{}, bv[0]);
+        // Step s8 issues the reads of step s8 + 1, then its four MFMAs with the unpack of step
+        // s8 + 1 between them (the matrix pipe takes 32 cycles per MFMA, eight issue slots of
+        // the vector pipe), and only then waits for the reads.  The order is pinned: left
+        // alone the scheduler sinks the MFMAs below the wait, which then sits right behind the
+        // reads it waits for.
+        static_for<8>([&](auto s8c) {
+            constexpr int s8 = decltype(s8c)::value;
+            constexpr int cur = s8 & 1;
+            if constexpr (s8 < 7) {
+                unsigned ta;
+                asm volatile("v_add_u32 %2, %c4, %3\n\t"
+                             "ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:8192"
+                             : "=&v"(av[cur ^ 1][0]), "=&v"(av[cur ^ 1][1]), "=&v"(ta)
+                             : "v"(a_addr[s8 < 7 ? s8 + 1 : 7]), "n"(kBufOff)
+                             : "memory");
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (s8 < 7) unpack(ic<(s8 < 7 ? s8 + 1 : 7)>{}, bv[cur ^ 1]);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    if constexpr (s8 == 0) {
+                        float16_t z16;
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) z16[e] = 0.0f;
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[cur][i], bv[cur][j],
+                                                                            z16, 0, 0, 0);
+                    } else {
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[cur][i], bv[cur][j],
+                                                                            acc[i][j], 0, 0, 0);
+                    }
+                }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+                __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // four vector instructions
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (s8 < 7)
+                asm volatile("s_waitcnt lgkmcnt(0)"
+                             : "+v"(av[cur ^ 1][0]), "+v"(av[cur ^ 1][1])::"memory");
+        });
+        // y += scale * acc
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const unsigned short sb = (unsigned short)(PAR ? (scur[j] >> 16) : scur[j]);
+            const float sf = __half2float(__builtin_bit_cast(__half, sb));
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) yacc[i][j][e] = fmaf(sf, acc[i][j][e], yacc[i][j][e]);
+        }
+        if constexpr (PAR == 1) {
+            // zero-point term of the groups g - 1 (lanes h = 0) and g (h = 1):
+            // y[m][n] += sum_x[m][g'] * (-scale[n][g'] * (128 + zero[n][g']))
+            float cv[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const unsigned short sb = (unsigned short)(h ? (scur[j] >> 16) : scur[j]);
+                const unsigned short zb = (unsigned short)(h ? (zcur[j] >> 16) : zcur[j]);
+                cv[j] = -__half2float(__builtin_bit_cast(__half, sb)) *
+                        (128.0f + __half2float(__builtin_bit_cast(__half, zb)));
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    yacc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xsum[i], cv[j], yacc[i][j], 0,
+                                                                      0, 0);
+            if (g + 1 < groups) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) scur[j] = snext[j], zcur[j] = znext[j];
+#pragma unroll
+                for (int i = 0; i < 2; ++i) xsum[i] = xsum_next[i];
+            }
+        }
+    };
+    // groups is even (checked on the host); buffers go round in threes, pairs in twos
+    for (int g0 = 0; g0 < groups; g0 += 6) {
+        static_for<6>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            if (g0 + u < groups) group(ic<u % kTpBufs>{}, ic<(u & 1)>{}, g0 + u);
+        });
+    }
+
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int gn = col0 + wc + 32 * j + r;
+        if (gn >= n) continue;
+        const float bv = bias ? bias[gn] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int gr = row0 + wr + 32 * i + 8 * (e >> 2) + 4 * h + (e & 3);
+                if (gr < m) {
+                    if constexpr (F32OUT)
+                        static_cast<float*>(y_out)[(int64_t)gr * n + gn] = yacc[i][j][e] + bv;
+                    else
+                        static_cast<uint16_t*>(y_out)[(int64_t)gr * n + gn] =
+                            f32_to_bf16_rne(yacc[i][j][e] + bv);
+                }
+            }
+    }
+}
+
+}  // namespace lg
+
+extern "C" logismos_status_t logismos_check_qgemm_q4g128_tall_shape(int m, int n, int k, char* msg,
+                                                                    size_t msg_cap) {
+    const char* kn = "qgemm_q4g128_tall";
+    if (m <= 0) return lg::reject(msg, msg_cap, "%s: rows must be positive, got %d", kn, m);
+    if (n <= 0) return lg::reject(msg, msg_cap, "%s: N must be positive, got %d", kn, n);
+    if (k <= 0 || k % 256 != 0)
+        return lg::reject(msg, msg_cap,
+                          "%s: K = %d is not a positive multiple of 256 (pairs of groups of 128)",
+                          kn, k);
+    const int64_t lim = INT32_MAX;
+    if ((int64_t)n * k > lim)
+        return lg::reject(msg, msg_cap, "%s: N*K = %lld exceeds i32::MAX", kn,
+                          (long long)((int64_t)n * k));
+    if ((int64_t)lg::tp_padded_rows(m) * k * 2 > lim || (int64_t)m * n > lim)
+        return lg::reject(msg, msg_cap, "%s: rows*K*2 or rows*N exceeds i32::MAX", kn);
+    if ((lg::tp_padded_rows(m) / lg::kTpTileM) > 65535)
+        return lg::reject(msg, msg_cap, "%s: more than 65535 row tiles", kn);
+    return 0;
+}
+
+extern "C" size_t logismos_qgemm_q4g128_tall_workspace_bytes(int m, int k) {
+    if (m <= 0 || k <= 0 || k % 128 != 0) return 0;
+    return lg::tp_sums_offset(m, k) + (size_t)lg::tp_padded_rows(m) * (k / 128) * 4;
+}
+
+extern "C" logismos_status_t logismos_launch_qgemm_q4g128_tall(
+    const void* x_bf16, const void* qw_u8, const void* scale_f16, const void* zero_f16,
+    const void* bias_f32, void* y, int y_is_f32, void* workspace, int m, int n, int k,
+    logismos_stream_t stream) {
+    if (logismos_check_qgemm_q4g128_tall_shape(m, n, k, nullptr, 0) != 0)
+        return hipErrorInvalidValue;
+    if (!x_bf16 || !qw_u8 || !scale_f16 || !zero_f16 || !y || !workspace)
+        return hipErrorInvalidValue;
+    if ((reinterpret_cast<uintptr_t>(qw_u8) | reinterpret_cast<uintptr_t>(x_bf16) |
+         reinterpret_cast<uintptr_t>(workspace)) & 15u)
+        return hipErrorInvalidValue;
+    if ((reinterpret_cast<uintptr_t>(scale_f16) | reinterpret_cast<uintptr_t>(zero_f16)) & 3u)
+        return hipErrorInvalidValue;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int m_pad = lg::tp_padded_rows(m);
+    uint16_t* xp = static_cast<uint16_t*>(workspace);
+    float* xs = reinterpret_cast<float*>(static_cast<char*>(workspace) + lg::tp_sums_offset(m, k));
+    const int64_t chunks = (int64_t)m_pad * (k / 8);
+    lg::q4_tall_prepare_kernel<<<dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st>>>(
+        static_cast<const uint16_t*>(x_bf16), xp, xs, m, m_pad, k);
+    const dim3 grid((n + lg::kTpTileN - 1) / lg::kTpTileN, m_pad / lg::kTpTileM);
+    constexpr size_t lds = (size_t)lg::kTpBufs * lg::kTpBufBytes;
+    if (y_is_f32) {
+        static const hipError_t opt = hipFuncSetAttribute(
+            reinterpret_cast<const void*>(lg::qgemm_q4g128_tallp_kernel<true>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (opt != hipSuccess) return opt;
+        lg::qgemm_q4g128_tallp_kernel<true><<<grid, dim3(512), lds, st>>>(
+            xp, xs, static_cast<const uint8_t*>(qw_u8), static_cast<const __half*>(scale_f16),
+            static_cast<const __half*>(zero_f16), static_cast<const float*>(bias_f32), y, m, n, k);
+    } else {
+        static const hipError_t opt = hipFuncSetAttribute(
+            reinterpret_cast<const void*>(lg::qgemm_q4g128_tallp_kernel<false>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (opt != hipSuccess) return opt;
+        lg::qgemm_q4g128_tallp_kernel<false><<<grid, dim3(512), lds, st>>>(
+            xp, xs, static_cast<const uint8_t*>(qw_u8), static_cast<const __half*>(scale_f16),
+            static_cast<const __half*>(zero_f16), static_cast<const float*>(bias_f32), y, m, n, k);
+    }
+    return hipGetLastError();
+}

@@ -54,6 +54,9 @@ _SIGNATURES = {
     "logismos_check_qgemm_q4g128_shape": (C.c_uint32, [_i, _i, _i, C.c_char_p, _sz]),
     "logismos_launch_qgemm_q4g128_bf16": (C.c_uint32, [_vp] * 5 + [_i, _i, _i, _vp]),
     "logismos_launch_qgemm_q4g128_bf16_mfma": (C.c_uint32, [_vp] * 5 + [_i, _i, _i, _vp]),
+    "logismos_check_qgemm_q4g128_tall_shape": (C.c_uint32, [_i, _i, _i, C.c_char_p, _sz]),
+    "logismos_qgemm_q4g128_tall_workspace_bytes": (_sz, [_i, _i]),
+    "logismos_launch_qgemm_q4g128_tall": (C.c_uint32, [_vp] * 6 + [_i, _vp, _i, _i, _i, _vp]),
     "logismos_launch_repack_q8_0": (C.c_uint32, [_vp, _vp, _vp, _i, _i, _vp]),
     "logismos_check_qgemv_q4g32_shape": (C.c_uint32, [_i, _i, C.c_char_p, _sz]),
     "logismos_launch_qgemv_q4g32_f32": (C.c_uint32, [_vp] * 5 + [_i, _i, _vp]),
@@ -284,6 +287,19 @@ def launch_qgemm_q4g128_bf16(x, qw, scale, zero, y, b: int, n: int, k: int, stre
           else library().logismos_launch_qgemm_q4g128_bf16)
     _status("qgemm_q4g128_bf16", fn(_ptr(x), _ptr(qw), _ptr(scale), _ptr(zero), _ptr(y), b, n, k,
                                     _raw(stream)))
+
+
+def qgemm_q4g128_tall_workspace_bytes(m: int, k: int) -> int:
+    return library().logismos_qgemm_q4g128_tall_workspace_bytes(m, k)
+
+
+def launch_qgemm_q4g128_tall(x, qw, scale, zero, y, workspace, m: int, n: int, k: int,
+                             stream=None, bias=None, f32_out: bool = False) -> None:
+    """`linear_t` over many rows through the tiled kernel with a workspace."""
+    _guard("qgemm_q4g128_tall", library().logismos_check_qgemm_q4g128_tall_shape, m, n, k)
+    _status("qgemm_q4g128_tall", library().logismos_launch_qgemm_q4g128_tall(
+        _ptr(x), _ptr(qw), _ptr(scale), _ptr(zero), _ptr(bias) if bias is not None else None,
+        _ptr(y), 1 if f32_out else 0, _ptr(workspace), m, n, k, _raw(stream)))
 
 
 def launch_repack_q8_0(blocks, qs, d, n: int, k: int, stream=None) -> None:

@@ -173,3 +173,83 @@ def test_q4g128_tiled_kernel_one_hot_rows_read_back_dequantised_columns():
     want = O.bf16_bits_to_f32(O.f32_to_bf16_bits(wd[:, cols].T.copy()))
     # (128 + q) - (128 + zero) in fp32, times scale: the same value the oracle rounds
     assert_parity(got, want, max_abs=1e-6, max_rel=4e-3, what="one-hot rows")
+
+
+def _gemm_q4_ws(xb, qw, s, z, b, n, k, bias, f32_out=False, ws_fill=0xFF):
+    """`logismos_launch_qgemm_q4g128_tall`: the same product through the entry point with a
+    workspace (first pass over x, then the tiled kernel that reads x straight into LDS)."""
+    ws = hip.DeviceBuffer(kernels.qgemm_q4g128_tall_workspace_bytes(b, k))
+    ws.fill(ws_fill)
+    d_y = hip.DeviceBuffer(b * n * (4 if f32_out else 2))
+    d_y.fill(0xFF)
+    kernels.launch_qgemm_q4g128_tall(up(xb), up(qw), up(s.view(np.uint16)), up(z.view(np.uint16)),
+                                     d_y, ws, b, n, k, bias=up(bias) if bias is not None else None,
+                                     f32_out=f32_out)
+    hip.synchronize()
+    if f32_out:
+        return d_y.to_numpy(np.float32, (b, n))
+    return O.bf16_bits_to_f32(d_y.to_numpy(np.uint16, (b, n)))
+
+
+@pytest.mark.parametrize("b,n,k,with_bias", [(1, 16, 256, True), (97, 128, 256, False),
+                                             (130, 200, 512, True), (257, 1000, 1280, True),
+                                             (300, 4100, 4096, False), (1000, 333, 2048, True),
+                                             (142, 576, 512, True)])
+def test_q4g128_workspace_kernel_ragged_shapes(b, n, k, with_bias):
+    # partial tiles in rows (128) and in weight rows (256), K of two groups up to 32, with and
+    # without a bias; the fp32 product (what the step executor keeps) tightly, the bf16 one at
+    # the decode path's tolerance; what the workspace held before does not matter
+    rng = np.random.default_rng(b + 7 * n + 13 * k)
+    qw, s, z = _q4(rng, n, k)
+    xb = O.f32_to_bf16_bits(rng.standard_normal((b, k), np.float32))
+    bias = rng.standard_normal(n).astype(np.float32) if with_bias else None
+    got32 = _gemm_q4_ws(xb, qw, s, z, b, n, k, bias, f32_out=True)
+    want32 = O.qgemm_q4g128_f32(xb, qw, s, z, b, n, k, bias)
+    assert_parity(got32, want32, max_abs=2e-4, max_rel=1e-3, what=f"q4g128 workspace f32 {b}x{n}x{k}")
+    got = _gemm_q4_ws(xb, qw, s, z, b, n, k, bias, ws_fill=0x00)
+    want = O.bf16_bits_to_f32(O.qgemm_q4g128_bf16(xb, qw, s, z, b, n, k, bias))
+    assert_parity(got, want, what=f"q4g128 workspace bf16 {b}x{n}x{k}")
+    # the bf16 product is the one rounding of the fp32 one
+    assert np.array_equal(O.f32_to_bf16_bits(got32).reshape(b, n),
+                          O.f32_to_bf16_bits(got).reshape(b, n))
+
+
+def test_q4g128_workspace_kernel_one_hot_rows_read_back_dequantised_columns():
+    # orientation, nibble order, the pair order the first pass writes, the LDS swizzles of x
+    # and of the weights, and the zero-point product in one exact check: row i of x is the unit
+    # vector of column c_i, so row i of y is column c_i of the dequantised matrix
+    rng = np.random.default_rng(11)
+    b, n, k = 384, 300, 768
+    w = rng.standard_normal((n, k), np.float32)
+    qw, s, z = O.quantize_q4g128(w, n, k)
+    wd = O.dequantize_q4g128(qw, s, z, n, k)
+    cols = rng.integers(0, k, size=b)
+    cols[:10] = [0, 1, 4, 7, 8, 63, 64, 127, 128, 767]
+    x = np.zeros((b, k), np.float32)
+    x[np.arange(b), cols] = 1.0
+    got = _gemm_q4_ws(O.f32_to_bf16_bits(x), qw, s, z, b, n, k, None, f32_out=True)
+    # scale * (128 + q) and scale * (128 + zero) * 1 are rounded apart (values of ~50 here, one
+    # fp32 ulp 4e-6) before they cancel to the dequantised weight of order 1
+    assert_parity(got, wd[:, cols].T.copy(), max_abs=8e-6, max_rel=1e-5, what="one-hot rows")
+
+
+def test_q4g128_workspace_kernel_config4_rows():
+    # config 4's 8240 packed rows through an attention-output-sized projection with a bias
+    rng = np.random.default_rng(12)
+    b, n, k = 8240, 4096, 4096
+    qw, s, z = _q4(rng, n, k)
+    xb = O.f32_to_bf16_bits(rng.standard_normal((b, k), np.float32))
+    bias = rng.standard_normal(n).astype(np.float32)
+    got = _gemm_q4_ws(xb, qw, s, z, b, n, k, bias)
+    rows = np.r_[0:3, 126:131, 4111:4114, 8190:8194, 8222:8240]
+    want = O.bf16_bits_to_f32(O.qgemm_q4g128_bf16(xb[rows], qw, s, z, len(rows), n, k, bias))
+    assert_parity(got[rows], want, what="q4g128 workspace m = 8240 + bias")
+    assert np.isfinite(got).all()
+
+
+def test_q4g128_workspace_entry_point_refuses_what_it_cannot_run():
+    with pytest.raises(kernels.UnsupportedShape):
+        kernels.launch_qgemm_q4g128_tall(None, None, None, None, None, None, 128, 128, 384)
+    with pytest.raises(kernels.UnsupportedShape):
+        kernels.launch_qgemm_q4g128_tall(None, None, None, None, None, None, 0, 128, 256)
+    assert kernels.qgemm_q4g128_tall_workspace_bytes(130, 512) == 256 * 512 * 2 + 256 * 4 * 4

@@ -171,6 +171,24 @@ def test_config4_prefill_rows_agree_with_decode_rows_at_full_size():
     assert_parity(rows_dec, want_dec, what="config 4 decode rows vs oracle")
 
 
+def test_config4_prefill_chunk_at_full_size_against_the_oracle():
+    # one chunk of config 4 at its largest: 512 new tokens behind 8 100 tokens of prior context
+    # (the config draws priors from 0..8192), 32 query / 8 KV heads, next to a decode row; pools
+    # of distinct random rows, the whole chunk against the CPU oracle
+    rng = np.random.default_rng(44)
+    c = workloads.paged_case(rng, [512, 1], [8100, 8611], hq=32, hkv=8)
+    _check(c, what="512-token chunk, prior 8100")
+
+
+def test_config5_attention_at_full_size_with_distinct_pool_rows():
+    # the decode step's attention at its own size (32 sequences, contexts U[256, 8192], 32 / 8
+    # heads) over pools in which no two rows are alike: a gather that is off by any number of
+    # rows reads different values
+    c = workloads.config5_attention()
+    assert int(c["context_lens"].sum()) > 100_000
+    _check(c, what="config 5 attention, distinct rows")
+
+
 @pytest.mark.parametrize("hq,hkv", [(1, 1), (4, 2), (12, 2), (12, 4), (32, 8), (8, 1), (16, 16),
                                     (14, 2)])
 def test_balanced_decode_kernel_gqa_group_sizes(hq, hkv):
