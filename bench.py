@@ -519,8 +519,8 @@ def bench_q4_tall(args):
         del d, dy, ws
     return {"workload": "config 4's 8240 packed rows through one layer's Q4G128 projections "
                         "(qkv 6144x4096, o 4096x4096, gate_up 24576x4096, down 4096x12288)",
-            "kernel": "q4_tall_prepare_kernel + qgemm_q4g128_tallp_kernel (128x128 tiles, x "
-                      "straight into LDS, v_mfma_f32_32x32x16_bf16)",
+            "kernel": "q4_tall_prepare_kernel + qgemm_q4g128_tallp_kernel (128x256 tiles, x and "
+                      "weights straight into a three-deep LDS ring, v_mfma_f32_32x32x16_bf16)",
             "projections": out, "ms_per_layer": round(ms_all, 4),
             "ms_per_layer_entry_point_without_workspace": round(ms_noworkspace, 4),
             "roofline": {"bound": "mfma", "achieved": round(flops_all / ms_all / 1e9, 1),
