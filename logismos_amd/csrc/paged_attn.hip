@@ -1038,9 +1038,9 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams 
 //
 // The C layout of S^T (lane (hl, c): keys 8g + 4hl + i of column c) is, read as
 // "slot e = 4*(g%2) + i of MFMA g/2", already a B-operand layout, so P never
-// leaves its lane; V is written to LDS transposed ([d][key], two keys per
-// 32-bit store, keys in P's slot order) so that the matching A operand is one
-// 16-byte read.
+// leaves its lane.  K and V rows go to LDS as they are (16-byte stores); the A
+// operand of the second product is read out of the row-major V tile with the
+// transposing LDS read (ds_read_b64_tr_b16, see v_operand in the kernel).
 //
 // Schedule of one step (tile t): request K rows of tile t+3 / V rows of tile t+1
 // from memory; then, in one block of interleaved instructions, the MFMAs of
@@ -1055,12 +1055,13 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams 
 constexpr int kPfKeys = 32;
 constexpr int kPfWaves = 8;
 constexpr int kKsStride = kHeadDim + 8;  // halfs per K row in LDS (272 B)
-constexpr int kVtStride = kPfKeys + 8;   // halfs per V^T row in LDS (80 B: 16-byte reads stay aligned)
+constexpr int kVsStride = kHeadDim + 16; // halfs per V row in LDS (288 B)
 constexpr int kKsElems = kPfKeys * kKsStride;
-constexpr int kVtElems = kHeadDim * kVtStride;
+constexpr int kVsElems = kPfKeys * kVsStride;
 constexpr int kStageStride = kHeadDim + 8;
 constexpr float kLazyLog2 = 8.0f;  // headroom of the lazily updated softmax maximum
 constexpr int kPfRankMax = 512;    // sequences ordered by length inside the kernel
+constexpr int kPfBtLds = 8192;     // block-table entries of the sequence held in LDS
 
 struct PfRegs {
     uint4_t x[2];  // the two keys of this thread's pair
@@ -1135,10 +1136,10 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
     const int wi0 = i0 + w * TPW;  // first token of this wave
     const int wave_min = wi0 < n_new ? limit_of(wi0) : 0;
 
-    __shared__ __attribute__((aligned(16))) _Float16 smem[2 * kKsElems + 2 * kVtElems];
-    static_assert(kPfWaves * 16 * kStageStride <= 2 * kKsElems + 2 * kVtElems, "stage fits");
+    __shared__ __attribute__((aligned(16))) _Float16 smem[2 * kKsElems + 2 * kVsElems];
+    static_assert(kPfWaves * 16 * kStageStride <= 2 * kKsElems + 2 * kVsElems, "stage fits");
     _Float16* Ks = smem;
-    _Float16* Vt = smem + 2 * kKsElems;
+    _Float16* Vs = smem + 2 * kKsElems;
 
     // ---- column of this lane and its query (B operand: column c, d = 16j + 8hl ..)
     const int col_tok_l = c / G;
@@ -1175,11 +1176,33 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
     // of keys 2kp and 2kp + 1 of its pool.  The eight keys a wave carries sit in one KV
     // block (8-aligned, block_size % 16 == 0, and a key past the end re-reads key kmax - 1
     // of that same block or, when the whole group is past the end, of its own block), so the
-    // physical block id is one scalar load per wave and tile.
+    // physical block id is wave-uniform (one LDS read per wave and tile).
     const int kp = (tid & 255) >> 4;
     const int piece = tid & 15;
     const bool moves_v = __builtin_amdgcn_readfirstlane(w >> 2) != 0;
     const int32_t* bt_row = p.block_tables + (int64_t)s * p.max_blocks_per_seq;
+    // The block ids of the keys this workgroup streams, copied to LDS once: read from
+    // memory inside the tile loop, each is a vector load (the compiler cannot show that
+    // nothing writes the table) on whose arrival the next step's addresses wait, and its
+    // wait covers the tile rows in flight as well.  Entries beyond the copy (contexts of
+    // more than kPfBtLds blocks) still come from memory.
+    __shared__ int bt_lds[kPfBtLds];
+    {
+        const int nb = min((kmax + p.block_size - 1) / p.block_size, kPfBtLds);
+        for (int i = tid; i < nb; i += 64 * kPfWaves) bt_lds[i] = bt_row[i];
+        __syncthreads();
+    }
+    auto block_id = [&](int bi) {
+        int blk;
+        if (__builtin_expect(bi >= kPfBtLds, 0)) {
+            blk = bt_row[bi];
+            asm volatile("" : "+v"(blk));  // (keeps the two loads apart: merged, they become
+                                           // one flat load that waits on both counters)
+        } else {
+            blk = bt_lds[bi];
+        }
+        return __builtin_amdgcn_readfirstlane(blk);
+    };
     const int wave_key0 = __builtin_amdgcn_readfirstlane(8 * (w & 3));
     struct PfAddr {
         int blk;   // physical block (wave-uniform)
@@ -1202,7 +1225,7 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
         const bool past = pos > last_key;
         const int bi = past ? last_bi : cur_bi;
         const int base = past ? last_base : cur_base;
-        PfAddr a{bt_row[bi], cur_tile * kPfKeys - base, cur_tile};
+        PfAddr a{block_id(bi), cur_tile * kPfKeys - base, cur_tile};
         ++cur_tile;
         return a;
     };
@@ -1247,10 +1270,11 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
         for (int i = 0; i < 8; ++i) o[i] = cv[i] * nh;
         return __builtin_bit_cast(uint4_t, o);
     };
-    // column (in halfs) of this thread's key pair inside a V^T row (see lstore)
-    const int vt_pos = ((2 * kp) & ~12) | (((2 * kp) & 4) << 1) | (((2 * kp) & 8) >> 1);
-    const int vt_col = 8 * ((vt_pos >> 3) ^ ((piece >> 1) & 3)) + (vt_pos & 7);
-    // K rows as they are; V transposed, (key 2kp, key 2kp+1) of element e as one word
+    // K and V rows as they are, 16 bytes per store.  The 16-byte chunks of a V row are
+    // stored in the order (bit 1, bit 3, bit 2, bit 0) of the chunk index, which puts the
+    // two halves of every 32-element block 128 bytes apart: the two groups of 16 lanes that
+    // read them in one request then use different banks (see v_operand).
+    const int v_chunk = (piece & 1) | (((piece >> 2) & 3) << 1) | (((piece >> 1) & 1) << 3);
     auto lstore = [&](int buf, const PfRegs& raw) {
         PfRegs r = raw;
         if constexpr (T3) {
@@ -1263,17 +1287,10 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
             for (int u = 0; u < 2; ++u)
                 *reinterpret_cast<uint4_t*>(ks + (2 * kp + u) * kKsStride + 8 * piece) = r.x[u];
         } else {
-            // Key k of a 16-key slab sits at position swap(bit 2, bit 3) of k, the order in
-            // which the P operand holds it, so that a lane's 8 keys are one 16-byte read; the
-            // four 16-byte chunks of a row are XOR-swizzled by (row / 16) % 4, which makes
-            // these transposed 4-byte stores two-way instead of eight-way bank conflicts
-            _Float16* vt = Vt + buf * kVtElems + vt_col;
+            _Float16* vs = Vs + buf * kVsElems;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const unsigned sel = (e & 1) ? 0x07060302u : 0x05040100u;
-                const unsigned pr = __builtin_amdgcn_perm(r.x[1][e >> 1], r.x[0][e >> 1], sel);
-                *reinterpret_cast<unsigned*>(vt + (8 * piece + e) * kVtStride) = pr;
-            }
+            for (int u = 0; u < 2; ++u)
+                *reinterpret_cast<uint4_t*>(vs + (2 * kp + u) * kVsStride + 8 * v_chunk) = r.x[u];
         }
     };
 
@@ -1294,9 +1311,28 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
 #pragma unroll
     for (int kh = 0; kh < 2; ++kh) p_prev[kh] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
     float16_t s_cur;
-    // lane part of a V^T operand address: row c of a 32-row block, the lane's half of a
-    // 16-key slab, under the chunk swizzle of lstore
-    const int vt_lane = c * kVtStride + 8 * (hl ^ (c >> 4));
+    // The A operand of O^T += V^T . P -- lane (hl, r): element r of a 32-element block for
+    // the keys {16kh + 4hl + i} and {16kh + 8 + 4hl + i}, i = 0..3, the key order in which
+    // P sits in its lane -- comes out of the row-major tile through two ds_read_b64_tr_b16:
+    // inside a group of 16 lanes, lane L receives element L % 4 of the four 8-byte pieces
+    // that the lanes L / 4, 4 + L / 4, 8 + L / 4, 12 + L / 4 point at, so with lane s of a
+    // group pointing at elements 4 (s % 4) .. + 3 of key s / 4, lane L ends up with element
+    // L of four keys.  (A transposed copy of the tile, written with 4-byte stores, cost the
+    // threads that moved V eight permutes and eight stores per tile, and a quarter of the
+    // kernel's time went into those stores and their bank conflicts.)  Lane part of the
+    // address, under the chunk order of lstore:
+    const int s16 = lane & 15;
+    const int v_lane = (4 * hl + (s16 >> 2)) * kVsStride + 64 * ((lane >> 4) & 1) + 4 * (s16 & 3);
+    auto v_operand = [&](const _Float16* vs, int kh, int dt) {
+        typedef short short4_t __attribute__((ext_vector_type(4)));
+        typedef __attribute__((address_space(3))) short4_t lds_short4_t;
+        const _Float16* a = vs + 16 * kh * kVsStride + 16 * dt;
+        const uint2_t lo = __builtin_bit_cast(
+            uint2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_t*)a));
+        const uint2_t hi = __builtin_bit_cast(
+            uint2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_t*)(a + 8 * kVsStride)));
+        return __builtin_bit_cast(half8_t, uint4_t{lo[0], lo[1], hi[0], hi[1]});
+    };
 
     // S^T of the first key tile (the steps compute every later one)
     auto qk_first = [&]() {
@@ -1312,15 +1348,13 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
     };
     // O += V^T(buffer buf) . P
     auto pv_from = [&](int buf, const half8_t (&pb)[2]) {
-        const _Float16* vt = Vt + buf * kVtElems + vt_lane;
+        const _Float16* vs = Vs + buf * kVsElems + v_lane;
 #pragma unroll
         for (int kh = 0; kh < 2; ++kh)
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt)
-                oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                    *reinterpret_cast<const half8_t*>(vt + 32 * dt * kVtStride +
-                                                      16 * (kh ^ (dt & 1))),
-                    pb[kh], oacc[dt], 0, 0, 0);
+                oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(v_operand(vs, kh, dt), pb[kh],
+                                                                  oacc[dt], 0, 0, 0);
     };
     // One step: tile t with S(t) in s_cur; K(t+1) in K buffer 1-H, V(t-1) in V buffer 1-H.
     // Leaves S(t+1) in s_cur and P(t) in p_prev.  MASKED: some column may not see all keys
@@ -1329,14 +1363,13 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
         constexpr bool MASKED = decltype(masked_c)::value != 0;
         constexpr int H = decltype(h_c)::value;
         const _Float16* ks = Ks + (1 - H) * kKsElems + c * kKsStride + 8 * hl;
-        const _Float16* vt = Vt + (1 - H) * kVtElems + vt_lane;
+        const _Float16* vs = Vs + (1 - H) * kVsElems + v_lane;
         // operands in the order the MFMAs below take them
         half8_t ka[8], va[2][4];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             ka[j] = *reinterpret_cast<const half8_t*>(ks + 16 * j);
-            va[j >> 2][j & 3] = *reinterpret_cast<const half8_t*>(
-                vt + 32 * (j & 3) * kVtStride + 16 * ((j >> 2) ^ (j & 1)));
+            va[j >> 2][j & 3] = v_operand(vs, j >> 2, j & 3);
         }
 
         // ---- F(t), first part: tile maximum and the lazily raised reference maximum
@@ -1390,14 +1423,15 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
         }
         l = fmaf(l, alpha, psum);
         if constexpr (!MASKED) {
-            // Order of the block: the first eight operand reads, then 16 MFMAs, each followed
-            // by the read of the operand eight MFMAs ahead (into the registers just freed) and
-            // by its share of the VALU work
-            __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+            // Order of the block: the operand reads of the first four MFMA pairs (a K
+            // operand is one read, a V operand two), then 16 MFMAs, each followed by one of
+            // the remaining reads (into registers freed before) and by its share of the
+            // VALU work
+            __builtin_amdgcn_sched_group_barrier(0x100, 12, 0);
 #pragma unroll
             for (int g = 0; g < 16; ++g) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                if (g < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                if (g < 12) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
                 __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
             }
         }
@@ -1437,12 +1471,14 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_attn_prefill_kernel(const
                 gload(a, ra);  // K(2) in flight
             }
             // V buffer 1 plays V(-1) in the first step (P(-1) = 0): finite values
-            unsigned* vz = reinterpret_cast<unsigned*>(Vt + kVtElems);
-            for (int i = tid; i < kVtElems / 2; i += 64 * kPfWaves) vz[i] = 0u;
+            unsigned* vz = reinterpret_cast<unsigned*>(Vs + kVsElems);
+            for (int i = tid; i < kVsElems / 2; i += 64 * kPfWaves) vz[i] = 0u;
         }
         PfAddr an = next_addr();
         __syncthreads();
         s_cur = qk_first();
+        // (the first step ends with a store into the K buffer just read)
+        __syncthreads();
         const int plain_tiles = min(ntiles, limit_of(i0) / kPfKeys) & ~1;
         auto two_steps = [&](auto masked_c, int tile) {
             // ---- tile: K(tile+3) / V(tile+1) requested, K(tile+2) / V(tile) to buffer 0
@@ -1582,8 +1618,9 @@ static hipError_t launch_group(const AttnParams& p, int max_seqlen_q, int phases
             paged_attn_kernel<G, T3><<<grid_d, block, 0, stream>>>(p);
         }
     }
-    if ((phases & LOGISMOS_ATTN_PHASE_PREFILL) && max_seqlen_q > 1)
+    if ((phases & LOGISMOS_ATTN_PHASE_PREFILL) && max_seqlen_q > 1) {
         launch_prefill<G, T3>(p, max_seqlen_q, stream);
+    }
     if ((phases & LOGISMOS_ATTN_PHASE_MERGE) && p.num_splits > 1) {
         dim3 grid_m(p.hq, p.num_seqs);
         paged_attn_merge_kernel<<<grid_m, dim3(256), 0, stream>>>(p);
