@@ -153,6 +153,39 @@ def against_ceiling(stream, nbytes: int, achieved_gbps: float) -> dict:
             "frac_of_measured_ceiling": round(achieved_gbps / c["GBps"], 4)}
 
 
+_MFMA_CEILING_CACHE = {}
+
+
+def mfma_ceiling(stream, bf16: bool) -> dict:
+    """What the matrix cores of THIS box sustain (TFLOP/s) when a kernel issues nothing but
+    v_mfma_f32_32x32x16 on every CU: with operands that never change, and with operands
+    rewritten between the MFMAs as real data rewrites them.  The datasheet's 2.5 PFLOP/s is
+    the peak every fraction is quoted against; the second figure is the ceiling an MFMA-bound
+    kernel on real data can actually be held to (the part slows the pipes when their inputs
+    toggle)."""
+    if bf16 not in _MFMA_CEILING_CACHE:
+        sink = hip.DeviceBuffer(16)
+        iters = 4000
+        flops = kernels.probe_mfma_flops(iters)
+        rates = {}
+        for name, flags in (("constant_operands", 0), ("changing_operands",
+                                                       kernels.PROBE_MFMA_CHANGING)):
+            flags |= kernels.PROBE_MFMA_BF16 if bf16 else 0
+            fn = [lambda flags=flags: kernels.launch_probe_mfma(sink, iters, flags, stream)]
+            ms, _, _ = time_launches(stream, fn, 10, 3)
+            rates[name] = round(flops / ms / 1e9, 1)
+        _MFMA_CEILING_CACHE[bf16] = rates
+    return _MFMA_CEILING_CACHE[bf16]
+
+
+def against_mfma_ceiling(stream, bf16: bool, achieved_tflops: float) -> dict:
+    """The fields every MFMA-bound figure carries beside its fraction of the 2.5 PFLOP/s peak."""
+    c = mfma_ceiling(stream, bf16)
+    return {"measured_mfma_ceiling_TFLOPs": c["changing_operands"],
+            "measured_mfma_rate_constant_operands_TFLOPs": c["constant_operands"],
+            "frac_of_measured_ceiling": round(achieved_tflops / c["changing_operands"], 4)}
+
+
 def replicate(buf: hip.DeviceBuffer, copies: int):
     out = [buf]
     for _ in range(copies - 1):
@@ -323,7 +356,9 @@ def bench_mixed_config4(args):
                      "peak": 2500.0, "unit": "TFLOP/s",
                      "frac": round(flops_pre / (ms_pre * 1e-3) / 1e12 / 2500.0, 4),
                      "traffic": None, "kernel": "paged_attn_prefill_kernel<4>",
-                     "flops_per_launch": flops_pre},
+                     "flops_per_launch": flops_pre,
+                     **against_mfma_ceiling(stream, False,
+                                            flops_pre / (ms_pre * 1e-3) / 1e12)},
         "decode_rows_GBps": round(dec_bytes / (ms_dec * 1e-3) / 1e9, 1),
         "decode_rows_frac_of_peak": round(dec_bytes / (ms_dec * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
         "decode_rows": against_ceiling(stream, dec_bytes, dec_bytes / (ms_dec * 1e-3) / 1e9),
@@ -526,7 +561,8 @@ def bench_q4_tall(args):
             "roofline": {"bound": "mfma", "achieved": round(flops_all / ms_all / 1e9, 1),
                          "peak": 2500.0, "unit": "TFLOP/s",
                          "frac": round(flops_all / ms_all / 1e9 / 2500.0, 4), "traffic": None,
-                         "flops_per_layer": flops_all},
+                         "flops_per_layer": flops_all,
+                         **against_mfma_ceiling(stream, True, flops_all / ms_all / 1e9)},
             "parity_max_abs_vs_oracle_sample": parity}
 
 

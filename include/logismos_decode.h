@@ -855,6 +855,20 @@ logismos_status_t logismos_launch_probe_read(const void* src, void* sink_u32, si
 logismos_status_t logismos_launch_probe_read_ex(const void* src, void* sink_u32, size_t bytes,
                                                 int flags, logismos_stream_t stream);
 
+/* The matrix-core counterpart (no counterpart in the reference): 256 workgroups of
+ * eight waves issue nothing but v_mfma_f32_32x32x16 (fp16, or bf16 with
+ * LOGISMOS_PROBE_MFMA_BF16) on four accumulators, `iters` x 4 per wave; with
+ * LOGISMOS_PROBE_MFMA_CHANGING both operands are rewritten between the MFMAs, as
+ * they are on real data.  The rate of the second form is the matrix-core ceiling
+ * the MFMA-bound kernels are measured against beside the datasheet peak: the part
+ * holds the pipes back when their inputs toggle.  `_flops` is the work of one
+ * launch.  `sink_f32` (4 bytes) is practically never written. */
+#define LOGISMOS_PROBE_MFMA_CHANGING 1
+#define LOGISMOS_PROBE_MFMA_BF16 2
+logismos_status_t logismos_launch_probe_mfma(void* sink_f32, int iters, int flags,
+                                             logismos_stream_t stream);
+double logismos_probe_mfma_flops(int iters);
+
 #ifdef __cplusplus
 }
 #endif

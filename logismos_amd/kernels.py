@@ -141,6 +141,8 @@ _SIGNATURES = {
     "logismos_launch_probe_copy": (C.c_uint32, [_vp, _vp, _sz, _vp]),
     "logismos_launch_probe_read": (C.c_uint32, [_vp, _vp, _sz, _vp]),
     "logismos_launch_probe_read_ex": (C.c_uint32, [_vp, _vp, _sz, _i, _vp]),
+    "logismos_launch_probe_mfma": (C.c_uint32, [_vp, _i, _i, _vp]),
+    "logismos_probe_mfma_flops": (C.c_double, [_i]),
 }
 
 ATTN_PHASE_DECODE, ATTN_PHASE_PREFILL, ATTN_PHASE_MERGE, ATTN_PHASE_ALL = 1, 2, 4, 7
@@ -398,6 +400,19 @@ PROBE_NON_TEMPORAL, PROBE_STRIDED = 1, 2
 def launch_probe_read(src, sink, nbytes: int, stream=None, flags: int = 0) -> None:
     _status("probe_read", library().logismos_launch_probe_read_ex(_ptr(src), _ptr(sink), nbytes,
                                                                   flags, _raw(stream)))
+
+
+PROBE_MFMA_CHANGING, PROBE_MFMA_BF16 = 1, 2
+
+
+def launch_probe_mfma(sink, iters: int, flags: int = 0, stream=None) -> None:
+    """Nothing but MFMAs on every CU (fp16 or bf16; constant or changing operands)."""
+    _status("probe_mfma", library().logismos_launch_probe_mfma(_ptr(sink), iters, flags,
+                                                               _raw(stream)))
+
+
+def probe_mfma_flops(iters: int) -> float:
+    return float(library().logismos_probe_mfma_flops(iters))
 
 
 def launch_pack_ragged(new_tokens, prior_ctx, block_tables, cu_seqlens, slot_mapping, context_lens,
