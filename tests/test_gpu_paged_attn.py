@@ -124,6 +124,18 @@ def test_chunked_prefill_512_token_chunks_with_prior_context():
     _check(c, what="512-token chunks")
 
 
+def test_chunked_prefill_with_a_block_table_wider_than_the_kernels_lds_copy():
+    # the prefill kernel keeps 8192 entries of a sequence's block-table row in LDS; the keys
+    # of the blocks beyond that (here the last 3 of 8195) take the ids from memory.  Pools
+    # repeat 5003 random rows (a 131 k-key pool takes a while to draw), which a wrong block
+    # id does not survive: the new tokens see all 131 k keys.
+    rng = np.random.default_rng(43)
+    c = workloads.paged_case(rng, [8, 1], [8192 * 16 + 40, 9], hq=1, hkv=1,
+                             pool_period_rows=5003, spare_frac=0.0)
+    assert c["max_blocks"] > 8192
+    _check(c, what="block table wider than 8192 entries")
+
+
 def test_chunked_prefill_peaked_softmax():
     rng = np.random.default_rng(42)
     c = workloads.paged_case(rng, [96, 1], [200, 10], hq=8, hkv=2)
