@@ -572,6 +572,23 @@ logismos_status_t logismos_launch_rms_norm_fp16(const void* x_fp16, const void* 
  * becomes uniform 1/n as in `softmax_fp16_ref` (crates/kernels/src/softmax/cpu.rs:40-59). */
 logismos_status_t logismos_launch_softmax_fp16(const void* x_fp16, void* y_fp16, int m, int n,
                                                logismos_stream_t stream);
+/* `cpu_f32::mask_additive_in_place` (crates/kernels/src/cpu_f32/mod.rs:451-486) on device
+ * scores: scores[r][c] becomes -inf where mask[r / repeat][c] == 0, with
+ * mask_rows = mask_len / n and repeat = rows / mask_rows (one mask row -- a batch row's
+ * key-padding mask -- serves the `repeat` consecutive score rows of its heads).  Like the
+ * reference: nothing to do (success) when n, rows or mask_len is 0 or the mask is shorter
+ * than a row; where the reference panics -- rows not a multiple of mask_rows -- and where
+ * its debug assertion fires -- a mask that is not whole rows -- InvalidValue and nothing
+ * launched.  `_f32` is the reference's own type; `_fp16` masks the fp16 scores that
+ * `logismos_launch_matmul_*_fp16` produce and `logismos_launch_softmax_fp16` consumes (a row
+ * masked everywhere then comes out uniform, as in the reference).  The fused paged attention
+ * masks by context length and causality only; a padded batch goes through these. */
+logismos_status_t logismos_launch_mask_additive_f32(void* scores_f32, const void* mask_u8,
+                                                    size_t mask_len, size_t rows, size_t n,
+                                                    logismos_stream_t stream);
+logismos_status_t logismos_launch_mask_additive_fp16(void* scores_fp16, const void* mask_u8,
+                                                     size_t mask_len, size_t rows, size_t n,
+                                                     logismos_stream_t stream);
 /* crates/kernels/src/rope/hip/rope.hip:45-68: in place on (batch, seq, heads, head_dim),
  * interleaved pairs (2i, 2i+1), table f32 `[seq][head_dim]` with cos at 2i and sin at 2i+1
  * (`build_cos_sin_table`, crates/kernels/src/rope/cpu.rs:19-40).  Shape guard of

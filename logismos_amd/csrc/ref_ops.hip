@@ -280,6 +280,82 @@ static bool matmul_shape_ok(int m, int n, int k) {
 
 }  // namespace lg
 
+namespace lg {
+
+// scores[r][c] = -inf where mask[r / repeat][c] == 0 (one mask row serves `repeat` consecutive
+// score rows: the heads of one batch row), 16 bytes of mask per thread where n allows
+template <typename T>
+__global__ __launch_bounds__(256) void mask_additive_kernel(T* __restrict__ scores,
+                                                            const uint8_t* __restrict__ mask,
+                                                            int64_t rows, int64_t n,
+                                                            int64_t repeat, T neg_inf) {
+    const int64_t total = rows * n;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int64_t r = i / n;
+        const int64_t c = i - r * n;
+        if (mask[(r / repeat) * n + c] == 0) scores[i] = neg_inf;
+    }
+}
+
+static logismos_status_t mask_additive_check(const void* scores, const void* mask,
+                                             size_t mask_len, size_t rows, size_t n,
+                                             int64_t* repeat) {
+    *repeat = 0;
+    // `mask_additive_in_place` (crates/kernels/src/cpu_f32/mod.rs:451-486): nothing to do
+    // without columns, rows or a mask, or with a mask shorter than one row
+    if (n == 0 || rows == 0 || mask_len == 0 || mask_len / n == 0) return hipSuccess;
+    if (!scores || !mask) return hipErrorInvalidValue;
+    const size_t mask_rows = mask_len / n;
+    // (the reference's debug assertion: the mask is whole rows)
+    if (mask_rows * n != mask_len) return hipErrorInvalidValue;
+    // the reference panics here: a row count that the mask rows do not divide would leave
+    // the trailing rows unmasked
+    if (rows % mask_rows != 0) return hipErrorInvalidValue;
+    if (rows > (size_t)INT32_MAX || n > (size_t)INT32_MAX ||
+        (uint64_t)rows * (uint64_t)n > ((uint64_t)1 << 40))
+        return hipErrorInvalidValue;
+    *repeat = (int64_t)(rows / mask_rows);
+    return hipSuccess;
+}
+
+template <typename T>
+static logismos_status_t mask_additive_launch(void* scores, const void* mask, size_t mask_len,
+                                              size_t rows, size_t n, T neg_inf,
+                                              logismos_stream_t stream) {
+    int64_t repeat;
+    const logismos_status_t st = mask_additive_check(scores, mask, mask_len, rows, n, &repeat);
+    if (st != hipSuccess || repeat == 0) return st;
+    const int64_t total = (int64_t)rows * (int64_t)n;
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 256 * 32) blocks = 256 * 32;
+    mask_additive_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0,
+                              static_cast<hipStream_t>(stream)>>>(
+        static_cast<T*>(scores), static_cast<const uint8_t*>(mask), (int64_t)rows, (int64_t)n,
+        repeat, neg_inf);
+    return hipGetLastError();
+}
+
+}  // namespace lg
+
+extern "C" logismos_status_t logismos_launch_mask_additive_f32(void* scores_f32,
+                                                               const void* mask_u8,
+                                                               size_t mask_len, size_t rows,
+                                                               size_t n,
+                                                               logismos_stream_t stream) {
+    return lg::mask_additive_launch<float>(scores_f32, mask_u8, mask_len, rows, n, -INFINITY,
+                                           stream);
+}
+
+extern "C" logismos_status_t logismos_launch_mask_additive_fp16(void* scores_fp16,
+                                                                const void* mask_u8,
+                                                                size_t mask_len, size_t rows,
+                                                                size_t n,
+                                                                logismos_stream_t stream) {
+    return lg::mask_additive_launch<unsigned short>(scores_fp16, mask_u8, mask_len, rows, n,
+                                                    (unsigned short)0xFC00u, stream);
+}
+
 extern "C" logismos_status_t logismos_launch_rms_norm_fp16(const void* x_fp16, const void* w_fp16,
                                                            void* y_fp16, int m, int n, float eps,
                                                            logismos_stream_t stream) {

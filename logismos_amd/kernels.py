@@ -87,6 +87,8 @@ _SIGNATURES = {
     "logismos_launch_greedy_f32": (C.c_uint32, [_vp, _vp, _i, _i, _vp]),
     "logismos_launch_rms_norm_fp16": (C.c_uint32, [_vp, _vp, _vp, _i, _i, _f, _vp]),
     "logismos_launch_softmax_fp16": (C.c_uint32, [_vp, _vp, _i, _i, _vp]),
+    "logismos_launch_mask_additive_f32": (C.c_uint32, [_vp, _vp, _sz, _sz, _sz, _vp]),
+    "logismos_launch_mask_additive_fp16": (C.c_uint32, [_vp, _vp, _sz, _sz, _sz, _vp]),
     "logismos_launch_rope_fp16": (C.c_uint32, [_vp, _vp, _i, _i, _i, _i, _vp]),
     "logismos_launch_matmul_naive_fp16": (C.c_uint32, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "logismos_launch_matmul_wmma_fp16": (C.c_uint32, [_vp, _vp, _vp, _i, _i, _i, _vp]),
@@ -493,6 +495,16 @@ def launch_greedy_f32(logits, out, rows: int, n: int, stream=None) -> None:
 def launch_rms_norm_fp16(x, w, y, m: int, n: int, eps: float, stream=None) -> None:
     _status("rms_norm_fp16", library().logismos_launch_rms_norm_fp16(
         _ptr(x), _ptr(w), _ptr(y), m, n, eps, _raw(stream)))
+
+
+def launch_mask_additive(scores, mask, mask_len: int, rows: int, n: int, fp16: bool = False,
+                         stream=None) -> None:
+    """`cpu_f32::mask_additive_in_place` on device scores (fp32, or fp16 with fp16=True)."""
+    fn = (library().logismos_launch_mask_additive_fp16 if fp16
+          else library().logismos_launch_mask_additive_f32)
+    _status("mask_additive", fn(_ptr(scores) if scores is not None else None,
+                                _ptr(mask) if mask is not None else None, mask_len, rows, n,
+                                _raw(stream)))
 
 
 def launch_softmax_fp16(x, y, m: int, n: int, stream=None) -> None:

@@ -158,3 +158,74 @@ def test_shape_guards_reject_before_any_launch():
         with pytest.raises(kernels.LaunchError) as e:
             kernels.launch_rope_fp16_in_place(buf, buf, *shape)
         assert e.value.code == 1
+
+
+@pytest.mark.parametrize("rows,n,mask_rows", [(12, 37, 3), (8, 128, 8), (6, 5, 1), (64, 1000, 2)])
+@pytest.mark.parametrize("fp16", [False, True])
+def test_mask_additive_matches_the_reference_function(rows, n, mask_rows, fp16):
+    """`cpu_f32::mask_additive_in_place` (crates/kernels/src/cpu_f32/mod.rs:451-486): one mask
+    row serves rows / mask_rows CONSECUTIVE score rows; bit for bit (the op only writes -inf)"""
+    from logismos_amd import hip, kernels
+    rng = np.random.default_rng(rows * 1000 + n)
+    scores = rng.standard_normal((rows, n)).astype(np.float32)
+    mask = (rng.random((mask_rows, n)) < 0.6).astype(np.uint8)
+    mask[0, :] = 0  # a mask row that hides every key
+    want = scores.copy()
+    O.mask_additive_in_place(want, mask, rows, n)
+    dt = np.float16 if fp16 else np.float32
+    d_s = _dev(scores.astype(dt))
+    kernels.launch_mask_additive(d_s, _dev(mask), mask.size, rows, n, fp16=fp16)
+    hip.synchronize()
+    got = d_s.to_numpy(dt, (rows, n))
+    want = want.astype(dt)  # (fp16: rounding the unmasked scores commutes with masking)
+    assert np.array_equal(got.view(np.uint16 if fp16 else np.uint32),
+                          want.view(np.uint16 if fp16 else np.uint32))
+    repeat = rows // mask_rows
+    assert np.isneginf(got[:repeat]).all()
+    if mask_rows > 1:
+        assert not np.isneginf(got[repeat:]).all()
+
+
+def test_mask_additive_edge_cases_of_the_reference():
+    """nothing to do without columns, rows or a mask (`:452-454, 459-461`); a row count the mask
+    rows do not divide is refused where the reference panics (`:462-465`)"""
+    from logismos_amd import hip, kernels
+    scores = np.arange(12, dtype=np.float32).reshape(3, 4)
+    d_s = _dev(scores)
+    mask = np.zeros(8, np.uint8)
+    for mask_len, rows, n in ((8, 3, 0), (8, 0, 4), (0, 3, 4), (3, 3, 4)):
+        kernels.launch_mask_additive(d_s, _dev(mask), mask_len, rows, n)
+    hip.synchronize()
+    assert np.array_equal(d_s.to_numpy(np.float32, (3, 4)), scores)
+    with pytest.raises(kernels.LaunchError):
+        kernels.launch_mask_additive(d_s, _dev(mask), 8, 3, 4)   # 3 rows, 2 mask rows
+    with pytest.raises(kernels.LaunchError):
+        kernels.launch_mask_additive(d_s, _dev(mask), 7, 4, 4)   # not whole mask rows
+    hip.synchronize()
+    assert np.array_equal(d_s.to_numpy(np.float32, (3, 4)), scores)
+
+
+def test_masked_scores_through_the_softmax_launcher():
+    """the unfused attention of a padded batch: fp16 scores, key-padding mask, softmax; a query
+    whose keys are all padding attends uniformly (crates/kernels/src/cpu_f32/mod.rs:395-416)"""
+    from logismos_amd import hip, kernels
+    rng = np.random.default_rng(99)
+    heads, seq, n = 4, 3, 8
+    scores = rng.standard_normal((2 * heads * seq, n)).astype(np.float16)
+    mask = np.ones((2, n), np.uint8)
+    mask[0, 5:] = 0     # batch row 0: keys 5.. are padding
+    mask[1, :] = 0      # batch row 1: nothing but padding
+    d_s = _dev(scores)
+    kernels.launch_mask_additive(d_s, _dev(mask), mask.size, scores.shape[0], n, fp16=True)
+    d_p = hip.DeviceBuffer(scores.size * 2)
+    kernels.launch_softmax_fp16(d_s, d_p, scores.shape[0], n)
+    hip.synchronize()
+    p = d_p.to_numpy(np.float16, scores.shape).astype(np.float32)
+    half = heads * seq
+    assert (p[:half, 5:] == 0).all() and np.allclose(p[:half, :5].sum(axis=1), 1.0, atol=2e-3)
+    assert (p[half:] == 0.125).all()
+    masked = scores.astype(np.float32)
+    O.mask_additive_in_place(masked, mask, scores.shape[0], n)
+    assert np.array_equal(p.astype(np.float16).view(np.uint16),
+                          O.softmax_fp16_ref(masked.astype(np.float16), scores.shape[0], n)
+                          .view(np.uint16).reshape(p.shape))
