@@ -338,6 +338,15 @@ def bench_mixed_config4(args):
     sub = lambda m: {**case, "new_tokens": case["new_tokens"][m],  # noqa: E731
                      "context_lens": case["context_lens"][m]}
     flops_pre = workloads.paged_attn_flops(sub(~is_dec))
+    # HBM bytes of the prefill kernel: the committed counter summary, if it was taken at this
+    # workload's byte count (every K/V row of the chunk sequences once, q in, out out)
+    pre_ctx = case["context_lens"][~is_dec].astype(np.int64)
+    pre_new = case["new_tokens"][~is_dec].astype(np.int64)
+    pre_bytes = int(pre_ctx.sum()) * 2 * row * 2 + 2 * int(pre_new.sum()) * case["hq"] * 128 * 2
+    prefill_traffic = measured_traffic("paged_attn_prefill_config4_pmc.txt")
+    if measured_traffic("paged_attn_prefill_config4_pmc.txt",
+                        "algorithmic_bytes_per_launch:") != pre_bytes:
+        prefill_traffic = None
     ctx_dec = case["context_lens"][is_dec].astype(np.int64)
     dec_bytes = int(ctx_dec.sum()) * 2 * row * 2
     return {
@@ -355,7 +364,7 @@ def bench_mixed_config4(args):
         "roofline": {"bound": "mfma", "achieved": round(flops_pre / (ms_pre * 1e-3) / 1e12, 1),
                      "peak": 2500.0, "unit": "TFLOP/s",
                      "frac": round(flops_pre / (ms_pre * 1e-3) / 1e12 / 2500.0, 4),
-                     "traffic": None, "kernel": "paged_attn_prefill_kernel<4>",
+                     "traffic": prefill_traffic, "kernel": "paged_attn_prefill_kernel<4>",
                      "flops_per_launch": flops_pre,
                      **against_mfma_ceiling(stream, False,
                                             flops_pre / (ms_pre * 1e-3) / 1e12)},
