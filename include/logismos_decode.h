@@ -691,9 +691,16 @@ typedef struct {
      * a time, every pass streaming the layer's weights once; from 97 rows on every projection
      * is one launch of the tiled matrix-core GEMM over all rows (`linear_t` over `seq` rows,
      * crates/transformers/src/mlp.rs:104-111).  The attention takes the whole ragged batch in
-     * one launch either way.  token_ids / lm_head need total_tokens <= 32. */
+     * one launch either way.  token_ids takes any number of rows; lm_head, as described
+     * above (a token for every packed row), needs total_tokens <= 32. */
     int total_tokens;
     int max_seqlen_q;
+    /* != 0, with lm_head: the vocabulary projection and the token choice are made for the LAST
+     * packed row of every sequence only (row cu_seqlens[s + 1] - 1: the row whose choice is the
+     * sequence's next token; every sequence must have a new token), for any total_tokens.
+     * out_tokens_u32 and logits_f32 then have num_seqs rows, in sequence order.  out_bf16 may
+     * still be given (all packed rows) or NULL. */
+    int tokens_for_last_rows;
 } logismos_decode_batch_t;
 
 size_t logismos_decode_step_workspace_bytes(const logismos_decode_config_t* cfg, int num_seqs,

@@ -36,6 +36,11 @@ struct Workspace {
     char* t_gu;    // f32  [T][2*inter]
     char* t_act;   // bf16 [T][inter]
     char* t_gemm;  // workspace of the tiled GEMM (its copy of x in unpack order + group sums)
+    // tokens for the last row of every sequence (vocab > 0)
+    char* norm_out;   // bf16 [T][hidden]: the normed rows when the caller takes none (chunked
+                      // steps; a many-row step has t_xn free by then)
+    char* last_rows;  // bf16 [num_seqs][hidden]: the normed last rows, gathered
+    char* last_xn;    // prepared activations of one chunk of them
     bool tall;
     size_t xn_stride;
     int chunks, rows;  // rows: rows of a full chunk (= T when there is one chunk)
@@ -70,6 +75,12 @@ Workspace carve(const logismos_decode_config_t& c, int num_seqs, int t, int num_
         const int kmax = c.intermediate > (int)qd ? (c.intermediate > c.hidden ? c.intermediate : c.hidden)
                                                   : ((int)qd > c.hidden ? (int)qd : c.hidden);
         w.t_gemm = take(logismos_qgemm_q4g128_tall_workspace_bytes(t, kmax));
+        if (c.vocab > 0) {
+            w.last_rows = take((size_t)num_seqs * c.hidden * 2);
+            w.last_xn = take(logismos_q4_xprep_bytes(kChunkRows, c.hidden));
+            w.head_ws =
+                take(logismos_qgemm_q4g128_greedy_workspace_bytes(kChunkRows, c.vocab, c.hidden));
+        }
         w.total = off;
         return w;
     }
@@ -101,9 +112,13 @@ Workspace carve(const logismos_decode_config_t& c, int num_seqs, int t, int num_
     w.act = take(logismos_q4_xprep_bytes(b, c.intermediate));
     w.attn_ws =
         take(logismos_paged_attn_workspace_bytes(num_seqs, c.num_q_heads, c.head_dim, num_splits));
-    w.head_ws = c.vocab > 0
-                    ? take(logismos_qgemm_q4g128_greedy_workspace_bytes(b, c.vocab, c.hidden))
-                    : nullptr;
+    if (c.vocab > 0) {
+        const int hb = num_seqs < kChunkRows ? (b > num_seqs ? b : num_seqs) : kChunkRows;
+        w.head_ws = take(logismos_qgemm_q4g128_greedy_workspace_bytes(hb, c.vocab, c.hidden));
+        w.norm_out = take((size_t)t * c.hidden * 2);
+        w.last_rows = take((size_t)num_seqs * c.hidden * 2);
+        w.last_xn = take(logismos_q4_xprep_bytes(kChunkRows, c.hidden));
+    }
     w.total = off;
     return w;
 }
@@ -134,10 +149,15 @@ bool config_ok(const logismos_decode_config_t* c, int num_seqs, int t, int max_s
         (int64_t)t * c->hidden > (int64_t)INT32_MAX)
         return false;
     if (c->vocab < 0) return false;
-    // tokens in / tokens out is a decode-step feature: one chunk
-    if (c->vocab > 0 && t <= kChunkRows &&
-        logismos_check_qgemm_q4g128_greedy_shape(t, c->vocab, c->hidden, nullptr, 0))
-        return false;
+    // tokens out: the vocabulary projection takes one chunk of rows at a time -- all packed
+    // rows of a step of up to 32, or the sequences' last rows 32 at a time
+    if (c->vocab > 0) {
+        const int full = num_seqs < kChunkRows ? num_seqs : kChunkRows;
+        const int rest = num_seqs % kChunkRows;
+        for (const int rows : {t <= kChunkRows ? t : full, full, rest ? rest : full})
+            if (logismos_check_qgemm_q4g128_greedy_shape(rows, c->vocab, c->hidden, nullptr, 0))
+                return false;
+    }
     const int b = t < kChunkRows ? t : kChunkRows;
     const int qd = c->num_q_heads * c->head_dim;
     const int kvd = c->num_kv_heads * c->head_dim;
@@ -208,14 +228,37 @@ extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_c
     if (tokens_in && !batch->embed_table_bf16) return hipErrorInvalidValue;
     if (tokens_out && !batch->out_tokens_u32) return hipErrorInvalidValue;
     if (!tokens_out && !batch->out_bf16) return hipErrorInvalidValue;
-    // the vocabulary projection with its token choice takes one chunk of rows
-    if (tokens_out && t > kChunkRows) return hipErrorInvalidValue;
+    const bool last_only = tokens_out && batch->tokens_for_last_rows != 0;
+    // the vocabulary projection with its token choice takes one chunk of rows: every packed
+    // row of a step of up to 32, or (tokens_for_last_rows) the last row of every sequence
+    if (tokens_out && !last_only && t > kChunkRows) return hipErrorInvalidValue;
     const Workspace w = carve(c, num_seqs, t, batch->num_splits, static_cast<char*>(workspace));
     const int qd = c.num_q_heads * c.head_dim;
     const int kvd = c.num_kv_heads * c.head_dim;
     const int width = qd + 2 * kvd;
     const float scale = 1.0f / sqrtf((float)c.head_dim);
     const bool one_chunk = w.chunks == 1;
+    // tokens for last rows: the normed rows of the whole batch, in the caller's buffer or in
+    // the workspace, are gathered afterwards
+    char* const norm_dst = batch->out_bf16 ? static_cast<char*>(batch->out_bf16)
+                                           : (w.tall ? w.t_xn : w.norm_out);
+    auto project_last_rows = [&]() -> logismos_status_t {
+        LG_TRY(lg::gather_last_rows_bf16_launch(norm_dst, batch->cu_seqlens, w.last_rows, num_seqs,
+                                                c.hidden, static_cast<hipStream_t>(stream)));
+        const logismos_q4_weight_t& H = *batch->lm_head;
+        for (int s0 = 0; s0 < num_seqs; s0 += kChunkRows) {
+            const int rows = num_seqs - s0 < kChunkRows ? num_seqs - s0 : kChunkRows;
+            LG_TRY(logismos_launch_q4_prepare_x_bf16(w.last_rows + (size_t)s0 * c.hidden * 2,
+                                                     w.last_xn, rows, c.hidden, stream));
+            LG_TRY(logismos_launch_qgemm_q4g128_greedy_xprep(
+                w.last_xn, H.qw, H.scale, H.zero,
+                static_cast<uint32_t*>(batch->out_tokens_u32) + s0,
+                batch->logits_f32 ? static_cast<float*>(batch->logits_f32) + (size_t)s0 * c.vocab
+                                  : nullptr,
+                w.head_ws, rows, c.vocab, c.hidden, stream));
+        }
+        return 0;
+    };
     // attention writes the o projection's input (the prepared layout's groups of 128 are whole
     // heads only at head_dim 128)
     const bool direct = one_chunk && max_q == 1 && c.head_dim == 128;
@@ -269,9 +312,10 @@ extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_c
             LG_TRY(gemm(w.t_act, L.down, nullptr, w.t_proj, c.hidden, c.intermediate));
             res_parts = 1;
         }
-        return logismos_launch_add_rms_norm_f32p(batch->hidden_f32, w.t_proj, res_parts,
-                                                 batch->final_norm_w_f32, batch->out_bf16, t,
-                                                 c.hidden, c.rms_eps, stream);
+        LG_TRY(logismos_launch_add_rms_norm_f32p(batch->hidden_f32, w.t_proj, res_parts,
+                                                 batch->final_norm_w_f32, norm_dst, t, c.hidden,
+                                                 c.rms_eps, stream));
+        return last_only ? project_last_rows() : 0;
     }
     // The normed input of a layer's first half is produced where the residual stream is
     // completed: before layer 0 here, afterwards by the add + norm that folds a chunk's down
@@ -341,14 +385,19 @@ extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_c
                 // last layer of a multi-chunk step: the final norm of this chunk's rows
                 LG_TRY(logismos_launch_add_rms_norm_f32p(
                     hc, w.proj, j_down, batch->final_norm_w_f32,
-                    static_cast<char*>(batch->out_bf16) + (size_t)r0 * c.hidden * 2, rows, c.hidden,
-                    c.rms_eps, stream));
+                    norm_dst + (size_t)r0 * c.hidden * 2, rows, c.hidden, c.rms_eps, stream));
             } else {
                 res_parts = j_down;
             }
         }
     }
-    if (!one_chunk) return 0;
+    if (!one_chunk) return last_only ? project_last_rows() : 0;
+    if (last_only) {
+        LG_TRY(logismos_launch_add_rms_norm_f32p(batch->hidden_f32, w.proj, res_parts,
+                                                 batch->final_norm_w_f32, norm_dst, t, c.hidden,
+                                                 c.rms_eps, stream));
+        return project_last_rows();
+    }
     if (tokens_out) {
         // the normed state in the layout of the vocabulary projection, then the projection
         // with the token choice fused into it

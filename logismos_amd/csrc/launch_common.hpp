@@ -70,4 +70,10 @@ hipError_t qgemm_q4_tall_f32_launch(const void* x_bf16, const void* qw, const vo
                                     const void* zero, const float* bias, void* y_f32, int b,
                                     int n, int k, hipStream_t stream);
 
+// dst[s][:] = src[cu_seqlens[s + 1] - 1][:], bf16 rows of `hidden` elements (step_ops.hip): the
+// last packed row of every sequence of a ragged batch.
+hipError_t gather_last_rows_bf16_launch(const void* src_bf16, const int32_t* cu_seqlens,
+                                        void* dst_bf16, int num_seqs, int hidden,
+                                        hipStream_t stream);
+
 }  // namespace lg

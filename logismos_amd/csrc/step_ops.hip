@@ -379,6 +379,19 @@ __global__ __launch_bounds__(256) void cast_f16_bf16_kernel(const __half* __rest
     if (idx < total) out[idx] = f32_to_bf16(__half2float(in[idx]));
 }
 
+// dst[s][:] = src[cu_seqlens[s + 1] - 1][:]: the last packed row of every sequence (bf16 rows
+// of `hidden` elements, hidden % 8 == 0).  One workgroup per sequence.  A sequence without new
+// tokens takes the row before its position (row 0 for the first): what it gets is not used.
+__global__ __launch_bounds__(256) void gather_last_rows_bf16_kernel(
+    const uint4_t* __restrict__ src, const int32_t* __restrict__ cu_seqlens,
+    uint4_t* __restrict__ dst, int chunks) {
+    const int s = blockIdx.x;
+    const int last = cu_seqlens[s + 1] - 1;
+    const int64_t row = last > 0 ? last : 0;
+    for (int i = threadIdx.x; i < chunks; i += 256)
+        dst[(int64_t)s * chunks + i] = src[row * chunks + i];
+}
+
 // One workgroup per row: first index of the maximum (strict >, ties keep the lower index).
 __global__ __launch_bounds__(256) void greedy_kernel(const float* __restrict__ logits,
                                                      uint32_t* __restrict__ out, int n) {
@@ -609,6 +622,19 @@ extern "C" logismos_status_t logismos_launch_cast_f16_bf16(const void* in_f16, v
         static_cast<const __half*>(in_f16), static_cast<uint16_t*>(out_bf16), (int64_t)count);
     return hipGetLastError();
 }
+
+namespace lg {
+hipError_t gather_last_rows_bf16_launch(const void* src_bf16, const int32_t* cu_seqlens,
+                                        void* dst_bf16, int num_seqs, int hidden,
+                                        hipStream_t stream) {
+    if (num_seqs <= 0 || hidden <= 0 || (hidden & 7) || !src_bf16 || !cu_seqlens || !dst_bf16)
+        return hipErrorInvalidValue;
+    gather_last_rows_bf16_kernel<<<dim3(num_seqs), dim3(256), 0, stream>>>(
+        static_cast<const uint4_t*>(src_bf16), cu_seqlens, static_cast<uint4_t*>(dst_bf16),
+        hidden / 8);
+    return hipGetLastError();
+}
+}  // namespace lg
 
 extern "C" logismos_status_t logismos_launch_greedy_f32(const void* logits_f32, void* out_u32,
                                                         int rows, int n,

@@ -179,7 +179,7 @@ class DecodeBatch(C.Structure):
                 ("rope_sin_f32", _vp), ("num_seqs", _i), ("num_splits", _i),
                 ("token_ids", _vp), ("embed_table_bf16", _vp), ("lm_head", C.POINTER(Q4Weight)),
                 ("out_tokens_u32", _vp), ("logits_f32", _vp), ("total_tokens", _i),
-                ("max_seqlen_q", _i)]
+                ("max_seqlen_q", _i), ("tokens_for_last_rows", _i)]
 
 
 def library() -> C.CDLL:

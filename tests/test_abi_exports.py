@@ -31,7 +31,7 @@ def test_binding_covers_exactly_the_header():
 
 def test_identity():
     lib = kernels.library()
-    assert lib.logismos_decode_abi_version() == 4
+    assert lib.logismos_decode_abi_version() == 5
     assert lib.logismos_decode_offload_arch() == b"gfx950"
 
 
