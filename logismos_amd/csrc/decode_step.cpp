@@ -149,15 +149,10 @@ bool config_ok(const logismos_decode_config_t* c, int num_seqs, int t, int max_s
         (int64_t)t * c->hidden > (int64_t)INT32_MAX)
         return false;
     if (c->vocab < 0) return false;
-    // tokens out: the vocabulary projection takes one chunk of rows at a time -- all packed
-    // rows of a step of up to 32, or the sequences' last rows 32 at a time
-    if (c->vocab > 0) {
-        const int full = num_seqs < kChunkRows ? num_seqs : kChunkRows;
-        const int rest = num_seqs % kChunkRows;
-        for (const int rows : {t <= kChunkRows ? t : full, full, rest ? rest : full})
-            if (logismos_check_qgemm_q4g128_greedy_shape(rows, c->vocab, c->hidden, nullptr, 0))
-                return false;
-    }
+    // tokens in / tokens out for every packed row is a decode-step feature: one chunk
+    if (c->vocab > 0 && t <= kChunkRows &&
+        logismos_check_qgemm_q4g128_greedy_shape(t, c->vocab, c->hidden, nullptr, 0))
+        return false;
     const int b = t < kChunkRows ? t : kChunkRows;
     const int qd = c->num_q_heads * c->head_dim;
     const int kvd = c->num_kv_heads * c->head_dim;
@@ -229,6 +224,14 @@ extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_c
     if (tokens_out && !batch->out_tokens_u32) return hipErrorInvalidValue;
     if (!tokens_out && !batch->out_bf16) return hipErrorInvalidValue;
     const bool last_only = tokens_out && batch->tokens_for_last_rows != 0;
+    if (last_only) {
+        // the sequences' last rows go through the vocabulary projection 32 at a time
+        const int full = num_seqs < kChunkRows ? num_seqs : kChunkRows;
+        const int rest = num_seqs % kChunkRows;
+        for (const int rows : {full, rest ? rest : full})
+            if (logismos_check_qgemm_q4g128_greedy_shape(rows, c.vocab, c.hidden, nullptr, 0))
+                return hipErrorInvalidValue;
+    }
     // the vocabulary projection with its token choice takes one chunk of rows: every packed
     // row of a step of up to 32, or (tokens_for_last_rows) the last row of every sequence
     if (tokens_out && !last_only && t > kChunkRows) return hipErrorInvalidValue;
