@@ -26,6 +26,14 @@
 //   operand is one weight row and one dword of nibbles, made bf16 `128 + q` with an and-or per
 //   pair, exact), one multiply-add per result for the group's scale, 32 MFMAs.
 //
+// * workgroups all take the same time and a CU holds one, so a launch whose tile count is not
+//   a multiple of the CU count ends on a round that leaves most CUs idle (config 4's o and
+//   down projections: 1040 tiles on 256 CUs, a fifth round for 16 tiles).  The tiles of that
+//   last partial round are split over K into parts, one workgroup each, that write fp32
+//   partial tiles into the workspace; `q4_tall_reduce_kernel` sums a tile's parts in part
+//   order (deterministic), adds the bias and writes y.  A launch of fewer tiles than CUs is
+//   all "last round": the split also fills the device at a few hundred rows.
+//
 // LDS is only touched through inline assembly inside the loop: the compiler would order
 // every LDS access it can see behind all outstanding global_load_lds.
 #include "device_utils.hpp"
@@ -46,9 +54,32 @@ constexpr int kTpWBytes = 256 * 64;       // one group's tile of weights: 256 ro
 constexpr int kTpBufBytes = kTpSlabBytes + kTpWBytes;
 constexpr int kTpBufs = 3;                // groups in LDS: one in use, two on their way
 
+constexpr int kTpTileElems = kTpTileM * kTpTileN;
+constexpr int kTpMaxParts = 512;          // partial tiles the workspace holds (fp32, 128 KiB each)
+constexpr int kTpMinPairsPerPart = 2;     // a part takes at least four groups of 128 columns
+
 __host__ __device__ inline int tp_padded_rows(int m) { return (m + kTpTileM - 1) / kTpTileM * kTpTileM; }
 __host__ __device__ inline size_t tp_sums_offset(int m, int k) {
     return ((size_t)tp_padded_rows(m) * k * 2 + 255) & ~(size_t)255;
+}
+__host__ __device__ inline size_t tp_partials_offset(int m, int k) {
+    return (tp_sums_offset(m, k) + (size_t)tp_padded_rows(m) * (k / 128) * 4 + 255) & ~(size_t)255;
+}
+
+// How a launch of `tiles` workgroup tiles is laid over `cus` CUs: the first `full` tiles whole,
+// the other `tiles - full` (the last, partial round) in `split` parts over K each.
+struct TpPlan {
+    int full, split;
+};
+inline TpPlan tp_plan(int tiles, int groups, int cus) {
+    const int rem = tiles % cus;
+    TpPlan p{tiles, 1};
+    if (rem == 0) return p;
+    int split = cus / rem;
+    const int most = (groups / 2) / kTpMinPairsPerPart;
+    if (split > most) split = most;
+    if (split > 1 && rem * split <= kTpMaxParts) p = TpPlan{tiles - rem, split};
+    return p;
 }
 
 // x [m][k] bf16 -> xp [m_pad][k] bf16 in pair order (rows >= m: zeros), xs [m_pad][k/128] fp32
@@ -74,18 +105,31 @@ template <bool F32OUT>
 __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
     const uint16_t* __restrict__ xp, const float* __restrict__ xs, const uint8_t* __restrict__ qw,
     const __half* __restrict__ scale, const __half* __restrict__ zero,
-    const float* __restrict__ bias, void* __restrict__ y_out, int m, int n, int k) {
+    const float* __restrict__ bias, void* __restrict__ y_out, float* __restrict__ partials, int m,
+    int n, int k, int tiles_n, int full_tiles, int split) {
     extern __shared__ uint4_t tp_lds[];  // kTpBufs x {slab of x, tile of weights}
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 31;
     const int h = lane >> 5;
-    const int row0 = blockIdx.y * kTpTileM;
-    const int col0 = blockIdx.x * kTpTileN;
+    // workgroup -> tile (columns fastest) and, past the whole tiles, part of a tile: groups
+    // [g_begin, groups) of K, both even
+    int tile = blockIdx.x, part = -1;
+    int g_begin = 0, groups = k >> 7;
+    if (tile >= full_tiles) {
+        const int p = tile - full_tiles;
+        tile = full_tiles + p / split;
+        part = p;
+        const int pairs = groups >> 1, q = p % split;
+        g_begin = 2 * (int)((int64_t)pairs * q / split);
+        groups = 2 * (int)((int64_t)pairs * (q + 1) / split);
+    }
+    const int row0 = (tile / tiles_n) * kTpTileM;
+    const int col0 = (tile % tiles_n) * kTpTileN;
     const int wr = (wave >> 2) * 64;  // this wave's 64 x 64 part of the 128 x 256 tile
     const int wc = (wave & 3) * 64;
-    const int groups = k >> 7;
+    const int groups_row = k >> 7;    // scales, zeros, sums: groups per row
 
     unsigned magic;
     asm volatile("v_mov_b32 %0, 0x43004300" : "=v"(magic));
@@ -142,27 +186,44 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
         b_addr[t] = lds_base + kTpSlabBytes + (unsigned)(wc + r) * 64u +
                     (unsigned)((2 * h + t) ^ ((r >> 2) & 3)) * 16u;
 
-    // scales and zeros of a pair of groups g, g + 1 (g even) in one dword each, from global
-    // memory into registers (a lane's 16 results of a tile belong to one weight row)
-    unsigned soff[2];
+    // Scales and zeros of a pair of groups g, g + 1 (g even) in one dword each, from global
+    // memory into registers (a lane's 16 results of a tile belong to one weight row), and the
+    // group sums of x for the zero-point product: lane (r, h) holds row wr + 32 i + r, group
+    // g + h of the pair.  Six loads per pair and wave, written as assembly with the waits for
+    // them spelled out below: for loads it can see the compiler waits with vmcnt(0), which
+    // also waits for every request of the groups ahead and takes the ring's depth away.
+    // A register loaded here must not be touched before `small_loads_landed` has named it.
+    unsigned soff[2], xsoff[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j)
-        soff[j] = (unsigned)min(col0 + wc + 32 * j + r, n - 1) * (unsigned)groups;
+        soff[j] = (unsigned)min(col0 + wc + 32 * j + r, n - 1) * (unsigned)groups_row * 2u;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+        xsoff[i] = ((unsigned)(row0 + wr + 32 * i + r) * (unsigned)groups_row + (unsigned)h) * 4u;
+    constexpr int kSmall = 6;  // small loads per pair and wave
     unsigned scur[2], zcur[2], snext[2], znext[2];
-    auto gload_sz = [&](int g, unsigned (&sv)[2], unsigned (&zv)[2]) {
+    float xsum[2], xsum_next[2];
+    auto gload_small = [&](int g, unsigned (&sv)[2], unsigned (&zv)[2], float (&xv)[2]) {
+        const __half* sb = scale + g;
+        const __half* zb = zero + g;
+        const float* xb = xs + g;
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            __builtin_memcpy(&sv[j], scale + soff[j] + (unsigned)g, 4);
-            __builtin_memcpy(&zv[j], zero + soff[j] + (unsigned)g, 4);
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(sv[j]) : "v"(soff[j]), "s"(sb) : "memory");
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(zv[j]) : "v"(soff[j]), "s"(zb) : "memory");
         }
-    };
-    // group sums of x for the zero-point product: lane (r, h) holds row wr + 32 i + r, group
-    // g + h of the pair
-    float xsum[2], xsum_next[2];
-    auto gload_xs = [&](int g, float (&v)[2]) {
 #pragma unroll
         for (int i = 0; i < 2; ++i)
-            v[i] = xs[(size_t)(row0 + wr + 32 * i + r) * groups + g + h];
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(xv[i]) : "v"(xsoff[i]), "s"(xb) : "memory");
+    };
+    // waits until at most `younger` of this wave's loads and requests are outstanding (they
+    // complete in the order they were issued) and hands the six registers over
+    auto small_loads_landed = [&](auto younger_c, unsigned (&sv)[2], unsigned (&zv)[2],
+                                  float (&xv)[2]) {
+        asm volatile("s_waitcnt vmcnt(%6)"
+                     : "+v"(sv[0]), "+v"(sv[1]), "+v"(zv[0]), "+v"(zv[1]), "+v"(xv[0]), "+v"(xv[1])
+                     : "n"(decltype(younger_c)::value)
+                     : "memory");
     };
 
     float16_t yacc[2][2];
@@ -173,10 +234,10 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
 #pragma unroll
             for (int e = 0; e < 16; ++e) yacc[i][j][e] = 0.0f;
 
-    gload_sz(0, scur, zcur);
-    gload_xs(0, xsum);
-    request_group(0, 0);
-    if (groups > 1) request_group(1, 1);
+    gload_small(g_begin, scur, zcur, xsum);
+    request_group(g_begin, 0);
+    request_group(g_begin + 1, 1);  // (a range holds at least one pair)
+    small_loads_landed(ic<2 * kReq>{}, scur, zcur, xsum);
 
     // One group of 128 columns out of buffer BUF (immediates in the LDS reads); PAR: the
     // group's place in its pair.  A wave's requests complete in the order they were issued,
@@ -190,17 +251,9 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
         // after the barrier everybody's requests for this group have landed, and everybody is
         // done reading the buffer of the group before it, which the group after next reuses
         __builtin_amdgcn_s_barrier();
-        if (g + 2 < groups) {
-            // (the small loads first: what waits for them need not wait for the requests)
-            if (PAR == 1) {
-                gload_sz(g + 1, snext, znext);
-                gload_xs(g + 1, xsum_next);
-            }
-            request_group(g + 2, (BUF + 2) % kTpBufs);
-        } else if (PAR == 1 && g + 1 < groups) {
-            gload_sz(g + 1, snext, znext);
-            gload_xs(g + 1, xsum_next);
-        }
+        // (the small loads first: what waits for them need not wait for the requests)
+        if (PAR == 1 && g + 1 < groups) gload_small(g + 1, snext, znext, xsum_next);
+        if (g + 2 < groups) request_group(g + 2, (BUF + 2) % kTpBufs);
         float16_t acc[2][2];
         bf16x8_t av[2][2];  // [step parity][i]
         bf16x8_t bv[2][2];  // [step parity][j]
@@ -308,6 +361,8 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
                     yacc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xsum[i], cv[j], yacc[i][j], 0,
                                                                       0, 0);
             if (g + 1 < groups) {
+                if (g + 2 < groups) small_loads_landed(ic<kReq>{}, snext, znext, xsum_next);
+                else small_loads_landed(ic<0>{}, snext, znext, xsum_next);
 #pragma unroll
                 for (int j = 0; j < 2; ++j) scur[j] = snext[j], zcur[j] = znext[j];
 #pragma unroll
@@ -316,13 +371,24 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
         }
     };
     // groups is even (checked on the host); buffers go round in threes, pairs in twos
-    for (int g0 = 0; g0 < groups; g0 += 6) {
+    for (int g0 = g_begin; g0 < groups; g0 += 6) {
         static_for<6>([&](auto uc) {
             constexpr int u = decltype(uc)::value;
             if (g0 + u < groups) group(ic<u % kTpBufs>{}, ic<(u & 1)>{}, g0 + u);
         });
     }
 
+    if (part >= 0) {
+        // a part of a tile: the wave's 64 x 64 results as they lie in registers, lane fastest
+        float* dst = partials + (size_t)part * kTpTileElems + (size_t)wave * 4096 + lane;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) dst[((i * 2 + j) * 16 + e) * 64] = yacc[i][j][e];
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const int gn = col0 + wc + 32 * j + r;
@@ -344,6 +410,57 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
     }
 }
 
+// Sums the `split` fp32 parts of each tile of the last round, in part order, adds the bias and
+// writes y.  One thread per result; a part's element index is (wave, i, j, e, lane) as the
+// product kernel left it.
+template <bool F32OUT>
+__global__ __launch_bounds__(256) void q4_tall_reduce_kernel(const float* __restrict__ partials,
+                                                            const float* __restrict__ bias,
+                                                            void* __restrict__ y_out, int m, int n,
+                                                            int tiles_n, int full_tiles,
+                                                            int split) {
+    const int t = blockIdx.x / (kTpTileElems / 256);
+    const int idx = (blockIdx.x % (kTpTileElems / 256)) * 256 + threadIdx.x;
+    const int lane = idx & 63, e = (idx >> 6) & 15, j = (idx >> 10) & 1, i = (idx >> 11) & 1;
+    const int wave = idx >> 12;
+    const int tile = full_tiles + t;
+    const int gr = (tile / tiles_n) * kTpTileM + (wave >> 2) * 64 + 32 * i + 8 * (e >> 2) +
+                   4 * (lane >> 5) + (e & 3);
+    const int gn = (tile % tiles_n) * kTpTileN + (wave & 3) * 64 + 32 * j + (lane & 31);
+    if (gr >= m || gn >= n) return;
+    const float* src = partials + (size_t)t * split * kTpTileElems + idx;
+    float acc = 0.0f;
+    for (int q = 0; q < split; ++q) acc += src[(size_t)q * kTpTileElems];
+    if (bias) acc += bias[gn];
+    if constexpr (F32OUT) static_cast<float*>(y_out)[(int64_t)gr * n + gn] = acc;
+    else static_cast<uint16_t*>(y_out)[(int64_t)gr * n + gn] = f32_to_bf16_rne(acc);
+}
+
+template <bool F32OUT>
+static hipError_t tallp_launch(const uint16_t* xp, const float* xs, float* partials,
+                               const uint8_t* qw, const __half* scale, const __half* zero,
+                               const float* bias, void* y, int m, int n, int k, hipStream_t st) {
+    constexpr size_t lds = (size_t)kTpBufs * kTpBufBytes;
+    static const hipError_t opt = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(qgemm_q4g128_tallp_kernel<F32OUT>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (opt != hipSuccess) return opt;
+    const int tiles_n = (n + kTpTileN - 1) / kTpTileN;
+    const int tiles = tiles_n * (tp_padded_rows(m) / kTpTileM);
+    const int cus = device_cu_count();
+    if (cus <= 0) return hipErrorInvalidDevice;
+    const TpPlan plan = tp_plan(tiles, k >> 7, cus);
+    const int parts = (tiles - plan.full) * plan.split;
+    qgemm_q4g128_tallp_kernel<F32OUT><<<dim3(plan.full + (plan.split > 1 ? parts : 0)), dim3(512),
+                                        lds, st>>>(xp, xs, qw, scale, zero, bias, y, partials, m,
+                                                   n, k, tiles_n, plan.full, plan.split);
+    if (plan.split > 1)
+        q4_tall_reduce_kernel<F32OUT>
+            <<<dim3((tiles - plan.full) * (kTpTileElems / 256)), dim3(256), 0, st>>>(
+                partials, bias, y, m, n, tiles_n, plan.full, plan.split);
+    return hipGetLastError();
+}
+
 }  // namespace lg
 
 extern "C" logismos_status_t logismos_check_qgemm_q4g128_tall_shape(int m, int n, int k, char* msg,
@@ -361,14 +478,12 @@ extern "C" logismos_status_t logismos_check_qgemm_q4g128_tall_shape(int m, int n
                           (long long)((int64_t)n * k));
     if ((int64_t)lg::tp_padded_rows(m) * k * 2 > lim || (int64_t)m * n > lim)
         return lg::reject(msg, msg_cap, "%s: rows*K*2 or rows*N exceeds i32::MAX", kn);
-    if ((lg::tp_padded_rows(m) / lg::kTpTileM) > 65535)
-        return lg::reject(msg, msg_cap, "%s: more than 65535 row tiles", kn);
     return 0;
 }
 
 extern "C" size_t logismos_qgemm_q4g128_tall_workspace_bytes(int m, int k) {
     if (m <= 0 || k <= 0 || k % 128 != 0) return 0;
-    return lg::tp_sums_offset(m, k) + (size_t)lg::tp_padded_rows(m) * (k / 128) * 4;
+    return lg::tp_partials_offset(m, k) + (size_t)lg::kTpMaxParts * lg::kTpTileElems * 4;
 }
 
 extern "C" logismos_status_t logismos_launch_qgemm_q4g128_tall(
@@ -391,24 +506,15 @@ extern "C" logismos_status_t logismos_launch_qgemm_q4g128_tall(
     const int64_t chunks = (int64_t)m_pad * (k / 8);
     lg::q4_tall_prepare_kernel<<<dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st>>>(
         static_cast<const uint16_t*>(x_bf16), xp, xs, m, m_pad, k);
-    const dim3 grid((n + lg::kTpTileN - 1) / lg::kTpTileN, m_pad / lg::kTpTileM);
-    constexpr size_t lds = (size_t)lg::kTpBufs * lg::kTpBufBytes;
-    if (y_is_f32) {
-        static const hipError_t opt = hipFuncSetAttribute(
-            reinterpret_cast<const void*>(lg::qgemm_q4g128_tallp_kernel<true>),
-            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (opt != hipSuccess) return opt;
-        lg::qgemm_q4g128_tallp_kernel<true><<<grid, dim3(512), lds, st>>>(
-            xp, xs, static_cast<const uint8_t*>(qw_u8), static_cast<const __half*>(scale_f16),
-            static_cast<const __half*>(zero_f16), static_cast<const float*>(bias_f32), y, m, n, k);
-    } else {
-        static const hipError_t opt = hipFuncSetAttribute(
-            reinterpret_cast<const void*>(lg::qgemm_q4g128_tallp_kernel<false>),
-            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (opt != hipSuccess) return opt;
-        lg::qgemm_q4g128_tallp_kernel<false><<<grid, dim3(512), lds, st>>>(
-            xp, xs, static_cast<const uint8_t*>(qw_u8), static_cast<const __half*>(scale_f16),
-            static_cast<const __half*>(zero_f16), static_cast<const float*>(bias_f32), y, m, n, k);
-    }
-    return hipGetLastError();
+    float* partials = reinterpret_cast<float*>(static_cast<char*>(workspace) +
+                                               lg::tp_partials_offset(m, k));
+    if (y_is_f32)
+        return lg::tallp_launch<true>(xp, xs, partials, static_cast<const uint8_t*>(qw_u8),
+                                      static_cast<const __half*>(scale_f16),
+                                      static_cast<const __half*>(zero_f16),
+                                      static_cast<const float*>(bias_f32), y, m, n, k, st);
+    return lg::tallp_launch<false>(xp, xs, partials, static_cast<const uint8_t*>(qw_u8),
+                                   static_cast<const __half*>(scale_f16),
+                                   static_cast<const __half*>(zero_f16),
+                                   static_cast<const float*>(bias_f32), y, m, n, k, st);
 }

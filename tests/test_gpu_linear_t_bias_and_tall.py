@@ -252,4 +252,6 @@ def test_q4g128_workspace_entry_point_refuses_what_it_cannot_run():
         kernels.launch_qgemm_q4g128_tall(None, None, None, None, None, None, 128, 128, 384)
     with pytest.raises(kernels.UnsupportedShape):
         kernels.launch_qgemm_q4g128_tall(None, None, None, None, None, None, 0, 128, 256)
-    assert kernels.qgemm_q4g128_tall_workspace_bytes(130, 512) == 256 * 512 * 2 + 256 * 4 * 4
+    # the copy of x, its group sums, and room for 512 fp32 partial tiles of 128 x 256
+    assert kernels.qgemm_q4g128_tall_workspace_bytes(130, 512) == (
+        256 * 512 * 2 + 256 * 4 * 4 + 512 * 128 * 256 * 4)
