@@ -56,7 +56,7 @@ constexpr int kTpBufs = 3;                // groups in LDS: one in use, two on t
 
 constexpr int kTpTileElems = kTpTileM * kTpTileN;
 constexpr int kTpMaxParts = 512;          // partial tiles the workspace holds (fp32, 128 KiB each)
-constexpr int kTpMinPairsPerPart = 2;     // a part takes at least four groups of 128 columns
+constexpr int kTpMinGroupsPerPart = 4;    // a part of a tile takes at least four groups of K
 
 __host__ __device__ inline int tp_padded_rows(int m) { return (m + kTpTileM - 1) / kTpTileM * kTpTileM; }
 __host__ __device__ inline size_t tp_sums_offset(int m, int k) {
@@ -71,24 +71,26 @@ __host__ __device__ inline size_t tp_partials_offset(int m, int k) {
 struct TpPlan {
     int full, split;
 };
-inline TpPlan tp_plan(int tiles, int groups, int cus) {
+inline TpPlan tp_plan(int tiles, int groups, int block_groups, int cus) {
     const int rem = tiles % cus;
     TpPlan p{tiles, 1};
     if (rem == 0) return p;
     int split = cus / rem;
-    const int most = (groups / 2) / kTpMinPairsPerPart;
+    // parts are whole blocks of the kernel's small loads and at least four groups
+    const int most = groups / (block_groups > kTpMinGroupsPerPart ? block_groups : kTpMinGroupsPerPart);
     if (split > most) split = most;
     if (split > 1 && rem * split <= kTpMaxParts) p = TpPlan{tiles - rem, split};
     return p;
 }
 
-// x [m][k] bf16 -> xp [m_pad][k] bf16 in pair order (rows >= m: zeros), xs [m_pad][k/128] fp32
-// sums of the bf16 values of each group.  One thread per 16-byte chunk; the 16 lanes of a row
-// of lanes hold one group of one row.
+// x [m][k] bf16 -> xp [m_pad][k] bf16 in pair order (rows >= m: zeros), xs: the fp32 sum of the
+// bf16 values of every row and group, laid out for the product kernel's loads as
+// [row tile of 128][block of w pairs of groups][group's place in its pair][row][pair].
+// One thread per 16-byte chunk; the 16 lanes of a row of lanes hold one group of one row.
 __global__ __launch_bounds__(256) void q4_tall_prepare_kernel(const uint16_t* __restrict__ x,
                                                              uint16_t* __restrict__ xp,
                                                              float* __restrict__ xs, int m,
-                                                             int m_pad, int k) {
+                                                             int m_pad, int k, int w) {
     const int64_t chunks_per_row = k >> 3;
     const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (id >= (int64_t)m_pad * chunks_per_row) return;  // (whole rows of 16 lanes: k % 128 == 0)
@@ -98,39 +100,62 @@ __global__ __launch_bounds__(256) void q4_tall_prepare_kernel(const uint16_t* __
     if (row < m) v = *reinterpret_cast<const uint4_t*>(x + row * k + c * 8);
     const float gs = row16_sum(sum8_bf16(v));
     *reinterpret_cast<uint4_t*>(xp + row * k + c * 8) = pair_order(v);
-    if ((threadIdx.x & 15) == 0) xs[row * (k >> 7) + (c >> 4)] = gs;
+    if ((threadIdx.x & 15) == 0) {
+        const int g = (int)(c >> 4), bl = 2 * w;
+        const int64_t block = (row / kTpTileM) * ((k >> 7) / bl) + g / bl;
+        const int in_block = g % bl;
+        xs[((block * 2 + (in_block & 1)) * kTpTileM + row % kTpTileM) * w + (in_block >> 1)] = gs;
+    }
 }
 
-template <bool F32OUT>
+// W values a lane loads at once, as one register operand of an assembly statement: a vector
+// of W, or the plain value for W = 1 (a vector of one is no register operand).
+template <typename T, int W>
+struct TpRegs {
+    typedef T raw_t __attribute__((ext_vector_type(W)));
+    raw_t raw;
+    __device__ __forceinline__ T operator[](int i) const { return raw[i]; }
+};
+template <typename T>
+struct TpRegs<T, 1> {
+    typedef T raw_t;
+    raw_t raw;
+    __device__ __forceinline__ T operator[](int) const { return raw; }
+};
+
+// W: pairs of groups whose scales, zeros and group sums a lane loads at once (1, 2 or 4: a
+// dword, two or four per load; K a multiple of 256 W).
+template <bool F32OUT, int W>
 __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
     const uint16_t* __restrict__ xp, const float* __restrict__ xs, const uint8_t* __restrict__ qw,
     const __half* __restrict__ scale, const __half* __restrict__ zero,
     const float* __restrict__ bias, void* __restrict__ y_out, float* __restrict__ partials, int m,
     int n, int k, int tiles_n, int full_tiles, int split) {
     extern __shared__ uint4_t tp_lds[];  // kTpBufs x {slab of x, tile of weights}
+    constexpr int BL = 2 * W;            // groups per block of small loads
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 31;
     const int h = lane >> 5;
     // workgroup -> tile (columns fastest) and, past the whole tiles, part of a tile: groups
-    // [g_begin, groups) of K, both even
+    // [g_begin, groups) of K, both multiples of BL
     int tile = blockIdx.x, part = -1;
     int g_begin = 0, groups = k >> 7;
     if (tile >= full_tiles) {
         const int p = tile - full_tiles;
         tile = full_tiles + p / split;
         part = p;
-        const int pairs = groups >> 1, q = p % split;
-        g_begin = 2 * (int)((int64_t)pairs * q / split);
-        groups = 2 * (int)((int64_t)pairs * (q + 1) / split);
+        const int blocks = groups / BL, q = p % split;
+        g_begin = BL * (int)((int64_t)blocks * q / split);
+        groups = BL * (int)((int64_t)blocks * (q + 1) / split);
     }
-    const int row0 = (tile / tiles_n) * kTpTileM;
+    const int row_tile = tile / tiles_n;
+    const int row0 = row_tile * kTpTileM;
     const int col0 = (tile % tiles_n) * kTpTileN;
     const int wr = (wave >> 2) * 64;  // this wave's 64 x 64 part of the 128 x 256 tile
     const int wc = (wave & 3) * 64;
-    const int groups_row = k >> 7;    // scales, zeros, sums: groups per row
-
+    const int groups_row = k >> 7;    // scales and zeros: groups per weight row
     unsigned magic;
     asm volatile("v_mov_b32 %0, 0x43004300" : "=v"(magic));
     const unsigned lds_base = (unsigned)(uintptr_t)(tp_lds_ptr_t)tp_lds;
@@ -156,28 +181,33 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
         const int gn = min(col0 + row, n - 1);  // a row past n re-reads the last row
         woff[q] = (unsigned)gn * (unsigned)(k >> 1) + (unsigned)piece * 16u;
     }
-    auto request_group = [&](int g, int buf) {
-        char* dst = lds_c + buf * kTpBufBytes;
+    // (as assembly: the 32-bit offsets above with a scalar base, where the builtin widens each
+    // to a 64-bit address in two more registers; M0 holds the LDS address of lane 0's 16 bytes
+    // and nothing else in this kernel uses M0)
+    auto request_group = [&](int g, int buf_off) {
         const char* xsrc = reinterpret_cast<const char*>(xp) + (size_t)g * 256;
         const char* wsrc = reinterpret_cast<const char*>(qw) + (size_t)g * 64;
+        const unsigned xdst = lds_base + (unsigned)buf_off + (unsigned)wave * 4096u;
+        const unsigned wdst = lds_base + (unsigned)buf_off + kTpSlabBytes + (unsigned)wave * 2048u;
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-            __builtin_amdgcn_global_load_lds((tp_glb_ptr_t)(xsrc + xoff[q]),
-                                             (tp_lds_ptr_t)(dst + (wave * 4 + q) * 1024), 16, 0, 0);
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                         :
+                         : "v"(xoff[q]), "s"(xsrc), "s"(xdst + q * 1024u)
+                         : "memory");
 #pragma unroll
         for (int q = 0; q < 2; ++q)
-            __builtin_amdgcn_global_load_lds(
-                (tp_glb_ptr_t)(wsrc + woff[q]),
-                (tp_lds_ptr_t)(dst + kTpSlabBytes + (wave * 2 + q) * 1024), 16, 0, 0);
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                         :
+                         : "v"(woff[q]), "s"(wsrc), "s"(wdst + q * 1024u)
+                         : "memory");
     };
     constexpr int kReq = 6;  // requests per group and wave
     // ---- A operand reads: lane (r, h) at step s8 wants chunk 8 h + s8 of row wr + 32 i + r,
     // stored at position (8 h + s8) ^ (r % 16): a0 ^ (s8 << 4), the i-tile as an immediate
+    // (a buffer's offset in the ring is a multiple of 16 KiB: adding it commutes with the XOR)
     const unsigned a0 = lds_base + (unsigned)(wr + r) * 256u +
                         (unsigned)(((8 * h) ^ (r & 8)) | (r & 7)) * 16u;
-    unsigned a_addr[8];
-#pragma unroll
-    for (int s8 = 0; s8 < 8; ++s8) a_addr[s8] = a0 ^ ((unsigned)s8 << 4);
     // ---- B operand reads: lane (r, h) of n-tile j wants the pieces 2 h, 2 h + 1 of row
     // wc + 32 j + r (dword s8 % 4 of piece 2 h + s8 / 4 feeds step s8); j as an immediate
     unsigned b_addr[2];
@@ -186,45 +216,69 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
         b_addr[t] = lds_base + kTpSlabBytes + (unsigned)(wc + r) * 64u +
                     (unsigned)((2 * h + t) ^ ((r >> 2) & 3)) * 16u;
 
-    // Scales and zeros of a pair of groups g, g + 1 (g even) in one dword each, from global
-    // memory into registers (a lane's 16 results of a tile belong to one weight row), and the
-    // group sums of x for the zero-point product: lane (r, h) holds row wr + 32 i + r, group
-    // g + h of the pair.  Six loads per pair and wave, written as assembly with the waits for
-    // them spelled out below: for loads it can see the compiler waits with vmcnt(0), which
-    // also waits for every request of the groups ahead and takes the ring's depth away.
-    // A register loaded here must not be touched before `small_loads_landed` has named it.
+    // ---- The small loads of a block of W pairs of groups, from global memory into registers:
+    // scales and zeros of this lane's two weight rows (a lane's 16 results of a tile belong to
+    // one weight row; pair p in dword p: group 2 p in the low half), and the group sums of x
+    // for the zero-point product (lane (r, h) holds row wr + 32 i + r, group 2 p + h of pair
+    // p; the first pass wrote them as [row tile][block][h][row][p], so a wave reads 512
+    // consecutive bytes x W).  Six loads per block and wave, written as assembly with the
+    // waits for them spelled out below: for loads it can see the compiler waits with
+    // vmcnt(0), which also waits for every request of the groups ahead and takes the ring's
+    // depth away.  A register loaded here must not be touched before `small_loads_landed`
+    // has named it.
+    struct Small {
+        TpRegs<unsigned, W> s[2], z[2];
+        TpRegs<float, W> xs[2];
+    };
     unsigned soff[2], xsoff[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j)
         soff[j] = (unsigned)min(col0 + wc + 32 * j + r, n - 1) * (unsigned)groups_row * 2u;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
-        xsoff[i] = ((unsigned)(row0 + wr + 32 * i + r) * (unsigned)groups_row + (unsigned)h) * 4u;
-    constexpr int kSmall = 6;  // small loads per pair and wave
-    unsigned scur[2], zcur[2], snext[2], znext[2];
-    float xsum[2], xsum_next[2];
-    auto gload_small = [&](int g, unsigned (&sv)[2], unsigned (&zv)[2], float (&xv)[2]) {
+    for (int i = 0; i < 2; ++i) xsoff[i] = (unsigned)((h * kTpTileM + wr + 32 * i + r) * W) * 4u;
+    constexpr int kSmall = 6;  // small loads per block and wave
+    auto gload_small = [&](int g, Small& v) {
         const __half* sb = scale + g;
         const __half* zb = zero + g;
-        const float* xb = xs + g;
+        const float* xb = xs + ((size_t)row_tile * (groups_row / BL) + g / BL) * (2 * kTpTileM * W);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            asm volatile("global_load_dword %0, %1, %2" : "=&v"(sv[j]) : "v"(soff[j]), "s"(sb) : "memory");
-            asm volatile("global_load_dword %0, %1, %2" : "=&v"(zv[j]) : "v"(soff[j]), "s"(zb) : "memory");
+            if constexpr (W == 1) {
+                asm volatile("global_load_dword %0, %1, %2" : "=&v"(v.s[j].raw) : "v"(soff[j]), "s"(sb) : "memory");
+                asm volatile("global_load_dword %0, %1, %2" : "=&v"(v.z[j].raw) : "v"(soff[j]), "s"(zb) : "memory");
+            } else if constexpr (W == 2) {
+                asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(v.s[j].raw) : "v"(soff[j]), "s"(sb) : "memory");
+                asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(v.z[j].raw) : "v"(soff[j]), "s"(zb) : "memory");
+            } else {
+                asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(v.s[j].raw) : "v"(soff[j]), "s"(sb) : "memory");
+                asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(v.z[j].raw) : "v"(soff[j]), "s"(zb) : "memory");
+            }
         }
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
-            asm volatile("global_load_dword %0, %1, %2" : "=&v"(xv[i]) : "v"(xsoff[i]), "s"(xb) : "memory");
+        for (int i = 0; i < 2; ++i) {
+            if constexpr (W == 1)
+                asm volatile("global_load_dword %0, %1, %2" : "=&v"(v.xs[i].raw) : "v"(xsoff[i]), "s"(xb) : "memory");
+            else if constexpr (W == 2)
+                asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(v.xs[i].raw) : "v"(xsoff[i]), "s"(xb) : "memory");
+            else
+                asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(v.xs[i].raw) : "v"(xsoff[i]), "s"(xb) : "memory");
+        }
     };
     // waits until at most `younger` of this wave's loads and requests are outstanding (they
-    // complete in the order they were issued) and hands the six registers over
-    auto small_loads_landed = [&](auto younger_c, unsigned (&sv)[2], unsigned (&zv)[2],
-                                  float (&xv)[2]) {
+    // complete in the order they were issued) and hands the registers over
+    auto small_loads_landed = [&](auto younger_c, Small& v) {
         asm volatile("s_waitcnt vmcnt(%6)"
-                     : "+v"(sv[0]), "+v"(sv[1]), "+v"(zv[0]), "+v"(zv[1]), "+v"(xv[0]), "+v"(xv[1])
+                     : "+v"(v.s[0].raw), "+v"(v.s[1].raw), "+v"(v.z[0].raw), "+v"(v.z[1].raw), "+v"(v.xs[0].raw),
+                       "+v"(v.xs[1].raw)
                      : "n"(decltype(younger_c)::value)
                      : "memory");
     };
+    // One block's values are in use while the next one's are on their way (W = 1), or the
+    // next block's are loaded over them behind their last use (W > 1: a block lasts four or
+    // eight groups, and a load issued at the end of one group has landed by the end of the
+    // next).
+    Small cur;
+    Small nxt;  // W == 1 only
 
     float16_t yacc[2][2];
 #pragma unroll
@@ -234,45 +288,60 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
 #pragma unroll
             for (int e = 0; e < 16; ++e) yacc[i][j][e] = 0.0f;
 
-    gload_small(g_begin, scur, zcur, xsum);
+    gload_small(g_begin, cur);
     request_group(g_begin, 0);
-    request_group(g_begin + 1, 1);  // (a range holds at least one pair)
-    small_loads_landed(ic<2 * kReq>{}, scur, zcur, xsum);
+    request_group(g_begin + 1, kTpBufBytes);  // (a range holds at least one pair)
+    small_loads_landed(ic<2 * kReq>{}, cur);
 
-    // One group of 128 columns out of buffer BUF (immediates in the LDS reads); PAR: the
-    // group's place in its pair.  A wave's requests complete in the order they were issued,
-    // so "at most the six youngest outstanding" means the group's own have landed while the
-    // next group's may still be on their way.
-    auto group = [&](auto buf_c, auto par_c, int g) {
-        constexpr int BUF = decltype(buf_c)::value;
-        constexpr int PAR = decltype(par_c)::value;
-        if (g + 1 < groups) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kReq) : "memory");
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // What a wave issues once per group, behind the group's barrier: the small loads first
+    // where it is their turn (what waits for them need not wait for the requests), then the
+    // requests of the group after next into the buffer everybody has just stopped reading.
+    auto issue_loads = [&](auto u_c, int g, int buf_off) {
+        constexpr int U = decltype(u_c)::value;
+        if constexpr (W == 1) {
+            if (U == 1 && g + 1 < groups) gload_small(g + 1, nxt);
+        }
+        if (g + 2 < groups) {
+            int dst = buf_off + 2 * kTpBufBytes;
+            if (dst >= kTpBufs * kTpBufBytes) dst -= kTpBufs * kTpBufBytes;
+            request_group(g + 2, dst);
+        }
+    };
+
+    // One group of 128 columns out of the buffer at byte `buf_off` of the ring; U: the group's
+    // place in its block.  A wave's loads and requests complete in the order they were
+    // issued, so "at most the n youngest outstanding" names what has landed.
+    auto group = [&](auto u_c, int g, int buf_off) {
+        constexpr int U = decltype(u_c)::value;
+        constexpr int PAR = U & 1;
+        // this wave's requests of the group have landed; those of the next group, and the
+        // small loads issued behind them at the end of a block, may be on their way
+        if (g + 1 >= groups) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        else if (W > 1 && U == 0 && g > g_begin)
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kReq + kSmall) : "memory");
+        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kReq) : "memory");
         // after the barrier everybody's requests for this group have landed, and everybody is
         // done reading the buffer of the group before it, which the group after next reuses
         __builtin_amdgcn_s_barrier();
-        // (the small loads first: what waits for them need not wait for the requests)
-        if (PAR == 1 && g + 1 < groups) gload_small(g + 1, snext, znext, xsum_next);
-        if (g + 2 < groups) request_group(g + 2, (BUF + 2) % kTpBufs);
+        issue_loads(u_c, g, buf_off);
         float16_t acc[2][2];
         bf16x8_t av[2][2];  // [step parity][i]
         bf16x8_t bv[2][2];  // [step parity][j]
         uint4_t wq[2][2];   // [j][half of the group]: the group's nibbles of this lane's rows
-        constexpr int kBufOff = BUF * kTpBufBytes;
-        // (the buffer's offset is added here, as a literal: LDS offsets of up to 144 KiB do not
-        // fit the 16-bit immediate of a read)
+        // (the buffer's offset is added here: LDS offsets of up to 144 KiB do not fit the
+        // 16-bit immediate of a read)
         unsigned t0, t1;
-        asm volatile("v_add_u32 %4, %c8, %6\n\tv_add_u32 %5, %c8, %7\n\t"
+        asm volatile("v_add_u32 %4, %8, %6\n\tv_add_u32 %5, %8, %7\n\t"
                      "ds_read_b128 %0, %4\n\tds_read_b128 %1, %5\n\t"
                      "ds_read_b128 %2, %4 offset:2048\n\tds_read_b128 %3, %5 offset:2048"
                      : "=&v"(wq[0][0]), "=&v"(wq[0][1]), "=&v"(wq[1][0]), "=&v"(wq[1][1]),
                        "=&v"(t0), "=&v"(t1)
-                     : "v"(b_addr[0]), "v"(b_addr[1]), "n"(kBufOff)
+                     : "v"(b_addr[0]), "v"(b_addr[1]), "s"(buf_off)
                      : "memory");
-        asm volatile("v_add_u32 %2, %c4, %3\n\t"
-                     "ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:8192"
-                     : "=&v"(av[0][0]), "=&v"(av[0][1]), "=&v"(t0)
-                     : "v"(a_addr[0]), "n"(kBufOff)
+        const unsigned a_buf = a0 + (unsigned)buf_off;
+        asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:8192"
+                     : "=&v"(av[0][0]), "=&v"(av[0][1])
+                     : "v"(a_buf)
                      : "memory");
         __builtin_amdgcn_sched_barrier(0);
         asm volatile("s_waitcnt lgkmcnt(0)"
@@ -297,17 +366,17 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
         // reads it waits for.
         static_for<8>([&](auto s8c) {
             constexpr int s8 = decltype(s8c)::value;
-            constexpr int cur = s8 & 1;
+            constexpr int cur_p = s8 & 1;
             if constexpr (s8 < 7) {
                 unsigned ta;
-                asm volatile("v_add_u32 %2, %c4, %3\n\t"
+                asm volatile("v_xor_b32 %2, %c4, %3\n\t"
                              "ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:8192"
-                             : "=&v"(av[cur ^ 1][0]), "=&v"(av[cur ^ 1][1]), "=&v"(ta)
-                             : "v"(a_addr[s8 < 7 ? s8 + 1 : 7]), "n"(kBufOff)
+                             : "=&v"(av[cur_p ^ 1][0]), "=&v"(av[cur_p ^ 1][1]), "=&v"(ta)
+                             : "v"(a_buf), "n"((s8 + 1) << 4)
                              : "memory");
             }
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr (s8 < 7) unpack(ic<(s8 < 7 ? s8 + 1 : 7)>{}, bv[cur ^ 1]);
+            if constexpr (s8 < 7) unpack(ic<(s8 < 7 ? s8 + 1 : 7)>{}, bv[cur_p ^ 1]);
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -316,11 +385,11 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
                         float16_t z16;
 #pragma unroll
                         for (int e = 0; e < 16; ++e) z16[e] = 0.0f;
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[cur][i], bv[cur][j],
-                                                                            z16, 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            av[cur_p][i], bv[cur_p][j], z16, 0, 0, 0);
                     } else {
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[cur][i], bv[cur][j],
-                                                                            acc[i][j], 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            av[cur_p][i], bv[cur_p][j], acc[i][j], 0, 0, 0);
                     }
                 }
 #pragma unroll
@@ -331,12 +400,20 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (s8 < 7)
                 asm volatile("s_waitcnt lgkmcnt(0)"
-                             : "+v"(av[cur ^ 1][0]), "+v"(av[cur ^ 1][1])::"memory");
+                             : "+v"(av[cur_p ^ 1][0]), "+v"(av[cur_p ^ 1][1])::"memory");
         });
+        if constexpr (W > 1 && U == 0) {
+            // the block's values, requested at the end of the group before this one
+            if (g > g_begin) {
+                if (g + 2 < groups) small_loads_landed(ic<kReq>{}, cur);
+                else small_loads_landed(ic<0>{}, cur);
+            }
+        }
         // y += scale * acc
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            const unsigned short sb = (unsigned short)(PAR ? (scur[j] >> 16) : scur[j]);
+            const unsigned sd = cur.s[j][U >> 1];
+            const unsigned short sb = (unsigned short)(PAR ? (sd >> 16) : sd);
             const float sf = __half2float(__builtin_bit_cast(__half, sb));
 #pragma unroll
             for (int i = 0; i < 2; ++i)
@@ -349,8 +426,9 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
             float cv[2];
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                const unsigned short sb = (unsigned short)(h ? (scur[j] >> 16) : scur[j]);
-                const unsigned short zb = (unsigned short)(h ? (zcur[j] >> 16) : zcur[j]);
+                const unsigned sd = cur.s[j][U >> 1], zd = cur.z[j][U >> 1];
+                const unsigned short sb = (unsigned short)(h ? (sd >> 16) : sd);
+                const unsigned short zb = (unsigned short)(h ? (zd >> 16) : zd);
                 cv[j] = -__half2float(__builtin_bit_cast(__half, sb)) *
                         (128.0f + __half2float(__builtin_bit_cast(__half, zb)));
             }
@@ -358,23 +436,25 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
             for (int i = 0; i < 2; ++i)
 #pragma unroll
                 for (int j = 0; j < 2; ++j)
-                    yacc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(xsum[i], cv[j], yacc[i][j], 0,
-                                                                      0, 0);
-            if (g + 1 < groups) {
-                if (g + 2 < groups) small_loads_landed(ic<kReq>{}, snext, znext, xsum_next);
-                else small_loads_landed(ic<0>{}, snext, znext, xsum_next);
-#pragma unroll
-                for (int j = 0; j < 2; ++j) scur[j] = snext[j], zcur[j] = znext[j];
-#pragma unroll
-                for (int i = 0; i < 2; ++i) xsum[i] = xsum_next[i];
+                    yacc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(cur.xs[i][U >> 1], cv[j],
+                                                                      yacc[i][j], 0, 0, 0);
+            if constexpr (W == 1) {
+                if (g + 1 < groups) {
+                    if (g + 2 < groups) small_loads_landed(ic<kReq>{}, nxt);
+                    else small_loads_landed(ic<0>{}, nxt);
+                    cur = nxt;
+                }
+            } else if constexpr (U == BL - 1) {
+                if (g + 1 < groups) gload_small(g + 1, cur);
             }
         }
     };
-    // groups is even (checked on the host); buffers go round in threes, pairs in twos
-    for (int g0 = g_begin; g0 < groups; g0 += 6) {
-        static_for<6>([&](auto uc) {
-            constexpr int u = decltype(uc)::value;
-            if (g0 + u < groups) group(ic<u % kTpBufs>{}, ic<(u & 1)>{}, g0 + u);
+    // ranges are whole blocks (K is a multiple of 256 W); buffers go round in threes
+    int buf_off = 0;
+    for (int g0 = g_begin; g0 < groups; g0 += BL) {
+        static_for<BL>([&](auto uc) {
+            group(uc, g0 + decltype(uc)::value, buf_off);
+            buf_off = buf_off + kTpBufBytes == kTpBufs * kTpBufBytes ? 0 : buf_off + kTpBufBytes;
         });
     }
 
@@ -436,29 +516,49 @@ __global__ __launch_bounds__(256) void q4_tall_reduce_kernel(const float* __rest
     else static_cast<uint16_t*>(y_out)[(int64_t)gr * n + gn] = f32_to_bf16_rne(acc);
 }
 
-template <bool F32OUT>
+// Pairs of groups per small load: as many as K (whole blocks) and the alignment of the scales
+// and zeros (a load of 4, 8 or 16 bytes per row) allow.
+inline int tp_pairs_per_load(int k, const void* scale, const void* zero) {
+    const uintptr_t a = reinterpret_cast<uintptr_t>(scale) | reinterpret_cast<uintptr_t>(zero);
+    if (k % 1024 == 0 && (a & 15u) == 0) return 4;
+    if (k % 512 == 0 && (a & 7u) == 0) return 2;
+    return 1;
+}
+
+template <bool F32OUT, int W>
 static hipError_t tallp_launch(const uint16_t* xp, const float* xs, float* partials,
                                const uint8_t* qw, const __half* scale, const __half* zero,
                                const float* bias, void* y, int m, int n, int k, hipStream_t st) {
     constexpr size_t lds = (size_t)kTpBufs * kTpBufBytes;
     static const hipError_t opt = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(qgemm_q4g128_tallp_kernel<F32OUT>),
+        reinterpret_cast<const void*>(qgemm_q4g128_tallp_kernel<F32OUT, W>),
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (opt != hipSuccess) return opt;
     const int tiles_n = (n + kTpTileN - 1) / kTpTileN;
     const int tiles = tiles_n * (tp_padded_rows(m) / kTpTileM);
     const int cus = device_cu_count();
     if (cus <= 0) return hipErrorInvalidDevice;
-    const TpPlan plan = tp_plan(tiles, k >> 7, cus);
+    const TpPlan plan = tp_plan(tiles, k >> 7, 2 * W, cus);
     const int parts = (tiles - plan.full) * plan.split;
-    qgemm_q4g128_tallp_kernel<F32OUT><<<dim3(plan.full + (plan.split > 1 ? parts : 0)), dim3(512),
-                                        lds, st>>>(xp, xs, qw, scale, zero, bias, y, partials, m,
-                                                   n, k, tiles_n, plan.full, plan.split);
+    qgemm_q4g128_tallp_kernel<F32OUT, W>
+        <<<dim3(plan.full + (plan.split > 1 ? parts : 0)), dim3(512), lds, st>>>(
+            xp, xs, qw, scale, zero, bias, y, partials, m, n, k, tiles_n, plan.full, plan.split);
     if (plan.split > 1)
         q4_tall_reduce_kernel<F32OUT>
             <<<dim3((tiles - plan.full) * (kTpTileElems / 256)), dim3(256), 0, st>>>(
                 partials, bias, y, m, n, tiles_n, plan.full, plan.split);
     return hipGetLastError();
+}
+
+template <bool F32OUT>
+static hipError_t tallp_launch_w(int w, const uint16_t* xp, const float* xs, float* partials,
+                                 const uint8_t* qw, const __half* scale, const __half* zero,
+                                 const float* bias, void* y, int m, int n, int k, hipStream_t st) {
+    switch (w) {
+        case 4: return tallp_launch<F32OUT, 4>(xp, xs, partials, qw, scale, zero, bias, y, m, n, k, st);
+        case 2: return tallp_launch<F32OUT, 2>(xp, xs, partials, qw, scale, zero, bias, y, m, n, k, st);
+        default: return tallp_launch<F32OUT, 1>(xp, xs, partials, qw, scale, zero, bias, y, m, n, k, st);
+    }
 }
 
 }  // namespace lg
@@ -504,17 +604,18 @@ extern "C" logismos_status_t logismos_launch_qgemm_q4g128_tall(
     uint16_t* xp = static_cast<uint16_t*>(workspace);
     float* xs = reinterpret_cast<float*>(static_cast<char*>(workspace) + lg::tp_sums_offset(m, k));
     const int64_t chunks = (int64_t)m_pad * (k / 8);
+    const int w = lg::tp_pairs_per_load(k, scale_f16, zero_f16);
     lg::q4_tall_prepare_kernel<<<dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st>>>(
-        static_cast<const uint16_t*>(x_bf16), xp, xs, m, m_pad, k);
+        static_cast<const uint16_t*>(x_bf16), xp, xs, m, m_pad, k, w);
     float* partials = reinterpret_cast<float*>(static_cast<char*>(workspace) +
                                                lg::tp_partials_offset(m, k));
     if (y_is_f32)
-        return lg::tallp_launch<true>(xp, xs, partials, static_cast<const uint8_t*>(qw_u8),
-                                      static_cast<const __half*>(scale_f16),
-                                      static_cast<const __half*>(zero_f16),
-                                      static_cast<const float*>(bias_f32), y, m, n, k, st);
-    return lg::tallp_launch<false>(xp, xs, partials, static_cast<const uint8_t*>(qw_u8),
-                                   static_cast<const __half*>(scale_f16),
-                                   static_cast<const __half*>(zero_f16),
-                                   static_cast<const float*>(bias_f32), y, m, n, k, st);
+        return lg::tallp_launch_w<true>(w, xp, xs, partials, static_cast<const uint8_t*>(qw_u8),
+                                        static_cast<const __half*>(scale_f16),
+                                        static_cast<const __half*>(zero_f16),
+                                        static_cast<const float*>(bias_f32), y, m, n, k, st);
+    return lg::tallp_launch_w<false>(w, xp, xs, partials, static_cast<const uint8_t*>(qw_u8),
+                                     static_cast<const __half*>(scale_f16),
+                                     static_cast<const __half*>(zero_f16),
+                                     static_cast<const float*>(bias_f32), y, m, n, k, st);
 }
