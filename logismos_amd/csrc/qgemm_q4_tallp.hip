@@ -181,26 +181,32 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
         const int gn = min(col0 + row, n - 1);  // a row past n re-reads the last row
         woff[q] = (unsigned)gn * (unsigned)(k >> 1) + (unsigned)piece * 16u;
     }
-    // (as assembly: the 32-bit offsets above with a scalar base, where the builtin widens each
-    // to a 64-bit address in two more registers; M0 holds the LDS address of lane 0's 16 bytes
-    // and nothing else in this kernel uses M0)
-    auto request_group = [&](int g, int buf_off) {
+    // As assembly: the 32-bit offsets above with a scalar base (the builtin widens each to a
+    // 64-bit address in two more registers); M0 holds the LDS address of lane 0's 16 bytes and
+    // nothing else in this kernel uses M0.  `on` switches the six requests off as a whole by
+    // way of EXEC, without a branch: a branch in the middle of a group's MFMAs costs the
+    // register allocator its footing (spills), and a wave issues its requests at one of two
+    // places in the group.
+    auto request_group = [&](int g, int buf_off, bool on) {
         const char* xsrc = reinterpret_cast<const char*>(xp) + (size_t)g * 256;
         const char* wsrc = reinterpret_cast<const char*>(qw) + (size_t)g * 64;
         const unsigned xdst = lds_base + (unsigned)buf_off + (unsigned)wave * 4096u;
         const unsigned wdst = lds_base + (unsigned)buf_off + kTpSlabBytes + (unsigned)wave * 2048u;
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                         :
-                         : "v"(xoff[q]), "s"(xsrc), "s"(xdst + q * 1024u)
-                         : "memory");
-#pragma unroll
-        for (int q = 0; q < 2; ++q)
-            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                         :
-                         : "v"(woff[q]), "s"(wsrc), "s"(wdst + q * 1024u)
-                         : "memory");
+        const unsigned long long mask = on ? ~0ull : 0ull;
+        unsigned long long saved;
+        asm volatile(
+            "s_mov_b64 %0, exec\n\ts_mov_b64 exec, %11\n\t"
+            "s_mov_b32 m0, %9\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %7\n\t"
+            "s_add_u32 m0, %9, 0x400\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %7\n\t"
+            "s_add_u32 m0, %9, 0x800\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %3, %7\n\t"
+            "s_add_u32 m0, %9, 0xc00\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %4, %7\n\t"
+            "s_mov_b32 m0, %10\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %5, %8\n\t"
+            "s_add_u32 m0, %10, 0x400\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %6, %8\n\t"
+            "s_mov_b64 exec, %0"
+            : "=&s"(saved)
+            : "v"(xoff[0]), "v"(xoff[1]), "v"(xoff[2]), "v"(xoff[3]), "v"(woff[0]), "v"(woff[1]),
+              "s"(xsrc), "s"(wsrc), "s"(xdst), "s"(wdst), "s"(mask)
+            : "memory", "scc");
     };
     constexpr int kReq = 6;  // requests per group and wave
     // ---- A operand reads: lane (r, h) at step s8 wants chunk 8 h + s8 of row wr + 32 i + r,
@@ -289,23 +295,22 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
             for (int e = 0; e < 16; ++e) yacc[i][j][e] = 0.0f;
 
     gload_small(g_begin, cur);
-    request_group(g_begin, 0);
-    request_group(g_begin + 1, kTpBufBytes);  // (a range holds at least one pair)
+    request_group(g_begin, 0, true);
+    request_group(g_begin + 1, kTpBufBytes, true);  // (a range holds at least one pair)
     small_loads_landed(ic<2 * kReq>{}, cur);
 
-    // What a wave issues once per group, behind the group's barrier: the small loads first
-    // where it is their turn (what waits for them need not wait for the requests), then the
-    // requests of the group after next into the buffer everybody has just stopped reading.
-    auto issue_loads = [&](auto u_c, int g, int buf_off) {
-        constexpr int U = decltype(u_c)::value;
-        if constexpr (W == 1) {
-            if (U == 1 && g + 1 < groups) gload_small(g + 1, nxt);
-        }
-        if (g + 2 < groups) {
-            int dst = buf_off + 2 * kTpBufBytes;
-            if (dst >= kTpBufs * kTpBufBytes) dst -= kTpBufs * kTpBufBytes;
-            request_group(g + 2, dst);
-        }
+    // The two waves of a SIMD (w and w + 4) issue a group's requests at different times: a
+    // burst of requests holds a wave up for hundreds of cycles (the address path takes 16
+    // cycles per 1 KiB request and a wave issues in order), and with all eight bursts behind
+    // the barrier the matrix pipes stood still meanwhile.  Waves 0-3 issue theirs behind the
+    // barrier, waves 4-7 in the middle of the group, when the other wave of the SIMD is busy
+    // with MFMAs: the requests of the group after next, into the buffer everybody stopped
+    // reading before the barrier.
+    const bool late = wave >= 4;
+    auto issue_requests = [&](int g, int buf_off, bool my_turn) {
+        int dst = buf_off + 2 * kTpBufBytes;
+        if (dst >= kTpBufs * kTpBufBytes) dst -= kTpBufs * kTpBufBytes;
+        request_group(g + 2, dst, my_turn && g + 2 < groups);
     };
 
     // One group of 128 columns out of the buffer at byte `buf_off` of the ring; U: the group's
@@ -323,7 +328,11 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
         // after the barrier everybody's requests for this group have landed, and everybody is
         // done reading the buffer of the group before it, which the group after next reuses
         __builtin_amdgcn_s_barrier();
-        issue_loads(u_c, g, buf_off);
+        // (the small loads first: what waits for them need not wait for the requests)
+        if constexpr (W == 1) {
+            if (U == 1 && g + 1 < groups) gload_small(g + 1, nxt);
+        }
+        issue_requests(g, buf_off, !late);
         float16_t acc[2][2];
         bf16x8_t av[2][2];  // [step parity][i]
         bf16x8_t bv[2][2];  // [step parity][j]
@@ -367,6 +376,10 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
         static_for<8>([&](auto s8c) {
             constexpr int s8 = decltype(s8c)::value;
             constexpr int cur_p = s8 & 1;
+            if constexpr (s8 == 4) {
+                issue_requests(g, buf_off, late);
+                __builtin_amdgcn_sched_barrier(0);
+            }
             if constexpr (s8 < 7) {
                 unsigned ta;
                 asm volatile("v_xor_b32 %2, %c4, %3\n\t"
