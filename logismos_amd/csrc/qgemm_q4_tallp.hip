@@ -183,29 +183,25 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
     }
     // As assembly: the 32-bit offsets above with a scalar base (the builtin widens each to a
     // 64-bit address in two more registers); M0 holds the LDS address of lane 0's 16 bytes and
-    // nothing else in this kernel uses M0.  `on` switches the six requests off as a whole by
-    // way of EXEC, without a branch: a branch in the middle of a group's MFMAs costs the
-    // register allocator its footing (spills), and a wave issues its requests at one of two
-    // places in the group.
-    auto request_group = [&](int g, int buf_off, bool on) {
+    // nothing else in this kernel uses M0.
+    auto request_group = [&](int g, int buf_off) {
         const char* xsrc = reinterpret_cast<const char*>(xp) + (size_t)g * 256;
         const char* wsrc = reinterpret_cast<const char*>(qw) + (size_t)g * 64;
-        const unsigned xdst = lds_base + (unsigned)buf_off + (unsigned)wave * 4096u;
-        const unsigned wdst = lds_base + (unsigned)buf_off + kTpSlabBytes + (unsigned)wave * 2048u;
-        const unsigned long long mask = on ? ~0ull : 0ull;
-        unsigned long long saved;
+        // (scalar registers for sure: a value the compiler takes for lane-dependent would be
+        // handed to the statement in vector registers)
+        const unsigned xdst = __builtin_amdgcn_readfirstlane(lds_base + (unsigned)buf_off +
+                                                             (unsigned)wave * 4096u);
+        const unsigned wdst = xdst + kTpSlabBytes - (unsigned)wave * 2048u;
         asm volatile(
-            "s_mov_b64 %0, exec\n\ts_mov_b64 exec, %11\n\t"
-            "s_mov_b32 m0, %9\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %7\n\t"
-            "s_add_u32 m0, %9, 0x400\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %7\n\t"
-            "s_add_u32 m0, %9, 0x800\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %3, %7\n\t"
-            "s_add_u32 m0, %9, 0xc00\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %4, %7\n\t"
-            "s_mov_b32 m0, %10\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %5, %8\n\t"
-            "s_add_u32 m0, %10, 0x400\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %6, %8\n\t"
-            "s_mov_b64 exec, %0"
-            : "=&s"(saved)
+            "s_mov_b32 m0, %8\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %6\n\t"
+            "s_add_u32 m0, %8, 0x400\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %6\n\t"
+            "s_add_u32 m0, %8, 0x800\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %6\n\t"
+            "s_add_u32 m0, %8, 0xc00\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %3, %6\n\t"
+            "s_mov_b32 m0, %9\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %4, %7\n\t"
+            "s_add_u32 m0, %9, 0x400\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %5, %7"
+            :
             : "v"(xoff[0]), "v"(xoff[1]), "v"(xoff[2]), "v"(xoff[3]), "v"(woff[0]), "v"(woff[1]),
-              "s"(xsrc), "s"(wsrc), "s"(xdst), "s"(wdst), "s"(mask)
+              "s"(xsrc), "s"(wsrc), "s"(xdst), "s"(wdst)
             : "memory", "scc");
     };
     constexpr int kReq = 6;  // requests per group and wave
@@ -295,22 +291,20 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
             for (int e = 0; e < 16; ++e) yacc[i][j][e] = 0.0f;
 
     gload_small(g_begin, cur);
-    request_group(g_begin, 0, true);
-    request_group(g_begin + 1, kTpBufBytes, true);  // (a range holds at least one pair)
+    request_group(g_begin, 0);
+    request_group(g_begin + 1, kTpBufBytes);  // (a range holds at least one pair)
     small_loads_landed(ic<2 * kReq>{}, cur);
 
-    // The two waves of a SIMD (w and w + 4) issue a group's requests at different times: a
-    // burst of requests holds a wave up for hundreds of cycles (the address path takes 16
-    // cycles per 1 KiB request and a wave issues in order), and with all eight bursts behind
-    // the barrier the matrix pipes stood still meanwhile.  Waves 0-3 issue theirs behind the
-    // barrier, waves 4-7 in the middle of the group, when the other wave of the SIMD is busy
-    // with MFMAs: the requests of the group after next, into the buffer everybody stopped
-    // reading before the barrier.
-    const bool late = wave >= 4;
-    auto issue_requests = [&](int g, int buf_off, bool my_turn) {
-        int dst = buf_off + 2 * kTpBufBytes;
-        if (dst >= kTpBufs * kTpBufBytes) dst -= kTpBufs * kTpBufBytes;
-        request_group(g + 2, dst, my_turn && g + 2 < groups);
+    // The requests of the group after next go into the buffer everybody stopped reading before
+    // this group's barrier.  (Measured and not kept: the two waves of a SIMD issuing theirs at
+    // different times -- behind the barrier and in the middle of the group -- so that one
+    // feeds the matrix pipe while the other is held up by its burst of requests; no change.)
+    auto issue_requests = [&](int g, int buf_off) {
+        if (g + 2 < groups) {
+            int dst = buf_off + 2 * kTpBufBytes;
+            if (dst >= kTpBufs * kTpBufBytes) dst -= kTpBufs * kTpBufBytes;
+            request_group(g + 2, dst);
+        }
     };
 
     // One group of 128 columns out of the buffer at byte `buf_off` of the ring; U: the group's
@@ -332,7 +326,7 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
         if constexpr (W == 1) {
             if (U == 1 && g + 1 < groups) gload_small(g + 1, nxt);
         }
-        issue_requests(g, buf_off, !late);
+        issue_requests(g, buf_off);
         float16_t acc[2][2];
         bf16x8_t av[2][2];  // [step parity][i]
         bf16x8_t bv[2][2];  // [step parity][j]
@@ -376,10 +370,6 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
         static_for<8>([&](auto s8c) {
             constexpr int s8 = decltype(s8c)::value;
             constexpr int cur_p = s8 & 1;
-            if constexpr (s8 == 4) {
-                issue_requests(g, buf_off, late);
-                __builtin_amdgcn_sched_barrier(0);
-            }
             if constexpr (s8 < 7) {
                 unsigned ta;
                 asm volatile("v_xor_b32 %2, %c4, %3\n\t"
@@ -422,7 +412,8 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
                 else small_loads_landed(ic<0>{}, cur);
             }
         }
-        // y += scale * acc
+        // y += scale * acc  (measured and not kept: the last two steps tile by tile with a
+        // tile's multiply-adds between the MFMAs of the tiles after it; no change)
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const unsigned sd = cur.s[j][U >> 1];
