@@ -159,7 +159,6 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
     unsigned magic;
     asm volatile("v_mov_b32 %0, 0x43004300" : "=v"(magic));
     const unsigned lds_base = (unsigned)(uintptr_t)(tp_lds_ptr_t)tp_lds;
-    char* const lds_c = reinterpret_cast<char*>(tp_lds);
 
     // ---- requests of a group, straight into LDS (a request writes 1 KiB of consecutive LDS).
     // x: request q of this wave covers rows 16 wave + 4 q .. + 3, lane -> row + lane / 16, LDS
@@ -238,7 +237,6 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
         soff[j] = (unsigned)min(col0 + wc + 32 * j + r, n - 1) * (unsigned)groups_row * 2u;
 #pragma unroll
     for (int i = 0; i < 2; ++i) xsoff[i] = (unsigned)((h * kTpTileM + wr + 32 * i + r) * W) * 4u;
-    constexpr int kSmall = 6;  // small loads per block and wave
     auto gload_small = [&](int g, Small& v) {
         const __half* sb = scale + g;
         const __half* zb = zero + g;
@@ -293,7 +291,9 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
     gload_small(g_begin, cur);
     request_group(g_begin, 0);
     request_group(g_begin + 1, kTpBufBytes);  // (a range holds at least one pair)
-    small_loads_landed(ic<2 * kReq>{}, cur);
+    // (everything issued so far: the order in which loads into registers and requests into
+    // LDS issued back to back complete is not relied on)
+    small_loads_landed(ic<0>{}, cur);
 
     // The requests of the group after next go into the buffer everybody stopped reading before
     // this group's barrier.  (Measured and not kept: the two waves of a SIMD issuing theirs at
@@ -313,11 +313,11 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
     auto group = [&](auto u_c, int g, int buf_off) {
         constexpr int U = decltype(u_c)::value;
         constexpr int PAR = U & 1;
-        // this wave's requests of the group have landed; those of the next group, and the
-        // small loads issued behind them at the end of a block, may be on their way
+        // this wave's requests of the group, issued two groups ago, have landed; those of
+        // the next group may be on their way.  (Requests complete in the order they were
+        // issued.  Behind a block's small loads the count is not raised by their number:
+        // whether they complete in order with the requests is not relied on.)
         if (g + 1 >= groups) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        else if (W > 1 && U == 0 && g > g_begin)
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kReq + kSmall) : "memory");
         else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kReq) : "memory");
         // after the barrier everybody's requests for this group have landed, and everybody is
         // done reading the buffer of the group before it, which the group after next reuses
@@ -407,10 +407,9 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
         });
         if constexpr (W > 1 && U == 0) {
             // the block's values, requested at the end of the group before this one
-            if (g > g_begin) {
-                if (g + 2 < groups) small_loads_landed(ic<kReq>{}, cur);
-                else small_loads_landed(ic<0>{}, cur);
-            }
+            // (with everything else this wave has outstanding: the requests of the group
+            // after next, issued most of a group ago -- once per block)
+            if (g > g_begin) small_loads_landed(ic<0>{}, cur);
         }
         // y += scale * acc  (measured and not kept: the last two steps tile by tile with a
         // tile's multiply-adds between the MFMAs of the tiles after it; no change)
@@ -444,8 +443,7 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
                                                                       yacc[i][j], 0, 0, 0);
             if constexpr (W == 1) {
                 if (g + 1 < groups) {
-                    if (g + 2 < groups) small_loads_landed(ic<kReq>{}, nxt);
-                    else small_loads_landed(ic<0>{}, nxt);
+                    small_loads_landed(ic<0>{}, nxt);
                     cur = nxt;
                 }
             } else if constexpr (U == BL - 1) {
