@@ -174,8 +174,50 @@ def mfma_ceiling(stream, bf16: bool) -> dict:
             fn = [lambda flags=flags: kernels.launch_probe_mfma(sink, iters, flags, stream)]
             ms, _, _ = time_launches(stream, fn, 10, 3)
             rates[name] = round(flops / ms / 1e9, 1)
+            rates[name + "_board_W"], rates["board_power_cap_W"] = board_power_watts(stream, fn[0])
         _MFMA_CEILING_CACHE[bf16] = rates
     return _MFMA_CEILING_CACHE[bf16]
+
+
+def board_power_watts(stream, launch, seconds: float = 1.5):
+    """Board power (W, mean of the second half of the samples) while `launch` loops for
+    `seconds`, and the board's power cap, both read from the amdgpu hwmon node; (None, None)
+    where the node is not readable.  The probe's and the GEMM's figures beside the cap say
+    whether a kernel runs into the cap -- below it the clock holds 2.4 GHz, at it the part
+    lowers the clock."""
+    import glob
+    import threading
+    nodes = glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input") or \
+        glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_average")
+    if not nodes:
+        return None, None
+
+    def read(path):
+        try:
+            with open(path) as f:
+                return int(f.read()) / 1e6
+        except (OSError, ValueError):
+            return None
+    cap = read(os.path.join(os.path.dirname(nodes[0]), "power1_cap"))
+    samples, stop = [], threading.Event()
+
+    def poll():
+        while not stop.is_set():
+            w = read(nodes[0])
+            if w is not None:
+                samples.append(w)
+            time.sleep(0.05)
+    t = threading.Thread(target=poll)
+    t.start()
+    t0 = time.time()
+    while time.time() - t0 < seconds:
+        for _ in range(5):
+            launch()
+        stream.synchronize()
+    stop.set()
+    t.join()
+    tail = samples[len(samples) // 2:]
+    return (round(sum(tail) / len(tail), 0) if tail else None), cap
 
 
 def against_mfma_ceiling(stream, bf16: bool, achieved_tflops: float) -> dict:
@@ -183,7 +225,10 @@ def against_mfma_ceiling(stream, bf16: bool, achieved_tflops: float) -> dict:
     c = mfma_ceiling(stream, bf16)
     return {"measured_mfma_ceiling_TFLOPs": c["changing_operands"],
             "measured_mfma_rate_constant_operands_TFLOPs": c["constant_operands"],
-            "frac_of_measured_ceiling": round(achieved_tflops / c["changing_operands"], 4)}
+            "frac_of_measured_ceiling": round(achieved_tflops / c["changing_operands"], 4),
+            "board_power_W": {"cap": c["board_power_cap_W"],
+                              "mfma_probe_constant_operands": c["constant_operands_board_W"],
+                              "mfma_probe_changing_operands": c["changing_operands_board_W"]}}
 
 
 def replicate(buf: hip.DeviceBuffer, copies: int):
@@ -532,7 +577,7 @@ def bench_q4_tall(args):
     shapes = [("qkv", 6144, 4096), ("o", 4096, 4096), ("gate_up", 24576, 4096),
               ("down", 4096, 12288)]
     out, flops_all, ms_all, ms_noworkspace = {}, 0.0, 0.0, 0.0
-    parity = None
+    parity, power = None, {}
     for name, n, k in shapes:
         qw = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
         s = (rng.random((n, k // 128), np.float32) * 0.004 + 0.004).astype(np.float16)
@@ -560,11 +605,24 @@ def bench_q4_tall(args):
         ms_all += ms
         out[name] = {"n": n, "k": k, "us": round(ms * 1e3, 1),
                      "TFLOPs": round(flops / ms / 1e9, 1)}
+        if name == "gate_up":
+            # the same launch on x = 0: operands of the A side that never toggle, the kernel's
+            # schedule without what the board's power cap takes off the clock
+            power["gate_up"], _ = board_power_watts(stream, fn)
+            d0 = hip.DeviceBuffer.from_numpy(np.zeros_like(xb))
+            fz = lambda: kernels.launch_qgemm_q4g128_tall(d0, d[1], d[2], d[3], dy, ws, b, n, k,  # noqa: E731
+                                                          stream)
+            msz, _, _ = time_launches(stream, [fz], 10, 2)
+            power["gate_up_x_zero"], _ = board_power_watts(stream, fz)
+            out[name]["us_x_zero"] = round(msz * 1e3, 1)
+            del d0
         del d, dy, ws
     return {"workload": "config 4's 8240 packed rows through one layer's Q4G128 projections "
                         "(qkv 6144x4096, o 4096x4096, gate_up 24576x4096, down 4096x12288)",
             "kernel": "q4_tall_prepare_kernel + qgemm_q4g128_tallp_kernel (128x256 tiles, x and "
-                      "weights straight into a three-deep LDS ring, v_mfma_f32_32x32x16_bf16)",
+                      "weights straight into a three-deep LDS ring, v_mfma_f32_32x32x16_bf16; the "
+                      "tiles of the last partial round of workgroups split over K + "
+                      "q4_tall_reduce_kernel)",
             "projections": out, "ms_per_layer": round(ms_all, 4),
             "ms_per_layer_entry_point_without_workspace": round(ms_noworkspace, 4),
             "roofline": {"bound": "mfma", "achieved": round(flops_all / ms_all / 1e9, 1),
@@ -572,6 +630,7 @@ def bench_q4_tall(args):
                          "frac": round(flops_all / ms_all / 1e9 / 2500.0, 4), "traffic": None,
                          "flops_per_layer": flops_all,
                          **against_mfma_ceiling(stream, True, flops_all / ms_all / 1e9)},
+            "board_power_W_during": power,
             "parity_max_abs_vs_oracle_sample": parity}
 
 

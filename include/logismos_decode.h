@@ -187,9 +187,12 @@ logismos_status_t logismos_launch_qgemm_q4g128_bf16_mfma(const void* x_bf16, con
  * LDS and takes the zero-point term as a small product of its own.  Any m >= 1 (built for
  * m >= ~100), K a multiple of 256, y bf16 `[m][N]` or, with y_is_f32, fp32 (what the step
  * executor keeps between operators); bias fp32 `[N]` or NULL.  The workspace
- * (`..._workspace_bytes(m, k)`, 16-byte aligned, caller-owned) is scratch: nothing in it
- * matters before or after the call.  The entry points above serve the same product without
- * a workspace (slower from about a hundred rows on). */
+ * (`..._workspace_bytes(m, k)`, 16-byte aligned, caller-owned: the copy of x, its group sums
+ * and 64 MiB for fp32 partial tiles -- the tiles of a last, partial round of workgroups are
+ * split over K and summed by a small kernel) is scratch: nothing in it matters before or
+ * after the call.  Scales and zeros 16-byte aligned with K a multiple of 1024 take the
+ * fastest path (8-byte aligned and a multiple of 512 the next).  The entry points above
+ * serve the same product without a workspace (slower from about a hundred rows on). */
 logismos_status_t logismos_check_qgemm_q4g128_tall_shape(int m, int n, int k, char* msg,
                                                          size_t msg_cap);
 size_t logismos_qgemm_q4g128_tall_workspace_bytes(int m, int k);

@@ -13,12 +13,19 @@
 //   in the order the nibble unpack produces ("pair order": (x0,x4)(x1,x5)(x2,x6)(x3,x7) per
 //   16-byte chunk), rows padded with zeros to a multiple of 128, and every row's sum over each
 //   group of 128 columns;
-// * the product kernel moves a group's 128 x 128 slab of that copy from global memory
-//   STRAIGHT into LDS (global_load_lds, 16 bytes per lane, no registers, no vector
-//   instructions), double buffered, one barrier per group.  A request writes 1 KiB of
-//   consecutive LDS (four rows), so instead of padding rows the 16-byte chunks of a row are
-//   stored XOR-swizzled by the row index; a lane's eight read addresses per buffer are
-//   loop-invariant registers and the ds_read_b128 of the MFMA A operand stays conflict-free;
+// * the product kernel (128 x 256 tiles, eight waves of 64 x 64, one workgroup per CU) moves
+//   a group's 128 x 128 slab of that copy and its 256 x 128 tile of nibbles from global
+//   memory STRAIGHT into LDS (global_load_lds, 16 bytes per lane, no registers, no vector
+//   instructions) into a ring of three buffers, requested two groups ahead, one barrier per
+//   group.  A request writes 1 KiB of consecutive LDS, so instead of padding rows the
+//   16-byte chunks of a row are stored XOR-swizzled by the row index and the ds_read_b128 of
+//   the MFMA operands stay conflict-free;
+// * scales, zeros and the group sums of x reach a lane's registers for four (or two) pairs
+//   of groups per load where K allows: a lane's row of scales is 64 bytes apart from the
+//   next lane's, so each such load costs the address path a cache line per lane -- one per
+//   pair and array, they took it twice as long as the tiles themselves and held every wave
+//   up behind each barrier.  The first pass writes the group sums in the layout these loads
+//   want ([row tile][block of pairs][group's place in its pair][row][pair]);
 // * the zero-point term -scale * (128 + zero) * sum_x is a rank-(K/128) product of its own:
 //   one v_mfma_f32_32x32x2_f32 per output tile and PAIR of groups, accumulating into the same
 //   registers, in place of a multiply-add per result and group;
