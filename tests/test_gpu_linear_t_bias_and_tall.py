@@ -194,11 +194,16 @@ def _gemm_q4_ws(xb, qw, s, z, b, n, k, bias, f32_out=False, ws_fill=0xFF):
 @pytest.mark.parametrize("b,n,k,with_bias", [(1, 16, 256, True), (97, 128, 256, False),
                                              (130, 200, 512, True), (257, 1000, 1280, True),
                                              (300, 4100, 4096, False), (1000, 333, 2048, True),
-                                             (142, 576, 512, True)])
+                                             (142, 576, 512, True), (200, 300, 1536, True),
+                                             (130, 520, 3072, False)])
 def test_q4g128_workspace_kernel_ragged_shapes(b, n, k, with_bias):
     # partial tiles in rows (128) and in weight rows (256), K of two groups up to 32, with and
     # without a bias; the fp32 product (what the step executor keeps) tightly, the bf16 one at
-    # the decode path's tolerance; what the workspace held before does not matter
+    # the decode path's tolerance; what the workspace held before does not matter.  K decides
+    # how many pairs of groups a lane loads scales / zeros / sums for at once (a multiple of
+    # 1024: four, 1536 = 3 x 512: two, else one), each with one and with several such blocks;
+    # every one of these launches is smaller than the device, so its tiles are split over K
+    # (evenly or not: 24 groups in parts of 8, 12 in parts of 4) and summed by the reduce kernel
     rng = np.random.default_rng(b + 7 * n + 13 * k)
     qw, s, z = _q4(rng, n, k)
     xb = O.f32_to_bf16_bits(rng.standard_normal((b, k), np.float32))
