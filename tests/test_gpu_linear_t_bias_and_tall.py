@@ -219,6 +219,47 @@ def test_q4g128_workspace_kernel_ragged_shapes(b, n, k, with_bias):
                           O.f32_to_bf16_bits(got).reshape(b, n))
 
 
+@pytest.mark.parametrize("shift", [0, 8, 4])
+def test_q4g128_workspace_kernel_takes_scales_and_zeros_at_any_4_byte_alignment(shift):
+    # the kernel loads a lane's scales and zeros for four pairs of groups at once where they
+    # are 16-byte aligned (and K allows), for two at 8 bytes, for one otherwise: the same
+    # arrays at 16-, 8- and 4-byte aligned addresses, each against the oracle
+    rng = np.random.default_rng(91)
+    b, n, k = 200, 520, 2048
+    qw, s, z = _q4(rng, n, k)
+    xb = O.f32_to_bf16_bits(rng.standard_normal((b, k), np.float32))
+    bias = rng.standard_normal(n).astype(np.float32)
+
+    def shifted(a):
+        raw = np.zeros(a.nbytes + 16, np.uint8)
+        raw[shift:shift + a.nbytes] = a.view(np.uint8).reshape(-1)
+        buf = up(raw)
+        return buf, buf.offset(shift)
+    s_buf, s_ptr = shifted(s.view(np.uint16))
+    z_buf, z_ptr = shifted(z.view(np.uint16))
+    ws = hip.DeviceBuffer(kernels.qgemm_q4g128_tall_workspace_bytes(b, k))
+    d_y = hip.DeviceBuffer(b * n * 4)
+    d_y.fill(0xFF)
+    kernels.launch_qgemm_q4g128_tall(up(xb), up(qw), s_ptr, z_ptr, d_y, ws, b, n, k,
+                                     bias=up(bias), f32_out=True)
+    hip.synchronize()
+    got = d_y.to_numpy(np.float32, (b, n))
+    want = O.qgemm_q4g128_f32(xb, qw, s, z, b, n, k, bias)
+    assert_parity(got, want, max_abs=2e-4, max_rel=1e-3, what=f"scales at +{shift} bytes")
+    del s_buf, z_buf
+
+
+def test_q4g128_workspace_kernel_is_deterministic():
+    # parts of a tile split over K are summed in part order: two launches, the same bits
+    rng = np.random.default_rng(92)
+    b, n, k = 300, 1000, 4096
+    qw, s, z = _q4(rng, n, k)
+    xb = O.f32_to_bf16_bits(rng.standard_normal((b, k), np.float32))
+    first = _gemm_q4_ws(xb, qw, s, z, b, n, k, None, f32_out=True)
+    again = _gemm_q4_ws(xb, qw, s, z, b, n, k, None, f32_out=True, ws_fill=0x00)
+    assert np.array_equal(first.view(np.uint32), again.view(np.uint32))
+
+
 def test_q4g128_workspace_kernel_one_hot_rows_read_back_dequantised_columns():
     # orientation, nibble order, the pair order the first pass writes, the LDS swizzles of x
     # and of the weights, and the zero-point product in one exact check: row i of x is the unit
