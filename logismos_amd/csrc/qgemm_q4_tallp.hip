@@ -230,10 +230,10 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
     // for the zero-point product (lane (r, h) holds row wr + 32 i + r, group 2 p + h of pair
     // p; the first pass wrote them as [row tile][block][h][row][p], so a wave reads 512
     // consecutive bytes x W).  Six loads per block and wave, written as assembly with the
-    // waits for them spelled out below: for loads it can see the compiler waits with
-    // vmcnt(0), which also waits for every request of the groups ahead and takes the ring's
-    // depth away.  A register loaded here must not be touched before `small_loads_landed`
-    // has named it.
+    // wait for them spelled out below, once per block: for loads it can see the compiler
+    // waits with vmcnt(0) wherever a value is used, in every group, which also waits for
+    // every request of the groups ahead and takes the ring's depth away.  A register loaded
+    // here must not be touched before `small_loads_landed` has named it.
     struct Small {
         TpRegs<unsigned, W> s[2], z[2];
         TpRegs<float, W> xs[2];
@@ -271,13 +271,15 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
                 asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(v.xs[i].raw) : "v"(xsoff[i]), "s"(xb) : "memory");
         }
     };
-    // waits until at most `younger` of this wave's loads and requests are outstanding (they
-    // complete in the order they were issued) and hands the registers over
-    auto small_loads_landed = [&](auto younger_c, Small& v) {
-        asm volatile("s_waitcnt vmcnt(%6)"
-                     : "+v"(v.s[0].raw), "+v"(v.s[1].raw), "+v"(v.z[0].raw), "+v"(v.z[1].raw), "+v"(v.xs[0].raw),
-                       "+v"(v.xs[1].raw)
-                     : "n"(decltype(younger_c)::value)
+    // Waits for everything this wave has outstanding and hands the registers over.  (Not
+    // "at most the requests issued behind them": whether loads into registers and requests
+    // into LDS complete in order with each other is not relied on.  The requests of the group
+    // after next, issued most of a group ago, are waited for with them -- once per block.)
+    auto small_loads_landed = [&](Small& v) {
+        asm volatile("s_waitcnt vmcnt(0)"
+                     : "+v"(v.s[0].raw), "+v"(v.s[1].raw), "+v"(v.z[0].raw), "+v"(v.z[1].raw),
+                       "+v"(v.xs[0].raw), "+v"(v.xs[1].raw)
+                     :
                      : "memory");
     };
     // One block's values are in use while the next one's are on their way (W = 1), or the
@@ -298,9 +300,7 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
     gload_small(g_begin, cur);
     request_group(g_begin, 0);
     request_group(g_begin + 1, kTpBufBytes);  // (a range holds at least one pair)
-    // (everything issued so far: the order in which loads into registers and requests into
-    // LDS issued back to back complete is not relied on)
-    small_loads_landed(ic<0>{}, cur);
+    small_loads_landed(cur);
 
     // The requests of the group after next go into the buffer everybody stopped reading before
     // this group's barrier.  (Measured and not kept: the two waves of a SIMD issuing theirs at
@@ -315,8 +315,8 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
     };
 
     // One group of 128 columns out of the buffer at byte `buf_off` of the ring; U: the group's
-    // place in its block.  A wave's loads and requests complete in the order they were
-    // issued, so "at most the n youngest outstanding" names what has landed.
+    // place in its block.  A wave's requests complete in the order they were issued, so "at
+    // most the six youngest outstanding" names what has landed.
     auto group = [&](auto u_c, int g, int buf_off) {
         constexpr int U = decltype(u_c)::value;
         constexpr int PAR = U & 1;
@@ -329,7 +329,6 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
         // after the barrier everybody's requests for this group have landed, and everybody is
         // done reading the buffer of the group before it, which the group after next reuses
         __builtin_amdgcn_s_barrier();
-        // (the small loads first: what waits for them need not wait for the requests)
         if constexpr (W == 1) {
             if (U == 1 && g + 1 < groups) gload_small(g + 1, nxt);
         }
@@ -414,9 +413,7 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
         });
         if constexpr (W > 1 && U == 0) {
             // the block's values, requested at the end of the group before this one
-            // (with everything else this wave has outstanding: the requests of the group
-            // after next, issued most of a group ago -- once per block)
-            if (g > g_begin) small_loads_landed(ic<0>{}, cur);
+            if (g > g_begin) small_loads_landed(cur);
         }
         // y += scale * acc  (measured and not kept: the last two steps tile by tile with a
         // tile's multiply-adds between the MFMAs of the tiles after it; no change)
@@ -450,7 +447,7 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
                                                                       yacc[i][j], 0, 0, 0);
             if constexpr (W == 1) {
                 if (g + 1 < groups) {
-                    small_loads_landed(ic<0>{}, nxt);
+                    small_loads_landed(nxt);
                     cur = nxt;
                 }
             } else if constexpr (U == BL - 1) {
