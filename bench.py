@@ -634,6 +634,56 @@ def bench_q4_tall(args):
             "parity_max_abs_vs_oracle_sample": parity}
 
 
+def bench_mixed_step_config4(args):
+    """Config 4's packed batch (48 decode rows + 16 prefill chunks of 512 tokens = 8240 rows)
+    through the whole step executor at Qwen3-8B geometry, 36 layers: the rows go through the
+    tiled Q4G128 GEMMs, rope + KV write, the chunked-prefill and decode attention kernels and
+    the small operators over all rows.  Timing only: the executor's many-row path is held
+    against the oracle at a few hundred rows in tests/ (a layer of 8240 rows on the CPU oracle
+    takes minutes); random nibbles as weights, pools of repeated random rows."""
+    from tests.gpu_harness import DecodeStepRunner
+    rng = np.random.default_rng(workloads.SEED + 44)
+    L, hidden, hq, hkv, inter = 36, 4096, 32, 8, 12288
+    c4 = workloads.config4()
+    new = c4["new_tokens"].astype(np.int32)
+    ctx = c4["context_lens"].astype(np.int32)
+    del c4
+    cfg, layers, batch = workloads.decode_step_problem(
+        rng, 1, hidden, hq, hkv, inter, ctx, new_tokens=new, random_nibbles=True,
+        pool_period_rows=8191)
+    stream = hip.Stream()
+    r = DecodeStepRunner(cfg, layers * L, batch, stream=stream, share_layer_data=True)
+    del layers
+    for _ in range(2):
+        r.launch()
+    stream.synchronize()
+    steps = 3
+    e0, e1 = hip.Event(), hip.Event()
+    e0.record(stream)
+    for _ in range(steps):
+        r.launch()
+    e1.record(stream)
+    e1.synchronize()
+    ms = e0.elapsed_ms(e1) / steps
+    out = O_bf16_finite(r)
+    rows = int(new.sum())
+    return {"workload": "config 4's mixed batch through the step executor: 64 sequences, "
+                        f"{rows} packed rows (48 decode + 16 x 512 prefill), sum of contexts "
+                        f"{int(ctx.sum())}, {L} layers at hidden {hidden}, {hq}/{hkv} heads, MLP "
+                        f"{inter}, Q4G128 weights, fp16 paged KV",
+            "ms_per_step": round(ms, 2), "ms_per_layer": round(ms / L, 3),
+            "new_tokens_per_s": round(rows / ms * 1e3, 0), "outputs_finite": out,
+            "parity": "not checked at this size (minutes on the CPU oracle); the same code path "
+                      "is checked against the oracle at 142-200 rows in "
+                      "tests/test_gpu_decode_step.py and per operator in "
+                      "tests/test_gpu_decode_step_many_rows_operators.py"}
+
+
+def O_bf16_finite(r) -> bool:
+    import oracle as O
+    return bool(np.isfinite(O.bf16_bits_to_f32(r.result_bits())).all())
+
+
 def bench_decode_step(args):
     """Config 5: full decode step, Qwen3-8B-style geometry, 32 live sequences."""
     import oracle as O
@@ -1155,7 +1205,7 @@ def main():
                          "profiler leave them out (--skip-kernels without --extras)")
     ap.add_argument("--workload", default="all",
                     choices=["all", "step", "config1", "config2", "config3", "config4",
-                             "config4_gemm", "turbo3", "headdim64", "two_streams"],
+                             "config4_gemm", "config4_step", "turbo3", "headdim64", "two_streams"],
                     help="all: the decode-step line with every leg inside it (default); "
                          "otherwise only that workload's own JSON line")
     args = ap.parse_args()
@@ -1168,12 +1218,13 @@ def main():
     kernels.library()
     args.steps_c5 = args.steps if args.steps is not None else 20
     args.warmup_c5 = args.warmup if args.warmup is not None else 3
-    if args.workload in ("config1", "config2", "config3", "config4", "config4_gemm", "turbo3",
-                         "headdim64", "two_streams"):
+    if args.workload in ("config1", "config2", "config3", "config4", "config4_gemm",
+                         "config4_step", "turbo3", "headdim64", "two_streams"):
         args.steps = args.steps if args.steps is not None else 200
         args.warmup = args.warmup if args.warmup is not None else 20
         leg = {"config1": bench_qgemv_q8, "config2": bench_paged_decode, "config3": bench_q4,
                "config4": bench_mixed_config4, "config4_gemm": bench_q4_tall,
+               "config4_step": bench_mixed_step_config4,
                "turbo3": bench_turbo3, "headdim64": bench_head_dim64,
                "two_streams": bench_two_streams}[args.workload]
         print(json.dumps(leg(args)))
@@ -1190,6 +1241,7 @@ def main():
         line["qgemv_q8_config1"] = bench_qgemv_q8(args)
         line["qgemm_q4_config3"] = bench_q4(args)
         line["qgemm_q4_tall_config4_rows"] = bench_q4_tall(args)
+        line["mixed_step_config4_rows"] = bench_mixed_step_config4(args)
         hd = bench_head_dim64(args)
         line["paged_attn_head_dim64"] = {k: hd[k] for k in (
             "value", "unit", "ms_per_step", "config", "roofline", "config2_batch_14q_2kv_heads",

@@ -348,28 +348,167 @@ __global__ __launch_bounds__(64) void rope_kv_write_kernel(
     }
 }
 
+// The same operator for many rows (a prefill chunk's worth and more), 128-wide heads, fp16
+// pools, fp32 parts in: one thread per four consecutive rotation pairs (i .. i + 3 with
+// i + 64 .. i + 67), 16-byte loads and 8-byte stores, 16 heads of a token per workgroup.  The
+// kernel above is one 64-thread workgroup per (token, head) with 4-byte accesses: at 8240
+// tokens x 48 heads that is 400 k workgroups for 300 MB.  Same sums in the same order, same
+// rotation, same rounding.
+constexpr int kRopeRowsKernelFrom = 64;  // tokens from which the many-row kernel is used
+__global__ __launch_bounds__(256) void rope_kv_write_rows_kernel(
+    const float* __restrict__ qkv_parts, int num_parts, int64_t part_stride,
+    const int32_t* __restrict__ positions, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, const int64_t* __restrict__ slot_mapping,
+    __half* __restrict__ q_out, __half* __restrict__ k_pool, __half* __restrict__ v_pool, int hq,
+    int hkv, int max_pos, const float* __restrict__ bias, int64_t total_quads) {
+    const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (gid >= total_quads) return;
+    const int heads = hq + 2 * hkv;
+    const int i = 4 * (int)(gid & 15);
+    const int64_t th = gid >> 4;
+    const int64_t t = th / heads;
+    const int head = (int)(th - t * heads);
+    const int64_t off = th * 128;
+    float4_t x0 = {0.0f, 0.0f, 0.0f, 0.0f}, x1 = x0;
+    for (int q = 0; q < num_parts; ++q) {
+        const float* src = qkv_parts + (int64_t)q * part_stride + off + i;
+        const float4_t a = *reinterpret_cast<const float4_t*>(src);
+        const float4_t b = *reinterpret_cast<const float4_t*>(src + 64);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            x0[e] += a[e];
+            x1[e] += b[e];
+        }
+    }
+    if (bias) {
+        const float4_t b0 = *reinterpret_cast<const float4_t*>(bias + head * 128 + i);
+        const float4_t b1 = *reinterpret_cast<const float4_t*>(bias + head * 128 + i + 64);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            x0[e] += b0[e];
+            x1[e] += b1[e];
+        }
+    }
+    auto store4 = [](__half* dst, const float4_t& v) {
+        uint2_t o;
+#pragma unroll
+        for (int e = 0; e < 2; ++e)
+            o[e] = (unsigned)__half_as_ushort(__float2half_rn(v[2 * e])) |
+                   ((unsigned)__half_as_ushort(__float2half_rn(v[2 * e + 1])) << 16);
+        *reinterpret_cast<uint2_t*>(dst) = o;
+    };
+    if (head < hq + hkv) {
+        int pos = positions[t];
+        pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
+        const float4_t c = *reinterpret_cast<const float4_t*>(cos_t + (int64_t)pos * 64 + i);
+        const float4_t sn = *reinterpret_cast<const float4_t*>(sin_t + (int64_t)pos * 64 + i);
+        float4_t y0, y1;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            y0[e] = x0[e] * c[e] - x1[e] * sn[e];
+            y1[e] = x0[e] * sn[e] + x1[e] * c[e];
+        }
+        __half* dst;
+        if (head < hq) {
+            dst = q_out + (t * hq + head) * 128;
+        } else {
+            const int64_t slot = slot_mapping[t];
+            if (slot < 0) return;
+            dst = k_pool + (slot * hkv + (head - hq)) * 128;
+        }
+        store4(dst + i, y0);
+        store4(dst + i + 64, y1);
+    } else {
+        const int64_t slot = slot_mapping[t];
+        if (slot < 0) return;
+        __half* dst = v_pool + (slot * hkv + (head - hq - hkv)) * 128;
+        store4(dst + i, x0);
+        store4(dst + i + 64, x1);
+    }
+}
+
 // out[t][j] = bf16( silu(gate[t][j]) * up[t][j] ), gate_up = [t][gate(0..inter) | up(0..inter)]
+// V: elements per thread (8 where inter is a multiple of 8: 32-byte loads of the fp32 parts,
+// one 16-byte store; over thousands of rows the operator reads a gigabyte).
+template <int V>
 __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restrict__ gate_up,
                                                        const float* __restrict__ parts,
                                                        int num_parts, int64_t part_stride,
                                                        uint16_t* __restrict__ out, int inter,
                                                        int64_t total) {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * V;
     if (idx >= total) return;
     const int64_t t = idx / inter;
     const int64_t j = idx - t * inter;
-    float g = 0.0f, u = 0.0f;
+    float g[V], u[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) g[e] = u[e] = 0.0f;
     if (gate_up) {
-        g = bf16_to_f32(gate_up[t * 2 * inter + j]);
-        u = bf16_to_f32(gate_up[t * 2 * inter + inter + j]);
+        const uint16_t* gp = gate_up + t * 2 * inter + j;
+        if constexpr (V == 8) {
+            const uint4_t gv = *reinterpret_cast<const uint4_t*>(gp);
+            const uint4_t uv = *reinterpret_cast<const uint4_t*>(gp + inter);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                g[e] = bf16_to_f32((uint16_t)(gv[e >> 1] >> (16 * (e & 1))));
+                u[e] = bf16_to_f32((uint16_t)(uv[e >> 1] >> (16 * (e & 1))));
+            }
+        } else {
+            g[0] = bf16_to_f32(gp[0]);
+            u[0] = bf16_to_f32(gp[inter]);
+        }
     } else {
         for (int q = 0; q < num_parts; ++q) {
-            g += parts[(int64_t)q * part_stride + t * 2 * inter + j];
-            u += parts[(int64_t)q * part_stride + t * 2 * inter + inter + j];
+            const float* gp = parts + (int64_t)q * part_stride + t * 2 * inter + j;
+            if constexpr (V == 8) {
+#pragma unroll
+                for (int v4 = 0; v4 < 2; ++v4) {
+                    const float4_t gv = *reinterpret_cast<const float4_t*>(gp + 4 * v4);
+                    const float4_t uv = *reinterpret_cast<const float4_t*>(gp + inter + 4 * v4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        g[4 * v4 + e] += gv[e];
+                        u[4 * v4 + e] += uv[e];
+                    }
+                }
+            } else {
+                g[0] += gp[0];
+                u[0] += gp[inter];
+            }
         }
     }
-    const float sg = g / (1.0f + expf(-g));
-    out[idx] = f32_to_bf16(sg * u);
+    uint16_t o[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+        const float sg = g[e] / (1.0f + expf(-g[e]));
+        o[e] = f32_to_bf16(sg * u[e]);
+    }
+    if constexpr (V == 8) {
+        uint4_t ov;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ov[e] = (unsigned)o[2 * e] | ((unsigned)o[2 * e + 1] << 16);
+        *reinterpret_cast<uint4_t*>(out + idx) = ov;
+    } else {
+        out[idx] = o[0];
+    }
+}
+
+// (one launcher for both element widths: 8 per thread where rows of `inter` elements and the
+// buffers allow 16- and 32-byte accesses)
+static hipError_t silu_mul_launch(const uint16_t* gate_up, const float* parts, int num_parts,
+                                  int64_t part_stride, uint16_t* out, int inter, int64_t total,
+                                  hipStream_t st) {
+    const uintptr_t a = reinterpret_cast<uintptr_t>(gate_up) | reinterpret_cast<uintptr_t>(parts) |
+                        reinterpret_cast<uintptr_t>(out) | (uintptr_t)(part_stride * 4);
+    if (inter % 8 == 0 && (a & 15u) == 0) {
+        const int64_t threads = total / 8;
+        silu_mul_kernel<8><<<dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st>>>(
+            gate_up, parts, num_parts, part_stride, out, inter, total);
+    } else {
+        silu_mul_kernel<1><<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st>>>(
+            gate_up, parts, num_parts, part_stride, out, inter, total);
+    }
+    return hipGetLastError();
 }
 
 __global__ __launch_bounds__(256) void cast_f16_bf16_kernel(const __half* __restrict__ in,
@@ -525,6 +664,27 @@ extern "C" logismos_status_t logismos_launch_rope_kv_write_f32p_bias(
     if (!qkv_parts_f32 || !positions || !cos_f32 || !sin_f32 || !slot_mapping || !q_out_f16 ||
         !k_pool_f16 || !v_pool_f16)
         return hipErrorInvalidValue;
+    // many rows of 128-wide heads: the kernel with 16-byte accesses (everything it reads and
+    // writes 16-byte aligned)
+    const uintptr_t align = reinterpret_cast<uintptr_t>(qkv_parts_f32) |
+                            reinterpret_cast<uintptr_t>(bias_f32) |
+                            reinterpret_cast<uintptr_t>(cos_f32) |
+                            reinterpret_cast<uintptr_t>(sin_f32) |
+                            reinterpret_cast<uintptr_t>(q_out_f16) |
+                            reinterpret_cast<uintptr_t>(k_pool_f16) |
+                            reinterpret_cast<uintptr_t>(v_pool_f16);
+    if (head_dim == 128 && total_tokens >= lg::kRopeRowsKernelFrom && (align & 15u) == 0 &&
+        ((int64_t)total_tokens * width) % 4 == 0) {
+        const int64_t quads = (int64_t)total_tokens * (num_q_heads + 2 * num_kv_heads) * 16;
+        lg::rope_kv_write_rows_kernel<<<dim3((unsigned)((quads + 255) / 256)), dim3(256), 0,
+                                        static_cast<hipStream_t>(stream)>>>(
+            static_cast<const float*>(qkv_parts_f32), num_parts, (int64_t)total_tokens * width,
+            positions, static_cast<const float*>(cos_f32), static_cast<const float*>(sin_f32),
+            slot_mapping, static_cast<__half*>(q_out_f16), static_cast<__half*>(k_pool_f16),
+            static_cast<__half*>(v_pool_f16), num_q_heads, num_kv_heads, max_pos,
+            static_cast<const float*>(bias_f32), quads);
+        return hipGetLastError();
+    }
     dim3 grid(num_q_heads + 2 * num_kv_heads, total_tokens);
     const auto kernel = head_dim == 128 ? lg::rope_kv_write_kernel<false, true>
                                         : lg::rope_kv_write_kernel<false, false>;
@@ -591,11 +751,9 @@ extern "C" logismos_status_t logismos_launch_silu_mul_f32p(const void* parts_f32
         return hipErrorInvalidValue;
     if (!parts_f32 || !out_bf16) return hipErrorInvalidValue;
     const int64_t total = (int64_t)rows * inter;
-    lg::silu_mul_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
-                          static_cast<hipStream_t>(stream)>>>(
-        nullptr, static_cast<const float*>(parts_f32), num_parts, (int64_t)rows * 2 * inter,
-        static_cast<uint16_t*>(out_bf16), inter, total);
-    return hipGetLastError();
+    return lg::silu_mul_launch(nullptr, static_cast<const float*>(parts_f32), num_parts,
+                               (int64_t)rows * 2 * inter, static_cast<uint16_t*>(out_bf16), inter,
+                               total, static_cast<hipStream_t>(stream));
 }
 
 extern "C" logismos_status_t logismos_launch_silu_mul_bf16(const void* gate_up_bf16,
@@ -605,11 +763,9 @@ extern "C" logismos_status_t logismos_launch_silu_mul_bf16(const void* gate_up_b
         return hipErrorInvalidValue;
     if (!gate_up_bf16 || !out_bf16) return hipErrorInvalidValue;
     const int64_t total = (int64_t)rows * inter;
-    lg::silu_mul_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
-                          static_cast<hipStream_t>(stream)>>>(
-        static_cast<const uint16_t*>(gate_up_bf16), nullptr, 0, 0,
-        static_cast<uint16_t*>(out_bf16), inter, total);
-    return hipGetLastError();
+    return lg::silu_mul_launch(static_cast<const uint16_t*>(gate_up_bf16), nullptr, 0, 0,
+                               static_cast<uint16_t*>(out_bf16), inter, total,
+                               static_cast<hipStream_t>(stream));
 }
 
 extern "C" logismos_status_t logismos_launch_cast_f16_bf16(const void* in_f16, void* out_bf16,

@@ -137,7 +137,8 @@ def qgemm_q4_algorithmic_bytes(b, n, k) -> int:
 
 def decode_step_problem(rng, num_layers, hidden, hq, hkv, inter, ctx, d=128, block_size=16,
                         max_pos=None, eps=1e-6, theta=1e6, random_nibbles=False, vocab=0,
-                        kv_turbo3=False, new_tokens=None, qkv_bias=False):
+                        kv_turbo3=False, new_tokens=None, qkv_bias=False,
+                        pool_period_rows=None):
     """A decode-step problem: `ctx[s]` is the context of sequence s INCLUDING its new tokens
     (one per sequence, or `new_tokens[s]` for a mixed chunked-prefill + decode batch: the batch
     then has sum(new_tokens) packed rows).  qkv_bias: every layer's q/k/v projection carries a
@@ -146,7 +147,8 @@ def decode_step_problem(rng, num_layers, hidden, hq, hkv, inter, ctx, d=128, blo
     random_nibbles, for timing-only runs), RMSNorm gains 1+N(0,0.02), RoPE theta 1e6.
     With vocab > 0 the batch also carries token ids, a bf16 embedding table and a Q4G128
     lm_head (tokens in, tokens out).  kv_turbo3: the pools are TurboQuant 3-bit pools
-    (uint8 [rows][hkv*56]) holding the encoded random rows."""
+    (uint8 [rows][hkv*56]) holding the encoded random rows.  pool_period_rows: the pools
+    repeat that many random rows (timing runs of full-size batches)."""
     import oracle as O
     ctx = np.asarray(ctx, np.int32)
     new = np.ones(len(ctx), np.int32) if new_tokens is None else np.asarray(new_tokens, np.int32)
@@ -164,7 +166,12 @@ def decode_step_problem(rng, num_layers, hidden, hq, hkv, inter, ctx, d=128, blo
         return O.quantize_q4g128(w, n, k)
 
     base = paged_case(rng, new, ctx - new, hq=hq, hkv=hkv, d=d, block_size=block_size,
-                      spare_frac=0.05)
+                      spare_frac=0.05, pool_period_rows=pool_period_rows)
+
+    def pool(rows):
+        n = min(rows, pool_period_rows or rows)
+        p = rng.standard_normal((n, hkv * d), np.float32).astype(np.float16)
+        return p if n == rows else np.resize(p, (rows, hkv * d))
     layers = []
     for _ in range(num_layers):
         rows = base["k_pool"].shape[0]
@@ -173,8 +180,7 @@ def decode_step_problem(rng, num_layers, hidden, hq, hkv, inter, ctx, d=128, blo
             norm2=(1 + 0.02 * rng.standard_normal(hidden)).astype(np.float32),
             qkv=q4((hq + 2 * hkv) * d, hidden), o=q4(hidden, hq * d),
             gate_up=q4(2 * inter, hidden), down=q4(hidden, inter),
-            k_pool=rng.standard_normal((rows, hkv * d), np.float32).astype(np.float16),
-            v_pool=rng.standard_normal((rows, hkv * d), np.float32).astype(np.float16)))
+            k_pool=pool(rows), v_pool=pool(rows)))
         if qkv_bias:
             layers[-1]["qkv_bias"] = rng.standard_normal((hq + 2 * hkv) * d).astype(np.float32)
     # the RoPE tables cover every position the block tables can hold
