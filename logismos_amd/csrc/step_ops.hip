@@ -264,6 +264,19 @@ __global__ __launch_bounds__(256) void silu_mul_xprep_kernel(const float* __rest
 // as they are, go to the pools at the token's slot: as fp16 rows, or (T3) rounded to fp16
 // like those and then encoded as turbo3 head rows -- the lane layout of the rotation is
 // the encoder's.
+// One rotation pair.  Spelled out with fmaf so that every kernel that rotates rounds alike
+// (left to the compiler, `x0 * c - x1 * s` contracts one way in a scalar loop and another in an
+// unrolled one).
+__device__ __forceinline__ void rope_rotate(float x0, float x1, float c, float s, float& y0,
+                                            float& y1) {
+    y0 = fmaf(x0, c, -(x1 * s));
+    y1 = fmaf(x0, s, x1 * c);
+    // (the fp32 values are the results: without this the compiler may fold the conversion to
+    // fp16 that follows into the multiply-add, v_fma_mixlo_f16, which rounds once where the
+    // reference rounds to fp32 and then to fp16)
+    asm volatile("" : "+v"(y0), "+v"(y1));
+}
+
 template <bool T3, bool D128>
 __global__ __launch_bounds__(64) void rope_kv_write_kernel(
     const uint16_t* __restrict__ qkv, const float* __restrict__ qkv_parts, int num_parts,
@@ -311,8 +324,8 @@ __global__ __launch_bounds__(64) void rope_kv_write_kernel(
             pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
             const float c = cos_t[(int64_t)pos * HALF + i];
             const float s = sin_t[(int64_t)pos * HALF + i];
-            const float y0 = x0 * c - x1 * s;
-            const float y1 = x0 * s + x1 * c;
+            float y0, y1;
+            rope_rotate(x0, x1, c, s, y0, y1);
             if (head < hq) {
                 __half* dst = q_out + (t * hq + head) * D;
                 dst[i] = __float2half_rn(y0);
@@ -405,8 +418,10 @@ __global__ __launch_bounds__(256) void rope_kv_write_rows_kernel(
         float4_t y0, y1;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            y0[e] = x0[e] * c[e] - x1[e] * sn[e];
-            y1[e] = x0[e] * sn[e] + x1[e] * c[e];
+            float a, b;
+            rope_rotate(x0[e], x1[e], c[e], sn[e], a, b);
+            y0[e] = a;
+            y1[e] = b;
         }
         __half* dst;
         if (head < hq) {

@@ -226,6 +226,58 @@ def test_f32_parts_variants_add_the_parts_in_order():
     assert np.array_equal(d_v3.to_numpy(np.uint8, v3.shape), v3_want)
 
 
+def test_rope_kv_write_over_many_rows_equals_the_per_head_kernel_bit_for_bit():
+    # from 64 tokens on 128-wide heads take the kernel with four rotation pairs per thread;
+    # below, one workgroup per (token, head).  The same 200 tokens in one launch and in
+    # launches of 50: same q rows, same pool rows, bit for bit -- with three parts, a bias, a
+    # token without a slot (skipped) and a position at the end of the table -- and both against
+    # the oracle.
+    rng = np.random.default_rng(77)
+    t, hq, hkv, d, bs, nblk, max_pos = 200, 8, 2, 128, 16, 20, 700
+    width = (hq + 2 * hkv) * d
+    parts = rng.standard_normal((3, t, width), np.float32)
+    bias = rng.standard_normal(width).astype(np.float32)
+    positions = rng.integers(0, max_pos, size=t).astype(np.int32)
+    positions[:3] = [0, max_pos - 1, 17]
+    slots = rng.permutation(nblk * bs)[:t].astype(np.int64)
+    slots[5] = -1
+    cos, sin = O.build_rope_table_f32(max_pos, d, 1_000_000.0)
+    k0 = rng.standard_normal((nblk * bs, hkv * d), np.float32).astype(np.float16)
+    v0 = rng.standard_normal((nblk * bs, hkv * d), np.float32).astype(np.float16)
+    dev = hip.DeviceBuffer.from_numpy
+
+    def run(chunk):
+        d_kp, d_vp, d_q = dev(k0), dev(v0), hip.DeviceBuffer(t * hq * d * 2)
+        for r0 in range(0, t, chunk):
+            n = min(chunk, t - r0)
+            sub = np.ascontiguousarray(parts[:, r0:r0 + n])
+            d_qs = hip.DeviceBuffer(n * hq * d * 2)
+            kernels.launch_rope_kv_write_f32p(dev(sub), 3, dev(positions[r0:r0 + n]), dev(cos),
+                                              dev(sin), dev(slots[r0:r0 + n]), d_qs, d_kp, d_vp, n,
+                                              hq, hkv, d, max_pos, bias=dev(bias))
+            hip.synchronize()
+            d_q.copy_from_device(d_qs, n * hq * d * 2, dst_offset=r0 * hq * d * 2)
+        hip.synchronize()
+        return (d_q.to_numpy(np.uint16, (t, hq, d)), d_kp.to_numpy(np.uint16, k0.shape),
+                d_vp.to_numpy(np.uint16, v0.shape))
+    q_rows, k_rows, v_rows = run(t)       # one launch: the many-row kernel
+    q_head, k_head, v_head = run(50)      # launches of 50 tokens: the per-head kernel
+    assert np.array_equal(q_rows, q_head)
+    assert np.array_equal(k_rows, k_head)
+    assert np.array_equal(v_rows, v_head)
+    k_want, v_want = k0.copy(), v0.copy()
+    keep = slots >= 0
+    q_want = OS.rope_kv_write((parts[0] + parts[1] + parts[2] + bias)[keep], positions[keep], cos,
+                              sin, slots[keep], k_want, v_want, hq, hkv, d)
+    assert_parity(q_rows.view(np.float16)[keep], q_want, max_abs=1e-3, max_rel=2e-3,
+                  what="rope rows q")
+    assert_parity(k_rows.view(np.float16), k_want, max_abs=1e-3, max_rel=2e-3, what="rope rows k")
+    assert_parity(v_rows.view(np.float16), v_want, max_abs=1e-3, max_rel=2e-3, what="rope rows v")
+    # the token without a slot left both pools alone (its q row is still written)
+    untouched = np.setdiff1d(np.arange(nblk * bs), slots[keep])
+    assert np.array_equal(k_rows[untouched], k0.view(np.uint16)[untouched])
+
+
 def _unprepare(buf, b, k):
     """prepared layout -> (bf16 bits [b][k], group sums [b][k/128])"""
     bp = 16 if b <= 16 else 32
