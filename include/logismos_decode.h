@@ -196,6 +196,17 @@ logismos_status_t logismos_launch_qgemm_q4g128_bf16_mfma(const void* x_bf16, con
 logismos_status_t logismos_check_qgemm_q4g128_tall_shape(int m, int n, int k, char* msg,
                                                          size_t msg_cap);
 size_t logismos_qgemm_q4g128_tall_workspace_bytes(int m, int k);
+/* The two halves of the launch below for a caller whose producer writes x where the kernel
+ * wants it: `..._tall_prepared` is the product alone over a workspace that already holds x in
+ * the kernel's operand order with its group sums (the first `m_pad*K*2` bytes and the sums
+ * behind them, as `logismos_launch_silu_mul_f32p_tall` writes them), `..._pairs_per_load` the
+ * one parameter of that layout that depends on the weights (how many pairs of groups of K the
+ * kernel loads scales and zeros for at once: 4, 2 or 1 by K and their alignment).  No
+ * counterpart in the reference: `linear_t` takes plain rows. */
+int logismos_qgemm_q4g128_tall_pairs_per_load(int k, const void* scale_f16, const void* zero_f16);
+logismos_status_t logismos_launch_qgemm_q4g128_tall_prepared(
+    const void* qw_u8, const void* scale_f16, const void* zero_f16, const void* bias_f32, void* y,
+    int y_is_f32, void* workspace, int m, int n, int k, logismos_stream_t stream);
 logismos_status_t logismos_launch_qgemm_q4g128_tall(const void* x_bf16, const void* qw_u8,
                                                     const void* scale_f16, const void* zero_f16,
                                                     const void* bias_f32, void* y, int y_is_f32,
@@ -519,6 +530,15 @@ logismos_status_t logismos_launch_rope_kv_write_f32p_turbo3_bias(
 logismos_status_t logismos_launch_silu_mul_f32p(const void* parts_f32, int num_parts,
                                                 void* out_bf16, int rows, int inter,
                                                 logismos_stream_t stream);
+
+/* SwiGLU over the fp32 parts with the result written as the operand of the many-row GEMM
+ * (`logismos_launch_qgemm_q4g128_tall_prepared` over the same workspace, K = inter a multiple
+ * of 256 * pairs_per_load): x in the kernel's order, rows padded with zeros to its 128-row
+ * tiles, the group sums behind it. */
+logismos_status_t logismos_launch_silu_mul_f32p_tall(const void* parts_f32, int num_parts,
+                                                     void* workspace, int rows, int inter,
+                                                     int pairs_per_load,
+                                                     logismos_stream_t stream);
 
 /* The same with the result in the prepared layout of the next GEMM (rows <= 32,
  * width % 128 == 0; see `logismos_q4_xprep_bytes`). */

@@ -311,8 +311,21 @@ extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_c
             LG_TRY(logismos_launch_add_rms_norm_f32p(batch->hidden_f32, w.t_proj, 1, L.norm2_w_f32,
                                                      w.t_xn, t, c.hidden, c.rms_eps, stream));
             LG_TRY(gemm(w.t_xn, L.gate_up, nullptr, w.t_gu, 2 * c.intermediate, c.hidden));
-            LG_TRY(logismos_launch_silu_mul_f32p(w.t_gu, 1, w.t_act, t, c.intermediate, stream));
-            LG_TRY(gemm(w.t_act, L.down, nullptr, w.t_proj, c.hidden, c.intermediate));
+            if (logismos_check_qgemm_q4g128_tall_shape(t, c.hidden, c.intermediate, nullptr, 0) == 0) {
+                // the activation goes straight into the down projection's workspace, in the
+                // kernel's operand order: no first pass over it
+                LG_TRY(logismos_launch_silu_mul_f32p_tall(
+                    w.t_gu, 1, w.t_gemm, t, c.intermediate,
+                    logismos_qgemm_q4g128_tall_pairs_per_load(c.intermediate, L.down.scale,
+                                                              L.down.zero),
+                    stream));
+                LG_TRY(logismos_launch_qgemm_q4g128_tall_prepared(L.down.qw, L.down.scale, L.down.zero,
+                                                                  nullptr, w.t_proj, 1, w.t_gemm, t,
+                                                                  c.hidden, c.intermediate, stream));
+            } else {
+                LG_TRY(logismos_launch_silu_mul_f32p(w.t_gu, 1, w.t_act, t, c.intermediate, stream));
+                LG_TRY(gemm(w.t_act, L.down, nullptr, w.t_proj, c.hidden, c.intermediate));
+            }
             res_parts = 1;
         }
         LG_TRY(logismos_launch_add_rms_norm_f32p(batch->hidden_f32, w.t_proj, res_parts,

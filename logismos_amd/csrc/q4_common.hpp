@@ -54,6 +54,36 @@ __host__ __device__ inline size_t xprep_bytes(int b, int k) {
     return xprep_xg_offset(b, k) + (size_t)(k / 128) * xprep_bp(b) * 4;
 }
 
+// Workspace of the Q4G128 GEMM for many rows (qgemm_q4_tallp.hip), first part: what its first
+// pass -- or the operator that produces x -- writes.
+//   xp  bf16  [m_pad][K]  x in pair order per 16-byte chunk, rows >= m zero, m_pad = m rounded
+//                         up to the kernel's 128-row tiles
+//   xs  float             the sum of the bf16 values of every row and group of 128 columns,
+//                         as [row tile][block of w pairs of groups][group's place in its
+//                         pair][row of the tile][pair]; w = pairs of groups the kernel loads
+//                         at once (tall_pairs_per_load)
+constexpr int kTallTileRows = 128;
+__host__ __device__ inline int tall_padded_rows(int m) {
+    return (m + kTallTileRows - 1) / kTallTileRows * kTallTileRows;
+}
+__host__ __device__ inline size_t tall_sums_offset(int m, int k) {
+    return ((size_t)tall_padded_rows(m) * k * 2 + 255) & ~(size_t)255;
+}
+__host__ __device__ inline int64_t tall_sum_index(int64_t row, int g, int k, int w) {
+    const int bl = 2 * w;
+    const int64_t block = (row / kTallTileRows) * ((k >> 7) / bl) + g / bl;
+    const int in_block = g % bl;
+    return ((block * 2 + (in_block & 1)) * kTallTileRows + row % kTallTileRows) * w + (in_block >> 1);
+}
+// as many pairs of groups per load as K (whole blocks) and the alignment of the scales and
+// zeros (a load of 4, 8 or 16 bytes per row) allow
+inline int tall_pairs_per_load(int k, const void* scale, const void* zero) {
+    const uintptr_t a = reinterpret_cast<uintptr_t>(scale) | reinterpret_cast<uintptr_t>(zero);
+    if (k % 1024 == 0 && (a & 15u) == 0) return 4;
+    if (k % 512 == 0 && (a & 7u) == 0) return 2;
+    return 1;
+}
+
 inline int device_cu_count() {
     static const int count = [] {
         int dev = 0, cus = 0;

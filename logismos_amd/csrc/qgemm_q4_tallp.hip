@@ -65,10 +65,9 @@ constexpr int kTpTileElems = kTpTileM * kTpTileN;
 constexpr int kTpMaxParts = 512;          // partial tiles the workspace holds (fp32, 128 KiB each)
 constexpr int kTpMinGroupsPerPart = 4;    // a part of a tile takes at least four groups of K
 
-__host__ __device__ inline int tp_padded_rows(int m) { return (m + kTpTileM - 1) / kTpTileM * kTpTileM; }
-__host__ __device__ inline size_t tp_sums_offset(int m, int k) {
-    return ((size_t)tp_padded_rows(m) * k * 2 + 255) & ~(size_t)255;
-}
+static_assert(kTpTileM == kTallTileRows, "the layout helpers of q4_common.hpp are for this tile");
+__host__ __device__ inline int tp_padded_rows(int m) { return tall_padded_rows(m); }
+__host__ __device__ inline size_t tp_sums_offset(int m, int k) { return tall_sums_offset(m, k); }
 __host__ __device__ inline size_t tp_partials_offset(int m, int k) {
     return (tp_sums_offset(m, k) + (size_t)tp_padded_rows(m) * (k / 128) * 4 + 255) & ~(size_t)255;
 }
@@ -107,12 +106,7 @@ __global__ __launch_bounds__(256) void q4_tall_prepare_kernel(const uint16_t* __
     if (row < m) v = *reinterpret_cast<const uint4_t*>(x + row * k + c * 8);
     const float gs = row16_sum(sum8_bf16(v));
     *reinterpret_cast<uint4_t*>(xp + row * k + c * 8) = pair_order(v);
-    if ((threadIdx.x & 15) == 0) {
-        const int g = (int)(c >> 4), bl = 2 * w;
-        const int64_t block = (row / kTpTileM) * ((k >> 7) / bl) + g / bl;
-        const int in_block = g % bl;
-        xs[((block * 2 + (in_block & 1)) * kTpTileM + row % kTpTileM) * w + (in_block >> 1)] = gs;
-    }
+    if ((threadIdx.x & 15) == 0) xs[tall_sum_index(row, (int)(c >> 4), k, w)] = gs;
 }
 
 // W values a lane loads at once, as one register operand of an assembly statement: a vector
@@ -522,13 +516,8 @@ __global__ __launch_bounds__(256) void q4_tall_reduce_kernel(const float* __rest
     else static_cast<uint16_t*>(y_out)[(int64_t)gr * n + gn] = f32_to_bf16_rne(acc);
 }
 
-// Pairs of groups per small load: as many as K (whole blocks) and the alignment of the scales
-// and zeros (a load of 4, 8 or 16 bytes per row) allow.
 inline int tp_pairs_per_load(int k, const void* scale, const void* zero) {
-    const uintptr_t a = reinterpret_cast<uintptr_t>(scale) | reinterpret_cast<uintptr_t>(zero);
-    if (k % 1024 == 0 && (a & 15u) == 0) return 4;
-    if (k % 512 == 0 && (a & 7u) == 0) return 2;
-    return 1;
+    return tall_pairs_per_load(k, scale, zero);
 }
 
 template <bool F32OUT, int W>
@@ -592,29 +581,36 @@ extern "C" size_t logismos_qgemm_q4g128_tall_workspace_bytes(int m, int k) {
     return lg::tp_partials_offset(m, k) + (size_t)lg::kTpMaxParts * lg::kTpTileElems * 4;
 }
 
-extern "C" logismos_status_t logismos_launch_qgemm_q4g128_tall(
-    const void* x_bf16, const void* qw_u8, const void* scale_f16, const void* zero_f16,
-    const void* bias_f32, void* y, int y_is_f32, void* workspace, int m, int n, int k,
-    logismos_stream_t stream) {
+static logismos_status_t tall_args_ok(const void* qw_u8, const void* scale_f16,
+                                      const void* zero_f16, const void* y, const void* workspace,
+                                      int m, int n, int k) {
     if (logismos_check_qgemm_q4g128_tall_shape(m, n, k, nullptr, 0) != 0)
         return hipErrorInvalidValue;
-    if (!x_bf16 || !qw_u8 || !scale_f16 || !zero_f16 || !y || !workspace)
-        return hipErrorInvalidValue;
-    if ((reinterpret_cast<uintptr_t>(qw_u8) | reinterpret_cast<uintptr_t>(x_bf16) |
-         reinterpret_cast<uintptr_t>(workspace)) & 15u)
+    if (!qw_u8 || !scale_f16 || !zero_f16 || !y || !workspace) return hipErrorInvalidValue;
+    if ((reinterpret_cast<uintptr_t>(qw_u8) | reinterpret_cast<uintptr_t>(workspace)) & 15u)
         return hipErrorInvalidValue;
     if ((reinterpret_cast<uintptr_t>(scale_f16) | reinterpret_cast<uintptr_t>(zero_f16)) & 3u)
         return hipErrorInvalidValue;
+    return hipSuccess;
+}
+
+extern "C" int logismos_qgemm_q4g128_tall_pairs_per_load(int k, const void* scale_f16,
+                                                         const void* zero_f16) {
+    return lg::tall_pairs_per_load(k, scale_f16, zero_f16);
+}
+
+extern "C" logismos_status_t logismos_launch_qgemm_q4g128_tall_prepared(
+    const void* qw_u8, const void* scale_f16, const void* zero_f16, const void* bias_f32, void* y,
+    int y_is_f32, void* workspace, int m, int n, int k, logismos_stream_t stream) {
+    if (const logismos_status_t e = tall_args_ok(qw_u8, scale_f16, zero_f16, y, workspace, m, n, k))
+        return e;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int m_pad = lg::tp_padded_rows(m);
-    uint16_t* xp = static_cast<uint16_t*>(workspace);
-    float* xs = reinterpret_cast<float*>(static_cast<char*>(workspace) + lg::tp_sums_offset(m, k));
-    const int64_t chunks = (int64_t)m_pad * (k / 8);
-    const int w = lg::tp_pairs_per_load(k, scale_f16, zero_f16);
-    lg::q4_tall_prepare_kernel<<<dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st>>>(
-        static_cast<const uint16_t*>(x_bf16), xp, xs, m, m_pad, k, w);
+    const uint16_t* xp = static_cast<const uint16_t*>(workspace);
+    const float* xs =
+        reinterpret_cast<const float*>(static_cast<char*>(workspace) + lg::tp_sums_offset(m, k));
     float* partials = reinterpret_cast<float*>(static_cast<char*>(workspace) +
                                                lg::tp_partials_offset(m, k));
+    const int w = lg::tp_pairs_per_load(k, scale_f16, zero_f16);
     if (y_is_f32)
         return lg::tallp_launch_w<true>(w, xp, xs, partials, static_cast<const uint8_t*>(qw_u8),
                                         static_cast<const __half*>(scale_f16),
@@ -624,4 +620,24 @@ extern "C" logismos_status_t logismos_launch_qgemm_q4g128_tall(
                                      static_cast<const __half*>(scale_f16),
                                      static_cast<const __half*>(zero_f16),
                                      static_cast<const float*>(bias_f32), y, m, n, k, st);
+}
+
+extern "C" logismos_status_t logismos_launch_qgemm_q4g128_tall(
+    const void* x_bf16, const void* qw_u8, const void* scale_f16, const void* zero_f16,
+    const void* bias_f32, void* y, int y_is_f32, void* workspace, int m, int n, int k,
+    logismos_stream_t stream) {
+    if (const logismos_status_t e = tall_args_ok(qw_u8, scale_f16, zero_f16, y, workspace, m, n, k))
+        return e;
+    if (!x_bf16 || (reinterpret_cast<uintptr_t>(x_bf16) & 15u)) return hipErrorInvalidValue;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int m_pad = lg::tp_padded_rows(m);
+    uint16_t* xp = static_cast<uint16_t*>(workspace);
+    float* xs = reinterpret_cast<float*>(static_cast<char*>(workspace) + lg::tp_sums_offset(m, k));
+    const int64_t chunks = (int64_t)m_pad * (k / 8);
+    const int w = lg::tp_pairs_per_load(k, scale_f16, zero_f16);
+    lg::q4_tall_prepare_kernel<<<dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st>>>(
+        static_cast<const uint16_t*>(x_bf16), xp, xs, m, m_pad, k, w);
+    if (const hipError_t e = hipGetLastError()) return e;
+    return logismos_launch_qgemm_q4g128_tall_prepared(qw_u8, scale_f16, zero_f16, bias_f32, y,
+                                                      y_is_f32, workspace, m, n, k, stream);
 }

@@ -508,6 +508,51 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restric
     }
 }
 
+// The same operator writing the down projection's operand where the tiled GEMM for many rows
+// wants it (q4_common.hpp: x in pair order, rows padded with zeros to the 128-row tiles, the
+// group sums in the layout of the GEMM's loads) instead of plain bf16 rows: the GEMM's first
+// pass over x (a read and a write of the whole operand) is not needed then.  One thread per
+// 16-byte chunk of the padded operand; the 16 lanes of a row of lanes hold one group.
+__global__ __launch_bounds__(256) void silu_mul_tall_kernel(const float* __restrict__ parts,
+                                                            int num_parts, int64_t part_stride,
+                                                            uint16_t* __restrict__ xp,
+                                                            float* __restrict__ xs, int rows,
+                                                            int rows_pad, int inter, int w) {
+    const int64_t chunks_per_row = inter >> 3;
+    const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (id >= (int64_t)rows_pad * chunks_per_row) return;  // (whole rows of 16 lanes: inter % 128 == 0)
+    const int64_t t = id / chunks_per_row;
+    const int64_t c = id - t * chunks_per_row;
+    uint4_t o = {0u, 0u, 0u, 0u};
+    if (t < rows) {
+        float g[8], u[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) g[e] = u[e] = 0.0f;
+        for (int q = 0; q < num_parts; ++q) {
+            const float* gp = parts + (int64_t)q * part_stride + t * 2 * inter + c * 8;
+#pragma unroll
+            for (int v4 = 0; v4 < 2; ++v4) {
+                const float4_t gv = *reinterpret_cast<const float4_t*>(gp + 4 * v4);
+                const float4_t uv = *reinterpret_cast<const float4_t*>(gp + inter + 4 * v4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    g[4 * v4 + e] += gv[e];
+                    u[4 * v4 + e] += uv[e];
+                }
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float s0 = g[2 * e] / (1.0f + expf(-g[2 * e]));
+            const float s1 = g[2 * e + 1] / (1.0f + expf(-g[2 * e + 1]));
+            o[e] = (unsigned)f32_to_bf16(s0 * u[2 * e]) | ((unsigned)f32_to_bf16(s1 * u[2 * e + 1]) << 16);
+        }
+    }
+    const float gs = row16_sum(sum8_bf16(o));
+    *reinterpret_cast<uint4_t*>(xp + t * inter + c * 8) = pair_order(o);
+    if ((threadIdx.x & 15) == 0) xs[tall_sum_index(t, (int)(c >> 4), inter, w)] = gs;
+}
+
 // (one launcher for both element widths: 8 per thread where rows of `inter` elements and the
 // buffers allow 16- and 32-byte accesses)
 static hipError_t silu_mul_launch(const uint16_t* gate_up, const float* parts, int num_parts,
@@ -769,6 +814,30 @@ extern "C" logismos_status_t logismos_launch_silu_mul_f32p(const void* parts_f32
     return lg::silu_mul_launch(nullptr, static_cast<const float*>(parts_f32), num_parts,
                                (int64_t)rows * 2 * inter, static_cast<uint16_t*>(out_bf16), inter,
                                total, static_cast<hipStream_t>(stream));
+}
+
+extern "C" logismos_status_t logismos_launch_silu_mul_f32p_tall(const void* parts_f32,
+                                                                int num_parts, void* workspace,
+                                                                int rows, int inter,
+                                                                int pairs_per_load,
+                                                                logismos_stream_t stream) {
+    if (rows <= 0 || inter <= 0 || inter % 256 != 0 || num_parts <= 0 ||
+        (pairs_per_load != 1 && pairs_per_load != 2 && pairs_per_load != 4) ||
+        inter % (256 * pairs_per_load) != 0)
+        return hipErrorInvalidValue;
+    const int rows_pad = lg::tall_padded_rows(rows);
+    if ((int64_t)rows_pad * inter * 2 > (int64_t)INT32_MAX) return hipErrorInvalidValue;
+    if (!parts_f32 || !workspace) return hipErrorInvalidValue;
+    if ((reinterpret_cast<uintptr_t>(parts_f32) | reinterpret_cast<uintptr_t>(workspace)) & 15u)
+        return hipErrorInvalidValue;
+    const int64_t chunks = (int64_t)rows_pad * (inter / 8);
+    lg::silu_mul_tall_kernel<<<dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0,
+                               static_cast<hipStream_t>(stream)>>>(
+        static_cast<const float*>(parts_f32), num_parts, (int64_t)rows * 2 * inter,
+        static_cast<uint16_t*>(workspace),
+        reinterpret_cast<float*>(static_cast<char*>(workspace) + lg::tall_sums_offset(rows, inter)),
+        rows, rows_pad, inter, pairs_per_load);
+    return hipGetLastError();
 }
 
 extern "C" logismos_status_t logismos_launch_silu_mul_bf16(const void* gate_up_bf16,

@@ -57,6 +57,10 @@ _SIGNATURES = {
     "logismos_check_qgemm_q4g128_tall_shape": (C.c_uint32, [_i, _i, _i, C.c_char_p, _sz]),
     "logismos_qgemm_q4g128_tall_workspace_bytes": (_sz, [_i, _i]),
     "logismos_launch_qgemm_q4g128_tall": (C.c_uint32, [_vp] * 6 + [_i, _vp, _i, _i, _i, _vp]),
+    "logismos_qgemm_q4g128_tall_pairs_per_load": (C.c_int, [_i, _vp, _vp]),
+    "logismos_launch_qgemm_q4g128_tall_prepared":
+        (C.c_uint32, [_vp] * 5 + [_i, _vp, _i, _i, _i, _vp]),
+    "logismos_launch_silu_mul_f32p_tall": (C.c_uint32, [_vp, _i, _vp, _i, _i, _i, _vp]),
     "logismos_launch_repack_q8_0": (C.c_uint32, [_vp, _vp, _vp, _i, _i, _vp]),
     "logismos_check_qgemv_q4g32_shape": (C.c_uint32, [_i, _i, C.c_char_p, _sz]),
     "logismos_launch_qgemv_q4g32_f32": (C.c_uint32, [_vp] * 5 + [_i, _i, _vp]),
@@ -304,6 +308,25 @@ def launch_qgemm_q4g128_tall(x, qw, scale, zero, y, workspace, m: int, n: int, k
     _status("qgemm_q4g128_tall", library().logismos_launch_qgemm_q4g128_tall(
         _ptr(x), _ptr(qw), _ptr(scale), _ptr(zero), _ptr(bias) if bias is not None else None,
         _ptr(y), 1 if f32_out else 0, _ptr(workspace), m, n, k, _raw(stream)))
+
+
+def qgemm_q4g128_tall_pairs_per_load(k: int, scale, zero) -> int:
+    return library().logismos_qgemm_q4g128_tall_pairs_per_load(k, _ptr(scale), _ptr(zero))
+
+
+def launch_qgemm_q4g128_tall_prepared(qw, scale, zero, y, workspace, m: int, n: int, k: int,
+                                      stream=None, bias=None, f32_out: bool = False) -> None:
+    """The tiled kernel alone over a workspace whose producer wrote x in the kernel's order."""
+    _guard("qgemm_q4g128_tall", library().logismos_check_qgemm_q4g128_tall_shape, m, n, k)
+    _status("qgemm_q4g128_tall_prepared", library().logismos_launch_qgemm_q4g128_tall_prepared(
+        _ptr(qw), _ptr(scale), _ptr(zero), _ptr(bias) if bias is not None else None, _ptr(y),
+        1 if f32_out else 0, _ptr(workspace), m, n, k, _raw(stream)))
+
+
+def launch_silu_mul_f32p_tall(parts, num_parts: int, workspace, rows: int, inter: int,
+                              pairs_per_load: int, stream=None) -> None:
+    _status("silu_mul_f32p_tall", library().logismos_launch_silu_mul_f32p_tall(
+        _ptr(parts), num_parts, _ptr(workspace), rows, inter, pairs_per_load, _raw(stream)))
 
 
 def launch_repack_q8_0(blocks, qs, d, n: int, k: int, stream=None) -> None:

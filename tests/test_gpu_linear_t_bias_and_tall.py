@@ -249,6 +249,52 @@ def test_q4g128_workspace_kernel_takes_scales_and_zeros_at_any_4_byte_alignment(
     del s_buf, z_buf
 
 
+@pytest.mark.parametrize("rows,inter,n", [(200, 1024, 300), (130, 1536, 256), (97, 768, 520)])
+def test_swiglu_written_as_the_workspace_kernels_operand(rows, inter, n):
+    # `silu_mul_f32p_tall` + `qgemm_q4g128_tall_prepared` against `silu_mul_f32p` + the entry
+    # point that makes its own first pass: the same workspace contents (x in pair order, rows
+    # padded with zeros, group sums), hence the same product, bit for bit; and both against
+    # the oracle.  inter a multiple of 1024 / 512 / 256: four, two, one pair of groups per load.
+    from oracle import decode_step as OS
+    rng = np.random.default_rng(rows + inter)
+    parts = rng.standard_normal((2, rows, 2 * inter), np.float32)
+    qw, s, z = _q4(rng, n, inter)
+    d_parts, d_qw = up(parts), up(qw)
+    d_s, d_z = up(s.view(np.uint16)), up(z.view(np.uint16))
+    nbytes = kernels.qgemm_q4g128_tall_workspace_bytes(rows, inter)
+    w = kernels.qgemm_q4g128_tall_pairs_per_load(inter, d_s, d_z)
+    assert w == (4 if inter % 1024 == 0 else 2 if inter % 512 == 0 else 1)
+
+    ws_a = hip.DeviceBuffer(nbytes)
+    ws_a.fill(0xFF)
+    d_ya = hip.DeviceBuffer(rows * n * 4)
+    kernels.launch_silu_mul_f32p_tall(d_parts, 2, ws_a, rows, inter, w)
+    kernels.launch_qgemm_q4g128_tall_prepared(d_qw, d_s, d_z, d_ya, ws_a, rows, n, inter,
+                                              f32_out=True)
+    ws_b = hip.DeviceBuffer(nbytes)
+    ws_b.fill(0x00)
+    d_act = hip.DeviceBuffer(rows * inter * 2)
+    d_yb = hip.DeviceBuffer(rows * n * 4)
+    kernels.launch_silu_mul_f32p(d_parts, 2, d_act, rows, inter)
+    kernels.launch_qgemm_q4g128_tall(d_act, d_qw, d_s, d_z, d_yb, ws_b, rows, n, inter,
+                                     f32_out=True)
+    hip.synchronize()
+    rows_pad = -(-rows // 128) * 128
+    head = rows_pad * inter * 2                      # x in pair order
+    sums_at = (head + 255) // 256 * 256
+    sums = rows_pad * (inter // 128) * 4
+    a, b = ws_a.to_numpy(np.uint8, (nbytes,)), ws_b.to_numpy(np.uint8, (nbytes,))
+    assert np.array_equal(a[:head], b[:head])
+    assert np.array_equal(a[sums_at:sums_at + sums], b[sums_at:sums_at + sums])
+    assert not a[rows * inter * 2:head].any()        # the padding rows
+    ya, yb = d_ya.to_numpy(np.float32, (rows, n)), d_yb.to_numpy(np.float32, (rows, n))
+    assert np.array_equal(ya.view(np.uint32), yb.view(np.uint32))
+    act = OS.silu_mul_bf16(parts[0] + parts[1], inter)
+    assert np.array_equal(d_act.to_numpy(np.uint16, (rows, inter)), act)
+    want = O.qgemm_q4g128_f32(act, qw, s, z, rows, n, inter, None)
+    assert_parity(ya, want, max_abs=2e-4, max_rel=1e-3, what=f"swiglu -> down {rows}x{n}x{inter}")
+
+
 def test_q4g128_workspace_kernel_is_deterministic():
     # parts of a tile split over K are summed in part order: two launches, the same bits
     rng = np.random.default_rng(92)
