@@ -199,7 +199,8 @@ size_t logismos_qgemm_q4g128_tall_workspace_bytes(int m, int k);
 /* The two halves of the launch below for a caller whose producer writes x where the kernel
  * wants it: `..._tall_prepared` is the product alone over a workspace that already holds x in
  * the kernel's operand order with its group sums (the first `m_pad*K*2` bytes and the sums
- * behind them, as `logismos_launch_silu_mul_f32p_tall` writes them), `..._pairs_per_load` the
+ * behind them, as `logismos_launch_silu_mul_f32p_tall` and
+ * `logismos_launch_add_rms_norm_f32p_tall` write them), `..._pairs_per_load` the
  * one parameter of that layout that depends on the weights (how many pairs of groups of K the
  * kernel loads scales and zeros for at once: 4, 2 or 1 by K and their alignment).  No
  * counterpart in the reference: `linear_t` takes plain rows. */
@@ -530,6 +531,15 @@ logismos_status_t logismos_launch_rope_kv_write_f32p_turbo3_bias(
 logismos_status_t logismos_launch_silu_mul_f32p(const void* parts_f32, int num_parts,
                                                 void* out_bf16, int rows, int inter,
                                                 logismos_stream_t stream);
+
+/* h += sum of the fp32 parts, then the RMS-normed row times its gains written as the operand
+ * of the many-row GEMM (see the SwiGLU form below; K = n a multiple of 256 * pairs_per_load,
+ * n <= 16384).  The arithmetic is that of `logismos_launch_add_rms_norm_f32p_xprep`. */
+logismos_status_t logismos_launch_add_rms_norm_f32p_tall(void* h_f32, const void* parts_f32,
+                                                         int num_parts, const void* w_f32,
+                                                         void* workspace, int rows, int n,
+                                                         float eps, int pairs_per_load,
+                                                         logismos_stream_t stream);
 
 /* SwiGLU over the fp32 parts with the result written as the operand of the many-row GEMM
  * (`logismos_launch_qgemm_q4g128_tall_prepared` over the same workspace, K = inter a multiple

@@ -289,13 +289,28 @@ extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_c
             return lg::qgemm_q4_tall_f32_launch(x_bf16, W.qw, W.scale, W.zero,
                                                 static_cast<const float*>(bias), y_f32, t, n, k, st);
         };
+        // add + norm followed by a projection of the normed rows: where the tiled GEMM with a
+        // workspace takes the shape, the normed rows go straight into its workspace in the
+        // kernel's operand order (no first pass over them)
+        auto norm_then_gemm = [&](int parts, const void* gains, const logismos_q4_weight_t& W,
+                                  void* y_f32, int n) -> logismos_status_t {
+            if (logismos_check_qgemm_q4g128_tall_shape(t, n, c.hidden, nullptr, 0) == 0 &&
+                c.hidden <= 16384) {
+                LG_TRY(logismos_launch_add_rms_norm_f32p_tall(
+                    batch->hidden_f32, w.t_proj, parts, gains, w.t_gemm, t, c.hidden, c.rms_eps,
+                    logismos_qgemm_q4g128_tall_pairs_per_load(c.hidden, W.scale, W.zero), stream));
+                return logismos_launch_qgemm_q4g128_tall_prepared(W.qw, W.scale, W.zero, nullptr,
+                                                                  y_f32, 1, w.t_gemm, t, n,
+                                                                  c.hidden, stream);
+            }
+            LG_TRY(logismos_launch_add_rms_norm_f32p(batch->hidden_f32, w.t_proj, parts, gains,
+                                                     w.t_xn, t, c.hidden, c.rms_eps, stream));
+            return gemm(w.t_xn, W, nullptr, y_f32, n, c.hidden);
+        };
         int res_parts = 0;
         for (int l = 0; l < c.num_layers; ++l) {
             const logismos_decode_layer_t& L = layers[l];
-            LG_TRY(logismos_launch_add_rms_norm_f32p(batch->hidden_f32, w.t_proj, res_parts,
-                                                     L.norm1_w_f32, w.t_xn, t, c.hidden, c.rms_eps,
-                                                     stream));
-            LG_TRY(gemm(w.t_xn, L.qkv, nullptr, w.t_qkv, width, c.hidden));
+            LG_TRY(norm_then_gemm(res_parts, L.norm1_w_f32, L.qkv, w.t_qkv, width));
             const auto rope_kv_write = c.kv_turbo3 ? logismos_launch_rope_kv_write_f32p_turbo3_bias
                                                    : logismos_launch_rope_kv_write_f32p_bias;
             LG_TRY(rope_kv_write(w.t_qkv, 1, L.qkv_bias_f32, batch->positions, batch->rope_cos_f32,
@@ -308,9 +323,7 @@ extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_c
                 c.num_kv_heads, c.head_dim, c.block_size, c.max_blocks_per_seq, batch->num_splits,
                 scale, 1, LOGISMOS_ATTN_PHASE_ALL, 1, c.kv_turbo3 ? 1 : 0, stream));
             LG_TRY(gemm(w.attn_out, L.o, nullptr, w.t_proj, c.hidden, qd));
-            LG_TRY(logismos_launch_add_rms_norm_f32p(batch->hidden_f32, w.t_proj, 1, L.norm2_w_f32,
-                                                     w.t_xn, t, c.hidden, c.rms_eps, stream));
-            LG_TRY(gemm(w.t_xn, L.gate_up, nullptr, w.t_gu, 2 * c.intermediate, c.hidden));
+            LG_TRY(norm_then_gemm(1, L.norm2_w_f32, L.gate_up, w.t_gu, 2 * c.intermediate));
             if (logismos_check_qgemm_q4g128_tall_shape(t, c.hidden, c.intermediate, nullptr, 0) == 0) {
                 // the activation goes straight into the down projection's workspace, in the
                 // kernel's operand order: no first pass over it

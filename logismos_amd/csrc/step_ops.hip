@@ -120,10 +120,27 @@ __global__ __launch_bounds__(kNormThreads) void add_rms_norm_kernel(
 constexpr int kPrepThreads = 512;
 constexpr int kPrepMaxPasses = 4;  // rows up to 16384 wide
 
+// TALL: the normed rows leave as the operand of the tiled GEMM for many rows instead
+// (q4_common.hpp: row-major in pair order, `pairs` pairs of groups per block of sums; the grid
+// covers the rows padded to the GEMM's 128-row tiles, and a padding row is written as zeros).
+template <bool TALL>
 __global__ __launch_bounds__(kPrepThreads) void add_rms_norm_xprep_kernel(
     float* __restrict__ h, const float* __restrict__ yp, int num_parts, int64_t part_stride,
-    const float* __restrict__ w, void* __restrict__ xprep, int rows, int n, float eps) {
+    const float* __restrict__ w, void* __restrict__ xprep, int rows, int n, float eps,
+    int pairs) {
     const int64_t row = blockIdx.x;
+    if constexpr (TALL) {
+        if (row >= rows) {
+            uint4_t* xt = reinterpret_cast<uint4_t*>(xprep) + row * (n >> 3);
+            float* xs = reinterpret_cast<float*>(reinterpret_cast<char*>(xprep) +
+                                                 tall_sums_offset(rows, n));
+            for (int c = threadIdx.x; c < (n >> 3); c += kPrepThreads) {
+                xt[c] = uint4_t{0u, 0u, 0u, 0u};
+                if ((c & 15) == 0) xs[tall_sum_index(row, c >> 4, n, pairs)] = 0.0f;
+            }
+            return;
+        }
+    }
     float* hr = h + row * n;
     float v[kPrepMaxPasses][8];
     float4_t wv[kPrepMaxPasses][2];  // the gains, requested with the first loads, not after the reduction
@@ -198,8 +215,16 @@ __global__ __launch_bounds__(kPrepThreads) void add_rms_norm_xprep_kernel(
         }
         const float gs = row16_sum(sum8_bf16(o));
         if (live) {
-            xp[(int64_t)c * bp + row] = pair_order(o);
-            if ((threadIdx.x & 15) == 0) xg[(int64_t)(c >> 4) * bp + row] = gs;
+            if constexpr (TALL) {
+                xp[row * (n >> 3) + c] = pair_order(o);
+                if ((threadIdx.x & 15) == 0)
+                    reinterpret_cast<float*>(reinterpret_cast<char*>(xprep) +
+                                             tall_sums_offset(rows, n))
+                        [tall_sum_index(row, c >> 4, n, pairs)] = gs;
+            } else {
+                xp[(int64_t)c * bp + row] = pair_order(o);
+                if ((threadIdx.x & 15) == 0) xg[(int64_t)(c >> 4) * bp + row] = gs;
+            }
         }
     }
 }
@@ -894,10 +919,32 @@ extern "C" logismos_status_t logismos_launch_add_rms_norm_f32p_xprep(
         return hipErrorInvalidValue;
     if (!h_f32 || !w_f32 || !x_prepared || num_parts < 0 || (num_parts > 0 && !parts_f32))
         return hipErrorInvalidValue;
-    lg::add_rms_norm_xprep_kernel<<<dim3(rows), dim3(lg::kPrepThreads), 0,
-                                    static_cast<hipStream_t>(stream)>>>(
+    lg::add_rms_norm_xprep_kernel<false><<<dim3(rows), dim3(lg::kPrepThreads), 0,
+                                           static_cast<hipStream_t>(stream)>>>(
         static_cast<float*>(h_f32), static_cast<const float*>(parts_f32), num_parts,
-        (int64_t)rows * n, static_cast<const float*>(w_f32), x_prepared, rows, n, eps);
+        (int64_t)rows * n, static_cast<const float*>(w_f32), x_prepared, rows, n, eps, 0);
+    return hipGetLastError();
+}
+
+extern "C" logismos_status_t logismos_launch_add_rms_norm_f32p_tall(
+    void* h_f32, const void* parts_f32, int num_parts, const void* w_f32, void* workspace,
+    int rows, int n, float eps, int pairs_per_load, logismos_stream_t stream) {
+    if (rows <= 0 || n <= 0 || num_parts < 0 ||
+        (pairs_per_load != 1 && pairs_per_load != 2 && pairs_per_load != 4) ||
+        n % (256 * pairs_per_load) != 0 || n > 8 * lg::kPrepThreads * lg::kPrepMaxPasses)
+        return hipErrorInvalidValue;
+    const int rows_pad = lg::tall_padded_rows(rows);
+    if ((int64_t)rows_pad * n * 2 > (int64_t)INT32_MAX) return hipErrorInvalidValue;
+    if (!h_f32 || !w_f32 || !workspace || (num_parts > 0 && !parts_f32))
+        return hipErrorInvalidValue;
+    if ((reinterpret_cast<uintptr_t>(h_f32) | reinterpret_cast<uintptr_t>(parts_f32) |
+         reinterpret_cast<uintptr_t>(w_f32) | reinterpret_cast<uintptr_t>(workspace)) & 15u)
+        return hipErrorInvalidValue;
+    lg::add_rms_norm_xprep_kernel<true><<<dim3(rows_pad), dim3(lg::kPrepThreads), 0,
+                                          static_cast<hipStream_t>(stream)>>>(
+        static_cast<float*>(h_f32), static_cast<const float*>(parts_f32), num_parts,
+        (int64_t)rows * n, static_cast<const float*>(w_f32), workspace, rows, n, eps,
+        pairs_per_load);
     return hipGetLastError();
 }
 

@@ -61,6 +61,8 @@ _SIGNATURES = {
     "logismos_launch_qgemm_q4g128_tall_prepared":
         (C.c_uint32, [_vp] * 5 + [_i, _vp, _i, _i, _i, _vp]),
     "logismos_launch_silu_mul_f32p_tall": (C.c_uint32, [_vp, _i, _vp, _i, _i, _i, _vp]),
+    "logismos_launch_add_rms_norm_f32p_tall":
+        (C.c_uint32, [_vp, _vp, _i, _vp, _vp, _i, _i, _f, _i, _vp]),
     "logismos_launch_repack_q8_0": (C.c_uint32, [_vp, _vp, _vp, _i, _i, _vp]),
     "logismos_check_qgemv_q4g32_shape": (C.c_uint32, [_i, _i, C.c_char_p, _sz]),
     "logismos_launch_qgemv_q4g32_f32": (C.c_uint32, [_vp] * 5 + [_i, _i, _vp]),
@@ -327,6 +329,13 @@ def launch_silu_mul_f32p_tall(parts, num_parts: int, workspace, rows: int, inter
                               pairs_per_load: int, stream=None) -> None:
     _status("silu_mul_f32p_tall", library().logismos_launch_silu_mul_f32p_tall(
         _ptr(parts), num_parts, _ptr(workspace), rows, inter, pairs_per_load, _raw(stream)))
+
+
+def launch_add_rms_norm_f32p_tall(h, parts, num_parts: int, w, workspace, rows: int, n: int,
+                                  eps: float, pairs_per_load: int, stream=None) -> None:
+    _status("add_rms_norm_f32p_tall", library().logismos_launch_add_rms_norm_f32p_tall(
+        _ptr(h), _ptr(parts) if parts is not None else None, num_parts, _ptr(w), _ptr(workspace),
+        rows, n, float(eps), pairs_per_load, _raw(stream)))
 
 
 def launch_repack_q8_0(blocks, qs, d, n: int, k: int, stream=None) -> None:

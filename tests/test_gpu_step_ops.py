@@ -329,3 +329,57 @@ def test_prepared_layout_producers_match_the_plain_ones():
     hip.synchronize()
     x2, xg2 = _unprepare(d_op2.to_numpy(np.uint8, (d_op2.nbytes,)), rows, inter)
     assert np.array_equal(x2, x) and np.array_equal(xg2, xg)
+
+
+def _untall(buf, rows, k, pairs):
+    """operand of the many-row GEMM -> (bf16 bits [rows_pad][k], group sums [rows_pad][k/128])"""
+    rows_pad = -(-rows // 128) * 128
+    xp = buf[: rows_pad * k * 2].view(np.uint16).reshape(rows_pad, k // 8, 8)
+    nat = np.empty_like(xp)
+    nat[..., [0, 4, 1, 5, 2, 6, 3, 7]] = xp
+    at = (rows_pad * k * 2 + 255) // 256 * 256
+    groups, bl = k // 128, 2 * pairs
+    xs = buf[at: at + rows_pad * groups * 4].view(np.float32).reshape(
+        rows_pad // 128, groups // bl, 2, 128, pairs)
+    # [row tile][block][place in pair][row][pair] -> [row][group = block * bl + 2 * pair + place]
+    sums = xs.transpose(0, 3, 1, 4, 2).reshape(rows_pad, groups)
+    return nat.reshape(rows_pad, k), sums
+
+
+@pytest.mark.parametrize("rows,n,pairs", [(32, 4096, 4), (150, 1536, 2), (130, 768, 1),
+                                          (20, 2048, 1)])
+def test_add_rms_norm_written_as_the_many_row_gemms_operand(rows, n, pairs):
+    # the same kernel as the prepared-layout producer of the decode chunks, storing into the
+    # tiled GEMM's workspace: x in pair order row by row, padding rows zero, group sums in the
+    # kernel's block order (for every number of pairs per block the GEMM may ask for).  Up to
+    # 32 rows the chunk producer runs beside it: same h, same bits, same sums.
+    rng = np.random.default_rng(rows + n)
+    j = 3
+    h = rng.standard_normal((rows, n), np.float32)
+    parts = rng.standard_normal((j, rows, n), np.float32)
+    w = (1 + 0.02 * rng.standard_normal(n)).astype(np.float32)
+    dev = hip.DeviceBuffer.from_numpy
+    d_w, d_parts, d_h = dev(w), dev(parts), dev(h)
+    ws = hip.DeviceBuffer(kernels.qgemm_q4g128_tall_workspace_bytes(rows, n))
+    ws.fill(0xFF)
+    kernels.launch_add_rms_norm_f32p_tall(d_h, d_parts, j, d_w, ws, rows, n, 1e-6, pairs)
+    hip.synchronize()
+    x, sums = _untall(ws.to_numpy(np.uint8, (ws.nbytes,)), rows, n, pairs)
+    assert not x[rows:].any() and not sums[rows:].any()
+    h_want = h.copy()
+    want = OS.add_rms_norm_bf16(h_want, parts[0] + parts[1] + parts[2], w, 1e-6)
+    assert_parity(d_h.to_numpy(np.float32, (rows, n)), h_want, max_abs=1e-5, max_rel=1e-5,
+                  what="h")
+    assert_parity(O.bf16_bits_to_f32(x[:rows]), O.bf16_bits_to_f32(want), max_abs=1e-6,
+                  max_rel=8e-3, what="normed rows")
+    assert np.abs(sums[:rows] -
+                  O.bf16_bits_to_f32(x[:rows]).reshape(rows, n // 128, 128).sum(axis=2)).max() < 1e-3
+    if rows <= 32:
+        d_h2 = dev(h)
+        d_prep = hip.DeviceBuffer(kernels.q4_xprep_bytes(rows, n))
+        kernels.launch_add_rms_norm_f32p_xprep(d_h2, d_parts, j, d_w, d_prep, rows, n, 1e-6)
+        hip.synchronize()
+        x2, xg2 = _unprepare(d_prep.to_numpy(np.uint8, (d_prep.nbytes,)), rows, n)
+        assert np.array_equal(x[:rows], x2) and np.array_equal(sums[:rows], xg2)
+        assert np.array_equal(d_h.to_numpy(np.float32, (rows, n)),
+                              d_h2.to_numpy(np.float32, (rows, n)))
