@@ -208,6 +208,14 @@ int logismos_qgemm_q4g128_tall_pairs_per_load(int k, const void* scale_f16, cons
 logismos_status_t logismos_launch_qgemm_q4g128_tall_prepared(
     const void* qw_u8, const void* scale_f16, const void* zero_f16, const void* bias_f32, void* y,
     int y_is_f32, void* workspace, int m, int n, int k, logismos_stream_t stream);
+/* The gate/up projection of a SwiGLU MLP with the activation applied where the products are
+ * summed (crates/transformers/src/mlp.rs:104-111: down(silu(gate(x)) * up(x))): weights
+ * `[2*inter][K]`, gate rows first; `act_bf16 [m][inter] = bf16(silu(x.gate^T) * (x.up^T))`, the
+ * fp32 products rounded once, as `logismos_launch_silu_mul_f32p` rounds them.  Over a prepared
+ * workspace like `..._tall_prepared`. */
+logismos_status_t logismos_launch_qgemm_q4g128_tall_swiglu_prepared(
+    const void* gate_up_qw_u8, const void* scale_f16, const void* zero_f16, void* act_bf16,
+    void* workspace, int m, int inter, int k, logismos_stream_t stream);
 logismos_status_t logismos_launch_qgemm_q4g128_tall(const void* x_bf16, const void* qw_u8,
                                                     const void* scale_f16, const void* zero_f16,
                                                     const void* bias_f32, void* y, int y_is_f32,

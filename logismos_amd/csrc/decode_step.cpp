@@ -323,6 +323,23 @@ extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_c
                 c.num_kv_heads, c.head_dim, c.block_size, c.max_blocks_per_seq, batch->num_splits,
                 scale, 1, LOGISMOS_ATTN_PHASE_ALL, 1, c.kv_turbo3 ? 1 : 0, stream));
             LG_TRY(gemm(w.attn_out, L.o, nullptr, w.t_proj, c.hidden, qd));
+            if (logismos_check_qgemm_q4g128_tall_shape(t, 2 * c.intermediate, c.hidden, nullptr, 0) ==
+                    0 &&
+                c.hidden <= 16384) {
+                // the gate/up projection with the SwiGLU where its products are summed: the
+                // fp32 gate and up products never go to memory
+                LG_TRY(logismos_launch_add_rms_norm_f32p_tall(
+                    batch->hidden_f32, w.t_proj, 1, L.norm2_w_f32, w.t_gemm, t, c.hidden, c.rms_eps,
+                    logismos_qgemm_q4g128_tall_pairs_per_load(c.hidden, L.gate_up.scale,
+                                                              L.gate_up.zero),
+                    stream));
+                LG_TRY(logismos_launch_qgemm_q4g128_tall_swiglu_prepared(
+                    L.gate_up.qw, L.gate_up.scale, L.gate_up.zero, w.t_act, w.t_gemm, t,
+                    c.intermediate, c.hidden, stream));
+                LG_TRY(gemm(w.t_act, L.down, nullptr, w.t_proj, c.hidden, c.intermediate));
+                res_parts = 1;
+                continue;
+            }
             LG_TRY(norm_then_gemm(1, L.norm2_w_f32, L.gate_up, w.t_gu, 2 * c.intermediate));
             if (logismos_check_qgemm_q4g128_tall_shape(t, c.hidden, c.intermediate, nullptr, 0) == 0) {
                 // the activation goes straight into the down projection's workspace, in the

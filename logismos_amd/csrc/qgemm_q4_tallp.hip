@@ -124,9 +124,16 @@ struct TpRegs<T, 1> {
     __device__ __forceinline__ T operator[](int) const { return raw; }
 };
 
+// What a launch writes.  kTpOutSwiglu: the weights are a gate/up pair [gate rows | up rows]
+// (2 n rows) and y [m][n] is bf16 silu(gate) * up -- a workgroup tile takes 128 gate rows and
+// the 128 up rows of the same outputs, a wave's first 32 columns the gate and its other 32 the
+// up values of the same 32 outputs, so a lane holds both products of a result and the fp32
+// gate/up products (a gigabyte at 8240 rows of a 12288-wide MLP) never go to memory.
+constexpr int kTpOutBf16 = 0, kTpOutF32 = 1, kTpOutSwiglu = 2;
+
 // W: pairs of groups whose scales, zeros and group sums a lane loads at once (1, 2 or 4: a
 // dword, two or four per load; K a multiple of 256 W).
-template <bool F32OUT, int W>
+template <int OUT, int W>
 __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
     const uint16_t* __restrict__ xp, const float* __restrict__ xs, const uint8_t* __restrict__ qw,
     const __half* __restrict__ scale, const __half* __restrict__ zero,
@@ -153,7 +160,18 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
     }
     const int row_tile = tile / tiles_n;
     const int row0 = row_tile * kTpTileM;
-    const int col0 = (tile % tiles_n) * kTpTileN;
+    // (SwiGLU: a tile is 128 outputs wide -- 128 gate and 128 up rows of the weights)
+    constexpr int kTileOutputs = OUT == kTpOutSwiglu ? kTpTileN / 2 : kTpTileN;
+    const int col0 = (tile % tiles_n) * kTileOutputs;
+    // weight row behind row L of the tile in LDS (a wave's B operand rows are L = wc + 32 j + r)
+    auto weight_row = [&](int L) {
+        if constexpr (OUT == kTpOutSwiglu) {
+            const int out_col = min(col0 + (L >> 6) * 32 + (L & 31), n - 1);
+            return ((L >> 5) & 1) ? n + out_col : out_col;
+        } else {
+            return min(col0 + L, n - 1);  // a row past n re-reads the last row
+        }
+    };
     const int wr = (wave >> 2) * 64;  // this wave's 64 x 64 part of the 128 x 256 tile
     const int wc = (wave & 3) * 64;
     const int groups_row = k >> 7;    // scales and zeros: groups per weight row
@@ -178,8 +196,7 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
     for (int q = 0; q < 2; ++q) {
         const int row = 32 * wave + 16 * q + (lane >> 2);
         const int piece = (lane & 3) ^ ((row >> 2) & 3);
-        const int gn = min(col0 + row, n - 1);  // a row past n re-reads the last row
-        woff[q] = (unsigned)gn * (unsigned)(k >> 1) + (unsigned)piece * 16u;
+        woff[q] = (unsigned)weight_row(row) * (unsigned)(k >> 1) + (unsigned)piece * 16u;
     }
     // As assembly: the 32-bit offsets above with a scalar base (the builtin widens each to a
     // 64-bit address in two more registers); M0 holds the LDS address of lane 0's 16 bytes and
@@ -235,7 +252,7 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
     unsigned soff[2], xsoff[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j)
-        soff[j] = (unsigned)min(col0 + wc + 32 * j + r, n - 1) * (unsigned)groups_row * 2u;
+        soff[j] = (unsigned)weight_row(wc + 32 * j + r) * (unsigned)groups_row * 2u;
 #pragma unroll
     for (int i = 0; i < 2; ++i) xsoff[i] = (unsigned)((h * kTpTileM + wr + 32 * i + r) * W) * 4u;
     auto gload_small = [&](int g, Small& v) {
@@ -469,6 +486,22 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
                 for (int e = 0; e < 16; ++e) dst[((i * 2 + j) * 16 + e) * 64] = yacc[i][j][e];
         return;
     }
+    if constexpr (OUT == kTpOutSwiglu) {
+        const int gn = col0 + (wc >> 1) + r;
+        if (gn >= n) return;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int gr = row0 + wr + 32 * i + 8 * (e >> 2) + 4 * h + (e & 3);
+                if (gr < m) {
+                    const float g = yacc[i][0][e], u = yacc[i][1][e];
+                    static_cast<uint16_t*>(y_out)[(int64_t)gr * n + gn] =
+                        f32_to_bf16_rne(g / (1.0f + expf(-g)) * u);
+                }
+            }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const int gn = col0 + wc + 32 * j + r;
@@ -480,7 +513,7 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
             for (int e = 0; e < 16; ++e) {
                 const int gr = row0 + wr + 32 * i + 8 * (e >> 2) + 4 * h + (e & 3);
                 if (gr < m) {
-                    if constexpr (F32OUT)
+                    if constexpr (OUT == kTpOutF32)
                         static_cast<float*>(y_out)[(int64_t)gr * n + gn] = yacc[i][j][e] + bv;
                     else
                         static_cast<uint16_t*>(y_out)[(int64_t)gr * n + gn] =
@@ -492,67 +525,85 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
 
 // Sums the `split` fp32 parts of each tile of the last round, in part order, adds the bias and
 // writes y.  One thread per result; a part's element index is (wave, i, j, e, lane) as the
-// product kernel left it.
-template <bool F32OUT>
+// product kernel left it.  (SwiGLU: j = 0 is the gate and j = 1 the up product of the same
+// result; one thread takes both.)
+template <int OUT>
 __global__ __launch_bounds__(256) void q4_tall_reduce_kernel(const float* __restrict__ partials,
                                                             const float* __restrict__ bias,
                                                             void* __restrict__ y_out, int m, int n,
                                                             int tiles_n, int full_tiles,
                                                             int split) {
-    const int t = blockIdx.x / (kTpTileElems / 256);
-    const int idx = (blockIdx.x % (kTpTileElems / 256)) * 256 + threadIdx.x;
+    constexpr int kPerTile = OUT == kTpOutSwiglu ? kTpTileElems / 2 : kTpTileElems;
+    const int t = blockIdx.x / (kPerTile / 256);
+    int idx = (blockIdx.x % (kPerTile / 256)) * 256 + threadIdx.x;
+    if constexpr (OUT == kTpOutSwiglu) idx = ((idx >> 10) << 11) | (idx & 1023);  // j = 0
     const int lane = idx & 63, e = (idx >> 6) & 15, j = (idx >> 10) & 1, i = (idx >> 11) & 1;
     const int wave = idx >> 12;
     const int tile = full_tiles + t;
     const int gr = (tile / tiles_n) * kTpTileM + (wave >> 2) * 64 + 32 * i + 8 * (e >> 2) +
                    4 * (lane >> 5) + (e & 3);
-    const int gn = (tile % tiles_n) * kTpTileN + (wave & 3) * 64 + 32 * j + (lane & 31);
-    if (gr >= m || gn >= n) return;
     const float* src = partials + (size_t)t * split * kTpTileElems + idx;
-    float acc = 0.0f;
-    for (int q = 0; q < split; ++q) acc += src[(size_t)q * kTpTileElems];
-    if (bias) acc += bias[gn];
-    if constexpr (F32OUT) static_cast<float*>(y_out)[(int64_t)gr * n + gn] = acc;
-    else static_cast<uint16_t*>(y_out)[(int64_t)gr * n + gn] = f32_to_bf16_rne(acc);
+    if constexpr (OUT == kTpOutSwiglu) {
+        const int gn = (tile % tiles_n) * (kTpTileN / 2) + (wave & 3) * 32 + (lane & 31);
+        if (gr >= m || gn >= n) return;
+        float g = 0.0f, u = 0.0f;
+        for (int q = 0; q < split; ++q) {
+            g += src[(size_t)q * kTpTileElems];
+            u += src[(size_t)q * kTpTileElems + 1024];
+        }
+        static_cast<uint16_t*>(y_out)[(int64_t)gr * n + gn] =
+            f32_to_bf16_rne(g / (1.0f + expf(-g)) * u);
+    } else {
+        const int gn = (tile % tiles_n) * kTpTileN + (wave & 3) * 64 + 32 * j + (lane & 31);
+        if (gr >= m || gn >= n) return;
+        float acc = 0.0f;
+        for (int q = 0; q < split; ++q) acc += src[(size_t)q * kTpTileElems];
+        if (bias) acc += bias[gn];
+        if constexpr (OUT == kTpOutF32) static_cast<float*>(y_out)[(int64_t)gr * n + gn] = acc;
+        else static_cast<uint16_t*>(y_out)[(int64_t)gr * n + gn] = f32_to_bf16_rne(acc);
+    }
 }
 
 inline int tp_pairs_per_load(int k, const void* scale, const void* zero) {
     return tall_pairs_per_load(k, scale, zero);
 }
 
-template <bool F32OUT, int W>
+template <int OUT, int W>
 static hipError_t tallp_launch(const uint16_t* xp, const float* xs, float* partials,
                                const uint8_t* qw, const __half* scale, const __half* zero,
                                const float* bias, void* y, int m, int n, int k, hipStream_t st) {
     constexpr size_t lds = (size_t)kTpBufs * kTpBufBytes;
     static const hipError_t opt = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(qgemm_q4g128_tallp_kernel<F32OUT, W>),
+        reinterpret_cast<const void*>(qgemm_q4g128_tallp_kernel<OUT, W>),
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (opt != hipSuccess) return opt;
-    const int tiles_n = (n + kTpTileN - 1) / kTpTileN;
+    constexpr int tile_outputs = OUT == kTpOutSwiglu ? kTpTileN / 2 : kTpTileN;
+    const int tiles_n = (n + tile_outputs - 1) / tile_outputs;
     const int tiles = tiles_n * (tp_padded_rows(m) / kTpTileM);
     const int cus = device_cu_count();
     if (cus <= 0) return hipErrorInvalidDevice;
     const TpPlan plan = tp_plan(tiles, k >> 7, 2 * W, cus);
     const int parts = (tiles - plan.full) * plan.split;
-    qgemm_q4g128_tallp_kernel<F32OUT, W>
+    qgemm_q4g128_tallp_kernel<OUT, W>
         <<<dim3(plan.full + (plan.split > 1 ? parts : 0)), dim3(512), lds, st>>>(
             xp, xs, qw, scale, zero, bias, y, partials, m, n, k, tiles_n, plan.full, plan.split);
-    if (plan.split > 1)
-        q4_tall_reduce_kernel<F32OUT>
-            <<<dim3((tiles - plan.full) * (kTpTileElems / 256)), dim3(256), 0, st>>>(
+    if (plan.split > 1) {
+        constexpr int per_tile = OUT == kTpOutSwiglu ? kTpTileElems / 2 : kTpTileElems;
+        q4_tall_reduce_kernel<OUT>
+            <<<dim3((tiles - plan.full) * (per_tile / 256)), dim3(256), 0, st>>>(
                 partials, bias, y, m, n, tiles_n, plan.full, plan.split);
+    }
     return hipGetLastError();
 }
 
-template <bool F32OUT>
+template <int OUT>
 static hipError_t tallp_launch_w(int w, const uint16_t* xp, const float* xs, float* partials,
                                  const uint8_t* qw, const __half* scale, const __half* zero,
                                  const float* bias, void* y, int m, int n, int k, hipStream_t st) {
     switch (w) {
-        case 4: return tallp_launch<F32OUT, 4>(xp, xs, partials, qw, scale, zero, bias, y, m, n, k, st);
-        case 2: return tallp_launch<F32OUT, 2>(xp, xs, partials, qw, scale, zero, bias, y, m, n, k, st);
-        default: return tallp_launch<F32OUT, 1>(xp, xs, partials, qw, scale, zero, bias, y, m, n, k, st);
+        case 4: return tallp_launch<OUT, 4>(xp, xs, partials, qw, scale, zero, bias, y, m, n, k, st);
+        case 2: return tallp_launch<OUT, 2>(xp, xs, partials, qw, scale, zero, bias, y, m, n, k, st);
+        default: return tallp_launch<OUT, 1>(xp, xs, partials, qw, scale, zero, bias, y, m, n, k, st);
     }
 }
 
@@ -612,14 +663,35 @@ extern "C" logismos_status_t logismos_launch_qgemm_q4g128_tall_prepared(
                                                lg::tp_partials_offset(m, k));
     const int w = lg::tp_pairs_per_load(k, scale_f16, zero_f16);
     if (y_is_f32)
-        return lg::tallp_launch_w<true>(w, xp, xs, partials, static_cast<const uint8_t*>(qw_u8),
+        return lg::tallp_launch_w<lg::kTpOutF32>(w, xp, xs, partials, static_cast<const uint8_t*>(qw_u8),
                                         static_cast<const __half*>(scale_f16),
                                         static_cast<const __half*>(zero_f16),
                                         static_cast<const float*>(bias_f32), y, m, n, k, st);
-    return lg::tallp_launch_w<false>(w, xp, xs, partials, static_cast<const uint8_t*>(qw_u8),
+    return lg::tallp_launch_w<lg::kTpOutBf16>(w, xp, xs, partials, static_cast<const uint8_t*>(qw_u8),
                                      static_cast<const __half*>(scale_f16),
                                      static_cast<const __half*>(zero_f16),
                                      static_cast<const float*>(bias_f32), y, m, n, k, st);
+}
+
+extern "C" logismos_status_t logismos_launch_qgemm_q4g128_tall_swiglu_prepared(
+    const void* gate_up_qw_u8, const void* scale_f16, const void* zero_f16, void* act_bf16,
+    void* workspace, int m, int inter, int k, logismos_stream_t stream) {
+    // the weights are 2 * inter rows (gate, then up); the output is m x inter
+    if (inter <= 0 || inter > INT32_MAX / 2) return hipErrorInvalidValue;
+    if (const logismos_status_t e = tall_args_ok(gate_up_qw_u8, scale_f16, zero_f16, act_bf16,
+                                                 workspace, m, 2 * inter, k))
+        return e;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint16_t* xp = static_cast<const uint16_t*>(workspace);
+    const float* xs =
+        reinterpret_cast<const float*>(static_cast<char*>(workspace) + lg::tp_sums_offset(m, k));
+    float* partials = reinterpret_cast<float*>(static_cast<char*>(workspace) +
+                                               lg::tp_partials_offset(m, k));
+    const int w = lg::tp_pairs_per_load(k, scale_f16, zero_f16);
+    return lg::tallp_launch_w<lg::kTpOutSwiglu>(
+        w, xp, xs, partials, static_cast<const uint8_t*>(gate_up_qw_u8),
+        static_cast<const __half*>(scale_f16), static_cast<const __half*>(zero_f16), nullptr,
+        act_bf16, m, inter, k, st);
 }
 
 extern "C" logismos_status_t logismos_launch_qgemm_q4g128_tall(

@@ -61,6 +61,8 @@ _SIGNATURES = {
     "logismos_launch_qgemm_q4g128_tall_prepared":
         (C.c_uint32, [_vp] * 5 + [_i, _vp, _i, _i, _i, _vp]),
     "logismos_launch_silu_mul_f32p_tall": (C.c_uint32, [_vp, _i, _vp, _i, _i, _i, _vp]),
+    "logismos_launch_qgemm_q4g128_tall_swiglu_prepared":
+        (C.c_uint32, [_vp] * 5 + [_i, _i, _i, _vp]),
     "logismos_launch_add_rms_norm_f32p_tall":
         (C.c_uint32, [_vp, _vp, _i, _vp, _vp, _i, _i, _f, _i, _vp]),
     "logismos_launch_repack_q8_0": (C.c_uint32, [_vp, _vp, _vp, _i, _i, _vp]),
@@ -323,6 +325,16 @@ def launch_qgemm_q4g128_tall_prepared(qw, scale, zero, y, workspace, m: int, n: 
     _status("qgemm_q4g128_tall_prepared", library().logismos_launch_qgemm_q4g128_tall_prepared(
         _ptr(qw), _ptr(scale), _ptr(zero), _ptr(bias) if bias is not None else None, _ptr(y),
         1 if f32_out else 0, _ptr(workspace), m, n, k, _raw(stream)))
+
+
+def launch_qgemm_q4g128_tall_swiglu_prepared(qw, scale, zero, act, workspace, m: int, inter: int,
+                                             k: int, stream=None) -> None:
+    """gate/up projection + SwiGLU in one kernel over a prepared workspace: act bf16 [m][inter]."""
+    _guard("qgemm_q4g128_tall", library().logismos_check_qgemm_q4g128_tall_shape, m, 2 * inter, k)
+    _status("qgemm_q4g128_tall_swiglu_prepared",
+            library().logismos_launch_qgemm_q4g128_tall_swiglu_prepared(
+                _ptr(qw), _ptr(scale), _ptr(zero), _ptr(act), _ptr(workspace), m, inter, k,
+                _raw(stream)))
 
 
 def launch_silu_mul_f32p_tall(parts, num_parts: int, workspace, rows: int, inter: int,

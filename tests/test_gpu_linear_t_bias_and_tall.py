@@ -295,6 +295,40 @@ def test_swiglu_written_as_the_workspace_kernels_operand(rows, inter, n):
     assert_parity(ya, want, max_abs=2e-4, max_rel=1e-3, what=f"swiglu -> down {rows}x{n}x{inter}")
 
 
+@pytest.mark.parametrize("rows,inter,k", [(200, 300, 1024), (130, 1000, 512), (97, 128, 768),
+                                          (520, 2560, 2048)])
+def test_gate_up_projection_with_the_swiglu_in_the_kernel(rows, inter, k):
+    # one kernel for the gate/up projection and silu(gate) * up against the two-step form
+    # (fp32 products of all 2 * inter weight rows, then `silu_mul_f32p`): a workgroup tile
+    # pairs 128 gate rows with the up rows of the same outputs, the sums are the same fp32
+    # sums in the same order, so the bf16 activations are the same bits -- whole tiles and
+    # tiles split over K (every launch here is smaller than the device; the last shape splits
+    # unevenly), ragged in rows and in outputs; and against the oracle.
+    from oracle import decode_step as OS
+    rng = np.random.default_rng(rows + inter + k)
+    qw, s, z = _q4(rng, 2 * inter, k)
+    xb = O.f32_to_bf16_bits(rng.standard_normal((rows, k), np.float32))
+    d_x, d_qw = up(xb), up(qw)
+    d_s, d_z = up(s.view(np.uint16)), up(z.view(np.uint16))
+    ws = hip.DeviceBuffer(kernels.qgemm_q4g128_tall_workspace_bytes(rows, k))
+    # two steps: products (which also leaves x prepared in the workspace), then the activation
+    d_gu = hip.DeviceBuffer(rows * 2 * inter * 4)
+    kernels.launch_qgemm_q4g128_tall(d_x, d_qw, d_s, d_z, d_gu, ws, rows, 2 * inter, k, f32_out=True)
+    d_two = hip.DeviceBuffer(rows * inter * 2)
+    kernels.launch_silu_mul_f32p(d_gu, 1, d_two, rows, inter)
+    # one step over the same prepared workspace
+    d_one = hip.DeviceBuffer(rows * inter * 2)
+    d_one.fill(0xFF)
+    kernels.launch_qgemm_q4g128_tall_swiglu_prepared(d_qw, d_s, d_z, d_one, ws, rows, inter, k)
+    hip.synchronize()
+    one = d_one.to_numpy(np.uint16, (rows, inter))
+    two = d_two.to_numpy(np.uint16, (rows, inter))
+    assert np.array_equal(one, two)
+    gu = O.qgemm_q4g128_f32(xb, qw, s, z, rows, 2 * inter, k, None)
+    want = OS.silu_mul_bf16(gu, inter)
+    assert_parity(O.bf16_bits_to_f32(one), O.bf16_bits_to_f32(want), what="gate/up + swiglu")
+
+
 def test_q4g128_workspace_kernel_is_deterministic():
     # parts of a tile split over K are summed in part order: two launches, the same bits
     rng = np.random.default_rng(92)
