@@ -329,6 +329,34 @@ def test_gate_up_projection_with_the_swiglu_in_the_kernel(rows, inter, k):
     assert_parity(O.bf16_bits_to_f32(one), O.bf16_bits_to_f32(want), what="gate/up + swiglu")
 
 
+def test_gate_up_with_the_swiglu_on_more_tiles_than_the_device_has_units():
+    # 9 x 30 = 270 tiles of 128 rows x 128 outputs: the first 256 whole, the other 14 split over
+    # K with the activation applied where their parts are summed; bit for bit the two-step form
+    # everywhere, and the oracle on the first and the last rows
+    from oracle import decode_step as OS
+    rows, inter, k = 1100, 3840, 512
+    rng = np.random.default_rng(97)
+    qw, s, z = _q4(rng, 2 * inter, k)
+    xb = O.f32_to_bf16_bits(rng.standard_normal((rows, k), np.float32))
+    d_x, d_qw = up(xb), up(qw)
+    d_s, d_z = up(s.view(np.uint16)), up(z.view(np.uint16))
+    ws = hip.DeviceBuffer(kernels.qgemm_q4g128_tall_workspace_bytes(rows, k))
+    d_gu = hip.DeviceBuffer(rows * 2 * inter * 4)
+    kernels.launch_qgemm_q4g128_tall(d_x, d_qw, d_s, d_z, d_gu, ws, rows, 2 * inter, k, f32_out=True)
+    d_two = hip.DeviceBuffer(rows * inter * 2)
+    kernels.launch_silu_mul_f32p(d_gu, 1, d_two, rows, inter)
+    d_one = hip.DeviceBuffer(rows * inter * 2)
+    d_one.fill(0xFF)
+    kernels.launch_qgemm_q4g128_tall_swiglu_prepared(d_qw, d_s, d_z, d_one, ws, rows, inter, k)
+    hip.synchronize()
+    one = d_one.to_numpy(np.uint16, (rows, inter))
+    assert np.array_equal(one, d_two.to_numpy(np.uint16, (rows, inter)))
+    for r0, r1 in ((0, 40), (rows - 40, rows)):
+        gu = O.qgemm_q4g128_f32(xb[r0:r1], qw, s, z, r1 - r0, 2 * inter, k, None)
+        assert_parity(O.bf16_bits_to_f32(one[r0:r1]), O.bf16_bits_to_f32(OS.silu_mul_bf16(gu, inter)),
+                      what=f"gate/up + swiglu, rows {r0}..{r1}")
+
+
 def test_q4g128_workspace_kernel_is_deterministic():
     # parts of a tile split over K are summed in part order: two launches, the same bits
     rng = np.random.default_rng(92)
