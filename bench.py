@@ -379,6 +379,11 @@ def bench_mixed_config4(args):
     ms_merge, _, _ = time_launches(
         stream, [lambda: r.launch(phases=kernels.ATTN_PHASE_MERGE)], steps, warmup)
 
+    # board power while the prefill kernel loops: says whether it runs into the power cap, as
+    # the tiled GEMM does, or waits for something else at full clock
+    pre_watts, _ = board_power_watts(
+        stream, lambda: r.launch(phases=kernels.ATTN_PHASE_PREFILL), 1.5)
+
     is_dec = case["new_tokens"] == 1
     sub = lambda m: {**case, "new_tokens": case["new_tokens"][m],  # noqa: E731
                      "context_lens": case["context_lens"][m]}
@@ -412,7 +417,8 @@ def bench_mixed_config4(args):
                      "traffic": prefill_traffic, "kernel": "paged_attn_prefill_kernel<4>",
                      "flops_per_launch": flops_pre,
                      **against_mfma_ceiling(stream, False,
-                                            flops_pre / (ms_pre * 1e-3) / 1e12)},
+                                            flops_pre / (ms_pre * 1e-3) / 1e12),
+                     "board_power_W_during": pre_watts},
         "decode_rows_GBps": round(dec_bytes / (ms_dec * 1e-3) / 1e9, 1),
         "decode_rows_frac_of_peak": round(dec_bytes / (ms_dec * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
         "decode_rows": against_ceiling(stream, dec_bytes, dec_bytes / (ms_dec * 1e-3) / 1e9),
