@@ -216,6 +216,17 @@ logismos_status_t logismos_launch_qgemm_q4g128_tall_prepared(
 logismos_status_t logismos_launch_qgemm_q4g128_tall_swiglu_prepared(
     const void* gate_up_qw_u8, const void* scale_f16, const void* zero_f16, void* act_bf16,
     void* workspace, int m, int inter, int k, logismos_stream_t stream);
+/* The same, with the activations written as the operand of the product that follows (the
+ * down projection, K = inter): `next_workspace` is that product's workspace
+ * (`logismos_qgemm_q4g128_tall_workspace_bytes(m, inter)` bytes, not the one this launch
+ * reads), and receives what `logismos_launch_silu_mul_f32p_tall` would write there from the
+ * fp32 gate/up products, bit for bit -- the bf16 activations in the kernel's operand order,
+ * zero rows up to the padded row count, and the group sums in the layout for
+ * `next_pairs_per_load` (`..._pairs_per_load` of the following product's K and weights).
+ * inter a multiple of 256 * next_pairs_per_load. */
+logismos_status_t logismos_launch_qgemm_q4g128_tall_swiglu_operand(
+    const void* gate_up_qw_u8, const void* scale_f16, const void* zero_f16, void* next_workspace,
+    int next_pairs_per_load, void* workspace, int m, int inter, int k, logismos_stream_t stream);
 logismos_status_t logismos_launch_qgemm_q4g128_tall(const void* x_bf16, const void* qw_u8,
                                                     const void* scale_f16, const void* zero_f16,
                                                     const void* bias_f32, void* y, int y_is_f32,

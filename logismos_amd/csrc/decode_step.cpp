@@ -34,7 +34,8 @@ struct Workspace {
     char* t_qkv;   // f32  [T][(hq+2hkv)*d]
     char* t_proj;  // f32  [T][hidden]
     char* t_gu;    // f32  [T][2*inter]
-    char* t_act;   // bf16 [T][inter]
+    char* t_act;   // bf16 [T][inter] (or the down projection's own workspace, see carve)
+    bool t_act_is_workspace;
     char* t_gemm;  // workspace of the tiled GEMM (its copy of x in unpack order + group sums)
     // tokens for the last row of every sequence (vocab > 0)
     char* norm_out;   // bf16 [T][hidden]: the normed rows when the caller takes none (chunked
@@ -71,7 +72,14 @@ Workspace carve(const logismos_decode_config_t& c, int num_seqs, int t, int num_
         w.attn_out = take((size_t)t * qd * 2);
         w.t_proj = take((size_t)t * c.hidden * 4);
         w.t_gu = take((size_t)t * 2 * c.intermediate * 4);
-        w.t_act = take((size_t)t * c.intermediate * 2);
+        // bf16 [T][inter], or (inter a multiple of 256) a whole workspace of the tiled GEMM over
+        // K = inter: the gate/up projection then writes the down projection's operand there
+        const size_t act_rows = (size_t)t * c.intermediate * 2;
+        const size_t act_ws = c.intermediate % 256 == 0
+                                  ? logismos_qgemm_q4g128_tall_workspace_bytes(t, c.intermediate)
+                                  : 0;
+        w.t_act_is_workspace = act_ws >= act_rows && act_ws > 0;
+        w.t_act = take(w.t_act_is_workspace ? act_ws : act_rows);
         const int kmax = c.intermediate > (int)qd ? (c.intermediate > c.hidden ? c.intermediate : c.hidden)
                                                   : ((int)qd > c.hidden ? (int)qd : c.hidden);
         w.t_gemm = take(logismos_qgemm_q4g128_tall_workspace_bytes(t, kmax));
@@ -333,10 +341,25 @@ extern "C" logismos_status_t logismos_launch_decode_step(const logismos_decode_c
                     logismos_qgemm_q4g128_tall_pairs_per_load(c.hidden, L.gate_up.scale,
                                                               L.gate_up.zero),
                     stream));
-                LG_TRY(logismos_launch_qgemm_q4g128_tall_swiglu_prepared(
-                    L.gate_up.qw, L.gate_up.scale, L.gate_up.zero, w.t_act, w.t_gemm, t,
-                    c.intermediate, c.hidden, stream));
-                LG_TRY(gemm(w.t_act, L.down, nullptr, w.t_proj, c.hidden, c.intermediate));
+                if (w.t_act_is_workspace &&
+                    logismos_check_qgemm_q4g128_tall_shape(t, c.hidden, c.intermediate, nullptr,
+                                                           0) == 0) {
+                    // ... and the activations written as the down projection's operand, in its
+                    // own workspace: no bf16 rows in between, no first pass over them
+                    LG_TRY(logismos_launch_qgemm_q4g128_tall_swiglu_operand(
+                        L.gate_up.qw, L.gate_up.scale, L.gate_up.zero, w.t_act,
+                        logismos_qgemm_q4g128_tall_pairs_per_load(c.intermediate, L.down.scale,
+                                                                  L.down.zero),
+                        w.t_gemm, t, c.intermediate, c.hidden, stream));
+                    LG_TRY(logismos_launch_qgemm_q4g128_tall_prepared(
+                        L.down.qw, L.down.scale, L.down.zero, nullptr, w.t_proj, 1, w.t_act, t,
+                        c.hidden, c.intermediate, stream));
+                } else {
+                    LG_TRY(logismos_launch_qgemm_q4g128_tall_swiglu_prepared(
+                        L.gate_up.qw, L.gate_up.scale, L.gate_up.zero, w.t_act, w.t_gemm, t,
+                        c.intermediate, c.hidden, stream));
+                    LG_TRY(gemm(w.t_act, L.down, nullptr, w.t_proj, c.hidden, c.intermediate));
+                }
                 res_parts = 1;
                 continue;
             }

@@ -129,7 +129,37 @@ struct TpRegs<T, 1> {
 // the 128 up rows of the same outputs, a wave's first 32 columns the gate and its other 32 the
 // up values of the same 32 outputs, so a lane holds both products of a result and the fp32
 // gate/up products (a gigabyte at 8240 rows of a 12288-wide MLP) never go to memory.
-constexpr int kTpOutBf16 = 0, kTpOutF32 = 1, kTpOutSwiglu = 2;
+// kTpOutSwigluOperand: the same product, written as the operand of a following launch of this
+// kernel over K = n (n a multiple of 256): y is that launch's workspace -- the bf16 values in
+// pair order, rows up to the padded count (the padding rows of x are zeros, and so are their
+// activations), and the group sums (a tile's 128 outputs are one group), added up in the order
+// of the first pass (`q4_tall_prepare_kernel`), so that the workspace is bit for bit what that
+// pass makes of the bf16 activations.
+constexpr int kTpOutBf16 = 0, kTpOutF32 = 1, kTpOutSwiglu = 2, kTpOutSwigluOperand = 3;
+__host__ __device__ constexpr bool tp_is_swiglu(int out) { return out >= kTpOutSwiglu; }
+
+// 16-bit slot of element j of a 16-byte chunk in pair order ((x0,x4)(x1,x5)(x2,x6)(x3,x7))
+__device__ __forceinline__ int tp_pair_slot(int j) { return 2 * (j & 3) + (j >> 2); }
+
+// The sum of a chunk's eight values as `sum8_bf16` adds them, for values that sit one per lane
+// in eight consecutive lanes (x_j in lane 8 c + j): the chunk's first lane gets
+// (((0 + (x0 + x1)) + (x2 + x3)) + (x4 + x5)) + (x6 + x7).
+__device__ __forceinline__ float tp_chunk_sum_across_lanes(float v) {
+    const float p = v + __shfl_down(v, 1, 64);  // x_j + x_(j+1): even j count
+    float s = 0.0f + p;
+    s += __shfl_down(p, 2, 64);
+    s += __shfl_down(p, 4, 64);
+    s += __shfl_down(p, 6, 64);
+    return s;
+}
+// ... and of a row's 16 chunk sums as `row16_sum` adds them (chunk c with c + 8, those with
+// the pair of c + 4, then c + 2, then c + 1), from sums[wave column wq = c / 4][c % 4]
+__device__ __forceinline__ float tp_group_sum(const float (&cs)[4][4]) {
+    float quad[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) quad[q] = (cs[0][q] + cs[2][q]) + (cs[1][q] + cs[3][q]);
+    return (quad[0] + quad[2]) + (quad[1] + quad[3]);
+}
 
 // W: pairs of groups whose scales, zeros and group sums a lane loads at once (1, 2 or 4: a
 // dword, two or four per load; K a multiple of 256 W).
@@ -138,7 +168,7 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
     const uint16_t* __restrict__ xp, const float* __restrict__ xs, const uint8_t* __restrict__ qw,
     const __half* __restrict__ scale, const __half* __restrict__ zero,
     const float* __restrict__ bias, void* __restrict__ y_out, float* __restrict__ partials, int m,
-    int n, int k, int tiles_n, int full_tiles, int split) {
+    int n, int k, int tiles_n, int full_tiles, int split, int out_pairs) {
     extern __shared__ uint4_t tp_lds[];  // kTpBufs x {slab of x, tile of weights}
     constexpr int BL = 2 * W;            // groups per block of small loads
     const int tid = threadIdx.x;
@@ -161,11 +191,11 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
     const int row_tile = tile / tiles_n;
     const int row0 = row_tile * kTpTileM;
     // (SwiGLU: a tile is 128 outputs wide -- 128 gate and 128 up rows of the weights)
-    constexpr int kTileOutputs = OUT == kTpOutSwiglu ? kTpTileN / 2 : kTpTileN;
+    constexpr int kTileOutputs = tp_is_swiglu(OUT) ? kTpTileN / 2 : kTpTileN;
     const int col0 = (tile % tiles_n) * kTileOutputs;
     // weight row behind row L of the tile in LDS (a wave's B operand rows are L = wc + 32 j + r)
     auto weight_row = [&](int L) {
-        if constexpr (OUT == kTpOutSwiglu) {
+        if constexpr (tp_is_swiglu(OUT)) {
             const int out_col = min(col0 + (L >> 6) * 32 + (L & 31), n - 1);
             return ((L >> 5) & 1) ? n + out_col : out_col;
         } else {
@@ -486,6 +516,37 @@ __global__ __launch_bounds__(512) void qgemm_q4g128_tallp_kernel(
                 for (int e = 0; e < 16; ++e) dst[((i * 2 + j) * 16 + e) * 64] = yacc[i][j][e];
         return;
     }
+    if constexpr (OUT == kTpOutSwigluOperand) {
+        // (n is a multiple of 128 here: every column of the tile is a result)
+        const int gn = col0 + (wc >> 1) + r;
+        uint16_t* const xo = static_cast<uint16_t*>(y_out);
+        float* const so = reinterpret_cast<float*>(static_cast<char*>(y_out) + tall_sums_offset(m, n));
+        // the ring is done with once every wave has read its last operands
+        __syncthreads();
+        float* const red = reinterpret_cast<float*>(tp_lds);  // [wave column][chunk of it][row]
+        const int wq = wave & 3, cq = r >> 3;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int row = wr + 32 * i + 8 * (e >> 2) + 4 * h + (e & 3);
+                const float g = yacc[i][0][e], u = yacc[i][1][e];
+                const uint16_t b = f32_to_bf16_rne(g / (1.0f + expf(-g)) * u);
+                xo[(int64_t)(row0 + row) * n + (gn & ~7) + tp_pair_slot(gn & 7)] = b;
+                const float cs = tp_chunk_sum_across_lanes(__uint_as_float((unsigned)b << 16));
+                if ((r & 7) == 0) red[(wq * 4 + cq) * kTpTileM + row] = cs;
+            }
+        __syncthreads();
+        if (tid < kTpTileM) {
+            float cs[4][4];
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) cs[a][c] = red[(a * 4 + c) * kTpTileM + tid];
+            so[tall_sum_index(row0 + tid, col0 >> 7, n, out_pairs)] = tp_group_sum(cs);
+        }
+        return;
+    }
     if constexpr (OUT == kTpOutSwiglu) {
         const int gn = col0 + (wc >> 1) + r;
         if (gn >= n) return;
@@ -533,6 +594,7 @@ __global__ __launch_bounds__(256) void q4_tall_reduce_kernel(const float* __rest
                                                             void* __restrict__ y_out, int m, int n,
                                                             int tiles_n, int full_tiles,
                                                             int split) {
+    static_assert(OUT != kTpOutSwigluOperand, "q4_tall_reduce_operand_kernel");
     constexpr int kPerTile = OUT == kTpOutSwiglu ? kTpTileElems / 2 : kTpTileElems;
     const int t = blockIdx.x / (kPerTile / 256);
     int idx = (blockIdx.x % (kPerTile / 256)) * 256 + threadIdx.x;
@@ -564,6 +626,53 @@ __global__ __launch_bounds__(256) void q4_tall_reduce_kernel(const float* __rest
     }
 }
 
+// The same for kTpOutSwigluOperand: a workgroup takes four rows-of-registers (e = 4 eq .. + 3)
+// of one (row half, i) of a tile across all four wave columns, i.e. eight rows of the tile with
+// all their 128 outputs, so that it can add up their group sums: thread (wave column wq, lane)
+// sums the parts of the gate and the up product of its result in part order, applies the
+// activation and writes the bf16 value in pair order; chunk and group sums as in the product
+// kernel.  grid: 16 workgroups per tile.
+__global__ __launch_bounds__(256) void q4_tall_reduce_operand_kernel(
+    const float* __restrict__ partials, void* __restrict__ y_out, int m, int n, int tiles_n,
+    int full_tiles, int split, int out_pairs) {
+    __shared__ float red[4][4][8];  // [wave column][chunk of it][row of the eight]
+    const int t = blockIdx.x >> 4;
+    const int half = (blockIdx.x >> 3) & 1, i = (blockIdx.x >> 2) & 1, eq = blockIdx.x & 3;
+    const int wq = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 31, h = lane >> 5;
+    const int tile = full_tiles + t;
+    const int row0 = (tile / tiles_n) * kTpTileM, col0 = (tile % tiles_n) * (kTpTileN / 2);
+    const int gn = col0 + 32 * wq + r;
+    uint16_t* const xo = static_cast<uint16_t*>(y_out);
+    float* const so = reinterpret_cast<float*>(static_cast<char*>(y_out) + tall_sums_offset(m, n));
+    const float* src = partials + (size_t)t * split * kTpTileElems +
+                       (size_t)(half * 4 + wq) * 4096 + (size_t)i * 2048 + lane;
+#pragma unroll
+    for (int el = 0; el < 4; ++el) {
+        const int e = 4 * eq + el;
+        float g = 0.0f, u = 0.0f;
+        for (int q = 0; q < split; ++q) {
+            g += src[(size_t)q * kTpTileElems + e * 64];
+            u += src[(size_t)q * kTpTileElems + 1024 + e * 64];
+        }
+        const int row = 64 * half + 32 * i + 8 * (e >> 2) + 4 * h + (e & 3);
+        const uint16_t b = f32_to_bf16_rne(g / (1.0f + expf(-g)) * u);
+        xo[(int64_t)(row0 + row) * n + (gn & ~7) + tp_pair_slot(gn & 7)] = b;
+        const float cs = tp_chunk_sum_across_lanes(__uint_as_float((unsigned)b << 16));
+        if ((r & 7) == 0) red[wq][r >> 3][2 * el + h] = cs;
+    }
+    __syncthreads();
+    if (threadIdx.x < 8) {
+        const int el = threadIdx.x >> 1, hh = threadIdx.x & 1, e = 4 * eq + el;
+        float cs[4][4];
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) cs[a][c] = red[a][c][threadIdx.x];
+        const int row = 64 * half + 32 * i + 8 * (e >> 2) + 4 * hh + (e & 3);
+        so[tall_sum_index(row0 + row, col0 >> 7, n, out_pairs)] = tp_group_sum(cs);
+    }
+}
+
 inline int tp_pairs_per_load(int k, const void* scale, const void* zero) {
     return tall_pairs_per_load(k, scale, zero);
 }
@@ -571,13 +680,14 @@ inline int tp_pairs_per_load(int k, const void* scale, const void* zero) {
 template <int OUT, int W>
 static hipError_t tallp_launch(const uint16_t* xp, const float* xs, float* partials,
                                const uint8_t* qw, const __half* scale, const __half* zero,
-                               const float* bias, void* y, int m, int n, int k, hipStream_t st) {
+                               const float* bias, void* y, int m, int n, int k, hipStream_t st,
+                               int out_pairs = 0) {
     constexpr size_t lds = (size_t)kTpBufs * kTpBufBytes;
     static const hipError_t opt = hipFuncSetAttribute(
         reinterpret_cast<const void*>(qgemm_q4g128_tallp_kernel<OUT, W>),
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (opt != hipSuccess) return opt;
-    constexpr int tile_outputs = OUT == kTpOutSwiglu ? kTpTileN / 2 : kTpTileN;
+    constexpr int tile_outputs = tp_is_swiglu(OUT) ? kTpTileN / 2 : kTpTileN;
     const int tiles_n = (n + tile_outputs - 1) / tile_outputs;
     const int tiles = tiles_n * (tp_padded_rows(m) / kTpTileM);
     const int cus = device_cu_count();
@@ -586,12 +696,18 @@ static hipError_t tallp_launch(const uint16_t* xp, const float* xs, float* parti
     const int parts = (tiles - plan.full) * plan.split;
     qgemm_q4g128_tallp_kernel<OUT, W>
         <<<dim3(plan.full + (plan.split > 1 ? parts : 0)), dim3(512), lds, st>>>(
-            xp, xs, qw, scale, zero, bias, y, partials, m, n, k, tiles_n, plan.full, plan.split);
+            xp, xs, qw, scale, zero, bias, y, partials, m, n, k, tiles_n, plan.full, plan.split,
+            out_pairs);
     if (plan.split > 1) {
-        constexpr int per_tile = OUT == kTpOutSwiglu ? kTpTileElems / 2 : kTpTileElems;
-        q4_tall_reduce_kernel<OUT>
-            <<<dim3((tiles - plan.full) * (per_tile / 256)), dim3(256), 0, st>>>(
-                partials, bias, y, m, n, tiles_n, plan.full, plan.split);
+        if constexpr (OUT == kTpOutSwigluOperand) {
+            q4_tall_reduce_operand_kernel<<<dim3((tiles - plan.full) * 16), dim3(256), 0, st>>>(
+                partials, y, m, n, tiles_n, plan.full, plan.split, out_pairs);
+        } else {
+            constexpr int per_tile = OUT == kTpOutSwiglu ? kTpTileElems / 2 : kTpTileElems;
+            q4_tall_reduce_kernel<OUT>
+                <<<dim3((tiles - plan.full) * (per_tile / 256)), dim3(256), 0, st>>>(
+                    partials, bias, y, m, n, tiles_n, plan.full, plan.split);
+        }
     }
     return hipGetLastError();
 }
@@ -599,11 +715,18 @@ static hipError_t tallp_launch(const uint16_t* xp, const float* xs, float* parti
 template <int OUT>
 static hipError_t tallp_launch_w(int w, const uint16_t* xp, const float* xs, float* partials,
                                  const uint8_t* qw, const __half* scale, const __half* zero,
-                                 const float* bias, void* y, int m, int n, int k, hipStream_t st) {
+                                 const float* bias, void* y, int m, int n, int k, hipStream_t st,
+                                 int out_pairs = 0) {
     switch (w) {
-        case 4: return tallp_launch<OUT, 4>(xp, xs, partials, qw, scale, zero, bias, y, m, n, k, st);
-        case 2: return tallp_launch<OUT, 2>(xp, xs, partials, qw, scale, zero, bias, y, m, n, k, st);
-        default: return tallp_launch<OUT, 1>(xp, xs, partials, qw, scale, zero, bias, y, m, n, k, st);
+        case 4:
+            return tallp_launch<OUT, 4>(xp, xs, partials, qw, scale, zero, bias, y, m, n, k, st,
+                                        out_pairs);
+        case 2:
+            return tallp_launch<OUT, 2>(xp, xs, partials, qw, scale, zero, bias, y, m, n, k, st,
+                                        out_pairs);
+        default:
+            return tallp_launch<OUT, 1>(xp, xs, partials, qw, scale, zero, bias, y, m, n, k, st,
+                                        out_pairs);
     }
 }
 
@@ -692,6 +815,36 @@ extern "C" logismos_status_t logismos_launch_qgemm_q4g128_tall_swiglu_prepared(
         w, xp, xs, partials, static_cast<const uint8_t*>(gate_up_qw_u8),
         static_cast<const __half*>(scale_f16), static_cast<const __half*>(zero_f16), nullptr,
         act_bf16, m, inter, k, st);
+}
+
+extern "C" logismos_status_t logismos_launch_qgemm_q4g128_tall_swiglu_operand(
+    const void* gate_up_qw_u8, const void* scale_f16, const void* zero_f16, void* next_workspace,
+    int next_pairs_per_load, void* workspace, int m, int inter, int k, logismos_stream_t stream) {
+    // the output is the operand of a product over K = inter: whole pairs of groups, and as many
+    // pairs per load as the caller's next launch will ask for (whole blocks of them)
+    if (inter <= 0 || inter > INT32_MAX / 2 || inter % 256 != 0) return hipErrorInvalidValue;
+    if (next_pairs_per_load != 1 && next_pairs_per_load != 2 && next_pairs_per_load != 4)
+        return hipErrorInvalidValue;
+    if (inter % (256 * next_pairs_per_load) != 0) return hipErrorInvalidValue;
+    if (const logismos_status_t e = tall_args_ok(gate_up_qw_u8, scale_f16, zero_f16,
+                                                 next_workspace, workspace, m, 2 * inter, k))
+        return e;
+    // (the next launch's own shape: rows * inter * 2 within 32 bits)
+    if (logismos_check_qgemm_q4g128_tall_shape(m, 1, inter, nullptr, 0) != 0)
+        return hipErrorInvalidValue;
+    if ((reinterpret_cast<uintptr_t>(next_workspace) & 15u) || next_workspace == workspace)
+        return hipErrorInvalidValue;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint16_t* xp = static_cast<const uint16_t*>(workspace);
+    const float* xs =
+        reinterpret_cast<const float*>(static_cast<char*>(workspace) + lg::tp_sums_offset(m, k));
+    float* partials = reinterpret_cast<float*>(static_cast<char*>(workspace) +
+                                               lg::tp_partials_offset(m, k));
+    const int w = lg::tp_pairs_per_load(k, scale_f16, zero_f16);
+    return lg::tallp_launch_w<lg::kTpOutSwigluOperand>(
+        w, xp, xs, partials, static_cast<const uint8_t*>(gate_up_qw_u8),
+        static_cast<const __half*>(scale_f16), static_cast<const __half*>(zero_f16), nullptr,
+        next_workspace, m, inter, k, st, next_pairs_per_load);
 }
 
 extern "C" logismos_status_t logismos_launch_qgemm_q4g128_tall(

@@ -63,6 +63,8 @@ _SIGNATURES = {
     "logismos_launch_silu_mul_f32p_tall": (C.c_uint32, [_vp, _i, _vp, _i, _i, _i, _vp]),
     "logismos_launch_qgemm_q4g128_tall_swiglu_prepared":
         (C.c_uint32, [_vp] * 5 + [_i, _i, _i, _vp]),
+    "logismos_launch_qgemm_q4g128_tall_swiglu_operand":
+        (C.c_uint32, [_vp] * 4 + [_i, _vp, _i, _i, _i, _vp]),
     "logismos_launch_add_rms_norm_f32p_tall":
         (C.c_uint32, [_vp, _vp, _i, _vp, _vp, _i, _i, _f, _i, _vp]),
     "logismos_launch_repack_q8_0": (C.c_uint32, [_vp, _vp, _vp, _i, _i, _vp]),
@@ -335,6 +337,17 @@ def launch_qgemm_q4g128_tall_swiglu_prepared(qw, scale, zero, act, workspace, m:
             library().logismos_launch_qgemm_q4g128_tall_swiglu_prepared(
                 _ptr(qw), _ptr(scale), _ptr(zero), _ptr(act), _ptr(workspace), m, inter, k,
                 _raw(stream)))
+
+
+def launch_qgemm_q4g128_tall_swiglu_operand(qw, scale, zero, next_workspace,
+                                            next_pairs_per_load: int, workspace, m: int,
+                                            inter: int, k: int, stream=None) -> None:
+    """gate/up projection + SwiGLU, written as the operand of the following product."""
+    _guard("qgemm_q4g128_tall", library().logismos_check_qgemm_q4g128_tall_shape, m, 2 * inter, k)
+    _status("qgemm_q4g128_tall_swiglu_operand",
+            library().logismos_launch_qgemm_q4g128_tall_swiglu_operand(
+                _ptr(qw), _ptr(scale), _ptr(zero), _ptr(next_workspace), next_pairs_per_load,
+                _ptr(workspace), m, inter, k, _raw(stream)))
 
 
 def launch_silu_mul_f32p_tall(parts, num_parts: int, workspace, rows: int, inter: int,

@@ -329,6 +329,66 @@ def test_gate_up_projection_with_the_swiglu_in_the_kernel(rows, inter, k):
     assert_parity(O.bf16_bits_to_f32(one), O.bf16_bits_to_f32(want), what="gate/up + swiglu")
 
 
+@pytest.mark.parametrize("rows,inter,k", [(200, 1024, 512), (130, 512, 1024), (97, 256, 768),
+                                          (520, 2560, 2048), (1100, 3840, 512)])
+def test_gate_up_projection_writing_the_down_projections_operand(rows, inter, k):
+    # the gate/up projection with the SwiGLU, its result written straight into the workspace of
+    # the product that follows (K = inter), against the route through memory: fp32 gate/up
+    # products, then `silu_mul_f32p_tall`.  The same bf16 values in the same places, zero
+    # padding rows, the group sums added in the same order: the operand part of the two
+    # workspaces is the same bytes -- for whole tiles (the last shape has more tiles than the
+    # device has units) and for tiles split over K (the others), four, two and one pair of
+    # groups per load of the following product.
+    rng = np.random.default_rng(rows + inter + k + 1)
+    qw, s, z = _q4(rng, 2 * inter, k)
+    xb = O.f32_to_bf16_bits(rng.standard_normal((rows, k), np.float32))
+    d_x, d_qw = up(xb), up(qw)
+    d_s, d_z = up(s.view(np.uint16)), up(z.view(np.uint16))
+    ws = hip.DeviceBuffer(kernels.qgemm_q4g128_tall_workspace_bytes(rows, k))
+    w_next = 4 if inter % 1024 == 0 else 2 if inter % 512 == 0 else 1
+    nbytes = kernels.qgemm_q4g128_tall_workspace_bytes(rows, inter)
+    d_gu = hip.DeviceBuffer(rows * 2 * inter * 4)
+    kernels.launch_qgemm_q4g128_tall(d_x, d_qw, d_s, d_z, d_gu, ws, rows, 2 * inter, k, f32_out=True)
+    ws_two = hip.DeviceBuffer(nbytes)
+    ws_two.fill(0xFF)
+    kernels.launch_silu_mul_f32p_tall(d_gu, 1, ws_two, rows, inter, w_next)
+    ws_one = hip.DeviceBuffer(nbytes)
+    ws_one.fill(0xEE)
+    kernels.launch_qgemm_q4g128_tall_swiglu_operand(d_qw, d_s, d_z, ws_one, w_next, ws, rows,
+                                                    inter, k)
+    hip.synchronize()
+    rows_pad = -(-rows // 128) * 128
+    head = rows_pad * inter * 2
+    sums_at = (head + 255) // 256 * 256
+    sums = rows_pad * (inter // 128) * 4
+    a, b = ws_one.to_numpy(np.uint8, (nbytes,)), ws_two.to_numpy(np.uint8, (nbytes,))
+    assert np.array_equal(a[:head], b[:head])
+    assert not a[rows * inter * 2:head].any()
+    sa = a[sums_at:sums_at + sums].view(np.float32)
+    sb = b[sums_at:sums_at + sums].view(np.float32)
+    assert np.array_equal(sa.view(np.uint32), sb.view(np.uint32))
+    # what lies behind the operand (the following product's partial tiles) is not touched
+    assert np.all(a[sums_at + sums:] == 0xEE)
+
+
+def test_gate_up_operand_refusals():
+    rng = np.random.default_rng(3)
+    rows, inter, k = 130, 384, 512  # inter is not a multiple of 256
+    qw, s, z = _q4(rng, 2 * inter, k)
+    d_qw, d_s, d_z = up(qw), up(s.view(np.uint16)), up(z.view(np.uint16))
+    ws = hip.DeviceBuffer(kernels.qgemm_q4g128_tall_workspace_bytes(rows, k))
+    nxt = hip.DeviceBuffer(kernels.qgemm_q4g128_tall_workspace_bytes(rows, 512))
+    with pytest.raises(kernels.LaunchError):
+        kernels.launch_qgemm_q4g128_tall_swiglu_operand(d_qw, d_s, d_z, nxt, 1, ws, rows, inter, k)
+    qw, s, z = _q4(rng, 1024, k)
+    d_qw, d_s, d_z = up(qw), up(s.view(np.uint16)), up(z.view(np.uint16))
+    with pytest.raises(kernels.LaunchError):  # 512 is not a whole block of four pairs
+        kernels.launch_qgemm_q4g128_tall_swiglu_operand(d_qw, d_s, d_z, nxt, 4, ws, rows, 512, k)
+    with pytest.raises(kernels.LaunchError):  # one workspace for both
+        kernels.launch_qgemm_q4g128_tall_swiglu_operand(d_qw, d_s, d_z, ws, 2, ws, rows, 512, k)
+    hip.synchronize()
+
+
 def test_gate_up_with_the_swiglu_on_more_tiles_than_the_device_has_units():
     # 9 x 30 = 270 tiles of 128 rows x 128 outputs: the first 256 whole, the other 14 split over
     # K with the activation applied where their parts are summed; bit for bit the two-step form
