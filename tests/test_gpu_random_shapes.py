@@ -1,5 +1,6 @@
-"""Seeded random shapes: the tiled Q4G128 GEMM with a workspace in every output mode, and the
-step executor at random geometries, against the CPU oracle through the C ABI.
+"""Seeded random shapes: the tiled Q4G128 GEMM with a workspace in every output mode, the
+step executor at random geometries and the paged-attention launcher on random ragged batches,
+against the CPU oracle through the C ABI.
 
 The parametrised tests of the other files pick their shapes by hand (tile edges, split tiles,
 alignment classes); these draw them, so that a combination nobody thought of is still seen:
@@ -149,3 +150,40 @@ def test_step_executor_random_geometries(seed):
         # (the whole-step bounds of test_gpu_decode_step.py: 6e-3 over fp16 pools, wider over
         # turbo3 pools, whose encoder turns a last-bit difference of a row into another code)
         assert rel < (2.5e-2 if t3 else 6e-3), f"{what}: rel L2 {rel:.2e}"
+
+
+@pytest.mark.parametrize("seed", [301, 302])
+def test_paged_attention_random_ragged_batches(seed):
+    # head widths 32..256, GQA groups 1..16, block sizes 16 / 32 / 64, decode rows, short and
+    # long chunks, prior contexts on and around block edges, narrow block tables (static
+    # split) and wide ones (balanced split), causal and not
+    from tests.gpu_harness import PagedAttnRunner
+    rng = np.random.default_rng(seed)
+    for case in range(25):
+        d = int(rng.choice([128, 128, 128, 32, 64, 96, 160, 256]))
+        hkv = int(rng.choice([1, 2, 4, 8]))
+        group = int(rng.integers(1, 9)) if d == 128 else int(rng.choice([1, 2, 3, 4, 7, 8, 16]))
+        hq = hkv * group
+        bs = int(rng.choice([16, 32, 64]))
+        nseq = int(rng.integers(1, 20))
+        kind = int(rng.integers(0, 3))
+        if kind == 0:
+            new = np.ones(nseq, np.int32)
+        elif kind == 1:
+            new = rng.choice([1, 1, 2, 5, 17, 40], size=nseq).astype(np.int32)
+        else:
+            new = rng.choice([1, 64, 100, 130], size=nseq).astype(np.int32)
+        prior = rng.choice([0, 1, 15, 16, 17, 100, 500, 1500, 3000], size=nseq).astype(np.int32)
+        wide = int(rng.choice([1, 1, 600]))
+        causal = bool(rng.integers(0, 4) > 0)
+        what = (f"seed {seed} case {case}: d={d} hq={hq} hkv={hkv} block={bs} new={new.tolist()} "
+                f"prior={prior.tolist()} min_max_blocks={wide} causal={causal}")
+        c = workloads.paged_case(rng, new, prior, hq, hkv, d, bs, min_max_blocks=wide)
+        r = PagedAttnRunner(c, causal=causal)
+        r.launch()
+        got = r.result().astype(np.float32)
+        want = O.paged_attn_varlen_fp16(c["q"], c["k_pool"], c["v_pool"], c["block_tables"],
+                                        c["cu_seqlens"], c["context_lens"], hq, hkv, d, bs,
+                                        c["scale"], causal).astype(np.float32)
+        assert np.isfinite(got).all(), what
+        assert _out_of_tolerance(got, want, 2e-3, 1e-2) == 0, what
