@@ -187,3 +187,44 @@ def test_paged_attention_random_ragged_batches(seed):
                                         c["scale"], causal).astype(np.float32)
         assert np.isfinite(got).all(), what
         assert _out_of_tolerance(got, want, 2e-3, 1e-2) == 0, what
+
+
+@pytest.mark.parametrize("seed", [401, 402])
+def test_small_batch_products_random_shapes(seed):
+    # the Q8G32 GEMV and the Q4G128 product at any batch (the GEMV for 1-2 rows, the
+    # matrix-core kernels in passes of 32 rows, a ragged last pass), N from 1 to thousands,
+    # K from one group up and off the kernels' fast paths, with and without a bias
+    rng = np.random.default_rng(seed)
+    for case in range(40):
+        n = int(rng.choice([1, 7, 16, 33, 100, 1000, 1024, 1536, 4096, 5000]))
+        bias = rng.standard_normal(n).astype(np.float32) if rng.integers(0, 2) else None
+        d_bias = up(bias) if bias is not None else None
+        if rng.integers(0, 2):
+            k = int(rng.choice([32, 64, 96, 512, 1536, 4096, 8192, 2080]))
+            w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
+            qs, d = O.quantize_q8g32(w, n, k)
+            x = rng.standard_normal(k).astype(np.float32)
+            what = f"seed {seed} case {case}: Q8G32 GEMV n={n} k={k} bias={bias is not None}"
+            y = hip.DeviceBuffer(n * 4)
+            y.fill(0xFF)
+            kernels.launch_qgemv_q8g32_f32(up(x), up(qs), up(d.view(np.uint16)), y, n, k,
+                                           bias=d_bias)
+            hip.synchronize()
+            got, tol = y.to_numpy(np.float32, (n,)), (2e-4, 1e-3)
+            want = O.qgemv_q8g32_f32(x, qs, d, n, k, bias)
+        else:
+            k = int(rng.choice([128, 256, 384, 1024, 2048, 4096, 4224]))
+            b = int(rng.choice([1, 2, 3, 4, 7, 8, 15, 16, 17, 31, 32, 33, 40, 64, 65, 70]))
+            w = rng.standard_normal((n, k), np.float32) * np.float32(0.02)
+            qw, s, z = O.quantize_q4g128(w, n, k)
+            xb = O.f32_to_bf16_bits(rng.standard_normal((b, k), np.float32))
+            what = f"seed {seed} case {case}: Q4G128 b={b} n={n} k={k} bias={bias is not None}"
+            y = hip.DeviceBuffer(b * n * 2)
+            y.fill(0xFF)
+            kernels.launch_qgemm_q4g128_bf16(up(xb), up(qw), up(s.view(np.uint16)),
+                                             up(z.view(np.uint16)), y, b, n, k, bias=d_bias)
+            hip.synchronize()
+            got, tol = O.bf16_bits_to_f32(y.to_numpy(np.uint16, (b, n))), (2e-3, 1e-2)
+            want = O.bf16_bits_to_f32(O.qgemm_q4g128_bf16(xb, qw, s, z, b, n, k, bias))
+        assert np.isfinite(got).all(), what
+        assert _out_of_tolerance(got, want, *tol) == 0, what
