@@ -296,3 +296,52 @@ def test_steps_that_take_the_admitted_prompt_as_a_chunk_of_the_batch():
             assert cache.len_of(s, 0) == lens[s]
     assert rig.clear_total >= 20
     rig.check_pools_and_blocks(lens)
+
+
+def test_twelve_steps_of_random_churn():
+    """A longer loop with the schedule drawn: every step retires none, one or two sequences
+    (always one that would outgrow its block table), and admits each replacement either with
+    its prompt `put` beforehand or as a chunk of the step's own batch; the blocks a retired
+    sequence held go back to the free list and out again many times over."""
+    rng = np.random.default_rng(79)
+    rig = _Rig(rng, 32)
+    cache = rig.cache
+    prompts = [12, 45, 3, 60, 28, 16]
+    assert [rig.admit(p) for p in prompts] == list(range(SEQS))
+    lens = list(prompts)
+    last = rng.integers(0, VOCAB, size=SEQS, dtype=np.uint32)
+    retired = 0
+    for step in range(12):
+        out = [s for s in range(SEQS) if lens[s] + 1 > 80]          # would outgrow 6 blocks
+        extra = [int(s) for s in rng.permutation(SEQS)[:int(rng.integers(0, 3))]]
+        out = list(dict.fromkeys(out + extra))[:3]
+        new = [1] * SEQS
+        tok = {s: last[s:s + 1] for s in range(SEQS)}
+        room = 32 - SEQS                                            # rows left for chunks
+        for s in out:
+            held = -(-lens[s] // BS)
+            free0 = cache.free_blocks()
+            cache.close_seq(s)
+            assert cache.free_blocks() == free0 + held
+            retired += 1
+            if room >= 2 and rng.integers(0, 2):
+                # the step takes the prompt itself: a chunk of its batch
+                assert cache.open_seq() == s and cache.len_of(s, 0) == 0
+                chunk = int(rng.integers(2, min(room, 20) + 1))
+                room -= chunk - 1
+                lens[s], new[s] = 0, chunk
+                tok[s] = rng.integers(0, VOCAB, size=chunk, dtype=np.uint32)
+            else:
+                plen = int(rng.integers(3, 50))
+                assert rig.admit(plen) == s
+                lens[s] = plen
+                tok[s] = rng.integers(0, VOCAB, size=1, dtype=np.uint32)
+        tok_in = np.concatenate([tok[s] for s in range(SEQS)])
+        tok_out, cu = rig.step(lens, new, tok_in, f"step {step}, retired {out}, new {new}")
+        last = tok_out[cu[1:] - 1]
+        lens = [n + k for n, k in zip(lens, new)]
+        for s in range(SEQS):
+            assert cache.len_of(s, 0) == lens[s]
+        assert cache.free_blocks() == NUM_BLOCKS - sum(-(-n // BS) for n in lens)
+    assert retired >= 8 and rig.clear_total >= 50
+    rig.check_pools_and_blocks(lens)
